@@ -1,0 +1,8 @@
+"""MI355X-native quantized decode path behind the reference's backend interface.
+
+``fandhe_ai_amd.backend`` mirrors the reference's ``BackendOps`` / ``MemoryOps``
+surface for ``Device::Rocm``; ``fandhe_ai_amd.capi`` is the ctypes view of the C
+ABI (include/fandhe_rocm.h) in ``lib/libfandhe_rocm.so``.
+"""
+from . import capi  # noqa: F401  (raises if the HIP library is not built)
+from .backend import *  # noqa: F401,F403

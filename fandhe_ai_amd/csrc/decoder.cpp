@@ -1,0 +1,368 @@
+// One decode step of a Llama-style decoder on resident state: the
+// composition of the quantized linears, RMSNorm, RoPE, paged attention and
+// greedy argmax that the benchmark's full-step configuration names.  All
+// buffers are allocated when the decoder is created; a step only enqueues
+// kernels, so it can be captured once into a HIP graph and replayed.
+#include <cmath>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "kernels.hpp"
+#include "runtime.hpp"
+#include "validate.hpp"
+
+using namespace fa;
+
+namespace fa {
+extern int g_decode_ppc;
+}
+
+struct fa_decoder {
+    uint32_t magic;
+    fa_context *ctx;
+    fa_decoder_config cfg;
+    struct Layer {
+        const fa_buffer *attn_norm = nullptr, *ffn_norm = nullptr;
+        const fa_qweight *wqkv = nullptr, *wo = nullptr, *wgu = nullptr, *wdown = nullptr;
+        fa_buffer *k_pool = nullptr, *v_pool = nullptr;
+    };
+    std::vector<Layer> layers;
+    const fa_buffer *embed = nullptr, *final_norm = nullptr;
+    const fa_qweight *lm_head = nullptr;
+    uint32_t batch = 0;
+    // resident state and activations
+    fa_buffer *tokens = nullptr, *tables = nullptr, *seq_lens = nullptr, *pos = nullptr, *slots = nullptr;
+    fa_buffer *cos_sin = nullptr, *h = nullptr, *xq = nullptr, *sx = nullptr, *qkv = nullptr, *q_bf = nullptr;
+    fa_buffer *attn = nullptr, *gu = nullptr, *logits = nullptr;
+    fa_graph *graph = nullptr;
+    uint32_t graph_batch = 0;
+    int graph_ppc = 0;
+};
+
+namespace {
+
+constexpr uint32_t kDecMagic = 0xFA0DEC01u;
+
+uint64_t round_up(uint64_t v, uint64_t to) { return (v + to - 1) / to * to; }
+
+fa_status check_dec(const fa_decoder *d) {
+    if (!d || d->magic != kDecMagic) return fail(FA_ERR_INVALID_ARGUMENT, "decoder: not a decoder");
+    return FA_OK;
+}
+
+fa_status check_weight(const fa_decoder *d, const fa_qweight *qw, uint64_t k, uint64_t n, const char *what) {
+    if (!qw || qw->magic != kQwMagic) return fail(FA_ERR_INVALID_ARGUMENT, std::string(what) + ": not a quantized weight");
+    if (qw->ctx != d->ctx) return fail(FA_ERR_DEVICE_MISMATCH, std::string(what) + ": weight belongs to another context");
+    if (qw->kind != FA_QW_INT8_CHANNEL) return fail(FA_ERR_INVALID_ARGUMENT, std::string(what) + ": must be an int8 weight");
+    if (qw->k != k || qw->n != n)
+        return fail(FA_ERR_SHAPE_MISMATCH, std::string(what) + ": expected [" + std::to_string(k) + ", " +
+                                               std::to_string(n) + "], got [" + std::to_string(qw->k) + ", " +
+                                               std::to_string(qw->n) + "]");
+    return FA_OK;
+}
+
+fa_status check_vec(const fa_decoder *d, const fa_buffer *b, uint64_t numel, const char *what) {
+    if (fa_status s = check_buf_typed(d->ctx, b, FA_F32, numel, what)) return s;
+    if (b->numel != numel) return fail(FA_ERR_SHAPE_MISMATCH, std::string(what) + ": wrong length");
+    return FA_OK;
+}
+
+void free_all(fa_context *ctx, fa_decoder *d) {
+    fa_buffer **bufs[] = {&d->tokens, &d->tables, &d->seq_lens, &d->pos, &d->slots, &d->cos_sin, &d->h, &d->xq,
+                          &d->sx,     &d->qkv,    &d->q_bf,     &d->attn, &d->gu,   &d->logits};
+    for (auto pb : bufs) {
+        if (*pb) fa_buffer_free(ctx, *pb);
+        *pb = nullptr;
+    }
+    for (auto &l : d->layers) {
+        if (l.k_pool) fa_buffer_free(ctx, l.k_pool);
+        if (l.v_pool) fa_buffer_free(ctx, l.v_pool);
+        l.k_pool = l.v_pool = nullptr;
+    }
+}
+
+// The kernels of one step, enqueued on the context's stream.
+fa_status enqueue_step(fa_context *ctx, fa_decoder *d) {
+    const fa_decoder_config &c = d->cfg;
+    const uint32_t B = d->batch;
+    const uint64_t D = c.d_model, H = c.n_heads, HKV = c.n_kv_heads, DH = c.head_dim, F = c.d_ffn, V = c.vocab;
+    const uint64_t EQ = H * DH, EKV = HKV * DH;
+    const uint64_t m_pad = round_up(B, 16);
+    const int cus = ctx->props.multiProcessorCount;
+    hipStream_t s = ctx->stream;
+    const uint64_t pool_rows = (uint64_t)c.num_blocks * c.block_size;
+
+    k::decode_prepare((const uint32_t *)d->tables->ptr, (uint32_t *)d->seq_lens->ptr, (int32_t *)d->pos->ptr,
+                      (uint32_t *)d->slots->ptr, (float *)d->cos_sin->ptr, B, c.block_size, c.max_blocks_per_seq,
+                      c.num_blocks, c.head_dim, c.rope_theta, s);
+    k::gather_rows_f32((const float *)d->embed->ptr, V, D, (const int32_t *)d->tokens->ptr, (float *)d->h->ptr, B, s);
+
+    k::PagedShape ps;
+    ps.num_blocks = c.num_blocks;
+    ps.block_size = c.block_size;
+    ps.e_kv = (uint32_t)EKV;
+    ps.batch = B;
+    ps.l_new = 1;
+    ps.num_heads = c.n_heads;
+    ps.num_kv_heads = c.n_kv_heads;
+    ps.head_dim = c.head_dim;
+    ps.max_blocks_per_seq = c.max_blocks_per_seq;
+    ps.scale = 1.0f / std::sqrt((float)c.head_dim);
+
+    auto epilogue = [&](const fa_qweight *w, void *out, const float *residual) {
+        k::EpilogueI8 ep;
+        ep.sx = (const float *)d->sx->ptr;
+        ep.sw = (const float *)w->scales->ptr;
+        ep.bias = nullptr;
+        ep.residual = residual;
+        ep.acc_out = nullptr;
+        ep.out = out;
+        ep.out_bf16 = 0;
+        return ep;
+    };
+    auto linear = [&](const fa_qweight *w, void *out, const float *residual) {
+        k::linear_w8a8_skinny((const int8_t *)d->xq->ptr, (const int8_t *)w->codes->ptr, B, w->n, w->n_pad, w->k_pad,
+                              epilogue(w, out, residual), cus, s);
+    };
+
+    for (uint32_t li = 0; li < c.n_layers; ++li) {
+        const fa_decoder::Layer &L = d->layers[li];
+        k::rmsnorm_quantize_i8((const float *)d->h->ptr, (const float *)L.attn_norm->ptr, c.rms_eps, nullptr,
+                               (int8_t *)d->xq->ptr, (float *)d->sx->ptr, B, m_pad, D, s);
+        linear(L.wqkv, d->qkv->ptr, nullptr);
+        k::qkv_rope_append((const float *)d->qkv->ptr, (const float *)d->cos_sin->ptr, (const uint32_t *)d->slots->ptr,
+                           (uint16_t *)d->q_bf->ptr, (uint16_t *)L.k_pool->ptr, (uint16_t *)L.v_pool->ptr, B,
+                           c.n_heads, c.n_kv_heads, c.head_dim, pool_rows, s);
+        k::paged_attention_decode_bf16((const uint16_t *)d->q_bf->ptr, (const uint16_t *)L.k_pool->ptr,
+                                       (const uint16_t *)L.v_pool->ptr, (const uint32_t *)d->tables->ptr,
+                                       (const uint32_t *)d->seq_lens->ptr, ps, (uint32_t)g_decode_ppc, ctx->workspace,
+                                       d->attn->ptr, 1, s);
+        k::quantize_rows_i8(d->attn->ptr, true, nullptr, (int8_t *)d->xq->ptr, (float *)d->sx->ptr, B, m_pad, EQ, EQ, s);
+        linear(L.wo, d->h->ptr, (const float *)d->h->ptr);
+        k::rmsnorm_quantize_i8((const float *)d->h->ptr, (const float *)L.ffn_norm->ptr, c.rms_eps, nullptr,
+                               (int8_t *)d->xq->ptr, (float *)d->sx->ptr, B, m_pad, D, s);
+        linear(L.wgu, d->gu->ptr, nullptr);
+        k::swiglu_quantize_i8((const float *)d->gu->ptr, (int8_t *)d->xq->ptr, (float *)d->sx->ptr, B, m_pad, F, s);
+        linear(L.wdown, d->h->ptr, (const float *)d->h->ptr);
+    }
+    k::rmsnorm_quantize_i8((const float *)d->h->ptr, (const float *)d->final_norm->ptr, c.rms_eps, nullptr,
+                           (int8_t *)d->xq->ptr, (float *)d->sx->ptr, B, m_pad, D, s);
+    linear(d->lm_head, d->logits->ptr, nullptr);
+    k::argmax_rows_f32((const float *)d->logits->ptr, (int32_t *)d->tokens->ptr, B, V, s);
+    return after_launch(ctx, "decoder step");
+}
+
+}  // namespace
+
+extern "C" {
+
+fa_status fa_decoder_create(fa_context *ctx, const fa_decoder_config *cfg, fa_decoder **out) {
+    if (fa_status s = check_ctx(ctx)) return s;
+    if (!cfg || !out) return fail(FA_ERR_INVALID_ARGUMENT, "decoder_create: null argument");
+    if (ctx->capturing) return fail(FA_ERR_CAPTURE_IN_PROGRESS, "decoder_create during graph capture");
+    const fa_decoder_config &c = *cfg;
+    if (c.n_layers == 0 || c.d_model == 0 || c.n_heads == 0 || c.n_kv_heads == 0 || c.d_ffn == 0 || c.vocab == 0 ||
+        c.max_batch == 0)
+        return fail(FA_ERR_INVALID_ARGUMENT, "decoder_create: zero dimension");
+    if (c.head_dim != 128 || c.block_size != 16)
+        return fail(FA_ERR_UNSUPPORTED, "decoder_create: head_dim must be 128 and block_size 16");
+    if (c.n_heads % c.n_kv_heads != 0 || c.n_heads / c.n_kv_heads > 8)
+        return fail(FA_ERR_UNSUPPORTED, "decoder_create: heads per kv head must be an integer of at most 8");
+    if (c.d_model % 64 != 0 || c.d_ffn % 64 != 0)
+        return fail(FA_ERR_UNSUPPORTED, "decoder_create: d_model and d_ffn must be multiples of 64");
+    if (c.max_batch > 32) return fail(FA_ERR_UNSUPPORTED, "decoder_create: at most 32 sequences per step");
+    if (!std::isfinite(c.rms_eps) || c.rms_eps < 0.0f) return fail(FA_ERR_INVALID_ARGUMENT, "decoder_create: bad rms_eps");
+    if (!(c.rope_theta > 0.0)) return fail(FA_ERR_INVALID_ARGUMENT, "decoder_create: bad rope_theta");
+    fa_paged_layout layout{c.num_blocks, c.block_size, (uint64_t)c.n_kv_heads * c.head_dim};
+    if (fa_status s = paged_layout_check(&layout)) return s;
+    if (c.max_blocks_per_seq == 0 || (uint64_t)c.max_blocks_per_seq * c.block_size > (uint64_t)INT32_MAX)
+        return fail(FA_ERR_INVALID_ARGUMENT, "decoder_create: bad max_blocks_per_seq");
+
+    fa_decoder *d = new (std::nothrow) fa_decoder();
+    if (!d) return fail(FA_ERR_ALLOCATION_FAILED, "decoder_create: host allocation failed");
+    d->magic = kDecMagic;
+    d->ctx = ctx;
+    d->cfg = c;
+    d->layers.resize(c.n_layers);
+    const uint64_t B = c.max_batch, D = c.d_model, F = c.d_ffn, V = c.vocab;
+    const uint64_t EQ = (uint64_t)c.n_heads * c.head_dim, EKV = (uint64_t)c.n_kv_heads * c.head_dim;
+    const uint64_t kmax = std::max(std::max(D, F), EQ);
+    fa_status s = FA_OK;
+    auto mk = [&](fa_dtype t, uint64_t n, fa_buffer **b) {
+        if (s == FA_OK) s = make_buffer(ctx, t, n, true, b);
+    };
+    mk(FA_I32, B, &d->tokens);
+    mk(FA_U32, B * c.max_blocks_per_seq, &d->tables);
+    mk(FA_U32, B, &d->seq_lens);
+    mk(FA_I32, B, &d->pos);
+    mk(FA_U32, B, &d->slots);
+    mk(FA_F32, B * c.head_dim, &d->cos_sin);
+    mk(FA_F32, B * D, &d->h);
+    mk(FA_I8, round_up(B, 16) * kmax, &d->xq);
+    mk(FA_F32, B, &d->sx);
+    mk(FA_F32, B * (EQ + 2 * EKV), &d->qkv);
+    mk(FA_BF16, B * EQ, &d->q_bf);
+    mk(FA_BF16, B * EQ, &d->attn);
+    mk(FA_F32, B * 2 * F, &d->gu);
+    mk(FA_F32, B * V, &d->logits);
+    for (auto &l : d->layers) {
+        mk(FA_BF16, layout.num_blocks * layout.block_size * layout.embed_dim, &l.k_pool);
+        mk(FA_BF16, layout.num_blocks * layout.block_size * layout.embed_dim, &l.v_pool);
+    }
+    if (s != FA_OK) {
+        free_all(ctx, d);
+        delete d;
+        return s;
+    }
+    *out = d;
+    return FA_OK;
+}
+
+fa_status fa_decoder_destroy(fa_context *ctx, fa_decoder *d) {
+    if (!d) return FA_OK;
+    if (fa_status s = check_dec(d)) return s;
+    if (d->graph) fa_graph_destroy(ctx, d->graph);
+    free_all(ctx, d);
+    d->magic = 0;
+    delete d;
+    return FA_OK;
+}
+
+fa_status fa_decoder_set_layer(fa_decoder *d, uint32_t layer, const fa_buffer *attn_norm, const fa_buffer *ffn_norm,
+                               const fa_qweight *wqkv, const fa_qweight *wo, const fa_qweight *wgu,
+                               const fa_qweight *wdown) {
+    if (fa_status s = check_dec(d)) return s;
+    const fa_decoder_config &c = d->cfg;
+    if (layer >= c.n_layers) return fail(FA_ERR_INVALID_ARGUMENT, "decoder_set_layer: layer out of range");
+    const uint64_t D = c.d_model, EQ = (uint64_t)c.n_heads * c.head_dim, EKV = (uint64_t)c.n_kv_heads * c.head_dim;
+    if (fa_status s = check_vec(d, attn_norm, D, "decoder_set_layer: attn_norm")) return s;
+    if (fa_status s = check_vec(d, ffn_norm, D, "decoder_set_layer: ffn_norm")) return s;
+    if (fa_status s = check_weight(d, wqkv, D, EQ + 2 * EKV, "decoder_set_layer: wqkv")) return s;
+    if (fa_status s = check_weight(d, wo, EQ, D, "decoder_set_layer: wo")) return s;
+    if (fa_status s = check_weight(d, wgu, D, 2ull * c.d_ffn, "decoder_set_layer: wgu")) return s;
+    if (fa_status s = check_weight(d, wdown, c.d_ffn, D, "decoder_set_layer: wdown")) return s;
+    fa_decoder::Layer &L = d->layers[layer];
+    L.attn_norm = attn_norm;
+    L.ffn_norm = ffn_norm;
+    L.wqkv = wqkv;
+    L.wo = wo;
+    L.wgu = wgu;
+    L.wdown = wdown;
+    if (d->graph) {
+        fa_graph_destroy(d->ctx, d->graph);
+        d->graph = nullptr;
+    }
+    return FA_OK;
+}
+
+fa_status fa_decoder_set_head(fa_decoder *d, const fa_buffer *embed, const fa_buffer *final_norm,
+                              const fa_qweight *lm_head) {
+    if (fa_status s = check_dec(d)) return s;
+    const fa_decoder_config &c = d->cfg;
+    if (fa_status s = check_vec(d, embed, (uint64_t)c.vocab * c.d_model, "decoder_set_head: embed")) return s;
+    if (fa_status s = check_vec(d, final_norm, c.d_model, "decoder_set_head: final_norm")) return s;
+    if (fa_status s = check_weight(d, lm_head, c.d_model, c.vocab, "decoder_set_head: lm_head")) return s;
+    d->embed = embed;
+    d->final_norm = final_norm;
+    d->lm_head = lm_head;
+    if (d->graph) {
+        fa_graph_destroy(d->ctx, d->graph);
+        d->graph = nullptr;
+    }
+    return FA_OK;
+}
+
+fa_status fa_decoder_kv_pools(fa_decoder *d, uint32_t layer, fa_buffer **k_pool, fa_buffer **v_pool) {
+    if (fa_status s = check_dec(d)) return s;
+    if (layer >= d->cfg.n_layers) return fail(FA_ERR_INVALID_ARGUMENT, "decoder_kv_pools: layer out of range");
+    if (k_pool) *k_pool = d->layers[layer].k_pool;
+    if (v_pool) *v_pool = d->layers[layer].v_pool;
+    return FA_OK;
+}
+
+fa_status fa_decoder_set_sequences(fa_context *ctx, fa_decoder *d, uint32_t batch, const uint32_t *block_tables,
+                                   const uint32_t *seq_lens) {
+    if (fa_status s = check_ctx(ctx)) return s;
+    if (fa_status s = check_dec(d)) return s;
+    const fa_decoder_config &c = d->cfg;
+    if (batch == 0 || batch > c.max_batch) return fail(FA_ERR_INVALID_ARGUMENT, "decoder_set_sequences: batch out of range");
+    if (!block_tables || !seq_lens) return fail(FA_ERR_INVALID_ARGUMENT, "decoder_set_sequences: null table");
+    // the next step writes position seq_len and then attends to seq_len + 1 tokens
+    for (uint32_t b = 0; b < batch; ++b) {
+        uint64_t need = ((uint64_t)seq_lens[b] + 1 + c.block_size - 1) / c.block_size;
+        if (need > c.max_blocks_per_seq)
+            return fail(FA_ERR_INVALID_ARGUMENT, "paged_kv: row " + std::to_string(b) + " has no room for one more token");
+        for (uint64_t i = 0; i < need; ++i)
+            if (block_tables[(uint64_t)b * c.max_blocks_per_seq + i] >= c.num_blocks)
+                return fail(FA_ERR_INVALID_ARGUMENT, "paged_kv: row " + std::to_string(b) + " entry " +
+                                                         std::to_string(i) + " is not a valid block id");
+    }
+    if (fa_status s = fa_upload_into(ctx, block_tables, (uint64_t)batch * c.max_blocks_per_seq, d->tables, 0)) return s;
+    if (fa_status s = fa_upload_into(ctx, seq_lens, batch, d->seq_lens, 0)) return s;
+    d->batch = batch;
+    return FA_OK;
+}
+
+fa_status fa_decoder_set_tokens(fa_context *ctx, fa_decoder *d, const int32_t *tokens) {
+    if (fa_status s = check_ctx(ctx)) return s;
+    if (fa_status s = check_dec(d)) return s;
+    if (d->batch == 0) return fail(FA_ERR_INVALID_ARGUMENT, "decoder_set_tokens: set the sequences first");
+    if (!tokens) return fail(FA_ERR_INVALID_ARGUMENT, "decoder_set_tokens: null tokens");
+    for (uint32_t b = 0; b < d->batch; ++b)
+        if (tokens[b] < 0 || (uint32_t)tokens[b] >= d->cfg.vocab)
+            return fail(FA_ERR_INVALID_ARGUMENT, "decoder_set_tokens: token id outside the vocabulary");
+    return fa_upload_into(ctx, tokens, d->batch, d->tokens, 0);
+}
+
+fa_status fa_decoder_step(fa_context *ctx, fa_decoder *d, int32_t use_graph) {
+    if (fa_status s = check_ctx(ctx)) return s;
+    if (fa_status s = check_dec(d)) return s;
+    if (d->ctx != ctx) return fail(FA_ERR_DEVICE_MISMATCH, "decoder_step: decoder belongs to another context");
+    if (d->batch == 0) return fail(FA_ERR_INVALID_ARGUMENT, "decoder_step: no sequences installed");
+    if (!d->embed || !d->final_norm || !d->lm_head) return fail(FA_ERR_INVALID_ARGUMENT, "decoder_step: head weights missing");
+    for (auto &l : d->layers)
+        if (!l.wqkv) return fail(FA_ERR_INVALID_ARGUMENT, "decoder_step: layer weights missing");
+    // attention workspace sized before anything is captured
+    k::PagedShape ps{};
+    ps.batch = d->batch;
+    ps.num_heads = d->cfg.n_heads;
+    ps.num_kv_heads = d->cfg.n_kv_heads;
+    ps.max_blocks_per_seq = d->cfg.max_blocks_per_seq;
+    if (fa_status s = ensure_workspace(ctx, k::paged_decode_workspace_bytes(ps, (uint32_t)g_decode_ppc))) return s;
+    if (!use_graph) return enqueue_step(ctx, d);
+    if (d->graph && (d->graph_batch != d->batch || d->graph_ppc != g_decode_ppc)) {
+        fa_graph_destroy(ctx, d->graph);
+        d->graph = nullptr;
+    }
+    if (!d->graph) {
+        if (fa_status s = fa_graph_capture_begin(ctx)) return s;
+        fa_status es = enqueue_step(ctx, d);
+        fa_graph *g = nullptr;
+        fa_status cs = fa_graph_capture_end(ctx, &g);
+        if (es != FA_OK) {
+            if (g) fa_graph_destroy(ctx, g);
+            return es;
+        }
+        if (cs != FA_OK) return cs;
+        d->graph = g;
+        d->graph_batch = d->batch;
+        d->graph_ppc = g_decode_ppc;
+    }
+    return fa_graph_launch(ctx, d->graph);
+}
+
+fa_status fa_decoder_read_tokens(fa_context *ctx, fa_decoder *d, int32_t *tokens) {
+    if (fa_status s = check_dec(d)) return s;
+    return fa_download(ctx, d->tokens, 0, tokens, d->batch);
+}
+fa_status fa_decoder_read_logits(fa_context *ctx, fa_decoder *d, float *logits) {
+    if (fa_status s = check_dec(d)) return s;
+    return fa_download(ctx, d->logits, 0, logits, (uint64_t)d->batch * d->cfg.vocab);
+}
+fa_status fa_decoder_read_seq_lens(fa_context *ctx, fa_decoder *d, uint32_t *seq_lens) {
+    if (fa_status s = check_dec(d)) return s;
+    return fa_download(ctx, d->seq_lens, 0, seq_lens, d->batch);
+}
+
+}  // extern "C"

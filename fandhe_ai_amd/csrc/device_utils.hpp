@@ -1,0 +1,98 @@
+// Device-side helpers shared by the gfx950 kernels (wave64 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace fa {
+namespace dev {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+typedef unsigned int v2u __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+
+// round-to-nearest-even, NaN stays a quiet NaN
+__device__ __forceinline__ uint16_t f32_to_bf16(float v) {
+    uint32_t u = __float_as_uint(v);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+__device__ __forceinline__ float bf16_to_f32(uint16_t v) { return __uint_as_float((uint32_t)v << 16); }
+__device__ __forceinline__ float bf16_lo(uint32_t pair) { return __uint_as_float(pair << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t pair) { return __uint_as_float(pair & 0xffff0000u); }
+
+template <typename T>
+__device__ __forceinline__ T wave_sum(T v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+    return v;
+}
+
+// Block-wide reductions for blocks of NWAVES wavefronts; `smem` needs NWAVES slots.
+template <typename T, int NWAVES>
+__device__ __forceinline__ T block_sum(T v, T *smem) {
+    v = wave_sum(v);
+    int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    __syncthreads();
+    if (lane == 0) smem[wave] = v;
+    __syncthreads();
+    T r = smem[0];
+#pragma unroll
+    for (int i = 1; i < NWAVES; ++i) r += smem[i];
+    return r;
+}
+template <int NWAVES>
+__device__ __forceinline__ float block_max(float v, float *smem) {
+    v = wave_max(v);
+    int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    __syncthreads();
+    if (lane == 0) smem[wave] = v;
+    __syncthreads();
+    float r = smem[0];
+#pragma unroll
+    for (int i = 1; i < NWAVES; ++i) r = fmaxf(r, smem[i]);
+    return r;
+}
+
+// symmetric int8 code of x for a given scale: rne(x / scale) clamped to +-127
+__device__ __forceinline__ int quant_i8(float x, float scale) {
+    if (scale == 0.0f) return 0;
+    float r = rintf(__fdiv_rn(x, scale));
+    r = fminf(fmaxf(r, -127.0f), 127.0f);
+    return (int)r;
+}
+
+// OCP e4m3fn encode, round-to-nearest-even, saturating at +-448
+__device__ __forceinline__ uint32_t f32_to_e4m3(float v) {
+    uint32_t u = __float_as_uint(v);
+    uint32_t sign = (u >> 24) & 0x80u;
+    uint32_t a = u & 0x7fffffffu;
+    if (a > 0x7f800000u) return 0x7fu;                    // NaN
+    if (a >= 0x43e80000u) return sign | 0x7eu;            // >= 464: saturate to 448
+    if (a < 0x3c800000u) {                                // < 2^-6: subnormal, spacing 2^-9
+        float q = rintf(__uint_as_float(a) * 512.0f);     // 0..8 (8 carries into the first normal)
+        return sign | (uint32_t)q;
+    }
+    // normal: keep 3 mantissa bits, RNE on the dropped 20
+    uint32_t r = a + 0x7ffffu + ((a >> 20) & 1u);
+    uint32_t e = (r >> 23) - 120u;                        // rebias 127 -> 7
+    uint32_t m = (r >> 20) & 7u;
+    return sign | (e << 3) | m;
+}
+
+}  // namespace dev
+}  // namespace fa

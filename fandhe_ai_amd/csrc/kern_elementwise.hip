@@ -1,0 +1,181 @@
+// Small bandwidth-bound operators around the linears: SwiGLU, residual add,
+// greedy argmax, embedding gather, dtype conversion, RoPE.
+#include "device_utils.hpp"
+#include "kernels.hpp"
+
+namespace fa {
+namespace k {
+using namespace fa::dev;
+
+namespace {
+
+// crates/tensor-core/src/scalar_op.rs:666-673 (sigmoid_stable) and :355 (Silu)
+__device__ __forceinline__ float silu(float x) {
+    float s;
+    if (x >= 0.0f) {
+        s = __fdiv_rn(1.0f, 1.0f + expf(-x));
+    } else {
+        float e = expf(x);
+        s = __fdiv_rn(e, 1.0f + e);
+    }
+    return x * s;
+}
+
+__global__ void silu_mul_kernel(const float *__restrict__ gate, const float *__restrict__ up,
+                                float *__restrict__ out, uint64_t n) {
+    uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) out[i] = silu(gate[i]) * up[i];
+}
+
+__global__ void swiglu_rows_kernel(const float *__restrict__ gu, float *__restrict__ out, uint64_t rows,
+                                   uint64_t f) {
+    uint64_t total = rows * f;
+    uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    for (; i < total; i += stride) {
+        uint64_t r = i / f, c = i - r * f;
+        const float *row = gu + r * 2 * f;
+        out[i] = silu(row[c]) * row[f + c];
+    }
+}
+
+__global__ void add_kernel(const float *__restrict__ a, const float *__restrict__ b, float *__restrict__ out,
+                           uint64_t n) {
+    uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) out[i] = a[i] + b[i];
+}
+
+// First index of the maximum, NaN ignored, all-NaN row -> 0
+// (crates/autodiff/src/generate/mod.rs:333-343, crates/backend-rocm/src/ops.rs:991-995).
+__global__ void __launch_bounds__(256) argmax_rows_kernel(const float *__restrict__ x, int32_t *__restrict__ out,
+                                                          uint64_t cols) {
+    const float *row = x + (uint64_t)blockIdx.x * cols;
+    float best = -INFINITY;
+    uint32_t best_i = 0xffffffffu;      // "nothing seen yet"
+    for (uint64_t i = threadIdx.x; i < cols; i += blockDim.x) {
+        float v = row[i];
+        if (v != v) continue;
+        if (best_i == 0xffffffffu || v > best) {
+            best = v;
+            best_i = (uint32_t)i;
+        }
+    }
+    __shared__ float s_val[256];
+    __shared__ uint32_t s_idx[256];
+    s_val[threadIdx.x] = best;
+    s_idx[threadIdx.x] = best_i;
+    __syncthreads();
+    for (int off = 128; off > 0; off >>= 1) {
+        if ((int)threadIdx.x < off) {
+            float ov = s_val[threadIdx.x + off];
+            uint32_t oi = s_idx[threadIdx.x + off];
+            float mv = s_val[threadIdx.x];
+            uint32_t mi = s_idx[threadIdx.x];
+            bool take = oi != 0xffffffffu && (mi == 0xffffffffu || ov > mv || (ov == mv && oi < mi));
+            if (take) {
+                s_val[threadIdx.x] = ov;
+                s_idx[threadIdx.x] = oi;
+            }
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) out[blockIdx.x] = s_idx[0] == 0xffffffffu ? 0 : (int32_t)s_idx[0];
+}
+
+__global__ void gather_rows_kernel(const float *__restrict__ table, uint64_t table_rows, uint64_t cols,
+                                   const int32_t *__restrict__ idx, float *__restrict__ out) {
+    uint64_t r = blockIdx.x;
+    int32_t id = idx[r];
+    bool ok = id >= 0 && (uint64_t)id < table_rows;
+    const float *src = table + (uint64_t)(ok ? id : 0) * cols;
+    float *dst = out + r * cols;
+    for (uint64_t c = threadIdx.x; c < cols; c += blockDim.x) dst[c] = ok ? src[c] : __uint_as_float(0x7fc00000u);
+}
+
+__global__ void f32_to_bf16_kernel(const float *__restrict__ in, uint16_t *__restrict__ out, uint64_t n) {
+    uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) out[i] = f32_to_bf16(in[i]);
+}
+__global__ void bf16_to_f32_kernel(const uint16_t *__restrict__ in, float *__restrict__ out, uint64_t n) {
+    uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) out[i] = bf16_to_f32(in[i]);
+}
+__global__ void fill_u32_kernel(uint32_t *p, uint32_t v, uint64_t n) {
+    uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) p[i] = v;
+}
+
+// Rotate-half RoPE: pair (i, i + Dh/2), angle = pos * theta^(-2i/Dh) in f64,
+// cos / sin rounded to f32, four f32 products and one add / sub, no contraction.
+__global__ void rope_kernel(const float *__restrict__ x, const int32_t *__restrict__ pos, float *__restrict__ out,
+                            uint32_t heads, uint32_t head_dim, double theta) {
+    uint32_t half = head_dim / 2;
+    uint64_t r = blockIdx.x;
+    double p = (double)pos[r];
+    for (uint32_t i = threadIdx.x; i < half; i += blockDim.x) {
+        double inv_freq = pow(theta, -2.0 * (double)i / (double)head_dim);
+        double ang = p * inv_freq;
+        float c = (float)cos(ang), s = (float)sin(ang);
+        for (uint32_t h = 0; h < heads; ++h) {
+            uint64_t base = (r * heads + h) * head_dim;
+            float xi = x[base + i], xj = x[base + i + half];
+            out[base + i] = __fsub_rn(__fmul_rn(xi, c), __fmul_rn(xj, s));
+            out[base + i + half] = __fadd_rn(__fmul_rn(xj, c), __fmul_rn(xi, s));
+        }
+    }
+}
+
+inline unsigned grid_for(uint64_t n, unsigned block, unsigned cap = 65535u * 4u) {
+    uint64_t g = (n + block - 1) / block;
+    if (g < 1) g = 1;
+    return (unsigned)(g > cap ? cap : g);
+}
+
+}  // namespace
+
+void silu_mul_f32(const float *gate, const float *up, float *out, uint64_t n, hipStream_t s) {
+    if (n == 0) return;
+    silu_mul_kernel<<<grid_for(n, 256), 256, 0, s>>>(gate, up, out, n);
+}
+void swiglu_rows_f32(const float *gu, float *out, uint64_t rows, uint64_t f, hipStream_t s) {
+    if (rows * f == 0) return;
+    swiglu_rows_kernel<<<grid_for(rows * f, 256), 256, 0, s>>>(gu, out, rows, f);
+}
+void add_f32(const float *a, const float *b, float *out, uint64_t n, hipStream_t s) {
+    if (n == 0) return;
+    add_kernel<<<grid_for(n, 256), 256, 0, s>>>(a, b, out, n);
+}
+void argmax_rows_f32(const float *x, int32_t *out, uint64_t rows, uint64_t cols, hipStream_t s) {
+    if (rows == 0) return;
+    argmax_rows_kernel<<<(unsigned)rows, 256, 0, s>>>(x, out, cols);
+}
+void gather_rows_f32(const float *table, uint64_t table_rows, uint64_t cols, const int32_t *idx, float *out,
+                     uint64_t rows, hipStream_t s) {
+    if (rows == 0 || cols == 0) return;
+    gather_rows_kernel<<<(unsigned)rows, 256, 0, s>>>(table, table_rows, cols, idx, out);
+}
+void convert_f32_to_bf16(const float *in, uint16_t *out, uint64_t n, hipStream_t s) {
+    if (n == 0) return;
+    f32_to_bf16_kernel<<<grid_for(n, 256), 256, 0, s>>>(in, out, n);
+}
+void convert_bf16_to_f32(const uint16_t *in, float *out, uint64_t n, hipStream_t s) {
+    if (n == 0) return;
+    bf16_to_f32_kernel<<<grid_for(n, 256), 256, 0, s>>>(in, out, n);
+}
+void fill_u32(uint32_t *p, uint32_t v, uint64_t n, hipStream_t s) {
+    if (n == 0) return;
+    fill_u32_kernel<<<grid_for(n, 256), 256, 0, s>>>(p, v, n);
+}
+void rope_f32(const float *x, const int32_t *pos, float *out, uint64_t rows, uint64_t heads, uint64_t head_dim,
+              double theta, hipStream_t s) {
+    if (rows == 0 || heads == 0 || head_dim < 2) return;
+    rope_kernel<<<(unsigned)rows, 64, 0, s>>>(x, pos, out, (uint32_t)heads, (uint32_t)head_dim, theta);
+}
+
+}  // namespace k
+}  // namespace fa

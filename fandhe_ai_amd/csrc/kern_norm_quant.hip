@@ -1,0 +1,225 @@
+// RMSNorm (reference contract), dynamic per-token int8 quantization, their
+// fusion, and per-tensor e4m3 quantization.
+#include "device_utils.hpp"
+#include "kernels.hpp"
+
+namespace fa {
+namespace k {
+using namespace fa::dev;
+
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kWaves = kBlock / kWave;
+
+// crates/backend-cpu/src/rmsnorm.rs:203-228: f64 sum of squares through fma,
+// rstd = (f32)(1 / sqrt(fma(acc, (f64)inv_n, (f64)eps))), out = (x * rstd) * w.
+// The row sum is split over the block's threads; only its order differs.
+__device__ __forceinline__ float row_rstd(const float *__restrict__ row, uint64_t hidden, float inv_n, float eps,
+                                          double *smem) {
+    double acc = 0.0;
+    for (uint64_t i = threadIdx.x; i < hidden; i += kBlock) {
+        double v = (double)row[i];
+        acc = fma(v, v, acc);
+    }
+    acc = block_sum<double, kWaves>(acc, smem);
+    return (float)(1.0 / sqrt(fma(acc, (double)inv_n, (double)eps)));
+}
+
+__global__ void __launch_bounds__(kBlock) rmsnorm_kernel(const float *__restrict__ x, const float *__restrict__ w,
+                                                         float *__restrict__ out, uint64_t hidden, float inv_n,
+                                                         float eps) {
+    __shared__ double smem[kWaves];
+    const float *row = x + (uint64_t)blockIdx.x * hidden;
+    float *orow = out + (uint64_t)blockIdx.x * hidden;
+    float rstd = row_rstd(row, hidden, inv_n, eps, smem);
+    if (w) {
+        for (uint64_t i = threadIdx.x; i < hidden; i += kBlock) orow[i] = __fmul_rn(__fmul_rn(row[i], rstd), w[i]);
+    } else {
+        for (uint64_t i = threadIdx.x; i < hidden; i += kBlock) orow[i] = __fmul_rn(row[i], rstd);
+    }
+}
+
+// byte offset of activation element (r, kk) in the 16-row x 64-k tile order
+__device__ __forceinline__ uint64_t tiled_chunk_offset(uint64_t r, uint64_t chunk, uint64_t k_tiles) {
+    // chunk = kk / 16: kt = chunk / 4, g = chunk % 4
+    uint64_t mt = r / 16, rr = r % 16, kt = chunk / 4, g = chunk % 4;
+    return (mt * k_tiles + kt) * 1024 + (g * 16 + rr) * 16;
+}
+
+template <bool IN_BF16>
+__device__ __forceinline__ float load_in(const void *x, uint64_t i) {
+    if (IN_BF16) return bf16_to_f32(((const uint16_t *)x)[i]);
+    return ((const float *)x)[i];
+}
+
+// One block per (padded) row.  Pass 1: absmax.  Pass 2: codes, 16 per thread
+// step so that the tiled output is written with 16-byte stores.
+template <bool IN_BF16>
+__global__ void __launch_bounds__(kBlock)
+    quantize_rows_kernel(const void *__restrict__ x, int8_t *__restrict__ xq_row, int8_t *__restrict__ xq_tiled,
+                         float *__restrict__ sx, uint64_t m, uint64_t k, uint64_t k_pad) {
+    __shared__ float smem[kWaves];
+    uint64_t r = blockIdx.x;
+    uint64_t k_tiles = k_pad / 64;
+    if (r >= m) {                                     // padding row of the tiled layout
+        if (xq_tiled)
+            for (uint64_t c = threadIdx.x; c < k_pad / 16; c += kBlock)
+                *(v4i *)(xq_tiled + tiled_chunk_offset(r, c, k_tiles)) = v4i{0, 0, 0, 0};
+        return;
+    }
+    uint64_t base = r * k;
+    float amax = 0.0f;
+    for (uint64_t i = threadIdx.x; i < k; i += kBlock) amax = fmaxf(amax, fabsf(load_in<IN_BF16>(x, base + i)));
+    amax = block_max<kWaves>(amax, smem);
+    float scale = __fdiv_rn(amax, 127.0f);
+    if (threadIdx.x == 0) sx[r] = scale;
+    for (uint64_t c = threadIdx.x; c < k_pad / 16; c += kBlock) {
+        uint32_t words[4];
+#pragma unroll
+        for (int wd = 0; wd < 4; ++wd) {
+            uint32_t word = 0;
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                uint64_t kk = c * 16 + wd * 4 + b;
+                int q = kk < k ? quant_i8(load_in<IN_BF16>(x, base + kk), scale) : 0;
+                word |= ((uint32_t)q & 0xffu) << (8 * b);
+            }
+            words[wd] = word;
+        }
+        if (xq_tiled)
+            *(v4u *)(xq_tiled + tiled_chunk_offset(r, c, k_tiles)) = v4u{words[0], words[1], words[2], words[3]};
+        if (xq_row) {
+#pragma unroll
+            for (int wd = 0; wd < 4; ++wd)
+#pragma unroll
+                for (int b = 0; b < 4; ++b) {
+                    uint64_t kk = c * 16 + wd * 4 + b;
+                    if (kk < k) xq_row[base + kk] = (int8_t)((words[wd] >> (8 * b)) & 0xffu);
+                }
+        }
+    }
+}
+
+// RMSNorm of an f32 row followed by its per-token quantization; the
+// normalized value is recomputed (same operations, same bits) in each pass.
+__global__ void __launch_bounds__(kBlock)
+    rmsnorm_quantize_kernel(const float *__restrict__ x, const float *__restrict__ w, float eps, float inv_n,
+                            float *__restrict__ out_f32, int8_t *__restrict__ xq_tiled, float *__restrict__ sx,
+                            uint64_t m, uint64_t hidden) {
+    __shared__ double smem_d[kWaves];
+    __shared__ float smem_f[kWaves];
+    uint64_t r = blockIdx.x;
+    uint64_t k_tiles = hidden / 64;
+    if (r >= m) {
+        for (uint64_t c = threadIdx.x; c < hidden / 16; c += kBlock)
+            *(v4i *)(xq_tiled + tiled_chunk_offset(r, c, k_tiles)) = v4i{0, 0, 0, 0};
+        return;
+    }
+    const float *row = x + r * hidden;
+    float rstd = row_rstd(row, hidden, inv_n, eps, smem_d);
+    float amax = 0.0f;
+    for (uint64_t i = threadIdx.x; i < hidden; i += kBlock) {
+        float y = __fmul_rn(__fmul_rn(row[i], rstd), w[i]);
+        if (out_f32) out_f32[r * hidden + i] = y;
+        amax = fmaxf(amax, fabsf(y));
+    }
+    amax = block_max<kWaves>(amax, smem_f);
+    float scale = __fdiv_rn(amax, 127.0f);
+    if (threadIdx.x == 0) sx[r] = scale;
+    for (uint64_t c = threadIdx.x; c < hidden / 16; c += kBlock) {
+        uint32_t words[4];
+#pragma unroll
+        for (int wd = 0; wd < 4; ++wd) {
+            uint32_t word = 0;
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                uint64_t kk = c * 16 + wd * 4 + b;
+                float y = __fmul_rn(__fmul_rn(row[kk], rstd), w[kk]);
+                word |= ((uint32_t)quant_i8(y, scale) & 0xffu) << (8 * b);
+            }
+            words[wd] = word;
+        }
+        *(v4u *)(xq_tiled + tiled_chunk_offset(r, c, k_tiles)) = v4u{words[0], words[1], words[2], words[3]};
+    }
+}
+
+// absmax over a tensor: block maxima merged with an integer max on the bit
+// pattern (valid for non-negative floats).  `absmax` must be zero on entry.
+__global__ void __launch_bounds__(kBlock) absmax_kernel(const float *__restrict__ x, uint64_t n,
+                                                        float *__restrict__ absmax) {
+    __shared__ float smem[kWaves];
+    float a = 0.0f;
+    uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    uint64_t stride = (uint64_t)gridDim.x * kBlock;
+    for (; i < n; i += stride) a = fmaxf(a, fabsf(x[i]));
+    a = block_max<kWaves>(a, smem);
+    if (threadIdx.x == 0) atomicMax((unsigned int *)absmax, __float_as_uint(a));
+}
+
+__global__ void scale_from_absmax_kernel(const float *__restrict__ absmax, float divisor, float *__restrict__ scale) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) *scale = __fdiv_rn(*absmax, divisor);
+}
+
+__global__ void __launch_bounds__(kBlock) quantize_e4m3_kernel(const float *__restrict__ x, uint8_t *__restrict__ q,
+                                                               const float *__restrict__ scale_p, uint64_t n) {
+    float scale = *scale_p;
+    uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    uint64_t stride = (uint64_t)gridDim.x * kBlock;
+    for (; i < n; i += stride) q[i] = scale == 0.0f ? 0 : (uint8_t)f32_to_e4m3(__fdiv_rn(x[i], scale));
+}
+
+__global__ void zero_f32_kernel(float *p) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) *p = 0.0f;
+}
+
+}  // namespace
+
+void rmsnorm_f32(const float *x, const float *w, float *out, uint64_t rows, uint64_t hidden, float eps,
+                 hipStream_t s) {
+    if (rows == 0 || hidden == 0) return;
+    float inv_n = 1.0f / (float)hidden;
+    rmsnorm_kernel<<<(unsigned)rows, kBlock, 0, s>>>(x, w, out, hidden, inv_n, eps);
+}
+
+void quantize_rows_i8(const void *x, bool in_bf16, int8_t *xq_rowmajor, int8_t *xq_tiled, float *sx, uint64_t m,
+                      uint64_t m_pad, uint64_t k, uint64_t k_pad, hipStream_t s) {
+    uint64_t rows = xq_tiled ? m_pad : m;
+    if (rows == 0 || k_pad == 0) return;
+    if (in_bf16)
+        quantize_rows_kernel<true><<<(unsigned)rows, kBlock, 0, s>>>(x, xq_rowmajor, xq_tiled, sx, m, k, k_pad);
+    else
+        quantize_rows_kernel<false><<<(unsigned)rows, kBlock, 0, s>>>(x, xq_rowmajor, xq_tiled, sx, m, k, k_pad);
+}
+
+void rmsnorm_quantize_i8(const float *x, const float *w, float eps, float *out_f32, int8_t *xq_tiled, float *sx,
+                         uint64_t m, uint64_t m_pad, uint64_t hidden, hipStream_t s) {
+    if (m_pad == 0 || hidden == 0) return;
+    float inv_n = 1.0f / (float)hidden;
+    rmsnorm_quantize_kernel<<<(unsigned)m_pad, kBlock, 0, s>>>(x, w, eps, inv_n, out_f32, xq_tiled, sx, m, hidden);
+}
+
+void tensor_absmax_f32(const float *x, uint64_t n, float *absmax, hipStream_t s) {
+    zero_f32_kernel<<<1, 64, 0, s>>>(absmax);
+    if (n == 0) return;
+    uint64_t g = (n + kBlock - 1) / kBlock;
+    if (g > 2048) g = 2048;
+    absmax_kernel<<<(unsigned)g, kBlock, 0, s>>>(x, n, absmax);
+}
+
+void scale_from_absmax(const float *absmax, float divisor, float *scale, hipStream_t s) {
+    scale_from_absmax_kernel<<<1, 64, 0, s>>>(absmax, divisor, scale);
+}
+
+void quantize_tensor_e4m3(const float *x, uint8_t *q, float *scale, float *absmax_scratch, uint64_t n,
+                          hipStream_t s) {
+    tensor_absmax_f32(x, n, absmax_scratch, s);
+    scale_from_absmax(absmax_scratch, 448.0f, scale, s);
+    if (n == 0) return;
+    uint64_t g = (n + kBlock - 1) / kBlock;
+    if (g > 4096) g = 4096;
+    quantize_e4m3_kernel<<<(unsigned)g, kBlock, 0, s>>>(x, q, scale, n);
+}
+
+}  // namespace k
+}  // namespace fa

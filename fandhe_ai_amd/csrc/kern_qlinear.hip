@@ -1,0 +1,307 @@
+// Decode-shape ("skinny", m <= 32 tokens) quantized linears.  Both kernels are
+// HBM-bound streams over the tile-ordered int8 weight: every wavefront load
+// is one contiguous 1 KiB tile that lands directly in the operand layout of
+// the matrix instruction, so the weight never passes through LDS.  The block
+// splits K over its wavefronts and reduces their partial tiles in LDS in a
+// fixed order (deterministic).
+#include "device_utils.hpp"
+#include "kernels.hpp"
+
+namespace fa {
+namespace k {
+using namespace fa::dev;
+
+int g_skinny_ntw = 0;      // tuning overrides (0 = heuristic)
+int g_skinny_waves = 0;
+
+namespace {
+
+struct EpiI8 {
+    const float *sx, *sw, *bias, *residual;
+    int32_t *acc_out;
+    void *out;
+    int out_bf16;
+};
+
+// ------------------------------------------------------------------ W8A8
+// acc[m, n] = sum_k xq[m, k] * w[k, n] on v_mfma_i32_16x16x64_i8.
+// D layout: lane l holds column l % 16, rows 4 * (l / 16) + j, j = 0..3.
+template <int MT, int NTW, int NWAVES>
+__global__ void __launch_bounds__(NWAVES * 64)
+    w8a8_skinny_kernel(const int8_t *__restrict__ xq_tiled, const int8_t *__restrict__ w_tiles, uint32_t m,
+                       uint32_t n, uint32_t n_tiles, uint32_t k_tiles, EpiI8 ep) {
+    constexpr int NACC = MT * NTW * 4;
+    __shared__ int red[NWAVES][NACC][64];
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+    const uint32_t nt0 = blockIdx.x * NTW;
+
+    v4i acc[MT][NTW];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < NTW; ++j) acc[i][j] = v4i{0, 0, 0, 0};
+
+    const int8_t *a_base = xq_tiled + (uint64_t)lane * 16;
+    const int8_t *b_base = w_tiles + (uint64_t)lane * 16;
+    // U k-tiles per trip: all their loads are issued before the first multiply
+    constexpr int U = (MT * NTW >= 4) ? 2 : 4;
+    const uint32_t cnt = k_tiles > (uint32_t)wave ? (k_tiles - wave + NWAVES - 1) / NWAVES : 0;
+    auto load_b = [&](uint32_t kt, v4i *b) {
+#pragma unroll
+        for (int j = 0; j < NTW; ++j) {
+            uint32_t nt = nt0 + j;
+            b[j] = nt < n_tiles ? *(const v4i *)(b_base + ((uint64_t)nt * k_tiles + kt) * 1024) : v4i{0, 0, 0, 0};
+        }
+    };
+    auto load_a = [&](uint32_t kt, v4i *a) {
+#pragma unroll
+        for (int i = 0; i < MT; ++i) a[i] = *(const v4i *)(a_base + ((uint64_t)i * k_tiles + kt) * 1024);
+    };
+    auto mma = [&](const v4i *a, const v4i *b) {
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int j = 0; j < NTW; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[i], b[j], acc[i][j], 0, 0, 0);
+    };
+    uint32_t it = 0;
+    for (; it + U <= cnt; it += U) {
+        v4i a[U][MT], b[U][NTW];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            uint32_t kt = wave + (it + u) * NWAVES;
+            load_b(kt, b[u]);
+            load_a(kt, a[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) mma(a[u], b[u]);
+    }
+    for (; it < cnt; ++it) {
+        v4i a[MT], b[NTW];
+        uint32_t kt = wave + it * NWAVES;
+        load_b(kt, b);
+        load_a(kt, a);
+        mma(a, b);
+    }
+
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < NTW; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) red[wave][(i * NTW + j) * 4 + e][lane] = acc[i][j][e];
+    __syncthreads();
+
+    for (int idx = wave; idx < NACC; idx += NWAVES) {
+        int sum = 0;
+#pragma unroll
+        for (int w = 0; w < NWAVES; ++w) sum += red[w][idx][lane];
+        int e = idx % 4, j = (idx / 4) % NTW, i = idx / (4 * NTW);
+        uint32_t row = i * 16 + 4 * (lane / 16) + e;
+        uint32_t col = (nt0 + j) * 16 + lane % 16;
+        if (row < m && col < n) {
+            uint64_t o = (uint64_t)row * n + col;
+            if (ep.acc_out) ep.acc_out[o] = sum;
+            float s = __fmul_rn(ep.sx[row], ep.sw[col]);
+            float v = __fmul_rn((float)sum, s);
+            if (ep.bias) v = __fadd_rn(v, ep.bias[col]);
+            if (ep.residual) v = __fadd_rn(ep.residual[o], v);
+            if (ep.out_bf16)
+                ((uint16_t *)ep.out)[o] = f32_to_bf16(v);
+            else
+                ((float *)ep.out)[o] = v;
+        }
+    }
+}
+
+// ----------------------------------------------------------------- W8A16
+// Two exact int8 -> bf16 conversions packed into one dword (low half first).
+__device__ __forceinline__ uint32_t pack_i8x2_bf16(int lo, int hi) {
+    uint32_t fl = __float_as_uint((float)lo), fh = __float_as_uint((float)hi);
+    // upper halves of both floats in one v_perm_b32; |v| <= 128 fits bf16 exactly, so truncation is exact
+    return __builtin_amdgcn_perm(fh, fl, 0x07060302u);
+}
+__device__ __forceinline__ void cvt_i8x8_bf16(uint32_t w0, uint32_t w1, v8bf *out) {
+    v4u r;
+    r[0] = pack_i8x2_bf16((int)(int8_t)(w0), (int)(int8_t)(w0 >> 8));
+    r[1] = pack_i8x2_bf16((int)(int8_t)(w0 >> 16), (int)(int8_t)(w0 >> 24));
+    r[2] = pack_i8x2_bf16((int)(int8_t)(w1), (int)(int8_t)(w1 >> 8));
+    r[3] = pack_i8x2_bf16((int)(int8_t)(w1 >> 16), (int)(int8_t)(w1 >> 24));
+    *out = __builtin_bit_cast(v8bf, r);
+}
+
+// out[m, n] = (sum_k a[m, k] * (float)w[k, n]) * sw[n] on v_mfma_f32_16x16x32_bf16.
+// A lane's 16 weight bytes are k = 64*kt + 16*g + 0..15; the first eight feed
+// one instruction, the last eight the next, and the activation operand uses the
+// same split, so the two instructions together cover the tile's 64 k-values.
+template <int MT, int NTW, int NWAVES>
+__global__ void __launch_bounds__(NWAVES * 64)
+    w8a16_skinny_kernel(const uint16_t *__restrict__ a, const int8_t *__restrict__ w_tiles,
+                        const float *__restrict__ sw, uint32_t m, uint32_t n, uint32_t n_tiles, uint32_t k_tiles,
+                        void *__restrict__ out, int out_bf16) {
+    constexpr int NACC = MT * NTW * 4;
+    __shared__ float red[NWAVES][NACC][64];
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+    const int g = lane / 16, r = lane % 16;
+    const uint32_t nt0 = blockIdx.x * NTW;
+    const uint64_t k = (uint64_t)k_tiles * 64;
+
+    v4f acc[MT][NTW];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < NTW; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    const int8_t *b_base = w_tiles + (uint64_t)lane * 16;
+    constexpr int U = (MT * NTW >= 4) ? 2 : 4;
+    const uint32_t cnt = k_tiles > (uint32_t)wave ? (k_tiles - wave + NWAVES - 1) / NWAVES : 0;
+    auto load_b = [&](uint32_t kt, v4u *braw) {
+#pragma unroll
+        for (int j = 0; j < NTW; ++j) {
+            uint32_t nt = nt0 + j;
+            braw[j] = nt < n_tiles ? *(const v4u *)(b_base + ((uint64_t)nt * k_tiles + kt) * 1024) : v4u{0, 0, 0, 0};
+        }
+    };
+    auto load_a = [&](uint32_t kt, v4u *lo, v4u *hi) {
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            uint32_t row = i * 16 + r;
+            lo[i] = v4u{0, 0, 0, 0};
+            hi[i] = v4u{0, 0, 0, 0};
+            if (row < m) {
+                const v4u *p = (const v4u *)(a + (uint64_t)row * k + (uint64_t)kt * 64 + g * 16);
+                lo[i] = p[0];
+                hi[i] = p[1];
+            }
+        }
+    };
+    auto mma = [&](const v4u *lo, const v4u *hi, const v4u *braw) {
+#pragma unroll
+        for (int j = 0; j < NTW; ++j) {
+            v8bf blo, bhi;
+            cvt_i8x8_bf16(braw[j][0], braw[j][1], &blo);
+            cvt_i8x8_bf16(braw[j][2], braw[j][3], &bhi);
+#pragma unroll
+            for (int i = 0; i < MT; ++i) {
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, lo[i]), blo, acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, hi[i]), bhi, acc[i][j], 0, 0, 0);
+            }
+        }
+    };
+    uint32_t it = 0;
+    for (; it + U <= cnt; it += U) {
+        v4u braw[U][NTW], lo[U][MT], hi[U][MT];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            uint32_t kt = wave + (it + u) * NWAVES;
+            load_b(kt, braw[u]);
+            load_a(kt, lo[u], hi[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) mma(lo[u], hi[u], braw[u]);
+    }
+    for (; it < cnt; ++it) {
+        v4u braw[NTW], lo[MT], hi[MT];
+        uint32_t kt = wave + it * NWAVES;
+        load_b(kt, braw);
+        load_a(kt, lo, hi);
+        mma(lo, hi, braw);
+    }
+
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < NTW; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) red[wave][(i * NTW + j) * 4 + e][lane] = acc[i][j][e];
+    __syncthreads();
+
+    for (int idx = wave; idx < NACC; idx += NWAVES) {
+        float sum = red[0][idx][lane];
+#pragma unroll
+        for (int w = 1; w < NWAVES; ++w) sum = __fadd_rn(sum, red[w][idx][lane]);
+        int e = idx % 4, j = (idx / 4) % NTW, i = idx / (4 * NTW);
+        uint32_t row = i * 16 + 4 * g + e;
+        uint32_t col = (nt0 + j) * 16 + r;
+        if (row < m && col < n) {
+            float v = __fmul_rn(sum, sw[col]);
+            uint64_t o = (uint64_t)row * n + col;
+            if (out_bf16)
+                ((uint16_t *)out)[o] = f32_to_bf16(v);
+            else
+                ((float *)out)[o] = v;
+        }
+    }
+}
+
+// Picks n-tiles per block and wavefronts per block so that the whole grid is
+// resident at once with about 8-16 wavefronts per compute unit.
+inline void pick_config(uint64_t n_tiles, uint64_t k_tiles, int num_cus, int *ntw, int *waves) {
+    int w = 8, t = 1;
+    if (k_tiles < 32) w = 4;
+    // blocks = n_tiles / t; resident waves per CU = blocks * w / num_cus
+    while (t < 2 && (n_tiles / (uint64_t)t) * (uint64_t)w > (uint64_t)num_cus * 16) t *= 2;
+    if ((n_tiles / (uint64_t)t) * (uint64_t)w > (uint64_t)num_cus * 16 && w == 8) w = 4;
+    if (g_skinny_ntw) t = g_skinny_ntw;
+    if (g_skinny_waves) w = g_skinny_waves;
+    *ntw = t;
+    *waves = w;
+}
+
+template <int MT>
+void launch_w8a8(const int8_t *xq, const int8_t *wt, uint32_t m, uint32_t n, uint32_t n_tiles, uint32_t k_tiles,
+                 const EpiI8 &ep, int ntw, int waves, hipStream_t s) {
+    unsigned grid = (n_tiles + ntw - 1) / ntw;
+    if (ntw == 1 && waves == 8)
+        w8a8_skinny_kernel<MT, 1, 8><<<grid, 512, 0, s>>>(xq, wt, m, n, n_tiles, k_tiles, ep);
+    else if (ntw == 1)
+        w8a8_skinny_kernel<MT, 1, 4><<<grid, 256, 0, s>>>(xq, wt, m, n, n_tiles, k_tiles, ep);
+    else if (waves == 8)
+        w8a8_skinny_kernel<MT, 2, 8><<<grid, 512, 0, s>>>(xq, wt, m, n, n_tiles, k_tiles, ep);
+    else
+        w8a8_skinny_kernel<MT, 2, 4><<<grid, 256, 0, s>>>(xq, wt, m, n, n_tiles, k_tiles, ep);
+}
+
+template <int MT>
+void launch_w8a16(const uint16_t *a, const int8_t *wt, const float *sw, uint32_t m, uint32_t n, uint32_t n_tiles,
+                  uint32_t k_tiles, void *out, int out_bf16, int ntw, int waves, hipStream_t s) {
+    unsigned grid = (n_tiles + ntw - 1) / ntw;
+    if (ntw == 1 && waves == 8)
+        w8a16_skinny_kernel<MT, 1, 8><<<grid, 512, 0, s>>>(a, wt, sw, m, n, n_tiles, k_tiles, out, out_bf16);
+    else if (ntw == 1)
+        w8a16_skinny_kernel<MT, 1, 4><<<grid, 256, 0, s>>>(a, wt, sw, m, n, n_tiles, k_tiles, out, out_bf16);
+    else if (waves == 8)
+        w8a16_skinny_kernel<MT, 2, 8><<<grid, 512, 0, s>>>(a, wt, sw, m, n, n_tiles, k_tiles, out, out_bf16);
+    else
+        w8a16_skinny_kernel<MT, 2, 4><<<grid, 256, 0, s>>>(a, wt, sw, m, n, n_tiles, k_tiles, out, out_bf16);
+}
+
+}  // namespace
+
+void linear_w8a8_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t m, uint64_t n, uint64_t n_pad,
+                        uint64_t k_pad, const EpilogueI8 &ep, int num_cus, hipStream_t s) {
+    if (m == 0 || n == 0) return;
+    uint32_t n_tiles = (uint32_t)(n_pad / 16), k_tiles = (uint32_t)(k_pad / 64);
+    int ntw, waves;
+    pick_config(n_tiles, k_tiles, num_cus, &ntw, &waves);
+    EpiI8 e{ep.sx, ep.sw, ep.bias, ep.residual, ep.acc_out, ep.out, ep.out_bf16};
+    if (m <= 16)
+        launch_w8a8<1>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e, ntw, waves, s);
+    else
+        launch_w8a8<2>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e, ntw, waves, s);
+}
+
+void linear_w8a16_skinny(const uint16_t *a, const int8_t *w_tiles, const float *sw, uint64_t m, uint64_t n,
+                         uint64_t n_pad, uint64_t k_pad, void *out, int out_bf16, int num_cus, hipStream_t s) {
+    if (m == 0 || n == 0) return;
+    uint32_t n_tiles = (uint32_t)(n_pad / 16), k_tiles = (uint32_t)(k_pad / 64);
+    int ntw, waves;
+    pick_config(n_tiles, k_tiles, num_cus, &ntw, &waves);
+    if (m <= 16)
+        launch_w8a16<1>(a, w_tiles, sw, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, out, out_bf16, ntw, waves, s);
+    else
+        launch_w8a16<2>(a, w_tiles, sw, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, out, out_bf16, ntw, waves, s);
+}
+
+}  // namespace k
+}  // namespace fa

@@ -1,0 +1,144 @@
+// Launchers of the gfx950 kernels.  Each enqueues on `stream` and returns;
+// shapes have been validated by the caller (capi_*.cpp) against what the
+// kernel and its grid assume.  Sizes are element counts unless named _bytes.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace fa {
+namespace k {
+
+// ---- weight tile order ---------------------------------------------------
+// int8 weights W[k, n] are stored as tiles of 16 columns x 64 k-values, one
+// tile = 1 KiB laid out in the order one wavefront loads it for the int8
+// matrix instruction: byte ((g*16 + c)*16 + j) of tile (nt, kt) holds
+// W[64*kt + 16*g + j][16*nt + c]   (g = 0..3, c = 0..15, j = 0..15),
+// tiles ordered [nt][kt].  e4m3 weights use tiles of 16 columns x 128
+// k-values (2 KiB): byte ((g*16 + c)*32 + j) holds W[128*kt + 32*g + j][16*nt + c].
+constexpr int kTileN = 16;
+constexpr int kTileK8 = 64;     // int8 k-values per tile
+constexpr int kTileKF8 = 128;   // e4m3 k-values per tile
+
+// ---- elementwise / small ops (kern_elementwise.hip) ------------------------
+void silu_mul_f32(const float *gate, const float *up, float *out, uint64_t n, hipStream_t s);
+// SwiGLU on a [rows, 2*f] gate|up matrix -> [rows, f]
+void swiglu_rows_f32(const float *gu, float *out, uint64_t rows, uint64_t f, hipStream_t s);
+void add_f32(const float *a, const float *b, float *out, uint64_t n, hipStream_t s);
+void argmax_rows_f32(const float *x, int32_t *out, uint64_t rows, uint64_t cols, hipStream_t s);
+void gather_rows_f32(const float *table, uint64_t table_rows, uint64_t cols, const int32_t *idx,
+                     float *out, uint64_t rows, hipStream_t s);
+void convert_f32_to_bf16(const float *in, uint16_t *out, uint64_t n, hipStream_t s);
+void convert_bf16_to_f32(const uint16_t *in, float *out, uint64_t n, hipStream_t s);
+void rope_f32(const float *x, const int32_t *pos, float *out, uint64_t rows, uint64_t heads,
+              uint64_t head_dim, double theta, hipStream_t s);
+void fill_u32(uint32_t *p, uint32_t v, uint64_t n, hipStream_t s);
+
+// ---- norms / quantizers (kern_norm_quant.hip) -------------------------------
+void rmsnorm_f32(const float *x, const float *w, float *out, uint64_t rows, uint64_t hidden,
+                 float eps, hipStream_t s);
+// Per-token int8 quantization.  in_bf16 selects the input type.  xq_rowmajor
+// (nullable) receives [m, k]; xq_tiled (nullable) receives the activation
+// tile order used by the skinny GEMM: tiles [mt][kt] of 16 rows x 64 k in
+// the same byte order as weight tiles, rows >= m zero-filled (m_pad rows).
+void quantize_rows_i8(const void *x, bool in_bf16, int8_t *xq_rowmajor, int8_t *xq_tiled, float *sx,
+                      uint64_t m, uint64_t m_pad, uint64_t k, uint64_t k_pad, hipStream_t s);
+// RMSNorm fused with the quantizer (f32 in): out_f32 nullable.
+void rmsnorm_quantize_i8(const float *x, const float *w, float eps, float *out_f32, int8_t *xq_tiled,
+                         float *sx, uint64_t m, uint64_t m_pad, uint64_t hidden, hipStream_t s);
+// Per-tensor absmax -> scale = absmax / 448 (one f32) then e4m3 codes.
+void quantize_tensor_e4m3(const float *x, uint8_t *q, float *scale, float *absmax_scratch, uint64_t n,
+                          hipStream_t s);
+
+// ---- weights (kern_qweight.hip) ----------------------------------------------
+// Column absmax / 127 of w[k, n] (f32, row-major) -> scales[n_pad] (padding 0)
+void weight_col_scales_i8(const float *w, uint64_t k, uint64_t n, uint64_t n_pad, float *scales,
+                          hipStream_t s);
+void weight_quantize_pack_i8(const float *w, const float *scales, uint64_t k, uint64_t n,
+                             uint64_t k_pad, uint64_t n_pad, int8_t *tiles, hipStream_t s);
+// Pack row-major codes [k, n] (1 byte each) into tile order; tile_k = 64 or 128.
+void weight_pack_codes(const uint8_t *codes, uint64_t k, uint64_t n, uint64_t k_pad, uint64_t n_pad,
+                       int tile_k, uint8_t *tiles, hipStream_t s);
+void weight_unpack_codes(const uint8_t *tiles, uint64_t k, uint64_t n, uint64_t k_pad, uint64_t n_pad,
+                         int tile_k, uint8_t *codes, hipStream_t s);
+void weight_quantize_pack_e4m3(const float *w, const float *scale, uint64_t k, uint64_t n,
+                               uint64_t k_pad, uint64_t n_pad, uint8_t *tiles, hipStream_t s);
+void tensor_absmax_f32(const float *x, uint64_t n, float *absmax, hipStream_t s);
+void scale_from_absmax(const float *absmax, float divisor, float *scale, hipStream_t s);
+
+// ---- f32 GEMM with the reference's summation order (kern_gemm_f32.hip) -------
+void gemm_f32(const float *a, const float *b, const float *bias, float *out, uint64_t m, uint64_t n,
+              uint64_t k, int relu, hipStream_t s);
+
+// ---- skinny (decode-shape) quantized linears (kern_qlinear.hip) ---------------
+struct EpilogueI8 {
+    const float *sx;      // [m] activation scales
+    const float *sw;      // [n_pad] weight scales
+    const float *bias;    // nullable [n]
+    const float *residual;  // nullable [m, n] f32, added last (may alias out when out is f32)
+    int32_t *acc_out;     // nullable [m, n]
+    void *out;            // [m, n] f32 or bf16
+    int out_bf16;
+};
+// xq_tiled: activation tiles (see quantize_rows_i8); m <= 32.
+void linear_w8a8_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t m, uint64_t n,
+                        uint64_t n_pad, uint64_t k_pad, const EpilogueI8 &ep, int num_cus,
+                        hipStream_t s);
+// a: bf16 [m, k] row-major (k == k_pad required), m <= 32.
+void linear_w8a16_skinny(const uint16_t *a, const int8_t *w_tiles, const float *sw, uint64_t m,
+                         uint64_t n, uint64_t n_pad, uint64_t k_pad, void *out, int out_bf16,
+                         int num_cus, hipStream_t s);
+
+// ---- prefill-shape MFMA GEMMs (kern_gemm_mfma.hip) -----------------------------
+// aq: int8 [m, k_pad] row-major.
+void gemm_w8a8_mfma(const int8_t *aq, const int8_t *w_tiles, uint64_t m, uint64_t n, uint64_t n_pad,
+                    uint64_t k_pad, const EpilogueI8 &ep, hipStream_t s);
+// aq: e4m3 [m, k_pad] row-major; scales are device scalars.
+void gemm_e4m3_mfma(const uint8_t *aq, const uint8_t *w_tiles, const float *a_scale,
+                    const float *w_scale, uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad,
+                    void *out, int out_bf16, hipStream_t s);
+
+// ---- paged KV (kern_paged.hip) ---------------------------------------------------
+struct PagedShape {
+    uint32_t num_blocks, block_size, e_kv, batch, l_new, num_heads, num_kv_heads, head_dim,
+        max_blocks_per_seq;
+    float scale;
+};
+// Row scatter; elem_bytes 2 or 4; slots bounds-checked against pool_rows.
+void paged_kv_append(const void *k_new, const void *v_new, void *k_pool, void *v_pool,
+                     const uint32_t *slots, uint64_t rows, uint64_t e, uint64_t pool_rows,
+                     int elem_bytes, hipStream_t s);
+// Generic attention with the reference's per-row summation order; is_bf16
+// selects the storage type; workspace holds query_rows * s_stride f32.
+void paged_attention_generic(const void *q, const void *k_pool, const void *v_pool,
+                             const uint32_t *tables, const uint32_t *seq_lens, const PagedShape &ps,
+                             int is_bf16, float *workspace, uint64_t s_stride, void *out,
+                             hipStream_t s);
+// Decode fast path: bf16, head_dim 128, block_size 16, l_new 1, group <= 16.
+// Workspace bytes needed for a given shape:
+uint64_t paged_decode_workspace_bytes(const PagedShape &ps, uint32_t pages_per_chunk);
+void paged_attention_decode_bf16(const uint16_t *q, const uint16_t *k_pool, const uint16_t *v_pool,
+                                 const uint32_t *tables, const uint32_t *seq_lens,
+                                 const PagedShape &ps, uint32_t pages_per_chunk, void *workspace,
+                                 void *out, int out_bf16, hipStream_t s);
+
+// ---- decode-step glue (kern_decoder.hip) --------------------------------------
+// Per step, before the layers: pos[b] = seq_lens[b]; slot[b] from the block
+// table (UINT32_MAX when the table cannot hold the position); seq_lens[b] += 1;
+// cos/sin table [batch, head_dim/2] for the positions.
+void decode_prepare(const uint32_t *tables, uint32_t *seq_lens, int32_t *pos, uint32_t *slots, float *cos_sin,
+                    uint32_t batch, uint32_t block_size, uint32_t max_blocks_per_seq, uint32_t num_blocks,
+                    uint32_t head_dim, double theta, hipStream_t s);
+// Splits qkv[b, (H + 2 Hkv) Dh] (f32): RoPE on q and k with the cos/sin table,
+// one rounding to bf16; q -> q_out[b, H Dh]; k, v -> pool rows slot[b].
+void qkv_rope_append(const float *qkv, const float *cos_sin, const uint32_t *slots, uint16_t *q_out,
+                     uint16_t *k_pool, uint16_t *v_pool, uint32_t batch, uint32_t heads, uint32_t kv_heads,
+                     uint32_t head_dim, uint64_t pool_rows, hipStream_t s);
+// act = silu(gate) * up on gu[m, 2f] followed by per-token int8 quantization
+// into activation tiles (f must be a multiple of 64).
+void swiglu_quantize_i8(const float *gu, int8_t *xq_tiled, float *sx, uint64_t m, uint64_t m_pad, uint64_t f,
+                        hipStream_t s);
+
+}  // namespace k
+}  // namespace fa

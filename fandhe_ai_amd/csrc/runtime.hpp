@@ -1,0 +1,131 @@
+// Internal runtime of the MI355X backend: context, stream, size-class pool,
+// buffer handles, error reporting.  Everything above this header is the C ABI
+// (include/fandhe_rocm.h); everything below is HIP.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <mutex>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "../../include/fandhe_rocm.h"
+
+namespace fa {
+
+// ------------------------------------------------------------------ errors
+void set_error(const std::string &msg);
+fa_status fail(fa_status s, const std::string &msg);
+
+// ------------------------------------------------------------- size classes
+// Size-class table of the reference pool (crates/tensor-core/src/pool_core.rs:102-209).
+struct PoolConfig {
+    uint64_t max_pool_bytes = 128ull << 20;
+    uint64_t small_max_bytes = 1ull << 20;
+    uint64_t large_granule_bytes = 2ull << 20;
+    uint64_t huge_min_bytes = 64ull << 20;
+    size_t huge_entries_per_class = 1;
+};
+bool size_class_for(uint64_t bytes, const PoolConfig &cfg, uint64_t *out);
+
+// Free list of device blocks keyed by class size, insertion-ordered so that
+// eviction is global LRU (pool_core.rs:211-590).  The pool never calls HIP
+// itself: evicted blocks are handed back to the caller, which frees them
+// after the lock is released.
+class SizeClassPool {
+  public:
+    explicit SizeClassPool(PoolConfig cfg = PoolConfig()) : cfg_(cfg) {}
+    const PoolConfig &config() const { return cfg_; }
+    void *take(uint64_t class_bytes);
+    void record_allocation(uint64_t logical, uint64_t cls);
+    void record_reuse(uint64_t logical, uint64_t cls);
+    void record_loan_end(uint64_t logical, uint64_t cls);
+    std::vector<std::pair<uint64_t, void *>> put(uint64_t class_bytes, void *ptr);
+    bool take_one_for_release(std::pair<uint64_t, void *> *out);
+    void record_release(uint64_t class_bytes);
+    fa_pool_stats stats();
+
+  private:
+    PoolConfig cfg_;
+    std::mutex mu_;
+    std::vector<std::pair<uint64_t, void *>> free_;
+    uint64_t alloc_count_ = 0, reuse_count_ = 0, cached_bytes_ = 0, waste_ = 0, released_ = 0;
+};
+
+size_t dtype_size(fa_dtype t);
+
+}  // namespace fa
+
+struct fa_context {
+    uint32_t magic;
+    int device;
+    hipStream_t stream;
+    fa::SizeClassPool pool;
+    bool poisoned;
+    bool capturing;
+    hipDeviceProp_t props;
+    // device staging for per-call host tables (slot mappings, block tables)
+    void *table_stage;
+    uint64_t table_stage_bytes;
+    // scratch for split-KV attention partials and similar kernel workspaces
+    void *workspace;
+    uint64_t workspace_bytes;
+};
+
+struct fa_buffer {
+    uint32_t magic;
+    fa_context *ctx;
+    void *ptr;
+    uint64_t numel;
+    fa_dtype dtype;
+    uint64_t logical_bytes;
+    uint64_t class_bytes;
+};
+
+struct fa_qweight {
+    uint32_t magic;
+    fa_context *ctx;
+    fa_qweight_kind kind;
+    uint64_t k, n;          // logical shape [k, n]
+    uint64_t k_pad, n_pad;  // padded to the tile grid
+    fa_buffer *codes;       // tile-ordered codes, k_pad * n_pad bytes
+    fa_buffer *scales;      // f32: n_pad (int8) or 1 (e4m3)
+};
+
+struct fa_graph {
+    uint32_t magic;
+    hipGraph_t graph;
+    hipGraphExec_t exec;
+};
+
+struct fa_timer {
+    hipEvent_t start, stop;
+};
+
+namespace fa {
+
+constexpr uint32_t kCtxMagic = 0xFA0C7C01u;
+constexpr uint32_t kBufMagic = 0xFA0B0F01u;
+constexpr uint32_t kQwMagic = 0xFA0A0E01u;
+constexpr uint32_t kGraphMagic = 0xFA06A901u;
+
+// Common entry checks; each returns FA_OK or records the error.
+fa_status check_ctx(const fa_context *ctx);
+fa_status check_buf(const fa_context *ctx, const fa_buffer *b, const char *what);
+fa_status check_buf_typed(const fa_context *ctx, const fa_buffer *b, fa_dtype t, uint64_t min_numel,
+                          const char *what);
+fa_status hip_fail(fa_context *ctx, hipError_t e, const char *what, fa_status as);
+// Checks hipGetLastError after a launch.
+fa_status after_launch(fa_context *ctx, const char *kernel);
+
+// Pool-backed raw allocation used by buffers and by internal scratch.
+fa_status pool_alloc(fa_context *ctx, uint64_t bytes, void **ptr, uint64_t *class_bytes);
+void pool_free(fa_context *ctx, void *ptr, uint64_t logical, uint64_t class_bytes);
+fa_status make_buffer(fa_context *ctx, fa_dtype dtype, uint64_t numel, bool zero, fa_buffer **out);
+// Ensures ctx->workspace holds at least `bytes` (grows outside capture only).
+fa_status ensure_workspace(fa_context *ctx, uint64_t bytes);
+fa_status ensure_table_stage(fa_context *ctx, uint64_t bytes);
+
+}  // namespace fa

@@ -1,0 +1,348 @@
+/*
+ * fandhe_rocm.h - C ABI of the MI355X (gfx950) quantized decode backend.
+ *
+ * Plain C, plain pointers and sizes.  Every entry point returns an fa_status;
+ * none of them aborts or throws.  The entry points are what a `BackendOps` /
+ * `MemoryOps` implementation for `Device::Rocm(0)` binds; each declaration
+ * cites the reference interface it stands behind (paths are relative to the
+ * reference repository root).
+ *
+ * Execution model (the contract of the reference's asynchronous backend,
+ * docs/backend-cuda-async-execution-design.md:71-118): one in-order HIP stream
+ * per context; submit calls do not block the host; the host-blocking points
+ * are fa_download, fa_synchronize_device and calls documented as returning
+ * host data.  Argument violations are reported before anything is written.
+ * A HIP failure after validation poisons the context: every later call
+ * returns FA_ERR_CONTEXT_POISONED until the context is destroyed.
+ */
+#ifndef FANDHE_ROCM_H
+#define FANDHE_ROCM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------ status */
+/* Mirrors BackendError (crates/tensor-core/src/device.rs:225-371). */
+typedef int32_t fa_status;
+enum {
+    FA_OK = 0,
+    FA_ERR_INVALID_ARGUMENT = 1,       /* BackendError::InvalidArgument */
+    FA_ERR_SHAPE_MISMATCH = 2,         /* BackendError::ShapeMismatch */
+    FA_ERR_DEVICE_MISMATCH = 3,        /* BackendError::DeviceMismatch (foreign handle) */
+    FA_ERR_ALLOCATION_FAILED = 4,      /* BackendError::DeviceAllocationFailed */
+    FA_ERR_KERNEL_LAUNCH_FAILED = 5,   /* BackendError::KernelLaunchFailed */
+    FA_ERR_DEVICE_UNAVAILABLE = 6,     /* BackendError::DeviceUnavailable */
+    FA_ERR_TRANSFER_FAILED = 7,        /* BackendError::TransferFailed */
+    FA_ERR_UNSUPPORTED = 8,            /* BackendError::Unsupported */
+    FA_ERR_CONTEXT_POISONED = 9,       /* BackendError::DeviceContextPoisoned */
+    FA_ERR_CAPTURE_IN_PROGRESS = 10    /* BackendError::DeviceContextCaptureInProgress */
+};
+/* Message of the last failure on the calling thread ("" if none). */
+const char *fa_last_error_message(void);
+const char *fa_status_name(fa_status s);
+/* ABI version of this header; bumped on any incompatible change. */
+uint32_t fa_abi_version(void);
+
+/* ----------------------------------------------------------------- context */
+/* DeviceProvider::{is_available, enumerate, select} for backend "rocm"
+ * (crates/tensor-core/src/device.rs:149-168,
+ *  crates/backend-rocm/src/device.rs:30-114).  Only gfx950 devices count. */
+typedef struct fa_context fa_context;
+fa_status fa_device_count(int32_t *count);
+fa_status fa_context_create(int32_t ordinal, fa_context **out);
+fa_status fa_context_destroy(fa_context *ctx);
+typedef struct {
+    int32_t ordinal;
+    int32_t compute_units;
+    int32_t clock_khz;
+    int32_t wavefront_size;
+    uint64_t total_memory_bytes;
+    char arch[32];
+    char name[128];
+} fa_device_info;
+fa_status fa_context_info(const fa_context *ctx, fa_device_info *out);
+
+/* ------------------------------------------------------------------ memory */
+/* MemoryOps + DeviceBuffer (crates/tensor-core/src/buffer.rs:91-373,389-521).
+ * The reference's buffers are f32 only; the element type is explicit here so
+ * that bf16 / int8 / fp8 storage sits behind the same opaque handle. */
+typedef enum {
+    FA_F32 = 0, FA_BF16 = 1, FA_I8 = 2, FA_E4M3 = 3, FA_I32 = 4, FA_U32 = 5
+} fa_dtype;
+typedef struct fa_buffer fa_buffer;
+
+/* MemoryOps::alloc_zeroed (buffer.rs:395).  numel == 0 touches no device. */
+fa_status fa_alloc_zeroed(fa_context *ctx, fa_dtype dtype, uint64_t numel, fa_buffer **out);
+/* Same pool, contents unspecified (operator outputs are fully overwritten,
+ * crates/tensor-core/src/backend_ops.rs:4343-4347). */
+fa_status fa_alloc_uninit(fa_context *ctx, fa_dtype dtype, uint64_t numel, fa_buffer **out);
+/* MemoryOps::upload (buffer.rs:404): host data is consumed on return. */
+fa_status fa_upload(fa_context *ctx, fa_dtype dtype, const void *host, uint64_t numel, fa_buffer **out);
+/* MemoryOps::upload_into (buffer.rs:446-459): dst_offset in elements. */
+fa_status fa_upload_into(fa_context *ctx, const void *host, uint64_t numel, fa_buffer *dst,
+                         uint64_t dst_offset);
+/* MemoryOps::download (buffer.rs:417): host data is final on return (the
+ * synchronization point).  src_offset / numel in elements. */
+fa_status fa_download(fa_context *ctx, const fa_buffer *src, uint64_t src_offset, void *host,
+                      uint64_t numel);
+/* Drop of the handle (buffer.rs:40-48): returns the block to the pool. */
+fa_status fa_buffer_free(fa_context *ctx, fa_buffer *buf);
+uint64_t fa_buffer_numel(const fa_buffer *buf);
+fa_dtype fa_buffer_dtype(const fa_buffer *buf);
+void *fa_buffer_device_ptr(const fa_buffer *buf);
+
+/* BackendOps::synchronize_device (backend_ops.rs:4897). */
+fa_status fa_synchronize_device(fa_context *ctx);
+/* The HIP stream (hipStream_t) every call of this context is ordered on. */
+void *fa_context_stream(fa_context *ctx);
+
+/* PoolStats (crates/tensor-core/src/pool_core.rs:122-139). */
+typedef struct {
+    uint64_t alloc_count, reuse_count, cached_bytes, pending_return_bytes,
+        capacity_waste_bytes, released_bytes;
+} fa_pool_stats;
+/* BackendOps::device_memory_pool_stats (backend_ops.rs:5050). */
+fa_status fa_device_memory_pool_stats(fa_context *ctx, fa_pool_stats *out);
+/* BackendOps::release_cached_device_memory (backend_ops.rs:5038). */
+fa_status fa_release_cached_device_memory(fa_context *ctx);
+/* size_class_for with the default configuration (pool_core.rs:157-209). */
+fa_status fa_size_class_for(uint64_t bytes, uint64_t *class_bytes);
+
+/* ------------------------------------------------------------ f32 linear */
+typedef enum { FA_ACT_NONE = 0, FA_ACT_RELU = 1 } fa_activation;
+/* BackendOps::gemm_device (backend_ops.rs:1998): out[m,n] = a[m,k] @ b[k,n],
+ * f32, one accumulator per output, k ascending, fused multiply-add. */
+fa_status fa_gemm_device(fa_context *ctx, const fa_buffer *a, const fa_buffer *b, uint64_t m,
+                         uint64_t n, uint64_t k, fa_buffer *out);
+/* BackendOps::linear_forward_device (backend_ops.rs:4296-4308):
+ * out = act(a @ w + bias); w / bias are views (buffer + element offset,
+ * DeviceBufferView, buffer.rs:277-373) with w stored [k, n]. bias may be NULL. */
+fa_status fa_linear_forward_device(fa_context *ctx, const fa_buffer *a, uint64_t m, uint64_t k,
+                                   const fa_buffer *w, uint64_t w_offset, uint64_t n,
+                                   const fa_buffer *bias, uint64_t bias_offset,
+                                   fa_activation act, fa_buffer *out);
+
+/* -------------------------------------------------------- quantized linear */
+/* Not in the reference (design record only,
+ * docs/backend-int8-quantization-decision.md:13,84); the contract is:
+ * symmetric int8, scale = absmax / 127, q = clamp(rne(x / scale), -127, 127),
+ * int32 accumulation, out = f32(acc) * (sx[m] * sw[n]) (+ bias[n]).
+ * A quantized weight is an opaque object: int8 (or e4m3) codes in an
+ * MFMA-friendly tile order plus f32 scales. */
+typedef struct fa_qweight fa_qweight;
+typedef enum { FA_QW_INT8_CHANNEL = 0, FA_QW_E4M3_TENSOR = 1 } fa_qweight_kind;
+/* Quantize an f32 weight view w[k, n] (the layout of linear_forward_device)
+ * on the device.  INT8_CHANNEL: one scale per output column.
+ * E4M3_TENSOR: one scale (absmax / 448). */
+fa_status fa_qweight_from_f32(fa_context *ctx, const fa_buffer *w, uint64_t w_offset, uint64_t k,
+                              uint64_t n, fa_qweight_kind kind, fa_qweight **out);
+/* Import host codes q[k, n] (int8 or e4m3 bytes) with their scales
+ * (n scales for INT8_CHANNEL, 1 for E4M3_TENSOR). */
+fa_status fa_qweight_from_codes(fa_context *ctx, const void *codes, const float *scales,
+                                uint64_t k, uint64_t n, fa_qweight_kind kind, fa_qweight **out);
+/* Read back codes as [k, n] and scales (test / export path; synchronizes). */
+fa_status fa_qweight_export(fa_context *ctx, const fa_qweight *qw, void *codes, float *scales);
+fa_status fa_qweight_free(fa_context *ctx, fa_qweight *qw);
+uint64_t fa_qweight_k(const fa_qweight *qw);
+uint64_t fa_qweight_n(const fa_qweight *qw);
+
+/* Dynamic per-token quantization of x[m, k] (f32 or bf16 buffer): writes
+ * row-major int8 codes xq[m, k] and scales sx[m]. */
+fa_status fa_quantize_rows_i8(fa_context *ctx, const fa_buffer *x, uint64_t m, uint64_t k,
+                              fa_buffer *xq, fa_buffer *sx);
+/* W8A8 linear on a weight of kind INT8_CHANNEL: quantizes x per token,
+ * multiplies on the int8 matrix cores, dequantizes in the epilogue.
+ * out: f32 or bf16 [m, n].  acc_out (nullable): i32 [m, n] raw accumulators.
+ * bias (nullable): f32 view of n elements. */
+fa_status fa_linear_w8a8(fa_context *ctx, const fa_buffer *x, uint64_t m, const fa_qweight *qw,
+                         const fa_buffer *bias, uint64_t bias_offset, fa_buffer *acc_out,
+                         fa_buffer *out);
+/* Decode-shape int8-weight linear with bf16 activations a[m, k]:
+ * out[m, n] = (sum_k a * w_int8) * sw[n], f32 accumulation; out f32 or bf16. */
+fa_status fa_linear_w8a16(fa_context *ctx, const fa_buffer *a, uint64_t m, const fa_qweight *qw,
+                          fa_buffer *out);
+/* Per-tensor e4m3 quantization of x (f32): codes xq (E4M3, same shape) and a
+ * one-element f32 scale buffer (absmax / 448). */
+fa_status fa_quantize_tensor_e4m3(fa_context *ctx, const fa_buffer *x, uint64_t numel,
+                                  fa_buffer *xq, fa_buffer *scale);
+/* fp8 GEMM: out[m, n] = (aq[m, k] @ W) * (a_scale * w_scale), f32
+ * accumulation; qw of kind E4M3_TENSOR; out f32 or bf16. */
+fa_status fa_gemm_e4m3(fa_context *ctx, const fa_buffer *aq, const fa_buffer *a_scale, uint64_t m,
+                       const fa_qweight *qw, fa_buffer *out);
+/* int8 GEMM on pre-quantized row-major activations aq[m, k] with scales
+ * sx[m] (prefill shape); same epilogue as fa_linear_w8a8. */
+fa_status fa_gemm_w8a8(fa_context *ctx, const fa_buffer *aq, const fa_buffer *sx, uint64_t m,
+                       const fa_qweight *qw, fa_buffer *acc_out, fa_buffer *out);
+
+/* ------------------------------------------------------------------ norms */
+/* BackendOps::rmsnorm (backend_ops.rs:5113-5122; CPU contract
+ * crates/backend-cpu/src/rmsnorm.rs:124-228): f64 sum of squares,
+ * rstd = (f32)(1 / sqrt(sum * (f64)(1/hidden as f32) + eps)),
+ * out = (x * rstd) * w.  w may be NULL.  x / out f32 [rows, hidden]. */
+fa_status fa_rmsnorm(fa_context *ctx, const fa_buffer *x, const fa_buffer *w, float eps,
+                     uint64_t rows, uint64_t hidden, fa_buffer *out);
+/* Not in the reference: rotary embedding, rotate-half pairing (i, i + Dh/2),
+ * inv_freq = theta^(-2i/Dh); x / out f32 [rows, heads, head_dim];
+ * positions: i32 buffer [rows]. */
+fa_status fa_rope(fa_context *ctx, const fa_buffer *x, const fa_buffer *positions, uint64_t rows,
+                  uint64_t heads, uint64_t head_dim, double theta, fa_buffer *out);
+
+/* ------------------------------------------------------------ elementwise */
+/* BackendOps::scalar_unary(Silu) then mul (backend_ops.rs:2304,2276;
+ * formula crates/tensor-core/src/scalar_op.rs:355,666-673). */
+fa_status fa_silu_mul(fa_context *ctx, const fa_buffer *gate, const fa_buffer *up, uint64_t numel,
+                      fa_buffer *out);
+/* BackendOps::add (backend_ops.rs:2277). */
+fa_status fa_add(fa_context *ctx, const fa_buffer *a, const fa_buffer *b, uint64_t numel,
+                 fa_buffer *out);
+/* BackendOps::argmax over the last axis (backend_ops.rs:2390): first index
+ * on ties, NaN ignored, all-NaN row -> 0.  out: i32 [rows]. */
+fa_status fa_argmax_rows(fa_context *ctx, const fa_buffer *x, uint64_t rows, uint64_t cols,
+                         fa_buffer *out);
+/* BackendOps::gather of rows (backend_ops.rs:3375): out[r, :] = table[idx[r], :]. */
+fa_status fa_gather_rows(fa_context *ctx, const fa_buffer *table, uint64_t table_rows,
+                         uint64_t cols, const fa_buffer *idx, uint64_t rows, fa_buffer *out);
+/* dtype conversion f32 <-> bf16 (round to nearest even, once). */
+fa_status fa_convert(fa_context *ctx, const fa_buffer *src, uint64_t numel, fa_buffer *dst);
+
+/* --------------------------------------------------------------- paged KV */
+/* PagedKvLayout (crates/tensor-core/src/paged_kv.rs:47-131). */
+typedef struct {
+    uint64_t num_blocks;
+    uint64_t block_size;      /* power of two, 1..256 */
+    uint64_t embed_dim;       /* width of one K / V row */
+} fa_paged_layout;
+/* PagedAttentionArgs (paged_kv.rs:137-214) + num_kv_heads for grouped-query
+ * attention (0 or == num_heads: the reference's MHA; then embed_dim is the
+ * query width too). */
+typedef struct {
+    fa_paged_layout layout;
+    uint64_t batch;
+    uint64_t l_new;
+    uint64_t num_heads;
+    uint64_t max_blocks_per_seq;
+    float scale;
+    uint64_t num_kv_heads;
+} fa_paged_args;
+/* PagedAttentionPlan (paged_kv.rs:201-213). */
+typedef struct {
+    uint64_t out_numel, s_max, query_rows, workspace_elems;
+} fa_paged_plan;
+/* validate_paged_kv_append / validate_paged_attention (paged_kv.rs:222-373);
+ * pure host functions, callable without a device. */
+fa_status fa_validate_paged_kv_append(uint64_t k_new_numel, uint64_t v_new_numel,
+                                      uint64_t k_pool_numel, uint64_t v_pool_numel,
+                                      const uint32_t *slot_mapping, uint64_t rows,
+                                      const fa_paged_layout *layout);
+fa_status fa_validate_paged_attention(uint64_t q_numel, uint64_t k_pool_numel,
+                                      uint64_t v_pool_numel, const uint32_t *block_tables,
+                                      uint64_t n_tables, const uint32_t *seq_lens, uint64_t n_seq,
+                                      const fa_paged_args *args, fa_paged_plan *plan);
+/* BackendOps::paged_kv_append (backend_ops.rs:4694-4709): copies row r of
+ * k_new / v_new [rows, E] to pool row slot_mapping[r].  Buffers f32 or bf16
+ * (all four the same type).  slot_mapping is a host array. */
+fa_status fa_paged_kv_append(fa_context *ctx, const fa_buffer *k_new, const fa_buffer *v_new,
+                             fa_buffer *k_pool, fa_buffer *v_pool, const uint32_t *slot_mapping,
+                             uint64_t rows, const fa_paged_layout *layout);
+/* BackendOps::paged_attention_forward (backend_ops.rs:4742-4757).  q / out
+ * [B, L_new, H * Dh]; pools [num_blocks, block_size, H_kv * Dh]; f32 or bf16
+ * (q, pools, out the same type).  block_tables [B, max_blocks_per_seq] and
+ * seq_lens [B] are host arrays; unused table entries hold UINT32_MAX. */
+fa_status fa_paged_attention_forward(fa_context *ctx, const fa_buffer *q, const fa_buffer *k_pool,
+                                     const fa_buffer *v_pool, const uint32_t *block_tables,
+                                     uint64_t n_tables, const uint32_t *seq_lens, uint64_t n_seq,
+                                     const fa_paged_args *args, fa_buffer *out);
+/* Device-resident tables (U32 buffers) for callers that replay a captured
+ * graph: nothing is read on the host, so table contents cannot be validated
+ * before the launch; the kernels bounds-check every block id and slot and
+ * write NaN / skip the row on a violation.  seq_lens may not exceed
+ * max_blocks_per_seq * block_size. */
+fa_status fa_paged_kv_append_device(fa_context *ctx, const fa_buffer *k_new, const fa_buffer *v_new,
+                                    fa_buffer *k_pool, fa_buffer *v_pool,
+                                    const fa_buffer *slot_mapping, uint64_t rows,
+                                    const fa_paged_layout *layout);
+fa_status fa_paged_attention_forward_device(fa_context *ctx, const fa_buffer *q,
+                                            const fa_buffer *k_pool, const fa_buffer *v_pool,
+                                            const fa_buffer *block_tables, const fa_buffer *seq_lens,
+                                            const fa_paged_args *args, fa_buffer *out);
+
+/* ------------------------------------------------------------------ graphs */
+/* Counterpart of the reference's captured inference chain
+ * (BackendOps::linear_chain_forward_captured, backend_ops.rs:4814;
+ * docs/inference-chain-single-sync-design.md:175-186).  Between begin and end
+ * every call on the context is recorded instead of executed; calls that
+ * synchronize or allocate return FA_ERR_CAPTURE_IN_PROGRESS. */
+typedef struct fa_graph fa_graph;
+fa_status fa_graph_capture_begin(fa_context *ctx);
+fa_status fa_graph_capture_end(fa_context *ctx, fa_graph **out);
+fa_status fa_graph_launch(fa_context *ctx, fa_graph *graph);
+fa_status fa_graph_destroy(fa_context *ctx, fa_graph *graph);
+
+/* ---------------------------------------------------------- decoder step */
+/* Llama-style decoder (pre-norm RMSNorm, GQA attention with RoPE over a
+ * paged bf16 KV cache, SwiGLU FFN), W8A8 int8 linears, one new token per
+ * sequence, greedy argmax.  The reference has no such model; it is the
+ * composition of the operators above that the benchmark names. */
+typedef struct {
+    uint32_t n_layers, d_model, n_heads, n_kv_heads, head_dim, d_ffn, vocab;
+    uint32_t block_size, max_blocks_per_seq, num_blocks;
+    uint32_t max_batch;
+    float rms_eps;
+    double rope_theta;
+} fa_decoder_config;
+typedef struct fa_decoder fa_decoder;
+fa_status fa_decoder_create(fa_context *ctx, const fa_decoder_config *cfg, fa_decoder **out);
+fa_status fa_decoder_destroy(fa_context *ctx, fa_decoder *dec);
+/* Weights: norm vectors and embedding are f32 buffers (copied by reference,
+ * the caller keeps them alive); linears are fa_qweight of kind INT8_CHANNEL
+ * with shapes qkv [d_model, (H + 2 H_kv) Dh], o [H Dh, d_model],
+ * gate_up [d_model, 2 d_ffn] (gate columns first), down [d_ffn, d_model],
+ * lm_head [d_model, vocab]. */
+fa_status fa_decoder_set_layer(fa_decoder *dec, uint32_t layer, const fa_buffer *attn_norm,
+                               const fa_buffer *ffn_norm, const fa_qweight *wqkv,
+                               const fa_qweight *wo, const fa_qweight *wgu, const fa_qweight *wdown);
+fa_status fa_decoder_set_head(fa_decoder *dec, const fa_buffer *embed, const fa_buffer *final_norm,
+                              const fa_qweight *lm_head);
+/* K / V pools of one layer: bf16 [num_blocks, block_size, H_kv * Dh]. */
+fa_status fa_decoder_kv_pools(fa_decoder *dec, uint32_t layer, fa_buffer **k_pool, fa_buffer **v_pool);
+/* Installs block tables [batch, max_blocks_per_seq] and the current
+ * sequence lengths [batch] (host arrays; validated here). */
+fa_status fa_decoder_set_sequences(fa_context *ctx, fa_decoder *dec, uint32_t batch,
+                                   const uint32_t *block_tables, const uint32_t *seq_lens);
+/* Installs the tokens [batch] to feed to the next step (host array). */
+fa_status fa_decoder_set_tokens(fa_context *ctx, fa_decoder *dec, const int32_t *tokens);
+/* One decode step, asynchronous: consumes the resident tokens, appends K/V,
+ * advances the sequence lengths by one and leaves the argmax tokens resident
+ * as the next step's input.  use_graph != 0 replays a captured HIP graph of
+ * the step (captured on first use). */
+fa_status fa_decoder_step(fa_context *ctx, fa_decoder *dec, int32_t use_graph);
+/* Host copies of the current tokens [batch] / logits [batch, vocab] /
+ * sequence lengths [batch] (synchronize). */
+fa_status fa_decoder_read_tokens(fa_context *ctx, fa_decoder *dec, int32_t *tokens);
+fa_status fa_decoder_read_logits(fa_context *ctx, fa_decoder *dec, float *logits);
+fa_status fa_decoder_read_seq_lens(fa_context *ctx, fa_decoder *dec, uint32_t *seq_lens);
+
+/* ------------------------------------------------------ profiling / tuning */
+/* Launch-shape knobs for experiments; value 0 restores the built-in choice.
+ * key 0: n-tiles per block of the decode-shape linears (1 or 2);
+ * key 1: wavefronts per block of the decode-shape linears (4 or 8);
+ * key 2: KV pages per work item of the decode attention (4, 8 or 16). */
+fa_status fa_set_tuning(int32_t key, int32_t value);
+/* A pair of HIP events recorded on the context's stream (the stream the
+ * kernels run on); used by the benchmark to time launches. */
+typedef struct fa_timer fa_timer;
+fa_status fa_timer_create(fa_context *ctx, fa_timer **out);
+fa_status fa_timer_start(fa_context *ctx, fa_timer *t);
+fa_status fa_timer_stop(fa_context *ctx, fa_timer *t);
+/* Blocks until the stop event has completed. */
+fa_status fa_timer_elapsed_ms(fa_context *ctx, fa_timer *t, float *ms);
+fa_status fa_timer_destroy(fa_context *ctx, fa_timer *t);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,111 @@
+"""GPU parity of the full decode step against the oracle's decode step.
+
+The step chains quantizers, whose rounding is discontinuous: a last-bit
+difference in an activation (attention's reduction order, exp) can flip an
+int8 code, which moves a few accumulators by one weight code.  The operators
+are each held to the reference's tolerance in their own tests; for the chained
+step the logits are held to 2e-3 of the row's logit range (stated here), the
+appended K/V rows to one bf16 step, and the greedy tokens must match wherever
+the oracle's top-2 margin exceeds that bound.
+"""
+import numpy as np
+import pytest
+
+import oracle_lib as o
+from decoder_common import GpuDecoder, build_model, oracle_step
+from gpu_common import ops
+
+pytestmark = pytest.mark.gpu
+
+
+def _check_step(m, dec, lens, tokens, use_graph, tag):
+    pools_before = [L["k_pool"].copy() for L in m.layers]
+    want_next, want_logits = oracle_step(m, lens, tokens)
+    dec.step(use_graph)
+    got_logits, got_next = dec.logits(), dec.tokens()
+    spread = want_logits.max(axis=1, keepdims=True) - want_logits.min(axis=1, keepdims=True)
+    err = np.abs(got_logits - want_logits) / spread
+    print("DECODE_STEP_PARITY\t%s\tmax_err/range=%.3e\tmean=%.3e" % (tag, err.max(), err.mean()), flush=True)
+    assert err.max() < 2e-3
+    top2 = np.sort(want_logits, axis=1)[:, -2:]
+    decisive = (top2[:, 1] - top2[:, 0]) > 4e-3 * spread[:, 0]
+    assert np.array_equal(got_next[decisive], want_next[decisive])
+    assert np.array_equal(got_next, o.argmax_rows(got_logits))
+    assert np.array_equal(dec.seq_lens(), lens)
+    for li, L in enumerate(m.layers):
+        gk, gv = dec.kv_pool(li)
+        changed = (L["k_pool"] != pools_before[li]).any(axis=2)
+        assert np.array_equal((gk != pools_before[li]).any(axis=2) | changed, changed)      # nothing else written
+        for name, g, w in (("k", gk, L["k_pool"]), ("v", gv, L["v_pool"])):
+            gf, wf = o.from_bf16(g[changed]), o.from_bf16(w[changed])
+            assert np.all(np.abs(gf - wf) <= np.maximum(np.abs(wf), 1e-2) * 2.0 ** -6), (li, name)
+        # keep the two caches identical from here on, so that later steps compare like with like
+        L["k_pool"][:] = gk
+        L["v_pool"][:] = gv
+    return got_next
+
+
+@pytest.mark.parametrize("shape", [
+    dict(n_layers=2, d_model=256, n_heads=4, n_kv_heads=2, d_ffn=512, vocab=1000, batch=4, ctxs=[1, 15, 16, 200]),
+    dict(n_layers=1, d_model=512, n_heads=8, n_kv_heads=8, d_ffn=256, vocab=333, batch=17, ctxs=list(range(3, 20))),
+    dict(n_layers=2, d_model=1024, n_heads=8, n_kv_heads=1, d_ffn=1536, vocab=4000, batch=32, ctxs=[40 + 9 * i for i in range(32)]),
+])
+def test_decode_steps_match_the_oracle_eager_and_graph(shape):
+    be = ops()
+    m = build_model(seed=11, steps=4, **shape)
+    dec = GpuDecoder(be, m)
+    try:
+        lens, tokens = m.seq_lens.copy(), m.tokens.copy()
+        for step in range(3):
+            tokens = _check_step(m, dec, lens, tokens, use_graph=(step > 0), tag="L%d:B%d:step%d" % (shape["n_layers"], shape["batch"], step))
+            dec.set_state(lens, tokens)            # the oracle continues from the GPU's tokens
+    finally:
+        dec.close()
+
+
+def test_graph_replay_is_bit_identical_to_eager():
+    be = ops()
+    shape = dict(n_layers=2, d_model=256, n_heads=4, n_kv_heads=2, d_ffn=512, vocab=1000, batch=8,
+                 ctxs=[7, 33, 64, 100, 5, 18, 250, 31])
+    runs = []
+    for use_graph in (False, True):
+        m = build_model(seed=5, steps=6, **shape)
+        dec = GpuDecoder(be, m)
+        try:
+            outs = []
+            for _ in range(5):
+                dec.step(use_graph)
+                be.synchronize_device()
+                outs.append((dec.logits().copy(), dec.tokens().copy(), dec.seq_lens().copy()))
+            runs.append(outs)
+        finally:
+            dec.close()
+    for (l0, t0, s0), (l1, t1, s1) in zip(*runs):
+        assert np.array_equal(l0, l1) and np.array_equal(t0, t1) and np.array_equal(s0, s1)
+    assert runs[0][-1][2].tolist() == [c + 5 for c in shape["ctxs"]]
+
+
+def test_decoder_argument_errors():
+    import ctypes as C
+    import fandhe_ai_amd as fa
+    be = ops()
+    lib = fa.capi.lib
+    h = C.c_void_p()
+    bad = fa.capi.DecoderConfig(1, 256, 4, 2, 64, 512, 100, 16, 8, 32, 4, 1e-5, 500000.0)       # head_dim 64
+    assert lib.fa_decoder_create(be._ctx, C.byref(bad), C.byref(h)) == fa.capi.UNSUPPORTED
+    bad = fa.capi.DecoderConfig(1, 256, 4, 2, 128, 512, 100, 16, 8, 32, 64, 1e-5, 500000.0)     # batch 64
+    assert lib.fa_decoder_create(be._ctx, C.byref(bad), C.byref(h)) == fa.capi.UNSUPPORTED
+    m = build_model(seed=1, n_layers=1, d_model=128, n_heads=2, n_kv_heads=1, d_ffn=128, vocab=50, batch=2,
+                    ctxs=[3, 4], steps=1)
+    dec = GpuDecoder(be, m)
+    try:
+        t = np.ascontiguousarray(m.tables)
+        full = np.array([m.cfg["max_blocks_per_seq"] * 16, 3], dtype=np.uint32)       # no room for one more token
+        assert lib.fa_decoder_set_sequences(be._ctx, dec.h, 2, t.ctypes.data_as(fa.capi.u32p),
+                                            full.ctypes.data_as(fa.capi.u32p)) == fa.capi.INVALID_ARGUMENT
+        tok = np.array([0, 50], dtype=np.int32)
+        assert lib.fa_decoder_set_tokens(be._ctx, dec.h, tok.ctypes.data_as(fa.capi.i32p)) == fa.capi.INVALID_ARGUMENT
+        wrong = be.import_quantized_weight(np.ones((64, 16), np.int8), np.ones(16, np.float32))
+        assert lib.fa_decoder_set_head(dec.h, dec.keep[-3]._h, dec.keep[-2]._h, wrong._h) == fa.capi.SHAPE_MISMATCH
+    finally:
+        dec.close()

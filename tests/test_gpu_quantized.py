@@ -1,0 +1,281 @@
+"""GPU parity of the quantized linears against the CPU oracle, through the C ABI.
+
+int8: quantizer codes, scales and int32 accumulators are bit-exact; the
+dequantized f32 output is bit-exact too (same single multiply).  bf16 outputs
+are checked as the one round-to-nearest-even of the kernel's own f32 result,
+whose parity with the oracle is judged with the composite tolerance.  fp8:
+codes bit-exact, products judged against the exactly-summed oracle with the
+bound stated in the test.
+"""
+import numpy as np
+import pytest
+
+import oracle_lib as o
+from gpu_common import assert_bf16_rounding_of, assert_parity, ops
+
+pytestmark = pytest.mark.gpu
+
+
+def _fa():
+    import fandhe_ai_amd as fa
+    return fa
+
+
+def test_per_token_quantizer_is_bit_exact():
+    be = ops()
+    rng = o.Rng(11)
+    hand = np.array([[127.0, -127.0, 0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 3.49, 63.5], [0.0] * 10,
+                     [-8.0, 4.0, 2.0, 1.0, 0.0, 8.0, -4.0, -2.0, -1.0, 0.03]], dtype=np.float32)
+    for x in (hand, rng.randn((16, 4096)), rng.randn((5, 100), std=3.0), rng.randn((33, 11008))):
+        xq, sx = be.quantize_rows_i8(be.upload(x))
+        wq, ws = o.quantize_rows_i8(x)
+        assert np.array_equal(be.download_owned(sx), ws)
+        assert np.array_equal(be.download_owned(xq), wq)
+    xb = o.to_bf16(rng.randn((8, 512)))
+    xq, sx = be.quantize_rows_i8(be.upload(xb))
+    wq, ws = o.quantize_rows_i8(o.from_bf16(xb))
+    assert np.array_equal(be.download_owned(sx), ws) and np.array_equal(be.download_owned(xq), wq)
+
+
+def test_weight_quantizer_and_tile_packing_round_trip():
+    fa = _fa()
+    be = ops()
+    rng = o.Rng(12)
+    for k, n in ((64, 16), (4096, 4096), (100, 37), (130, 70), (11008, 64)):
+        w = rng.randn((k, n), std=0.02)
+        store = be.upload(w)
+        qw = be.quantize_weight(fa.DeviceBufferView(store, 0, (k, n)))
+        codes, scales = qw.export()
+        o.set_threads(8)
+        wq, ws = o.quantize_cols_i8(w)
+        o.set_threads(1)
+        assert np.array_equal(scales, ws), (k, n)
+        assert np.array_equal(codes, wq), (k, n)
+        qw2 = be.import_quantized_weight(wq, ws)
+        c2, s2 = qw2.export()
+        assert np.array_equal(c2, wq) and np.array_equal(s2, ws)
+    w = rng.randn((256, 48))
+    qw = be.quantize_weight(fa.DeviceBufferView(be.upload(w), 0, (256, 48)), fa.capi.QW_E4M3_TENSOR)
+    codes, scale = qw.export()
+    wq, ws = o.quantize_tensor_e4m3(w)
+    assert scale[0] == ws and np.array_equal(codes, wq)
+
+
+def test_int8_matrix_core_known_answers_from_the_reference_probe():
+    """docs/perf/logs/int8-mma-probe-2608/RULE.txt:6-10,25-28 on the gfx950 int8 matrix instruction."""
+    fa = _fa()
+    be = ops()
+
+    def acc_of(a, b):
+        m, k = a.shape
+        n = b.shape[1]
+        kp = (k + 63) // 64 * 64
+        ap = np.zeros((m, kp), np.int8)
+        ap[:, :k] = a
+        bp = np.zeros((kp, n), np.int8)
+        bp[:k] = b
+        qw = be.import_quantized_weight(bp, np.ones(n, np.float32))
+        out, acc = be.gemm_w8a8(be.upload(ap), be.upload(np.ones(m, np.float32)), qw, fa.capi.F32, want_acc=True)
+        acc = be.download_owned(acc)
+        assert np.array_equal(be.download_owned(out), acc.astype(np.float32))
+        return acc
+
+    assert np.all(acc_of(np.ones((16, 32), np.int8), np.ones((32, 8), np.int8)) == 32)
+    a127 = np.full((16, 128), 127, np.int8)
+    assert np.all(acc_of(a127, np.full((128, 8), 127, np.int8)) == 2064512)
+    assert np.all(acc_of(a127, np.full((128, 8), -127, np.int8)) == -2064512)
+    r, kk, cc = np.arange(16)[:, None], np.arange(32)[None, :], np.arange(8)[None, :]
+    pa = ((r * 37 + kk * 91 + 11) % 251 - 125).astype(np.int64)
+    pb = ((np.arange(32)[:, None] * 53 + cc * 29 + 7) % 247 - 123).astype(np.int64)
+    pa[0, 0], pa[1, 1], pb[0, 0], pb[31, 7] = -128, 127, -128, 127
+    pc = np.arange(16)[:, None] * 1000003 - cc * 7919 - 5000000
+    got = acc_of(pa.astype(np.int8), pb.astype(np.int8)).astype(np.int64) + pc
+    assert np.array_equal(got, pc + pa @ pb)
+    # asymmetric random operands: a transposed or permuted operand layout cannot pass
+    rng = np.random.default_rng(0)
+    a = rng.integers(-128, 128, size=(37, 192), dtype=np.int8)
+    b = rng.integers(-128, 128, size=(192, 50), dtype=np.int8)
+    assert np.array_equal(acc_of(a, b).astype(np.int64), a.astype(np.int64) @ b.astype(np.int64))
+
+
+def test_w8a8_linear_benchmark_configuration_is_bit_exact():
+    """x f32 [16,4096] ~N(0,1), W f32 [4096,4096] ~N(0,0.02), seed 0: int32 accumulators bit-exact."""
+    fa = _fa()
+    be = ops()
+    rng = o.Rng(0)
+    x = rng.randn((16, 4096))
+    w = rng.randn((4096, 4096), std=0.02)
+    qw = be.quantize_weight(fa.DeviceBufferView(be.upload(w), 0, (4096, 4096)))
+    out, acc = be.linear_w8a8(be.upload(x), qw, want_acc=True)
+    o.set_threads(8)
+    wq, ws = o.quantize_cols_i8(w)
+    want_acc, want_out = o.linear_w8a8(x, wq, ws)
+    o.set_threads(1)
+    got_acc, got_out = be.download_owned(acc), be.download_owned(out)
+    assert np.array_equal(got_acc, want_acc)
+    r = assert_parity("W8A8_PARITY", "16x4096x4096", got_out, want_out)
+    assert r.bit_mismatch == 0
+    # the quantized linear tracks the f32 linear it replaces
+    ref = x.astype(np.float64) @ w.astype(np.float64)
+    assert np.abs(got_out - ref).max() < 0.03 * np.abs(ref).max()
+
+
+@pytest.mark.parametrize("m", [1, 8, 16, 17, 32, 33, 100, 300])
+def test_w8a8_linear_row_sweep_bias_and_output_types(m):
+    fa = _fa()
+    be = ops()
+    rng = o.Rng(100 + m)
+    k, n = (4096, 6144) if m <= 32 else (512, 200)
+    x = rng.randn((m, k))
+    w = rng.randn((k, n), std=0.02)
+    bias = rng.randn((n,))
+    o.set_threads(8)
+    wq, ws = o.quantize_cols_i8(w)
+    want_acc, want = o.linear_w8a8(x, wq, ws, bias)
+    o.set_threads(1)
+    qw = be.import_quantized_weight(wq, ws)
+    dbias = fa.DeviceBufferView(be.upload(bias), 0, (n,))
+    out, acc = be.linear_w8a8(be.upload(x), qw, bias=dbias, want_acc=True)
+    assert np.array_equal(be.download_owned(acc), want_acc)
+    got = be.download_owned(out)
+    assert assert_parity("W8A8_PARITY", f"{m}x{n}x{k}", got, want).bit_mismatch == 0
+    out_bf = be.linear_w8a8(be.upload(x), qw, bias=dbias, out_dtype=fa.capi.BF16)
+    assert_bf16_rounding_of("w8a8 bf16", be.download_owned(out_bf), got)
+    # bf16 activations are promoted exactly before the quantizer
+    xb = o.to_bf16(x)
+    out2 = be.download_owned(be.linear_w8a8(be.upload(xb), qw))
+    assert np.array_equal(out2, o.linear_w8a8(o.from_bf16(xb), wq, ws)[1])
+
+
+def test_w8a8_ragged_shapes():
+    be = ops()
+    rng = o.Rng(13)
+    for m, k, n in ((3, 100, 37), (16, 64, 16), (32, 130, 70), (7, 4097, 33)):
+        x = rng.randn((m, k))
+        w = rng.randn((k, n), std=0.05)
+        wq, ws = o.quantize_cols_i8(w)
+        want_acc, want = o.linear_w8a8(x, wq, ws)
+        out, acc = be.linear_w8a8(be.upload(x), be.import_quantized_weight(wq, ws), want_acc=True)
+        assert np.array_equal(be.download_owned(acc), want_acc), (m, k, n)
+        assert np.array_equal(be.download_owned(out), want), (m, k, n)
+
+
+# Llama-7B layer shapes of the decode sweep: K -> N
+GEMV_SHAPES = [(4096, 12288), (4096, 4096), (4096, 22016), (11008, 4096)]
+
+
+@pytest.mark.parametrize("k,n", GEMV_SHAPES)
+def test_w8a16_decode_sweep(k, n):
+    fa = _fa()
+    be = ops()
+    rng = o.Rng(k + n)
+    w = rng.randn((k, n), std=0.02)
+    o.set_threads(8)
+    wq, ws = o.quantize_cols_i8(w)
+    qw = be.import_quantized_weight(wq, ws)
+    for m in (1, 8, 32):
+        a = o.to_bf16(rng.randn((m, k)))
+        want = o.linear_w8a16(a, wq, ws)
+        da = be.upload(a)
+        got = be.download_owned(be.linear_w8a16(da, qw, fa.capi.F32))
+        assert_parity("W8A16_PARITY", f"{m}x{n}x{k}", got, want)
+        assert_bf16_rounding_of("w8a16 bf16", be.download_owned(be.linear_w8a16(da, qw, fa.capi.BF16)), got)
+    o.set_threads(1)
+
+
+def test_w8a16_rejects_shapes_outside_its_contract():
+    fa = _fa()
+    be = ops()
+    wq = np.ones((100, 16), np.int8)
+    qw = be.import_quantized_weight(wq, np.ones(16, np.float32))
+    with pytest.raises(fa.Unsupported):
+        be.linear_w8a16(be.upload(np.zeros((1, 100), np.uint16)), qw)
+    qw = be.import_quantized_weight(np.ones((128, 16), np.int8), np.ones(16, np.float32))
+    with pytest.raises(fa.Unsupported):
+        be.linear_w8a16(be.upload(np.zeros((33, 128), np.uint16)), qw)
+    with pytest.raises(fa.ShapeMismatch):
+        be.linear_w8a16(be.upload(np.zeros((2, 64), np.uint16)), qw)
+
+
+def test_w8a16_one_hot_rows_pick_weight_rows_exactly():
+    fa = _fa()
+    be = ops()
+    rng = np.random.default_rng(3)
+    k, n = 256, 48
+    wq = rng.integers(-127, 128, size=(k, n), dtype=np.int8)
+    ws = np.ones(n, np.float32)
+    qw = be.import_quantized_weight(wq, ws)
+    a = np.zeros((16, k), np.float32)
+    picks = [0, 1, 15, 16, 17, 63, 64, 65, 100, 127, 128, 200, 254, 255, 7, 8]
+    for r, p in enumerate(picks):
+        a[r, p] = 1.0
+    got = be.download_owned(be.linear_w8a16(be.upload(o.to_bf16(a)), qw, fa.capi.F32))
+    assert np.array_equal(got, wq[picks].astype(np.float32))
+
+
+def test_int8_prefill_gemm_rows_sampled_at_full_size():
+    """M=2048, K=4096, N=14336: accumulators of sampled rows bit-exact against the oracle."""
+    fa = _fa()
+    be = ops()
+    m, k, n = 2048, 4096, 14336
+    rng = np.random.default_rng(5)
+    aq = rng.integers(-127, 128, size=(m, k), dtype=np.int8)
+    wq = rng.integers(-127, 128, size=(k, n), dtype=np.int8)
+    sx = rng.uniform(0.01, 0.05, size=m).astype(np.float32)
+    sw = rng.uniform(1e-4, 1e-3, size=n).astype(np.float32)
+    qw = be.import_quantized_weight(wq, sw)
+    out, acc = be.gemm_w8a8(be.upload(aq), be.upload(sx), qw, fa.capi.F32, want_acc=True)
+    got_acc, got = be.download_owned(acc), be.download_owned(out)
+    rows = np.r_[0:16, 127:130, 1000:1016, 2040:2048]
+    o.set_threads(8)
+    want_acc = o.gemm_i8_i32(np.ascontiguousarray(aq[rows]), wq)
+    o.set_threads(1)
+    assert np.array_equal(got_acc[rows], want_acc)
+    assert np.array_equal(got[rows], o.dequant_i32(want_acc, np.ascontiguousarray(sx[rows]), sw))
+    # checksum over the whole output: column sums of the accumulators equal (sum_m a[m, :]) @ w
+    colsum = aq.astype(np.int64).sum(axis=0)
+    assert np.array_equal(got_acc.astype(np.int64).sum(axis=0), colsum @ wq.astype(np.int64))
+    out_bf = be.download_owned(be.gemm_w8a8(be.upload(aq), be.upload(sx), qw, fa.capi.BF16))
+    assert_bf16_rounding_of("gemm_w8a8 bf16", out_bf, got)
+
+
+def test_fp8_quantizer_bit_exact_and_gemm_within_stated_bound():
+    """e4m3 per-tensor: codes and scale bit-exact.  GEMM: the oracle sums the exact products in f64 and
+    rounds once; the matrix cores accumulate in f32, so the bound is the f32 accumulation error over K:
+    abs error <= 2^-20 * sum_k |a||b| * (sa*sb)  (about 16 ulp of the absolute-value product), and the
+    composite tolerance must hold for at least 99.9 % of the outputs."""
+    fa = _fa()
+    be = ops()
+    rng = o.Rng(21)
+    for m, k, n in ((64, 256, 48), (130, 1024, 200), (2048, 4096, 512)):
+        a, w = rng.randn((m, k)), rng.randn((k, n))
+        aq, a_scale = be.quantize_tensor_e4m3(be.upload(a))
+        want_aq, want_sa = o.quantize_tensor_e4m3(a)
+        assert be.download(a_scale)[0] == want_sa and np.array_equal(be.download(aq), want_aq)
+        qw = be.quantize_weight(fa.DeviceBufferView(be.upload(w), 0, (k, n)), fa.capi.QW_E4M3_TENSOR)
+        wq, sw = qw.export()
+        want_wq, want_sw = o.quantize_tensor_e4m3(w)
+        assert sw[0] == want_sw and np.array_equal(wq, want_wq)
+        got = be.download_owned(be.gemm_e4m3(aq, a_scale, qw, fa.capi.F32))
+        o.set_threads(8)
+        want = o.gemm_e4m3(want_aq, want_wq, want_sa, want_sw)
+        o.set_threads(1)
+        absprod = (np.abs(o.from_e4m3(want_aq)).astype(np.float64) @ np.abs(o.from_e4m3(want_wq)).astype(np.float64))
+        bound = absprod * float(want_sa) * float(want_sw) * 2.0 ** -20 + 1e-30
+        err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+        print("FP8_PARITY\t%dx%dx%d\tmax_err/bound=%.3e" % (m, n, k, float((err / bound).max())), flush=True)
+        assert np.all(err <= bound)
+        r = o.compare(got, want)
+        print(r.line("FP8_PARITY", f"{m}x{n}x{k}"), flush=True)
+        assert r.fail_count <= 1e-3 * r.total
+        out_bf = be.download_owned(be.gemm_e4m3(aq, a_scale, qw, fa.capi.BF16))
+        assert_bf16_rounding_of("gemm_e4m3 bf16", out_bf, got)
+    # e4m3-representable operands with absmax 448 (scale exactly 1): every product is a multiple of 2^9
+    # and every partial sum stays below 2^33, so f32 accumulation in any order is exact
+    a = np.tile(np.array([[64, 128, -256, 448]], np.float32), (16, 32))
+    w = np.tile(np.array([[224], [-112], [56], [448]], np.float32), (32, 16))
+    aq, sa = be.quantize_tensor_e4m3(be.upload(a))
+    qw = be.quantize_weight(fa.DeviceBufferView(be.upload(w), 0, (128, 16)), fa.capi.QW_E4M3_TENSOR)
+    assert be.download(sa)[0] == 1.0 and np.array_equal(o.from_e4m3(be.download(aq)), a)
+    got = be.download_owned(be.gemm_e4m3(aq, sa, qw, fa.capi.F32))
+    assert np.array_equal(got, (a.astype(np.float64) @ w.astype(np.float64)).astype(np.float32))

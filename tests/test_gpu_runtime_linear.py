@@ -1,0 +1,212 @@
+"""GPU parity: memory ops, pool, f32 GEMM / linear (reference summation order),
+RMSNorm, RoPE and the small elementwise operators, all through the C ABI."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle_lib as o
+from gpu_common import assert_parity, ops
+
+pytestmark = pytest.mark.gpu
+
+
+def test_device_is_gfx950_and_provider_surface():
+    import fandhe_ai_amd as fa
+    prov = fa.RocmDeviceProvider()
+    assert prov.backend_name() == "rocm" and prov.is_available()
+    assert prov.enumerate()[0] == fa.Device.Rocm(0)
+    info = ops().info()
+    assert info.arch.decode().startswith("gfx950") and info.wavefront_size == 64
+    print("DEVICE", info.name.decode(), info.arch.decode(), "CUs", info.compute_units, "clock_khz", info.clock_khz)
+    with pytest.raises(fa.DeviceUnavailable):
+        fa.RocmBackendOps(99)
+
+
+def test_memory_ops_round_trip_views_and_pool():
+    import fandhe_ai_amd as fa
+    be = ops()
+    x = np.arange(1000, dtype=np.float32).reshape(10, 100)
+    b = be.upload(x)
+    assert np.array_equal(be.download(b), x)
+    z = be.alloc_zeroed((7, 5))
+    assert not be.download(z).any()
+    be.upload_into(np.array([1, 2, 3], np.float32), z, 4)
+    got = be.download(z).ravel()
+    assert got[4:7].tolist() == [1, 2, 3] and got[:4].sum() == 0 and got[7:].sum() == 0
+    with pytest.raises(fa.InvalidArgument):
+        be.upload_into(np.zeros(3, np.float32), z, 33)
+    with pytest.raises(fa.InvalidArgument):
+        fa.DeviceBufferView(z, 30, (2, 3))
+    seen = []
+    be.with_host_view(b, lambda s: seen.append(float(s.sum())))
+    assert seen == [float(x.sum())]
+    # numel == 0 never touches the device (crates/tensor-core/src/buffer.rs:50-59)
+    e = be.alloc_zeroed((0, 4))
+    assert be.download(e).size == 0
+    # pool: a freed block is reused for the same size class, stats follow pool_core.rs:122-139
+    s0 = be.device_memory_pool_stats()
+    t = be.alloc_zeroed((1000,))            # 4000 B -> class 4096
+    t.free()
+    s1 = be.device_memory_pool_stats()
+    t2 = be.alloc_zeroed((1010,))           # 4040 B -> the same class
+    s2 = be.device_memory_pool_stats()
+    assert s2.reuse_count == s1.reuse_count + 1
+    assert s2.capacity_waste_bytes - s1.capacity_waste_bytes == 4096 - 4040
+    t2.free()
+    be.release_cached_device_memory()
+    s3 = be.device_memory_pool_stats()
+    assert s3.cached_bytes == 0 and s3.released_bytes > s0.released_bytes
+    cls = C.c_uint64()
+    for n in (0, 1, 255, 256, 1793, 200704, (1 << 20) + 1, (64 << 20) - 1, (64 << 20) + 7):
+        assert fa.capi.lib.fa_size_class_for(n, C.byref(cls)) == 0 and cls.value == o.lib.orc_size_class_for(n)
+    # a buffer of another context is a foreign handle
+    other = fa.RocmBackendOps(0)
+    try:
+        fb = other.upload(np.zeros(4, np.float32))
+        with pytest.raises(fa.DeviceMismatch):
+            be.download(fb)
+        fb.free()
+    finally:
+        other.close()
+
+
+# crates/backend-rocm/tests/gemm_real_device.rs:16-38
+GEMM_SHAPES = [(1, 1, 1), (1, 1, 0), (64, 64, 16), (63, 65, 17), (130, 70, 33), (5, 129, 200), (128, 128, 64),
+               (257, 255, 513), (128, 128, 32), (65, 64, 16), (64, 63, 16), (64, 64, 15), (64, 64, 17), (1, 257, 33),
+               (257, 1, 33), (193, 129, 48), (64, 64, 4096), (33, 17, 4097), (128, 96, 8192), (0, 5, 3), (5, 0, 3)]
+
+
+def _data(n, seed):
+    out = np.empty(n, dtype=np.float32)
+    o.lib.orc_test_data_f32(o.ptr(out, o.f32p), n, seed)
+    return out
+
+
+def test_gemm_device_is_bit_identical_to_the_fma_reference():
+    be = ops()
+    o.set_threads(8)
+    for i, (m, n, k) in enumerate(GEMM_SHAPES):
+        a = _data(m * k, 1 + i).reshape(m, k)
+        b = _data(k * n, 100 + i).reshape(k, n)
+        want = o.gemm_f32(a, b)
+        got = be.download_owned(be.gemm_device(be.upload(a), be.upload(b)))
+        r = assert_parity("ROCM_PARITY", f"{m}x{n}x{k}", got, want)
+        assert r.bit_mismatch == 0
+    o.set_threads(1)
+
+
+def test_linear_forward_device_views_bias_relu():
+    import fandhe_ai_amd as fa
+    be = ops()
+    rng = o.Rng(5)
+    m, k, n = 16, 200, 72
+    a = rng.randn((m, k))
+    flat = rng.randn((37 + k * n + 11 + n,), std=0.1)       # one flat parameter buffer, weight and bias are views
+    w = flat[37:37 + k * n].reshape(k, n)
+    bias = flat[37 + k * n + 11:37 + k * n + 11 + n]
+    store = be.upload(flat)
+    wv = fa.DeviceBufferView(store, 37, (k, n))
+    bv = fa.DeviceBufferView(store, 37 + k * n + 11, (n,))
+    da = be.upload(a)
+    for act, code in (("none", 0), ("relu", 1)):
+        got = be.download_owned(be.linear_forward_device(da, wv, bv, act))
+        want = o.linear_f32(a, np.ascontiguousarray(w), np.ascontiguousarray(bias), code)
+        assert assert_parity("LINEAR_F32", f"{m}x{n}x{k}:{act}", got, want).bit_mismatch == 0
+    got = be.download_owned(be.linear_forward_device(da, wv, None, "none"))
+    assert np.array_equal(got, o.gemm_f32(a, np.ascontiguousarray(w)))
+    with pytest.raises(fa.Unsupported):
+        be.linear_forward_device(da, wv, bv, "gelu")
+    with pytest.raises(fa.ShapeMismatch):
+        be.linear_forward_device(da, fa.DeviceBufferView(store, 0, (k + 1, n)), None)
+
+
+def test_rmsnorm_reference_fixtures_and_sweep():
+    import fandhe_ai_amd as fa
+    be = ops()
+    # crates/backend-cpu/src/rmsnorm.rs:433-441
+    x = np.array([[1, 2, 3, 4]], dtype=np.float32)
+    got = be.rmsnorm(x, None, 0.0)
+    assert np.array_equal(got, o.rmsnorm_f32(x, None, 0.0)[1])
+    # NaN poisons its row only (rmsnorm.rs:443-462)
+    x = np.array([[1, float("nan"), 3], [1, 2, 3]], dtype=np.float32)
+    got = be.rmsnorm(x, None, 1e-5)
+    assert np.all(np.isnan(got[0])) and np.all(np.isfinite(got[1]))
+    with pytest.raises(fa.InvalidArgument):
+        be.rmsnorm(x, None, -1.0)
+    with pytest.raises(fa.ShapeMismatch):
+        be.rmsnorm(x, np.ones(2, np.float32), 1e-5)
+    x = np.array([[1e30, -1e30, 1e30, 1e-30]], dtype=np.float32)
+    assert np.all(np.isfinite(be.rmsnorm(x, None, 1e-5)))
+    rng = o.Rng(6)
+    for rows, hidden in ((3, 1), (3, 4), (2, 8), (3, 1023), (3, 1024), (2, 4097), (32, 4096), (2048, 4096)):
+        x = rng.randn((rows, hidden))
+        w = rng.randn((hidden,))
+        o.set_threads(8)
+        rc, want = o.rmsnorm_f32(x, w, 1e-5)
+        o.set_threads(1)
+        got = be.rmsnorm(x, w, 1e-5)
+        r = assert_parity("RMSNORM", f"{rows}x{hidden}", got, want)
+        assert r.max_rel_err < 1e-6
+    assert be.rmsnorm(np.zeros((0, 8), np.float32), None, 1e-5).size == 0
+
+
+def test_rope_and_elementwise_against_the_oracle():
+    be = ops()
+    rng = o.Rng(7)
+    x = rng.randn((6, 5, 128))
+    pos = np.array([0, 1, 7, 100, 4095, 8191], dtype=np.int32)
+    got = be.download_owned(be.rope(be.upload(x), be.upload(pos), 500000.0))
+    want = o.rope_f32(x, pos, 500000.0)
+    assert_parity("ROPE", "6x5x128", got, want)
+    assert np.array_equal(got[0], x[0])
+    g, u = rng.randn((32, 14336)), rng.randn((32, 14336))
+    got = be.download_owned(be.silu_mul(be.upload(g), be.upload(u)))
+    assert_parity("SILU_MUL", "32x14336", got, o.silu_mul_f32(g, u))
+    a, b = rng.randn((32, 4096)), rng.randn((32, 4096))
+    assert np.array_equal(be.download_owned(be.add(be.upload(a), be.upload(b))), a + b)
+    # greedy argmax: first maximum, NaN ignored, all-NaN -> 0
+    logits = rng.randn((32, 32000))
+    logits[3, 100] = logits[3, 20000] = 50.0
+    logits[4, :] = np.nan
+    logits[5, 7] = np.nan
+    got = be.download_owned(be.argmax(be.upload(logits)))
+    assert np.array_equal(got, o.argmax_rows(logits)) and got[3] == 100 and got[4] == 0
+    small = np.array([[1.0, 3.0, 3.0, 2.0], [-1.0, -2.0, -0.5, -9.0]], np.float32)
+    assert be.download_owned(be.argmax(be.upload(small))).tolist() == [1, 2]
+    table = rng.randn((50, 96))
+    idx = np.array([3, 49, 0, 3], dtype=np.int32)
+    assert np.array_equal(be.download_owned(be.gather(be.upload(table), be.upload(idx))), table[idx])
+    v = rng.randn((1000,))
+    import fandhe_ai_amd as fa
+    bf = be.download_owned(be.convert(be.upload(v), fa.capi.BF16))
+    assert np.array_equal(bf, o.to_bf16(v))
+    assert np.array_equal(be.download_owned(be.convert(be.upload(bf), fa.capi.F32)), o.from_bf16(bf))
+
+
+def test_sync_points_are_rejected_during_graph_capture_and_graph_replays():
+    import fandhe_ai_amd as fa
+    be = ops()
+    lib = fa.capi.lib
+    a = be.upload(np.full(256, 2.0, np.float32))
+    b = be.upload(np.full(256, 3.0, np.float32))
+    out = be.alloc_zeroed((256,))
+    fa.check(lib.fa_graph_capture_begin(be._ctx))
+    try:
+        with pytest.raises(fa.DeviceContextCaptureInProgress):
+            be.download(a)
+        with pytest.raises(fa.DeviceContextCaptureInProgress):
+            be.synchronize_device()
+        with pytest.raises(fa.DeviceContextCaptureInProgress):
+            be.alloc_zeroed((4,))
+        fa.check(lib.fa_add(be._ctx, a._h, b._h, 256, out._h))
+        fa.check(lib.fa_add(be._ctx, out._h, b._h, 256, out._h))
+    finally:
+        g = C.c_void_p()
+        fa.check(lib.fa_graph_capture_end(be._ctx, C.byref(g)))
+    assert not be.download(out).any()              # capture records, it does not execute
+    for rep in range(3):
+        fa.check(lib.fa_graph_launch(be._ctx, g))
+        assert np.all(be.download(out) == 8.0)
+        be.upload_into(np.zeros(256, np.float32), out, 0)
+    fa.check(lib.fa_graph_destroy(be._ctx, g))
