@@ -74,7 +74,7 @@ def test_f32_append_then_attention_matches_the_reference_algorithm(case):
                           dtype=np.uint32)
         lens = np.full(batch, seq, dtype=np.uint32)
         be.paged_kv_append(be.upload(k.reshape(-1, embed)), be.upload(v.reshape(-1, embed)), k_pool, v_pool, slots, layout)
-        assert o.paged_kv_append(k.reshape(-1, embed), v.reshape(-1, embed), hk, hv, slots, layout.c()) == 0
+        assert o.paged_kv_append(k.reshape(-1, embed), v.reshape(-1, embed), hk, hv, slots, o.PagedLayout(num_blocks, bs, embed)) == 0
         assert np.array_equal(be.download(k_pool).reshape(-1, embed), hk)          # append is a bit-exact copy
         assert np.array_equal(be.download(v_pool).reshape(-1, embed), hv)
         args = fa.PagedAttentionArgs(layout, batch, l, heads, max_blocks, scale)
@@ -168,7 +168,8 @@ def test_bf16_gqa_decode_against_the_oracle(heads, kv_heads):
     for h in range(heads):
         g = h // (heads // kv_heads)
         assert np.array_equal(got_bf[0, 0, h * 128:(h + 1) * 128], vp[tables[0, 0], 0, g * 128:(g + 1) * 128])
-    # device-resident tables give the same bits as host tables
+    # device-resident tables give the same bits as host tables (same launch shape)
+    got_bf = be.download_owned(be.paged_attention_forward(dq, dk, dv, tables, lens, args))
     got_dev = be.download_owned(be.paged_attention_forward_device(dq, dk, dv, be.upload(tables), be.upload(lens), args))
     assert np.array_equal(got_dev, got_bf)
 
