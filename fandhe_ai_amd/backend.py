@@ -458,6 +458,11 @@ class RocmBackendOps:
         check(lib.fa_gather_rows(self._ctx, table._h, table.shape[0], cols, idx._h, rows, out._h))
         return out
 
+    def fill_normal(self, buf, seed, mean=0.0, std=1.0, offset=0, numel=None):
+        """Synthetic N(mean, std) data generated on the device (benchmarks)."""
+        check(lib.fa_fill_normal(self._ctx, buf._h, offset, buf.numel() - offset if numel is None else numel, seed,
+                                 mean, std))
+
     def convert(self, src, dtype):
         out = self.alloc_uninit(src.shape, dtype)
         check(lib.fa_convert(self._ctx, src._h, src.numel(), out._h))

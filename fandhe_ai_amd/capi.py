@@ -110,6 +110,7 @@ SIGNATURES = {
     "fa_argmax_rows": (C.c_int32, [ctx_p, buf_p, u64, u64, buf_p]),
     "fa_gather_rows": (C.c_int32, [ctx_p, buf_p, u64, u64, buf_p, u64, buf_p]),
     "fa_convert": (C.c_int32, [ctx_p, buf_p, u64, buf_p]),
+    "fa_fill_normal": (C.c_int32, [ctx_p, buf_p, u64, u64, u64, C.c_float, C.c_float]),
     "fa_validate_paged_kv_append": (C.c_int32, [u64, u64, u64, u64, u32p, u64, C.POINTER(PagedLayout)]),
     "fa_validate_paged_attention": (C.c_int32, [u64, u64, u64, u32p, u64, u32p, u64, C.POINTER(PagedArgs),
                                                 C.POINTER(PagedPlan)]),

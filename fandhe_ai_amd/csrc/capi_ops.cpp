@@ -465,6 +465,20 @@ fa_status fa_gather_rows(fa_context *ctx, const fa_buffer *table, uint64_t table
     return after_launch(ctx, "gather_rows_f32");
 }
 
+fa_status fa_fill_normal(fa_context *ctx, fa_buffer *buf, uint64_t offset, uint64_t numel, uint64_t seed, float mean,
+                         float std) {
+    if (fa_status s = check_ctx(ctx)) return s;
+    if (fa_status s = check_buf(ctx, buf, "fill_normal: buf")) return s;
+    if (buf->dtype != FA_F32 && buf->dtype != FA_BF16) return fail(FA_ERR_INVALID_ARGUMENT, "fill_normal: f32 or bf16 only");
+    uint64_t end;
+    if (__builtin_add_overflow(offset, numel, &end) || end > buf->numel)
+        return fail(FA_ERR_INVALID_ARGUMENT, "fill_normal: range exceeds the buffer");
+    if (offset % 2 != 0) return fail(FA_ERR_INVALID_ARGUMENT, "fill_normal: offset must be even");
+    k::fill_normal((char *)buf->ptr + offset * dtype_size(buf->dtype), buf->dtype == FA_BF16, numel, seed, mean, std,
+                   ctx->stream);
+    return after_launch(ctx, "fill_normal");
+}
+
 fa_status fa_convert(fa_context *ctx, const fa_buffer *src, uint64_t numel, fa_buffer *dst) {
     if (fa_status s = check_ctx(ctx)) return s;
     if (fa_status s = check_buf(ctx, src, "convert: src")) return s;

@@ -110,6 +110,37 @@ __global__ void fill_u32_kernel(uint32_t *p, uint32_t v, uint64_t n) {
     for (; i < n; i += stride) p[i] = v;
 }
 
+__device__ __forceinline__ uint64_t splitmix64(uint64_t x) {
+    x += 0x9E3779B97F4A7C15ull;
+    x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+    x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+    return x ^ (x >> 31);
+}
+// two normals per hash (Box-Muller): element pair (2p, 2p+1) shares one draw
+__global__ void fill_normal_kernel(void *__restrict__ out, int out_bf16, uint64_t n, uint64_t seed, float mean,
+                                   float std) {
+    uint64_t pair = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    for (; pair * 2 < n; pair += stride) {
+        uint64_t h = splitmix64(seed * 0xD1342543DE82EF95ull + pair);
+        float u1 = ((float)(uint32_t)(h >> 40) + 1.0f) * (1.0f / 16777216.0f);     // (0, 1]
+        float u2 = (float)(uint32_t)((h >> 8) & 0xffffffu) * (1.0f / 16777216.0f);  // [0, 1)
+        float r = sqrtf(-2.0f * logf(u1));
+        float sn, cs;
+        sincosf(6.283185307179586f * u2, &sn, &cs);
+        float z[2] = {mean + std * (r * cs), mean + std * (r * sn)};
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            uint64_t i = pair * 2 + e;
+            if (i >= n) break;
+            if (out_bf16)
+                ((uint16_t *)out)[i] = f32_to_bf16(z[e]);
+            else
+                ((float *)out)[i] = z[e];
+        }
+    }
+}
+
 // Rotate-half RoPE: pair (i, i + Dh/2), angle = pos * theta^(-2i/Dh) in f64,
 // cos / sin rounded to f32, four f32 products and one add / sub, no contraction.
 __global__ void rope_kernel(const float *__restrict__ x, const int32_t *__restrict__ pos, float *__restrict__ out,
@@ -170,6 +201,10 @@ void convert_bf16_to_f32(const uint16_t *in, float *out, uint64_t n, hipStream_t
 void fill_u32(uint32_t *p, uint32_t v, uint64_t n, hipStream_t s) {
     if (n == 0) return;
     fill_u32_kernel<<<grid_for(n, 256), 256, 0, s>>>(p, v, n);
+}
+void fill_normal(void *out, int out_bf16, uint64_t n, uint64_t seed, float mean, float std, hipStream_t s) {
+    if (n == 0) return;
+    fill_normal_kernel<<<grid_for((n + 1) / 2, 256, 65535u), 256, 0, s>>>(out, out_bf16, n, seed, mean, std);
 }
 void rope_f32(const float *x, const int32_t *pos, float *out, uint64_t rows, uint64_t heads, uint64_t head_dim,
               double theta, hipStream_t s) {

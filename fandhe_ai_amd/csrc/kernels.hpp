@@ -34,6 +34,8 @@ void convert_bf16_to_f32(const uint16_t *in, float *out, uint64_t n, hipStream_t
 void rope_f32(const float *x, const int32_t *pos, float *out, uint64_t rows, uint64_t heads,
               uint64_t head_dim, double theta, hipStream_t s);
 void fill_u32(uint32_t *p, uint32_t v, uint64_t n, hipStream_t s);
+// N(mean, std) from a counter-based hash of (seed, index); out is f32 or bf16
+void fill_normal(void *out, int out_bf16, uint64_t n, uint64_t seed, float mean, float std, hipStream_t s);
 
 // ---- norms / quantizers (kern_norm_quant.hip) -------------------------------
 void rmsnorm_f32(const float *x, const float *w, float *out, uint64_t rows, uint64_t hidden,

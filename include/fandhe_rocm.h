@@ -206,6 +206,12 @@ fa_status fa_argmax_rows(fa_context *ctx, const fa_buffer *x, uint64_t rows, uin
 /* BackendOps::gather of rows (backend_ops.rs:3375): out[r, :] = table[idx[r], :]. */
 fa_status fa_gather_rows(fa_context *ctx, const fa_buffer *table, uint64_t table_rows,
                          uint64_t cols, const fa_buffer *idx, uint64_t rows, fa_buffer *out);
+/* Synthetic data: fills an f32 or bf16 buffer with N(mean, std) values from a
+ * counter-based generator (value i depends only on seed and i).  For
+ * benchmarks that need tens of GB of resident inputs; not part of the
+ * reference's interface. */
+fa_status fa_fill_normal(fa_context *ctx, fa_buffer *buf, uint64_t offset, uint64_t numel,
+                         uint64_t seed, float mean, float std);
 /* dtype conversion f32 <-> bf16 (round to nearest even, once). */
 fa_status fa_convert(fa_context *ctx, const fa_buffer *src, uint64_t numel, fa_buffer *dst);
 
