@@ -285,6 +285,7 @@ def main():
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--ppc", type=int, default=0, help="tuning: KV pages per attention work item (0 = built-in)")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (--gpus 1); nothing here shards across devices")
@@ -294,6 +295,7 @@ def main():
     info = be.info()
     log("device", info.arch.decode(), "CUs", info.compute_units, "clock_khz", info.clock_khz)
     lib = fa.capi.lib
+    fa.check(lib.fa_set_tuning(2, a.ppc))
     cfg = dict(MODEL, n_layers=a.layers)
     batch = 32
     ctxs = np.random.default_rng(0).integers(1024, 8193, size=batch).tolist()

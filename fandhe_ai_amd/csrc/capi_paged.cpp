@@ -44,7 +44,7 @@ k::PagedShape make_shape(const fa_paged_args *a) {
 
 bool decode_fast_path(const k::PagedShape &ps, const fa_buffer *q) {
     uint32_t group = ps.num_heads / ps.num_kv_heads;
-    return q->dtype == FA_BF16 && ps.head_dim == 128 && ps.block_size == 16 && ps.l_new == 1 && group <= 8 &&
+    return q->dtype == FA_BF16 && ps.head_dim == 128 && ps.block_size == 16 && ps.l_new == 1 && group <= 16 &&
            ps.max_blocks_per_seq >= 1;
 }
 
@@ -58,7 +58,7 @@ fa_status launch_attention(fa_context *ctx, const fa_buffer *q, const fa_buffer 
         if (fa_status s = ensure_workspace(ctx, need)) return s;
         k::paged_attention_decode_bf16((const uint16_t *)q->ptr, (const uint16_t *)k_pool->ptr,
                                        (const uint16_t *)v_pool->ptr, d_tables, d_lens, ps, (uint32_t)g_decode_ppc,
-                                       ctx->workspace, out->ptr, out->dtype == FA_BF16, ctx->stream);
+                                       ctx->workspace, out->ptr, out->dtype == FA_BF16, nullptr, ctx->stream);
         return after_launch(ctx, "paged_attention_decode_bf16");
     }
     if (out->dtype != q->dtype) return fail(FA_ERR_INVALID_ARGUMENT, "paged_attention: out must have the type of q");

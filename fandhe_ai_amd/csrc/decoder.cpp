@@ -34,7 +34,7 @@ struct fa_decoder {
     // resident state and activations
     fa_buffer *tokens = nullptr, *tables = nullptr, *seq_lens = nullptr, *pos = nullptr, *slots = nullptr;
     fa_buffer *cos_sin = nullptr, *h = nullptr, *xq = nullptr, *sx = nullptr, *qkv = nullptr, *q_bf = nullptr;
-    fa_buffer *attn = nullptr, *gu = nullptr, *logits = nullptr;
+    fa_buffer *attn = nullptr, *act = nullptr, *pmax = nullptr, *logits = nullptr;
     fa_graph *graph = nullptr;
     uint32_t graph_batch = 0;
     int graph_ppc = 0;
@@ -70,7 +70,7 @@ fa_status check_vec(const fa_decoder *d, const fa_buffer *b, uint64_t numel, con
 
 void free_all(fa_context *ctx, fa_decoder *d) {
     fa_buffer **bufs[] = {&d->tokens, &d->tables, &d->seq_lens, &d->pos, &d->slots, &d->cos_sin, &d->h, &d->xq,
-                          &d->sx,     &d->qkv,    &d->q_bf,     &d->attn, &d->gu,   &d->logits};
+                          &d->sx,     &d->qkv,    &d->q_bf,     &d->attn, &d->act,  &d->pmax, &d->logits};
     for (auto pb : bufs) {
         if (*pb) fa_buffer_free(ctx, *pb);
         *pb = nullptr;
@@ -137,13 +137,17 @@ fa_status enqueue_step(fa_context *ctx, fa_decoder *d) {
         k::paged_attention_decode_bf16((const uint16_t *)d->q_bf->ptr, (const uint16_t *)L.k_pool->ptr,
                                        (const uint16_t *)L.v_pool->ptr, (const uint32_t *)d->tables->ptr,
                                        (const uint32_t *)d->seq_lens->ptr, ps, (uint32_t)g_decode_ppc, ctx->workspace,
-                                       d->attn->ptr, 1, s);
-        k::quantize_rows_i8(d->attn->ptr, true, nullptr, (int8_t *)d->xq->ptr, (float *)d->sx->ptr, B, m_pad, EQ, EQ, s);
+                                       d->attn->ptr, 1, (float *)d->pmax->ptr, s);
+        k::quantize_rows_from_pmax(d->attn->ptr, true, (const float *)d->pmax->ptr, c.n_heads, (int8_t *)d->xq->ptr,
+                                   (float *)d->sx->ptr, B, m_pad, EQ, s);
         linear(L.wo, d->h->ptr, (const float *)d->h->ptr);
         k::rmsnorm_quantize_i8((const float *)d->h->ptr, (const float *)L.ffn_norm->ptr, c.rms_eps, nullptr,
                                (int8_t *)d->xq->ptr, (float *)d->sx->ptr, B, m_pad, D, s);
-        linear(L.wgu, d->gu->ptr, nullptr);
-        k::swiglu_quantize_i8((const float *)d->gu->ptr, (int8_t *)d->xq->ptr, (float *)d->sx->ptr, B, m_pad, F, s);
+        k::linear_w8a8_swiglu_skinny((const int8_t *)d->xq->ptr, (const int8_t *)L.wgu->codes->ptr,
+                                     (const float *)d->sx->ptr, (const float *)L.wgu->scales->ptr, B, L.wgu->n,
+                                     L.wgu->n_pad, L.wgu->k_pad, (float *)d->act->ptr, (float *)d->pmax->ptr, 4, s);
+        k::quantize_rows_from_pmax(d->act->ptr, false, (const float *)d->pmax->ptr, (uint32_t)(F / 16),
+                                   (int8_t *)d->xq->ptr, (float *)d->sx->ptr, B, m_pad, F, s);
         linear(L.wdown, d->h->ptr, (const float *)d->h->ptr);
     }
     k::rmsnorm_quantize_i8((const float *)d->h->ptr, (const float *)d->final_norm->ptr, c.rms_eps, nullptr,
@@ -167,10 +171,11 @@ fa_status fa_decoder_create(fa_context *ctx, const fa_decoder_config *cfg, fa_de
         return fail(FA_ERR_INVALID_ARGUMENT, "decoder_create: zero dimension");
     if (c.head_dim != 128 || c.block_size != 16)
         return fail(FA_ERR_UNSUPPORTED, "decoder_create: head_dim must be 128 and block_size 16");
-    if (c.n_heads % c.n_kv_heads != 0 || c.n_heads / c.n_kv_heads > 8)
-        return fail(FA_ERR_UNSUPPORTED, "decoder_create: heads per kv head must be an integer of at most 8");
+    if (c.n_heads % c.n_kv_heads != 0 || c.n_heads / c.n_kv_heads > 16)
+        return fail(FA_ERR_UNSUPPORTED, "decoder_create: heads per kv head must be an integer of at most 16");
     if (c.d_model % 64 != 0 || c.d_ffn % 64 != 0)
         return fail(FA_ERR_UNSUPPORTED, "decoder_create: d_model and d_ffn must be multiples of 64");
+    if (c.d_model > 16384) return fail(FA_ERR_UNSUPPORTED, "decoder_create: d_model above 16384");
     if (c.max_batch > 32) return fail(FA_ERR_UNSUPPORTED, "decoder_create: at most 32 sequences per step");
     if (!std::isfinite(c.rms_eps) || c.rms_eps < 0.0f) return fail(FA_ERR_INVALID_ARGUMENT, "decoder_create: bad rms_eps");
     if (!(c.rope_theta > 0.0)) return fail(FA_ERR_INVALID_ARGUMENT, "decoder_create: bad rope_theta");
@@ -204,7 +209,8 @@ fa_status fa_decoder_create(fa_context *ctx, const fa_decoder_config *cfg, fa_de
     mk(FA_F32, B * (EQ + 2 * EKV), &d->qkv);
     mk(FA_BF16, B * EQ, &d->q_bf);
     mk(FA_BF16, B * EQ, &d->attn);
-    mk(FA_F32, B * 2 * F, &d->gu);
+    mk(FA_F32, B * F, &d->act);
+    mk(FA_F32, B * std::max<uint64_t>(F / 16, c.n_heads), &d->pmax);
     mk(FA_F32, B * V, &d->logits);
     for (auto &l : d->layers) {
         mk(FA_BF16, layout.num_blocks * layout.block_size * layout.embed_dim, &l.k_pool);

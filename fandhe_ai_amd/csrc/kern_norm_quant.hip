@@ -101,47 +101,106 @@ __global__ void __launch_bounds__(kBlock)
     }
 }
 
-// RMSNorm of an f32 row followed by its per-token quantization; the
-// normalized value is recomputed (same operations, same bits) in each pass.
+// RMSNorm of an f32 row followed by its per-token quantization.  Thread t owns the 16-element chunks
+// t, t + 256, ... of the row and keeps them in registers (NCH chunks), so the row is read once:
+// f64 sum of squares -> rstd -> y = (x * rstd) * w -> absmax -> codes, written as 16-byte tile chunks.
+template <int NCH>
 __global__ void __launch_bounds__(kBlock)
     rmsnorm_quantize_kernel(const float *__restrict__ x, const float *__restrict__ w, float eps, float inv_n,
                             float *__restrict__ out_f32, int8_t *__restrict__ xq_tiled, float *__restrict__ sx,
                             uint64_t m, uint64_t hidden) {
     __shared__ double smem_d[kWaves];
     __shared__ float smem_f[kWaves];
-    uint64_t r = blockIdx.x;
-    uint64_t k_tiles = hidden / 64;
+    const uint64_t r = blockIdx.x;
+    const uint64_t k_tiles = hidden / 64, n_chunks = hidden / 16;
     if (r >= m) {
-        for (uint64_t c = threadIdx.x; c < hidden / 16; c += kBlock)
+        for (uint64_t c = threadIdx.x; c < n_chunks; c += kBlock)
             *(v4i *)(xq_tiled + tiled_chunk_offset(r, c, k_tiles)) = v4i{0, 0, 0, 0};
         return;
     }
     const float *row = x + r * hidden;
-    float rstd = row_rstd(row, hidden, inv_n, eps, smem_d);
-    float amax = 0.0f;
-    for (uint64_t i = threadIdx.x; i < hidden; i += kBlock) {
-        float y = __fmul_rn(__fmul_rn(row[i], rstd), w[i]);
-        if (out_f32) out_f32[r * hidden + i] = y;
-        amax = fmaxf(amax, fabsf(y));
+    v4f xv[NCH][4], wv[NCH][4];
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+        uint64_t c = threadIdx.x + (uint64_t)i * kBlock;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            xv[i][v] = c < n_chunks ? *(const v4f *)(row + c * 16 + v * 4) : v4f{0.f, 0.f, 0.f, 0.f};
+            wv[i][v] = c < n_chunks ? *(const v4f *)(w + c * 16 + v * 4) : v4f{0.f, 0.f, 0.f, 0.f};
+        }
     }
+    double acc = 0.0;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i)
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                double d = (double)xv[i][v][e];
+                acc = fma(d, d, acc);
+            }
+    acc = block_sum<double, kWaves>(acc, smem_d);
+    const float rstd = (float)(1.0 / sqrt(fma(acc, (double)inv_n, (double)eps)));
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i)
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float y = __fmul_rn(__fmul_rn(xv[i][v][e], rstd), wv[i][v][e]);
+                xv[i][v][e] = y;
+                amax = fmaxf(amax, fabsf(y));
+            }
     amax = block_max<kWaves>(amax, smem_f);
-    float scale = __fdiv_rn(amax, 127.0f);
+    const float scale = __fdiv_rn(amax, 127.0f);
     if (threadIdx.x == 0) sx[r] = scale;
-    for (uint64_t c = threadIdx.x; c < hidden / 16; c += kBlock) {
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+        uint64_t c = threadIdx.x + (uint64_t)i * kBlock;
+        if (c >= n_chunks) continue;
         uint32_t words[4];
 #pragma unroll
-        for (int wd = 0; wd < 4; ++wd) {
+        for (int v = 0; v < 4; ++v) {
             uint32_t word = 0;
 #pragma unroll
-            for (int b = 0; b < 4; ++b) {
-                uint64_t kk = c * 16 + wd * 4 + b;
-                float y = __fmul_rn(__fmul_rn(row[kk], rstd), w[kk]);
-                word |= ((uint32_t)quant_i8(y, scale) & 0xffu) << (8 * b);
-            }
-            words[wd] = word;
+            for (int e = 0; e < 4; ++e) word |= ((uint32_t)quant_i8(xv[i][v][e], scale) & 0xffu) << (8 * e);
+            words[v] = word;
+            if (out_f32) *(v4f *)(out_f32 + r * hidden + c * 16 + v * 4) = xv[i][v];
         }
         *(v4u *)(xq_tiled + tiled_chunk_offset(r, c, k_tiles)) = v4u{words[0], words[1], words[2], words[3]};
     }
+}
+
+// Quantizer for rows whose absmax is already known as `parts` partial maxima: every block first
+// reduces its row's partials (cheap, L2-resident), then quantizes a slab of 256 chunks.
+template <bool IN_BF16>
+__global__ void __launch_bounds__(kBlock)
+    quantize_from_pmax_kernel(const void *__restrict__ x, const float *__restrict__ pmax, uint32_t parts,
+                              int8_t *__restrict__ xq_tiled, float *__restrict__ sx, uint64_t m, uint64_t k) {
+    __shared__ float smem[kWaves];
+    const uint64_t r = blockIdx.y, k_tiles = k / 64, n_chunks = k / 16;
+    const uint64_t c = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (r >= m) {
+        if (c < n_chunks) *(v4i *)(xq_tiled + tiled_chunk_offset(r, c, k_tiles)) = v4i{0, 0, 0, 0};
+        return;
+    }
+    float amax = 0.0f;
+    for (uint32_t i = threadIdx.x; i < parts; i += kBlock) amax = fmaxf(amax, pmax[r * parts + i]);
+    amax = block_max<kWaves>(amax, smem);
+    const float scale = __fdiv_rn(amax, 127.0f);
+    if (blockIdx.x == 0 && threadIdx.x == 0) sx[r] = scale;
+    if (c >= n_chunks) return;
+    uint32_t words[4];
+#pragma unroll
+    for (int wd = 0; wd < 4; ++wd) {
+        uint32_t word = 0;
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+            word |= ((uint32_t)quant_i8(load_in<IN_BF16>(x, r * k + c * 16 + wd * 4 + b), scale) & 0xffu) << (8 * b);
+        words[wd] = word;
+    }
+    *(v4u *)(xq_tiled + tiled_chunk_offset(r, c, k_tiles)) = v4u{words[0], words[1], words[2], words[3]};
 }
 
 // absmax over a tensor: block maxima merged with an integer max on the bit
@@ -196,7 +255,24 @@ void rmsnorm_quantize_i8(const float *x, const float *w, float eps, float *out_f
                          uint64_t m, uint64_t m_pad, uint64_t hidden, hipStream_t s) {
     if (m_pad == 0 || hidden == 0) return;
     float inv_n = 1.0f / (float)hidden;
-    rmsnorm_quantize_kernel<<<(unsigned)m_pad, kBlock, 0, s>>>(x, w, eps, inv_n, out_f32, xq_tiled, sx, m, hidden);
+    uint64_t per_thread = (hidden / 16 + kBlock - 1) / kBlock;       // 16-element chunks per thread
+    unsigned grid = (unsigned)m_pad;
+    if (per_thread <= 1)
+        rmsnorm_quantize_kernel<1><<<grid, kBlock, 0, s>>>(x, w, eps, inv_n, out_f32, xq_tiled, sx, m, hidden);
+    else if (per_thread <= 2)
+        rmsnorm_quantize_kernel<2><<<grid, kBlock, 0, s>>>(x, w, eps, inv_n, out_f32, xq_tiled, sx, m, hidden);
+    else
+        rmsnorm_quantize_kernel<4><<<grid, kBlock, 0, s>>>(x, w, eps, inv_n, out_f32, xq_tiled, sx, m, hidden);
+}
+
+void quantize_rows_from_pmax(const void *x, bool in_bf16, const float *pmax, uint32_t parts, int8_t *xq_tiled,
+                             float *sx, uint64_t m, uint64_t m_pad, uint64_t k, hipStream_t s) {
+    if (m_pad == 0 || k == 0) return;
+    dim3 grid((unsigned)((k / 16 + kBlock - 1) / kBlock), (unsigned)m_pad);
+    if (in_bf16)
+        quantize_from_pmax_kernel<true><<<grid, kBlock, 0, s>>>(x, pmax, parts, xq_tiled, sx, m, k);
+    else
+        quantize_from_pmax_kernel<false><<<grid, kBlock, 0, s>>>(x, pmax, parts, xq_tiled, sx, m, k);
 }
 
 void tensor_absmax_f32(const float *x, uint64_t n, float *absmax, hipStream_t s) {

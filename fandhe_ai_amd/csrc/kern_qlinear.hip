@@ -21,19 +21,37 @@ struct EpiI8 {
     int32_t *acc_out;
     void *out;
     int out_bf16;
+    float *pmax;          // SwiGLU mode: per (row, block) absmax of the activation
 };
+
+// crates/tensor-core/src/scalar_op.rs:666-673 / :355
+__device__ __forceinline__ float silu_f32(float x) {
+    float s;
+    if (x >= 0.0f) {
+        s = __fdiv_rn(1.0f, 1.0f + expf(-x));
+    } else {
+        float e = expf(x);
+        s = __fdiv_rn(e, 1.0f + e);
+    }
+    return x * s;
+}
 
 // ------------------------------------------------------------------ W8A8
 // acc[m, n] = sum_k xq[m, k] * w[k, n] on v_mfma_i32_16x16x64_i8.
 // D layout: lane l holds column l % 16, rows 4 * (l / 16) + j, j = 0..3.
-template <int MT, int NTW, int NWAVES>
+// SWIGLU: the weight holds gate columns [0, n/2) and up columns [n/2, n); the block multiplies the
+// gate tile blockIdx.x and the up tile of the same columns and writes act = silu(gate) * up
+// ([m, n/2] f32) plus the block's per-row absmax, so that the next quantizer needs no pass over gate|up.
+template <int MT, int NTW, int NWAVES, bool SWIGLU>
 __global__ void __launch_bounds__(NWAVES * 64)
     w8a8_skinny_kernel(const int8_t *__restrict__ xq_tiled, const int8_t *__restrict__ w_tiles, uint32_t m,
                        uint32_t n, uint32_t n_tiles, uint32_t k_tiles, EpiI8 ep) {
+    static_assert(!SWIGLU || NTW == 2, "SwiGLU pairs one gate tile with one up tile");
     constexpr int NACC = MT * NTW * 4;
     __shared__ int red[NWAVES][NACC][64];
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
-    const uint32_t nt0 = blockIdx.x * NTW;
+    const uint32_t nt0 = SWIGLU ? blockIdx.x : blockIdx.x * NTW;
+    const uint32_t nt_step = SWIGLU ? n_tiles / 2 : 1;
 
     v4i acc[MT][NTW];
 #pragma unroll
@@ -49,7 +67,7 @@ __global__ void __launch_bounds__(NWAVES * 64)
     auto load_b = [&](uint32_t kt, v4i *b) {
 #pragma unroll
         for (int j = 0; j < NTW; ++j) {
-            uint32_t nt = nt0 + j;
+            uint32_t nt = nt0 + j * nt_step;
             b[j] = nt < n_tiles ? *(const v4i *)(b_base + ((uint64_t)nt * k_tiles + kt) * 1024) : v4i{0, 0, 0, 0};
         }
     };
@@ -92,6 +110,33 @@ __global__ void __launch_bounds__(NWAVES * 64)
             for (int e = 0; e < 4; ++e) red[wave][(i * NTW + j) * 4 + e][lane] = acc[i][j][e];
     __syncthreads();
 
+    if constexpr (SWIGLU) {
+        const uint32_t f = n / 2;
+        for (int q = wave; q < MT * 4; q += NWAVES) {
+            int i = q / 4, e = q % 4;
+            int sg = 0, su = 0;
+#pragma unroll
+            for (int w = 0; w < NWAVES; ++w) {
+                sg += red[w][(i * 2 + 0) * 4 + e][lane];
+                su += red[w][(i * 2 + 1) * 4 + e][lane];
+            }
+            uint32_t row = i * 16 + 4 * (lane / 16) + e;
+            uint32_t col = nt0 * 16 + lane % 16;
+            float a = 0.0f;
+            if (row < m && col < f) {
+                float vg = __fmul_rn((float)sg, __fmul_rn(ep.sx[row], ep.sw[col]));
+                float vu = __fmul_rn((float)su, __fmul_rn(ep.sx[row], ep.sw[col + f]));
+                float act = silu_f32(vg) * vu;
+                ((float *)ep.out)[(uint64_t)row * f + col] = act;
+                a = fabsf(act);
+            }
+            // absmax over the 16 columns of the tile (lanes sharing lane / 16)
+#pragma unroll
+            for (int off = 1; off < 16; off <<= 1) a = fmaxf(a, __shfl_xor(a, off, 64));
+            if (lane % 16 == 0 && row < m) ep.pmax[(uint64_t)row * (n_tiles / 2) + nt0] = a;
+        }
+        return;
+    }
     for (int idx = wave; idx < NACC; idx += NWAVES) {
         int sum = 0;
 #pragma unroll
@@ -253,13 +298,13 @@ void launch_w8a8(const int8_t *xq, const int8_t *wt, uint32_t m, uint32_t n, uin
                  const EpiI8 &ep, int ntw, int waves, hipStream_t s) {
     unsigned grid = (n_tiles + ntw - 1) / ntw;
     if (ntw == 1 && waves == 8)
-        w8a8_skinny_kernel<MT, 1, 8><<<grid, 512, 0, s>>>(xq, wt, m, n, n_tiles, k_tiles, ep);
+        w8a8_skinny_kernel<MT, 1, 8, false><<<grid, 512, 0, s>>>(xq, wt, m, n, n_tiles, k_tiles, ep);
     else if (ntw == 1)
-        w8a8_skinny_kernel<MT, 1, 4><<<grid, 256, 0, s>>>(xq, wt, m, n, n_tiles, k_tiles, ep);
+        w8a8_skinny_kernel<MT, 1, 4, false><<<grid, 256, 0, s>>>(xq, wt, m, n, n_tiles, k_tiles, ep);
     else if (waves == 8)
-        w8a8_skinny_kernel<MT, 2, 8><<<grid, 512, 0, s>>>(xq, wt, m, n, n_tiles, k_tiles, ep);
+        w8a8_skinny_kernel<MT, 2, 8, false><<<grid, 512, 0, s>>>(xq, wt, m, n, n_tiles, k_tiles, ep);
     else
-        w8a8_skinny_kernel<MT, 2, 4><<<grid, 256, 0, s>>>(xq, wt, m, n, n_tiles, k_tiles, ep);
+        w8a8_skinny_kernel<MT, 2, 4, false><<<grid, 256, 0, s>>>(xq, wt, m, n, n_tiles, k_tiles, ep);
 }
 
 template <int MT>
@@ -284,11 +329,32 @@ void linear_w8a8_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t 
     uint32_t n_tiles = (uint32_t)(n_pad / 16), k_tiles = (uint32_t)(k_pad / 64);
     int ntw, waves;
     pick_config(n_tiles, k_tiles, num_cus, &ntw, &waves);
-    EpiI8 e{ep.sx, ep.sw, ep.bias, ep.residual, ep.acc_out, ep.out, ep.out_bf16};
+    EpiI8 e{ep.sx, ep.sw, ep.bias, ep.residual, ep.acc_out, ep.out, ep.out_bf16, nullptr};
     if (m <= 16)
         launch_w8a8<1>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e, ntw, waves, s);
     else
         launch_w8a8<2>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e, ntw, waves, s);
+}
+
+void linear_w8a8_swiglu_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, const float *sx, const float *sw,
+                               uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad, float *act, float *pmax,
+                               int waves, hipStream_t s) {
+    if (m == 0 || n == 0) return;
+    uint32_t n_tiles = (uint32_t)(n_pad / 16), k_tiles = (uint32_t)(k_pad / 64);
+    if (g_skinny_waves) waves = g_skinny_waves;
+    EpiI8 e{sx, sw, nullptr, nullptr, nullptr, act, 0, pmax};
+    unsigned grid = n_tiles / 2;
+    if (m <= 16) {
+        if (waves == 8)
+            w8a8_skinny_kernel<1, 2, 8, true><<<grid, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e);
+        else
+            w8a8_skinny_kernel<1, 2, 4, true><<<grid, 256, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e);
+    } else {
+        if (waves == 8)
+            w8a8_skinny_kernel<2, 2, 8, true><<<grid, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e);
+        else
+            w8a8_skinny_kernel<2, 2, 4, true><<<grid, 256, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e);
+    }
 }
 
 void linear_w8a16_skinny(const uint16_t *a, const int8_t *w_tiles, const float *sw, uint64_t m, uint64_t n,

@@ -46,6 +46,10 @@ void rmsnorm_f32(const float *x, const float *w, float *out, uint64_t rows, uint
 // the same byte order as weight tiles, rows >= m zero-filled (m_pad rows).
 void quantize_rows_i8(const void *x, bool in_bf16, int8_t *xq_rowmajor, int8_t *xq_tiled, float *sx,
                       uint64_t m, uint64_t m_pad, uint64_t k, uint64_t k_pad, hipStream_t s);
+// Per-token quantization when the row absmax is already known as `parts` partial maxima per row
+// (pmax[m, parts]): x f32 or bf16 [m, k] -> activation tiles + sx[m].  k a multiple of 64.
+void quantize_rows_from_pmax(const void *x, bool in_bf16, const float *pmax, uint32_t parts, int8_t *xq_tiled,
+                             float *sx, uint64_t m, uint64_t m_pad, uint64_t k, hipStream_t s);
 // RMSNorm fused with the quantizer (f32 in): out_f32 nullable.
 void rmsnorm_quantize_i8(const float *x, const float *w, float eps, float *out_f32, int8_t *xq_tiled,
                          float *sx, uint64_t m, uint64_t m_pad, uint64_t hidden, hipStream_t s);
@@ -87,6 +91,12 @@ struct EpilogueI8 {
 void linear_w8a8_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t m, uint64_t n,
                         uint64_t n_pad, uint64_t k_pad, const EpilogueI8 &ep, int num_cus,
                         hipStream_t s);
+// gate_up projection fused with SwiGLU: the weight is [k, n] with gate columns [0, n/2) and up columns
+// [n/2, n), n/2 a multiple of 16; act[m, n/2] = silu(gate) * up (f32) and pmax[m, n/32] receives the
+// absmax of every 16-column block of act (consumed by quantize_rows_from_pmax).
+void linear_w8a8_swiglu_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, const float *sx, const float *sw,
+                               uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad, float *act, float *pmax,
+                               int waves, hipStream_t s);
 // a: bf16 [m, k] row-major (k == k_pad required), m <= 32.
 void linear_w8a16_skinny(const uint16_t *a, const int8_t *w_tiles, const float *sw, uint64_t m,
                          uint64_t n, uint64_t n_pad, uint64_t k_pad, void *out, int out_bf16,
@@ -123,7 +133,8 @@ uint64_t paged_decode_workspace_bytes(const PagedShape &ps, uint32_t pages_per_c
 void paged_attention_decode_bf16(const uint16_t *q, const uint16_t *k_pool, const uint16_t *v_pool,
                                  const uint32_t *tables, const uint32_t *seq_lens,
                                  const PagedShape &ps, uint32_t pages_per_chunk, void *workspace,
-                                 void *out, int out_bf16, hipStream_t s);
+                                 void *out, int out_bf16, float *pmax /*nullable: [batch, heads] absmax*/,
+                                 hipStream_t s);
 
 // ---- decode-step glue (kern_decoder.hip) --------------------------------------
 // Per step, before the layers: pos[b] = seq_lens[b]; slot[b] from the block

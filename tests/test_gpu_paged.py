@@ -240,7 +240,7 @@ def test_bf16_generic_path_covers_shapes_outside_the_fast_path():
     be = ops()
     rng = o.Rng(31)
     for heads, kv_heads, dh, bs, l_new, ctxs in ((4, 2, 64, 16, 1, [33, 5]), (8, 2, 128, 4, 1, [9, 30]),
-                                                 (4, 4, 128, 16, 3, [20, 20]), (32, 2, 128, 16, 1, [40, 3])):
+                                                 (4, 4, 128, 16, 3, [20, 20]), (32, 1, 128, 16, 1, [40, 3])):
         batch, num_blocks = len(ctxs), 64
         tables, lens, max_blocks, e_kv, e_q = _decode_case(rng, batch, heads, kv_heads, ctxs, num_blocks, dh, bs)
         kp = o.to_bf16(rng.randn((num_blocks, bs, e_kv)))
