@@ -173,6 +173,21 @@ def bench_attention(fa, be, batch, heads, kv_heads, ctxs, num_blocks, iters, see
     return sec, nbytes
 
 
+def bench_copy(fa, be, iters):
+    """Plain row copy (identity gather) of 256 MiB: reads 256 MiB + 256 KiB of indices, writes 256 MiB."""
+    lib = fa.capi.lib
+    rows, cols = 65536, 1024
+    src = be.alloc_uninit((rows, cols))
+    fa.check(lib.fa_fill_normal(be._ctx, src._h, 0, rows * cols, 9, 0.0, 1.0))
+    idx = be.upload(np.arange(rows, dtype=np.int32))
+    dst = be.alloc_uninit((rows, cols))
+    sec = time_launches(fa, be, lambda: fa.check(lib.fa_gather_rows(be._ctx, src._h, rows, cols, idx._h, rows, dst._h)),
+                        iters)
+    for b in (src, idx, dst):
+        b.free()
+    return sec, 2 * rows * cols * 4 + rows * 4
+
+
 def bench_linears(fa, be, iters):
     """Decode-shape int8-weight linears: bf16 activations (W8A16) and W8A8, Llama-7B layer shapes."""
     lib = fa.capi.lib
@@ -285,7 +300,11 @@ def main():
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true")
-    ap.add_argument("--ppc", type=int, default=0, help="tuning: KV pages per attention work item (0 = built-in)")
+    ap.add_argument("--attn-waves", type=int, default=0,
+                    help="tuning: wavefronts per compute unit of the decode attention (0 = built-in)")
+    ap.add_argument("--only", choices=("attention", "copy"), default=None,
+                    help="profiling aid: run only the dominant kernel at the workload's shape, or a plain "
+                         "copy kernel of known size (counter calibration), a few launches, no JSON line")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (--gpus 1); nothing here shards across devices")
@@ -295,10 +314,19 @@ def main():
     info = be.info()
     log("device", info.arch.decode(), "CUs", info.compute_units, "clock_khz", info.clock_khz)
     lib = fa.capi.lib
-    fa.check(lib.fa_set_tuning(2, a.ppc))
+    fa.check(lib.fa_set_tuning(2, a.attn_waves))
     cfg = dict(MODEL, n_layers=a.layers)
     batch = 32
     ctxs = np.random.default_rng(0).integers(1024, 8193, size=batch).tolist()
+    if a.only is not None:
+        mid_ctx = [c + a.warmup + a.steps // 2 for c in ctxs]
+        if a.only == "attention":
+            sec, nb = bench_attention(fa, be, batch, cfg["n_heads"], cfg["n_kv_heads"], mid_ctx, None, 10, seed=4)
+        else:
+            sec, nb = bench_copy(fa, be, 10)
+        log("%s: %.2f us per launch, %d algorithmic bytes, %.0f GB/s" % (a.only, sec * 1e6, nb, nb / sec / 1e9))
+        be.close()
+        return
     t0 = time.time()
     dec, keep, tables, max_blocks, num_blocks = build_decoder(fa, be, cfg, batch, ctxs, a.steps + a.warmup)
     log("model resident in %.1f s; sum ctx = %d" % (time.time() - t0, sum(ctxs)))
@@ -332,7 +360,7 @@ def main():
 
     # dominant operator at this workload's shape: paged decode attention of one layer
     att_sec, att_bytes = bench_attention(fa, be, batch, cfg["n_heads"], cfg["n_kv_heads"], mid_ctx, None, 50, seed=4)
-    roofline = dict(bound="hbm", kernel="paged_attention_decode_bf16 (chunk + merge kernels of one layer)",
+    roofline = dict(bound="hbm", kernel="paged_attention_decode_bf16 (decode_stream_kernel + merge of one layer)",
                     achieved=att_bytes / att_sec / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
                     frac=att_bytes / att_sec / 1e9 / HBM_PEAK_GBS, traffic=None,
                     bytes_per_launch=att_bytes, us_per_launch=att_sec * 1e6)

@@ -14,7 +14,7 @@ namespace fa {
 namespace k {
 extern int g_skinny_ntw, g_skinny_waves;
 }
-int g_decode_ppc = 8;
+int g_decode_waves = 0;
 }  // namespace fa
 
 namespace {
@@ -68,7 +68,7 @@ fa_status fa_set_tuning(int32_t key, int32_t value) {
     switch (key) {
         case 0: k::g_skinny_ntw = value; return FA_OK;
         case 1: k::g_skinny_waves = value; return FA_OK;
-        case 2: fa::g_decode_ppc = value ? value : 8; return FA_OK;
+        case 2: fa::g_decode_waves = value; return FA_OK;
     }
     return fail(FA_ERR_INVALID_ARGUMENT, "fa_set_tuning: unknown key");
 }

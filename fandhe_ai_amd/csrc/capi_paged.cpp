@@ -10,7 +10,7 @@
 using namespace fa;
 
 namespace fa {
-extern int g_decode_ppc;
+extern int g_decode_waves;
 }
 
 namespace {
@@ -54,10 +54,10 @@ fa_status launch_attention(fa_context *ctx, const fa_buffer *q, const fa_buffer 
                            uint64_t s_stride, fa_buffer *out) {
     k::PagedShape ps = make_shape(args);
     if (decode_fast_path(ps, q)) {
-        uint64_t need = k::paged_decode_workspace_bytes(ps, (uint32_t)g_decode_ppc);
+        uint64_t need = k::paged_decode_workspace_bytes(ps, (uint32_t)g_decode_waves);
         if (fa_status s = ensure_workspace(ctx, need)) return s;
         k::paged_attention_decode_bf16((const uint16_t *)q->ptr, (const uint16_t *)k_pool->ptr,
-                                       (const uint16_t *)v_pool->ptr, d_tables, d_lens, ps, (uint32_t)g_decode_ppc,
+                                       (const uint16_t *)v_pool->ptr, d_tables, d_lens, ps, (uint32_t)g_decode_waves,
                                        ctx->workspace, out->ptr, out->dtype == FA_BF16, nullptr, ctx->stream);
         return after_launch(ctx, "paged_attention_decode_bf16");
     }

@@ -15,7 +15,7 @@
 using namespace fa;
 
 namespace fa {
-extern int g_decode_ppc;
+extern int g_decode_waves;
 }
 
 struct fa_decoder {
@@ -37,7 +37,7 @@ struct fa_decoder {
     fa_buffer *attn = nullptr, *act = nullptr, *pmax = nullptr, *logits = nullptr;
     fa_graph *graph = nullptr;
     uint32_t graph_batch = 0;
-    int graph_ppc = 0;
+    int graph_waves = 0;
 };
 
 namespace {
@@ -136,7 +136,7 @@ fa_status enqueue_step(fa_context *ctx, fa_decoder *d) {
                            c.n_heads, c.n_kv_heads, c.head_dim, pool_rows, s);
         k::paged_attention_decode_bf16((const uint16_t *)d->q_bf->ptr, (const uint16_t *)L.k_pool->ptr,
                                        (const uint16_t *)L.v_pool->ptr, (const uint32_t *)d->tables->ptr,
-                                       (const uint32_t *)d->seq_lens->ptr, ps, (uint32_t)g_decode_ppc, ctx->workspace,
+                                       (const uint32_t *)d->seq_lens->ptr, ps, (uint32_t)g_decode_waves, ctx->workspace,
                                        d->attn->ptr, 1, (float *)d->pmax->ptr, s);
         k::quantize_rows_from_pmax(d->attn->ptr, true, (const float *)d->pmax->ptr, c.n_heads, (int8_t *)d->xq->ptr,
                                    (float *)d->sx->ptr, B, m_pad, EQ, s);
@@ -335,9 +335,9 @@ fa_status fa_decoder_step(fa_context *ctx, fa_decoder *d, int32_t use_graph) {
     ps.num_heads = d->cfg.n_heads;
     ps.num_kv_heads = d->cfg.n_kv_heads;
     ps.max_blocks_per_seq = d->cfg.max_blocks_per_seq;
-    if (fa_status s = ensure_workspace(ctx, k::paged_decode_workspace_bytes(ps, (uint32_t)g_decode_ppc))) return s;
+    if (fa_status s = ensure_workspace(ctx, k::paged_decode_workspace_bytes(ps, (uint32_t)g_decode_waves))) return s;
     if (!use_graph) return enqueue_step(ctx, d);
-    if (d->graph && (d->graph_batch != d->batch || d->graph_ppc != g_decode_ppc)) {
+    if (d->graph && (d->graph_batch != d->batch || d->graph_waves != g_decode_waves)) {
         fa_graph_destroy(ctx, d->graph);
         d->graph = nullptr;
     }
@@ -353,7 +353,7 @@ fa_status fa_decoder_step(fa_context *ctx, fa_decoder *d, int32_t use_graph) {
         if (cs != FA_OK) return cs;
         d->graph = g;
         d->graph_batch = d->batch;
-        d->graph_ppc = g_decode_ppc;
+        d->graph_waves = g_decode_waves;
     }
     return fa_graph_launch(ctx, d->graph);
 }

@@ -116,279 +116,335 @@ __global__ void __launch_bounds__(128)
 }
 
 // ------------------------------------------------------- decode fast path
-// Work item = (sequence b, kv head, chunk of PPC pages); one wavefront each,
-// four per block.  Both products run on the matrix cores and the K / V bytes
-// are read once for the whole group of query heads:
+// Both products of the decode attention run on the matrix cores and the K / V
+// bytes are read once for the whole group of query heads:
 //   1. S^T = K Q^T: the K slice of a page (16 tokens x 128 dims, 4 KiB) is
 //      loaded straight into the A operand of v_mfma_f32_16x16x32_bf16 (lane
 //      (g, r): token r, dims 32*s + 8*g .. +7 for step s); Q^T is the B operand
 //      (column = query head of the group).  Lane (g, c) receives the scores of
 //      tokens 4g .. 4g+3 for head c.
-//   2. The scaled, masked scores of the whole chunk stay in registers; the
-//      chunk maximum per head and the exponentials follow.
-//   3. O^T = V^T P^T on v_mfma_f32_16x16x16_bf16: the weights of step 2 are
+//   2. O^T = V^T P^T on v_mfma_f32_16x16x16_bf16: the softmax weights are
 //      already in B-operand order (k = tokens 4g .. 4g+3, column = head); each
 //      f32 weight is split exactly into three bf16 terms (hi + mid + lo) fed
-//      to three instructions, so no precision is lost to the bf16 operand.  V^T needs four tokens of one dim per lane, so the
-//      V page is staged through LDS (row pitch 272 B: conflict-free both for
-//      the 16-byte row writes and for the 4-byte column reads) and every 4-byte
-//      read, holding dims (d, d+1) of one token, serves an even / odd pair of
-//      output rows after a byte permute.
-// The chunk's unnormalized O, its maximum and its sum go to the workspace; a
-// second kernel merges the chunks of a sequence.
+//      to three instructions, so no precision is lost to the bf16 operand.
+//      V^T needs four tokens of one dim per lane, so the V page is staged
+//      through LDS (row pitch 272 B: conflict-free both for the 16-byte row
+//      writes and for the 4-byte column reads) and every 4-byte read, holding
+//      dims (d, d+1) of one token, serves an even / odd pair of output rows
+//      after a byte permute.
 constexpr int kDh = 128, kPage = 16;
 constexpr int kVPitch = 136;            // bf16 elements per staged V row (272 B)
 
 typedef short v4s __attribute__((ext_vector_type(4)));
 
-struct DecodeParams {
+// The pages of all sequences, laid end to end, are cut into n_ranges equal
+// ranges; range r goes to one wavefront per kv head, and the launch is sized so
+// that every wavefront is resident at once and all of them carry the same number
+// of pages whatever the length distribution.  A range that crosses a sequence
+// boundary yields one partial result per sequence it touches; partial (r, b)
+// lives in slot r + b, which is unique because r and b never decrease along
+// the page axis and one of them grows from one partial to the next.
+// Inside a segment the wavefront walks groups of SP pages with a running
+// maximum / sum (the accumulators are rescaled when the maximum grows), and the
+// K and V loads of later pages are always in flight while a group is being
+// multiplied, so the memory pipe never drains between the two products.
+struct StreamParams {
     const uint16_t *q, *k_pool, *v_pool;
     const uint32_t *tables, *seq_lens;
-    float *part_o;      // [items][g_pad][128]
-    float *part_ml;     // [items][2][g_pad]
-    uint32_t num_blocks, e_kv, batch, num_heads, num_kv_heads, group, g_pad, max_blocks_per_seq, max_chunks;
+    float *part_o;      // [slots * num_kv_heads][g_pad][128]
+    float *part_ml;     // [slots * num_kv_heads][2][g_pad]
+    uint32_t num_blocks, e_kv, batch, num_heads, num_kv_heads, group, g_pad, max_blocks_per_seq;
+    uint32_t n_ranges, min_pages;
     float scale;
 };
 
-template <int PPC>
-__global__ void __launch_bounds__(256) decode_chunk_kernel(DecodeParams p) {
-    constexpr int KD = PPC < 4 ? PPC : 4;               // K pages in flight
-    constexpr int VD = PPC < 2 ? PPC : 2;               // V pages in flight
-    // one staging tile per wavefront: LDS operations of a wavefront execute in order, so the column
-    // reads of page i are done before the row writes of page i + 1 land
+__device__ __forceinline__ uint32_t seq_pages(const StreamParams &p, uint32_t b, uint32_t max_ctx) {
+    uint32_t len = p.seq_lens[b];
+    if (len > max_ctx) len = max_ctx;
+    return (len + kPage - 1) / kPage;
+}
+
+// pages per range for this launch: the same value in every wavefront of both kernels
+__device__ __forceinline__ uint32_t range_pages(const StreamParams &p, uint32_t total) {
+    uint32_t per = (total + p.n_ranges - 1) / p.n_ranges;
+    return per < p.min_pages ? p.min_pages : per;
+}
+
+template <int SP, int KD, int VD, int WPE>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) decode_stream_kernel(StreamParams p) {
+    static_assert(SP % KD == 0 && SP % VD == 0, "static register indices need SP to be a multiple of the depths");
     __shared__ __attribute__((aligned(16))) uint16_t v_s[4][kPage * kVPitch];
     const int lane = threadIdx.x % 64;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
     const int g = lane / 16, c = lane % 16;
-    // Work list: item t = (sequence, chunk) pairs that exist, in sequence order, times the kv heads.
-    // The wavefront finds its pair with a prefix sum over the chunk counts of the sequences (64 per
-    // pass, one per lane).  Consecutive blocks hold consecutive items, so the hardware's round-robin
-    // placement of blocks gives every XCD the same share of the bytes whatever the length distribution.
     const uint32_t item_id = blockIdx.x * 4 + wave;
-    const uint32_t kvh = item_id % p.num_kv_heads, t = item_id / p.num_kv_heads;
+    const uint32_t kvh = item_id % p.num_kv_heads, r = item_id / p.num_kv_heads;
+    if (r >= p.n_ranges) return;
     const uint32_t max_ctx = p.max_blocks_per_seq * kPage;
-    uint32_t b = 0, chunk = 0, ctx = 0, base = 0;
-    bool found = false, bad = false;
-    for (uint32_t b0 = 0; b0 < p.batch && !found; b0 += 64) {
+    uint32_t total = 0;
+    for (uint32_t b = lane; b < p.batch; b += 64) total += seq_pages(p, b, max_ctx);
+    total = __builtin_amdgcn_readfirstlane(wave_sum<uint32_t>(total));
+    const uint32_t per = range_pages(p, total);
+    const uint64_t rlo64 = (uint64_t)r * per;
+    if (rlo64 >= total) return;
+    const uint32_t rlo = (uint32_t)rlo64, rhi = rlo + per < total ? rlo + per : total;
+
+    const uint64_t page_elems = (uint64_t)kPage * p.e_kv;
+    const uint64_t k_lane = (uint64_t)c * p.e_kv + (uint64_t)kvh * kDh + 8 * g;       // token c, dims 8g..
+    const uint64_t v_lane = (uint64_t)(4 * g) * p.e_kv + (uint64_t)kvh * kDh + 8 * c;  // tokens 4g.., dims 8c..
+    uint16_t *vs = &v_s[wave][0];
+
+    uint32_t base = 0;
+    for (uint32_t b0 = 0; b0 < p.batch; b0 += 64) {
         uint32_t len = b0 + lane < p.batch ? p.seq_lens[b0 + lane] : 0;
         uint32_t len_c = len > max_ctx ? max_ctx : len;
-        uint32_t nch = ((len_c + kPage - 1) / kPage + PPC - 1) / PPC;
-        uint32_t incl = nch;
+        uint32_t npg = (len_c + kPage - 1) / kPage;
+        uint32_t incl = npg;
 #pragma unroll
         for (int off = 1; off < 64; off <<= 1) {
             uint32_t up = __shfl_up(incl, off, 64);
             if (lane >= off) incl += up;
         }
-        bool hit = t >= base + incl - nch && t < base + incl;
-        uint64_t mask = __ballot(hit);
-        if (mask != 0) {
-            int src = __builtin_ctzll(mask);
-            b = b0 + src;
-            chunk = t - (base + __shfl(incl - nch, src, 64));
-            uint32_t len_src = __shfl(len, src, 64);
-            bad = len_src > max_ctx;
-            ctx = bad ? max_ctx : len_src;
-            found = true;
-        }
+        const uint32_t s_b = base + incl - npg, e_b = base + incl;
+        uint64_t mask = __ballot(npg != 0 && s_b < rhi && e_b > rlo);
         base += __shfl(incl, 63, 64);
-    }
-    if (!found) return;
-    b = __builtin_amdgcn_readfirstlane(b);
-    chunk = __builtin_amdgcn_readfirstlane(chunk);
-    ctx = __builtin_amdgcn_readfirstlane(ctx);
-    const uint32_t p0 = chunk * PPC;
-    const uint32_t *tab = p.tables + (uint64_t)b * p.max_blocks_per_seq + p0;
-    uint32_t raw[PPC];
-#pragma unroll
-    for (int i = 0; i < PPC; ++i) raw[i] = p0 + i < p.max_blocks_per_seq ? tab[i] : 0xffffffffu;
+        while (mask != 0) {
+            const int src = __builtin_ctzll(mask);
+            mask &= mask - 1;
+            const uint32_t b = b0 + src;
+            const uint32_t sb = __builtin_amdgcn_readfirstlane(__shfl(s_b, src, 64));
+            const uint32_t eb = __builtin_amdgcn_readfirstlane(__shfl(e_b, src, 64));
+            const uint32_t len_b = __builtin_amdgcn_readfirstlane(__shfl(len, src, 64));
+            bool bad = len_b > max_ctx;
+            const uint32_t ctx = bad ? max_ctx : len_b;
+            const uint32_t lo = (rlo > sb ? rlo : sb) - sb;            // first page of the segment, in the sequence
+            const uint32_t hi = (rhi < eb ? rhi : eb) - sb;
+            const uint32_t n = hi - lo;                                // pages of this segment (>= 1)
+            const uint32_t *tab = p.tables + (uint64_t)b * p.max_blocks_per_seq + lo;
 
-    // Q^T operand: column c = head of the group (zero beyond the group)
-    v8bf qb[4];
-    {
-        const uint32_t hc = (uint32_t)c < p.group ? (uint32_t)c : 0;
-        const uint16_t *qrow = p.q + ((uint64_t)b * p.num_heads + (uint64_t)kvh * p.group + hc) * kDh + 8 * g;
+            // Q^T operand: column c = head of the group (zero beyond the group)
+            v8bf qb[4];
+            {
+                const uint32_t hc = (uint32_t)c < p.group ? (uint32_t)c : 0;
+                const uint16_t *qrow = p.q + ((uint64_t)b * p.num_heads + (uint64_t)kvh * p.group + hc) * kDh + 8 * g;
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            v4u t = *(const v4u *)(qrow + 32 * s);
-            if ((uint32_t)c >= p.group) t = v4u{0, 0, 0, 0};
-            qb[s] = __builtin_bit_cast(v8bf, t);
-        }
-    }
-
-    const uint32_t n_pages = (ctx + kPage - 1) / kPage;
-    const uint32_t np = n_pages - p0 < (uint32_t)PPC ? n_pages - p0 : (uint32_t)PPC;
-    // positions past the end repeat the last page (their scores are masked): loads stay unconditional
-    uint32_t ids[PPC];
-    {
-        uint32_t cur = 0;
-#pragma unroll
-        for (int i = 0; i < PPC; ++i) {
-            if ((uint32_t)i < np) {
-                cur = raw[i];
-                if (cur >= p.num_blocks) {
-                    bad = true;
-                    cur = 0;
+                for (int s = 0; s < 4; ++s) {
+                    v4u t = *(const v4u *)(qrow + 32 * s);
+                    if ((uint32_t)c >= p.group) t = v4u{0, 0, 0, 0};
+                    qb[s] = __builtin_bit_cast(v8bf, t);
                 }
             }
-            ids[i] = cur;
-        }
-    }
+            // Block ids of 64 pages at a time, one per lane (idv), with the following 64 (idv_next) already
+            // resident.  Everything below is straight-line code per group: loads past the end of the
+            // segment repeat its last page and their scores are masked, and the id windows advance by
+            // selects, so the compiler can count outstanding loads exactly and never drains them at a join.
+            auto tab_at = [&](uint32_t i) -> uint32_t { return tab[i < n ? i : n - 1]; };
+            uint32_t idv = tab_at(lane), idv_next = tab_at(64 + lane);
+            if (__ballot((uint32_t)lane < n && idv >= p.num_blocks) != 0) bad = true;
+            if (idv >= p.num_blocks) idv = 0;
+            uint32_t win = 0;                                          // first page of the id window
+            auto page_id = [&](uint32_t i) -> uint32_t {               // i uniform, win <= i < win + 128
+                const uint32_t ic = i < n ? i : n - 1, rel = ic - win;
+                const uint32_t a = __builtin_amdgcn_readlane(idv, (int)(rel & 63));
+                const uint32_t bnext = __builtin_amdgcn_readlane(idv_next, (int)(rel & 63));
+                uint32_t id = rel < 64 ? a : bnext;
+                return id < p.num_blocks ? id : 0;                     // ids of the next window are checked on use too
+            };
+            auto load_k = [&](uint32_t i, v4u *dst) {
+                const uint16_t *src_p = p.k_pool + (uint64_t)page_id(i) * page_elems + k_lane;
+#pragma unroll
+                for (int s = 0; s < 4; ++s) dst[s] = *(const v4u *)(src_p + 32 * s);
+            };
+            auto load_v = [&](uint32_t i, v4u *dst) {
+                const uint16_t *src_p = p.v_pool + (uint64_t)page_id(i) * page_elems + v_lane;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) dst[j] = *(const v4u *)(src_p + (uint64_t)j * p.e_kv);
+            };
 
-    const uint64_t page_elems = (uint64_t)kPage * p.e_kv;
-    const uint64_t k_lane = (uint64_t)c * p.e_kv + (uint64_t)kvh * kDh + 8 * g;       // token c, dims 8g..
-    const uint64_t v_lane = (uint64_t)(4 * g) * p.e_kv + (uint64_t)kvh * kDh + 8 * c;  // tokens 4g.., dims 8c..
+            // the first requests go out in the order the loop consumes them (oldest first), so that the wait
+            // counts at the loop head are as loose on the first pass as on the later ones
+            v4u kreg[KD][4], vreg[VD][4];
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < KD; ++i) {
+                load_k(i, kreg[i]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int i = 0; i < VD; ++i) {
+                load_v(i, vreg[i]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
 
-    auto load_k = [&](int i, v4u *dst) {
-        const uint16_t *base = p.k_pool + (uint64_t)ids[i] * page_elems + k_lane;
+            float m_run = -INFINITY, l_run = 0.0f;
+            v4f o[8];
 #pragma unroll
-        for (int s = 0; s < 4; ++s) dst[s] = *(const v4u *)(base + 32 * s);
-    };
-    auto load_v = [&](int i, v4u *dst) {
-        const uint16_t *base = p.v_pool + (uint64_t)ids[i] * page_elems + v_lane;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) dst[j] = *(const v4u *)(base + (uint64_t)j * p.e_kv);
-    };
+            for (int t = 0; t < 8; ++t) o[t] = v4f{0.f, 0.f, 0.f, 0.f};
 
-    // ---- pass 1: scores
-    v4u kreg[KD][4];
+            // 64 is a multiple of SP, so a group never straddles two id windows; the loads issued from a
+            // group reach at most max(KD, VD) <= SP pages past it, i.e. at most into the next window
+            for (uint32_t p0 = 0; p0 < n; p0 += SP) {
+                // ids two windows ahead, requested before this group's K / V loads so that consuming
+                // them at the end of the group waits for nothing younger than the loads of the last group
+                const uint32_t cand = tab_at(win + 128 + lane);
+                __builtin_amdgcn_sched_barrier(0);
+                // ---- scores of the group
+                float sc[SP][4];
+                float mx = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < KD; ++i) load_k(i, kreg[i]);
-    float sc[PPC][4];
-    float mx = -INFINITY;
+                for (int i = 0; i < SP; ++i) {
+                    const uint32_t pg = p0 + i;
+                    v4f acc = v4f{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int i = 0; i < PPC; ++i) {
-        v4f acc = v4f{0.f, 0.f, 0.f, 0.f};
+                    for (int s = 0; s < 4; ++s)
+                        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, kreg[i % KD][s]), qb[s],
+                                                                      acc, 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);                 // keep the request right behind its consumer
+                    load_k(pg + KD, kreg[i % KD]);
+                    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int s = 0; s < 4; ++s)
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, kreg[i % KD][s]), qb[s], acc, 0, 0, 0);
-        if (i + KD < PPC) load_k(i + KD, kreg[i % KD]);
+                    for (int j = 0; j < 4; ++j) {
+                        uint32_t tok = (lo + pg) * kPage + 4 * g + j;
+                        float s = pg < n && tok < ctx ? acc[j] * p.scale : -INFINITY;
+                        sc[i][j] = s;
+                        mx = fmaxf(mx, s);
+                    }
+                }
+                // ---- running maximum and sum per head (lanes with equal c hold one head)
+                mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+                const float m_new = fmaxf(m_run, mx);
+                const float alpha = expf(m_run - m_new);               // first group: exp(-inf) = 0
+                m_run = m_new;
+                float gsum = 0.0f;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            uint32_t tok = (p0 + i) * kPage + 4 * g + j;
-            float s = (uint32_t)i < np && tok < ctx ? acc[j] * p.scale : -INFINITY;
-            sc[i][j] = s;
-            mx = fmaxf(mx, s);
-        }
-    }
-    // the first V pages are requested before the softmax arithmetic
-    v4u vreg[VD][4];
+                for (int i = 0; i < SP; ++i)
 #pragma unroll
-    for (int i = 0; i < VD; ++i) load_v(i, vreg[i]);
-
-    // chunk maximum and sum per head: lanes with equal c hold one head
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    float lsum = 0.0f;
+                    for (int j = 0; j < 4; ++j) {
+                        float e = expf(sc[i][j] - m_new);              // masked scores: exp(-inf) = 0
+                        sc[i][j] = e;
+                        gsum += e;
+                    }
+                l_run = __builtin_fmaf(l_run, alpha, gsum);
 #pragma unroll
-    for (int i = 0; i < PPC; ++i)
+                for (int t = 0; t < 8; ++t) o[t] = o[t] * alpha;
+                // ---- O^T += V^T P^T
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            float e = expf(sc[i][j] - mx);              // masked scores: exp(-inf) = 0
-            sc[i][j] = e;
-            lsum += e;
-        }
-    lsum += __shfl_xor(lsum, 16, 64);
-    lsum += __shfl_xor(lsum, 32, 64);
-
-    // ---- pass 2: O^T[d][head] += V^T[d][token] * P^T[token][head]
-    // acc index 2*bp + e covers dims 32*bp + 2*(4g + j) + e, j = 0..3, in lane (g, c)
-    v4f o[8];
+                for (int i = 0; i < SP; ++i) {
+                    const uint32_t pg = p0 + i;
+                    // rows of tokens at or past the sequence end are staged as zeros: their weights are zero,
+                    // but the pool may hold anything there and 0 * NaN must not reach the accumulators
 #pragma unroll
-    for (int t = 0; t < 8; ++t) o[t] = v4f{0.f, 0.f, 0.f, 0.f};
-    uint16_t *vs = &v_s[wave][0];
+                    for (int j = 0; j < 4; ++j) {
+                        uint32_t tok = (lo + pg) * kPage + 4 * g + j;
+                        v4u row = pg < n && tok < ctx ? vreg[i % VD][j] : v4u{0, 0, 0, 0};
+                        *(v4u *)(vs + (4 * g + j) * kVPitch + 8 * c) = row;
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    load_v(pg + VD, vreg[i % VD]);
+                    __builtin_amdgcn_sched_barrier(0);
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                    __builtin_amdgcn_wave_barrier();
+                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                    // each f32 weight as three bf16 operands by repeated truncation: hi + mid + lo == p exactly
+                    uint32_t whi[4], wmid[4], wlo[4];
 #pragma unroll
-    for (int i = 0; i < PPC; ++i) {
-        // stage the page: lane (g, c) owns tokens 4g + j, dims 8c .. 8c + 7
-        // rows of tokens at or past the sequence end are staged as zeros: their weights are zero, but the
-        // pool may hold anything there and 0 * NaN must not reach the accumulators
+                    for (int j = 0; j < 4; ++j) {
+                        float pj = sc[i][j];
+                        whi[j] = __float_as_uint(pj) & 0xffff0000u;
+                        float r1 = pj - __uint_as_float(whi[j]);
+                        wmid[j] = __float_as_uint(r1) & 0xffff0000u;
+                        wlo[j] = __float_as_uint(r1 - __uint_as_float(wmid[j]));
+                    }
+                    v2u ph = v2u{__builtin_amdgcn_perm(whi[1], whi[0], 0x07060302u), __builtin_amdgcn_perm(whi[3], whi[2], 0x07060302u)};
+                    v2u pm = v2u{__builtin_amdgcn_perm(wmid[1], wmid[0], 0x07060302u), __builtin_amdgcn_perm(wmid[3], wmid[2], 0x07060302u)};
+                    v2u pl = v2u{__builtin_amdgcn_perm(wlo[1], wlo[0], 0x07060302u), __builtin_amdgcn_perm(wlo[3], wlo[2], 0x07060302u)};
+                    v4s b_hi = __builtin_bit_cast(v4s, ph), b_mid = __builtin_bit_cast(v4s, pm), b_lo = __builtin_bit_cast(v4s, pl);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            uint32_t tok = (p0 + i) * kPage + 4 * g + j;
-            v4u row = (uint32_t)i < np && tok < ctx ? vreg[i % VD][j] : v4u{0, 0, 0, 0};
-            *(v4u *)(vs + (4 * g + j) * kVPitch + 8 * c) = row;
-        }
-        if (i + VD < PPC) load_v(i + VD, vreg[i % VD]);
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        // each f32 weight as three bf16 operands by repeated truncation: hi + mid + lo == p exactly
-        // (3 x 8 significant bits), so the only rounding left is the f32 accumulation
-        uint32_t hi[4], mid[4], lo[4];
+                    for (int bp = 0; bp < 4; ++bp) {
+                        uint32_t w[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            float pj = sc[i][j];
-            hi[j] = __float_as_uint(pj) & 0xffff0000u;
-            float r1 = pj - __uint_as_float(hi[j]);
-            mid[j] = __float_as_uint(r1) & 0xffff0000u;
-            lo[j] = __float_as_uint(r1 - __uint_as_float(mid[j]));
-        }
-        v2u ph = v2u{__builtin_amdgcn_perm(hi[1], hi[0], 0x07060302u), __builtin_amdgcn_perm(hi[3], hi[2], 0x07060302u)};
-        v2u pm = v2u{__builtin_amdgcn_perm(mid[1], mid[0], 0x07060302u), __builtin_amdgcn_perm(mid[3], mid[2], 0x07060302u)};
-        v2u pl = v2u{__builtin_amdgcn_perm(lo[1], lo[0], 0x07060302u), __builtin_amdgcn_perm(lo[3], lo[2], 0x07060302u)};
-        v4s b_hi = __builtin_bit_cast(v4s, ph), b_mid = __builtin_bit_cast(v4s, pm), b_lo = __builtin_bit_cast(v4s, pl);
+                        for (int j = 0; j < 4; ++j) w[j] = *(const uint32_t *)(vs + (4 * g + j) * kVPitch + 32 * bp + 2 * c);
+                        v2u ae = v2u{__builtin_amdgcn_perm(w[1], w[0], 0x05040100u), __builtin_amdgcn_perm(w[3], w[2], 0x05040100u)};
+                        v2u ao = v2u{__builtin_amdgcn_perm(w[1], w[0], 0x07060302u), __builtin_amdgcn_perm(w[3], w[2], 0x07060302u)};
+                        v4s a_even = __builtin_bit_cast(v4s, ae), a_odd = __builtin_bit_cast(v4s, ao);
+                        // smallest terms first
+                        o[2 * bp] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_even, b_lo, o[2 * bp], 0, 0, 0);
+                        o[2 * bp + 1] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_odd, b_lo, o[2 * bp + 1], 0, 0, 0);
+                        o[2 * bp] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_even, b_mid, o[2 * bp], 0, 0, 0);
+                        o[2 * bp + 1] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_odd, b_mid, o[2 * bp + 1], 0, 0, 0);
+                        o[2 * bp] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_even, b_hi, o[2 * bp], 0, 0, 0);
+                        o[2 * bp + 1] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_odd, b_hi, o[2 * bp + 1], 0, 0, 0);
+                    }
+                }
+                // advance the id windows when the next group starts a new one
+                const bool adv = p0 + SP >= win + 64;
+                if (adv && __ballot(win + 64 + lane < n && idv_next >= p.num_blocks) != 0) bad = true;
+                idv = adv ? idv_next : idv;
+                idv_next = adv ? cand : idv_next;
+                win = adv ? win + 64 : win;
+            }
+            l_run += __shfl_xor(l_run, 16, 64);
+            l_run += __shfl_xor(l_run, 32, 64);
+            // lane (g, c) holds, for head c: dims 32 bp + 8 g + {0..7} = {o[2bp][0], o[2bp+1][0], o[2bp][1], ...}
+            const uint64_t item = (uint64_t)(r + b) * p.num_kv_heads + kvh;
+            if ((uint32_t)c < p.group) {
+                float *po = p.part_o + (item * p.g_pad + c) * kDh + 8 * g;
 #pragma unroll
-        for (int bp = 0; bp < 4; ++bp) {
-            // dims (32 bp + 2c, +1) of tokens 4g .. 4g + 3
-            uint32_t w[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) w[j] = *(const uint32_t *)(vs + (4 * g + j) * kVPitch + 32 * bp + 2 * c);
-            v2u ae = v2u{__builtin_amdgcn_perm(w[1], w[0], 0x05040100u), __builtin_amdgcn_perm(w[3], w[2], 0x05040100u)};
-            v2u ao = v2u{__builtin_amdgcn_perm(w[1], w[0], 0x07060302u), __builtin_amdgcn_perm(w[3], w[2], 0x07060302u)};
-            v4s a_even = __builtin_bit_cast(v4s, ae), a_odd = __builtin_bit_cast(v4s, ao);
-            // smallest terms first
-            o[2 * bp] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_even, b_lo, o[2 * bp], 0, 0, 0);
-            o[2 * bp + 1] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_odd, b_lo, o[2 * bp + 1], 0, 0, 0);
-            o[2 * bp] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_even, b_mid, o[2 * bp], 0, 0, 0);
-            o[2 * bp + 1] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_odd, b_mid, o[2 * bp + 1], 0, 0, 0);
-            o[2 * bp] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_even, b_hi, o[2 * bp], 0, 0, 0);
-            o[2 * bp + 1] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_odd, b_hi, o[2 * bp + 1], 0, 0, 0);
-        }
-    }
-    // lane (g, c) holds, for head c: dims 32 bp + 8 g + {0..7} = {o[2bp][0], o[2bp+1][0], o[2bp][1], ...}
-    const uint64_t item = ((uint64_t)b * p.num_kv_heads + kvh) * p.max_chunks + chunk;
-    if ((uint32_t)c < p.group) {
-        float *po = p.part_o + (item * p.g_pad + c) * kDh + 8 * g;
-#pragma unroll
-        for (int bp = 0; bp < 4; ++bp) {
-            *(v4f *)(po + 32 * bp) = v4f{o[2 * bp][0], o[2 * bp + 1][0], o[2 * bp][1], o[2 * bp + 1][1]};
-            *(v4f *)(po + 32 * bp + 4) = v4f{o[2 * bp][2], o[2 * bp + 1][2], o[2 * bp][3], o[2 * bp + 1][3]};
-        }
-        if (g == 0) {
-            float nanv = __uint_as_float(0x7fc00000u);
-            p.part_ml[item * (2 * p.g_pad) + c] = bad ? nanv : mx;
-            p.part_ml[item * (2 * p.g_pad) + p.g_pad + c] = bad ? nanv : lsum;
+                for (int bp = 0; bp < 4; ++bp) {
+                    *(v4f *)(po + 32 * bp) = v4f{o[2 * bp][0], o[2 * bp + 1][0], o[2 * bp][1], o[2 * bp + 1][1]};
+                    *(v4f *)(po + 32 * bp + 4) = v4f{o[2 * bp][2], o[2 * bp + 1][2], o[2 * bp][3], o[2 * bp + 1][3]};
+                }
+                if (g == 0) {
+                    float nanv = __uint_as_float(0x7fc00000u);
+                    p.part_ml[item * (2 * p.g_pad) + c] = bad ? nanv : m_run;
+                    p.part_ml[item * (2 * p.g_pad) + p.g_pad + c] = bad ? nanv : l_run;
+                }
+            }
         }
     }
 }
 
-// Merges the chunks of one (sequence, query head).  Block = 256 threads: thread
-// (part, d) sums every second chunk for dim d, then the two parts are added.
-template <int PPC>
-__global__ void __launch_bounds__(256) decode_merge_kernel(DecodeParams p, void *__restrict__ out, int out_bf16,
-                                                          float *__restrict__ pmax) {
+// Merges the partial results of one (sequence, query head): block = 256 threads,
+// thread (part, d) sums every second partial for dim d, then the two parts are added.
+__global__ void __launch_bounds__(256) decode_stream_merge_kernel(StreamParams p, void *__restrict__ out, int out_bf16,
+                                                                 float *__restrict__ pmax) {
     __shared__ float s_acc[128], s_den, s_max[2];
+    __shared__ uint32_t s_tot[4], s_pre[4];
     const uint32_t h = blockIdx.x, b = blockIdx.y, d = threadIdx.x % 128, part = threadIdx.x / 128;
     const uint32_t kvh = h / p.group, hg = h % p.group;
-    uint32_t ctx = p.seq_lens[b];
-    uint32_t max_ctx = p.max_blocks_per_seq * kPage;
-    if (ctx > max_ctx) ctx = max_ctx;
-    const uint32_t n_pages = (ctx + kPage - 1) / kPage;
-    const uint32_t n_chunks = (n_pages + PPC - 1) / PPC;
-    const uint64_t item0 = ((uint64_t)b * p.num_kv_heads + kvh) * p.max_chunks;
-    const float *ml = p.part_ml + item0 * (2 * p.g_pad) + hg;
+    const uint32_t max_ctx = p.max_blocks_per_seq * kPage;
+    uint32_t tot = 0, pre = 0;
+    for (uint32_t bb = threadIdx.x; bb < p.batch; bb += 256) {
+        uint32_t v = seq_pages(p, bb, max_ctx);
+        tot += v;
+        if (bb < b) pre += v;
+    }
+    tot = (uint32_t)wave_sum<uint32_t>(tot);
+    pre = (uint32_t)wave_sum<uint32_t>(pre);
+    if (threadIdx.x % 64 == 0) {
+        s_tot[threadIdx.x / 64] = tot;
+        s_pre[threadIdx.x / 64] = pre;
+    }
+    __syncthreads();
+    tot = s_tot[0] + s_tot[1] + s_tot[2] + s_tot[3];
+    pre = s_pre[0] + s_pre[1] + s_pre[2] + s_pre[3];
+    const uint32_t npg = seq_pages(p, b, max_ctx);
+    const uint32_t per = range_pages(p, tot);
+    const uint32_t r_lo = npg ? pre / per : 1, r_hi = npg ? (pre + npg - 1) / per : 0;   // empty sequence: no partials
     float mx = -INFINITY;
-    for (uint32_t ch = 0; ch < n_chunks; ++ch) {
-        float m = ml[(uint64_t)ch * (2 * p.g_pad)];
+    for (uint32_t r = r_lo; r <= r_hi; ++r) {
+        float m = p.part_ml[((uint64_t)(r + b) * p.num_kv_heads + kvh) * (2 * p.g_pad) + hg];
         mx = (m != m || mx != mx) ? __uint_as_float(0x7fc00000u) : fmaxf(mx, m);   // NaN marks a violation
     }
     float acc = 0.0f, den = 0.0f;
-    const float *po = p.part_o + (item0 * p.g_pad + hg) * kDh + d;
-    for (uint32_t ch = part; ch < n_chunks; ch += 2) {
-        float m = ml[(uint64_t)ch * (2 * p.g_pad)];
-        float l = ml[(uint64_t)ch * (2 * p.g_pad) + p.g_pad];
+    for (uint32_t r = r_lo + part; r <= r_hi; r += 2) {
+        const uint64_t item = (uint64_t)(r + b) * p.num_kv_heads + kvh;
+        float m = p.part_ml[item * (2 * p.g_pad) + hg];
+        float l = p.part_ml[item * (2 * p.g_pad) + p.g_pad + hg];
         float w = expf(m - mx);
         den = __builtin_fmaf(w, l, den);
-        acc = __builtin_fmaf(w, po[(uint64_t)ch * p.g_pad * kDh], acc);
+        acc = __builtin_fmaf(w, p.part_o[(item * p.g_pad + hg) * kDh + d], acc);
     }
     if (part == 1) {
         s_acc[d] = acc;
@@ -399,16 +455,16 @@ __global__ void __launch_bounds__(256) decode_merge_kernel(DecodeParams p, void 
     if (part == 0) {
         acc += s_acc[d];
         den += s_den;
-        float r = n_chunks == 0 ? 0.0f : __fdiv_rn(acc, den);
-        uint64_t o = ((uint64_t)b * p.num_heads + h) * kDh + d;
+        float res = npg == 0 ? 0.0f : __fdiv_rn(acc, den);
+        uint64_t oi = ((uint64_t)b * p.num_heads + h) * kDh + d;
         if (out_bf16) {
-            uint16_t rb = f32_to_bf16(r);
-            ((uint16_t *)out)[o] = rb;
-            r = bf16_to_f32(rb);
+            uint16_t rb = f32_to_bf16(res);
+            ((uint16_t *)out)[oi] = rb;
+            res = bf16_to_f32(rb);
         } else {
-            ((float *)out)[o] = r;
+            ((float *)out)[oi] = res;
         }
-        a = fabsf(r);
+        a = fabsf(res);
     }
     if (pmax) {                      // absmax of the stored head slice, for the quantizer that follows
         a = wave_max(a);
@@ -422,15 +478,6 @@ inline int group_pad(uint32_t group) {
     int gp = 1;
     while ((uint32_t)gp < group) gp *= 2;
     return gp;
-}
-
-template <int PPC>
-void launch_decode(const DecodeParams &p, void *out, int out_bf16, float *pmax, hipStream_t s) {
-    // upper bound of the work list; wavefronts past its real end exit at once
-    uint64_t items = (uint64_t)p.batch * p.num_kv_heads * p.max_chunks;
-    decode_chunk_kernel<PPC><<<(unsigned)((items + 3) / 4), 256, 0, s>>>(p);
-    dim3 grid2(p.num_heads, p.batch);
-    decode_merge_kernel<PPC><<<grid2, 256, 0, s>>>(p, out, out_bf16, pmax);
 }
 
 }  // namespace
@@ -466,48 +513,65 @@ void paged_attention_generic(const void *q, const void *k_pool, const void *v_po
                                                                           workspace, s_stride, out);
 }
 
-static uint32_t normalize_ppc(uint32_t ppc) { return ppc == 4 || ppc == 16 ? ppc : 8; }
+static uint32_t compute_units() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, v = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+            cus = v;
+        else
+            cus = 256;
+    }
+    return (uint32_t)cus;
+}
 
-uint64_t paged_decode_workspace_bytes(const PagedShape &ps, uint32_t pages_per_chunk) {
-    uint32_t ppc = normalize_ppc(pages_per_chunk);
+// Ranges of the streamed kernel: one wavefront per (range, kv head), `waves_per_cu` of them on every
+// compute unit, all resident at once.  Four per compute unit (one per SIMD) measured best: longer
+// ranges mean fewer partial results, and the loads in flight per wavefront already cover the latency.
+static uint32_t stream_ranges(const PagedShape &ps, uint32_t waves_per_cu) {
+    if (waves_per_cu == 0) waves_per_cu = 4;
+    if (waves_per_cu > 8) waves_per_cu = 8;               // register budget of the kernel: two per SIMD
+    uint32_t r = compute_units() * waves_per_cu / ps.num_kv_heads;
+    return r ? r : 1;
+}
+
+uint64_t paged_decode_workspace_bytes(const PagedShape &ps, uint32_t waves_per_cu) {
     uint32_t group = ps.num_heads / ps.num_kv_heads;
     uint64_t gp = (uint64_t)group_pad(group);
-    uint64_t max_chunks = ((uint64_t)ps.max_blocks_per_seq + ppc - 1) / ppc;
-    uint64_t items = (uint64_t)ps.batch * ps.num_kv_heads * max_chunks;
+    uint64_t items = ((uint64_t)stream_ranges(ps, waves_per_cu) + ps.batch) * ps.num_kv_heads;
     return items * (gp * kDh + 2 * gp) * sizeof(float);
 }
 
 void paged_attention_decode_bf16(const uint16_t *q, const uint16_t *k_pool, const uint16_t *v_pool,
                                  const uint32_t *tables, const uint32_t *seq_lens, const PagedShape &ps,
-                                 uint32_t pages_per_chunk, void *workspace, void *out, int out_bf16, float *pmax,
+                                 uint32_t waves_per_cu, void *workspace, void *out, int out_bf16, float *pmax,
                                  hipStream_t s) {
     if (ps.batch == 0) return;
-    uint32_t ppc = normalize_ppc(pages_per_chunk);
-    DecodeParams p;
-    p.q = q;
-    p.k_pool = k_pool;
-    p.v_pool = v_pool;
-    p.tables = tables;
-    p.seq_lens = seq_lens;
-    p.num_blocks = ps.num_blocks;
-    p.e_kv = ps.e_kv;
-    p.batch = ps.batch;
-    p.num_heads = ps.num_heads;
-    p.num_kv_heads = ps.num_kv_heads;
-    p.group = ps.num_heads / ps.num_kv_heads;
-    p.max_blocks_per_seq = ps.max_blocks_per_seq;
-    p.max_chunks = (ps.max_blocks_per_seq + ppc - 1) / ppc;
-    p.scale = ps.scale;
-    int gp = group_pad(p.group);
-    p.g_pad = (uint32_t)gp;
-    uint64_t items = (uint64_t)ps.batch * ps.num_kv_heads * p.max_chunks;
-    p.part_o = (float *)workspace;
-    p.part_ml = p.part_o + items * (uint64_t)gp * kDh;
-    switch (ppc) {
-        case 4: launch_decode<4>(p, out, out_bf16, pmax, s); break;
-        case 16: launch_decode<16>(p, out, out_bf16, pmax, s); break;
-        default: launch_decode<8>(p, out, out_bf16, pmax, s); break;
-    }
+    StreamParams sp;
+    sp.q = q;
+    sp.k_pool = k_pool;
+    sp.v_pool = v_pool;
+    sp.tables = tables;
+    sp.seq_lens = seq_lens;
+    sp.num_blocks = ps.num_blocks;
+    sp.e_kv = ps.e_kv;
+    sp.batch = ps.batch;
+    sp.num_heads = ps.num_heads;
+    sp.num_kv_heads = ps.num_kv_heads;
+    sp.group = ps.num_heads / ps.num_kv_heads;
+    sp.g_pad = (uint32_t)group_pad(sp.group);
+    sp.max_blocks_per_seq = ps.max_blocks_per_seq;
+    sp.n_ranges = stream_ranges(ps, waves_per_cu);
+    sp.min_pages = 4;
+    sp.scale = ps.scale;
+    uint64_t items = ((uint64_t)sp.n_ranges + ps.batch) * ps.num_kv_heads;
+    sp.part_o = (float *)workspace;
+    sp.part_ml = sp.part_o + items * (uint64_t)sp.g_pad * kDh;
+    uint64_t waves = (uint64_t)sp.n_ranges * ps.num_kv_heads;
+    decode_stream_kernel<4, 4, 2, 2><<<(unsigned)((waves + 3) / 4), 256, 0, s>>>(sp);
+    dim3 grid2(ps.num_heads, ps.batch);
+    decode_stream_merge_kernel<<<grid2, 256, 0, s>>>(sp, out, out_bf16, pmax);
 }
 
 }  // namespace k

@@ -129,10 +129,10 @@ void paged_attention_generic(const void *q, const void *k_pool, const void *v_po
                              hipStream_t s);
 // Decode fast path: bf16, head_dim 128, block_size 16, l_new 1, group <= 16.
 // Workspace bytes needed for a given shape:
-uint64_t paged_decode_workspace_bytes(const PagedShape &ps, uint32_t pages_per_chunk);
+uint64_t paged_decode_workspace_bytes(const PagedShape &ps, uint32_t waves_per_cu);
 void paged_attention_decode_bf16(const uint16_t *q, const uint16_t *k_pool, const uint16_t *v_pool,
                                  const uint32_t *tables, const uint32_t *seq_lens,
-                                 const PagedShape &ps, uint32_t pages_per_chunk, void *workspace,
+                                 const PagedShape &ps, uint32_t waves_per_cu, void *workspace,
                                  void *out, int out_bf16, float *pmax /*nullable: [batch, heads] absmax*/,
                                  hipStream_t s);
 

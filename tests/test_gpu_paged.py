@@ -157,10 +157,10 @@ def test_bf16_gqa_decode_against_the_oracle(heads, kv_heads):
     o.set_threads(1)
     assert rc == 0
     dq, dk, dv = be.upload(q), be.upload(kp), be.upload(vp)
-    for ppc in (4, 8, 16):
+    for ppc in (0, 1, 2, 8):          # wavefronts per compute unit: ranges of many / few pages
         fa.check(fa.capi.lib.fa_set_tuning(2, ppc))
         got = be.download_owned(be.paged_attention_forward(dq, dk, dv, tables, lens, args, out_dtype=fa.capi.F32))
-        assert_parity("PAGED_DECODE_PARITY", f"H{heads}/{kv_heads}:ppc{ppc}", got, want)
+        assert_parity("PAGED_DECODE_PARITY", f"H{heads}/{kv_heads}:waves{ppc}", got, want)
         got_bf = be.download_owned(be.paged_attention_forward(dq, dk, dv, tables, lens, args))
         assert_bf16_rounding_of("paged decode bf16", got_bf, got)
     fa.check(fa.capi.lib.fa_set_tuning(2, 0))
@@ -215,6 +215,13 @@ def test_bf16_decode_properties_at_benchmark_size():
     o.set_threads(1)
     assert rc == 0
     assert_parity("PAGED_DECODE_PARITY", "bench:sampled", got[sample], want)
+    # other launch shapes (1 and 8 wavefronts per compute unit: ranges of several hundred / a few dozen pages)
+    for tune in (1, 8):
+        fa.check(fa.capi.lib.fa_set_tuning(2, tune))
+        alt = be.download_owned(be.paged_attention_forward(dq, dk, dv, tables, lens, args, out_dtype=fa.capi.F32))
+        assert_parity("PAGED_DECODE_PARITY", f"bench:sampled:tune{tune}", alt[sample], want)
+        assert np.allclose(alt, got, rtol=2e-3, atol=2e-5)
+    fa.check(fa.capi.lib.fa_set_tuning(2, 0))
     # every output row is a convex combination of V rows: |out| <= max |V| per dim of its kv head
     vmax = np.abs(o.from_bf16(vp[used])).reshape(-1, kv_heads, 128).max(axis=0)
     assert np.all(np.abs(got.reshape(batch, heads, 128)) <= np.repeat(vmax, heads // kv_heads, axis=0)[None] + 1e-6)
