@@ -188,6 +188,29 @@ def bench_copy(fa, be, iters):
     return sec, 2 * rows * cols * 4 + rows * 4
 
 
+def bench_w8a8_decode(fa, be, cfg, m, iters):
+    """W8A8 linears of one decoder layer at the step's batch (dynamic per-token quantizer + int8 GEMV)."""
+    lib = fa.capi.lib
+    D, F = cfg["d_model"], cfg["d_ffn"]
+    EQ, EKV = cfg["n_heads"] * cfg["head_dim"], cfg["n_kv_heads"] * cfg["head_dim"]
+    res = []
+    for k, n in ((D, EQ + 2 * EKV), (EQ, D), (D, 2 * F), (F, D)):
+        w = be.alloc_uninit((k, n))
+        fa.check(lib.fa_fill_normal(be._ctx, w._h, 0, k * n, k + n, 0.0, 0.02))
+        qw = be.quantize_weight(fa.DeviceBufferView(w, 0, (k, n)))
+        w.free()
+        x = be.alloc_uninit((m, k))
+        fa.check(lib.fa_fill_normal(be._ctx, x._h, 0, m * k, 5, 0.0, 1.0))
+        out = be.alloc_uninit((m, n))
+        sec = time_launches(fa, be, lambda: fa.check(lib.fa_linear_w8a8(be._ctx, x._h, m, qw._h, None, 0, None, out._h)),
+                            iters)
+        nbytes = k * n + 4 * n + m * k + 4 * m * n
+        res.append(dict(op="w8a8", m=m, k=k, n=n, us=sec * 1e6, gbs=nbytes / sec / 1e9))
+        for b in (x, out, qw):
+            b.free()
+    return res
+
+
 def bench_linears(fa, be, iters):
     """Decode-shape int8-weight linears: bf16 activations (W8A16) and W8A8, Llama-7B layer shapes."""
     lib = fa.capi.lib
@@ -302,7 +325,9 @@ def main():
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--attn-waves", type=int, default=0,
                     help="tuning: wavefronts per compute unit of the decode attention (0 = built-in)")
-    ap.add_argument("--only", choices=("attention", "copy"), default=None,
+    ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
+                    help="tuning: raw fa_set_tuning key/value pairs (experiments)")
+    ap.add_argument("--only", choices=("attention", "copy", "linears"), default=None,
                     help="profiling aid: run only the dominant kernel at the workload's shape, or a plain "
                          "copy kernel of known size (counter calibration), a few launches, no JSON line")
     a = ap.parse_args()
@@ -315,11 +340,20 @@ def main():
     log("device", info.arch.decode(), "CUs", info.compute_units, "clock_khz", info.clock_khz)
     lib = fa.capi.lib
     fa.check(lib.fa_set_tuning(2, a.attn_waves))
+    for kv in a.tune:
+        key, value = kv.split("=")
+        fa.check(lib.fa_set_tuning(int(key), int(value)))
     cfg = dict(MODEL, n_layers=a.layers)
     batch = 32
     ctxs = np.random.default_rng(0).integers(1024, 8193, size=batch).tolist()
     if a.only is not None:
         mid_ctx = [c + a.warmup + a.steps // 2 for c in ctxs]
+        if a.only == "linears":
+            for r in bench_w8a8_decode(fa, be, cfg, batch, 20):
+                log("w8a8 m=%d %5d->%5d: %.2f us per call (quantizer + GEMV), %.0f GB/s" %
+                    (r["m"], r["k"], r["n"], r["us"], r["gbs"]))
+            be.close()
+            return
         if a.only == "attention":
             sec, nb = bench_attention(fa, be, batch, cfg["n_heads"], cfg["n_kv_heads"], mid_ctx, None, 10, seed=4)
         else:

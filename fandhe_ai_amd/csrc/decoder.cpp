@@ -33,7 +33,7 @@ struct fa_decoder {
     uint32_t batch = 0;
     // resident state and activations
     fa_buffer *tokens = nullptr, *tables = nullptr, *seq_lens = nullptr, *pos = nullptr, *slots = nullptr;
-    fa_buffer *cos_sin = nullptr, *h = nullptr, *xq = nullptr, *sx = nullptr, *qkv = nullptr, *q_bf = nullptr;
+    fa_buffer *cos_sin = nullptr, *h = nullptr, *xq = nullptr, *sx = nullptr, *q_bf = nullptr;
     fa_buffer *attn = nullptr, *act = nullptr, *pmax = nullptr, *logits = nullptr;
     fa_graph *graph = nullptr;
     uint32_t graph_batch = 0;
@@ -70,7 +70,7 @@ fa_status check_vec(const fa_decoder *d, const fa_buffer *b, uint64_t numel, con
 
 void free_all(fa_context *ctx, fa_decoder *d) {
     fa_buffer **bufs[] = {&d->tokens, &d->tables, &d->seq_lens, &d->pos, &d->slots, &d->cos_sin, &d->h, &d->xq,
-                          &d->sx,     &d->qkv,    &d->q_bf,     &d->attn, &d->act,  &d->pmax, &d->logits};
+                          &d->sx,     &d->q_bf,     &d->attn, &d->act,  &d->pmax, &d->logits};
     for (auto pb : bufs) {
         if (*pb) fa_buffer_free(ctx, *pb);
         *pb = nullptr;
@@ -130,10 +130,14 @@ fa_status enqueue_step(fa_context *ctx, fa_decoder *d) {
         const fa_decoder::Layer &L = d->layers[li];
         k::rmsnorm_quantize_i8((const float *)d->h->ptr, (const float *)L.attn_norm->ptr, c.rms_eps, nullptr,
                                (int8_t *)d->xq->ptr, (float *)d->sx->ptr, B, m_pad, D, s);
-        linear(L.wqkv, d->qkv->ptr, nullptr);
-        k::qkv_rope_append((const float *)d->qkv->ptr, (const float *)d->cos_sin->ptr, (const uint32_t *)d->slots->ptr,
-                           (uint16_t *)d->q_bf->ptr, (uint16_t *)L.k_pool->ptr, (uint16_t *)L.v_pool->ptr, B,
-                           c.n_heads, c.n_kv_heads, c.head_dim, pool_rows, s);
+        {
+            k::QkvRopeTargets t{(const float *)d->cos_sin->ptr, (const uint32_t *)d->slots->ptr, (uint16_t *)d->q_bf->ptr,
+                                (uint16_t *)L.k_pool->ptr, (uint16_t *)L.v_pool->ptr, c.n_heads, c.n_kv_heads,
+                                c.head_dim, pool_rows};
+            k::linear_w8a8_qkv_rope_skinny((const int8_t *)d->xq->ptr, (const int8_t *)L.wqkv->codes->ptr,
+                                           (const float *)d->sx->ptr, (const float *)L.wqkv->scales->ptr, B,
+                                           L.wqkv->n_pad, L.wqkv->k_pad, t, s);
+        }
         k::paged_attention_decode_bf16((const uint16_t *)d->q_bf->ptr, (const uint16_t *)L.k_pool->ptr,
                                        (const uint16_t *)L.v_pool->ptr, (const uint32_t *)d->tables->ptr,
                                        (const uint32_t *)d->seq_lens->ptr, ps, (uint32_t)g_decode_waves, ctx->workspace,
@@ -191,7 +195,7 @@ fa_status fa_decoder_create(fa_context *ctx, const fa_decoder_config *cfg, fa_de
     d->cfg = c;
     d->layers.resize(c.n_layers);
     const uint64_t B = c.max_batch, D = c.d_model, F = c.d_ffn, V = c.vocab;
-    const uint64_t EQ = (uint64_t)c.n_heads * c.head_dim, EKV = (uint64_t)c.n_kv_heads * c.head_dim;
+    const uint64_t EQ = (uint64_t)c.n_heads * c.head_dim;
     const uint64_t kmax = std::max(std::max(D, F), EQ);
     fa_status s = FA_OK;
     auto mk = [&](fa_dtype t, uint64_t n, fa_buffer **b) {
@@ -206,7 +210,6 @@ fa_status fa_decoder_create(fa_context *ctx, const fa_decoder_config *cfg, fa_de
     mk(FA_F32, B * D, &d->h);
     mk(FA_I8, round_up(B, 16) * kmax, &d->xq);
     mk(FA_F32, B, &d->sx);
-    mk(FA_F32, B * (EQ + 2 * EKV), &d->qkv);
     mk(FA_BF16, B * EQ, &d->q_bf);
     mk(FA_BF16, B * EQ, &d->attn);
     mk(FA_F32, B * F, &d->act);

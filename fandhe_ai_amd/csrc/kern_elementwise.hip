@@ -28,18 +28,6 @@ __global__ void silu_mul_kernel(const float *__restrict__ gate, const float *__r
     for (; i < n; i += stride) out[i] = silu(gate[i]) * up[i];
 }
 
-__global__ void swiglu_rows_kernel(const float *__restrict__ gu, float *__restrict__ out, uint64_t rows,
-                                   uint64_t f) {
-    uint64_t total = rows * f;
-    uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
-    for (; i < total; i += stride) {
-        uint64_t r = i / f, c = i - r * f;
-        const float *row = gu + r * 2 * f;
-        out[i] = silu(row[c]) * row[f + c];
-    }
-}
-
 __global__ void add_kernel(const float *__restrict__ a, const float *__restrict__ b, float *__restrict__ out,
                            uint64_t n) {
     uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -172,10 +160,6 @@ inline unsigned grid_for(uint64_t n, unsigned block, unsigned cap = 65535u * 4u)
 void silu_mul_f32(const float *gate, const float *up, float *out, uint64_t n, hipStream_t s) {
     if (n == 0) return;
     silu_mul_kernel<<<grid_for(n, 256), 256, 0, s>>>(gate, up, out, n);
-}
-void swiglu_rows_f32(const float *gu, float *out, uint64_t rows, uint64_t f, hipStream_t s) {
-    if (rows * f == 0) return;
-    swiglu_rows_kernel<<<grid_for(rows * f, 256), 256, 0, s>>>(gu, out, rows, f);
 }
 void add_f32(const float *a, const float *b, float *out, uint64_t n, hipStream_t s) {
     if (n == 0) return;

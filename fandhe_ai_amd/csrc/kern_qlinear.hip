@@ -22,7 +22,15 @@ struct EpiI8 {
     void *out;
     int out_bf16;
     float *pmax;          // SwiGLU mode: per (row, block) absmax of the activation
+    // RoPE mode (fused q/k/v projection of a decode step)
+    const float *cos_sin;     // [m][head_dim]: cos of the row's position for i < head_dim/2, then sin
+    const uint32_t *slots;    // [m] cache row of the new token
+    uint16_t *q_out, *k_pool, *v_pool;
+    uint32_t heads, kv_heads, head_dim;
+    uint64_t pool_rows;
 };
+
+enum { kEpiPlain = 0, kEpiSwiglu = 1, kEpiRope = 2 };
 
 // crates/tensor-core/src/scalar_op.rs:666-673 / :355
 __device__ __forceinline__ float silu_f32(float x) {
@@ -42,16 +50,24 @@ __device__ __forceinline__ float silu_f32(float x) {
 // SWIGLU: the weight holds gate columns [0, n/2) and up columns [n/2, n); the block multiplies the
 // gate tile blockIdx.x and the up tile of the same columns and writes act = silu(gate) * up
 // ([m, n/2] f32) plus the block's per-row absmax, so that the next quantizer needs no pass over gate|up.
-template <int MT, int NTW, int NWAVES, bool SWIGLU>
+// ROPE (mode 2): the weight is the fused q | k | v projection; the block multiplies tile a and tile
+// a + head_dim/32 of one head, i.e. the two halves that the rotation pairs, rotates q and k heads by the
+// row's position (products rounded separately, no contraction), rounds once to bf16 and stores q rows
+// and the new K / V cache rows directly, so the f32 projection never reaches memory.
+template <int MT, int NTW, int NWAVES, int MODE>
 __global__ void __launch_bounds__(NWAVES * 64)
     w8a8_skinny_kernel(const int8_t *__restrict__ xq_tiled, const int8_t *__restrict__ w_tiles, uint32_t m,
                        uint32_t n, uint32_t n_tiles, uint32_t k_tiles, EpiI8 ep) {
-    static_assert(!SWIGLU || NTW == 2, "SwiGLU pairs one gate tile with one up tile");
+    constexpr bool SWIGLU = MODE == kEpiSwiglu, ROPE = MODE == kEpiRope;
+    static_assert(MODE == kEpiPlain || NTW == 2, "the fused epilogues pair two tiles");
     constexpr int NACC = MT * NTW * 4;
     __shared__ int red[NWAVES][NACC][64];
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
-    const uint32_t nt0 = SWIGLU ? blockIdx.x : blockIdx.x * NTW;
-    const uint32_t nt_step = SWIGLU ? n_tiles / 2 : 1;
+    const uint32_t half_tiles = ROPE ? ep.head_dim / 32 : 0;
+    const uint32_t nt0 = SWIGLU ? blockIdx.x
+                         : ROPE ? (blockIdx.x / half_tiles) * 2 * half_tiles + blockIdx.x % half_tiles
+                                : blockIdx.x * NTW;
+    const uint32_t nt_step = SWIGLU ? n_tiles / 2 : ROPE ? half_tiles : 1;
 
     v4i acc[MT][NTW];
 #pragma unroll
@@ -134,6 +150,50 @@ __global__ void __launch_bounds__(NWAVES * 64)
 #pragma unroll
             for (int off = 1; off < 16; off <<= 1) a = fmaxf(a, __shfl_xor(a, off, 64));
             if (lane % 16 == 0 && row < m) ep.pmax[(uint64_t)row * (n_tiles / 2) + nt0] = a;
+        }
+        return;
+    }
+    if constexpr (ROPE) {
+        const uint32_t half = ep.head_dim / 2;
+        const uint32_t eq = ep.heads * ep.head_dim, ekv = ep.kv_heads * ep.head_dim;
+        for (int q = wave; q < MT * 4; q += NWAVES) {
+            int i = q / 4, e = q % 4;
+            int s0 = 0, s1 = 0;
+#pragma unroll
+            for (int w = 0; w < NWAVES; ++w) {
+                s0 += red[w][(i * 2 + 0) * 4 + e][lane];
+                s1 += red[w][(i * 2 + 1) * 4 + e][lane];
+            }
+            const uint32_t row = i * 16 + 4 * (lane / 16) + e;
+            const uint32_t col = nt0 * 16 + lane % 16;             // first half of the head; partner at col + half
+            if (row < m && col + half < n) {
+                float x0 = __fmul_rn((float)s0, __fmul_rn(ep.sx[row], ep.sw[col]));
+                float x1 = __fmul_rn((float)s1, __fmul_rn(ep.sx[row], ep.sw[col + half]));
+                const uint32_t h = col / ep.head_dim, d = col % ep.head_dim;
+                uint16_t *dst = nullptr;
+                if (h < ep.heads) {
+                    dst = ep.q_out + (uint64_t)row * eq + (uint64_t)h * ep.head_dim + d;
+                } else {
+                    const uint64_t slot = ep.slots[row];
+                    if (slot < ep.pool_rows) {
+                        const uint32_t hk = h - ep.heads;
+                        dst = (hk < ep.kv_heads ? ep.k_pool + slot * ekv + (uint64_t)hk * ep.head_dim
+                                                : ep.v_pool + slot * ekv + (uint64_t)(hk - ep.kv_heads) * ep.head_dim) + d;
+                    }
+                }
+                if (h < ep.heads + ep.kv_heads) {
+                    const float c = ep.cos_sin[(uint64_t)row * ep.head_dim + d];
+                    const float sn = ep.cos_sin[(uint64_t)row * ep.head_dim + half + d];
+                    const float r0 = __fsub_rn(__fmul_rn(x0, c), __fmul_rn(x1, sn));
+                    const float r1 = __fadd_rn(__fmul_rn(x1, c), __fmul_rn(x0, sn));
+                    x0 = r0;
+                    x1 = r1;
+                }
+                if (dst) {
+                    dst[0] = f32_to_bf16(x0);
+                    dst[half] = f32_to_bf16(x1);
+                }
+            }
         }
         return;
     }
@@ -298,13 +358,13 @@ void launch_w8a8(const int8_t *xq, const int8_t *wt, uint32_t m, uint32_t n, uin
                  const EpiI8 &ep, int ntw, int waves, hipStream_t s) {
     unsigned grid = (n_tiles + ntw - 1) / ntw;
     if (ntw == 1 && waves == 8)
-        w8a8_skinny_kernel<MT, 1, 8, false><<<grid, 512, 0, s>>>(xq, wt, m, n, n_tiles, k_tiles, ep);
+        w8a8_skinny_kernel<MT, 1, 8, kEpiPlain><<<grid, 512, 0, s>>>(xq, wt, m, n, n_tiles, k_tiles, ep);
     else if (ntw == 1)
-        w8a8_skinny_kernel<MT, 1, 4, false><<<grid, 256, 0, s>>>(xq, wt, m, n, n_tiles, k_tiles, ep);
+        w8a8_skinny_kernel<MT, 1, 4, kEpiPlain><<<grid, 256, 0, s>>>(xq, wt, m, n, n_tiles, k_tiles, ep);
     else if (waves == 8)
-        w8a8_skinny_kernel<MT, 2, 8, false><<<grid, 512, 0, s>>>(xq, wt, m, n, n_tiles, k_tiles, ep);
+        w8a8_skinny_kernel<MT, 2, 8, kEpiPlain><<<grid, 512, 0, s>>>(xq, wt, m, n, n_tiles, k_tiles, ep);
     else
-        w8a8_skinny_kernel<MT, 2, 4, false><<<grid, 256, 0, s>>>(xq, wt, m, n, n_tiles, k_tiles, ep);
+        w8a8_skinny_kernel<MT, 2, 4, kEpiPlain><<<grid, 256, 0, s>>>(xq, wt, m, n, n_tiles, k_tiles, ep);
 }
 
 template <int MT>
@@ -329,7 +389,14 @@ void linear_w8a8_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t 
     uint32_t n_tiles = (uint32_t)(n_pad / 16), k_tiles = (uint32_t)(k_pad / 64);
     int ntw, waves;
     pick_config(n_tiles, k_tiles, num_cus, &ntw, &waves);
-    EpiI8 e{ep.sx, ep.sw, ep.bias, ep.residual, ep.acc_out, ep.out, ep.out_bf16, nullptr};
+    EpiI8 e{};
+    e.sx = ep.sx;
+    e.sw = ep.sw;
+    e.bias = ep.bias;
+    e.residual = ep.residual;
+    e.acc_out = ep.acc_out;
+    e.out = ep.out;
+    e.out_bf16 = ep.out_bf16;
     if (m <= 16)
         launch_w8a8<1>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e, ntw, waves, s);
     else
@@ -342,18 +409,54 @@ void linear_w8a8_swiglu_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, co
     if (m == 0 || n == 0) return;
     uint32_t n_tiles = (uint32_t)(n_pad / 16), k_tiles = (uint32_t)(k_pad / 64);
     if (g_skinny_waves) waves = g_skinny_waves;
-    EpiI8 e{sx, sw, nullptr, nullptr, nullptr, act, 0, pmax};
+    EpiI8 e{};
+    e.sx = sx;
+    e.sw = sw;
+    e.out = act;
+    e.pmax = pmax;
     unsigned grid = n_tiles / 2;
     if (m <= 16) {
         if (waves == 8)
-            w8a8_skinny_kernel<1, 2, 8, true><<<grid, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e);
+            w8a8_skinny_kernel<1, 2, 8, kEpiSwiglu><<<grid, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e);
         else
-            w8a8_skinny_kernel<1, 2, 4, true><<<grid, 256, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e);
+            w8a8_skinny_kernel<1, 2, 4, kEpiSwiglu><<<grid, 256, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e);
     } else {
         if (waves == 8)
-            w8a8_skinny_kernel<2, 2, 8, true><<<grid, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e);
+            w8a8_skinny_kernel<2, 2, 8, kEpiSwiglu><<<grid, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e);
         else
-            w8a8_skinny_kernel<2, 2, 4, true><<<grid, 256, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e);
+            w8a8_skinny_kernel<2, 2, 4, kEpiSwiglu><<<grid, 256, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e);
+    }
+}
+
+void linear_w8a8_qkv_rope_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, const float *sx, const float *sw,
+                                 uint64_t m, uint64_t n_pad, uint64_t k_pad, const QkvRopeTargets &t, hipStream_t s) {
+    if (m == 0) return;
+    uint32_t n = (t.heads + 2 * t.kv_heads) * t.head_dim;
+    uint32_t n_tiles = (uint32_t)(n_pad / 16), k_tiles = (uint32_t)(k_pad / 64);
+    EpiI8 e{};
+    e.sx = sx;
+    e.sw = sw;
+    e.cos_sin = t.cos_sin;
+    e.slots = t.slots;
+    e.q_out = t.q_out;
+    e.k_pool = t.k_pool;
+    e.v_pool = t.v_pool;
+    e.heads = t.heads;
+    e.kv_heads = t.kv_heads;
+    e.head_dim = t.head_dim;
+    e.pool_rows = t.pool_rows;
+    unsigned grid = n / 32;                                  // one block per pair of 16-column tiles
+    int waves = g_skinny_waves ? g_skinny_waves : 8;
+    if (m <= 16) {
+        if (waves == 8)
+            w8a8_skinny_kernel<1, 2, 8, kEpiRope><<<grid, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, n, n_tiles, k_tiles, e);
+        else
+            w8a8_skinny_kernel<1, 2, 4, kEpiRope><<<grid, 256, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, n, n_tiles, k_tiles, e);
+    } else {
+        if (waves == 8)
+            w8a8_skinny_kernel<2, 2, 8, kEpiRope><<<grid, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, n, n_tiles, k_tiles, e);
+        else
+            w8a8_skinny_kernel<2, 2, 4, kEpiRope><<<grid, 256, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, n, n_tiles, k_tiles, e);
     }
 }
 

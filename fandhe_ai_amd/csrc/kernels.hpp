@@ -23,8 +23,6 @@ constexpr int kTileKF8 = 128;   // e4m3 k-values per tile
 
 // ---- elementwise / small ops (kern_elementwise.hip) ------------------------
 void silu_mul_f32(const float *gate, const float *up, float *out, uint64_t n, hipStream_t s);
-// SwiGLU on a [rows, 2*f] gate|up matrix -> [rows, f]
-void swiglu_rows_f32(const float *gu, float *out, uint64_t rows, uint64_t f, hipStream_t s);
 void add_f32(const float *a, const float *b, float *out, uint64_t n, hipStream_t s);
 void argmax_rows_f32(const float *x, int32_t *out, uint64_t rows, uint64_t cols, hipStream_t s);
 void gather_rows_f32(const float *table, uint64_t table_rows, uint64_t cols, const int32_t *idx,
@@ -97,6 +95,19 @@ void linear_w8a8_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t 
 void linear_w8a8_swiglu_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, const float *sx, const float *sw,
                                uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad, float *act, float *pmax,
                                int waves, hipStream_t s);
+// Fused q | k | v projection of a decode step: the weight is [k, (heads + 2 kv_heads) head_dim], head_dim a
+// multiple of 32; q and k heads are rotated (rotate-half pairing, cos/sin of the row's position from
+// cos_sin[m][head_dim]) and rounded once to bf16; q goes to q_out [m, heads * head_dim], the new K / V rows
+// to pool row slots[r] (rows whose slot is out of range are skipped).
+struct QkvRopeTargets {
+    const float *cos_sin;
+    const uint32_t *slots;
+    uint16_t *q_out, *k_pool, *v_pool;
+    uint32_t heads, kv_heads, head_dim;
+    uint64_t pool_rows;
+};
+void linear_w8a8_qkv_rope_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, const float *sx, const float *sw,
+                                 uint64_t m, uint64_t n_pad, uint64_t k_pad, const QkvRopeTargets &t, hipStream_t s);
 // a: bf16 [m, k] row-major (k == k_pad required), m <= 32.
 void linear_w8a16_skinny(const uint16_t *a, const int8_t *w_tiles, const float *sw, uint64_t m,
                          uint64_t n, uint64_t n_pad, uint64_t k_pad, void *out, int out_bf16,
@@ -143,15 +154,6 @@ void paged_attention_decode_bf16(const uint16_t *q, const uint16_t *k_pool, cons
 void decode_prepare(const uint32_t *tables, uint32_t *seq_lens, int32_t *pos, uint32_t *slots, float *cos_sin,
                     uint32_t batch, uint32_t block_size, uint32_t max_blocks_per_seq, uint32_t num_blocks,
                     uint32_t head_dim, double theta, hipStream_t s);
-// Splits qkv[b, (H + 2 Hkv) Dh] (f32): RoPE on q and k with the cos/sin table,
-// one rounding to bf16; q -> q_out[b, H Dh]; k, v -> pool rows slot[b].
-void qkv_rope_append(const float *qkv, const float *cos_sin, const uint32_t *slots, uint16_t *q_out,
-                     uint16_t *k_pool, uint16_t *v_pool, uint32_t batch, uint32_t heads, uint32_t kv_heads,
-                     uint32_t head_dim, uint64_t pool_rows, hipStream_t s);
-// act = silu(gate) * up on gu[m, 2f] followed by per-token int8 quantization
-// into activation tiles (f must be a multiple of 64).
-void swiglu_quantize_i8(const float *gu, int8_t *xq_tiled, float *sx, uint64_t m, uint64_t m_pad, uint64_t f,
-                        hipStream_t s);
 
 }  // namespace k
 }  // namespace fa
