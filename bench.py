@@ -29,6 +29,10 @@ sys.path.insert(0, ROOT)
 METRIC = "int8/fp8 GEMM TOPS + decode tok/s (bs32, paged-KV) and % roofline, 1 GPU"
 HBM_PEAK_GBS = 8000.0
 MFMA_PEAK_TOPS = 5000.0          # dense int8 and fp8 on MI355X
+# HBM bytes per launch of decode_stream_kernel at this benchmark's shape, from hardware counters
+# (rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE, each scaled by the same counter's reading for a plain
+# row-copy kernel of known size; the figures are in profiles/decode_stream_kernel_config5_pmc.txt).
+ATTENTION_TRAFFIC_BYTES = 627609598
 U32MAX = 0xFFFFFFFF
 
 MODEL = dict(n_layers=32, d_model=4096, n_heads=32, n_kv_heads=8, head_dim=128, d_ffn=14336, vocab=32000,
@@ -148,7 +152,7 @@ def attention_bytes(sum_ctx, ctxs, heads, kv_heads, head_dim=128, bs=16):
 
 
 # ------------------------------------------------------------------ operators
-def bench_attention(fa, be, batch, heads, kv_heads, ctxs, num_blocks, iters, seed):
+def bench_attention(fa, be, batch, heads, kv_heads, ctxs, num_blocks, iters, seed, kernel_only=False):
     lib = fa.capi.lib
     rng = np.random.default_rng(seed)
     tables, max_blocks, num_blocks = make_tables(rng, ctxs, 0, 16, num_blocks)
@@ -168,9 +172,17 @@ def bench_attention(fa, be, batch, heads, kv_heads, ctxs, num_blocks, iters, see
                                                        C.byref(args), out._h))
     sec = time_launches(fa, be, launch, iters)
     nbytes = attention_bytes(int(np.sum(ctxs)), ctxs, heads, kv_heads)
+    sec_kernel = None
+    if kernel_only:
+        # the streaming kernel by itself (its merge kernel is not launched, the output stays unwritten)
+        fa.check(lib.fa_set_tuning(3, 1))
+        try:
+            sec_kernel = time_launches(fa, be, launch, iters)
+        finally:
+            fa.check(lib.fa_set_tuning(3, 0))
     for b in (kp, vp, q, d_tables, d_lens, out):
         b.free()
-    return sec, nbytes
+    return (sec, nbytes, sec_kernel) if kernel_only else (sec, nbytes)
 
 
 def bench_copy(fa, be, iters):
@@ -355,7 +367,9 @@ def main():
             be.close()
             return
         if a.only == "attention":
-            sec, nb = bench_attention(fa, be, batch, cfg["n_heads"], cfg["n_kv_heads"], mid_ctx, None, 10, seed=4)
+            sec, nb, sec_k = bench_attention(fa, be, batch, cfg["n_heads"], cfg["n_kv_heads"], mid_ctx, None, 10, seed=4,
+                                             kernel_only=True)
+            log("attention streaming kernel alone: %.2f us per launch, %.0f GB/s" % (sec_k * 1e6, nb / sec_k / 1e9))
         else:
             sec, nb = bench_copy(fa, be, 10)
         log("%s: %.2f us per launch, %d algorithmic bytes, %.0f GB/s" % (a.only, sec * 1e6, nb, nb / sec / 1e9))
@@ -393,11 +407,17 @@ def main():
     be.release_cached_device_memory()
 
     # dominant operator at this workload's shape: paged decode attention of one layer
-    att_sec, att_bytes = bench_attention(fa, be, batch, cfg["n_heads"], cfg["n_kv_heads"], mid_ctx, None, 50, seed=4)
-    roofline = dict(bound="hbm", kernel="paged_attention_decode_bf16 (decode_stream_kernel + merge of one layer)",
-                    achieved=att_bytes / att_sec / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
-                    frac=att_bytes / att_sec / 1e9 / HBM_PEAK_GBS, traffic=None,
-                    bytes_per_launch=att_bytes, us_per_launch=att_sec * 1e6)
+    att_sec, att_bytes, att_kernel_sec = bench_attention(fa, be, batch, cfg["n_heads"], cfg["n_kv_heads"], mid_ctx,
+                                                         None, 50, seed=4, kernel_only=True)
+    # Dominant kernel: decode_stream_kernel of the paged attention (about 60 % of the step).  Its launch
+    # is timed by itself; the whole operator (that kernel + the merge of the partial results) is given
+    # beside it.  traffic: HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE of this kernel at
+    # this shape, scaled by a copy kernel of known size (profiles/decode_stream_kernel_config5_pmc.txt).
+    roofline = dict(bound="hbm", kernel="decode_stream_kernel (paged GQA decode attention, one layer)",
+                    achieved=att_bytes / att_kernel_sec / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
+                    frac=att_bytes / att_kernel_sec / 1e9 / HBM_PEAK_GBS, traffic=ATTENTION_TRAFFIC_BYTES,
+                    bytes_per_launch=att_bytes, us_per_launch=att_kernel_sec * 1e6,
+                    operator_us=att_sec * 1e6, operator_achieved=att_bytes / att_sec / 1e9)
     extras = {"step_algorithmic_gb": bytes_step / 1e9, "step_hbm_frac": bytes_step / sec_per_step / 1e9 / HBM_PEAK_GBS}
     if not a.no_extras:
         c3 = np.random.default_rng(0).integers(128, 4097, size=64).tolist()

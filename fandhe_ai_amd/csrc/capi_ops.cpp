@@ -15,6 +15,7 @@ namespace k {
 extern int g_skinny_ntw, g_skinny_waves;
 }
 int g_decode_waves = 0;
+extern int g_decode_partials_only;
 }  // namespace fa
 
 namespace {
@@ -63,12 +64,14 @@ extern "C" {
 
 // Tuning knobs for experiments (0 restores the built-in choice):
 // key 0 = n-tiles per block of the skinny linears, 1 = wavefronts per block,
-// 2 = pages per chunk of the decode attention.
+// 2 = wavefronts per compute unit of the decode attention, 3 = decode attention launches its streaming
+// kernel only (timing aid).
 fa_status fa_set_tuning(int32_t key, int32_t value) {
     switch (key) {
         case 0: k::g_skinny_ntw = value; return FA_OK;
         case 1: k::g_skinny_waves = value; return FA_OK;
         case 2: fa::g_decode_waves = value; return FA_OK;
+        case 3: fa::g_decode_partials_only = value; return FA_OK;
     }
     return fail(FA_ERR_INVALID_ARGUMENT, "fa_set_tuning: unknown key");
 }

@@ -513,6 +513,10 @@ void paged_attention_generic(const void *q, const void *k_pool, const void *v_po
                                                                           workspace, s_stride, out);
 }
 
+}  // namespace k
+int g_decode_partials_only = 0;   // profiling: launch only the streaming kernel (the output is not written)
+namespace k {
+
 static uint32_t compute_units() {
     static int cus = 0;
     if (cus == 0) {
@@ -570,6 +574,7 @@ void paged_attention_decode_bf16(const uint16_t *q, const uint16_t *k_pool, cons
     sp.part_ml = sp.part_o + items * (uint64_t)sp.g_pad * kDh;
     uint64_t waves = (uint64_t)sp.n_ranges * ps.num_kv_heads;
     decode_stream_kernel<4, 4, 2, 2><<<(unsigned)((waves + 3) / 4), 256, 0, s>>>(sp);
+    if (g_decode_partials_only) return;
     dim3 grid2(ps.num_heads, ps.batch);
     decode_stream_merge_kernel<<<grid2, 256, 0, s>>>(sp, out, out_bf16, pmax);
 }
