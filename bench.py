@@ -61,14 +61,32 @@ class Timer:
 
 
 def time_launches(fa, be, fn, iters, warmup=5):
+    """Seconds per launch of fn, from HIP events on the library's stream.  The launches are recorded
+    into one HIP graph and the graph is replayed, so that the host's per-call cost (several microseconds
+    through ctypes) does not show in kernels that take only a few microseconds."""
+    lib = fa.capi.lib
     for _ in range(warmup):
         fn()
     be.synchronize_device()
-    t = Timer(fa, be)
-    t.start()
-    for _ in range(iters):
-        fn()
-    return t.stop_ms() / iters * 1e-3        # seconds per launch
+    graph = C.c_void_p()
+    fa.check(lib.fa_graph_capture_begin(be._ctx))
+    try:
+        for _ in range(iters):
+            fn()
+    finally:
+        st = lib.fa_graph_capture_end(be._ctx, C.byref(graph))
+    fa.check(st)
+    try:
+        fa.check(lib.fa_graph_launch(be._ctx, graph))
+        be.synchronize_device()
+        reps = 3
+        t = Timer(fa, be)
+        t.start()
+        for _ in range(reps):
+            fa.check(lib.fa_graph_launch(be._ctx, graph))
+        return t.stop_ms() / (iters * reps) * 1e-3
+    finally:
+        lib.fa_graph_destroy(be._ctx, graph)
 
 
 def make_tables(rng, ctxs, extra_tokens, bs, num_blocks=None):
@@ -339,7 +357,7 @@ def main():
                     help="tuning: wavefronts per compute unit of the decode attention (0 = built-in)")
     ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
                     help="tuning: raw fa_set_tuning key/value pairs (experiments)")
-    ap.add_argument("--only", choices=("attention", "copy", "linears"), default=None,
+    ap.add_argument("--only", choices=("attention", "copy", "linears", "prefill"), default=None,
                     help="profiling aid: run only the dominant kernel at the workload's shape, or a plain "
                          "copy kernel of known size (counter calibration), a few launches, no JSON line")
     a = ap.parse_args()
@@ -360,6 +378,12 @@ def main():
     ctxs = np.random.default_rng(0).integers(1024, 8193, size=batch).tolist()
     if a.only is not None:
         mid_ctx = [c + a.warmup + a.steps // 2 for c in ctxs]
+        if a.only == "prefill":
+            for r in bench_prefill(fa, be, 20):
+                log("%s m=%d k=%d n=%d: %.1f us, %.0f TOPS (%.1f %% of peak)" %
+                    (r["op"], r["m"], r["k"], r["n"], r["us"], r["tops"], 100 * r["frac"]))
+            be.close()
+            return
         if a.only == "linears":
             for r in bench_w8a8_decode(fa, be, cfg, batch, 20):
                 log("w8a8 m=%d %5d->%5d: %.2f us per call (quantizer + GEMV), %.0f GB/s" %

@@ -12,7 +12,7 @@ using namespace fa;
 
 namespace fa {
 namespace k {
-extern int g_skinny_ntw, g_skinny_waves;
+extern int g_skinny_ntw, g_skinny_waves, g_gemm_small_tiles;
 }
 int g_decode_waves = 0;
 extern int g_decode_partials_only;
@@ -65,13 +65,14 @@ extern "C" {
 // Tuning knobs for experiments (0 restores the built-in choice):
 // key 0 = n-tiles per block of the skinny linears, 1 = wavefronts per block,
 // 2 = wavefronts per compute unit of the decode attention, 3 = decode attention launches its streaming
-// kernel only (timing aid).
+// kernel only (timing aid), 4 = prefill GEMMs keep the 128 x 128 block tile for every shape.
 fa_status fa_set_tuning(int32_t key, int32_t value) {
     switch (key) {
         case 0: k::g_skinny_ntw = value; return FA_OK;
         case 1: k::g_skinny_waves = value; return FA_OK;
         case 2: fa::g_decode_waves = value; return FA_OK;
         case 3: fa::g_decode_partials_only = value; return FA_OK;
+        case 4: k::g_gemm_small_tiles = value; return FA_OK;
     }
     return fail(FA_ERR_INVALID_ARGUMENT, "fa_set_tuning: unknown key");
 }
@@ -302,7 +303,7 @@ fa_status fa_linear_w8a8(fa_context *ctx, const fa_buffer *x, uint64_t m, const 
         k::quantize_rows_i8(x->ptr, x->dtype == FA_BF16, (int8_t *)xq.ptr, nullptr, (float *)sx.ptr, m, m, qw->k,
                             qw->k_pad, ctx->stream);
         k::gemm_w8a8_mfma((const int8_t *)xq.ptr, (const int8_t *)qw->codes->ptr, m, qw->n, qw->n_pad, qw->k_pad, ep,
-                          ctx->stream);
+                          ctx->props.multiProcessorCount, ctx->stream);
     }
     return after_launch(ctx, "linear_w8a8");
 }
@@ -330,7 +331,7 @@ fa_status fa_gemm_w8a8(fa_context *ctx, const fa_buffer *aq, const fa_buffer *sx
     ep.out = out->ptr;
     ep.out_bf16 = out->dtype == FA_BF16;
     k::gemm_w8a8_mfma((const int8_t *)aq->ptr, (const int8_t *)qw->codes->ptr, m, qw->n, qw->n_pad, qw->k_pad, ep,
-                      ctx->stream);
+                      ctx->props.multiProcessorCount, ctx->stream);
     return after_launch(ctx, "gemm_w8a8_mfma");
 }
 
@@ -376,7 +377,7 @@ fa_status fa_gemm_e4m3(fa_context *ctx, const fa_buffer *aq, const fa_buffer *a_
     if (m > (1ull << 22)) return fail(FA_ERR_INVALID_ARGUMENT, "gemm_e4m3: m too large for one launch");
     k::gemm_e4m3_mfma((const uint8_t *)aq->ptr, (const uint8_t *)qw->codes->ptr, (const float *)a_scale->ptr,
                       (const float *)qw->scales->ptr, m, qw->n, qw->n_pad, qw->k_pad, out->ptr, out->dtype == FA_BF16,
-                      ctx->stream);
+                      ctx->props.multiProcessorCount, ctx->stream);
     return after_launch(ctx, "gemm_e4m3_mfma");
 }
 

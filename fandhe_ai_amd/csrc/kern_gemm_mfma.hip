@@ -15,6 +15,8 @@ namespace fa {
 namespace k {
 using namespace fa::dev;
 
+int g_gemm_small_tiles = 0;   // tuning: nonzero keeps the 128 x 128 kernel for every shape
+
 namespace {
 
 struct EpiI8 {
@@ -178,21 +180,337 @@ __global__ void __launch_bounds__(256)
             }
 }
 
+// Matrix instructions with the accumulator pinned to the accumulation registers ("+a"): with 256
+// accumulator registers per lane the register allocator otherwise shuffles tiles between the two
+// register files around every instruction.  Same instructions as the builtins emit.  volatile keeps
+// them in program order, ahead of the drain that precedes the epilogue.
+__device__ __forceinline__ void mfma_acc(v4i &c, const v4i &a, const v4i &b) {
+    asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mfma_acc(v4f &c, const v8i &a, const v8i &b) {
+    const int unit = 0x7f7f7f7f;                      // block scales 2^0
+    asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %3 op_sel_hi:[0,0,0]"
+                 : "+a"(c)
+                 : "v"(a), "v"(b), "v"(unit));
+}
+
+// ------------------------------------------------------------ large tiles
+// Block tile 256 rows x NTB * 16 columns, four wavefronts in 2 x 2, one per
+// SIMD, each owning 128 rows x NTB / 2 column tiles of accumulators (up to 256
+// registers).  Per k-step a wavefront reads 8 A fragments once and streams its
+// B fragments past them, so the LDS traffic per matrix instruction is a quarter
+// of the 64 x 64 wavefront tile above, which is what lets the matrix cores run
+// instead of waiting on LDS.  Rows / tiles past the edge are loaded from a
+// clamped address (never stored), so the main loop has no predicated loads.
+// The block index is remapped so that the blocks that land on one XCD (the
+// hardware deals consecutive block ids round-robin over the 8 XCDs) are
+// consecutive tiles, m fastest: they share one B panel and walk k together,
+// which keeps the panel in that XCD's L2.
+template <bool FP8, int NTB, typename Epi>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+    gemm_mfma_big_kernel(const uint8_t *__restrict__ aq, const uint8_t *__restrict__ w_tiles, uint32_t m, uint32_t n,
+                         uint32_t n_tiles, uint32_t k_steps, uint32_t m_blocks, uint32_t n_blocks, Epi ep) {
+    // One stage is 128 bytes of k for both types: one e4m3 instruction step, or two int8 steps (two
+    // adjacent 1 KiB weight tiles).  Fewer, larger stages halve the per-stage fixed cost (barrier, load
+    // issue, first fragment reads) for int8 and let its A rows be fetched as whole 128-byte lines.
+    constexpr int TK = 128, TILE = 2048;             // bytes of k per stage; bytes per operand tile and stage
+    constexpr int WNT = NTB / 2;                     // column tiles per wavefront
+    constexpr int A_STAGE = 16 * TILE, B_STAGE = NTB * TILE, STAGE = A_STAGE + B_STAGE;
+    constexpr int NST = 2;                           // stages in LDS
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];   // [NST][A_STAGE + B_STAGE]
+
+    const int tid = threadIdx.x, lane = tid % 64;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
+    const int wm = wave / 2, wn = wave % 2;
+    uint32_t bid = blockIdx.x;
+    const uint32_t total = m_blocks * n_blocks;
+    if (total % 8 == 0) bid = (bid % 8) * (total / 8) + bid / 8;
+    const uint32_t mb = bid % m_blocks, nb = bid / m_blocks;
+    const uint32_t m0 = mb * 256, nt0 = nb * NTB;
+    const uint64_t k_bytes = (uint64_t)k_steps * TK;
+
+    // Global -> LDS without passing through registers: one load instruction moves 16 bytes per lane to
+    // LDS base + lane * 16, i.e. one 1 KiB slice of an operand tile in the matrix instruction's lane
+    // order; a tile of a stage is two slices h = 0, 1.  e4m3: slice h holds bytes 16 h .. 16 h + 15 of every
+    // lane's 32-byte chunk.  int8: slice h is the operand tile of k-step h of the stage.
+    // Wavefront w moves tiles w, w + 4, w + 8, w + 12 of A and of B.  Rows / tiles past the edge are loaded
+    // from a clamped address and never stored.
+    // A rows are row-major in memory: a row's 128 bytes of a stage are eight 16-byte pieces q.  Load
+    // instruction x takes the pieces with q % 2 == x, four consecutive lanes sharing one row, so every
+    // lane quad touches one whole cache line per instruction (the L1 fetches it once; the second
+    // instruction hits) instead of one line per lane.  Lane 4 r + p fills LDS slot 4 r + p of slice x
+    // with piece q = 2 ((p - r / 2) mod 4) + x: the rotation by r / 2 spreads the fragment reads of eight
+    // consecutive rows over all LDS banks.
+    // e4m3: k-group g of the matrix instruction is pieces 2 g, 2 g + 1, i.e. slot 4 r + (g + r / 2) mod 4
+    // of both slices.  int8: k-group g of k-step s is piece q = 4 s + g, i.e. slice q % 2, slot
+    // 4 r + (q / 2 + r / 2) mod 4.
+    constexpr int B_L = FP8 ? 32 : 16, B_H = FP8 ? 16 : 1024;    // byte offsets of lane l and slice h in a tile
+    const uint8_t *a_src[4];
+    const uint8_t *b_src[4];
+    {
+        const int r = lane / 4, p4 = lane % 4;
+        const int pp = (p4 - r / 2) & 3;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            uint32_t row = m0 + (wave + 4 * i) * 16 + r;
+            row = row < m ? row : m - 1;
+            a_src[i] = aq + (uint64_t)row * k_bytes + pp * 32;
+            uint32_t t = nt0 + wave + 4 * i;
+            t = t < n_tiles ? t : n_tiles - 1;
+            b_src[i] = w_tiles + (uint64_t)t * k_steps * TILE + lane * B_L;
+        }
+    }
+    // byte offsets of this lane's two A operand reads inside a tile
+    int a_off[2];
+    {
+        const int g = lane / 16, r = lane % 16;
+        if constexpr (FP8) {
+            a_off[0] = (4 * r + ((g + r / 2) & 3)) * 16;
+            a_off[1] = a_off[0] + 1024;
+        } else {
+#pragma unroll
+            for (int sub = 0; sub < 2; ++sub) {
+                const int q = 4 * sub + g;
+                a_off[sub] = (q & 1) * 1024 + (4 * r + (((q >> 1) + r / 2) & 3)) * 16;
+            }
+        }
+    }
+    auto issue_stage = [&](uint32_t ks, int buf) {
+        typedef __attribute__((address_space(1))) const void *gptr;
+        typedef __attribute__((address_space(3))) void *lptr;
+        uint8_t *base = lds + buf * STAGE;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                __builtin_amdgcn_global_load_lds((gptr)(a_src[i] + (uint64_t)ks * TK + h * 16),
+                                                 (lptr)(base + (wave + 4 * i) * TILE + h * 1024), 16, 0, 0);
+                if (wave + 4 * i < NTB)               // uniform: NTB = 14 has no tiles 14, 15
+                    __builtin_amdgcn_global_load_lds((gptr)(b_src[i] + (uint64_t)ks * TILE + h * B_H),
+                                                     (lptr)(base + A_STAGE + (wave + 4 * i) * TILE + h * 1024), 16, 0, 0);
+            }
+    };
+
+    typedef typename std::conditional<FP8, v4f, v4i>::type acc_t;
+    acc_t acc[8][WNT];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < WNT; ++j) {
+            if constexpr (FP8) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+            else acc[i][j] = v4i{0, 0, 0, 0};
+        }
+
+    // Stage ks + 1 is in flight while stage ks is multiplied.
+    const uint32_t last = k_steps - 1;
+    issue_stage(0, 0);
+    for (uint32_t ks = 0; ks < k_steps; ++ks) {
+        const int buf = ks % NST;
+        __builtin_amdgcn_s_waitcnt(0x0F70);           // vmcnt(0): this wavefront's part of stage ks has landed
+        // a bare barrier: __syncthreads would add a fence on top of it
+        __builtin_amdgcn_s_barrier();                 // stage ks visible to all; stage ks - 1 no longer read
+        if (ks < last) issue_stage(ks + 1, buf ^ 1);
+        const uint8_t *la = lds + buf * STAGE + (wm * 8) * TILE;
+        const uint8_t *lb = lds + buf * STAGE + A_STAGE + (wn * WNT) * TILE + lane * 16;
+        v4i a[8][2], b[2][2];                         // [..][slice]
+        b[0][0] = *(const v4i *)(lb);
+        b[0][1] = *(const v4i *)(lb + 1024);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            a[i][0] = *(const v4i *)(la + i * TILE + a_off[0]);
+            a[i][1] = *(const v4i *)(la + i * TILE + a_off[1]);
+        }
+#pragma unroll
+        for (int j = 0; j < WNT; ++j) {
+            if (j + 1 < WNT) {                        // next fragment under the multiplies
+                b[(j + 1) % 2][0] = *(const v4i *)(lb + (j + 1) * TILE);
+                b[(j + 1) % 2][1] = *(const v4i *)(lb + (j + 1) * TILE + 1024);
+            }
+            if constexpr (FP8) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const v4i &x0 = a[i][0], &x1 = a[i][1], &y0 = b[j % 2][0], &y1 = b[j % 2][1];
+                    mfma_acc(acc[i][j], v8i{x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]},
+                             v8i{y0[0], y0[1], y0[2], y0[3], y1[0], y1[1], y1[2], y1[3]});
+                }
+            } else {
+                // the two k-steps of a tile are eight instructions apart, so no instruction waits for the
+                // accumulator of the one before it
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) mfma_acc(acc[i][j], a[i][h], b[j % 2][h]);
+            }
+        }
+        // The compiler cannot see that the asm statements are matrix instructions, so it does not insert
+        // the wait states their results need before other instructions read the accumulators; the last
+        // pass drains the matrix pipeline inside the loop body, ahead of any copy placed on the loop exit.
+        if (ks == last) asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    }
+
+    // epilogue: lane l holds column l % 16 and rows 4 * (l / 16) + e of each 16 x 16 tile
+    const int g = lane / 16, c = lane % 16;
+    float fscale = 0.0f;
+    bool extras = false;
+    const bool out_bf16 = ep.out_bf16 != 0;
+    if constexpr (FP8) fscale = __fmul_rn(*ep.a_scale, *ep.w_scale);
+    else extras = ep.acc_out != nullptr || ep.bias != nullptr || ep.residual != nullptr;
+    const uint32_t col0 = (nt0 + wn * WNT) * 16;      // first column of this wavefront
+    const bool full_cols = nt0 + wn * WNT + WNT <= n_tiles && col0 + WNT * 16 <= n;
+    if (!extras && full_cols && n % 8 == 0) {
+        // Fast path: a lane's values of one 16-row band are 2 or 4 bytes each, 16 lanes per 32 / 64 byte
+        // piece of a row; they are transposed through LDS (free now) so that the band leaves as whole
+        // rows of WNT * 16 columns in 16-byte stores.
+        __syncthreads();                              // every wavefront is done with the operand stages
+        constexpr int COLS = WNT * 16;
+        constexpr int PITCH = COLS * 4 + 16;          // bytes; also enough for bf16
+        uint8_t *band = lds + wave * (16 * PITCH);
+        float swc[WNT];
+        if constexpr (!FP8) {
+#pragma unroll
+            for (int j = 0; j < WNT; ++j) swc[j] = ep.sw[col0 + j * 16 + c];
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t row_base = m0 + (wm * 8 + i) * 16;
+            float sxr[4];
+            if constexpr (!FP8) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    uint32_t row = row_base + 4 * g + e;
+                    sxr[e] = ep.sx[row < m ? row : m - 1];
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < WNT; ++j)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float v;
+                    if constexpr (FP8) v = __fmul_rn(acc[i][j][e], fscale);
+                    else v = __fmul_rn((float)acc[i][j][e], __fmul_rn(sxr[e], swc[j]));
+                    uint8_t *dst = band + (4 * g + e) * PITCH;
+                    if (out_bf16)
+                        *(uint16_t *)(dst + (j * 16 + c) * 2) = f32_to_bf16(v);
+                    else
+                        *(float *)(dst + (j * 16 + c) * 4) = v;
+                }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            const int row_bytes = out_bf16 ? COLS * 2 : COLS * 4;
+            const int vec_per_row = row_bytes / 16;
+            for (int t = lane; t < 16 * vec_per_row; t += 64) {
+                const int r = t / vec_per_row, vcol = t % vec_per_row;
+                const uint32_t row = row_base + r;
+                if (row < m) {
+                    v4u val = *(const v4u *)(band + r * PITCH + vcol * 16);
+                    uint8_t *o = (uint8_t *)ep.out + ((uint64_t)row * n + col0) * (out_bf16 ? 2 : 4) + vcol * 16;
+                    *(v4u *)o = val;
+                }
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        }
+        return;
+    }
+#pragma unroll
+    for (int j = 0; j < WNT; ++j) {
+        const uint32_t col = (nt0 + wn * WNT + j) * 16 + c;
+        const bool col_ok = col < n && nt0 + wn * WNT + j < n_tiles;
+        float swc = 0.0f;
+        if constexpr (!FP8) swc = col_ok ? ep.sw[col] : 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const uint32_t row = m0 + (wm * 8 + i) * 16 + 4 * g + e;
+                if (col_ok && row < m) {
+                    const uint64_t o = (uint64_t)row * n + col;
+                    float v;
+                    if constexpr (FP8) {
+                        v = __fmul_rn(acc[i][j][e], fscale);
+                    } else {
+                        v = __fmul_rn((float)acc[i][j][e], __fmul_rn(ep.sx[row], swc));
+                        if (extras) {                  // uniform: raw accumulators, bias, residual
+                            if (ep.acc_out) ep.acc_out[o] = acc[i][j][e];
+                            if (ep.bias) v = __fadd_rn(v, ep.bias[col]);
+                            if (ep.residual) v = __fadd_rn(ep.residual[o], v);
+                        }
+                    }
+                    if (out_bf16)
+                        ((uint16_t *)ep.out)[o] = f32_to_bf16(v);
+                    else
+                        ((float *)ep.out)[o] = v;
+                }
+            }
+        }
+    }
+}
+
+// Column tiles per block for the large-tile kernel: the width that leaves the fewest idle block slots
+// in the last round over the compute units (0: the matrix is too small for it).
+inline int pick_big_ntb(uint64_t m, uint64_t n_tiles, int num_cus) {
+    if (m < 256 || n_tiles < 14) return 0;
+    uint64_t mb = (m + 255) / 256;
+    int best = 0;
+    double best_cost = 0;
+    for (int ntb : {16, 14}) {
+        uint64_t blocks = mb * ((n_tiles + ntb - 1) / ntb);
+        uint64_t rounds = (blocks + num_cus - 1) / num_cus;
+        double cost = (double)rounds * ntb;           // time ~ rounds x tile width
+        if (best == 0 || cost < best_cost) {
+            best = ntb;
+            best_cost = cost;
+        }
+    }
+    return best;
+}
+
+template <bool FP8, int NTB, typename Epi>
+void launch_big(const uint8_t *aq, const uint8_t *w_tiles, uint64_t m, uint64_t n, uint64_t n_tiles, uint64_t k_steps,
+                const Epi &e, hipStream_t s) {
+    const size_t smem = 2 * (size_t)(16 + NTB) * 2048;
+    static bool configured = false;
+    if (!configured) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_mfma_big_kernel<FP8, NTB, Epi>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        configured = true;
+    }
+    uint32_t mb = (uint32_t)((m + 255) / 256), nb = (uint32_t)((n_tiles + NTB - 1) / NTB);
+    gemm_mfma_big_kernel<FP8, NTB, Epi><<<mb * nb, 256, smem, s>>>(aq, w_tiles, (uint32_t)m, (uint32_t)n, (uint32_t)n_tiles,
+                                                                  (uint32_t)k_steps, mb, nb, e);
+}
+
 }  // namespace
 
 void gemm_w8a8_mfma(const int8_t *aq, const int8_t *w_tiles, uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad,
-                    const EpilogueI8 &ep, hipStream_t s) {
+                    const EpilogueI8 &ep, int num_cus, hipStream_t s) {
     if (m == 0 || n == 0) return;
     EpiI8 e{ep.sx, ep.sw, ep.bias, ep.residual, ep.acc_out, ep.out, ep.out_bf16};
+    if (int ntb = (g_gemm_small_tiles || k_pad % 128) ? 0 : pick_big_ntb(m, n_pad / 16, num_cus)) {
+        if (ntb == 16)
+            launch_big<false, 16, EpiI8>((const uint8_t *)aq, (const uint8_t *)w_tiles, m, n, n_pad / 16, k_pad / 128, e, s);
+        else
+            launch_big<false, 14, EpiI8>((const uint8_t *)aq, (const uint8_t *)w_tiles, m, n, n_pad / 16, k_pad / 128, e, s);
+        return;
+    }
     dim3 grid((unsigned)((n_pad / 16 + NT - 1) / NT), (unsigned)((m + BM - 1) / BM));
     gemm_mfma_kernel<false, EpiI8><<<grid, 256, 0, s>>>((const uint8_t *)aq, (const uint8_t *)w_tiles, (uint32_t)m,
                                                         (uint32_t)n, (uint32_t)(n_pad / 16), (uint32_t)(k_pad / 64), e);
 }
 
 void gemm_e4m3_mfma(const uint8_t *aq, const uint8_t *w_tiles, const float *a_scale, const float *w_scale, uint64_t m,
-                    uint64_t n, uint64_t n_pad, uint64_t k_pad, void *out, int out_bf16, hipStream_t s) {
+                    uint64_t n, uint64_t n_pad, uint64_t k_pad, void *out, int out_bf16, int num_cus, hipStream_t s) {
     if (m == 0 || n == 0) return;
     EpiF8 e{a_scale, w_scale, out, out_bf16};
+    if (int ntb = g_gemm_small_tiles ? 0 : pick_big_ntb(m, n_pad / 16, num_cus)) {
+        if (ntb == 16)
+            launch_big<true, 16, EpiF8>(aq, w_tiles, m, n, n_pad / 16, k_pad / 128, e, s);
+        else
+            launch_big<true, 14, EpiF8>(aq, w_tiles, m, n, n_pad / 16, k_pad / 128, e, s);
+        return;
+    }
     dim3 grid((unsigned)((n_pad / 16 + NT - 1) / NT), (unsigned)((m + BM - 1) / BM));
     gemm_mfma_kernel<true, EpiF8><<<grid, 256, 0, s>>>(aq, w_tiles, (uint32_t)m, (uint32_t)n, (uint32_t)(n_pad / 16),
                                                        (uint32_t)(k_pad / 128), e);

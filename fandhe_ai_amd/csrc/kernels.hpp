@@ -116,11 +116,11 @@ void linear_w8a16_skinny(const uint16_t *a, const int8_t *w_tiles, const float *
 // ---- prefill-shape MFMA GEMMs (kern_gemm_mfma.hip) -----------------------------
 // aq: int8 [m, k_pad] row-major.
 void gemm_w8a8_mfma(const int8_t *aq, const int8_t *w_tiles, uint64_t m, uint64_t n, uint64_t n_pad,
-                    uint64_t k_pad, const EpilogueI8 &ep, hipStream_t s);
+                    uint64_t k_pad, const EpilogueI8 &ep, int num_cus, hipStream_t s);
 // aq: e4m3 [m, k_pad] row-major; scales are device scalars.
 void gemm_e4m3_mfma(const uint8_t *aq, const uint8_t *w_tiles, const float *a_scale,
                     const float *w_scale, uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad,
-                    void *out, int out_bf16, hipStream_t s);
+                    void *out, int out_bf16, int num_cus, hipStream_t s);
 
 // ---- paged KV (kern_paged.hip) ---------------------------------------------------
 struct PagedShape {
