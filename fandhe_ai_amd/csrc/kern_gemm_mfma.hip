@@ -275,20 +275,19 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
             }
         }
     }
-    auto issue_stage = [&](uint32_t ks, int buf) {
+    // Part `part` (0 .. 7) of the loads of stage ks: tile wave + 4 (part / 2), slice part % 2, of A and of B.
+    // The parts are spread over the multiply groups of the previous stage, which keeps a steady stream
+    // of requests going to the L2 instead of one burst per stage.
+    auto issue_part = [&](uint32_t ks, int buf, int part) {
         typedef __attribute__((address_space(1))) const void *gptr;
         typedef __attribute__((address_space(3))) void *lptr;
         uint8_t *base = lds + buf * STAGE;
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                __builtin_amdgcn_global_load_lds((gptr)(a_src[i] + (uint64_t)ks * TK + h * 16),
-                                                 (lptr)(base + (wave + 4 * i) * TILE + h * 1024), 16, 0, 0);
-                if (wave + 4 * i < NTB)               // uniform: NTB = 14 has no tiles 14, 15
-                    __builtin_amdgcn_global_load_lds((gptr)(b_src[i] + (uint64_t)ks * TILE + h * B_H),
-                                                     (lptr)(base + A_STAGE + (wave + 4 * i) * TILE + h * 1024), 16, 0, 0);
-            }
+        const int i = part / 2, h = part % 2;
+        __builtin_amdgcn_global_load_lds((gptr)(a_src[i] + (uint64_t)ks * TK + h * 16),
+                                         (lptr)(base + (wave + 4 * i) * TILE + h * 1024), 16, 0, 0);
+        if (wave + 4 * i < NTB)                       // uniform: NTB = 14 has no tiles 14, 15
+            __builtin_amdgcn_global_load_lds((gptr)(b_src[i] + (uint64_t)ks * TILE + h * B_H),
+                                             (lptr)(base + A_STAGE + (wave + 4 * i) * TILE + h * 1024), 16, 0, 0);
     };
 
     typedef typename std::conditional<FP8, v4f, v4i>::type acc_t;
@@ -303,13 +302,14 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 
     // Stage ks + 1 is in flight while stage ks is multiplied.
     const uint32_t last = k_steps - 1;
-    issue_stage(0, 0);
+#pragma unroll
+    for (int part = 0; part < 8; ++part) issue_part(0, 0, part);
     for (uint32_t ks = 0; ks < k_steps; ++ks) {
         const int buf = ks % NST;
         __builtin_amdgcn_s_waitcnt(0x0F70);           // vmcnt(0): this wavefront's part of stage ks has landed
         // a bare barrier: __syncthreads would add a fence on top of it
         __builtin_amdgcn_s_barrier();                 // stage ks visible to all; stage ks - 1 no longer read
-        if (ks < last) issue_stage(ks + 1, buf ^ 1);
+        const bool more = ks < last;
         const uint8_t *la = lds + buf * STAGE + (wm * 8) * TILE;
         const uint8_t *lb = lds + buf * STAGE + A_STAGE + (wn * WNT) * TILE + lane * 16;
         v4i a[8][2], b[2][2];                         // [..][slice]
@@ -322,6 +322,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         }
 #pragma unroll
         for (int j = 0; j < WNT; ++j) {
+            if (more) {
+                // 8 parts over the first multiply groups
+                constexpr int PER = (8 + WNT - 2) / (WNT - 1);
+#pragma unroll
+                for (int q = 0; q < PER; ++q)
+                    if (j * PER + q < 8) issue_part(ks + 1, buf ^ 1, j * PER + q);
+            }
             if (j + 1 < WNT) {                        // next fragment under the multiplies
                 b[(j + 1) % 2][0] = *(const v4i *)(lb + (j + 1) * TILE);
                 b[(j + 1) % 2][1] = *(const v4i *)(lb + (j + 1) * TILE + 1024);
