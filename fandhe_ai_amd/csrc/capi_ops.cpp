@@ -12,7 +12,7 @@ using namespace fa;
 
 namespace fa {
 namespace k {
-extern int g_skinny_ntw, g_skinny_waves, g_gemm_small_tiles;
+extern int g_skinny_ntw, g_skinny_waves, g_skinny_astat, g_gemm_small_tiles;
 }
 int g_decode_waves = 0;
 extern int g_decode_partials_only;
@@ -65,7 +65,8 @@ extern "C" {
 // Tuning knobs for experiments (0 restores the built-in choice):
 // key 0 = n-tiles per block of the skinny linears, 1 = wavefronts per block,
 // 2 = wavefronts per compute unit of the decode attention, 3 = decode attention launches its streaming
-// kernel only (timing aid), 4 = prefill GEMMs keep the 128 x 128 block tile for every shape.
+// kernel only (timing aid), 4 = prefill GEMMs keep the 128 x 128 block tile for every shape,
+// 5 = activation-stationary decode linears (1 never, 2 whenever they can run).
 fa_status fa_set_tuning(int32_t key, int32_t value) {
     switch (key) {
         case 0: k::g_skinny_ntw = value; return FA_OK;
@@ -73,6 +74,7 @@ fa_status fa_set_tuning(int32_t key, int32_t value) {
         case 2: fa::g_decode_waves = value; return FA_OK;
         case 3: fa::g_decode_partials_only = value; return FA_OK;
         case 4: k::g_gemm_small_tiles = value; return FA_OK;
+        case 5: k::g_skinny_astat = value; return FA_OK;
     }
     return fail(FA_ERR_INVALID_ARGUMENT, "fa_set_tuning: unknown key");
 }

@@ -149,7 +149,7 @@ fa_status enqueue_step(fa_context *ctx, fa_decoder *d) {
                                (int8_t *)d->xq->ptr, (float *)d->sx->ptr, B, m_pad, D, s);
         k::linear_w8a8_swiglu_skinny((const int8_t *)d->xq->ptr, (const int8_t *)L.wgu->codes->ptr,
                                      (const float *)d->sx->ptr, (const float *)L.wgu->scales->ptr, B, L.wgu->n,
-                                     L.wgu->n_pad, L.wgu->k_pad, (float *)d->act->ptr, (float *)d->pmax->ptr, 4, s);
+                                     L.wgu->n_pad, L.wgu->k_pad, (float *)d->act->ptr, (float *)d->pmax->ptr, 4, cus, s);
         k::quantize_rows_from_pmax(d->act->ptr, false, (const float *)d->pmax->ptr, (uint32_t)(F / 16),
                                    (int8_t *)d->xq->ptr, (float *)d->sx->ptr, B, m_pad, F, s);
         linear(L.wdown, d->h->ptr, (const float *)d->h->ptr);

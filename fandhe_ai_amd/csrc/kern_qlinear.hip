@@ -4,6 +4,8 @@
 // the matrix instruction, so the weight never passes through LDS.  The block
 // splits K over its wavefronts and reduces their partial tiles in LDS in a
 // fixed order (deterministic).
+#include <algorithm>
+
 #include "device_utils.hpp"
 #include "kernels.hpp"
 
@@ -13,6 +15,7 @@ using namespace fa::dev;
 
 int g_skinny_ntw = 0;      // tuning overrides (0 = heuristic)
 int g_skinny_waves = 0;
+int g_skinny_astat = 0;     // activation-stationary kernel: 0 by shape, 1 never, 2 whenever it can run
 
 namespace {
 
@@ -219,6 +222,136 @@ __global__ void __launch_bounds__(NWAVES * 64)
     }
 }
 
+// ------------------------------------------------- W8A8, activation stationary
+// For weights with many more column tiles than the chip has compute units: the
+// kernel above re-reads the activation tiles (m x k, twice the bytes of a weight
+// tile at m = 32) once per block from L2, and L2 delivers little more than HBM on
+// this part, so those re-reads cost as much as the weight stream itself.  Here a
+// block of eight wavefronts keeps its activations in registers for its whole life:
+// wavefront w owns the k-tiles w, w + 8, ... (at most KTW of them) and walks the
+// block's units (pairs of column tiles: b, b + gridDim, ...) streaming only weight
+// tiles, one unit ahead in a second register set.  The eight partial tiles of a unit
+// meet in LDS (two buffers, one barrier per unit) and wavefront w finishes the rows
+// 4 (l / 16) + w % 4 of row tile w / 4 for both tiles of the unit, so SwiGLU has
+// gate and up of an element in the same lane.
+template <int MT, int KTW, int MODE>
+__global__ void __launch_bounds__(512)
+    w8a8_astat_kernel(const int8_t *__restrict__ xq_tiled, const int8_t *__restrict__ w_tiles, uint32_t m, uint32_t n,
+                      uint32_t n_tiles, uint32_t k_tiles, uint32_t n_units, EpiI8 ep) {
+    constexpr bool SWIGLU = MODE == kEpiSwiglu;
+    constexpr int NW = 8, NACC = MT * 2 * 4;
+    __shared__ int red[2][NW][NACC][64];
+    const int lane = threadIdx.x % 64;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+    const uint32_t last_kt = k_tiles - 1, last_tile = n_tiles - 1;
+
+    // activations of this wavefront's k-tiles (clamped repeats past the end are never multiplied)
+    v4i a[KTW][MT];
+#pragma unroll
+    for (int t = 0; t < KTW; ++t) {
+        uint32_t kt = wave + NW * t;
+        kt = kt < k_tiles ? kt : last_kt;
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+            a[t][i] = *(const v4i *)(xq_tiled + ((uint64_t)i * k_tiles + kt) * 1024 + (uint64_t)lane * 16);
+    }
+    auto tile_of = [&](uint32_t u, int j) -> uint32_t {
+        uint32_t nt = SWIGLU ? u + j * (n_tiles / 2) : 2 * u + j;
+        return nt < last_tile ? nt : last_tile;
+    };
+    auto load_unit = [&](uint32_t u, v4i (&b)[KTW][2]) {
+        u = u < n_units ? u : n_units - 1;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int8_t *base = w_tiles + (uint64_t)tile_of(u, j) * k_tiles * 1024 + (uint64_t)lane * 16;
+#pragma unroll
+            for (int t = 0; t < KTW; ++t) {
+                uint32_t kt = wave + NW * t;
+                kt = kt < k_tiles ? kt : last_kt;
+                b[t][j] = *(const v4i *)(base + (uint64_t)kt * 1024);
+            }
+        }
+    };
+    auto finish_unit = [&](uint32_t u, const v4i (&b)[KTW][2], int buf) {
+        v4i acc[MT][2];
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) acc[i][j] = v4i{0, 0, 0, 0};
+#pragma unroll
+        for (int t = 0; t < KTW; ++t) {
+            if ((uint32_t)(wave + NW * t) < k_tiles) {
+#pragma unroll
+                for (int i = 0; i < MT; ++i)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[t][i], b[t][j], acc[i][j], 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) red[buf][wave][(i * 2 + j) * 4 + e][lane] = acc[i][j][e];
+        __syncthreads();
+        if (wave < MT * 4) {
+            const int i = wave / 4, e = wave % 4;
+            int s0 = 0, s1 = 0;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) {
+                s0 += red[buf][w][(i * 2 + 0) * 4 + e][lane];
+                s1 += red[buf][w][(i * 2 + 1) * 4 + e][lane];
+            }
+            const uint32_t row = i * 16 + 4 * (lane / 16) + e;
+            if constexpr (SWIGLU) {
+                const uint32_t f = n / 2, col = u * 16 + lane % 16;
+                float av = 0.0f;
+                if (row < m && col < f) {
+                    float vg = __fmul_rn((float)s0, __fmul_rn(ep.sx[row], ep.sw[col]));
+                    float vu = __fmul_rn((float)s1, __fmul_rn(ep.sx[row], ep.sw[col + f]));
+                    float act = silu_f32(vg) * vu;
+                    ((float *)ep.out)[(uint64_t)row * f + col] = act;
+                    av = fabsf(act);
+                }
+#pragma unroll
+                for (int off = 1; off < 16; off <<= 1) av = fmaxf(av, __shfl_xor(av, off, 64));
+                if (lane % 16 == 0 && row < m) ep.pmax[(uint64_t)row * (n_tiles / 2) + u] = av;
+            } else {
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const uint32_t col = (2 * u + j) * 16 + lane % 16;
+                    const int sum = j ? s1 : s0;
+                    if (row < m && col < n) {
+                        uint64_t o = (uint64_t)row * n + col;
+                        if (ep.acc_out) ep.acc_out[o] = sum;
+                        float v = __fmul_rn((float)sum, __fmul_rn(ep.sx[row], ep.sw[col]));
+                        if (ep.bias) v = __fadd_rn(v, ep.bias[col]);
+                        if (ep.residual) v = __fadd_rn(ep.residual[o], v);
+                        if (ep.out_bf16)
+                            ((uint16_t *)ep.out)[o] = f32_to_bf16(v);
+                        else
+                            ((float *)ep.out)[o] = v;
+                    }
+                }
+            }
+        }
+    };
+
+    // two units per trip so that the two weight register sets have fixed names; buffer u % 2 of `red` is
+    // rewritten two units later, after the barrier of the unit in between
+    v4i b0[KTW][2], b1[KTW][2];
+    uint32_t u = blockIdx.x;
+    load_unit(u, b0);
+    for (; u < n_units; u += 2 * gridDim.x) {
+        load_unit(u + gridDim.x, b1);
+        finish_unit(u, b0, 0);
+        if (u + gridDim.x >= n_units) break;
+        load_unit(u + 2 * gridDim.x, b0);
+        finish_unit(u + gridDim.x, b1, 1);
+    }
+}
+
 // ----------------------------------------------------------------- W8A16
 // Two exact int8 -> bf16 conversions packed into one dword (low half first).
 __device__ __forceinline__ uint32_t pack_i8x2_bf16(int lo, int hi) {
@@ -353,6 +486,15 @@ inline void pick_config(uint64_t n_tiles, uint64_t k_tiles, int num_cus, int *nt
     *waves = w;
 }
 
+// The activation-stationary kernel pays off when every block has several units to amortize its
+// activation registers over and the k-tiles fit eight per wavefront.
+inline bool astat_applies(uint64_t n_units, uint64_t k_tiles, int num_cus) {
+    if (g_skinny_astat == 1) return false;
+    if (k_tiles > 64 || k_tiles == 0) return false;
+    if (g_skinny_astat == 2) return true;
+    return n_units >= 3 * (uint64_t)num_cus;
+}
+
 template <int MT>
 void launch_w8a8(const int8_t *xq, const int8_t *wt, uint32_t m, uint32_t n, uint32_t n_tiles, uint32_t k_tiles,
                  const EpiI8 &ep, int ntw, int waves, hipStream_t s) {
@@ -387,8 +529,6 @@ void linear_w8a8_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t 
                         uint64_t k_pad, const EpilogueI8 &ep, int num_cus, hipStream_t s) {
     if (m == 0 || n == 0) return;
     uint32_t n_tiles = (uint32_t)(n_pad / 16), k_tiles = (uint32_t)(k_pad / 64);
-    int ntw, waves;
-    pick_config(n_tiles, k_tiles, num_cus, &ntw, &waves);
     EpiI8 e{};
     e.sx = ep.sx;
     e.sw = ep.sw;
@@ -397,6 +537,17 @@ void linear_w8a8_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t 
     e.acc_out = ep.acc_out;
     e.out = ep.out;
     e.out_bf16 = ep.out_bf16;
+    if (astat_applies((n_tiles + 1) / 2, k_tiles, num_cus)) {
+        unsigned n_units = (n_tiles + 1) / 2;
+        unsigned blocks = (unsigned)std::min<uint64_t>(n_units, (uint64_t)num_cus);
+        if (m <= 16)
+            w8a8_astat_kernel<1, 8, kEpiPlain><<<blocks, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, n_units, e);
+        else
+            w8a8_astat_kernel<2, 8, kEpiPlain><<<blocks, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, n_units, e);
+        return;
+    }
+    int ntw, waves;
+    pick_config(n_tiles, k_tiles, num_cus, &ntw, &waves);
     if (m <= 16)
         launch_w8a8<1>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e, ntw, waves, s);
     else
@@ -405,7 +556,7 @@ void linear_w8a8_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t 
 
 void linear_w8a8_swiglu_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, const float *sx, const float *sw,
                                uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad, float *act, float *pmax,
-                               int waves, hipStream_t s) {
+                               int waves, int num_cus, hipStream_t s) {
     if (m == 0 || n == 0) return;
     uint32_t n_tiles = (uint32_t)(n_pad / 16), k_tiles = (uint32_t)(k_pad / 64);
     if (g_skinny_waves) waves = g_skinny_waves;
@@ -414,6 +565,14 @@ void linear_w8a8_swiglu_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, co
     e.sw = sw;
     e.out = act;
     e.pmax = pmax;
+    if (astat_applies(n_tiles / 2, k_tiles, num_cus)) {
+        unsigned blocks = (unsigned)std::min<uint64_t>(n_tiles / 2, (uint64_t)num_cus);
+        if (m <= 16)
+            w8a8_astat_kernel<1, 8, kEpiSwiglu><<<blocks, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, n_tiles / 2, e);
+        else
+            w8a8_astat_kernel<2, 8, kEpiSwiglu><<<blocks, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, n_tiles / 2, e);
+        return;
+    }
     unsigned grid = n_tiles / 2;
     if (m <= 16) {
         if (waves == 8)

@@ -94,7 +94,7 @@ void linear_w8a8_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t 
 // absmax of every 16-column block of act (consumed by quantize_rows_from_pmax).
 void linear_w8a8_swiglu_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, const float *sx, const float *sw,
                                uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad, float *act, float *pmax,
-                               int waves, hipStream_t s);
+                               int waves, int num_cus, hipStream_t s);
 // Fused q | k | v projection of a decode step: the weight is [k, (heads + 2 kv_heads) head_dim], head_dim a
 // multiple of 32; q and k heads are rotated (rotate-half pairing, cos/sin of the row's position from
 // cos_sin[m][head_dim]) and rounded once to bf16; q goes to q_out [m, heads * head_dim], the new K / V rows

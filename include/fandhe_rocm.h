@@ -339,7 +339,8 @@ fa_status fa_decoder_read_seq_lens(fa_context *ctx, fa_decoder *dec, uint32_t *s
  * key 2: wavefronts per compute unit of the decode attention (1 .. 8);
  * key 3: nonzero launches only the streaming kernel of the decode attention and
  *        leaves the output unwritten (for timing that kernel by itself);
- * key 4: nonzero keeps the 128 x 128 block tile of the prefill GEMMs for every shape. */
+ * key 4: nonzero keeps the 128 x 128 block tile of the prefill GEMMs for every shape;
+ * key 5: activation-stationary decode linears: 1 never, 2 whenever the shape allows. */
 fa_status fa_set_tuning(int32_t key, int32_t value);
 /* A pair of HIP events recorded on the context's stream (the stream the
  * kernels run on); used by the benchmark to time launches. */

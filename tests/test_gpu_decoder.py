@@ -57,17 +57,24 @@ def _check_step(m, dec, lens, tokens, use_graph, tag):
     dict(n_layers=1, d_model=512, n_heads=8, n_kv_heads=8, d_ffn=256, vocab=333, batch=17, ctxs=list(range(3, 20))),
     dict(n_layers=2, d_model=1024, n_heads=8, n_kv_heads=1, d_ffn=1536, vocab=4000, batch=32, ctxs=[40 + 9 * i for i in range(32)]),
 ])
-def test_decode_steps_match_the_oracle_eager_and_graph(shape):
+@pytest.mark.parametrize("astat", [1, 2], ids=["block-per-tile", "activation-stationary"])
+def test_decode_steps_match_the_oracle_eager_and_graph(shape, astat):
+    """Both families of decode-shape linears (the test models are narrow, so the activation-stationary
+    kernels, which the shape heuristic reserves for wide weights, are forced for one of the runs)."""
+    import fandhe_ai_amd as fa
     be = ops()
+    fa.check(fa.capi.lib.fa_set_tuning(5, astat))
     m = build_model(seed=11, steps=4, **shape)
     dec = GpuDecoder(be, m)
     try:
         lens, tokens = m.seq_lens.copy(), m.tokens.copy()
         for step in range(3):
-            tokens = _check_step(m, dec, lens, tokens, use_graph=(step > 0), tag="L%d:B%d:step%d" % (shape["n_layers"], shape["batch"], step))
+            tokens = _check_step(m, dec, lens, tokens, use_graph=(step > 0),
+                                 tag="L%d:B%d:step%d:%d" % (shape["n_layers"], shape["batch"], step, astat))
             dec.set_state(lens, tokens)            # the oracle continues from the GPU's tokens
     finally:
         dec.close()
+        fa.check(fa.capi.lib.fa_set_tuning(5, 0))
 
 
 def test_graph_replay_is_bit_identical_to_eager():

@@ -160,6 +160,34 @@ def test_w8a8_ragged_shapes():
         assert np.array_equal(be.download_owned(out), want), (m, k, n)
 
 
+def test_w8a8_activation_stationary_kernel_is_bit_exact():
+    """The decode-shape linear that keeps the activations in registers and walks several column-tile
+    pairs per block (chosen by shape for wide weights; forced here so that few units per block, ragged
+    widths and k-tile counts that do not fill every wavefront are covered too)."""
+    fa = _fa()
+    be = ops()
+    rng = o.Rng(77)
+    lib = fa.capi.lib
+    fa.check(lib.fa_set_tuning(5, 2))
+    try:
+        for m, k, n in ((32, 4096, 28672), (16, 4096, 6144), (3, 100, 37), (32, 130, 70), (7, 4096, 33), (17, 1000, 16400),
+                        (1, 64, 16)):
+            x = rng.randn((m, k))
+            w = rng.randn((k, n), std=0.05)
+            bias = rng.randn((n,))
+            o.set_threads(8)
+            wq, ws = o.quantize_cols_i8(w)
+            want_acc, want = o.linear_w8a8(x, wq, ws, bias)
+            o.set_threads(1)
+            qw = be.import_quantized_weight(wq, ws)
+            dbias = fa.DeviceBufferView(be.upload(bias), 0, (n,))
+            out, acc = be.linear_w8a8(be.upload(x), qw, bias=dbias, want_acc=True)
+            assert np.array_equal(be.download_owned(acc), want_acc), (m, k, n)
+            assert np.array_equal(be.download_owned(out), want), (m, k, n)
+    finally:
+        fa.check(lib.fa_set_tuning(5, 0))
+
+
 # Llama-7B layer shapes of the decode sweep: K -> N
 GEMV_SHAPES = [(4096, 12288), (4096, 4096), (4096, 22016), (11008, 4096)]
 
