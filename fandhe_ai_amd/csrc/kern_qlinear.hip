@@ -472,6 +472,98 @@ __global__ void __launch_bounds__(NWAVES * 64)
     }
 }
 
+// Activation-stationary form of the kernel above (see w8a8_astat_kernel): the bf16 activations of
+// the wavefront's k-tiles stay in registers (at m = 32 they are four times the bytes of a weight tile,
+// so re-reading them per column tile through L2 costs far more than the weight stream), the block
+// walks the column tiles b, b + gridDim, ... one tile ahead in a second register set, and the eight
+// partial tiles are added in LDS in wavefront order, exactly the k-split and summation order of the
+// eight-wavefront kernel above.
+template <int MT, int KTW>
+__global__ void __launch_bounds__(512)
+    w8a16_astat_kernel(const uint16_t *__restrict__ a, const int8_t *__restrict__ w_tiles, const float *__restrict__ sw,
+                       uint32_t m, uint32_t n, uint32_t n_tiles, uint32_t k_tiles, void *__restrict__ out, int out_bf16) {
+    constexpr int NW = 8, NACC = MT * 4;
+    __shared__ float red[2][NW][NACC][64];
+    const int lane = threadIdx.x % 64;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+    const int g = lane / 16, r = lane % 16;
+    const uint64_t k = (uint64_t)k_tiles * 64;
+    const uint32_t last_kt = k_tiles - 1;
+
+    v4u lo[KTW][MT], hi[KTW][MT];
+#pragma unroll
+    for (int t = 0; t < KTW; ++t) {
+        uint32_t kt = wave + NW * t;
+        kt = kt < k_tiles ? kt : last_kt;
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            uint32_t row = i * 16 + r;
+            row = row < m ? row : m - 1;                   // rows past m are never stored
+            const v4u *p = (const v4u *)(a + (uint64_t)row * k + (uint64_t)kt * 64 + g * 16);
+            lo[t][i] = p[0];
+            hi[t][i] = p[1];
+        }
+    }
+    auto load_tile = [&](uint32_t nt, v4u (&b)[KTW]) {
+        nt = nt < n_tiles ? nt : n_tiles - 1;
+        const int8_t *base = w_tiles + (uint64_t)nt * k_tiles * 1024 + (uint64_t)lane * 16;
+#pragma unroll
+        for (int t = 0; t < KTW; ++t) {
+            uint32_t kt = wave + NW * t;
+            kt = kt < k_tiles ? kt : last_kt;
+            b[t] = *(const v4u *)(base + (uint64_t)kt * 1024);
+        }
+    };
+    auto finish_tile = [&](uint32_t nt, const v4u (&b)[KTW], int buf) {
+        v4f acc[MT];
+#pragma unroll
+        for (int i = 0; i < MT; ++i) acc[i] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int t = 0; t < KTW; ++t) {
+            if ((uint32_t)(wave + NW * t) < k_tiles) {
+                v8bf blo, bhi;
+                cvt_i8x8_bf16(b[t][0], b[t][1], &blo);
+                cvt_i8x8_bf16(b[t][2], b[t][3], &bhi);
+#pragma unroll
+                for (int i = 0; i < MT; ++i) {
+                    acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, lo[t][i]), blo, acc[i], 0, 0, 0);
+                    acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, hi[t][i]), bhi, acc[i], 0, 0, 0);
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) red[buf][wave][i * 4 + e][lane] = acc[i][e];
+        __syncthreads();
+        if (wave < NACC) {
+            float sum = 0.0f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) sum += red[buf][w][wave][lane];
+            const int i = wave / 4, e = wave % 4;
+            const uint32_t row = i * 16 + 4 * g + e, col = nt * 16 + r;
+            if (row < m && col < n) {
+                float v = __fmul_rn(sum, sw[col]);
+                uint64_t o = (uint64_t)row * n + col;
+                if (out_bf16)
+                    ((uint16_t *)out)[o] = f32_to_bf16(v);
+                else
+                    ((float *)out)[o] = v;
+            }
+        }
+    };
+    v4u b0[KTW], b1[KTW];
+    uint32_t nt = blockIdx.x;
+    load_tile(nt, b0);
+    for (; nt < n_tiles; nt += 2 * gridDim.x) {
+        load_tile(nt + gridDim.x, b1);
+        finish_tile(nt, b0, 0);
+        if (nt + gridDim.x >= n_tiles) break;
+        load_tile(nt + 2 * gridDim.x, b0);
+        finish_tile(nt + gridDim.x, b1, 1);
+    }
+}
+
 // Picks n-tiles per block and wavefronts per block so that the whole grid is
 // resident at once with about 8-16 wavefronts per compute unit.
 inline void pick_config(uint64_t n_tiles, uint64_t k_tiles, int num_cus, int *ntw, int *waves) {
@@ -623,6 +715,16 @@ void linear_w8a16_skinny(const uint16_t *a, const int8_t *w_tiles, const float *
                          uint64_t n_pad, uint64_t k_pad, void *out, int out_bf16, int num_cus, hipStream_t s) {
     if (m == 0 || n == 0) return;
     uint32_t n_tiles = (uint32_t)(n_pad / 16), k_tiles = (uint32_t)(k_pad / 64);
+    // by shape only above 16 rows: with one row tile the activations are as small as the weight tile
+    // and the block-per-tile kernel, which spreads over more wavefronts, measured faster
+    if (astat_applies(n_tiles, k_tiles, num_cus) && !(g_skinny_ntw || g_skinny_waves) && (m > 16 || g_skinny_astat == 2)) {
+        unsigned blocks = (unsigned)std::min<uint64_t>(n_tiles, (uint64_t)num_cus);
+        if (m <= 16)
+            w8a16_astat_kernel<1, 8><<<blocks, 512, 0, s>>>(a, w_tiles, sw, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, out, out_bf16);
+        else
+            w8a16_astat_kernel<2, 8><<<blocks, 512, 0, s>>>(a, w_tiles, sw, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, out, out_bf16);
+        return;
+    }
     int ntw, waves;
     pick_config(n_tiles, k_tiles, num_cus, &ntw, &waves);
     if (m <= 16)

@@ -208,6 +208,14 @@ def test_w8a16_decode_sweep(k, n):
         got = be.download_owned(be.linear_w8a16(da, qw, fa.capi.F32))
         assert_parity("W8A16_PARITY", f"{m}x{n}x{k}", got, want)
         assert_bf16_rounding_of("w8a16 bf16", be.download_owned(be.linear_w8a16(da, qw, fa.capi.BF16)), got)
+        # the activation-stationary kernel keeps the k-split and summation order of the eight-wavefront
+        # block-per-tile kernel: forced for every shape it can run, it must meet the same tolerance
+        fa.check(fa.capi.lib.fa_set_tuning(5, 2))
+        try:
+            alt = be.download_owned(be.linear_w8a16(da, qw, fa.capi.F32))
+        finally:
+            fa.check(fa.capi.lib.fa_set_tuning(5, 0))
+        assert_parity("W8A16_PARITY", f"{m}x{n}x{k}:stationary", alt, want)
     o.set_threads(1)
 
 
