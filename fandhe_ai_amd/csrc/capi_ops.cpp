@@ -12,7 +12,7 @@ using namespace fa;
 
 namespace fa {
 namespace k {
-extern int g_skinny_ntw, g_skinny_waves, g_skinny_astat, g_gemm_small_tiles;
+extern int g_skinny_ntw, g_skinny_waves, g_skinny_astat, g_gemm_small_tiles, g_gemm_waves;
 }
 int g_decode_waves = 0;
 extern int g_decode_partials_only;
@@ -75,6 +75,7 @@ fa_status fa_set_tuning(int32_t key, int32_t value) {
         case 3: fa::g_decode_partials_only = value; return FA_OK;
         case 4: k::g_gemm_small_tiles = value; return FA_OK;
         case 5: k::g_skinny_astat = value; return FA_OK;
+        case 6: k::g_gemm_waves = value; return FA_OK;
     }
     return fail(FA_ERR_INVALID_ARGUMENT, "fa_set_tuning: unknown key");
 }

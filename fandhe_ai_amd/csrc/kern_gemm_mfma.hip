@@ -16,6 +16,7 @@ namespace k {
 using namespace fa::dev;
 
 int g_gemm_small_tiles = 0;   // tuning: nonzero keeps the 128 x 128 kernel for every shape
+int g_gemm_waves = 0;         // tuning: 4 = four wavefronts per large-tile block instead of eight
 
 namespace {
 
@@ -206,8 +207,8 @@ __device__ __forceinline__ void mfma_acc(v4f &c, const v8i &a, const v8i &b) {
 // hardware deals consecutive block ids round-robin over the 8 XCDs) are
 // consecutive tiles, m fastest: they share one B panel and walk k together,
 // which keeps the panel in that XCD's L2.
-template <bool FP8, int NTB, typename Epi>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+template <bool FP8, int NTB, int WM, typename Epi>
+__global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(WM / 2, WM / 2)))
     gemm_mfma_big_kernel(const uint8_t *__restrict__ aq, const uint8_t *__restrict__ w_tiles, uint32_t m, uint32_t n,
                          uint32_t n_tiles, uint32_t k_steps, uint32_t m_blocks, uint32_t n_blocks, Epi ep) {
     // One stage is 128 bytes of k for both types: one e4m3 instruction step, or two int8 steps (two
@@ -215,6 +216,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     // issue, first fragment reads) for int8 and let its A rows be fetched as whole 128-byte lines.
     constexpr int TK = 128, TILE = 2048;             // bytes of k per stage; bytes per operand tile and stage
     constexpr int WNT = NTB / 2;                     // column tiles per wavefront
+    constexpr int NWAVES = 2 * WM;                   // WM wavefronts along m, 2 along n
+    constexpr int AI = 16 / WM;                      // row tiles per wavefront
+    constexpr int TPW = 16 / NWAVES;                 // operand tiles each wavefront moves per stage
     constexpr int A_STAGE = 16 * TILE, B_STAGE = NTB * TILE, STAGE = A_STAGE + B_STAGE;
     constexpr int NST = 2;                           // stages in LDS
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];   // [NST][A_STAGE + B_STAGE]
@@ -239,23 +243,26 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     // instruction x takes the pieces with q % 2 == x, four consecutive lanes sharing one row, so every
     // lane quad touches one whole cache line per instruction (the L1 fetches it once; the second
     // instruction hits) instead of one line per lane.  Lane 4 r + p fills LDS slot 4 r + p of slice x
-    // with piece q = 2 ((p - r / 2) mod 4) + x: the rotation by r / 2 spreads the fragment reads of eight
-    // consecutive rows over all LDS banks.
-    // e4m3: k-group g of the matrix instruction is pieces 2 g, 2 g + 1, i.e. slot 4 r + (g + r / 2) mod 4
-    // of both slices.  int8: k-group g of k-step s is piece q = 4 s + g, i.e. slice q % 2, slot
-    // 4 r + (q / 2 + r / 2) mod 4.
+    // with piece q = 2 ((p - rot) mod 4) + x.  The rotation spreads the fragment reads over the LDS
+    // banks: rot = r / 2 for e4m3, whose k-group g of the matrix instruction is pieces 2 g, 2 g + 1, i.e.
+    // slot 4 r + (g + r / 2) mod 4 of both slices; rot = r / 2 + 2 x for int8, whose k-group g of k-step s
+    // is the single piece q = 4 s + g in slice q % 2, slot 4 r + (q / 2 + rot) mod 4 (without the 2 x
+    // term the lanes of k-groups g and g + 1 would read the same banks of the two slices).
     constexpr int B_L = FP8 ? 32 : 16, B_H = FP8 ? 16 : 1024;    // byte offsets of lane l and slice h in a tile
-    const uint8_t *a_src[4];
-    const uint8_t *b_src[4];
+    const uint8_t *a_src[TPW][2];
+    const uint8_t *b_src[TPW];
     {
         const int r = lane / 4, p4 = lane % 4;
-        const int pp = (p4 - r / 2) & 3;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            uint32_t row = m0 + (wave + 4 * i) * 16 + r;
+        for (int i = 0; i < TPW; ++i) {
+            uint32_t row = m0 + (wave + NWAVES * i) * 16 + r;
             row = row < m ? row : m - 1;
-            a_src[i] = aq + (uint64_t)row * k_bytes + pp * 32;
-            uint32_t t = nt0 + wave + 4 * i;
+#pragma unroll
+            for (int x = 0; x < 2; ++x) {
+                const int pp = (p4 - r / 2 - (FP8 ? 0 : 2 * x)) & 3;
+                a_src[i][x] = aq + (uint64_t)row * k_bytes + pp * 32 + x * 16;
+            }
+            uint32_t t = nt0 + wave + NWAVES * i;
             t = t < n_tiles ? t : n_tiles - 1;
             b_src[i] = w_tiles + (uint64_t)t * k_steps * TILE + lane * B_L;
         }
@@ -270,12 +277,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         } else {
 #pragma unroll
             for (int sub = 0; sub < 2; ++sub) {
-                const int q = 4 * sub + g;
-                a_off[sub] = (q & 1) * 1024 + (4 * r + (((q >> 1) + r / 2) & 3)) * 16;
+                const int q = 4 * sub + g, x = q & 1;
+                a_off[sub] = x * 1024 + (4 * r + (((q >> 1) + r / 2 + 2 * x) & 3)) * 16;
             }
         }
     }
-    // Part `part` (0 .. 7) of the loads of stage ks: tile wave + 4 (part / 2), slice part % 2, of A and of B.
+    // Part `part` of the loads of stage ks: tile wave + NWAVES (part / 2), slice part % 2, of A and of B.
     // The parts are spread over the multiply groups of the previous stage, which keeps a steady stream
     // of requests going to the L2 instead of one burst per stage.
     auto issue_part = [&](uint32_t ks, int buf, int part) {
@@ -283,17 +290,17 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         typedef __attribute__((address_space(3))) void *lptr;
         uint8_t *base = lds + buf * STAGE;
         const int i = part / 2, h = part % 2;
-        __builtin_amdgcn_global_load_lds((gptr)(a_src[i] + (uint64_t)ks * TK + h * 16),
-                                         (lptr)(base + (wave + 4 * i) * TILE + h * 1024), 16, 0, 0);
-        if (wave + 4 * i < NTB)                       // uniform: NTB = 14 has no tiles 14, 15
+        __builtin_amdgcn_global_load_lds((gptr)(a_src[i][h] + (uint64_t)ks * TK),
+                                         (lptr)(base + (wave + NWAVES * i) * TILE + h * 1024), 16, 0, 0);
+        if (wave + NWAVES * i < NTB)                  // uniform: NTB = 14 has no tiles 14, 15
             __builtin_amdgcn_global_load_lds((gptr)(b_src[i] + (uint64_t)ks * TILE + h * B_H),
-                                             (lptr)(base + A_STAGE + (wave + 4 * i) * TILE + h * 1024), 16, 0, 0);
+                                             (lptr)(base + A_STAGE + (wave + NWAVES * i) * TILE + h * 1024), 16, 0, 0);
     };
 
     typedef typename std::conditional<FP8, v4f, v4i>::type acc_t;
-    acc_t acc[8][WNT];
+    acc_t acc[AI][WNT];
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+    for (int i = 0; i < AI; ++i)
 #pragma unroll
         for (int j = 0; j < WNT; ++j) {
             if constexpr (FP8) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
@@ -303,20 +310,20 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     // Stage ks + 1 is in flight while stage ks is multiplied.
     const uint32_t last = k_steps - 1;
 #pragma unroll
-    for (int part = 0; part < 8; ++part) issue_part(0, 0, part);
+    for (int part = 0; part < 2 * TPW; ++part) issue_part(0, 0, part);
     for (uint32_t ks = 0; ks < k_steps; ++ks) {
         const int buf = ks % NST;
         __builtin_amdgcn_s_waitcnt(0x0F70);           // vmcnt(0): this wavefront's part of stage ks has landed
         // a bare barrier: __syncthreads would add a fence on top of it
         __builtin_amdgcn_s_barrier();                 // stage ks visible to all; stage ks - 1 no longer read
         const bool more = ks < last;
-        const uint8_t *la = lds + buf * STAGE + (wm * 8) * TILE;
+        const uint8_t *la = lds + buf * STAGE + (wm * AI) * TILE;
         const uint8_t *lb = lds + buf * STAGE + A_STAGE + (wn * WNT) * TILE + lane * 16;
-        v4i a[8][2], b[2][2];                         // [..][slice]
+        v4i a[AI][2], b[2][2];                         // [..][slice]
         b[0][0] = *(const v4i *)(lb);
         b[0][1] = *(const v4i *)(lb + 1024);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
+        for (int i = 0; i < AI; ++i) {
             a[i][0] = *(const v4i *)(la + i * TILE + a_off[0]);
             a[i][1] = *(const v4i *)(la + i * TILE + a_off[1]);
         }
@@ -324,10 +331,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         for (int j = 0; j < WNT; ++j) {
             if (more) {
                 // 8 parts over the first multiply groups
-                constexpr int PER = (8 + WNT - 2) / (WNT - 1);
+                constexpr int PER = (2 * TPW + WNT - 2) / (WNT - 1);
 #pragma unroll
                 for (int q = 0; q < PER; ++q)
-                    if (j * PER + q < 8) issue_part(ks + 1, buf ^ 1, j * PER + q);
+                    if (j * PER + q < 2 * TPW) issue_part(ks + 1, buf ^ 1, j * PER + q);
             }
             if (j + 1 < WNT) {                        // next fragment under the multiplies
                 b[(j + 1) % 2][0] = *(const v4i *)(lb + (j + 1) * TILE);
@@ -335,7 +342,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
             }
             if constexpr (FP8) {
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
+                for (int i = 0; i < AI; ++i) {
                     const v4i &x0 = a[i][0], &x1 = a[i][1], &y0 = b[j % 2][0], &y1 = b[j % 2][1];
                     mfma_acc(acc[i][j], v8i{x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]},
                              v8i{y0[0], y0[1], y0[2], y0[3], y1[0], y1[1], y1[2], y1[3]});
@@ -346,7 +353,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 #pragma unroll
                 for (int h = 0; h < 2; ++h)
 #pragma unroll
-                    for (int i = 0; i < 8; ++i) mfma_acc(acc[i][j], a[i][h], b[j % 2][h]);
+                    for (int i = 0; i < AI; ++i) mfma_acc(acc[i][j], a[i][h], b[j % 2][h]);
             }
         }
         // The compiler cannot see that the asm statements are matrix instructions, so it does not insert
@@ -378,8 +385,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
             for (int j = 0; j < WNT; ++j) swc[j] = ep.sw[col0 + j * 16 + c];
         }
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const uint32_t row_base = m0 + (wm * 8 + i) * 16;
+        for (int i = 0; i < AI; ++i) {
+            const uint32_t row_base = m0 + (wm * AI + i) * 16;
             float sxr[4];
             if constexpr (!FP8) {
 #pragma unroll
@@ -428,10 +435,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         float swc = 0.0f;
         if constexpr (!FP8) swc = col_ok ? ep.sw[col] : 0.0f;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
+        for (int i = 0; i < AI; ++i) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const uint32_t row = m0 + (wm * 8 + i) * 16 + 4 * g + e;
+                const uint32_t row = m0 + (wm * AI + i) * 16 + 4 * g + e;
                 if (col_ok && row < m) {
                     const uint64_t o = (uint64_t)row * n + col;
                     float v;
@@ -474,19 +481,30 @@ inline int pick_big_ntb(uint64_t m, uint64_t n_tiles, int num_cus) {
     return best;
 }
 
-template <bool FP8, int NTB, typename Epi>
-void launch_big(const uint8_t *aq, const uint8_t *w_tiles, uint64_t m, uint64_t n, uint64_t n_tiles, uint64_t k_steps,
+template <bool FP8, int NTB, int WM, typename Epi>
+void launch_big_wm(const uint8_t *aq, const uint8_t *w_tiles, uint64_t m, uint64_t n, uint64_t n_tiles, uint64_t k_steps,
                 const Epi &e, hipStream_t s) {
     const size_t smem = 2 * (size_t)(16 + NTB) * 2048;
     static bool configured = false;
     if (!configured) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_mfma_big_kernel<FP8, NTB, Epi>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_mfma_big_kernel<FP8, NTB, WM, Epi>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
         configured = true;
     }
     uint32_t mb = (uint32_t)((m + 255) / 256), nb = (uint32_t)((n_tiles + NTB - 1) / NTB);
-    gemm_mfma_big_kernel<FP8, NTB, Epi><<<mb * nb, 256, smem, s>>>(aq, w_tiles, (uint32_t)m, (uint32_t)n, (uint32_t)n_tiles,
+    gemm_mfma_big_kernel<FP8, NTB, WM, Epi><<<mb * nb, 128 * WM, smem, s>>>(aq, w_tiles, (uint32_t)m, (uint32_t)n, (uint32_t)n_tiles,
                                                                   (uint32_t)k_steps, mb, nb, e);
+}
+
+template <bool FP8, int NTB, typename Epi>
+void launch_big(const uint8_t *aq, const uint8_t *w_tiles, uint64_t m, uint64_t n, uint64_t n_tiles, uint64_t k_steps,
+                const Epi &e, hipStream_t s) {
+    if (g_gemm_waves == 4)
+        launch_big_wm<FP8, NTB, 2, Epi>(aq, w_tiles, m, n, n_tiles, k_steps, e, s);
+    else if (g_gemm_waves == 16)
+        launch_big_wm<FP8, NTB, 8, Epi>(aq, w_tiles, m, n, n_tiles, k_steps, e, s);
+    else
+        launch_big_wm<FP8, NTB, 4, Epi>(aq, w_tiles, m, n, n_tiles, k_steps, e, s);
 }
 
 }  // namespace
