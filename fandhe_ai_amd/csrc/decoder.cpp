@@ -138,12 +138,20 @@ fa_status enqueue_step(fa_context *ctx, fa_decoder *d) {
                                            (const float *)d->sx->ptr, (const float *)L.wqkv->scales->ptr, B,
                                            L.wqkv->n_pad, L.wqkv->k_pad, t, s);
         }
-        k::paged_attention_decode_bf16((const uint16_t *)d->q_bf->ptr, (const uint16_t *)L.k_pool->ptr,
-                                       (const uint16_t *)L.v_pool->ptr, (const uint32_t *)d->tables->ptr,
-                                       (const uint32_t *)d->seq_lens->ptr, ps, (uint32_t)g_decode_waves, ctx->workspace,
-                                       d->attn->ptr, 1, (float *)d->pmax->ptr, s);
-        k::quantize_rows_from_pmax(d->attn->ptr, true, (const float *)d->pmax->ptr, c.n_heads, (int8_t *)d->xq->ptr,
-                                   (float *)d->sx->ptr, B, m_pad, EQ, s);
+        if (c.n_heads <= 32) {
+            k::paged_attention_decode_bf16((const uint16_t *)d->q_bf->ptr, (const uint16_t *)L.k_pool->ptr,
+                                           (const uint16_t *)L.v_pool->ptr, (const uint32_t *)d->tables->ptr,
+                                           (const uint32_t *)d->seq_lens->ptr, ps, (uint32_t)g_decode_waves, ctx->workspace,
+                                           nullptr, 1, nullptr, (int8_t *)d->xq->ptr, (float *)d->sx->ptr, (uint32_t)m_pad,
+                                           s);
+        } else {
+            k::paged_attention_decode_bf16((const uint16_t *)d->q_bf->ptr, (const uint16_t *)L.k_pool->ptr,
+                                           (const uint16_t *)L.v_pool->ptr, (const uint32_t *)d->tables->ptr,
+                                           (const uint32_t *)d->seq_lens->ptr, ps, (uint32_t)g_decode_waves, ctx->workspace,
+                                           d->attn->ptr, 1, (float *)d->pmax->ptr, s);
+            k::quantize_rows_from_pmax(d->attn->ptr, true, (const float *)d->pmax->ptr, c.n_heads, (int8_t *)d->xq->ptr,
+                                       (float *)d->sx->ptr, B, m_pad, EQ, s);
+        }
         linear(L.wo, d->h->ptr, (const float *)d->h->ptr);
         k::rmsnorm_quantize_i8((const float *)d->h->ptr, (const float *)L.ffn_norm->ptr, c.rms_eps, nullptr,
                                (int8_t *)d->xq->ptr, (float *)d->sx->ptr, B, m_pad, D, s);

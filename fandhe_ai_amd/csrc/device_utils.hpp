@@ -76,6 +76,14 @@ __device__ __forceinline__ int quant_i8(float x, float scale) {
     return (int)r;
 }
 
+// byte offset of the 16-byte chunk `chunk` (= k / 16) of activation row r in the 16-row x 64-k tile order
+// of the quantized activations
+__device__ __forceinline__ uint64_t tiled_chunk_offset(uint64_t r, uint64_t chunk, uint64_t k_tiles) {
+    // kt = chunk / 4, k-group g = chunk % 4
+    uint64_t mt = r / 16, rr = r % 16, kt = chunk / 4, g = chunk % 4;
+    return (mt * k_tiles + kt) * 1024 + (g * 16 + rr) * 16;
+}
+
 // OCP e4m3fn encode, round-to-nearest-even, saturating at +-448
 __device__ __forceinline__ uint32_t f32_to_e4m3(float v) {
     uint32_t u = __float_as_uint(v);

@@ -40,13 +40,6 @@ __global__ void __launch_bounds__(kBlock) rmsnorm_kernel(const float *__restrict
     }
 }
 
-// byte offset of activation element (r, kk) in the 16-row x 64-k tile order
-__device__ __forceinline__ uint64_t tiled_chunk_offset(uint64_t r, uint64_t chunk, uint64_t k_tiles) {
-    // chunk = kk / 16: kt = chunk / 4, g = chunk % 4
-    uint64_t mt = r / 16, rr = r % 16, kt = chunk / 4, g = chunk % 4;
-    return (mt * k_tiles + kt) * 1024 + (g * 16 + rr) * 16;
-}
-
 template <bool IN_BF16>
 __device__ __forceinline__ float load_in(const void *x, uint64_t i) {
     if (IN_BF16) return bf16_to_f32(((const uint16_t *)x)[i]);

@@ -474,6 +474,104 @@ __global__ void __launch_bounds__(256) decode_stream_merge_kernel(StreamParams p
     }
 }
 
+// The merge above for a whole sequence per block, followed by the per-token int8 quantizer of the
+// projection that consumes the attention output: thread (head, 4 dims) merges its partial results,
+// rounds once to bf16 (the attention output's type), the block takes the row's absmax, and the row
+// leaves as int8 activation tiles plus its scale.  Rows at or past the batch are written as zeros.
+__global__ void __launch_bounds__(1024) decode_stream_merge_quantize_kernel(StreamParams p, int8_t *__restrict__ xq_tiled,
+                                                                           float *__restrict__ sx) {
+    __shared__ uint32_t s_tot[16], s_pre[16];
+    __shared__ float s_max[16];
+    const uint32_t b = blockIdx.x;
+    const uint32_t e_q = p.num_heads * kDh, k_tiles = e_q / 64;
+    const int wave = threadIdx.x / 64, n_waves = blockDim.x / 64;
+    if (b >= p.batch) {
+        for (uint32_t c = threadIdx.x; c < e_q / 16; c += blockDim.x)
+            *(v4u *)(xq_tiled + tiled_chunk_offset(b, c, k_tiles)) = v4u{0, 0, 0, 0};
+        return;
+    }
+    const uint32_t max_ctx = p.max_blocks_per_seq * kPage;
+    uint32_t tot = 0, pre = 0;
+    for (uint32_t bb = threadIdx.x; bb < p.batch; bb += blockDim.x) {
+        uint32_t v = seq_pages(p, bb, max_ctx);
+        tot += v;
+        if (bb < b) pre += v;
+    }
+    tot = wave_sum<uint32_t>(tot);
+    pre = wave_sum<uint32_t>(pre);
+    if (threadIdx.x % 64 == 0) {
+        s_tot[wave] = tot;
+        s_pre[wave] = pre;
+    }
+    __syncthreads();
+    tot = 0;
+    pre = 0;
+    for (int w = 0; w < n_waves; ++w) {
+        tot += s_tot[w];
+        pre += s_pre[w];
+    }
+    const uint32_t npg = seq_pages(p, b, max_ctx);
+    const uint32_t per = range_pages(p, tot);
+    const uint32_t r_lo = npg ? pre / per : 1, r_hi = npg ? (pre + npg - 1) / per : 0;   // empty sequence: no partials
+
+    // blockDim.x == num_heads * 32: thread (h, q) owns dims 4 q .. 4 q + 3 of head h
+    const uint32_t h = threadIdx.x / 32, d4 = (threadIdx.x % 32) * 4;
+    const uint32_t kvh = h / p.group, hg = h % p.group;
+    // partial results four at a time, all loads of a batch issued before the first use (the loop is a
+    // chain of L2 round trips otherwise); slots past r_hi repeat the last one with weight zero
+    const float *ml = p.part_ml + ((uint64_t)b * p.num_kv_heads + kvh) * (2 * p.g_pad) + hg;
+    const float *po = p.part_o + (((uint64_t)b * p.num_kv_heads + kvh) * p.g_pad + hg) * kDh + d4;
+    const uint64_t ml_step = (uint64_t)p.num_kv_heads * (2 * p.g_pad), po_step = (uint64_t)p.num_kv_heads * p.g_pad * kDh;
+    float mx = -INFINITY;
+    for (uint32_t r0 = r_lo; r0 <= r_hi; r0 += 4) {
+        float m[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) m[u] = ml[(uint64_t)(r0 + u <= r_hi ? r0 + u : r_hi) * ml_step];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            mx = (m[u] != m[u] || mx != mx) ? __uint_as_float(0x7fc00000u) : fmaxf(mx, m[u]);   // NaN marks a violation
+    }
+    v4f acc = v4f{0.f, 0.f, 0.f, 0.f};
+    float den = 0.0f;
+    for (uint32_t r0 = r_lo; r0 <= r_hi; r0 += 4) {
+        float m[4], l[4];
+        v4f o[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const uint64_t r = r0 + u <= r_hi ? r0 + u : r_hi;
+            m[u] = ml[r * ml_step];
+            l[u] = ml[r * ml_step + p.g_pad];
+            o[u] = *(const v4f *)(po + r * po_step);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            float w = r0 + u <= r_hi ? expf(m[u] - mx) : 0.0f;
+            den = __builtin_fmaf(w, l[u], den);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[e] = __builtin_fmaf(w, o[u][e], acc[e]);
+        }
+    }
+    float v[4], amax = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        float res = npg == 0 ? 0.0f : __fdiv_rn(acc[e], den);
+        v[e] = bf16_to_f32(f32_to_bf16(res));         // the attention output is bf16: round once, then quantize
+        amax = fmaxf(amax, fabsf(v[e]));
+    }
+    amax = wave_max(amax);
+    if (threadIdx.x % 64 == 0) s_max[wave] = amax;
+    __syncthreads();
+    amax = 0.0f;
+    for (int w = 0; w < n_waves; ++w) amax = fmaxf(amax, s_max[w]);
+    const float scale = __fdiv_rn(amax, 127.0f);
+    if (threadIdx.x == 0) sx[b] = scale;
+    uint32_t word = 0;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) word |= ((uint32_t)quant_i8(v[e], scale) & 0xffu) << (8 * e);
+    const uint32_t col = h * kDh + d4;
+    *(uint32_t *)(xq_tiled + tiled_chunk_offset(b, col / 16, k_tiles) + col % 16) = word;
+}
+
 inline int group_pad(uint32_t group) {
     int gp = 1;
     while ((uint32_t)gp < group) gp *= 2;
@@ -551,6 +649,14 @@ void paged_attention_decode_bf16(const uint16_t *q, const uint16_t *k_pool, cons
                                  const uint32_t *tables, const uint32_t *seq_lens, const PagedShape &ps,
                                  uint32_t waves_per_cu, void *workspace, void *out, int out_bf16, float *pmax,
                                  hipStream_t s) {
+    paged_attention_decode_bf16(q, k_pool, v_pool, tables, seq_lens, ps, waves_per_cu, workspace, out, out_bf16, pmax,
+                                nullptr, nullptr, 0, s);
+}
+
+void paged_attention_decode_bf16(const uint16_t *q, const uint16_t *k_pool, const uint16_t *v_pool,
+                                 const uint32_t *tables, const uint32_t *seq_lens, const PagedShape &ps,
+                                 uint32_t waves_per_cu, void *workspace, void *out, int out_bf16, float *pmax,
+                                 int8_t *xq_tiled, float *sx, uint32_t m_pad, hipStream_t s) {
     if (ps.batch == 0) return;
     StreamParams sp;
     sp.q = q;
@@ -575,6 +681,11 @@ void paged_attention_decode_bf16(const uint16_t *q, const uint16_t *k_pool, cons
     uint64_t waves = (uint64_t)sp.n_ranges * ps.num_kv_heads;
     decode_stream_kernel<4, 4, 2, 2><<<(unsigned)((waves + 3) / 4), 256, 0, s>>>(sp);
     if (g_decode_partials_only) return;
+    if (xq_tiled != nullptr && ps.num_heads <= 32) {
+        // fused merge + per-token quantizer (the bf16 output itself is not written)
+        decode_stream_merge_quantize_kernel<<<m_pad, ps.num_heads * 32, 0, s>>>(sp, xq_tiled, sx);
+        return;
+    }
     dim3 grid2(ps.num_heads, ps.batch);
     decode_stream_merge_kernel<<<grid2, 256, 0, s>>>(sp, out, out_bf16, pmax);
 }

@@ -146,6 +146,14 @@ void paged_attention_decode_bf16(const uint16_t *q, const uint16_t *k_pool, cons
                                  const PagedShape &ps, uint32_t waves_per_cu, void *workspace,
                                  void *out, int out_bf16, float *pmax /*nullable: [batch, heads] absmax*/,
                                  hipStream_t s);
+// The same with the merged result handed straight to the per-token int8 quantizer instead of being
+// stored: rounded once to bf16, quantized per sequence into activation tiles xq_tiled (rows padded to
+// m_pad, a multiple of 16) with scales sx.  Needs num_heads <= 32; otherwise call the form above and
+// quantize separately.
+void paged_attention_decode_bf16(const uint16_t *q, const uint16_t *k_pool, const uint16_t *v_pool,
+                                 const uint32_t *tables, const uint32_t *seq_lens, const PagedShape &ps,
+                                 uint32_t waves_per_cu, void *workspace, void *out, int out_bf16, float *pmax,
+                                 int8_t *xq_tiled, float *sx, uint32_t m_pad, hipStream_t s);
 
 // ---- decode-step glue (kern_decoder.hip) --------------------------------------
 // Per step, before the layers: pos[b] = seq_lens[b]; slot[b] from the block
