@@ -72,7 +72,11 @@ class DeviceContextCaptureInProgress(BackendError):
     code = capi.CAPTURE_IN_PROGRESS
 
 
-_ERRORS = {e.code: e for e in (InvalidArgument, ShapeMismatch, DeviceMismatch, DeviceAllocationFailed,
+class StorePoisoned(BackendError):
+    code = capi.STORE_POISONED
+
+
+_ERRORS = {e.code: e for e in (StorePoisoned, InvalidArgument, ShapeMismatch, DeviceMismatch, DeviceAllocationFailed,
                                KernelLaunchFailed, DeviceUnavailable, TransferFailed, Unsupported,
                                DeviceContextPoisoned, DeviceContextCaptureInProgress)}
 

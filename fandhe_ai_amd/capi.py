@@ -19,7 +19,7 @@ lib = C.CDLL(LIB_PATH)
 
 # status codes (BackendError, crates/tensor-core/src/device.rs:225-371)
 OK, INVALID_ARGUMENT, SHAPE_MISMATCH, DEVICE_MISMATCH, ALLOCATION_FAILED, KERNEL_LAUNCH_FAILED, \
-    DEVICE_UNAVAILABLE, TRANSFER_FAILED, UNSUPPORTED, CONTEXT_POISONED, CAPTURE_IN_PROGRESS = range(11)
+    DEVICE_UNAVAILABLE, TRANSFER_FAILED, UNSUPPORTED, CONTEXT_POISONED, CAPTURE_IN_PROGRESS, STORE_POISONED = range(12)
 
 F32, BF16, I8, E4M3, I32, U32 = range(6)
 QW_INT8_CHANNEL, QW_E4M3_TENSOR = 0, 1
@@ -52,6 +52,11 @@ class PagedLayout(C.Structure):
 class PagedArgs(C.Structure):
     _fields_ = [("layout", PagedLayout), ("batch", u64), ("l_new", u64), ("num_heads", u64),
                 ("max_blocks_per_seq", u64), ("scale", C.c_float), ("num_kv_heads", u64)]
+
+
+class BlockTableState(C.Structure):
+    _fields_ = [("seq_len", u64), ("has_batch", u64), ("batch", u64), ("used_blocks", u64), ("free_blocks", u64),
+                ("next_unused", u64), ("returned", u64)]
 
 
 class PagedPlan(C.Structure):
@@ -120,6 +125,28 @@ SIGNATURES = {
     "fa_paged_kv_append_device": (C.c_int32, [ctx_p, buf_p, buf_p, buf_p, buf_p, buf_p, u64, C.POINTER(PagedLayout)]),
     "fa_paged_attention_forward_device": (C.c_int32, [ctx_p, buf_p, buf_p, buf_p, buf_p, buf_p,
                                                       C.POINTER(PagedArgs), buf_p]),
+    "fa_block_table_create": (C.c_int32, [C.POINTER(C.c_void_p)]),
+    "fa_block_table_destroy": (C.c_int32, [C.c_void_p]),
+    "fa_block_table_clone": (C.c_int32, [C.c_void_p, C.POINTER(C.c_void_p)]),
+    "fa_block_table_alloc": (C.c_int32, [C.c_void_p, u64, u32p, i32p]),
+    "fa_block_table_return": (C.c_int32, [C.c_void_p, C.c_uint32]),
+    "fa_block_table_reset": (C.c_int32, [C.c_void_p]),
+    "fa_block_table_state_get": (C.c_int32, [C.c_void_p, u64, C.POINTER(BlockTableState)]),
+    "fa_block_table_extend_for_append": (C.c_int32, [C.c_void_p, u64, u64, u64, u64, u32p, u64, C.POINTER(u64)]),
+    "fa_block_table_flatten": (C.c_int32, [C.c_void_p, u64, u32p, u64, C.POINTER(u64)]),
+    "fa_block_table_rewind_to": (C.c_int32, [C.c_void_p, u64, u64]),
+    "fa_paged_cache_check_config": (C.c_int32, [u64, u64, u64, C.c_int32]),
+    "fa_paged_cache_create": (C.c_int32, [ctx_p, u64, u64, u64, C.c_int32, C.POINTER(C.c_void_p)]),
+    "fa_paged_cache_destroy": (C.c_int32, [ctx_p, C.c_void_p]),
+    "fa_paged_cache_state_get": (C.c_int32, [C.c_void_p, C.POINTER(BlockTableState), i32p]),
+    "fa_paged_cache_pools": (C.c_int32, [C.c_void_p, C.POINTER(buf_p), C.POINTER(buf_p)]),
+    "fa_paged_cache_block_tables": (C.c_int32, [C.c_void_p, u64, u32p, u64, C.POINTER(u64)]),
+    "fa_paged_cache_append": (C.c_int32, [ctx_p, C.c_void_p, buf_p, buf_p, u64, u64]),
+    "fa_paged_cache_attention": (C.c_int32, [ctx_p, C.c_void_p, buf_p, u64, u64, u64, u64, C.c_float, buf_p]),
+    "fa_paged_cache_rewind_to": (C.c_int32, [C.c_void_p, u64]),
+    "fa_paged_cache_clear": (C.c_int32, [C.c_void_p]),
+    "fa_paged_cache_snapshot_table": (C.c_int32, [C.c_void_p, C.POINTER(C.c_void_p)]),
+    "fa_paged_cache_restore_table": (C.c_int32, [C.c_void_p, C.c_void_p]),
     "fa_graph_capture_begin": (C.c_int32, [ctx_p]),
     "fa_graph_capture_end": (C.c_int32, [ctx_p, C.POINTER(C.c_void_p)]),
     "fa_graph_launch": (C.c_int32, [ctx_p, C.c_void_p]),

@@ -288,6 +288,7 @@ const char *fa_status_name(fa_status s) {
         case FA_ERR_UNSUPPORTED: return "Unsupported";
         case FA_ERR_CONTEXT_POISONED: return "DeviceContextPoisoned";
         case FA_ERR_CAPTURE_IN_PROGRESS: return "DeviceContextCaptureInProgress";
+        case FA_ERR_STORE_POISONED: return "StorePoisoned";
     }
     return "Unknown";
 }

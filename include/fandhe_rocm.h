@@ -39,7 +39,8 @@ enum {
     FA_ERR_TRANSFER_FAILED = 7,        /* BackendError::TransferFailed */
     FA_ERR_UNSUPPORTED = 8,            /* BackendError::Unsupported */
     FA_ERR_CONTEXT_POISONED = 9,       /* BackendError::DeviceContextPoisoned */
-    FA_ERR_CAPTURE_IN_PROGRESS = 10    /* BackendError::DeviceContextCaptureInProgress */
+    FA_ERR_CAPTURE_IN_PROGRESS = 10,   /* BackendError::DeviceContextCaptureInProgress */
+    FA_ERR_STORE_POISONED = 11         /* BackendError::StorePoisoned (a paged cache after a failed device write) */
 };
 /* Message of the last failure on the calling thread ("" if none). */
 const char *fa_last_error_message(void);
@@ -275,6 +276,77 @@ fa_status fa_paged_attention_forward_device(fa_context *ctx, const fa_buffer *q,
                                             const fa_buffer *k_pool, const fa_buffer *v_pool,
                                             const fa_buffer *block_tables, const fa_buffer *seq_lens,
                                             const fa_paged_args *args, fa_buffer *out);
+
+/* ---------------------------------------------------- paged KV cache (layer) */
+/* The caller side of the paged operators: page table with free-block
+ * bookkeeping and the one-layer device-resident cache built on it.
+ * BlockTable (crates/autodiff/src/nn/paged_kv.rs:147-363): free blocks are the
+ * stack of returned ids (last in, first out) and then the never-used ids in
+ * ascending order; all rows of the batch have the same length; every call
+ * either succeeds or leaves the table unchanged.  Pure host code: usable
+ * without a device. */
+typedef struct fa_block_table fa_block_table;
+typedef struct {
+    uint64_t seq_len;       /* BlockTable::seq_len (paged_kv.rs:192-195) */
+    uint64_t has_batch;     /* batch fixed by the first append */
+    uint64_t batch;
+    uint64_t used_blocks;   /* sum of the rows' block counts */
+    uint64_t free_blocks;   /* BlockTable::free_blocks (paged_kv.rs:167-169) */
+    uint64_t next_unused, returned;
+} fa_block_table_state;
+fa_status fa_block_table_create(fa_block_table **out);
+fa_status fa_block_table_destroy(fa_block_table *bt);
+fa_status fa_block_table_clone(const fa_block_table *bt, fa_block_table **out);
+/* BlockTable::alloc (paged_kv.rs:172-183); *got = 0 when no block is free. */
+fa_status fa_block_table_alloc(fa_block_table *bt, uint64_t max_blocks, uint32_t *id, int32_t *got);
+/* Pushes an id on the returned stack (what rewind_to does for every block it releases). */
+fa_status fa_block_table_return(fa_block_table *bt, uint32_t id);
+fa_status fa_block_table_reset(fa_block_table *bt);
+fa_status fa_block_table_state_get(const fa_block_table *bt, uint64_t max_blocks, fa_block_table_state *out);
+/* BlockTable::extend_for_append (paged_kv.rs:205-291): slots of the b * l_new
+ * new tokens, rows first, slot = block_id * block_size + pos % block_size. */
+fa_status fa_block_table_extend_for_append(fa_block_table *bt, uint64_t max_blocks, uint64_t block_size,
+                                           uint64_t b, uint64_t l_new, uint32_t *slots,
+                                           uint64_t slots_capacity, uint64_t *n_slots);
+/* BlockTable::flatten_tables (paged_kv.rs:295-319): [rows, max_blocks_per_seq], UINT32_MAX in unused entries. */
+fa_status fa_block_table_flatten(const fa_block_table *bt, uint64_t max_blocks_per_seq, uint32_t *out,
+                                 uint64_t out_capacity, uint64_t *n_out);
+/* BlockTable::rewind_to (paged_kv.rs:323-363). */
+fa_status fa_block_table_rewind_to(fa_block_table *bt, uint64_t new_len, uint64_t block_size);
+
+/* PagedKvCache (crates/autodiff/src/nn/paged_kv_device.rs:67-372): K / V pools
+ * [max_blocks, block_size, embed_dim] on the device (f32 as in the reference,
+ * or bf16), append and attention queued on the context's stream, the only
+ * synchronization point is the download of the attention output.  A device
+ * failure after validation poisons the cache (append / attention then return
+ * FA_ERR_STORE_POISONED; rewind_to and clear stay allowed). */
+typedef struct fa_paged_cache fa_paged_cache;
+/* PagedKvCacheConfig::new (paged_kv.rs:79-108). */
+fa_status fa_paged_cache_check_config(uint64_t block_size, uint64_t max_blocks, uint64_t embed_dim,
+                                      fa_dtype dtype);
+/* PagedKvCache::new (paged_kv_device.rs:91-123). */
+fa_status fa_paged_cache_create(fa_context *ctx, uint64_t block_size, uint64_t max_blocks,
+                                uint64_t embed_dim, fa_dtype dtype, fa_paged_cache **out);
+fa_status fa_paged_cache_destroy(fa_context *ctx, fa_paged_cache *cache);
+/* seq_len / batch / num_used_blocks / num_free_blocks / is_poisoned (paged_kv_device.rs:136-160). */
+fa_status fa_paged_cache_state_get(const fa_paged_cache *cache, fa_block_table_state *out, int32_t *poisoned);
+fa_status fa_paged_cache_pools(fa_paged_cache *cache, fa_buffer **k_pool, fa_buffer **v_pool);
+fa_status fa_paged_cache_block_tables(const fa_paged_cache *cache, uint64_t max_blocks_per_seq, uint32_t *out,
+                                      uint64_t out_capacity, uint64_t *n_out);
+/* PagedKvCache::append (paged_kv_device.rs:187-247): k_new / v_new [b, l_new, embed_dim] of the pools' type. */
+fa_status fa_paged_cache_append(fa_context *ctx, fa_paged_cache *cache, const fa_buffer *k_new,
+                                const fa_buffer *v_new, uint64_t b, uint64_t l_new);
+/* PagedKvCache::attention (paged_kv_device.rs:254-340): q / out [b, l_new, num_heads * head_dim] with
+ * head_dim = embed_dim / num_kv_heads (num_kv_heads 0 or == num_heads: the reference's MHA). */
+fa_status fa_paged_cache_attention(fa_context *ctx, const fa_paged_cache *cache, const fa_buffer *q, uint64_t b,
+                                   uint64_t l_new, uint64_t num_heads, uint64_t num_kv_heads, float scale,
+                                   fa_buffer *out);
+/* PagedKvCache::rewind_to / clear (paged_kv_device.rs:346-371): logical state only. */
+fa_status fa_paged_cache_rewind_to(fa_paged_cache *cache, uint64_t new_len);
+fa_status fa_paged_cache_clear(fa_paged_cache *cache);
+/* snapshot_table / restore_table (paged_kv_device.rs:356-363). */
+fa_status fa_paged_cache_snapshot_table(const fa_paged_cache *cache, fa_block_table **out);
+fa_status fa_paged_cache_restore_table(fa_paged_cache *cache, const fa_block_table *saved);
 
 /* ------------------------------------------------------------------ graphs */
 /* Counterpart of the reference's captured inference chain
