@@ -16,7 +16,8 @@ namespace k {
 using namespace fa::dev;
 
 int g_gemm_small_tiles = 0;   // tuning: nonzero keeps the 128 x 128 kernel for every shape
-int g_gemm_waves = 0;         // tuning: 4 = four wavefronts per large-tile block instead of eight
+int g_gemm_waves = 0;
+int g_gemm_ntb = 0;           // tuning: 14 or 16 fixes the column tiles per large-tile block         // tuning: 4 = four wavefronts per large-tile block instead of eight
 
 namespace {
 
@@ -195,6 +196,19 @@ __device__ __forceinline__ void mfma_acc(v4f &c, const v8i &a, const v8i &b) {
                  : "v"(a), "v"(b), "v"(unit));
 }
 
+// Waits until the matrix pipeline has retired everything issued before, and ties the accumulators of one
+// row of tiles to that point (they are in/out operands, so no read of them can be placed ahead of it).
+template <typename T>
+__device__ __forceinline__ void drain_row(T (&r)[7]) {
+    asm volatile("s_nop 15\n\ts_nop 15"
+                 : "+a"(r[0]), "+a"(r[1]), "+a"(r[2]), "+a"(r[3]), "+a"(r[4]), "+a"(r[5]), "+a"(r[6]));
+}
+template <typename T>
+__device__ __forceinline__ void drain_row(T (&r)[8]) {
+    asm volatile("s_nop 15\n\ts_nop 15"
+                 : "+a"(r[0]), "+a"(r[1]), "+a"(r[2]), "+a"(r[3]), "+a"(r[4]), "+a"(r[5]), "+a"(r[6]), "+a"(r[7]));
+}
+
 // ------------------------------------------------------------ large tiles
 // Block tile 256 rows x NTB * 16 columns, four wavefronts in 2 x 2, one per
 // SIMD, each owning 128 rows x NTB / 2 column tiles of accumulators (up to 256
@@ -219,9 +233,8 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
     constexpr int NWAVES = 2 * WM;                   // WM wavefronts along m, 2 along n
     constexpr int AI = 16 / WM;                      // row tiles per wavefront
     constexpr int TPW = 16 / NWAVES;                 // operand tiles each wavefront moves per stage
-    constexpr int A_STAGE = 16 * TILE, B_STAGE = NTB * TILE, STAGE = A_STAGE + B_STAGE;
-    constexpr int NST = 2;                           // stages in LDS
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];   // [NST][A_STAGE + B_STAGE]
+    constexpr int A_STAGE = 16 * TILE, B_STAGE = NTB * TILE;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];   // [3][A_STAGE] then [2][B_STAGE]
 
     const int tid = threadIdx.x, lane = tid % 64;
     const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
@@ -262,7 +275,10 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
                 const int pp = (p4 - r / 2 - (FP8 ? 0 : 2 * x)) & 3;
                 a_src[i][x] = aq + (uint64_t)row * k_bytes + pp * 32 + x * 16;
             }
-            uint32_t t = nt0 + wave + NWAVES * i;
+            // a block of NTB = 14 has no tiles 14, 15: the wavefronts that would move them repeat their
+            // first tile instead (same bytes to the same place, served by the L1), which keeps the main
+            // loop free of branches
+            uint32_t t = nt0 + (wave + NWAVES * i < NTB ? wave + NWAVES * i : wave);
             t = t < n_tiles ? t : n_tiles - 1;
             b_src[i] = w_tiles + (uint64_t)t * k_steps * TILE + lane * B_L;
         }
@@ -282,19 +298,26 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
             }
         }
     }
-    // Part `part` of the loads of stage ks: tile wave + NWAVES (part / 2), slice part % 2, of A and of B.
-    // The parts are spread over the multiply groups of the previous stage, which keeps a steady stream
-    // of requests going to the L2 instead of one burst per stage.
-    auto issue_part = [&](uint32_t ks, int buf, int part) {
-        typedef __attribute__((address_space(1))) const void *gptr;
-        typedef __attribute__((address_space(3))) void *lptr;
-        uint8_t *base = lds + buf * STAGE;
-        const int i = part / 2, h = part % 2;
+    // LDS holds three stages of A and two of B: A runs two stages ahead of the multiplies, B one, so that
+    // requests stay in flight across the wait at the top of a stage (with both operands one stage ahead
+    // the path from L2 runs dry there; a third stage of both does not fit).
+    constexpr int NSA = 3, NSB = 2;
+    uint8_t *const lds_b0 = lds + NSA * A_STAGE;
+    // Load instruction `idx` of a stage: tile wave + NWAVES (idx / 2), slice idx % 2.  They are spread over
+    // the multiply groups of the stage before, which keeps a steady stream of requests going to the L2
+    // instead of one burst per stage.
+    typedef __attribute__((address_space(1))) const void *gptr;
+    typedef __attribute__((address_space(3))) void *lptr;
+    auto issue_a = [&](uint32_t ks, int slot, int idx) {
+        const int i = idx / 2, h = idx % 2;
         __builtin_amdgcn_global_load_lds((gptr)(a_src[i][h] + (uint64_t)ks * TK),
-                                         (lptr)(base + (wave + NWAVES * i) * TILE + h * 1024), 16, 0, 0);
-        if (wave + NWAVES * i < NTB)                  // uniform: NTB = 14 has no tiles 14, 15
-            __builtin_amdgcn_global_load_lds((gptr)(b_src[i] + (uint64_t)ks * TILE + h * B_H),
-                                             (lptr)(base + A_STAGE + (wave + NWAVES * i) * TILE + h * 1024), 16, 0, 0);
+                                         (lptr)(lds + slot * A_STAGE + (wave + NWAVES * i) * TILE + h * 1024), 16, 0, 0);
+    };
+    auto issue_b = [&](uint32_t ks, int slot, int idx) {
+        const int i = idx / 2, h = idx % 2;
+        const int t = wave + NWAVES * i < NTB ? wave + NWAVES * i : wave;
+        __builtin_amdgcn_global_load_lds((gptr)(b_src[i] + (uint64_t)ks * TILE + h * B_H),
+                                         (lptr)(lds_b0 + slot * B_STAGE + t * TILE + h * 1024), 16, 0, 0);
     };
 
     typedef typename std::conditional<FP8, v4f, v4i>::type acc_t;
@@ -307,45 +330,81 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
             else acc[i][j] = v4i{0, 0, 0, 0};
         }
 
-    // Stage ks + 1 is in flight while stage ks is multiplied.
+    // Per stage a wavefront issues its B loads of stage ks + 1 first and its A loads of stage ks + 2 after
+    // them, so the wait at the top of stage ks + 1 can leave exactly those 2 TPW A loads outstanding.  Past
+    // the end the loads are repeated from the last stage into slots nobody reads again, which keeps the
+    // count of outstanding loads the same in every pass.
+    constexpr int NLD = 2 * TPW;                     // A load instructions per wavefront and stage
     const uint32_t last = k_steps - 1;
 #pragma unroll
-    for (int part = 0; part < 2 * TPW; ++part) issue_part(0, 0, part);
-    for (uint32_t ks = 0; ks < k_steps; ++ks) {
-        const int buf = ks % NST;
-        __builtin_amdgcn_s_waitcnt(0x0F70);           // vmcnt(0): this wavefront's part of stage ks has landed
-        // a bare barrier: __syncthreads would add a fence on top of it
-        __builtin_amdgcn_s_barrier();                 // stage ks visible to all; stage ks - 1 no longer read
-        const bool more = ks < last;
-        const uint8_t *la = lds + buf * STAGE + (wm * AI) * TILE;
-        const uint8_t *lb = lds + buf * STAGE + A_STAGE + (wn * WNT) * TILE + lane * 16;
-        v4i a[AI][2], b[2][2];                         // [..][slice]
-        b[0][0] = *(const v4i *)(lb);
-        b[0][1] = *(const v4i *)(lb + 1024);
+    for (int idx = 0; idx < NLD; ++idx) issue_a(0, 0, idx);
 #pragma unroll
-        for (int i = 0; i < AI; ++i) {
-            a[i][0] = *(const v4i *)(la + i * TILE + a_off[0]);
-            a[i][1] = *(const v4i *)(la + i * TILE + a_off[1]);
-        }
+    for (int idx = 0; idx < NLD; ++idx) issue_b(0, 0, idx);
+#pragma unroll
+    for (int idx = 0; idx < NLD; ++idx) issue_a(last < 1 ? last : 1, 1, idx);
+    // The barrier that opens stage ks + 1 sits before the last multiply group of stage ks, and the first
+    // fragments of stage ks + 1 (all of A, the first of B) are read under that group: with the barrier
+    // at the top of a stage every wavefront of the block would wait there for its first fragments at
+    // the same time, with the matrix cores idle.  Per stage:
+    //   groups 0 .. WNT - 2: loads of B (stage ks + 1) and A (stage ks + 2), B fragment j + 1, multiplies j
+    //   group WNT - 1: own reads of stage ks complete and own loads of stage ks + 1 landed, barrier,
+    //                  multiplies interleaved with the A fragment reads of stage ks + 1, then its first B
+    // The loads overwrite the buffers of stage ks - 1; they are issued after the barrier that opened
+    // stage ks, which a wavefront reaches only after all its reads of stage ks - 1 have completed.
+    int slot_a = 0;
+    const uint8_t *la = lds + (wm * AI) * TILE;
+    const uint8_t *lb = lds_b0 + (wn * WNT) * TILE + lane * 16;
+    __builtin_amdgcn_s_waitcnt(0x0F70 | NLD);         // stage 0 of this wavefront has landed (A of stage 1 may not)
+    __builtin_amdgcn_s_barrier();                     // a bare barrier: __syncthreads would add a fence on top
+    v4i a[AI][2], b[2][2];                            // [..][slice]
+#pragma unroll
+    for (int i = 0; i < AI; ++i) {
+        a[i][0] = *(const v4i *)(la + i * TILE + a_off[0]);
+        a[i][1] = *(const v4i *)(la + i * TILE + a_off[1]);
+    }
+    b[0][0] = *(const v4i *)(lb);
+    b[0][1] = *(const v4i *)(lb + 1024);
+    uint32_t ks = 0;
+    do {                                              // k_steps >= 1: the launcher returns early otherwise
+        const int buf = ks % NSB;
+        const uint32_t ks_b = ks + 1 < last ? ks + 1 : last, ks_a = ks + 2 < last ? ks + 2 : last;
+        const int slot_a2 = slot_a == 0 ? 2 : slot_a - 1;             // (slot_a + 2) % 3
 #pragma unroll
         for (int j = 0; j < WNT; ++j) {
-            if (more) {
-                // 8 parts over the first multiply groups
-                constexpr int PER = (2 * TPW + WNT - 2) / (WNT - 1);
+            {
+                // 2 NLD load instructions over the first multiply groups, B before A
+                constexpr int PER = (2 * NLD + WNT - 3) / (WNT - 2);
 #pragma unroll
-                for (int q = 0; q < PER; ++q)
-                    if (j * PER + q < 2 * TPW) issue_part(ks + 1, buf ^ 1, j * PER + q);
+                for (int q = 0; q < PER; ++q) {
+                    const int idx = j * PER + q;
+                    if (idx < NLD) issue_b(ks_b, buf ^ 1, idx);
+                    else if (idx < 2 * NLD) issue_a(ks_a, slot_a2, idx - NLD);
+                }
             }
+            const int cur = j % 2;
             if (j + 1 < WNT) {                        // next fragment under the multiplies
-                b[(j + 1) % 2][0] = *(const v4i *)(lb + (j + 1) * TILE);
-                b[(j + 1) % 2][1] = *(const v4i *)(lb + (j + 1) * TILE + 1024);
+                b[cur ^ 1][0] = *(const v4i *)(lb + (j + 1) * TILE);
+                b[cur ^ 1][1] = *(const v4i *)(lb + (j + 1) * TILE + 1024);
+            } else {
+                // lgkmcnt(0), vmcnt(NLD): every read of stage ks by this wavefront is complete and its
+                // loads of stage ks + 1 have landed (the A loads of stage ks + 2 may be outstanding)
+                __builtin_amdgcn_s_waitcnt(0x0070 | NLD);
+                __builtin_amdgcn_s_barrier();         // stage ks + 1 visible to all; stage ks no longer read
+                slot_a = slot_a == 2 ? 0 : slot_a + 1;
+                la = lds + slot_a * A_STAGE + (wm * AI) * TILE;
+                lb = lds_b0 + (buf ^ 1) * B_STAGE + (wn * WNT) * TILE + lane * 16;
             }
+            const bool tail = j + 1 == WNT;           // past the last stage the reads fetch stale, unused data
             if constexpr (FP8) {
 #pragma unroll
                 for (int i = 0; i < AI; ++i) {
-                    const v4i &x0 = a[i][0], &x1 = a[i][1], &y0 = b[j % 2][0], &y1 = b[j % 2][1];
+                    const v4i &x0 = a[i][0], &x1 = a[i][1], &y0 = b[cur][0], &y1 = b[cur][1];
                     mfma_acc(acc[i][j], v8i{x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]},
                              v8i{y0[0], y0[1], y0[2], y0[3], y1[0], y1[1], y1[2], y1[3]});
+                    if (tail) {
+                        a[i][0] = *(const v4i *)(la + i * TILE + a_off[0]);
+                        a[i][1] = *(const v4i *)(la + i * TILE + a_off[1]);
+                    }
                 }
             } else {
                 // the two k-steps of a tile are eight instructions apart, so no instruction waits for the
@@ -353,14 +412,24 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
 #pragma unroll
                 for (int h = 0; h < 2; ++h)
 #pragma unroll
-                    for (int i = 0; i < AI; ++i) mfma_acc(acc[i][j], a[i][h], b[j % 2][h]);
+                    for (int i = 0; i < AI; ++i) {
+                        mfma_acc(acc[i][j], a[i][h], b[cur][h]);
+                        if (tail) a[i][h] = *(const v4i *)(la + i * TILE + a_off[h]);
+                    }
+            }
+            if (tail) {                               // after the multiplies: with an odd WNT they read b[0]
+                b[0][0] = *(const v4i *)(lb);
+                b[0][1] = *(const v4i *)(lb + 1024);
             }
         }
-        // The compiler cannot see that the asm statements are matrix instructions, so it does not insert
-        // the wait states their results need before other instructions read the accumulators; the last
-        // pass drains the matrix pipeline inside the loop body, ahead of any copy placed on the loop exit.
-        if (ks == last) asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-    }
+    } while (++ks < k_steps);
+    // The compiler cannot see that the asm statements are matrix instructions, so it does not insert the
+    // wait states their results need before other instructions read the accumulators (it may even peel
+    // the last pass and start copying accumulators between its multiplies).  Every accumulator therefore
+    // passes through a statement that waits out the matrix pipeline before anything else may read it.
+#pragma unroll
+    for (int i = 0; i < AI; ++i) drain_row(acc[i]);
+    __builtin_amdgcn_s_waitcnt(0x0F70);               // the repeated loads of the tail have landed too
 
     // epilogue: lane l holds column l % 16 and rows 4 * (l / 16) + e of each 16 x 16 tile
     const int g = lane / 16, c = lane % 16;
@@ -466,6 +535,7 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
 // in the last round over the compute units (0: the matrix is too small for it).
 inline int pick_big_ntb(uint64_t m, uint64_t n_tiles, int num_cus) {
     if (m < 256 || n_tiles < 14) return 0;
+    if (g_gemm_ntb == 14 || g_gemm_ntb == 16) return g_gemm_ntb;
     uint64_t mb = (m + 255) / 256;
     int best = 0;
     double best_cost = 0;
@@ -484,7 +554,7 @@ inline int pick_big_ntb(uint64_t m, uint64_t n_tiles, int num_cus) {
 template <bool FP8, int NTB, int WM, typename Epi>
 void launch_big_wm(const uint8_t *aq, const uint8_t *w_tiles, uint64_t m, uint64_t n, uint64_t n_tiles, uint64_t k_steps,
                 const Epi &e, hipStream_t s) {
-    const size_t smem = 2 * (size_t)(16 + NTB) * 2048;
+    const size_t smem = (3 * 16 + 2 * (size_t)NTB) * 2048;          // three stages of A, two of B
     static bool configured = false;
     if (!configured) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_mfma_big_kernel<FP8, NTB, WM, Epi>),
@@ -513,7 +583,7 @@ void gemm_w8a8_mfma(const int8_t *aq, const int8_t *w_tiles, uint64_t m, uint64_
                     const EpilogueI8 &ep, int num_cus, hipStream_t s) {
     if (m == 0 || n == 0) return;
     EpiI8 e{ep.sx, ep.sw, ep.bias, ep.residual, ep.acc_out, ep.out, ep.out_bf16};
-    if (int ntb = (g_gemm_small_tiles || k_pad % 128) ? 0 : pick_big_ntb(m, n_pad / 16, num_cus)) {
+    if (int ntb = (g_gemm_small_tiles || k_pad % 128 || k_pad == 0) ? 0 : pick_big_ntb(m, n_pad / 16, num_cus)) {
         if (ntb == 16)
             launch_big<false, 16, EpiI8>((const uint8_t *)aq, (const uint8_t *)w_tiles, m, n, n_pad / 16, k_pad / 128, e, s);
         else
@@ -529,7 +599,7 @@ void gemm_e4m3_mfma(const uint8_t *aq, const uint8_t *w_tiles, const float *a_sc
                     uint64_t n, uint64_t n_pad, uint64_t k_pad, void *out, int out_bf16, int num_cus, hipStream_t s) {
     if (m == 0 || n == 0) return;
     EpiF8 e{a_scale, w_scale, out, out_bf16};
-    if (int ntb = g_gemm_small_tiles ? 0 : pick_big_ntb(m, n_pad / 16, num_cus)) {
+    if (int ntb = (g_gemm_small_tiles || k_pad == 0) ? 0 : pick_big_ntb(m, n_pad / 16, num_cus)) {
         if (ntb == 16)
             launch_big<true, 16, EpiF8>(aq, w_tiles, m, n, n_pad / 16, k_pad / 128, e, s);
         else
