@@ -292,6 +292,31 @@ def bench_prefill(fa, be, iters):
     return res
 
 
+def bench_matrix_rate(fa, be, iters=20000):
+    """Register-only rate of the matrix instructions the prefill GEMMs use, with all-zero and with
+    random operand bits (the sustained clock of the part depends on the bits it multiplies)."""
+    lib = fa.capi.lib
+    rng = np.random.default_rng(7)
+    rand = rng.integers(0, 256, size=65536, dtype=np.uint8)
+    rand[(rand & 0x7F) == 0x7F] = 0x3C                  # no e4m3 NaN codes
+    sink = be.alloc_zeroed((1,), fa.capi.I32)
+    res = []
+    for fill, data in (("zero operands", np.zeros(65536, np.uint8)), ("random operand bits", rand)):
+        src = be.upload(data)
+        for kind, name in enumerate(("v_mfma_i32_16x16x64_i8", "v_mfma_i32_32x32x32_i8", "v_mfma_scale_f32_16x16x128_f8f6f4 (e4m3)")):
+            ops = C.c_double()
+            fa.check(lib.fa_probe_matrix_rate(be._ctx, kind, src._h, 200, sink._h, C.byref(ops)))
+            be.synchronize_device()
+            t = Timer(fa, be)
+            t.start()
+            fa.check(lib.fa_probe_matrix_rate(be._ctx, kind, src._h, iters, sink._h, C.byref(ops)))
+            ms = t.stop_ms()
+            res.append(dict(instr=name, fill=fill, ms=ms, tops=ops.value / (ms * 1e-3) / 1e12))
+        src.free()
+    sink.free()
+    return res
+
+
 # ---------------------------------------------------------------- CPU baseline
 def cpu_baseline(cfg, batch, ctxs, threads):
     """The CPU oracle (a restatement of the reference's backend-cpu algorithms; the Rust crate cannot be
@@ -357,7 +382,7 @@ def main():
                     help="tuning: wavefronts per compute unit of the decode attention (0 = built-in)")
     ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
                     help="tuning: raw fa_set_tuning key/value pairs (experiments)")
-    ap.add_argument("--only", choices=("attention", "copy", "linears", "prefill"), default=None,
+    ap.add_argument("--only", choices=("attention", "copy", "linears", "prefill", "mfma"), default=None,
                     help="profiling aid: run only the dominant kernel at the workload's shape, or a plain "
                          "copy kernel of known size (counter calibration), a few launches, no JSON line")
     a = ap.parse_args()
@@ -382,6 +407,12 @@ def main():
             for r in bench_prefill(fa, be, 20):
                 log("%s m=%d k=%d n=%d: %.1f us, %.0f TOPS (%.1f %% of peak)" %
                     (r["op"], r["m"], r["k"], r["n"], r["us"], r["tops"], 100 * r["frac"]))
+            be.close()
+            return
+        if a.only == "mfma":
+            for r in bench_matrix_rate(fa, be):
+                log("%-42s %-20s: %.2f ms, %.0f T op/s (%.1f %% of peak)" %
+                    (r["instr"], r["fill"], r["ms"], r["tops"], 100 * r["tops"] / MFMA_PEAK_TOPS))
             be.close()
             return
         if a.only == "linears":

@@ -487,6 +487,20 @@ fa_status fa_fill_normal(fa_context *ctx, fa_buffer *buf, uint64_t offset, uint6
     return after_launch(ctx, "fill_normal");
 }
 
+fa_status fa_probe_matrix_rate(fa_context *ctx, int32_t kind, const fa_buffer *operands, uint32_t iters, fa_buffer *sink,
+                               double *ops) {
+    if (fa_status s = check_ctx(ctx)) return s;
+    if (fa_status s = check_buf(ctx, operands, "probe_matrix_rate: operands")) return s;
+    if (fa_status s = check_buf(ctx, sink, "probe_matrix_rate: sink")) return s;
+    if (kind < 0 || kind > 2) return fail(FA_ERR_INVALID_ARGUMENT, "probe_matrix_rate: kind is 0, 1 or 2");
+    if (operands->numel * dtype_size(operands->dtype) < 65536)
+        return fail(FA_ERR_SHAPE_MISMATCH, "probe_matrix_rate: operands must hold 64 KiB");
+    if (sink->numel * dtype_size(sink->dtype) < 4) return fail(FA_ERR_SHAPE_MISMATCH, "probe_matrix_rate: sink too small");
+    if (!ops) return fail(FA_ERR_INVALID_ARGUMENT, "probe_matrix_rate: null ops");
+    *ops = k::matrix_rate_probe(kind, operands->ptr, iters, ctx->props.multiProcessorCount, (int *)sink->ptr, ctx->stream);
+    return after_launch(ctx, "matrix_rate_probe");
+}
+
 fa_status fa_convert(fa_context *ctx, const fa_buffer *src, uint64_t numel, fa_buffer *dst) {
     if (fa_status s = check_ctx(ctx)) return s;
     if (fa_status s = check_buf(ctx, src, "convert: src")) return s;

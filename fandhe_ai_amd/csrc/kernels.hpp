@@ -155,6 +155,12 @@ void paged_attention_decode_bf16(const uint16_t *q, const uint16_t *k_pool, cons
                                  uint32_t waves_per_cu, void *workspace, void *out, int out_bf16, float *pmax,
                                  int8_t *xq_tiled, float *sx, uint32_t m_pad, hipStream_t s);
 
+// ---- measurement aid (kern_probe.hip) -------------------------------------------
+// Launches a register-only loop of one matrix instruction kind (0: i32_16x16x64_i8, 1: i32_32x32x32_i8,
+// 2: scaled f32_16x16x128 on e4m3) whose operand bits come from `operands` (64 KiB); returns the number
+// of multiply-add operations x 2 the launch performs.  sink: one int, never written in practice.
+double matrix_rate_probe(int kind, const void *operands, uint32_t iters, int num_cus, int *sink, hipStream_t s);
+
 // ---- decode-step glue (kern_decoder.hip) --------------------------------------
 // Per step, before the layers: pos[b] = seq_lens[b]; slot[b] from the block
 // table (UINT32_MAX when the table cannot hold the position); seq_lens[b] += 1;

@@ -213,6 +213,15 @@ fa_status fa_gather_rows(fa_context *ctx, const fa_buffer *table, uint64_t table
  * reference's interface. */
 fa_status fa_fill_normal(fa_context *ctx, fa_buffer *buf, uint64_t offset, uint64_t numel,
                          uint64_t seed, float mean, float std);
+/* Measurement aid, not part of the reference's interface: queues a loop of one
+ * matrix instruction kind with operands held in registers (kind 0:
+ * v_mfma_i32_16x16x64_i8, 1: v_mfma_i32_32x32x32_i8, 2: the scaled
+ * 16x16x128 e4m3 form).  The operand bits are taken from `operands` (64 KiB of
+ * any element type): the sustained rate of the matrix cores depends on them.
+ * *ops receives the multiply-add operations x 2 of the launch; time it with an
+ * fa_timer. */
+fa_status fa_probe_matrix_rate(fa_context *ctx, int32_t kind, const fa_buffer *operands,
+                               uint32_t iters, fa_buffer *sink, double *ops);
 /* dtype conversion f32 <-> bf16 (round to nearest even, once). */
 fa_status fa_convert(fa_context *ctx, const fa_buffer *src, uint64_t numel, fa_buffer *dst);
 
