@@ -292,6 +292,41 @@ def bench_prefill(fa, be, iters):
     return res
 
 
+def bench_prefill_attention(fa, be, batch=4, l_new=2048, heads=32, kv_heads=8):
+    """Causal attention of `l_new` new tokens per row over their own pages (empty cache before them), bf16,
+    page 16: the streamed matrix-core kernel, and the generic kernel (reference summation order) beside it."""
+    lib = fa.capi.lib
+    rng = np.random.default_rng(5)
+    tables, max_blocks, num_blocks = make_tables(rng, [l_new] * batch, 0, 16)
+    e_kv, e_q = kv_heads * 128, heads * 128
+    layout = fa.PagedKvLayout.new(num_blocks, 16, e_kv)
+    pools = [be.alloc_uninit((num_blocks, 16, e_kv), fa.capi.BF16) for _ in range(2)]
+    q = be.alloc_uninit((batch, l_new, e_q), fa.capi.BF16)
+    for i, b in enumerate(pools + [q]):
+        fa.check(lib.fa_fill_normal(be._ctx, b._h, 0, b.numel(), 21 + i, 0.0, 1.0))
+    out = be.alloc_uninit((batch, l_new, e_q), fa.capi.BF16)
+    args = fa.PagedAttentionArgs(layout, batch, l_new, heads, max_blocks, fa.default_scale(128), kv_heads)
+    d_tables, d_lens = be.upload(tables), be.upload(np.full(batch, l_new, np.uint32))
+    flops = 4.0 * batch * heads * 128 * l_new * (l_new + 1) / 2          # QK^T and PV over the causal triangle
+    res = []
+    for name, generic, reps in (("streamed", 0, 5), ("generic", 1, 1)):
+        fa.check(lib.fa_set_tuning(8, generic))
+        fn = lambda: fa.check(lib.fa_paged_attention_forward_device(be._ctx, q._h, pools[0]._h, pools[1]._h, d_tables._h,
+                                                                    d_lens._h, C.byref(args.c()), out._h))
+        fn()
+        be.synchronize_device()
+        t = Timer(fa, be)
+        t.start()
+        for _ in range(reps):
+            fn()
+        ms = t.stop_ms() / reps
+        res.append(dict(kernel=name, ms=ms, tflops=flops / (ms * 1e-3) / 1e12))
+    fa.check(lib.fa_set_tuning(8, 0))
+    for b in pools + [q, out, d_tables, d_lens]:
+        b.free()
+    return res
+
+
 def bench_matrix_rate(fa, be, iters=20000):
     """Register-only rate of the matrix instructions the prefill GEMMs use, with all-zero and with
     random operand bits (the sustained clock of the part depends on the bits it multiplies)."""
@@ -407,6 +442,9 @@ def main():
             for r in bench_prefill(fa, be, 20):
                 log("%s m=%d k=%d n=%d: %.1f us, %.0f TOPS (%.1f %% of peak)" %
                     (r["op"], r["m"], r["k"], r["n"], r["us"], r["tops"], 100 * r["frac"]))
+            for r in bench_prefill_attention(fa, be):
+                log("prefill attention 4 x 2048 new tokens, 32/8 heads, %s kernel: %.2f ms, %.1f TFLOP/s" %
+                    (r["kernel"], r["ms"], r["tflops"]))
             be.close()
             return
         if a.only == "mfma":

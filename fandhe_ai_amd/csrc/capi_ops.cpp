@@ -15,6 +15,7 @@ namespace k {
 extern int g_skinny_ntw, g_skinny_waves, g_skinny_astat, g_gemm_small_tiles, g_gemm_waves, g_gemm_ntb;
 }
 int g_decode_waves = 0;
+int g_prefill_generic = 0;
 extern int g_decode_partials_only;
 }  // namespace fa
 
@@ -77,6 +78,7 @@ fa_status fa_set_tuning(int32_t key, int32_t value) {
         case 5: k::g_skinny_astat = value; return FA_OK;
         case 6: k::g_gemm_waves = value; return FA_OK;
         case 7: k::g_gemm_ntb = value; return FA_OK;
+        case 8: fa::g_prefill_generic = value; return FA_OK;
     }
     return fail(FA_ERR_INVALID_ARGUMENT, "fa_set_tuning: unknown key");
 }

@@ -10,7 +10,7 @@
 using namespace fa;
 
 namespace fa {
-extern int g_decode_waves;
+extern int g_decode_waves, g_prefill_generic;
 }
 
 namespace {
@@ -42,9 +42,10 @@ k::PagedShape make_shape(const fa_paged_args *a) {
     return ps;
 }
 
-bool decode_fast_path(const k::PagedShape &ps, const fa_buffer *q) {
+// shapes of the streamed matrix-core kernel: one new token per row (decode) or several (prefill)
+bool stream_fast_path(const k::PagedShape &ps, const fa_buffer *q) {
     uint32_t group = ps.num_heads / ps.num_kv_heads;
-    return q->dtype == FA_BF16 && ps.head_dim == 128 && ps.block_size == 16 && ps.l_new == 1 && group <= 16 &&
+    return q->dtype == FA_BF16 && ps.head_dim == 128 && ps.block_size == 16 && ps.l_new >= 1 && group <= 16 &&
            ps.max_blocks_per_seq >= 1;
 }
 
@@ -53,7 +54,15 @@ fa_status launch_attention(fa_context *ctx, const fa_buffer *q, const fa_buffer 
                            const uint32_t *d_tables, const uint32_t *d_lens, const fa_paged_args *args,
                            uint64_t s_stride, fa_buffer *out) {
     k::PagedShape ps = make_shape(args);
-    if (decode_fast_path(ps, q)) {
+    if (stream_fast_path(ps, q) && ps.l_new > 1 && !g_prefill_generic) {
+        uint64_t need = k::paged_prefill_workspace_bytes(ps, (uint32_t)g_decode_waves);
+        if (fa_status s = ensure_workspace(ctx, need)) return s;
+        k::paged_attention_prefill_bf16((const uint16_t *)q->ptr, (const uint16_t *)k_pool->ptr,
+                                        (const uint16_t *)v_pool->ptr, d_tables, d_lens, ps, (uint32_t)g_decode_waves,
+                                        ctx->workspace, out->ptr, out->dtype == FA_BF16, ctx->stream);
+        return after_launch(ctx, "paged_attention_prefill_bf16");
+    }
+    if (stream_fast_path(ps, q) && ps.l_new == 1) {
         uint64_t need = k::paged_decode_workspace_bytes(ps, (uint32_t)g_decode_waves);
         if (fa_status s = ensure_workspace(ctx, need)) return s;
         k::paged_attention_decode_bf16((const uint16_t *)q->ptr, (const uint16_t *)k_pool->ptr,

@@ -156,10 +156,31 @@ struct StreamParams {
     uint32_t num_blocks, e_kv, batch, num_heads, num_kv_heads, group, g_pad, max_blocks_per_seq;
     uint32_t n_ranges, min_pages;
     float scale;
+    // Prefill (l_new > 1): the 16 columns of the score tile are tpt = 16 / group consecutive new tokens x
+    // the heads of the group (column = token-in-tile * group + head), and every such token tile of a
+    // sequence is streamed as a sequence of its own ("virtual sequence" b * qt + tile) whose length is the
+    // causal limit of its last token; columns are masked individually at their own limit.  One launch
+    // covers the new tokens [t0, t0 + qt * tpt) of every sequence.  Decode: l_new = tpt = qt = 1, t0 = 0.
+    uint32_t l_new, tpt, qt, t0, n_vseq;
 };
 
-__device__ __forceinline__ uint32_t seq_pages(const StreamParams &p, uint32_t b, uint32_t max_ctx) {
-    uint32_t len = p.seq_lens[b];
+// Length of (virtual) sequence vs: all cached positions up to the last new token of its tile.  A row whose
+// length is below l_new (possible only with unvalidated device tables) streams nothing.
+template <bool PF>
+__device__ __forceinline__ uint32_t vseq_len(const StreamParams &p, uint32_t vs) {
+    if constexpr (!PF) {
+        return p.seq_lens[vs];
+    } else {
+        const uint32_t len = p.seq_lens[vs / p.qt];
+        if (len < p.l_new) return 0;
+        uint32_t after = p.t0 + (vs % p.qt + 1) * p.tpt;
+        if (after > p.l_new) after = p.l_new;
+        return len - p.l_new + after;
+    }
+}
+template <bool PF>
+__device__ __forceinline__ uint32_t seq_pages(const StreamParams &p, uint32_t vs, uint32_t max_ctx) {
+    uint32_t len = vseq_len<PF>(p, vs);
     if (len > max_ctx) len = max_ctx;
     return (len + kPage - 1) / kPage;
 }
@@ -170,7 +191,7 @@ __device__ __forceinline__ uint32_t range_pages(const StreamParams &p, uint32_t 
     return per < p.min_pages ? p.min_pages : per;
 }
 
-template <int SP, int KD, int VD, int WPE>
+template <int SP, int KD, int VD, int WPE, bool PF>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) decode_stream_kernel(StreamParams p) {
     static_assert(SP % KD == 0 && SP % VD == 0, "static register indices need SP to be a multiple of the depths");
     __shared__ __attribute__((aligned(16))) uint16_t v_s[4][kPage * kVPitch];
@@ -181,8 +202,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, W
     const uint32_t kvh = item_id % p.num_kv_heads, r = item_id / p.num_kv_heads;
     if (r >= p.n_ranges) return;
     const uint32_t max_ctx = p.max_blocks_per_seq * kPage;
+    const uint32_t nv = PF ? p.n_vseq : p.batch;
     uint32_t total = 0;
-    for (uint32_t b = lane; b < p.batch; b += 64) total += seq_pages(p, b, max_ctx);
+    for (uint32_t b = lane; b < nv; b += 64) total += seq_pages<PF>(p, b, max_ctx);
     total = __builtin_amdgcn_readfirstlane(wave_sum<uint32_t>(total));
     const uint32_t per = range_pages(p, total);
     const uint64_t rlo64 = (uint64_t)r * per;
@@ -195,8 +217,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, W
     uint16_t *vs = &v_s[wave][0];
 
     uint32_t base = 0;
-    for (uint32_t b0 = 0; b0 < p.batch; b0 += 64) {
-        uint32_t len = b0 + lane < p.batch ? p.seq_lens[b0 + lane] : 0;
+    for (uint32_t b0 = 0; b0 < nv; b0 += 64) {
+        uint32_t len = b0 + lane < nv ? vseq_len<PF>(p, b0 + lane) : 0;
         uint32_t len_c = len > max_ctx ? max_ctx : len;
         uint32_t npg = (len_c + kPage - 1) / kPage;
         uint32_t incl = npg;
@@ -211,20 +233,24 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, W
         while (mask != 0) {
             const int src = __builtin_ctzll(mask);
             mask &= mask - 1;
-            const uint32_t b = b0 + src;
+            const uint32_t vq = b0 + src;                                // (virtual) sequence
+            const uint32_t b = PF ? vq / p.qt : vq;
             const uint32_t sb = __builtin_amdgcn_readfirstlane(__shfl(s_b, src, 64));
             const uint32_t eb = __builtin_amdgcn_readfirstlane(__shfl(e_b, src, 64));
             const uint32_t len_b = __builtin_amdgcn_readfirstlane(__shfl(len, src, 64));
             bool bad = len_b > max_ctx;
-            const uint32_t ctx = bad ? max_ctx : len_b;
+            if constexpr (PF) bad = p.seq_lens[b] > max_ctx;
+            const uint32_t ctx = len_b > max_ctx ? max_ctx : len_b;
             const uint32_t lo = (rlo > sb ? rlo : sb) - sb;            // first page of the segment, in the sequence
             const uint32_t hi = (rhi < eb ? rhi : eb) - sb;
             const uint32_t n = hi - lo;                                // pages of this segment (>= 1)
             const uint32_t *tab = p.tables + (uint64_t)b * p.max_blocks_per_seq + lo;
 
-            // Q^T operand: column c = head of the group (zero beyond the group)
+            // Q^T operand: column c = head of the group (zero beyond the group); prefill: column c = new
+            // token c / group of the tile, head c % group, masked at that token's own causal limit
             v8bf qb[4];
-            {
+            uint32_t ctx_l = ctx;                                      // this lane's column sees tokens below ctx_l
+            if constexpr (!PF) {
                 const uint32_t hc = (uint32_t)c < p.group ? (uint32_t)c : 0;
                 const uint16_t *qrow = p.q + ((uint64_t)b * p.num_heads + (uint64_t)kvh * p.group + hc) * kDh + 8 * g;
 #pragma unroll
@@ -233,6 +259,23 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, W
                     if ((uint32_t)c >= p.group) t = v4u{0, 0, 0, 0};
                     qb[s] = __builtin_bit_cast(v8bf, t);
                 }
+            } else {
+                const uint32_t tl = (uint32_t)c / p.group, hc = (uint32_t)c % p.group;
+                const uint32_t t = p.t0 + (vq % p.qt) * p.tpt + tl;
+                const bool valid = tl < p.tpt && t < p.l_new;
+                const uint32_t tc = valid ? t : 0;
+                const uint16_t *qrow =
+                    p.q + (((uint64_t)b * p.l_new + tc) * p.num_heads + (uint64_t)kvh * p.group + hc) * kDh + 8 * g;
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    v4u t4 = *(const v4u *)(qrow + 32 * s);
+                    if (!valid) t4 = v4u{0, 0, 0, 0};
+                    qb[s] = __builtin_bit_cast(v8bf, t4);
+                }
+                // cached positions before the new tokens + new tokens up to and including t; never above ctx,
+                // which is already clamped to what the table can describe
+                const uint32_t lim = p.seq_lens[b] - p.l_new + t + 1;
+                if (valid) ctx_l = lim < ctx ? lim : ctx;
             }
             // Block ids of 64 pages at a time, one per lane (idv), with the following 64 (idv_next) already
             // resident.  Everything below is straight-line code per group: loads past the end of the
@@ -305,7 +348,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, W
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
                         uint32_t tok = (lo + pg) * kPage + 4 * g + j;
-                        float s = pg < n && tok < ctx ? acc[j] * p.scale : -INFINITY;
+                        float s = pg < n && tok < ctx_l ? acc[j] * p.scale : -INFINITY;
                         sc[i][j] = s;
                         mx = fmaxf(mx, s);
                     }
@@ -314,14 +357,17 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, W
                 mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
                 mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
                 const float m_new = fmaxf(m_run, mx);
-                const float alpha = expf(m_run - m_new);               // first group: exp(-inf) = 0
+                // prefill: a column can have every score of a segment masked (the segment lies past its
+                // causal limit); its maximum stays -inf and the exponentials are taken against 0 instead
+                const float m_use = (PF && m_new == -INFINITY) ? 0.0f : m_new;
+                const float alpha = expf(m_run - m_use);               // first group: exp(-inf) = 0
                 m_run = m_new;
                 float gsum = 0.0f;
 #pragma unroll
                 for (int i = 0; i < SP; ++i)
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        float e = expf(sc[i][j] - m_new);              // masked scores: exp(-inf) = 0
+                        float e = expf(sc[i][j] - m_use);              // masked scores: exp(-inf) = 0
                         sc[i][j] = e;
                         gsum += e;
                     }
@@ -387,8 +433,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, W
             l_run += __shfl_xor(l_run, 16, 64);
             l_run += __shfl_xor(l_run, 32, 64);
             // lane (g, c) holds, for head c: dims 32 bp + 8 g + {0..7} = {o[2bp][0], o[2bp+1][0], o[2bp][1], ...}
-            const uint64_t item = (uint64_t)(r + b) * p.num_kv_heads + kvh;
-            if ((uint32_t)c < p.group) {
+            const uint64_t item = (uint64_t)(r + vq) * p.num_kv_heads + kvh;
+            if ((uint32_t)c < (PF ? p.tpt * p.group : p.group)) {
                 float *po = p.part_o + (item * p.g_pad + c) * kDh + 8 * g;
 #pragma unroll
                 for (int bp = 0; bp < 4; ++bp) {
@@ -407,16 +453,29 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, W
 
 // Merges the partial results of one (sequence, query head): block = 256 threads,
 // thread (part, d) sums every second partial for dim d, then the two parts are added.
+// Prefill: blockIdx.y = sequence * (tokens of this launch) + token; the partials of the token's tile are
+// merged for the tile column of (token, head).
+template <bool PF>
 __global__ void __launch_bounds__(256) decode_stream_merge_kernel(StreamParams p, void *__restrict__ out, int out_bf16,
                                                                  float *__restrict__ pmax) {
     __shared__ float s_acc[128], s_den, s_max[2];
     __shared__ uint32_t s_tot[4], s_pre[4];
-    const uint32_t h = blockIdx.x, b = blockIdx.y, d = threadIdx.x % 128, part = threadIdx.x / 128;
-    const uint32_t kvh = h / p.group, hg = h % p.group;
+    const uint32_t h = blockIdx.x, d = threadIdx.x % 128, part = threadIdx.x / 128;
+    const uint32_t kvh = h / p.group;
+    uint32_t b = blockIdx.y, hg = h % p.group, out_row = blockIdx.y, seq = blockIdx.y;
+    if constexpr (PF) {
+        const uint32_t ct = p.qt * p.tpt < p.l_new - p.t0 ? p.qt * p.tpt : p.l_new - p.t0;   // tokens of this launch
+        seq = blockIdx.y / ct;
+        const uint32_t tt = blockIdx.y % ct;
+        b = seq * p.qt + tt / p.tpt;                               // virtual sequence
+        hg = (tt % p.tpt) * p.group + h % p.group;                 // tile column
+        out_row = seq * p.l_new + p.t0 + tt;
+    }
+    const uint32_t nv = PF ? p.n_vseq : p.batch;
     const uint32_t max_ctx = p.max_blocks_per_seq * kPage;
     uint32_t tot = 0, pre = 0;
-    for (uint32_t bb = threadIdx.x; bb < p.batch; bb += 256) {
-        uint32_t v = seq_pages(p, bb, max_ctx);
+    for (uint32_t bb = threadIdx.x; bb < nv; bb += 256) {
+        uint32_t v = seq_pages<PF>(p, bb, max_ctx);
         tot += v;
         if (bb < b) pre += v;
     }
@@ -429,10 +488,11 @@ __global__ void __launch_bounds__(256) decode_stream_merge_kernel(StreamParams p
     __syncthreads();
     tot = s_tot[0] + s_tot[1] + s_tot[2] + s_tot[3];
     pre = s_pre[0] + s_pre[1] + s_pre[2] + s_pre[3];
-    const uint32_t npg = seq_pages(p, b, max_ctx);
+    const uint32_t npg = seq_pages<PF>(p, b, max_ctx);
     const uint32_t per = range_pages(p, tot);
     const uint32_t r_lo = npg ? pre / per : 1, r_hi = npg ? (pre + npg - 1) / per : 0;   // empty sequence: no partials
     float mx = -INFINITY;
+    if (PF && p.seq_lens[seq] < p.l_new) mx = __uint_as_float(0x7fc00000u);             // violation: NaN out
     for (uint32_t r = r_lo; r <= r_hi; ++r) {
         float m = p.part_ml[((uint64_t)(r + b) * p.num_kv_heads + kvh) * (2 * p.g_pad) + hg];
         mx = (m != m || mx != mx) ? __uint_as_float(0x7fc00000u) : fmaxf(mx, m);   // NaN marks a violation
@@ -455,8 +515,8 @@ __global__ void __launch_bounds__(256) decode_stream_merge_kernel(StreamParams p
     if (part == 0) {
         acc += s_acc[d];
         den += s_den;
-        float res = npg == 0 ? 0.0f : __fdiv_rn(acc, den);
-        uint64_t oi = ((uint64_t)b * p.num_heads + h) * kDh + d;
+        float res = npg == 0 ? (mx != mx ? mx : 0.0f) : __fdiv_rn(acc, den);
+        uint64_t oi = ((uint64_t)out_row * p.num_heads + h) * kDh + d;
         if (out_bf16) {
             uint16_t rb = f32_to_bf16(res);
             ((uint16_t *)out)[oi] = rb;
@@ -470,7 +530,7 @@ __global__ void __launch_bounds__(256) decode_stream_merge_kernel(StreamParams p
         a = wave_max(a);
         if (part == 0 && threadIdx.x % 64 == 0) s_max[threadIdx.x / 64] = a;
         __syncthreads();
-        if (threadIdx.x == 0) pmax[(uint64_t)b * p.num_heads + h] = fmaxf(s_max[0], s_max[1]);
+        if (threadIdx.x == 0) pmax[(uint64_t)out_row * p.num_heads + h] = fmaxf(s_max[0], s_max[1]);
     }
 }
 
@@ -493,7 +553,7 @@ __global__ void __launch_bounds__(1024) decode_stream_merge_quantize_kernel(Stre
     const uint32_t max_ctx = p.max_blocks_per_seq * kPage;
     uint32_t tot = 0, pre = 0;
     for (uint32_t bb = threadIdx.x; bb < p.batch; bb += blockDim.x) {
-        uint32_t v = seq_pages(p, bb, max_ctx);
+        uint32_t v = seq_pages<false>(p, bb, max_ctx);
         tot += v;
         if (bb < b) pre += v;
     }
@@ -510,7 +570,7 @@ __global__ void __launch_bounds__(1024) decode_stream_merge_quantize_kernel(Stre
         tot += s_tot[w];
         pre += s_pre[w];
     }
-    const uint32_t npg = seq_pages(p, b, max_ctx);
+    const uint32_t npg = seq_pages<false>(p, b, max_ctx);
     const uint32_t per = range_pages(p, tot);
     const uint32_t r_lo = npg ? pre / per : 1, r_hi = npg ? (pre + npg - 1) / per : 0;   // empty sequence: no partials
 
@@ -675,11 +735,14 @@ void paged_attention_decode_bf16(const uint16_t *q, const uint16_t *k_pool, cons
     sp.n_ranges = stream_ranges(ps, waves_per_cu);
     sp.min_pages = 4;
     sp.scale = ps.scale;
+    sp.l_new = sp.tpt = sp.qt = 1;
+    sp.t0 = 0;
+    sp.n_vseq = ps.batch;
     uint64_t items = ((uint64_t)sp.n_ranges + ps.batch) * ps.num_kv_heads;
     sp.part_o = (float *)workspace;
     sp.part_ml = sp.part_o + items * (uint64_t)sp.g_pad * kDh;
     uint64_t waves = (uint64_t)sp.n_ranges * ps.num_kv_heads;
-    decode_stream_kernel<4, 4, 2, 2><<<(unsigned)((waves + 3) / 4), 256, 0, s>>>(sp);
+    decode_stream_kernel<4, 4, 2, 2, false><<<(unsigned)((waves + 3) / 4), 256, 0, s>>>(sp);
     if (g_decode_partials_only) return;
     if (xq_tiled != nullptr && ps.num_heads <= 32) {
         // fused merge + per-token quantizer (the bf16 output itself is not written)
@@ -687,7 +750,65 @@ void paged_attention_decode_bf16(const uint16_t *q, const uint16_t *k_pool, cons
         return;
     }
     dim3 grid2(ps.num_heads, ps.batch);
-    decode_stream_merge_kernel<<<grid2, 256, 0, s>>>(sp, out, out_bf16, pmax);
+    decode_stream_merge_kernel<false><<<grid2, 256, 0, s>>>(sp, out, out_bf16, pmax);
+}
+
+// Prefill (l_new > 1) on the same streaming kernel: token tiles of 16 / group new tokens are streamed as
+// sequences of their own, at most kPrefillTiles of them per launch so that the partial results stay within
+// a bounded workspace; the launches for successive token ranges follow each other on the stream.
+constexpr uint32_t kPrefillTiles = 1024;
+
+static uint32_t prefill_tiles_per_seq(const PagedShape &ps) {          // token tiles of one sequence per launch
+    uint32_t per_seq = kPrefillTiles / ps.batch;
+    return per_seq ? per_seq : 1;
+}
+
+uint64_t paged_prefill_workspace_bytes(const PagedShape &ps, uint32_t waves_per_cu) {
+    uint32_t tpt = 16 / (ps.num_heads / ps.num_kv_heads);
+    uint32_t tiles = (ps.l_new + tpt - 1) / tpt;
+    uint32_t qt = tiles < prefill_tiles_per_seq(ps) ? tiles : prefill_tiles_per_seq(ps);
+    uint64_t items = ((uint64_t)stream_ranges(ps, waves_per_cu) + (uint64_t)ps.batch * qt) * ps.num_kv_heads;
+    return items * (16 * kDh + 2 * 16) * sizeof(float);
+}
+
+void paged_attention_prefill_bf16(const uint16_t *q, const uint16_t *k_pool, const uint16_t *v_pool,
+                                  const uint32_t *tables, const uint32_t *seq_lens, const PagedShape &ps,
+                                  uint32_t waves_per_cu, void *workspace, void *out, int out_bf16, hipStream_t s) {
+    if (ps.batch == 0 || ps.l_new == 0) return;
+    StreamParams sp;
+    sp.q = q;
+    sp.k_pool = k_pool;
+    sp.v_pool = v_pool;
+    sp.tables = tables;
+    sp.seq_lens = seq_lens;
+    sp.num_blocks = ps.num_blocks;
+    sp.e_kv = ps.e_kv;
+    sp.batch = ps.batch;
+    sp.num_heads = ps.num_heads;
+    sp.num_kv_heads = ps.num_kv_heads;
+    sp.group = ps.num_heads / ps.num_kv_heads;
+    sp.g_pad = 16;
+    sp.max_blocks_per_seq = ps.max_blocks_per_seq;
+    sp.n_ranges = stream_ranges(ps, waves_per_cu);
+    sp.min_pages = 4;
+    sp.scale = ps.scale;
+    sp.l_new = ps.l_new;
+    sp.tpt = 16 / sp.group;
+    const uint32_t tiles = (ps.l_new + sp.tpt - 1) / sp.tpt;
+    const uint32_t qt_max = tiles < prefill_tiles_per_seq(ps) ? tiles : prefill_tiles_per_seq(ps);
+    const uint64_t items_max = ((uint64_t)sp.n_ranges + (uint64_t)ps.batch * qt_max) * ps.num_kv_heads;
+    sp.part_o = (float *)workspace;
+    sp.part_ml = sp.part_o + items_max * 16 * kDh;
+    const uint64_t waves = (uint64_t)sp.n_ranges * ps.num_kv_heads;
+    for (uint32_t tile0 = 0; tile0 < tiles; tile0 += qt_max) {
+        sp.qt = tiles - tile0 < qt_max ? tiles - tile0 : qt_max;
+        sp.t0 = tile0 * sp.tpt;
+        sp.n_vseq = ps.batch * sp.qt;
+        const uint32_t ct = sp.qt * sp.tpt < ps.l_new - sp.t0 ? sp.qt * sp.tpt : ps.l_new - sp.t0;
+        decode_stream_kernel<4, 4, 2, 2, true><<<(unsigned)((waves + 3) / 4), 256, 0, s>>>(sp);
+        dim3 grid2(ps.num_heads, ps.batch * ct);
+        decode_stream_merge_kernel<true><<<grid2, 256, 0, s>>>(sp, out, out_bf16, nullptr);
+    }
 }
 
 }  // namespace k

@@ -155,6 +155,13 @@ void paged_attention_decode_bf16(const uint16_t *q, const uint16_t *k_pool, cons
                                  uint32_t waves_per_cu, void *workspace, void *out, int out_bf16, float *pmax,
                                  int8_t *xq_tiled, float *sx, uint32_t m_pad, hipStream_t s);
 
+// Prefill fast path: bf16, head_dim 128, block_size 16, l_new > 1, group <= 16.  Causal over the cached
+// positions: new token t of a row sees positions below seq_len - l_new + t + 1.
+uint64_t paged_prefill_workspace_bytes(const PagedShape &ps, uint32_t waves_per_cu);
+void paged_attention_prefill_bf16(const uint16_t *q, const uint16_t *k_pool, const uint16_t *v_pool,
+                                  const uint32_t *tables, const uint32_t *seq_lens, const PagedShape &ps,
+                                  uint32_t waves_per_cu, void *workspace, void *out, int out_bf16, hipStream_t s);
+
 // ---- measurement aid (kern_probe.hip) -------------------------------------------
 // Launches a register-only loop of one matrix instruction kind (0: i32_16x16x64_i8, 1: i32_32x32x32_i8,
 // 2: scaled f32_16x16x128 on e4m3) whose operand bits come from `operands` (64 KiB); returns the number

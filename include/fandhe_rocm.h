@@ -423,7 +423,9 @@ fa_status fa_decoder_read_seq_lens(fa_context *ctx, fa_decoder *dec, uint32_t *s
  * key 4: nonzero keeps the 128 x 128 block tile of the prefill GEMMs for every shape;
  * key 5: activation-stationary decode linears: 1 never, 2 whenever the shape allows;
  * key 6: wavefronts per block of the large-tile prefill GEMMs (4 or 16; default 8);
- * key 7: column tiles of 16 per block of the large-tile prefill GEMMs (14 or 16). */
+ * key 7: column tiles of 16 per block of the large-tile prefill GEMMs (14 or 16);
+ * key 8: nonzero sends attention with more than one new token per row to the generic
+ *        kernel (the reference's summation order) instead of the streamed one. */
 fa_status fa_set_tuning(int32_t key, int32_t value);
 /* A pair of HIP events recorded on the context's stream (the stream the
  * kernels run on); used by the benchmark to time launches. */

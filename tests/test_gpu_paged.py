@@ -242,6 +242,91 @@ def test_bf16_decode_properties_at_benchmark_size():
     assert np.allclose(got3, 1.5, rtol=1e-5, atol=0)
 
 
+PREFILL_CASES = [
+    # heads, kv_heads, l_new, total lengths per row (>= l_new)
+    (32, 8, 2, [2, 17, 300]), (32, 8, 3, [3, 16, 50]), (32, 8, 4, [4, 20, 33]), (32, 8, 5, [5, 21, 100]),
+    (32, 8, 16, [16, 17, 64]), (32, 8, 17, [17, 31, 200]), (32, 8, 37, [37, 38, 500]), (32, 8, 200, [200, 333, 777]),
+    (8, 8, 19, [19, 40]), (8, 4, 9, [9, 100]), (16, 2, 11, [11, 64]), (16, 1, 6, [6, 90]), (6, 2, 13, [13, 70]),
+    (5, 1, 7, [7, 40]),
+]
+
+
+@pytest.mark.parametrize("heads,kv_heads,l_new,lens", PREFILL_CASES,
+                         ids=["H%d_%d_L%d" % c[:3] for c in PREFILL_CASES])
+def test_bf16_prefill_on_the_streaming_kernel_against_the_oracle(heads, kv_heads, l_new, lens):
+    """l_new > 1 with page 16 / head_dim 128: token tiles of 16 / group new tokens on the matrix cores,
+    each masked at its own causal limit; rows differ in how much was cached before the new tokens."""
+    fa = _fa()
+    be = ops()
+    rng = o.Rng(1000 * heads + 10 * l_new + kv_heads)
+    batch, num_blocks = len(lens), 160
+    tables, seq_lens, max_blocks, e_kv, e_q = _decode_case(rng, batch, heads, kv_heads, lens, num_blocks, extra_slots=2)
+    kp = o.to_bf16(rng.randn((num_blocks, 16, e_kv)))
+    vp = o.to_bf16(rng.randn((num_blocks, 16, e_kv)))
+    q = o.to_bf16(rng.randn((batch, l_new, e_q)))
+    layout = fa.PagedKvLayout.new(num_blocks, 16, e_kv)
+    args = fa.PagedAttentionArgs(layout, batch, l_new, heads, max_blocks, fa.default_scale(128), kv_heads)
+    oargs = o.paged_args(num_blocks, 16, e_kv, batch, l_new, heads, max_blocks, args.scale, kv_heads)
+    o.set_threads(8)
+    rc, want = o.paged_attention_bf16(q, kp, vp, tables, seq_lens, oargs)
+    o.set_threads(1)
+    assert rc == 0
+    dq, dk, dv = be.upload(q), be.upload(kp), be.upload(vp)
+    for waves in (0, 1, 8):           # few long ranges / many short ones: different cuts through the token tiles
+        fa.check(fa.capi.lib.fa_set_tuning(2, waves))
+        got = be.download_owned(be.paged_attention_forward(dq, dk, dv, tables, seq_lens, args, out_dtype=fa.capi.F32))
+        assert_parity("PAGED_PREFILL_PARITY", f"H{heads}/{kv_heads}:L{l_new}:waves{waves}", got, want)
+    fa.check(fa.capi.lib.fa_set_tuning(2, 0))
+    got = be.download_owned(be.paged_attention_forward(dq, dk, dv, tables, seq_lens, args, out_dtype=fa.capi.F32))
+    got_bf = be.download_owned(be.paged_attention_forward(dq, dk, dv, tables, seq_lens, args))
+    assert_bf16_rounding_of("paged prefill bf16", got_bf, got)      # same launch shape: same f32 values
+    # the first new token of a row that had nothing cached sees only itself: its output is its own V row
+    for h in range(heads):
+        gq = h // (heads // kv_heads)
+        assert np.array_equal(got_bf[0, 0, h * 128:(h + 1) * 128], vp[tables[0, 0], 0, gq * 128:(gq + 1) * 128])
+    # device-resident tables: same bits
+    got_dev = be.download_owned(be.paged_attention_forward_device(dq, dk, dv, be.upload(tables), be.upload(seq_lens), args))
+    assert np.array_equal(got_dev, got_bf)
+    # the last new token equals a one-token decode call over the same cache
+    q_last = np.ascontiguousarray(q[:, -1:, :])
+    args1 = fa.PagedAttentionArgs(layout, batch, 1, heads, max_blocks, fa.default_scale(128), kv_heads)
+    dec = be.download_owned(be.paged_attention_forward(be.upload(q_last), dk, dv, tables, seq_lens, args1,
+                                                       out_dtype=fa.capi.F32))
+    assert_parity("PREFILL_LAST_VS_DECODE", f"H{heads}/{kv_heads}:L{l_new}", got[:, -1:, :], dec)
+
+
+def test_bf16_prefill_in_several_launches_matches_one_token_at_a_time():
+    """More token tiles than one launch holds (batch 6 x 800 new tokens, 4 tokens per tile): the launches over
+    successive token ranges together equal 800 single-token calls on sampled positions."""
+    fa = _fa()
+    be = ops()
+    rng = o.Rng(77)
+    heads, kv_heads, l_new, batch, num_blocks = 32, 8, 800, 6, 400
+    lens = [800, 801, 815, 816, 900, 1000]
+    tables, seq_lens, max_blocks, e_kv, e_q = _decode_case(rng, batch, heads, kv_heads, lens, num_blocks)
+    kp = o.to_bf16(rng.randn((num_blocks, 16, e_kv)))
+    vp = o.to_bf16(rng.randn((num_blocks, 16, e_kv)))
+    q = o.to_bf16(rng.randn((batch, l_new, e_q)))
+    layout = fa.PagedKvLayout.new(num_blocks, 16, e_kv)
+    args = fa.PagedAttentionArgs(layout, batch, l_new, heads, max_blocks, fa.default_scale(128), kv_heads)
+    dq, dk, dv = be.upload(q), be.upload(kp), be.upload(vp)
+    got = be.download_owned(be.paged_attention_forward(dq, dk, dv, tables, seq_lens, args, out_dtype=fa.capi.F32))
+    assert np.all(np.isfinite(got))
+    args1 = fa.PagedAttentionArgs(layout, batch, 1, heads, max_blocks, fa.default_scale(128), kv_heads)
+    for t in (0, 1, 3, 4, 170, 171, 682, 683, 684, 799):
+        lens_t = (seq_lens - l_new + t + 1).astype(np.uint32)
+        dec = be.download_owned(be.paged_attention_forward(be.upload(np.ascontiguousarray(q[:, t:t + 1, :])), dk, dv,
+                                                           tables, lens_t, args1, out_dtype=fa.capi.F32))
+        assert_parity("PREFILL_VS_DECODE", f"t{t}", got[:, t:t + 1, :], dec)
+    oargs = o.paged_args(num_blocks, 16, e_kv, 1, l_new, heads, max_blocks, args.scale, kv_heads)
+    o.set_threads(8)
+    rc, want = o.paged_attention_bf16(np.ascontiguousarray(q[4:5]), kp, vp, np.ascontiguousarray(tables[4:5]),
+                                      np.ascontiguousarray(seq_lens[4:5]), oargs)
+    o.set_threads(1)
+    assert rc == 0
+    assert_parity("PAGED_PREFILL_PARITY", "row4 of 6 x 800", got[4:5], want)
+
+
 def test_bf16_generic_path_covers_shapes_outside_the_fast_path():
     fa = _fa()
     be = ops()
