@@ -159,9 +159,11 @@ struct StreamParams {
     // Prefill (l_new > 1): the 16 columns of the score tile are tpt = 16 / group consecutive new tokens x
     // the heads of the group (column = token-in-tile * group + head), and every such token tile of a
     // sequence is streamed as a sequence of its own ("virtual sequence" b * qt + tile) whose length is the
-    // causal limit of its last token; columns are masked individually at their own limit.  One launch
-    // covers the new tokens [t0, t0 + qt * tpt) of every sequence.  Decode: l_new = tpt = qt = 1, t0 = 0.
-    uint32_t l_new, tpt, qt, t0, n_vseq;
+    // causal limit of its last token; columns are masked individually at their own limit.  A wavefront
+    // carries TT token tiles at once (tpv = TT * tpt tokens per virtual sequence), so K / V are read once
+    // per tpv new tokens.  One launch covers the new tokens [t0, t0 + qt * tpv) of every sequence.
+    // Decode: l_new = tpt = tpv = qt = 1, t0 = 0.
+    uint32_t l_new, tpt, tpv, qt, t0, n_vseq;
 };
 
 // Length of (virtual) sequence vs: all cached positions up to the last new token of its tile.  A row whose
@@ -173,7 +175,7 @@ __device__ __forceinline__ uint32_t vseq_len(const StreamParams &p, uint32_t vs)
     } else {
         const uint32_t len = p.seq_lens[vs / p.qt];
         if (len < p.l_new) return 0;
-        uint32_t after = p.t0 + (vs % p.qt + 1) * p.tpt;
+        uint32_t after = p.t0 + (vs % p.qt + 1) * p.tpv;
         if (after > p.l_new) after = p.l_new;
         return len - p.l_new + after;
     }
@@ -191,8 +193,9 @@ __device__ __forceinline__ uint32_t range_pages(const StreamParams &p, uint32_t 
     return per < p.min_pages ? p.min_pages : per;
 }
 
-template <int SP, int KD, int VD, int WPE, bool PF>
+template <int SP, int KD, int VD, int WPE, bool PF, int TT = 1>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) decode_stream_kernel(StreamParams p) {
+    static_assert(PF || TT == 1, "several token tiles per wavefront exist only in the prefill form");
     static_assert(SP % KD == 0 && SP % VD == 0, "static register indices need SP to be a multiple of the depths");
     __shared__ __attribute__((aligned(16))) uint16_t v_s[4][kPage * kVPitch];
     const int lane = threadIdx.x % 64;
@@ -248,34 +251,38 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, W
 
             // Q^T operand: column c = head of the group (zero beyond the group); prefill: column c = new
             // token c / group of the tile, head c % group, masked at that token's own causal limit
-            v8bf qb[4];
-            uint32_t ctx_l = ctx;                                      // this lane's column sees tokens below ctx_l
+            v8bf qb[TT][4];
+            uint32_t ctx_l[TT];                                        // this lane's column sees tokens below ctx_l
             if constexpr (!PF) {
+                ctx_l[0] = ctx;
                 const uint32_t hc = (uint32_t)c < p.group ? (uint32_t)c : 0;
                 const uint16_t *qrow = p.q + ((uint64_t)b * p.num_heads + (uint64_t)kvh * p.group + hc) * kDh + 8 * g;
 #pragma unroll
                 for (int s = 0; s < 4; ++s) {
                     v4u t = *(const v4u *)(qrow + 32 * s);
                     if ((uint32_t)c >= p.group) t = v4u{0, 0, 0, 0};
-                    qb[s] = __builtin_bit_cast(v8bf, t);
+                    qb[0][s] = __builtin_bit_cast(v8bf, t);
                 }
             } else {
                 const uint32_t tl = (uint32_t)c / p.group, hc = (uint32_t)c % p.group;
-                const uint32_t t = p.t0 + (vq % p.qt) * p.tpt + tl;
-                const bool valid = tl < p.tpt && t < p.l_new;
-                const uint32_t tc = valid ? t : 0;
-                const uint16_t *qrow =
-                    p.q + (((uint64_t)b * p.l_new + tc) * p.num_heads + (uint64_t)kvh * p.group + hc) * kDh + 8 * g;
 #pragma unroll
-                for (int s = 0; s < 4; ++s) {
-                    v4u t4 = *(const v4u *)(qrow + 32 * s);
-                    if (!valid) t4 = v4u{0, 0, 0, 0};
-                    qb[s] = __builtin_bit_cast(v8bf, t4);
+                for (int tt = 0; tt < TT; ++tt) {
+                    const uint32_t t = p.t0 + (vq % p.qt) * p.tpv + tt * p.tpt + tl;
+                    const bool valid = tl < p.tpt && t < p.l_new;
+                    const uint32_t tc = valid ? t : 0;
+                    const uint16_t *qrow =
+                        p.q + (((uint64_t)b * p.l_new + tc) * p.num_heads + (uint64_t)kvh * p.group + hc) * kDh + 8 * g;
+#pragma unroll
+                    for (int s = 0; s < 4; ++s) {
+                        v4u t4 = *(const v4u *)(qrow + 32 * s);
+                        if (!valid) t4 = v4u{0, 0, 0, 0};
+                        qb[tt][s] = __builtin_bit_cast(v8bf, t4);
+                    }
+                    // cached positions before the new tokens + new tokens up to and including t; never above
+                    // ctx, which is already clamped to what the table can describe
+                    const uint32_t lim = p.seq_lens[b] - p.l_new + t + 1;
+                    ctx_l[tt] = valid && lim < ctx ? lim : ctx;
                 }
-                // cached positions before the new tokens + new tokens up to and including t; never above ctx,
-                // which is already clamped to what the table can describe
-                const uint32_t lim = p.seq_lens[b] - p.l_new + t + 1;
-                if (valid) ctx_l = lim < ctx ? lim : ctx;
             }
             // Block ids of 64 pages at a time, one per lane (idv), with the following 64 (idv_next) already
             // resident.  Everything below is straight-line code per group: loads past the end of the
@@ -319,10 +326,15 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, W
                 __builtin_amdgcn_sched_barrier(0);
             }
 
-            float m_run = -INFINITY, l_run = 0.0f;
-            v4f o[8];
+            float m_run[TT], l_run[TT];
+            v4f o[TT][8];
 #pragma unroll
-            for (int t = 0; t < 8; ++t) o[t] = v4f{0.f, 0.f, 0.f, 0.f};
+            for (int tt = 0; tt < TT; ++tt) {
+                m_run[tt] = -INFINITY;
+                l_run[tt] = 0.0f;
+#pragma unroll
+                for (int t = 0; t < 8; ++t) o[tt][t] = v4f{0.f, 0.f, 0.f, 0.f};
+            }
 
             // 64 is a multiple of SP, so a group never straddles two id windows; the loads issued from a
             // group reach at most max(KD, VD) <= SP pages past it, i.e. at most into the next window
@@ -332,48 +344,60 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, W
                 const uint32_t cand = tab_at(win + 128 + lane);
                 __builtin_amdgcn_sched_barrier(0);
                 // ---- scores of the group
-                float sc[SP][4];
-                float mx = -INFINITY;
+                float sc[TT][SP][4];
+                float mx[TT];
+#pragma unroll
+                for (int tt = 0; tt < TT; ++tt) mx[tt] = -INFINITY;
 #pragma unroll
                 for (int i = 0; i < SP; ++i) {
                     const uint32_t pg = p0 + i;
-                    v4f acc = v4f{0.f, 0.f, 0.f, 0.f};
+                    v4f acc[TT];
 #pragma unroll
-                    for (int s = 0; s < 4; ++s)
-                        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, kreg[i % KD][s]), qb[s],
-                                                                      acc, 0, 0, 0);
+                    for (int tt = 0; tt < TT; ++tt) {
+                        acc[tt] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                        for (int s = 0; s < 4; ++s)
+                            acc[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, kreg[i % KD][s]),
+                                                                              qb[tt][s], acc[tt], 0, 0, 0);
+                    }
                     __builtin_amdgcn_sched_barrier(0);                 // keep the request right behind its consumer
                     load_k(pg + KD, kreg[i % KD]);
                     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        uint32_t tok = (lo + pg) * kPage + 4 * g + j;
-                        float s = pg < n && tok < ctx_l ? acc[j] * p.scale : -INFINITY;
-                        sc[i][j] = s;
-                        mx = fmaxf(mx, s);
-                    }
+                    for (int tt = 0; tt < TT; ++tt)
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            uint32_t tok = (lo + pg) * kPage + 4 * g + j;
+                            float s = pg < n && tok < ctx_l[tt] ? acc[tt][j] * p.scale : -INFINITY;
+                            sc[tt][i][j] = s;
+                            mx[tt] = fmaxf(mx[tt], s);
+                        }
                 }
-                // ---- running maximum and sum per head (lanes with equal c hold one head)
-                mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-                const float m_new = fmaxf(m_run, mx);
-                // prefill: a column can have every score of a segment masked (the segment lies past its
-                // causal limit); its maximum stays -inf and the exponentials are taken against 0 instead
-                const float m_use = (PF && m_new == -INFINITY) ? 0.0f : m_new;
-                const float alpha = expf(m_run - m_use);               // first group: exp(-inf) = 0
-                m_run = m_new;
-                float gsum = 0.0f;
+                // ---- running maximum and sum per column (lanes with equal c hold one column)
 #pragma unroll
-                for (int i = 0; i < SP; ++i)
+                for (int tt = 0; tt < TT; ++tt) {
+                    float m = mx[tt];
+                    m = fmaxf(m, __shfl_xor(m, 16, 64));
+                    m = fmaxf(m, __shfl_xor(m, 32, 64));
+                    const float m_new = fmaxf(m_run[tt], m);
+                    // prefill: a column can have every score of a segment masked (the segment lies past its
+                    // causal limit); its maximum stays -inf and the exponentials are taken against 0 instead
+                    const float m_use = (PF && m_new == -INFINITY) ? 0.0f : m_new;
+                    const float alpha = expf(m_run[tt] - m_use);       // first group: exp(-inf) = 0
+                    m_run[tt] = m_new;
+                    float gsum = 0.0f;
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        float e = expf(sc[i][j] - m_use);              // masked scores: exp(-inf) = 0
-                        sc[i][j] = e;
-                        gsum += e;
-                    }
-                l_run = __builtin_fmaf(l_run, alpha, gsum);
+                    for (int i = 0; i < SP; ++i)
 #pragma unroll
-                for (int t = 0; t < 8; ++t) o[t] = o[t] * alpha;
+                        for (int j = 0; j < 4; ++j) {
+                            float e = expf(sc[tt][i][j] - m_use);      // masked scores: exp(-inf) = 0
+                            sc[tt][i][j] = e;
+                            gsum += e;
+                        }
+                    l_run[tt] = __builtin_fmaf(l_run[tt], alpha, gsum);
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) o[tt][t] = o[tt][t] * alpha;
+                }
                 // ---- O^T += V^T P^T
 #pragma unroll
                 for (int i = 0; i < SP; ++i) {
@@ -393,19 +417,25 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, W
                     __builtin_amdgcn_wave_barrier();
                     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
                     // each f32 weight as three bf16 operands by repeated truncation: hi + mid + lo == p exactly
-                    uint32_t whi[4], wmid[4], wlo[4];
+                    v4s b_hi[TT], b_mid[TT], b_lo[TT];
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        float pj = sc[i][j];
-                        whi[j] = __float_as_uint(pj) & 0xffff0000u;
-                        float r1 = pj - __uint_as_float(whi[j]);
-                        wmid[j] = __float_as_uint(r1) & 0xffff0000u;
-                        wlo[j] = __float_as_uint(r1 - __uint_as_float(wmid[j]));
+                    for (int tt = 0; tt < TT; ++tt) {
+                        uint32_t whi[4], wmid[4], wlo[4];
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            float pj = sc[tt][i][j];
+                            whi[j] = __float_as_uint(pj) & 0xffff0000u;
+                            float r1 = pj - __uint_as_float(whi[j]);
+                            wmid[j] = __float_as_uint(r1) & 0xffff0000u;
+                            wlo[j] = __float_as_uint(r1 - __uint_as_float(wmid[j]));
+                        }
+                        v2u ph = v2u{__builtin_amdgcn_perm(whi[1], whi[0], 0x07060302u), __builtin_amdgcn_perm(whi[3], whi[2], 0x07060302u)};
+                        v2u pm = v2u{__builtin_amdgcn_perm(wmid[1], wmid[0], 0x07060302u), __builtin_amdgcn_perm(wmid[3], wmid[2], 0x07060302u)};
+                        v2u pl = v2u{__builtin_amdgcn_perm(wlo[1], wlo[0], 0x07060302u), __builtin_amdgcn_perm(wlo[3], wlo[2], 0x07060302u)};
+                        b_hi[tt] = __builtin_bit_cast(v4s, ph);
+                        b_mid[tt] = __builtin_bit_cast(v4s, pm);
+                        b_lo[tt] = __builtin_bit_cast(v4s, pl);
                     }
-                    v2u ph = v2u{__builtin_amdgcn_perm(whi[1], whi[0], 0x07060302u), __builtin_amdgcn_perm(whi[3], whi[2], 0x07060302u)};
-                    v2u pm = v2u{__builtin_amdgcn_perm(wmid[1], wmid[0], 0x07060302u), __builtin_amdgcn_perm(wmid[3], wmid[2], 0x07060302u)};
-                    v2u pl = v2u{__builtin_amdgcn_perm(wlo[1], wlo[0], 0x07060302u), __builtin_amdgcn_perm(wlo[3], wlo[2], 0x07060302u)};
-                    v4s b_hi = __builtin_bit_cast(v4s, ph), b_mid = __builtin_bit_cast(v4s, pm), b_lo = __builtin_bit_cast(v4s, pl);
 #pragma unroll
                     for (int bp = 0; bp < 4; ++bp) {
                         uint32_t w[4];
@@ -414,13 +444,16 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, W
                         v2u ae = v2u{__builtin_amdgcn_perm(w[1], w[0], 0x05040100u), __builtin_amdgcn_perm(w[3], w[2], 0x05040100u)};
                         v2u ao = v2u{__builtin_amdgcn_perm(w[1], w[0], 0x07060302u), __builtin_amdgcn_perm(w[3], w[2], 0x07060302u)};
                         v4s a_even = __builtin_bit_cast(v4s, ae), a_odd = __builtin_bit_cast(v4s, ao);
-                        // smallest terms first
-                        o[2 * bp] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_even, b_lo, o[2 * bp], 0, 0, 0);
-                        o[2 * bp + 1] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_odd, b_lo, o[2 * bp + 1], 0, 0, 0);
-                        o[2 * bp] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_even, b_mid, o[2 * bp], 0, 0, 0);
-                        o[2 * bp + 1] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_odd, b_mid, o[2 * bp + 1], 0, 0, 0);
-                        o[2 * bp] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_even, b_hi, o[2 * bp], 0, 0, 0);
-                        o[2 * bp + 1] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_odd, b_hi, o[2 * bp + 1], 0, 0, 0);
+#pragma unroll
+                        for (int tt = 0; tt < TT; ++tt) {
+                            // smallest terms first
+                            o[tt][2 * bp] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_even, b_lo[tt], o[tt][2 * bp], 0, 0, 0);
+                            o[tt][2 * bp + 1] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_odd, b_lo[tt], o[tt][2 * bp + 1], 0, 0, 0);
+                            o[tt][2 * bp] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_even, b_mid[tt], o[tt][2 * bp], 0, 0, 0);
+                            o[tt][2 * bp + 1] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_odd, b_mid[tt], o[tt][2 * bp + 1], 0, 0, 0);
+                            o[tt][2 * bp] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_even, b_hi[tt], o[tt][2 * bp], 0, 0, 0);
+                            o[tt][2 * bp + 1] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_odd, b_hi[tt], o[tt][2 * bp + 1], 0, 0, 0);
+                        }
                     }
                 }
                 // advance the id windows when the next group starts a new one
@@ -430,21 +463,25 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, W
                 idv_next = adv ? cand : idv_next;
                 win = adv ? win + 64 : win;
             }
-            l_run += __shfl_xor(l_run, 16, 64);
-            l_run += __shfl_xor(l_run, 32, 64);
-            // lane (g, c) holds, for head c: dims 32 bp + 8 g + {0..7} = {o[2bp][0], o[2bp+1][0], o[2bp][1], ...}
+            // lane (g, c) holds, for column c: dims 32 bp + 8 g + {0..7} = {o[2bp][0], o[2bp+1][0], o[2bp][1], ...}
             const uint64_t item = (uint64_t)(r + vq) * p.num_kv_heads + kvh;
-            if ((uint32_t)c < (PF ? p.tpt * p.group : p.group)) {
-                float *po = p.part_o + (item * p.g_pad + c) * kDh + 8 * g;
 #pragma unroll
-                for (int bp = 0; bp < 4; ++bp) {
-                    *(v4f *)(po + 32 * bp) = v4f{o[2 * bp][0], o[2 * bp + 1][0], o[2 * bp][1], o[2 * bp + 1][1]};
-                    *(v4f *)(po + 32 * bp + 4) = v4f{o[2 * bp][2], o[2 * bp + 1][2], o[2 * bp][3], o[2 * bp + 1][3]};
-                }
-                if (g == 0) {
-                    float nanv = __uint_as_float(0x7fc00000u);
-                    p.part_ml[item * (2 * p.g_pad) + c] = bad ? nanv : m_run;
-                    p.part_ml[item * (2 * p.g_pad) + p.g_pad + c] = bad ? nanv : l_run;
+            for (int tt = 0; tt < TT; ++tt) {
+                float l = l_run[tt];
+                l += __shfl_xor(l, 16, 64);
+                l += __shfl_xor(l, 32, 64);
+                if ((uint32_t)c < (PF ? p.tpt * p.group : p.group)) {
+                    float *po = p.part_o + ((item * TT + tt) * p.g_pad + c) * kDh + 8 * g;
+#pragma unroll
+                    for (int bp = 0; bp < 4; ++bp) {
+                        *(v4f *)(po + 32 * bp) = v4f{o[tt][2 * bp][0], o[tt][2 * bp + 1][0], o[tt][2 * bp][1], o[tt][2 * bp + 1][1]};
+                        *(v4f *)(po + 32 * bp + 4) = v4f{o[tt][2 * bp][2], o[tt][2 * bp + 1][2], o[tt][2 * bp][3], o[tt][2 * bp + 1][3]};
+                    }
+                    if (g == 0) {
+                        float nanv = __uint_as_float(0x7fc00000u);
+                        p.part_ml[(item * TT + tt) * (2 * p.g_pad) + c] = bad ? nanv : m_run[tt];
+                        p.part_ml[(item * TT + tt) * (2 * p.g_pad) + p.g_pad + c] = bad ? nanv : l;
+                    }
                 }
             }
         }
@@ -453,29 +490,17 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, W
 
 // Merges the partial results of one (sequence, query head): block = 256 threads,
 // thread (part, d) sums every second partial for dim d, then the two parts are added.
-// Prefill: blockIdx.y = sequence * (tokens of this launch) + token; the partials of the token's tile are
-// merged for the tile column of (token, head).
-template <bool PF>
 __global__ void __launch_bounds__(256) decode_stream_merge_kernel(StreamParams p, void *__restrict__ out, int out_bf16,
                                                                  float *__restrict__ pmax) {
     __shared__ float s_acc[128], s_den, s_max[2];
     __shared__ uint32_t s_tot[4], s_pre[4];
     const uint32_t h = blockIdx.x, d = threadIdx.x % 128, part = threadIdx.x / 128;
     const uint32_t kvh = h / p.group;
-    uint32_t b = blockIdx.y, hg = h % p.group, out_row = blockIdx.y, seq = blockIdx.y;
-    if constexpr (PF) {
-        const uint32_t ct = p.qt * p.tpt < p.l_new - p.t0 ? p.qt * p.tpt : p.l_new - p.t0;   // tokens of this launch
-        seq = blockIdx.y / ct;
-        const uint32_t tt = blockIdx.y % ct;
-        b = seq * p.qt + tt / p.tpt;                               // virtual sequence
-        hg = (tt % p.tpt) * p.group + h % p.group;                 // tile column
-        out_row = seq * p.l_new + p.t0 + tt;
-    }
-    const uint32_t nv = PF ? p.n_vseq : p.batch;
+    const uint32_t b = blockIdx.y, hg = h % p.group;
     const uint32_t max_ctx = p.max_blocks_per_seq * kPage;
     uint32_t tot = 0, pre = 0;
-    for (uint32_t bb = threadIdx.x; bb < nv; bb += 256) {
-        uint32_t v = seq_pages<PF>(p, bb, max_ctx);
+    for (uint32_t bb = threadIdx.x; bb < p.batch; bb += 256) {
+        uint32_t v = seq_pages<false>(p, bb, max_ctx);
         tot += v;
         if (bb < b) pre += v;
     }
@@ -488,11 +513,10 @@ __global__ void __launch_bounds__(256) decode_stream_merge_kernel(StreamParams p
     __syncthreads();
     tot = s_tot[0] + s_tot[1] + s_tot[2] + s_tot[3];
     pre = s_pre[0] + s_pre[1] + s_pre[2] + s_pre[3];
-    const uint32_t npg = seq_pages<PF>(p, b, max_ctx);
+    const uint32_t npg = seq_pages<false>(p, b, max_ctx);
     const uint32_t per = range_pages(p, tot);
     const uint32_t r_lo = npg ? pre / per : 1, r_hi = npg ? (pre + npg - 1) / per : 0;   // empty sequence: no partials
     float mx = -INFINITY;
-    if (PF && p.seq_lens[seq] < p.l_new) mx = __uint_as_float(0x7fc00000u);             // violation: NaN out
     for (uint32_t r = r_lo; r <= r_hi; ++r) {
         float m = p.part_ml[((uint64_t)(r + b) * p.num_kv_heads + kvh) * (2 * p.g_pad) + hg];
         mx = (m != m || mx != mx) ? __uint_as_float(0x7fc00000u) : fmaxf(mx, m);   // NaN marks a violation
@@ -515,8 +539,8 @@ __global__ void __launch_bounds__(256) decode_stream_merge_kernel(StreamParams p
     if (part == 0) {
         acc += s_acc[d];
         den += s_den;
-        float res = npg == 0 ? (mx != mx ? mx : 0.0f) : __fdiv_rn(acc, den);
-        uint64_t oi = ((uint64_t)out_row * p.num_heads + h) * kDh + d;
+        float res = npg == 0 ? 0.0f : __fdiv_rn(acc, den);
+        uint64_t oi = ((uint64_t)b * p.num_heads + h) * kDh + d;
         if (out_bf16) {
             uint16_t rb = f32_to_bf16(res);
             ((uint16_t *)out)[oi] = rb;
@@ -530,7 +554,61 @@ __global__ void __launch_bounds__(256) decode_stream_merge_kernel(StreamParams p
         a = wave_max(a);
         if (part == 0 && threadIdx.x % 64 == 0) s_max[threadIdx.x / 64] = a;
         __syncthreads();
-        if (threadIdx.x == 0) pmax[(uint64_t)out_row * p.num_heads + h] = fmaxf(s_max[0], s_max[1]);
+        if (threadIdx.x == 0) pmax[(uint64_t)b * p.num_heads + h] = fmaxf(s_max[0], s_max[1]);
+    }
+}
+
+// Prefill: one block per (kv head, virtual sequence) merges the partial results of all its columns
+// (token tiles x tokens of a tile x heads of the group): two columns at a time, thread = (column parity, dim).
+__global__ void __launch_bounds__(256) prefill_stream_merge_kernel(StreamParams p, void *__restrict__ out, int out_bf16) {
+    __shared__ uint32_t s_tot[4], s_pre[4];
+    const uint32_t kvh = blockIdx.x, vq = blockIdx.y, d = threadIdx.x % 128, part = threadIdx.x / 128;
+    const uint32_t max_ctx = p.max_blocks_per_seq * kPage;
+    uint32_t tot = 0, pre = 0;
+    for (uint32_t bb = threadIdx.x; bb < p.n_vseq; bb += 256) {
+        uint32_t v = seq_pages<true>(p, bb, max_ctx);
+        tot += v;
+        if (bb < vq) pre += v;
+    }
+    tot = (uint32_t)wave_sum<uint32_t>(tot);
+    pre = (uint32_t)wave_sum<uint32_t>(pre);
+    if (threadIdx.x % 64 == 0) {
+        s_tot[threadIdx.x / 64] = tot;
+        s_pre[threadIdx.x / 64] = pre;
+    }
+    __syncthreads();
+    tot = s_tot[0] + s_tot[1] + s_tot[2] + s_tot[3];
+    pre = s_pre[0] + s_pre[1] + s_pre[2] + s_pre[3];
+    const uint32_t npg = seq_pages<true>(p, vq, max_ctx);
+    const uint32_t per = range_pages(p, tot);
+    const uint32_t r_lo = npg ? pre / per : 1, r_hi = npg ? (pre + npg - 1) / per : 0;   // nothing streamed: no partials
+    const uint32_t seq = vq / p.qt, tiles = p.tpv / p.tpt, cols = p.tpt * p.group;
+    const bool violation = p.seq_lens[seq] < p.l_new;              // possible only with unvalidated device tables
+    for (uint32_t ci = part; ci < tiles * cols; ci += 2) {
+        const uint32_t tile = ci / cols, col = ci % cols;
+        const uint32_t t = p.t0 + (vq % p.qt) * p.tpv + tile * p.tpt + col / p.group;
+        if (t >= p.l_new) continue;
+        float mx = -INFINITY;
+        for (uint32_t r = r_lo; r <= r_hi; ++r) {
+            float m = p.part_ml[(((uint64_t)(r + vq) * p.num_kv_heads + kvh) * tiles + tile) * (2 * p.g_pad) + col];
+            mx = (m != m || mx != mx) ? __uint_as_float(0x7fc00000u) : fmaxf(mx, m);   // NaN marks a violation
+        }
+        float acc = 0.0f, den = 0.0f;
+        for (uint32_t r = r_lo; r <= r_hi; ++r) {
+            const uint64_t item = ((uint64_t)(r + vq) * p.num_kv_heads + kvh) * tiles + tile;
+            float m = p.part_ml[item * (2 * p.g_pad) + col];
+            float l = p.part_ml[item * (2 * p.g_pad) + p.g_pad + col];
+            float w = expf(m - mx);
+            den = __builtin_fmaf(w, l, den);
+            acc = __builtin_fmaf(w, p.part_o[(item * p.g_pad + col) * kDh + d], acc);
+        }
+        float res = npg == 0 ? 0.0f : __fdiv_rn(acc, den);
+        if (violation) res = __uint_as_float(0x7fc00000u);
+        const uint64_t oi = (((uint64_t)seq * p.l_new + t) * p.num_heads + (uint64_t)kvh * p.group + col % p.group) * kDh + d;
+        if (out_bf16)
+            ((uint16_t *)out)[oi] = f32_to_bf16(res);
+        else
+            ((float *)out)[oi] = res;
     }
 }
 
@@ -735,7 +813,7 @@ void paged_attention_decode_bf16(const uint16_t *q, const uint16_t *k_pool, cons
     sp.n_ranges = stream_ranges(ps, waves_per_cu);
     sp.min_pages = 4;
     sp.scale = ps.scale;
-    sp.l_new = sp.tpt = sp.qt = 1;
+    sp.l_new = sp.tpt = sp.tpv = sp.qt = 1;
     sp.t0 = 0;
     sp.n_vseq = ps.batch;
     uint64_t items = ((uint64_t)sp.n_ranges + ps.batch) * ps.num_kv_heads;
@@ -750,24 +828,30 @@ void paged_attention_decode_bf16(const uint16_t *q, const uint16_t *k_pool, cons
         return;
     }
     dim3 grid2(ps.num_heads, ps.batch);
-    decode_stream_merge_kernel<false><<<grid2, 256, 0, s>>>(sp, out, out_bf16, pmax);
+    decode_stream_merge_kernel<<<grid2, 256, 0, s>>>(sp, out, out_bf16, pmax);
 }
 
-// Prefill (l_new > 1) on the same streaming kernel: token tiles of 16 / group new tokens are streamed as
-// sequences of their own, at most kPrefillTiles of them per launch so that the partial results stay within
-// a bounded workspace; the launches for successive token ranges follow each other on the stream.
-constexpr uint32_t kPrefillTiles = 1024;
+// Prefill (l_new > 1) on the same streaming kernel: groups of kPrefillTT token tiles of 16 / group new tokens
+// are streamed as sequences of their own, at most kPrefillSeqs of them per launch so that the partial
+// results stay within a bounded workspace; the launches for successive token ranges follow each other on
+// the stream.  A call whose new tokens fit one tile uses the one-tile form (two wavefronts per SIMD).
+constexpr uint32_t kPrefillSeqs = 512, kPrefillTT = 2;
 
-static uint32_t prefill_tiles_per_seq(const PagedShape &ps) {          // token tiles of one sequence per launch
-    uint32_t per_seq = kPrefillTiles / ps.batch;
-    return per_seq ? per_seq : 1;
+static uint32_t prefill_tt(const PagedShape &ps) {
+    uint32_t tpt = 16 / (ps.num_heads / ps.num_kv_heads);
+    return ps.l_new > tpt ? kPrefillTT : 1;
+}
+static uint32_t prefill_seqs_per_row(const PagedShape &ps) {           // virtual sequences of one row per launch
+    const uint32_t tpv = 16 / (ps.num_heads / ps.num_kv_heads) * prefill_tt(ps);
+    const uint32_t all = (ps.l_new + tpv - 1) / tpv;
+    uint32_t cap = kPrefillSeqs / ps.batch;
+    if (cap == 0) cap = 1;
+    return all < cap ? all : cap;
 }
 
 uint64_t paged_prefill_workspace_bytes(const PagedShape &ps, uint32_t waves_per_cu) {
-    uint32_t tpt = 16 / (ps.num_heads / ps.num_kv_heads);
-    uint32_t tiles = (ps.l_new + tpt - 1) / tpt;
-    uint32_t qt = tiles < prefill_tiles_per_seq(ps) ? tiles : prefill_tiles_per_seq(ps);
-    uint64_t items = ((uint64_t)stream_ranges(ps, waves_per_cu) + (uint64_t)ps.batch * qt) * ps.num_kv_heads;
+    uint64_t items = ((uint64_t)stream_ranges(ps, waves_per_cu) + (uint64_t)ps.batch * prefill_seqs_per_row(ps)) *
+                     ps.num_kv_heads * prefill_tt(ps);
     return items * (16 * kDh + 2 * 16) * sizeof(float);
 }
 
@@ -789,25 +873,31 @@ void paged_attention_prefill_bf16(const uint16_t *q, const uint16_t *k_pool, con
     sp.group = ps.num_heads / ps.num_kv_heads;
     sp.g_pad = 16;
     sp.max_blocks_per_seq = ps.max_blocks_per_seq;
-    sp.n_ranges = stream_ranges(ps, waves_per_cu);
     sp.min_pages = 4;
     sp.scale = ps.scale;
     sp.l_new = ps.l_new;
     sp.tpt = 16 / sp.group;
-    const uint32_t tiles = (ps.l_new + sp.tpt - 1) / sp.tpt;
-    const uint32_t qt_max = tiles < prefill_tiles_per_seq(ps) ? tiles : prefill_tiles_per_seq(ps);
-    const uint64_t items_max = ((uint64_t)sp.n_ranges + (uint64_t)ps.batch * qt_max) * ps.num_kv_heads;
+    const uint32_t tt = prefill_tt(ps);
+    sp.tpv = sp.tpt * tt;
+    // the several-tile form keeps one wavefront per SIMD (register budget)
+    sp.n_ranges = stream_ranges(ps, tt == 1 ? waves_per_cu : (waves_per_cu && waves_per_cu < 4 ? waves_per_cu : 4));
+    const uint32_t vseqs = (ps.l_new + sp.tpv - 1) / sp.tpv;
+    const uint32_t qt_max = prefill_seqs_per_row(ps);
+    const uint64_t items_max = ((uint64_t)stream_ranges(ps, waves_per_cu) + (uint64_t)ps.batch * qt_max) * ps.num_kv_heads * tt;
     sp.part_o = (float *)workspace;
     sp.part_ml = sp.part_o + items_max * 16 * kDh;
     const uint64_t waves = (uint64_t)sp.n_ranges * ps.num_kv_heads;
-    for (uint32_t tile0 = 0; tile0 < tiles; tile0 += qt_max) {
-        sp.qt = tiles - tile0 < qt_max ? tiles - tile0 : qt_max;
-        sp.t0 = tile0 * sp.tpt;
+    for (uint32_t v0 = 0; v0 < vseqs; v0 += qt_max) {
+        sp.qt = vseqs - v0 < qt_max ? vseqs - v0 : qt_max;
+        sp.t0 = v0 * sp.tpv;
         sp.n_vseq = ps.batch * sp.qt;
-        const uint32_t ct = sp.qt * sp.tpt < ps.l_new - sp.t0 ? sp.qt * sp.tpt : ps.l_new - sp.t0;
-        decode_stream_kernel<4, 4, 2, 2, true><<<(unsigned)((waves + 3) / 4), 256, 0, s>>>(sp);
-        dim3 grid2(ps.num_heads, ps.batch * ct);
-        decode_stream_merge_kernel<true><<<grid2, 256, 0, s>>>(sp, out, out_bf16, nullptr);
+        if (tt == 1)
+            decode_stream_kernel<4, 4, 2, 2, true, 1><<<(unsigned)((waves + 3) / 4), 256, 0, s>>>(sp);
+        else
+            decode_stream_kernel<4, 4, 2, 1, true, kPrefillTT><<<(unsigned)((waves + 3) / 4), 256, 0, s>>>(sp);
+        if (g_decode_partials_only) continue;
+        dim3 grid2(ps.num_kv_heads, sp.n_vseq);
+        prefill_stream_merge_kernel<<<grid2, 256, 0, s>>>(sp, out, out_bf16);
     }
 }
 
