@@ -327,6 +327,32 @@ def bench_prefill_attention(fa, be, batch=4, l_new=2048, heads=32, kv_heads=8):
     return res
 
 
+def bench_prompt_prefill(fa, be, dec, cfg, tables, batch=4, l_new=2048, reps=2):
+    """Prompt ingestion through the whole decoder: `batch` empty sequences, `l_new` prompt tokens each, on the
+    resident model (the sequences borrow the first pages of the installed tables)."""
+    lib = fa.capi.lib
+    need = (l_new + 1 + cfg["block_size"] - 1) // cfg["block_size"]
+    assert need <= tables.shape[1] and batch <= tables.shape[0]
+    tb = np.ascontiguousarray(tables[:batch])
+    lens = np.zeros(batch, dtype=np.uint32)
+    prompt = np.random.default_rng(3).integers(0, cfg["vocab"], size=(batch, l_new)).astype(np.int32)
+
+    def run():
+        fa.check(lib.fa_decoder_set_sequences(be._ctx, dec, batch, tb.ctypes.data_as(fa.capi.u32p),
+                                              lens.ctypes.data_as(fa.capi.u32p)))
+        t = Timer(fa, be)
+        t.start()
+        fa.check(lib.fa_decoder_prefill(be._ctx, dec, prompt.ctypes.data_as(fa.capi.i32p), l_new))
+        return t.stop_ms()
+
+    run()
+    ms = min(run() for _ in range(reps))
+    toks = np.empty(batch, dtype=np.int32)
+    fa.check(lib.fa_decoder_read_tokens(be._ctx, dec, toks.ctypes.data_as(fa.capi.i32p)))
+    assert np.all((toks >= 0) & (toks < cfg["vocab"]))
+    return dict(batch=batch, l_new=l_new, ms=ms, tokens_per_s=batch * l_new / (ms * 1e-3))
+
+
 def bench_matrix_rate(fa, be, iters=20000):
     """Register-only rate of the matrix instructions the prefill GEMMs use, with all-zero and with
     random operand bits (the sustained clock of the part depends on the bits it multiplies)."""
@@ -494,6 +520,15 @@ def main():
     bytes_step = step_bytes(cfg, batch, sum(mid_ctx))
     log("step %.3f ms (events %.3f ms, wall %.3f ms); algorithmic bytes/step %.2f GB -> %.0f GB/s" %
         (sec_per_step * 1e3, ms / a.steps, wall / a.steps * 1e3, bytes_step / 1e9, bytes_step / sec_per_step / 1e9))
+    prompt = None
+    if not a.no_extras and min(ctxs) >= 2048 // 2:
+        # the pages of the first sequences hold at least 2049 tokens each only if their context is that long;
+        # pick the four longest rows of the table
+        order = np.argsort(ctxs)[::-1][:4]
+        if min(ctxs[i] for i in order) > 2048:
+            prompt = bench_prompt_prefill(fa, be, dec, cfg, np.ascontiguousarray(tables[order]))
+            log("prompt prefill %d x %d tokens: %.1f ms, %.0f tokens/s" %
+                (prompt["batch"], prompt["l_new"], prompt["ms"], prompt["tokens_per_s"]))
     lib.fa_decoder_destroy(be._ctx, dec)
     for x in keep:
         x.free()
@@ -512,6 +547,8 @@ def main():
                     bytes_per_launch=att_bytes, us_per_launch=att_kernel_sec * 1e6,
                     operator_us=att_sec * 1e6, operator_achieved=att_bytes / att_sec / 1e9)
     extras = {"step_algorithmic_gb": bytes_step / 1e9, "step_hbm_frac": bytes_step / sec_per_step / 1e9 / HBM_PEAK_GBS}
+    if prompt is not None:
+        extras["prompt_prefill"] = prompt
     if not a.no_extras:
         c3 = np.random.default_rng(0).integers(128, 4097, size=64).tolist()
         sec, nb = bench_attention(fa, be, 64, 32, 8, c3, 40000, 50, seed=3)

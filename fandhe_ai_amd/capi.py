@@ -125,6 +125,7 @@ SIGNATURES = {
     "fa_paged_kv_append_device": (C.c_int32, [ctx_p, buf_p, buf_p, buf_p, buf_p, buf_p, u64, C.POINTER(PagedLayout)]),
     "fa_paged_attention_forward_device": (C.c_int32, [ctx_p, buf_p, buf_p, buf_p, buf_p, buf_p,
                                                       C.POINTER(PagedArgs), buf_p]),
+    "fa_decoder_prefill": (C.c_int32, [ctx_p, C.c_void_p, i32p, C.c_uint32]),
     "fa_probe_matrix_rate": (C.c_int32, [ctx_p, C.c_int32, buf_p, C.c_uint32, buf_p, C.POINTER(C.c_double)]),
     "fa_block_table_create": (C.c_int32, [C.POINTER(C.c_void_p)]),
     "fa_block_table_destroy": (C.c_int32, [C.c_void_p]),

@@ -3,7 +3,9 @@
 // greedy argmax that the benchmark's full-step configuration names.  All
 // buffers are allocated when the decoder is created; a step only enqueues
 // kernels, so it can be captured once into a HIP graph and replayed.
+#include <algorithm>
 #include <cmath>
+#include <exception>
 #include <new>
 #include <string>
 #include <vector>
@@ -38,6 +40,9 @@ struct fa_decoder {
     fa_graph *graph = nullptr;
     uint32_t graph_batch = 0;
     int graph_waves = 0;
+    // host mirror of the installed block tables and of the sequence lengths (advanced with every step and
+    // prompt chunk), used to validate that a prompt fits before anything is queued
+    std::vector<uint32_t> host_tables, host_lens;
 };
 
 namespace {
@@ -167,6 +172,114 @@ fa_status enqueue_step(fa_context *ctx, fa_decoder *d) {
     linear(d->lm_head, d->logits->ptr, nullptr);
     k::argmax_rows_f32((const float *)d->logits->ptr, (int32_t *)d->tokens->ptr, B, V, s);
     return after_launch(ctx, "decoder step");
+}
+
+// device memory from the context's pool, returned when the call that took it ends (the stream is in
+// order, so a later user of the same memory is queued behind this call's kernels)
+struct Temp {
+    fa_context *ctx;
+    void *ptr = nullptr;
+    uint64_t bytes = 0, cls = 0;
+    explicit Temp(fa_context *c) : ctx(c) {}
+    fa_status get(uint64_t n) {
+        bytes = n ? n : 16;
+        return pool_alloc(ctx, bytes, &ptr, &cls);
+    }
+    ~Temp() {
+        if (ptr) pool_free(ctx, ptr, bytes, cls);
+    }
+    template <typename T>
+    T *as() const { return (T *)ptr; }
+};
+
+// One pass of a prompt chunk (lc tokens per sequence, rows = batch * lc, row b * lc + t) through all layers
+// on the prefill-shape GEMMs and the prefill form of the attention kernel.  The arithmetic per row is
+// that of the decode step (same quantizers, same dequantization, same RoPE and SwiGLU expressions), so
+// a prompt token leaves the same K / V rows in the cache as if it had been decoded.
+struct PrefillBuffers {
+    Temp tok, h, norm, xq, sx, qkv, q_bf, attn, gu, act, slots, cos_sin, last_rows;
+    explicit PrefillBuffers(fa_context *c)
+        : tok(c), h(c), norm(c), xq(c), sx(c), qkv(c), q_bf(c), attn(c), gu(c), act(c), slots(c), cos_sin(c), last_rows(c) {}
+};
+
+fa_status enqueue_prefill_chunk(fa_context *ctx, fa_decoder *d, PrefillBuffers &t, uint32_t lc, bool last_chunk) {
+    const fa_decoder_config &c = d->cfg;
+    const uint32_t B = d->batch;
+    const uint64_t M = (uint64_t)B * lc;
+    const uint64_t D = c.d_model, F = c.d_ffn, V = c.vocab;
+    const uint64_t EKV = (uint64_t)c.n_kv_heads * c.head_dim;
+    const int cus = ctx->props.multiProcessorCount;
+    hipStream_t s = ctx->stream;
+    const uint64_t pool_rows = (uint64_t)c.num_blocks * c.block_size;
+
+    k::prefill_prepare((const uint32_t *)d->tables->ptr, (const uint32_t *)d->seq_lens->ptr, t.slots.as<uint32_t>(),
+                       t.cos_sin.as<float>(), B, lc, c.block_size, c.max_blocks_per_seq, c.num_blocks, c.head_dim,
+                       c.rope_theta, s);
+    k::advance_seq_lens((uint32_t *)d->seq_lens->ptr, t.last_rows.as<int32_t>(), B, lc, s);
+    k::gather_rows_f32((const float *)d->embed->ptr, V, D, t.tok.as<int32_t>(), t.h.as<float>(), M, s);
+
+    k::PagedShape ps;
+    ps.num_blocks = c.num_blocks;
+    ps.block_size = c.block_size;
+    ps.e_kv = (uint32_t)EKV;
+    ps.batch = B;
+    ps.l_new = lc;
+    ps.num_heads = c.n_heads;
+    ps.num_kv_heads = c.n_kv_heads;
+    ps.head_dim = c.head_dim;
+    ps.max_blocks_per_seq = c.max_blocks_per_seq;
+    ps.scale = 1.0f / std::sqrt((float)c.head_dim);
+
+    // y = dequant(quantize_rows(x) @ w) (+ residual); x f32 or bf16 [M, w->k]
+    auto linear = [&](const void *x, bool x_bf16, const fa_qweight *w, float *out, const float *residual) {
+        k::quantize_rows_i8(x, x_bf16, t.xq.as<int8_t>(), nullptr, t.sx.as<float>(), M, M, w->k, w->k_pad, s);
+        k::EpilogueI8 ep;
+        ep.sx = t.sx.as<float>();
+        ep.sw = (const float *)w->scales->ptr;
+        ep.bias = nullptr;
+        ep.residual = residual;
+        ep.acc_out = nullptr;
+        ep.out = out;
+        ep.out_bf16 = 0;
+        k::gemm_w8a8_mfma(t.xq.as<int8_t>(), (const int8_t *)w->codes->ptr, M, w->n, w->n_pad, w->k_pad, ep, cus, s);
+    };
+
+    for (uint32_t li = 0; li < c.n_layers; ++li) {
+        const fa_decoder::Layer &L = d->layers[li];
+        k::rmsnorm_f32(t.h.as<float>(), (const float *)L.attn_norm->ptr, t.norm.as<float>(), M, D, c.rms_eps, s);
+        linear(t.norm.ptr, false, L.wqkv, t.qkv.as<float>(), nullptr);
+        k::rope_append(t.qkv.as<float>(), t.cos_sin.as<float>(), t.slots.as<uint32_t>(), t.q_bf.as<uint16_t>(),
+                       (uint16_t *)L.k_pool->ptr, (uint16_t *)L.v_pool->ptr, M, c.n_heads, c.n_kv_heads, c.head_dim,
+                       pool_rows, s);
+        k::paged_attention_prefill_bf16(t.q_bf.as<uint16_t>(), (const uint16_t *)L.k_pool->ptr,
+                                        (const uint16_t *)L.v_pool->ptr, (const uint32_t *)d->tables->ptr,
+                                        (const uint32_t *)d->seq_lens->ptr, ps, (uint32_t)g_decode_waves, ctx->workspace,
+                                        t.attn.ptr, 1, s);
+        linear(t.attn.ptr, true, L.wo, t.h.as<float>(), t.h.as<float>());
+        k::rmsnorm_f32(t.h.as<float>(), (const float *)L.ffn_norm->ptr, t.norm.as<float>(), M, D, c.rms_eps, s);
+        linear(t.norm.ptr, false, L.wgu, t.gu.as<float>(), nullptr);
+        k::swiglu_rows_f32(t.gu.as<float>(), t.act.as<float>(), M, F, s);
+        linear(t.act.ptr, false, L.wdown, t.h.as<float>(), t.h.as<float>());
+    }
+    if (last_chunk) {
+        // logits of every sequence's last prompt token, and the greedy next token, as a decode step leaves them
+        const uint64_t m_pad = round_up(B, 16);
+        k::gather_rows_f32(t.h.as<float>(), M, D, t.last_rows.as<int32_t>(), (float *)d->h->ptr, B, s);
+        k::rmsnorm_quantize_i8((const float *)d->h->ptr, (const float *)d->final_norm->ptr, c.rms_eps, nullptr,
+                               (int8_t *)d->xq->ptr, (float *)d->sx->ptr, B, m_pad, D, s);
+        k::EpilogueI8 ep;
+        ep.sx = (const float *)d->sx->ptr;
+        ep.sw = (const float *)d->lm_head->scales->ptr;
+        ep.bias = nullptr;
+        ep.residual = nullptr;
+        ep.acc_out = nullptr;
+        ep.out = d->logits->ptr;
+        ep.out_bf16 = 0;
+        k::linear_w8a8_skinny((const int8_t *)d->xq->ptr, (const int8_t *)d->lm_head->codes->ptr, B, d->lm_head->n,
+                              d->lm_head->n_pad, d->lm_head->k_pad, ep, cus, s);
+        k::argmax_rows_f32((const float *)d->logits->ptr, (int32_t *)d->tokens->ptr, B, V, s);
+    }
+    return after_launch(ctx, "decoder prefill");
 }
 
 }  // namespace
@@ -318,6 +431,13 @@ fa_status fa_decoder_set_sequences(fa_context *ctx, fa_decoder *d, uint32_t batc
     if (fa_status s = fa_upload_into(ctx, block_tables, (uint64_t)batch * c.max_blocks_per_seq, d->tables, 0)) return s;
     if (fa_status s = fa_upload_into(ctx, seq_lens, batch, d->seq_lens, 0)) return s;
     d->batch = batch;
+    try {
+        d->host_tables.assign(block_tables, block_tables + (uint64_t)batch * c.max_blocks_per_seq);
+        d->host_lens.assign(seq_lens, seq_lens + batch);
+    } catch (const std::exception &) {
+        d->batch = 0;
+        return fail(FA_ERR_ALLOCATION_FAILED, "decoder_set_sequences: out of host memory");
+    }
     return FA_OK;
 }
 
@@ -347,6 +467,7 @@ fa_status fa_decoder_step(fa_context *ctx, fa_decoder *d, int32_t use_graph) {
     ps.num_kv_heads = d->cfg.n_kv_heads;
     ps.max_blocks_per_seq = d->cfg.max_blocks_per_seq;
     if (fa_status s = ensure_workspace(ctx, k::paged_decode_workspace_bytes(ps, (uint32_t)g_decode_waves))) return s;
+    for (auto &len : d->host_lens) len += 1;            // mirrors the device-side advance of this step
     if (!use_graph) return enqueue_step(ctx, d);
     if (d->graph && (d->graph_batch != d->batch || d->graph_waves != g_decode_waves)) {
         fa_graph_destroy(ctx, d->graph);
@@ -367,6 +488,85 @@ fa_status fa_decoder_step(fa_context *ctx, fa_decoder *d, int32_t use_graph) {
         d->graph_waves = g_decode_waves;
     }
     return fa_graph_launch(ctx, d->graph);
+}
+
+fa_status fa_decoder_prefill(fa_context *ctx, fa_decoder *d, const int32_t *tokens, uint32_t l_new) {
+    if (fa_status s = check_ctx(ctx)) return s;
+    if (fa_status s = check_dec(d)) return s;
+    if (d->ctx != ctx) return fail(FA_ERR_DEVICE_MISMATCH, "decoder_prefill: decoder belongs to another context");
+    if (ctx->capturing) return fail(FA_ERR_CAPTURE_IN_PROGRESS, "decoder_prefill during graph capture");
+    if (d->batch == 0) return fail(FA_ERR_INVALID_ARGUMENT, "decoder_prefill: no sequences installed");
+    if (!d->embed || !d->final_norm || !d->lm_head) return fail(FA_ERR_INVALID_ARGUMENT, "decoder_prefill: head weights missing");
+    for (auto &l : d->layers)
+        if (!l.wqkv) return fail(FA_ERR_INVALID_ARGUMENT, "decoder_prefill: layer weights missing");
+    if (!tokens || l_new == 0) return fail(FA_ERR_INVALID_ARGUMENT, "decoder_prefill: no tokens");
+    const fa_decoder_config &c = d->cfg;
+    const uint32_t B = d->batch;
+    for (uint64_t i = 0; i < (uint64_t)B * l_new; ++i)
+        if (tokens[i] < 0 || (uint32_t)tokens[i] >= c.vocab)
+            return fail(FA_ERR_INVALID_ARGUMENT, "decoder_prefill: token id outside the vocabulary");
+    // every position the prompt writes must have a valid page
+    for (uint32_t b = 0; b < B; ++b) {
+        const uint64_t end = (uint64_t)d->host_lens[b] + l_new;
+        const uint64_t need = (end + c.block_size - 1) / c.block_size;
+        if (need > c.max_blocks_per_seq)
+            return fail(FA_ERR_INVALID_ARGUMENT, "paged_kv: row " + std::to_string(b) + " has no room for the prompt");
+        for (uint64_t i = 0; i < need; ++i)
+            if (d->host_tables[(uint64_t)b * c.max_blocks_per_seq + i] >= c.num_blocks)
+                return fail(FA_ERR_INVALID_ARGUMENT, "paged_kv: row " + std::to_string(b) + " entry " + std::to_string(i) +
+                                                         " is not a valid block id");
+    }
+    // chunks of at most kRows rows per pass bound the activation memory (the widest is [rows, 2 d_ffn] f32)
+    constexpr uint64_t kRows = 4096;
+    const uint32_t lc_max = (uint32_t)std::max<uint64_t>(1, std::min<uint64_t>(l_new, kRows / B));
+    const uint64_t M = (uint64_t)B * lc_max;
+    const uint64_t D = c.d_model, F = c.d_ffn, EQ = (uint64_t)c.n_heads * c.head_dim, EKV = (uint64_t)c.n_kv_heads * c.head_dim;
+    const uint64_t kmax = std::max(std::max(D, F), EQ);
+    PrefillBuffers t(ctx);
+    fa_status st = FA_OK;
+    auto get = [&](Temp &b, uint64_t bytes) {
+        if (st == FA_OK) st = b.get(bytes);
+    };
+    get(t.tok, M * 4);
+    get(t.h, M * D * 4);
+    get(t.norm, M * D * 4);
+    get(t.xq, M * kmax);
+    get(t.sx, M * 4);
+    get(t.qkv, M * (EQ + 2 * EKV) * 4);
+    get(t.q_bf, M * EQ * 2);
+    get(t.attn, M * EQ * 2);
+    get(t.gu, M * 2 * F * 4);
+    get(t.act, M * F * 4);
+    get(t.slots, M * 4);
+    get(t.cos_sin, M * c.head_dim * 4);
+    get(t.last_rows, (uint64_t)B * 4);
+    if (st != FA_OK) return st;
+    k::PagedShape ps{};
+    ps.batch = B;
+    ps.l_new = lc_max;
+    ps.num_heads = c.n_heads;
+    ps.num_kv_heads = c.n_kv_heads;
+    ps.max_blocks_per_seq = c.max_blocks_per_seq;
+    if (fa_status s = ensure_workspace(ctx, k::paged_prefill_workspace_bytes(ps, (uint32_t)g_decode_waves))) return s;
+
+    std::vector<int32_t> stage;
+    try {
+        stage.resize(M);
+    } catch (const std::exception &) {
+        return fail(FA_ERR_ALLOCATION_FAILED, "decoder_prefill: out of host memory");
+    }
+    for (uint32_t t0 = 0; t0 < l_new; t0 += lc_max) {
+        const uint32_t lc = std::min(lc_max, l_new - t0);
+        for (uint32_t b = 0; b < B; ++b)
+            for (uint32_t i = 0; i < lc; ++i) stage[(uint64_t)b * lc + i] = tokens[(uint64_t)b * l_new + t0 + i];
+        // the staging vector is reused by the next chunk: the copy must have consumed it before this call goes on
+        hipError_t e = hipMemcpyAsync(t.tok.ptr, stage.data(), (uint64_t)B * lc * 4, hipMemcpyHostToDevice, ctx->stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+        if (e != hipSuccess) return hip_fail(ctx, e, "prompt token upload", FA_ERR_TRANSFER_FAILED);
+        if (fa_status s = enqueue_prefill_chunk(ctx, d, t, lc, t0 + lc == l_new)) return s;
+        for (auto &len : d->host_lens) len += lc;
+    }
+    return FA_OK;
 }
 
 fa_status fa_decoder_read_tokens(fa_context *ctx, fa_decoder *d, int32_t *tokens) {

@@ -24,6 +24,8 @@ constexpr int kTileKF8 = 128;   // e4m3 k-values per tile
 // ---- elementwise / small ops (kern_elementwise.hip) ------------------------
 void silu_mul_f32(const float *gate, const float *up, float *out, uint64_t n, hipStream_t s);
 void add_f32(const float *a, const float *b, float *out, uint64_t n, hipStream_t s);
+// act[r, j] = silu(gu[r, j]) * gu[r, f + j] for gu [rows, 2 f] (gate columns first)
+void swiglu_rows_f32(const float *gu, float *act, uint64_t rows, uint64_t f, hipStream_t s);
 void argmax_rows_f32(const float *x, int32_t *out, uint64_t rows, uint64_t cols, hipStream_t s);
 void gather_rows_f32(const float *table, uint64_t table_rows, uint64_t cols, const int32_t *idx,
                      float *out, uint64_t rows, hipStream_t s);
@@ -175,6 +177,19 @@ double matrix_rate_probe(int kind, const void *operands, uint32_t iters, int num
 void decode_prepare(const uint32_t *tables, uint32_t *seq_lens, int32_t *pos, uint32_t *slots, float *cos_sin,
                     uint32_t batch, uint32_t block_size, uint32_t max_blocks_per_seq, uint32_t num_blocks,
                     uint32_t head_dim, double theta, hipStream_t s);
+
+// Prompt chunks (several new tokens per sequence): row b * l_chunk + t is at position seq_lens[b] + t;
+// slots [batch * l_chunk] and the cos/sin table [batch * l_chunk, head_dim] as in decode_prepare.
+void prefill_prepare(const uint32_t *tables, const uint32_t *seq_lens, uint32_t *slots, float *cos_sin, uint32_t batch,
+                     uint32_t l_chunk, uint32_t block_size, uint32_t max_blocks_per_seq, uint32_t num_blocks,
+                     uint32_t head_dim, double theta, hipStream_t s);
+// seq_lens[b] += l_chunk; last_rows[b] = row of the chunk's last token of sequence b
+void advance_seq_lens(uint32_t *seq_lens, int32_t *last_rows, uint32_t batch, uint32_t l_chunk, hipStream_t s);
+// RoPE on the q and k heads of qkv [rows, (heads + 2 kv_heads) head_dim] (f32), one rounding to bf16;
+// q to q_out [rows, heads head_dim], K / V to pool row slots[r].
+void rope_append(const float *qkv, const float *cos_sin, const uint32_t *slots, uint16_t *q_out, uint16_t *k_pool,
+                 uint16_t *v_pool, uint64_t rows, uint32_t heads, uint32_t kv_heads, uint32_t head_dim, uint64_t pool_rows,
+                 hipStream_t s);
 
 }  // namespace k
 }  // namespace fa

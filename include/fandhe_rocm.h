@@ -407,6 +407,16 @@ fa_status fa_decoder_set_tokens(fa_context *ctx, fa_decoder *dec, const int32_t 
  * as the next step's input.  use_graph != 0 replays a captured HIP graph of
  * the step (captured on first use). */
 fa_status fa_decoder_step(fa_context *ctx, fa_decoder *dec, int32_t use_graph);
+/* Prompt ingestion: l_new tokens per installed sequence (tokens [batch, l_new],
+ * host array), written behind what each sequence has cached, on the
+ * prefill-shape GEMMs and the prefill form of the attention kernel, in chunks of
+ * at most 4096 rows.  Leaves the logits of every sequence's last prompt token
+ * and its greedy next token resident, exactly as a decode step does, so
+ * fa_decoder_step continues from there.  The per-row arithmetic is the decode
+ * step's: a prompt token leaves the K / V rows it would leave if it were
+ * decoded.  Rejected before anything is queued if a row has no pages for its
+ * prompt.  Asynchronous apart from the upload of the token ids. */
+fa_status fa_decoder_prefill(fa_context *ctx, fa_decoder *dec, const int32_t *tokens, uint32_t l_new);
 /* Host copies of the current tokens [batch] / logits [batch, vocab] /
  * sequence lengths [batch] (synchronize). */
 fa_status fa_decoder_read_tokens(fa_context *ctx, fa_decoder *dec, int32_t *tokens);

@@ -143,6 +143,13 @@ class GpuDecoder:
     def step(self, use_graph):
         self.fa.check(self.fa.capi.lib.fa_decoder_step(self.be._ctx, self.h, 1 if use_graph else 0))
 
+    def prefill(self, prompt):
+        """prompt: int32 [batch, l_new]"""
+        p = np.ascontiguousarray(prompt, dtype=np.int32)
+        assert p.shape[0] == self.m.batch
+        self.fa.check(self.fa.capi.lib.fa_decoder_prefill(self.be._ctx, self.h, p.ctypes.data_as(self.fa.capi.i32p),
+                                                          p.shape[1]))
+
     def tokens(self):
         out = np.empty(self.m.batch, dtype=np.int32)
         self.fa.check(self.fa.capi.lib.fa_decoder_read_tokens(self.be._ctx, self.h, out.ctypes.data_as(self.fa.capi.i32p)))

@@ -77,6 +77,83 @@ def test_decode_steps_match_the_oracle_eager_and_graph(shape, astat):
         fa.check(fa.capi.lib.fa_set_tuning(5, 0))
 
 
+PREFILL_SHAPES = [
+    dict(n_layers=2, d_model=256, n_heads=4, n_kv_heads=2, d_ffn=512, vocab=1000, batch=4, ctxs=[0, 5, 16, 40], l_new=7),
+    dict(n_layers=2, d_model=512, n_heads=8, n_kv_heads=2, d_ffn=768, vocab=500, batch=3, ctxs=[0, 1, 31], l_new=33),
+    dict(n_layers=1, d_model=256, n_heads=2, n_kv_heads=2, d_ffn=256, vocab=300, batch=2, ctxs=[0, 100], l_new=1),
+    # 8 x 600 rows: two chunks (512 + 88 tokens per sequence)
+    dict(n_layers=1, d_model=256, n_heads=4, n_kv_heads=1, d_ffn=256, vocab=300, batch=8, ctxs=[0, 3, 9, 20, 0, 64, 7, 15],
+         l_new=600),
+]
+
+
+@pytest.mark.parametrize("shape", PREFILL_SHAPES, ids=["B%d_L%d" % (s["batch"], s["l_new"]) for s in PREFILL_SHAPES])
+def test_prompt_prefill_matches_the_oracle_decoding_the_prompt_token_by_token(shape):
+    """The oracle has no prompt path of its own: it decodes the prompt one token at a time (teacher forced),
+    which is what the prefill is defined to equal.  Tolerances as for the chained decode step above."""
+    be = ops()
+    shape = dict(shape)
+    l_new = shape.pop("l_new")
+    m = build_model(seed=21, steps=l_new + 2, **shape)
+    dec = GpuDecoder(be, m)
+    try:
+        rng = o.Rng(5)
+        prompt = rng.randint(0, shape["vocab"], shape["batch"] * l_new).astype(np.int32).reshape(shape["batch"], l_new)
+        pools_before = [(L["k_pool"].copy(), L["v_pool"].copy()) for L in m.layers]
+        lens = m.seq_lens.copy()
+        for t in range(l_new):
+            want_next, want_logits = oracle_step(m, lens, np.ascontiguousarray(prompt[:, t]))
+        dec.prefill(prompt)
+        got_logits, got_next = dec.logits(), dec.tokens()
+        spread = want_logits.max(axis=1, keepdims=True) - want_logits.min(axis=1, keepdims=True)
+        err = np.abs(got_logits - want_logits) / spread
+        print("PREFILL_PARITY\tB%d:L%d\tmax_err/range=%.3e\tmean=%.3e" % (shape["batch"], l_new, err.max(), err.mean()),
+              flush=True)
+        assert err.mean() < 2e-4 and err.max() < 2e-2
+        top2 = np.sort(want_logits, axis=1)[:, -2:]
+        decisive = (top2[:, 1] - top2[:, 0]) > 4e-2 * spread[:, 0]
+        assert np.array_equal(got_next[decisive], want_next[decisive])
+        assert np.array_equal(got_next, o.argmax_rows(got_logits))
+        assert np.array_equal(dec.seq_lens(), lens) and np.array_equal(lens, m.seq_lens + l_new)
+        for li, L in enumerate(m.layers):
+            gk, gv = dec.kv_pool(li)
+            for name, g, w, before in (("k", gk, L["k_pool"], pools_before[li][0]), ("v", gv, L["v_pool"], pools_before[li][1])):
+                changed = (w != before).any(axis=2)
+                assert np.array_equal((g != before).any(axis=2) | changed, changed), (li, name)   # nothing else written
+                gf, wf = o.from_bf16(g[changed]), o.from_bf16(w[changed])
+                assert np.all(np.abs(gf - wf) <= np.abs(wf).max(axis=1, keepdims=True) * 2.0 ** -6), (li, name)
+                if li == 0:
+                    # the first layer's rows depend on nothing but the embedding and the projection: exact
+                    assert np.array_equal(g[changed], w[changed]), name
+            L["k_pool"][:] = gk
+            L["v_pool"][:] = gv
+        # decoding continues from the prefilled state
+        _check_step(m, dec, lens, got_next.copy(), use_graph=False, tag="after prefill B%d:L%d" % (shape["batch"], l_new))
+    finally:
+        dec.close()
+
+
+def test_prefill_argument_errors():
+    import fandhe_ai_amd as fa
+    be = ops()
+    m = build_model(seed=1, n_layers=1, d_model=128, n_heads=2, n_kv_heads=1, d_ffn=128, vocab=50, batch=2,
+                    ctxs=[3, 4], steps=6)
+    dec = GpuDecoder(be, m)
+    try:
+        room = m.cfg["max_blocks_per_seq"] * 16 - 4
+        with pytest.raises(fa.InvalidArgument):
+            dec.prefill(np.zeros((2, room + 1), np.int32))                  # no pages for the whole prompt
+        with pytest.raises(fa.InvalidArgument):
+            dec.prefill(np.full((2, 2), 50, np.int32))                      # token outside the vocabulary
+        with pytest.raises(fa.InvalidArgument):
+            dec.prefill(np.zeros((2, 0), np.int32))
+        assert dec.seq_lens().tolist() == [3, 4]
+        dec.prefill(np.zeros((2, 5), np.int32))
+        assert dec.seq_lens().tolist() == [8, 9]
+    finally:
+        dec.close()
+
+
 def test_graph_replay_is_bit_identical_to_eager():
     be = ops()
     shape = dict(n_layers=2, d_model=256, n_heads=4, n_kv_heads=2, d_ffn=512, vocab=1000, batch=8,
