@@ -197,9 +197,9 @@ struct Temp {
 // that of the decode step (same quantizers, same dequantization, same RoPE and SwiGLU expressions), so
 // a prompt token leaves the same K / V rows in the cache as if it had been decoded.
 struct PrefillBuffers {
-    Temp tok, h, norm, xq, sx, qkv, q_bf, attn, gu, act, slots, cos_sin, last_rows;
+    Temp tok, h, xq, sx, qkv, q_bf, attn, gu, slots, cos_sin, last_rows;
     explicit PrefillBuffers(fa_context *c)
-        : tok(c), h(c), norm(c), xq(c), sx(c), qkv(c), q_bf(c), attn(c), gu(c), act(c), slots(c), cos_sin(c), last_rows(c) {}
+        : tok(c), h(c), xq(c), sx(c), qkv(c), q_bf(c), attn(c), gu(c), slots(c), cos_sin(c), last_rows(c) {}
 };
 
 fa_status enqueue_prefill_chunk(fa_context *ctx, fa_decoder *d, PrefillBuffers &t, uint32_t lc, bool last_chunk) {
@@ -230,9 +230,8 @@ fa_status enqueue_prefill_chunk(fa_context *ctx, fa_decoder *d, PrefillBuffers &
     ps.max_blocks_per_seq = c.max_blocks_per_seq;
     ps.scale = 1.0f / std::sqrt((float)c.head_dim);
 
-    // y = dequant(quantize_rows(x) @ w) (+ residual); x f32 or bf16 [M, w->k]
-    auto linear = [&](const void *x, bool x_bf16, const fa_qweight *w, float *out, const float *residual) {
-        k::quantize_rows_i8(x, x_bf16, t.xq.as<int8_t>(), nullptr, t.sx.as<float>(), M, M, w->k, w->k_pad, s);
+    // y = dequant(xq @ w) (+ residual) for the rows quantized into t.xq / t.sx just before
+    auto gemm = [&](const fa_qweight *w, float *out, const float *residual) {
         k::EpilogueI8 ep;
         ep.sx = t.sx.as<float>();
         ep.sw = (const float *)w->scales->ptr;
@@ -246,8 +245,9 @@ fa_status enqueue_prefill_chunk(fa_context *ctx, fa_decoder *d, PrefillBuffers &
 
     for (uint32_t li = 0; li < c.n_layers; ++li) {
         const fa_decoder::Layer &L = d->layers[li];
-        k::rmsnorm_f32(t.h.as<float>(), (const float *)L.attn_norm->ptr, t.norm.as<float>(), M, D, c.rms_eps, s);
-        linear(t.norm.ptr, false, L.wqkv, t.qkv.as<float>(), nullptr);
+        k::rmsnorm_quantize_rows_i8(t.h.as<float>(), (const float *)L.attn_norm->ptr, c.rms_eps, t.xq.as<int8_t>(),
+                                    t.sx.as<float>(), M, D, s);
+        gemm(L.wqkv, t.qkv.as<float>(), nullptr);
         k::rope_append(t.qkv.as<float>(), t.cos_sin.as<float>(), t.slots.as<uint32_t>(), t.q_bf.as<uint16_t>(),
                        (uint16_t *)L.k_pool->ptr, (uint16_t *)L.v_pool->ptr, M, c.n_heads, c.n_kv_heads, c.head_dim,
                        pool_rows, s);
@@ -255,11 +255,13 @@ fa_status enqueue_prefill_chunk(fa_context *ctx, fa_decoder *d, PrefillBuffers &
                                         (const uint16_t *)L.v_pool->ptr, (const uint32_t *)d->tables->ptr,
                                         (const uint32_t *)d->seq_lens->ptr, ps, (uint32_t)g_decode_waves, ctx->workspace,
                                         t.attn.ptr, 1, s);
-        linear(t.attn.ptr, true, L.wo, t.h.as<float>(), t.h.as<float>());
-        k::rmsnorm_f32(t.h.as<float>(), (const float *)L.ffn_norm->ptr, t.norm.as<float>(), M, D, c.rms_eps, s);
-        linear(t.norm.ptr, false, L.wgu, t.gu.as<float>(), nullptr);
-        k::swiglu_rows_f32(t.gu.as<float>(), t.act.as<float>(), M, F, s);
-        linear(t.act.ptr, false, L.wdown, t.h.as<float>(), t.h.as<float>());
+        k::quantize_rows_i8(t.attn.ptr, true, t.xq.as<int8_t>(), nullptr, t.sx.as<float>(), M, M, L.wo->k, L.wo->k_pad, s);
+        gemm(L.wo, t.h.as<float>(), t.h.as<float>());
+        k::rmsnorm_quantize_rows_i8(t.h.as<float>(), (const float *)L.ffn_norm->ptr, c.rms_eps, t.xq.as<int8_t>(),
+                                    t.sx.as<float>(), M, D, s);
+        gemm(L.wgu, t.gu.as<float>(), nullptr);
+        k::swiglu_quantize_rows_i8(t.gu.as<float>(), t.xq.as<int8_t>(), t.sx.as<float>(), M, F, s);
+        gemm(L.wdown, t.h.as<float>(), t.h.as<float>());
     }
     if (last_chunk) {
         // logits of every sequence's last prompt token, and the greedy next token, as a decode step leaves them
@@ -529,14 +531,12 @@ fa_status fa_decoder_prefill(fa_context *ctx, fa_decoder *d, const int32_t *toke
     };
     get(t.tok, M * 4);
     get(t.h, M * D * 4);
-    get(t.norm, M * D * 4);
     get(t.xq, M * kmax);
     get(t.sx, M * 4);
     get(t.qkv, M * (EQ + 2 * EKV) * 4);
     get(t.q_bf, M * EQ * 2);
     get(t.attn, M * EQ * 2);
     get(t.gu, M * 2 * F * 4);
-    get(t.act, M * F * 4);
     get(t.slots, M * 4);
     get(t.cos_sin, M * c.head_dim * 4);
     get(t.last_rows, (uint64_t)B * 4);

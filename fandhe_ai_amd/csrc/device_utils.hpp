@@ -76,6 +76,18 @@ __device__ __forceinline__ int quant_i8(float x, float scale) {
     return (int)r;
 }
 
+// x * sigmoid(x) with the two-branch sigmoid of crates/tensor-core/src/scalar_op.rs:666-673 (and :355)
+__device__ __forceinline__ float silu_f32(float x) {
+    float s;
+    if (x >= 0.0f) {
+        s = __fdiv_rn(1.0f, 1.0f + expf(-x));
+    } else {
+        float e = expf(x);
+        s = __fdiv_rn(e, 1.0f + e);
+    }
+    return x * s;
+}
+
 // byte offset of the 16-byte chunk `chunk` (= k / 16) of activation row r in the 16-row x 64-k tile order
 // of the quantized activations
 __device__ __forceinline__ uint64_t tiled_chunk_offset(uint64_t r, uint64_t chunk, uint64_t k_tiles) {

@@ -10,25 +10,7 @@ using namespace fa::dev;
 namespace {
 
 // crates/tensor-core/src/scalar_op.rs:666-673 (sigmoid_stable) and :355 (Silu)
-__device__ __forceinline__ float silu(float x) {
-    float s;
-    if (x >= 0.0f) {
-        s = __fdiv_rn(1.0f, 1.0f + expf(-x));
-    } else {
-        float e = expf(x);
-        s = __fdiv_rn(e, 1.0f + e);
-    }
-    return x * s;
-}
-
-__global__ void swiglu_rows_kernel(const float *__restrict__ gu, float *__restrict__ act, uint64_t rows, uint64_t f) {
-    uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
-    for (; i < rows * f; i += stride) {
-        const uint64_t r = i / f, j = i % f;
-        act[i] = silu(gu[r * 2 * f + j]) * gu[r * 2 * f + f + j];
-    }
-}
+__device__ __forceinline__ float silu(float x) { return silu_f32(x); }
 
 __global__ void silu_mul_kernel(const float *__restrict__ gate, const float *__restrict__ up,
                                 float *__restrict__ out, uint64_t n) {
@@ -165,11 +147,6 @@ inline unsigned grid_for(uint64_t n, unsigned block, unsigned cap = 65535u * 4u)
 }
 
 }  // namespace
-
-void swiglu_rows_f32(const float *gu, float *act, uint64_t rows, uint64_t f, hipStream_t s) {
-    if (rows * f == 0) return;
-    swiglu_rows_kernel<<<grid_for(rows * f, 256), 256, 0, s>>>(gu, act, rows, f);
-}
 
 void silu_mul_f32(const float *gate, const float *up, float *out, uint64_t n, hipStream_t s) {
     if (n == 0) return;

@@ -46,6 +46,31 @@ __device__ __forceinline__ float load_in(const void *x, uint64_t i) {
     return ((const float *)x)[i];
 }
 
+// 16 consecutive elements starting at element i (a multiple of 16 of a 16-aligned row) as f32
+template <bool IN_BF16>
+__device__ __forceinline__ void load16(const void *x, uint64_t i, float (&v)[16]) {
+    if (IN_BF16) {
+        const v4u *p = (const v4u *)((const uint16_t *)x + i);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            v4u t = p[h];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                v[h * 8 + 2 * e] = bf16_lo(t[e]);
+                v[h * 8 + 2 * e + 1] = bf16_hi(t[e]);
+            }
+        }
+    } else {
+        const v4f *p = (const v4f *)((const float *)x + i);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            v4f t = p[q];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[q * 4 + e] = t[e];
+        }
+    }
+}
+
 // One block per (padded) row.  Pass 1: absmax.  Pass 2: codes, 16 per thread
 // step so that the tiled output is written with 16-byte stores.
 template <bool IN_BF16>
@@ -63,6 +88,31 @@ __global__ void __launch_bounds__(kBlock)
     }
     uint64_t base = r * k;
     float amax = 0.0f;
+    if (k % 16 == 0) {
+        // whole 16-element chunks: 16-byte loads, and the row-major codes leave in 16-byte stores
+        for (uint64_t c = threadIdx.x; c < k / 16; c += kBlock) {
+            float v[16];
+            load16<IN_BF16>(x, base + c * 16, v);
+#pragma unroll
+            for (int e = 0; e < 16; ++e) amax = fmaxf(amax, fabsf(v[e]));
+        }
+        amax = block_max<kWaves>(amax, smem);
+        const float scale = __fdiv_rn(amax, 127.0f);
+        if (threadIdx.x == 0) sx[r] = scale;
+        for (uint64_t c = threadIdx.x; c < k_pad / 16; c += kBlock) {
+            uint32_t words[4] = {0, 0, 0, 0};
+            if (c < k / 16) {
+                float v[16];
+                load16<IN_BF16>(x, base + c * 16, v);
+#pragma unroll
+                for (int e = 0; e < 16; ++e) words[e / 4] |= ((uint32_t)quant_i8(v[e], scale) & 0xffu) << (8 * (e % 4));
+            }
+            if (xq_tiled)
+                *(v4u *)(xq_tiled + tiled_chunk_offset(r, c, k_tiles)) = v4u{words[0], words[1], words[2], words[3]};
+            if (xq_row && c < k / 16) *(v4u *)(xq_row + base + c * 16) = v4u{words[0], words[1], words[2], words[3]};
+        }
+        return;
+    }
     for (uint64_t i = threadIdx.x; i < k; i += kBlock) amax = fmaxf(amax, fabsf(load_in<IN_BF16>(x, base + i)));
     amax = block_max<kWaves>(amax, smem);
     float scale = __fdiv_rn(amax, 127.0f);
@@ -97,7 +147,8 @@ __global__ void __launch_bounds__(kBlock)
 // RMSNorm of an f32 row followed by its per-token quantization.  Thread t owns the 16-element chunks
 // t, t + 256, ... of the row and keeps them in registers (NCH chunks), so the row is read once:
 // f64 sum of squares -> rstd -> y = (x * rstd) * w -> absmax -> codes, written as 16-byte tile chunks.
-template <int NCH>
+// ROW: the codes go to a row-major [m, hidden] matrix (the operand layout of the prefill GEMMs) instead of tiles.
+template <int NCH, bool ROW = false>
 __global__ void __launch_bounds__(kBlock)
     rmsnorm_quantize_kernel(const float *__restrict__ x, const float *__restrict__ w, float eps, float inv_n,
                             float *__restrict__ out_f32, int8_t *__restrict__ xq_tiled, float *__restrict__ sx,
@@ -107,8 +158,9 @@ __global__ void __launch_bounds__(kBlock)
     const uint64_t r = blockIdx.x;
     const uint64_t k_tiles = hidden / 64, n_chunks = hidden / 16;
     if (r >= m) {
-        for (uint64_t c = threadIdx.x; c < n_chunks; c += kBlock)
-            *(v4i *)(xq_tiled + tiled_chunk_offset(r, c, k_tiles)) = v4i{0, 0, 0, 0};
+        if (!ROW)
+            for (uint64_t c = threadIdx.x; c < n_chunks; c += kBlock)
+                *(v4i *)(xq_tiled + tiled_chunk_offset(r, c, k_tiles)) = v4i{0, 0, 0, 0};
         return;
     }
     const float *row = x + r * hidden;
@@ -161,7 +213,40 @@ __global__ void __launch_bounds__(kBlock)
             words[v] = word;
             if (out_f32) *(v4f *)(out_f32 + r * hidden + c * 16 + v * 4) = xv[i][v];
         }
-        *(v4u *)(xq_tiled + tiled_chunk_offset(r, c, k_tiles)) = v4u{words[0], words[1], words[2], words[3]};
+        int8_t *dst = ROW ? xq_tiled + r * hidden + c * 16 : xq_tiled + tiled_chunk_offset(r, c, k_tiles);
+        *(v4u *)dst = v4u{words[0], words[1], words[2], words[3]};
+    }
+}
+
+// SwiGLU of gu [m, 2 f] (gate columns first) followed by the per-token quantizer of the product, row-major:
+// pass 1 takes the row's absmax of silu(gate) * up, pass 2 recomputes the products (the row is in L2) and
+// writes their codes, so the f32 products never go to memory.  f a multiple of 16.
+__global__ void __launch_bounds__(kBlock)
+    swiglu_quantize_rows_kernel(const float *__restrict__ gu, int8_t *__restrict__ xq_row, float *__restrict__ sx,
+                                uint64_t f) {
+    __shared__ float smem[kWaves];
+    const uint64_t r = blockIdx.x;
+    const float *gate = gu + r * 2 * f, *up = gate + f;
+    float amax = 0.0f;
+    for (uint64_t c = threadIdx.x; c < f / 16; c += kBlock) {
+        float g[16], u[16];
+        load16<false>(gate, c * 16, g);
+        load16<false>(up, c * 16, u);
+#pragma unroll
+        for (int e = 0; e < 16; ++e) amax = fmaxf(amax, fabsf(silu_f32(g[e]) * u[e]));
+    }
+    amax = block_max<kWaves>(amax, smem);
+    const float scale = __fdiv_rn(amax, 127.0f);
+    if (threadIdx.x == 0) sx[r] = scale;
+    for (uint64_t c = threadIdx.x; c < f / 16; c += kBlock) {
+        float g[16], u[16];
+        load16<false>(gate, c * 16, g);
+        load16<false>(up, c * 16, u);
+        uint32_t words[4] = {0, 0, 0, 0};
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+            words[e / 4] |= ((uint32_t)quant_i8(silu_f32(g[e]) * u[e], scale) & 0xffu) << (8 * (e % 4));
+        *(v4u *)(xq_row + r * f + c * 16) = v4u{words[0], words[1], words[2], words[3]};
     }
 }
 
@@ -256,6 +341,25 @@ void rmsnorm_quantize_i8(const float *x, const float *w, float eps, float *out_f
         rmsnorm_quantize_kernel<2><<<grid, kBlock, 0, s>>>(x, w, eps, inv_n, out_f32, xq_tiled, sx, m, hidden);
     else
         rmsnorm_quantize_kernel<4><<<grid, kBlock, 0, s>>>(x, w, eps, inv_n, out_f32, xq_tiled, sx, m, hidden);
+}
+
+void rmsnorm_quantize_rows_i8(const float *x, const float *w, float eps, int8_t *xq_rowmajor, float *sx, uint64_t m,
+                              uint64_t hidden, hipStream_t s) {
+    if (m == 0 || hidden == 0) return;
+    float inv_n = 1.0f / (float)hidden;
+    uint64_t per_thread = (hidden / 16 + kBlock - 1) / kBlock;
+    unsigned grid = (unsigned)m;
+    if (per_thread <= 1)
+        rmsnorm_quantize_kernel<1, true><<<grid, kBlock, 0, s>>>(x, w, eps, inv_n, nullptr, xq_rowmajor, sx, m, hidden);
+    else if (per_thread <= 2)
+        rmsnorm_quantize_kernel<2, true><<<grid, kBlock, 0, s>>>(x, w, eps, inv_n, nullptr, xq_rowmajor, sx, m, hidden);
+    else
+        rmsnorm_quantize_kernel<4, true><<<grid, kBlock, 0, s>>>(x, w, eps, inv_n, nullptr, xq_rowmajor, sx, m, hidden);
+}
+
+void swiglu_quantize_rows_i8(const float *gu, int8_t *xq_rowmajor, float *sx, uint64_t m, uint64_t f, hipStream_t s) {
+    if (m == 0 || f == 0) return;
+    swiglu_quantize_rows_kernel<<<(unsigned)m, kBlock, 0, s>>>(gu, xq_rowmajor, sx, f);
 }
 
 void quantize_rows_from_pmax(const void *x, bool in_bf16, const float *pmax, uint32_t parts, int8_t *xq_tiled,

@@ -35,17 +35,6 @@ struct EpiI8 {
 
 enum { kEpiPlain = 0, kEpiSwiglu = 1, kEpiRope = 2 };
 
-// crates/tensor-core/src/scalar_op.rs:666-673 / :355
-__device__ __forceinline__ float silu_f32(float x) {
-    float s;
-    if (x >= 0.0f) {
-        s = __fdiv_rn(1.0f, 1.0f + expf(-x));
-    } else {
-        float e = expf(x);
-        s = __fdiv_rn(e, 1.0f + e);
-    }
-    return x * s;
-}
 
 // ------------------------------------------------------------------ W8A8
 // acc[m, n] = sum_k xq[m, k] * w[k, n] on v_mfma_i32_16x16x64_i8.

@@ -24,8 +24,6 @@ constexpr int kTileKF8 = 128;   // e4m3 k-values per tile
 // ---- elementwise / small ops (kern_elementwise.hip) ------------------------
 void silu_mul_f32(const float *gate, const float *up, float *out, uint64_t n, hipStream_t s);
 void add_f32(const float *a, const float *b, float *out, uint64_t n, hipStream_t s);
-// act[r, j] = silu(gu[r, j]) * gu[r, f + j] for gu [rows, 2 f] (gate columns first)
-void swiglu_rows_f32(const float *gu, float *act, uint64_t rows, uint64_t f, hipStream_t s);
 void argmax_rows_f32(const float *x, int32_t *out, uint64_t rows, uint64_t cols, hipStream_t s);
 void gather_rows_f32(const float *table, uint64_t table_rows, uint64_t cols, const int32_t *idx,
                      float *out, uint64_t rows, hipStream_t s);
@@ -53,6 +51,13 @@ void quantize_rows_from_pmax(const void *x, bool in_bf16, const float *pmax, uin
 // RMSNorm fused with the quantizer (f32 in): out_f32 nullable.
 void rmsnorm_quantize_i8(const float *x, const float *w, float eps, float *out_f32, int8_t *xq_tiled,
                          float *sx, uint64_t m, uint64_t m_pad, uint64_t hidden, hipStream_t s);
+// The same fused pair with row-major codes [m, hidden] (operand layout of the prefill GEMMs); hidden a
+// multiple of 16 and at most 16384.
+void rmsnorm_quantize_rows_i8(const float *x, const float *w, float eps, int8_t *xq_rowmajor, float *sx, uint64_t m,
+                              uint64_t hidden, hipStream_t s);
+// act = silu(gate) * up of gu [m, 2 f] (gate columns first) quantized per token, row-major codes [m, f];
+// the f32 products are not stored.  f a multiple of 16.
+void swiglu_quantize_rows_i8(const float *gu, int8_t *xq_rowmajor, float *sx, uint64_t m, uint64_t f, hipStream_t s);
 // Per-tensor absmax -> scale = absmax / 448 (one f32) then e4m3 codes.
 void quantize_tensor_e4m3(const float *x, uint8_t *q, float *scale, float *absmax_scratch, uint64_t n,
                           hipStream_t s);
