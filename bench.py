@@ -353,6 +353,23 @@ def bench_prompt_prefill(fa, be, dec, cfg, tables, batch=4, l_new=2048, reps=2):
     return dict(batch=batch, l_new=l_new, ms=ms, tokens_per_s=batch * l_new / (ms * 1e-3))
 
 
+def bench_sampling(fa, be, rows=32, vocab=32000, iters=50):
+    """Device sampler at the decode step's logits shape, beside the greedy argmax it replaces."""
+    lib = fa.capi.lib
+    logits = be.alloc_uninit((rows, vocab))
+    fa.check(lib.fa_fill_normal(be._ctx, logits._h, 0, rows * vocab, 5, 0.0, 3.0))
+    gen = be.new_generator(1)
+    out = be.alloc_uninit((rows,), fa.capi.I32)
+    res = {}
+    for name, strategy, temperature, k in (("greedy", 0, 1.0, 0), ("temperature", 1, 0.8, 0), ("top_k_50", 2, 1.0, 50)):
+        sec = time_launches(fa, be, lambda: fa.check(lib.fa_sample_rows(be._ctx, logits._h, rows, vocab, strategy, temperature,
+                                                                       k, gen._h, out._h)), iters)
+        res[name + "_us"] = sec * 1e6
+    for b in (logits, gen, out):
+        b.free()
+    return res
+
+
 def bench_matrix_rate(fa, be, iters=20000):
     """Register-only rate of the matrix instructions the prefill GEMMs use, with all-zero and with
     random operand bits (the sustained clock of the part depends on the bits it multiplies)."""
@@ -555,6 +572,7 @@ def main():
         extras["paged_attention_bs64"] = dict(us=sec * 1e6, gbs=nb / sec / 1e9, frac=nb / sec / 1e9 / HBM_PEAK_GBS,
                                               bytes=nb)
         extras["decode_linears"] = bench_linears(fa, be, 100)
+        extras["sampling_32x32000"] = bench_sampling(fa, be)
         extras["prefill_gemm"] = bench_prefill(fa, be, 20)
     out = {
         "metric": METRIC, "value": batch / sec_per_step, "unit": "tokens/s", "n_gpus": 1, "steps": a.steps,

@@ -456,6 +456,21 @@ class RocmBackendOps:
         check(lib.fa_argmax_rows(self._ctx, x._h, rows, cols, out._h))
         return out
 
+    def new_generator(self, seed=0):
+        """Device-resident state of a ``Generator::new(seed)`` (crates/tensor-core/src/rng.rs:684-689)."""
+        g = self.alloc_zeroed((2,), capi.U32)
+        check(lib.fa_rng_seed(self._ctx, g._h, seed))
+        return g
+
+    def sample_rows(self, logits, strategy, temperature=1.0, top_k=0, generator=None):
+        """Next tokens [rows] (device buffer) from logits [rows, vocab]; strategy: SAMPLE_GREEDY /
+        SAMPLE_TEMPERATURE / SAMPLE_TOP_K (crates/autodiff/src/generate/mod.rs:376-424)."""
+        rows, vocab = logits.shape
+        out = self.alloc_uninit((rows,), capi.I32)
+        check(lib.fa_sample_rows(self._ctx, logits._h, rows, vocab, strategy, temperature, top_k,
+                                 generator._h if generator is not None else None, out._h))
+        return out
+
     def gather(self, table, idx):
         rows, cols = idx.shape[0], table.shape[1]
         out = self.alloc_uninit((rows, cols))
@@ -499,6 +514,9 @@ class RocmBackendOps:
         check(lib.fa_paged_attention_forward_device(self._ctx, q._h, k_pool._h, v_pool._h, block_tables._h,
                                                     seq_lens._h, C.byref(args.c()), out._h))
         return out
+
+
+SAMPLE_GREEDY, SAMPLE_TEMPERATURE, SAMPLE_TOP_K = 0, 1, 2
 
 
 def default_scale(head_dim):

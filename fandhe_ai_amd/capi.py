@@ -125,6 +125,9 @@ SIGNATURES = {
     "fa_paged_kv_append_device": (C.c_int32, [ctx_p, buf_p, buf_p, buf_p, buf_p, buf_p, u64, C.POINTER(PagedLayout)]),
     "fa_paged_attention_forward_device": (C.c_int32, [ctx_p, buf_p, buf_p, buf_p, buf_p, buf_p,
                                                       C.POINTER(PagedArgs), buf_p]),
+    "fa_sample_rows": (C.c_int32, [ctx_p, buf_p, u64, u64, C.c_int32, C.c_float, u64, buf_p, buf_p]),
+    "fa_rng_seed": (C.c_int32, [ctx_p, buf_p, u64]),
+    "fa_decoder_set_sampling": (C.c_int32, [ctx_p, C.c_void_p, C.c_int32, C.c_float, u64, u64]),
     "fa_decoder_prefill": (C.c_int32, [ctx_p, C.c_void_p, i32p, C.c_uint32]),
     "fa_probe_matrix_rate": (C.c_int32, [ctx_p, C.c_int32, buf_p, C.c_uint32, buf_p, C.POINTER(C.c_double)]),
     "fa_block_table_create": (C.c_int32, [C.POINTER(C.c_void_p)]),

@@ -489,6 +489,46 @@ fa_status fa_fill_normal(fa_context *ctx, fa_buffer *buf, uint64_t offset, uint6
     return after_launch(ctx, "fill_normal");
 }
 
+static fa_status check_sampling(fa_sampling strategy, float temperature, uint64_t top_k, uint64_t vocab) {
+    // GenerateConfig::validate (crates/autodiff/src/generate/mod.rs:170-215)
+    if (strategy != FA_SAMPLE_GREEDY && strategy != FA_SAMPLE_TEMPERATURE && strategy != FA_SAMPLE_TOP_K)
+        return fail(FA_ERR_INVALID_ARGUMENT, "sampling: unknown strategy");
+    if (strategy != FA_SAMPLE_GREEDY && !(std::isfinite(temperature) && temperature > 0.0f))
+        return fail(FA_ERR_INVALID_ARGUMENT, "sampling: temperature must be finite and positive");
+    if (strategy == FA_SAMPLE_TOP_K && (top_k == 0 || top_k > vocab))
+        return fail(FA_ERR_INVALID_ARGUMENT, "sampling: top_k must be in 1..=vocab");
+    return FA_OK;
+}
+
+fa_status fa_sample_rows(fa_context *ctx, const fa_buffer *logits, uint64_t rows, uint64_t vocab, fa_sampling strategy,
+                         float temperature, uint64_t top_k, fa_buffer *rng, fa_buffer *tokens) {
+    if (fa_status s = check_ctx(ctx)) return s;
+    uint64_t numel;
+    if (!mul3(rows, vocab, &numel)) return fail(FA_ERR_SHAPE_MISMATCH, "sample_rows: shape overflows");
+    if (fa_status s = check_buf_typed(ctx, logits, FA_F32, numel, "sample_rows: logits")) return s;
+    if (fa_status s = check_buf_typed(ctx, tokens, FA_I32, rows, "sample_rows: tokens")) return s;
+    if (vocab == 0 || vocab > (uint64_t)INT32_MAX) return fail(FA_ERR_INVALID_ARGUMENT, "sample_rows: vocab must be in 1..=i32::MAX");
+    if (rows > 65535) return fail(FA_ERR_INVALID_ARGUMENT, "sample_rows: at most 65535 rows per call");
+    if (fa_status s = check_sampling(strategy, temperature, top_k, vocab)) return s;
+    if (rows == 0) return FA_OK;
+    if (strategy == FA_SAMPLE_GREEDY) {
+        k::argmax_rows_f32((const float *)logits->ptr, (int32_t *)tokens->ptr, rows, vocab, ctx->stream);
+        return after_launch(ctx, "argmax_rows");
+    }
+    if (fa_status s = check_buf_typed(ctx, rng, FA_U32, 2, "sample_rows: rng")) return s;
+    k::sample_rows((const float *)logits->ptr, (int32_t *)tokens->ptr, (uint64_t *)rng->ptr, (uint32_t)rows, (uint32_t)vocab,
+                   strategy == FA_SAMPLE_TOP_K, temperature, (uint32_t)top_k, ctx->stream);
+    return after_launch(ctx, "sample_rows");
+}
+
+fa_status fa_rng_seed(fa_context *ctx, fa_buffer *rng, uint64_t seed) {
+    if (fa_status s = check_ctx(ctx)) return s;
+    if (fa_status s = check_buf_typed(ctx, rng, FA_U32, 2, "rng_seed: rng")) return s;
+    const uint64_t state = seed == 0 ? 0x9E3779B97F4A7C15ull : seed;
+    const uint32_t words[2] = {(uint32_t)state, (uint32_t)(state >> 32)};
+    return fa_upload_into(ctx, words, 2, rng, 0);
+}
+
 fa_status fa_probe_matrix_rate(fa_context *ctx, int32_t kind, const fa_buffer *operands, uint32_t iters, fa_buffer *sink,
                                double *ops) {
     if (fa_status s = check_ctx(ctx)) return s;

@@ -40,6 +40,11 @@ struct fa_decoder {
     fa_graph *graph = nullptr;
     uint32_t graph_batch = 0;
     int graph_waves = 0;
+    // how the step and the prompt pass pick the next token; rng holds the generator state on the device
+    fa_sampling strategy = FA_SAMPLE_GREEDY;
+    float temperature = 1.0f;
+    uint32_t top_k = 0;
+    fa_buffer *rng = nullptr;
     // host mirror of the installed block tables and of the sequence lengths (advanced with every step and
     // prompt chunk), used to validate that a prompt fits before anything is queued
     std::vector<uint32_t> host_tables, host_lens;
@@ -75,7 +80,7 @@ fa_status check_vec(const fa_decoder *d, const fa_buffer *b, uint64_t numel, con
 
 void free_all(fa_context *ctx, fa_decoder *d) {
     fa_buffer **bufs[] = {&d->tokens, &d->tables, &d->seq_lens, &d->pos, &d->slots, &d->cos_sin, &d->h, &d->xq,
-                          &d->sx,     &d->q_bf,     &d->attn, &d->act,  &d->pmax, &d->logits};
+                          &d->sx,     &d->q_bf,     &d->attn, &d->act,  &d->pmax, &d->logits, &d->rng};
     for (auto pb : bufs) {
         if (*pb) fa_buffer_free(ctx, *pb);
         *pb = nullptr;
@@ -85,6 +90,15 @@ void free_all(fa_context *ctx, fa_decoder *d) {
         if (l.v_pool) fa_buffer_free(ctx, l.v_pool);
         l.k_pool = l.v_pool = nullptr;
     }
+}
+
+// logits [batch, vocab] -> next tokens, by the decoder's sampling strategy
+void enqueue_pick(fa_decoder *d, hipStream_t s) {
+    if (d->strategy == FA_SAMPLE_GREEDY)
+        k::argmax_rows_f32((const float *)d->logits->ptr, (int32_t *)d->tokens->ptr, d->batch, d->cfg.vocab, s);
+    else
+        k::sample_rows((const float *)d->logits->ptr, (int32_t *)d->tokens->ptr, (uint64_t *)d->rng->ptr, d->batch,
+                       d->cfg.vocab, d->strategy == FA_SAMPLE_TOP_K, d->temperature, d->top_k, s);
 }
 
 // The kernels of one step, enqueued on the context's stream.
@@ -170,7 +184,7 @@ fa_status enqueue_step(fa_context *ctx, fa_decoder *d) {
     k::rmsnorm_quantize_i8((const float *)d->h->ptr, (const float *)d->final_norm->ptr, c.rms_eps, nullptr,
                            (int8_t *)d->xq->ptr, (float *)d->sx->ptr, B, m_pad, D, s);
     linear(d->lm_head, d->logits->ptr, nullptr);
-    k::argmax_rows_f32((const float *)d->logits->ptr, (int32_t *)d->tokens->ptr, B, V, s);
+    enqueue_pick(d, s);
     return after_launch(ctx, "decoder step");
 }
 
@@ -279,7 +293,7 @@ fa_status enqueue_prefill_chunk(fa_context *ctx, fa_decoder *d, PrefillBuffers &
         ep.out_bf16 = 0;
         k::linear_w8a8_skinny((const int8_t *)d->xq->ptr, (const int8_t *)d->lm_head->codes->ptr, B, d->lm_head->n,
                               d->lm_head->n_pad, d->lm_head->k_pad, ep, cus, s);
-        k::argmax_rows_f32((const float *)d->logits->ptr, (int32_t *)d->tokens->ptr, B, V, s);
+        enqueue_pick(d, s);
     }
     return after_launch(ctx, "decoder prefill");
 }
@@ -338,6 +352,7 @@ fa_status fa_decoder_create(fa_context *ctx, const fa_decoder_config *cfg, fa_de
     mk(FA_F32, B * F, &d->act);
     mk(FA_F32, B * std::max<uint64_t>(F / 16, c.n_heads), &d->pmax);
     mk(FA_F32, B * V, &d->logits);
+    mk(FA_U32, 2, &d->rng);
     for (auto &l : d->layers) {
         mk(FA_BF16, layout.num_blocks * layout.block_size * layout.embed_dim, &l.k_pool);
         mk(FA_BF16, layout.num_blocks * layout.block_size * layout.embed_dim, &l.v_pool);
@@ -400,6 +415,28 @@ fa_status fa_decoder_set_head(fa_decoder *d, const fa_buffer *embed, const fa_bu
     d->lm_head = lm_head;
     if (d->graph) {
         fa_graph_destroy(d->ctx, d->graph);
+        d->graph = nullptr;
+    }
+    return FA_OK;
+}
+
+fa_status fa_decoder_set_sampling(fa_context *ctx, fa_decoder *d, fa_sampling strategy, float temperature, uint64_t top_k,
+                                  uint64_t seed) {
+    if (fa_status s = check_ctx(ctx)) return s;
+    if (fa_status s = check_dec(d)) return s;
+    if (d->ctx != ctx) return fail(FA_ERR_DEVICE_MISMATCH, "decoder_set_sampling: decoder belongs to another context");
+    if (strategy != FA_SAMPLE_GREEDY && strategy != FA_SAMPLE_TEMPERATURE && strategy != FA_SAMPLE_TOP_K)
+        return fail(FA_ERR_INVALID_ARGUMENT, "decoder_set_sampling: unknown strategy");
+    if (strategy != FA_SAMPLE_GREEDY && !(std::isfinite(temperature) && temperature > 0.0f))
+        return fail(FA_ERR_INVALID_ARGUMENT, "decoder_set_sampling: temperature must be finite and positive");
+    if (strategy == FA_SAMPLE_TOP_K && (top_k == 0 || top_k > d->cfg.vocab))
+        return fail(FA_ERR_INVALID_ARGUMENT, "decoder_set_sampling: top_k must be in 1..=vocab");
+    if (fa_status s = fa_rng_seed(ctx, d->rng, seed)) return s;
+    d->strategy = strategy;
+    d->temperature = temperature;
+    d->top_k = (uint32_t)top_k;
+    if (d->graph) {                                     // the captured step holds the old choice
+        fa_graph_destroy(ctx, d->graph);
         d->graph = nullptr;
     }
     return FA_OK;

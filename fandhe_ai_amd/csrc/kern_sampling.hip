@@ -1,0 +1,214 @@
+// Next-token sampling on the device: temperature / top-k softmax weights and one multinomial draw per row,
+// with the reference's host arithmetic (crates/autodiff/src/generate/mod.rs:347-369, 432-452;
+// crates/tensor-core/src/rng.rs:65-104, 509-539): weights (f32) = f64 exp((logit - max) / t) / f64 sum,
+// top-k keeps the k largest by (value descending, index ascending), the draw is the first index whose f64
+// cumulative weight exceeds u * total, u the next 53-bit uniform of an xorshift64* generator whose state
+// lives on the device; rows draw in row order from the one generator.  Only the order of the f64 sums
+// differs from the host loop (a block-wide tree instead of a sequential pass).
+#include "device_utils.hpp"
+#include "kernels.hpp"
+
+namespace fa {
+namespace k {
+using namespace fa::dev;
+
+namespace {
+
+constexpr int kThreads = 1024;
+
+__device__ __forceinline__ uint64_t xorshift64star_next(uint64_t &state) {
+    uint64_t x = state;
+    x ^= x << 13;
+    x ^= x >> 7;
+    x ^= x << 17;
+    state = x;
+    return x * 0x2545F4914F6CDD1Dull;
+}
+
+// larger float <-> larger key (finite values)
+__device__ __forceinline__ uint32_t order_key(float v) {
+    uint32_t u = __float_as_uint(v);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+// exclusive prefix sums of one value per thread over the block; returns the block total through *total
+template <typename T>
+__device__ __forceinline__ T block_exclusive_scan(T v, T *buf, T *total) {
+    const int t = threadIdx.x;
+    buf[t] = v;
+    __syncthreads();
+    for (int off = 1; off < kThreads; off <<= 1) {
+        T add = t >= off ? buf[t - off] : (T)0;
+        __syncthreads();
+        buf[t] += add;
+        __syncthreads();
+    }
+    T incl = buf[t];
+    *total = buf[kThreads - 1];
+    __syncthreads();
+    return incl - v;
+}
+
+__global__ void __launch_bounds__(kThreads)
+    sample_rows_kernel(const float *__restrict__ logits, int32_t *__restrict__ tokens, const uint64_t *__restrict__ rng_state,
+                       uint32_t vocab, int top_k_mode, float temperature, uint32_t top_k) {
+    __shared__ double s_d[kThreads];
+    __shared__ uint32_t s_u[kThreads];
+    __shared__ uint32_t hist[256];
+    __shared__ float s_max[kThreads / 64];
+    __shared__ uint32_t s_sel[4];            // radix-select state: prefix, remaining; flags
+    __shared__ double s_x;
+    const uint32_t b = blockIdx.x, t = threadIdx.x;
+    const float *row = logits + (uint64_t)b * vocab;
+    const uint32_t seg = (vocab + kThreads - 1) / kThreads;
+    const uint32_t lo = t * seg < vocab ? t * seg : vocab, hi = lo + seg < vocab ? lo + seg : vocab;
+
+    // ---- every logit finite (the reference rejects the step otherwise); row maximum
+    float mx = -INFINITY;
+    bool finite = true;
+    for (uint32_t i = lo; i < hi; ++i) {
+        float v = row[i];
+        finite = finite && (fabsf(v) <= 3.402823466e38f);            // false for NaN and +-inf
+        mx = fmaxf(mx, v);
+    }
+    if (t < 4) s_sel[t] = 0;
+    __syncthreads();
+    if (!finite) atomicOr(&s_sel[2], 1u);
+    mx = wave_max(mx);
+    if (t % 64 == 0) s_max[t / 64] = mx;
+    __syncthreads();
+    if (s_sel[2]) {
+        if (t == 0) tokens[b] = -1;
+        return;
+    }
+    mx = s_max[0];
+    for (int w = 1; w < kThreads / 64; ++w) mx = fmaxf(mx, s_max[w]);
+    const double dmax = (double)mx, dt = (double)temperature;
+
+    // ---- top-k: key of the k-th largest value and how many elements with that key are kept (lowest indices)
+    uint32_t thr_key = 0, keep_equal = 0xffffffffu, eq_rank = 0;
+    if (top_k_mode) {
+        uint32_t prefix = 0, mask = 0, remaining = top_k;
+        for (int pass = 0; pass < 4; ++pass) {
+            const int shift = 24 - 8 * pass;
+            if (t < 256) hist[t] = 0;
+            __syncthreads();
+            for (uint32_t i = lo; i < hi; ++i) {
+                uint32_t key = order_key(row[i]);
+                if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
+            }
+            __syncthreads();
+            if (t == 0) {
+                uint32_t cum = 0, bin = 255;
+                for (;; --bin) {
+                    if (cum + hist[bin] >= remaining || bin == 0) break;
+                    cum += hist[bin];
+                }
+                s_sel[0] = prefix | (bin << shift);
+                s_sel[1] = remaining - cum;
+            }
+            __syncthreads();
+            prefix = s_sel[0];
+            remaining = s_sel[1];
+            mask |= 255u << shift;
+            __syncthreads();
+        }
+        thr_key = prefix;
+        keep_equal = remaining;
+        uint32_t eq = 0;
+        for (uint32_t i = lo; i < hi; ++i) eq += order_key(row[i]) == thr_key ? 1u : 0u;
+        uint32_t eq_total;
+        eq_rank = block_exclusive_scan<uint32_t>(eq, s_u, &eq_total);
+    }
+    // kept(i): walks the segment in index order with a running rank among the elements equal to the threshold
+    auto for_each_kept = [&](auto &&f) {
+        uint32_t rank = eq_rank;
+        for (uint32_t i = lo; i < hi; ++i) {
+            const float v = row[i];
+            bool kept = true;
+            if (top_k_mode) {
+                const uint32_t key = order_key(v);
+                if (key == thr_key) {
+                    kept = rank < keep_equal;
+                    ++rank;
+                } else {
+                    kept = key > thr_key;
+                }
+            }
+            f(i, v, kept);
+        }
+    };
+
+    // ---- f64 sum of the exponentials of the kept logits
+    double part = 0.0;
+    for_each_kept([&](uint32_t, float v, bool kept) {
+        if (kept) part += exp(((double)v - dmax) / dt);
+    });
+    double sum_exp;
+    (void)block_exclusive_scan<double>(part, s_d, &sum_exp);
+
+    // ---- f32 weights, their f64 cumulative sums, and the draw
+    auto weight = [&](float v, bool kept) -> float { return kept ? (float)(exp(((double)v - dmax) / dt) / sum_exp) : 0.0f; };
+    double wsum = 0.0;
+    uint32_t last_pos = 0;
+    bool any_pos = false;
+    for_each_kept([&](uint32_t i, float v, bool kept) {
+        const float w = weight(v, kept);
+        wsum += (double)w;
+        if (w > 0.0f) {
+            last_pos = i;
+            any_pos = true;
+        }
+    });
+    double total;
+    const double before = block_exclusive_scan<double>(wsum, s_d, &total);
+    if (t == 0) {
+        uint64_t st = rng_state[0];
+        uint64_t bits = 0;
+        for (uint32_t r = 0; r <= b; ++r) bits = xorshift64star_next(st);     // row b takes the (b + 1)-th draw of the step
+        s_x = (double)(bits >> 11) / 9007199254740992.0 * total;
+        s_sel[0] = 0xffffffffu;                 // first index whose cumulative weight exceeds x
+        s_sel[1] = 0;                           // last index with a positive weight (+ 1)
+    }
+    __syncthreads();
+    const double x = s_x;
+    if (any_pos) atomicMax(&s_sel[1], last_pos + 1);
+    {
+        // Every thread looks for the first positive-weight element of its segment whose cumulative weight
+        // exceeds x and the block keeps the smallest such index: in a segment past the crossing that is its
+        // first positive element, which loses against the true crossing further left, and the rounding of
+        // the scanned offsets against the running sums cannot leave x between two segments unnoticed.
+        double acc = before;
+        uint32_t found = 0xffffffffu;
+        for_each_kept([&](uint32_t i, float v, bool kept) {
+            const float w = weight(v, kept);
+            acc += (double)w;
+            if (found == 0xffffffffu && w > 0.0f && acc > x) found = i;
+        });
+        if (found != 0xffffffffu) atomicMin(&s_sel[0], found);
+    }
+    __syncthreads();
+    if (t == 0) {
+        uint32_t idx = s_sel[0];
+        if (idx == 0xffffffffu) idx = s_sel[1] ? s_sel[1] - 1 : vocab - 1;
+        tokens[b] = (int32_t)idx;
+    }
+}
+
+__global__ void advance_rng_kernel(uint64_t *state, uint32_t draws) {
+    uint64_t st = state[0];
+    for (uint32_t i = 0; i < draws; ++i) (void)xorshift64star_next(st);
+    state[0] = st;
+}
+
+}  // namespace
+
+void sample_rows(const float *logits, int32_t *tokens, uint64_t *rng_state, uint32_t rows, uint32_t vocab, int top_k_mode,
+                 float temperature, uint32_t top_k, hipStream_t s) {
+    if (rows == 0 || vocab == 0) return;
+    sample_rows_kernel<<<rows, kThreads, 0, s>>>(logits, tokens, rng_state, vocab, top_k_mode, temperature, top_k);
+    advance_rng_kernel<<<1, 1, 0, s>>>(rng_state, rows);
+}
+
+}  // namespace k
+}  // namespace fa

@@ -169,6 +169,13 @@ void paged_attention_prefill_bf16(const uint16_t *q, const uint16_t *k_pool, con
                                   const uint32_t *tables, const uint32_t *seq_lens, const PagedShape &ps,
                                   uint32_t waves_per_cu, void *workspace, void *out, int out_bf16, hipStream_t s);
 
+// ---- sampling (kern_sampling.hip) ------------------------------------------------
+// One token per row of logits [rows, vocab] by temperature (top_k_mode 0) or top-k (1) sampling with the
+// reference's arithmetic; row b takes the (b + 1)-th draw of the xorshift64* generator at rng_state, which is
+// advanced by `rows` draws afterwards.  A row with a non-finite logit gets token -1.
+void sample_rows(const float *logits, int32_t *tokens, uint64_t *rng_state, uint32_t rows, uint32_t vocab, int top_k_mode,
+                 float temperature, uint32_t top_k, hipStream_t s);
+
 // ---- measurement aid (kern_probe.hip) -------------------------------------------
 // Launches a register-only loop of one matrix instruction kind (0: i32_16x16x64_i8, 1: i32_32x32x32_i8,
 // 2: scaled f32_16x16x128 on e4m3) whose operand bits come from `operands` (64 KiB); returns the number

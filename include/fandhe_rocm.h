@@ -213,6 +213,22 @@ fa_status fa_gather_rows(fa_context *ctx, const fa_buffer *table, uint64_t table
  * reference's interface. */
 fa_status fa_fill_normal(fa_context *ctx, fa_buffer *buf, uint64_t offset, uint64_t numel,
                          uint64_t seed, float mean, float std);
+/* Next-token sampling from logits [rows, vocab] (f32), on the device, with the
+ * arithmetic of the reference's host sampler (crates/autodiff/src/generate/mod.rs:
+ * 333-452, sample_step / sampling_weights_f32; crates/tensor-core/src/rng.rs:
+ * 509-539 multinomial): strategy 0 greedy (first maximum), 1 temperature, 2
+ * top-k (k largest by value descending, index ascending; temperature applies
+ * too, the reference fixes it at 1).  rng: a U32 buffer of at least two
+ * elements holding the 64-bit state of the xorshift64* generator
+ * (fa_rng_seed); rows draw in row order, one draw each; greedy draws nothing.
+ * tokens: I32 [rows].  A row with a non-finite logit gets token -1 (the
+ * reference fails the step).  Asynchronous. */
+typedef enum fa_sampling { FA_SAMPLE_GREEDY = 0, FA_SAMPLE_TEMPERATURE = 1, FA_SAMPLE_TOP_K = 2 } fa_sampling;
+fa_status fa_sample_rows(fa_context *ctx, const fa_buffer *logits, uint64_t rows, uint64_t vocab,
+                         fa_sampling strategy, float temperature, uint64_t top_k, fa_buffer *rng,
+                         fa_buffer *tokens);
+/* Generator::new(seed) (rng.rs:65-69, 684-689): seed 0 selects 0x9E3779B97F4A7C15. */
+fa_status fa_rng_seed(fa_context *ctx, fa_buffer *rng, uint64_t seed);
 /* Measurement aid, not part of the reference's interface: queues a loop of one
  * matrix instruction kind with operands held in registers (kind 0:
  * v_mfma_i32_16x16x64_i8, 1: v_mfma_i32_32x32x32_i8, 2: the scaled
@@ -407,6 +423,12 @@ fa_status fa_decoder_set_tokens(fa_context *ctx, fa_decoder *dec, const int32_t 
  * as the next step's input.  use_graph != 0 replays a captured HIP graph of
  * the step (captured on first use). */
 fa_status fa_decoder_step(fa_context *ctx, fa_decoder *dec, int32_t use_graph);
+/* How fa_decoder_step and fa_decoder_prefill pick the next token from the
+ * logits (fa_sample_rows; greedy until this is called) and the seed of the
+ * decoder's generator, whose state stays on the device so that a sampled step
+ * can be captured and replayed like a greedy one. */
+fa_status fa_decoder_set_sampling(fa_context *ctx, fa_decoder *dec, fa_sampling strategy, float temperature,
+                                  uint64_t top_k, uint64_t seed);
 /* Prompt ingestion: l_new tokens per installed sequence (tokens [batch, l_new],
  * host array), written behind what each sequence has cached, on the
  * prefill-shape GEMMs and the prefill form of the attention kernel, in chunks of

@@ -143,6 +143,9 @@ class GpuDecoder:
     def step(self, use_graph):
         self.fa.check(self.fa.capi.lib.fa_decoder_step(self.be._ctx, self.h, 1 if use_graph else 0))
 
+    def set_sampling(self, strategy, temperature=1.0, top_k=0, seed=0):
+        self.fa.check(self.fa.capi.lib.fa_decoder_set_sampling(self.be._ctx, self.h, strategy, temperature, top_k, seed))
+
     def prefill(self, prompt):
         """prompt: int32 [batch, l_new]"""
         p = np.ascontiguousarray(prompt, dtype=np.int32)

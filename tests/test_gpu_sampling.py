@@ -1,0 +1,101 @@
+"""GPU parity of the device sampler (fa_sample_rows) against the oracle restatement of the reference's
+host sampler: the same tokens for the same logits, strategy and generator seed, over consecutive steps
+(the generator state advances on the device), with ties in the logits, zero weights, and rows whose
+logits are not finite."""
+import os
+import sys
+
+import numpy as np
+import pytest
+
+import oracle_lib as o
+from decoder_common import GpuDecoder, build_model
+from gpu_common import ops
+
+sys.path.insert(0, os.path.join(os.path.dirname(__file__), "..", "oracle"))
+import sampling as os_  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+
+
+def _fa():
+    import fandhe_ai_amd as fa
+    return fa
+
+
+def _logits(rng, rows, vocab, kind):
+    x = rng.standard_normal((rows, vocab)).astype(np.float32) * 3
+    if kind == "ties":
+        x = np.round(x)                                    # many equal values: tie-breaking by index matters
+    elif kind == "peaked":
+        x *= 20                                            # most weights underflow to zero
+    elif kind == "flat":
+        x[:] = 1.25
+    return x
+
+
+CASES = [(rows, vocab, kind) for rows, vocab in ((1, 17), (5, 1000), (32, 32000), (3, 50257), (2, 1024), (7, 1))
+         for kind in ("normal", "ties", "peaked", "flat")]
+
+
+@pytest.mark.parametrize("rows,vocab,kind", CASES, ids=["%dx%d_%s" % c for c in CASES])
+def test_sampled_tokens_equal_the_oracle(rows, vocab, kind):
+    fa = _fa()
+    be = ops()
+    rng = np.random.default_rng(rows * 7 + vocab)
+    strategies = [(fa.SAMPLE_TEMPERATURE, 1.0, 0), (fa.SAMPLE_TEMPERATURE, 0.6, 0), (fa.SAMPLE_TEMPERATURE, 1.7, 0),
+                  (fa.SAMPLE_TOP_K, 1.0, 1), (fa.SAMPLE_TOP_K, 1.0, min(5, vocab)), (fa.SAMPLE_TOP_K, 0.8, min(50, vocab)),
+                  (fa.SAMPLE_TOP_K, 1.0, vocab)]
+    for strategy, temperature, k in strategies:
+        seed = 11 + k
+        gen = be.new_generator(seed)
+        ref = os_.Generator(seed)
+        for step in range(3):
+            x = _logits(rng, rows, vocab, kind)
+            got = be.download_owned(be.sample_rows(be.upload(x), strategy, temperature, k, gen))
+            want = os_.sample_step(x, strategy, temperature, k or None, ref)
+            assert np.array_equal(got, want), (strategy, temperature, k, step, got[:8], want[:8])
+        state = be.download(gen)
+        assert (int(state[1]) << 32 | int(state[0])) == ref.state
+
+
+def test_greedy_top1_and_non_finite_rows():
+    fa = _fa()
+    be = ops()
+    rng = np.random.default_rng(3)
+    x = np.round(rng.standard_normal((6, 999)).astype(np.float32) * 2)
+    greedy = be.download_owned(be.sample_rows(be.upload(x), fa.SAMPLE_GREEDY))
+    assert np.array_equal(greedy, o.argmax_rows(x))
+    gen = be.new_generator(0)
+    top1 = be.download_owned(be.sample_rows(be.upload(x), fa.SAMPLE_TOP_K, 1.0, 1, gen))
+    assert np.array_equal(top1, greedy)                    # first maximum, as the reference's ordering keeps it
+    bad = x.copy()
+    bad[1, 5] = np.nan
+    bad[4, 998] = -np.inf
+    got = be.download_owned(be.sample_rows(be.upload(bad), fa.SAMPLE_TEMPERATURE, 1.0, 0, gen))
+    assert got[1] == -1 and got[4] == -1 and (got[[0, 2, 3, 5]] >= 0).all()
+    for args in ((fa.SAMPLE_TEMPERATURE, 0.0, 0), (fa.SAMPLE_TEMPERATURE, float("nan"), 0), (fa.SAMPLE_TOP_K, 1.0, 0),
+                 (fa.SAMPLE_TOP_K, 1.0, 1000), (7, 1.0, 0)):
+        with pytest.raises(fa.InvalidArgument):
+            be.sample_rows(be.upload(x), *args, generator=gen)
+
+
+def test_decoder_steps_with_sampling_follow_the_oracle_generator():
+    fa = _fa()
+    be = ops()
+    m = build_model(seed=4, n_layers=1, d_model=256, n_heads=2, n_kv_heads=1, d_ffn=256, vocab=700, batch=5,
+                    ctxs=[3, 20, 9, 33, 1], steps=8)
+    dec = GpuDecoder(be, m)
+    try:
+        for strategy, temperature, k, seed in ((fa.SAMPLE_TOP_K, 1.0, 40, 5), (fa.SAMPLE_TEMPERATURE, 0.9, 0, 0)):
+            dec.set_sampling(strategy, temperature, k, seed)
+            ref = os_.Generator(seed)
+            for step in range(3):
+                dec.step(use_graph=(step > 0))
+                want = os_.sample_step(dec.logits(), strategy, temperature, k or None, ref)
+                assert np.array_equal(dec.tokens(), want), (strategy, step)
+        dec.set_sampling(fa.SAMPLE_GREEDY)
+        dec.step(False)
+        assert np.array_equal(dec.tokens(), o.argmax_rows(dec.logits()))
+    finally:
+        dec.close()
