@@ -353,6 +353,36 @@ def bench_prompt_prefill(fa, be, dec, cfg, tables, batch=4, l_new=2048, reps=2):
     return dict(batch=batch, l_new=l_new, ms=ms, tokens_per_s=batch * l_new / (ms * 1e-3))
 
 
+def bench_continuous_batching(fa, be, dec, dcfg, requests=96, max_active=32):
+    """Continuous batching on the resident model: requests with prompts of 64..512 tokens that each generate
+    64..192 tokens (greedy, temperature and top-k mixed) join and leave a batch of at most `max_active` rows;
+    wall time from the first submit to the last finished request, prompts included."""
+    from fandhe_ai_amd.scheduler import BatchScheduler, GenerateConfig, SamplingStrategy, SchedulerLimits
+    rng = np.random.default_rng(12)
+    d = fa.Decoder.from_handle(be, dec, dcfg)
+    s = BatchScheduler(d, SchedulerLimits(max_active, requests, 1024))
+    prompt_tokens = new_tokens = 0
+    for i in range(requests):
+        plen, gen = int(rng.integers(64, 513)), int(rng.integers(64, 193))
+        strategy = (SamplingStrategy.Greedy(), SamplingStrategy.Temperature(0.8), SamplingStrategy.TopK(50))[i % 3]
+        s.submit(rng.integers(0, dcfg.vocab, plen).astype(np.int32), GenerateConfig.new(plen + gen, strategy).with_seed(i + 1))
+        prompt_tokens += plen
+        new_tokens += gen
+    be.synchronize_device()
+    t0 = time.perf_counter()
+    steps = rows = done = 0
+    while s.active_len() or s.queued_len():
+        done += s.step()
+        rows += s.active_len()
+        steps += 1
+        assert steps < 100000
+    be.synchronize_device()
+    sec = time.perf_counter() - t0
+    assert done == requests and not s.take_failed() and len(s.take_finished()) == requests
+    return dict(requests=requests, max_active=max_active, prompt_tokens=prompt_tokens, generated_tokens=new_tokens,
+                seconds=sec, generated_tokens_per_s=new_tokens / sec, iterations=steps, mean_active_rows=rows / steps)
+
+
 def bench_sampling(fa, be, rows=32, vocab=32000, iters=50):
     """Device sampler at the decode step's logits shape, beside the greedy argmax it replaces."""
     lib = fa.capi.lib
@@ -546,6 +576,15 @@ def main():
             prompt = bench_prompt_prefill(fa, be, dec, cfg, np.ascontiguousarray(tables[order]))
             log("prompt prefill %d x %d tokens: %.1f ms, %.0f tokens/s" %
                 (prompt["batch"], prompt["l_new"], prompt["ms"], prompt["tokens_per_s"]))
+    batching = None
+    if not a.no_extras:
+        dcfg = fa.capi.DecoderConfig(cfg["n_layers"], cfg["d_model"], cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"],
+                                     cfg["d_ffn"], cfg["vocab"], cfg["block_size"], max_blocks, num_blocks, batch,
+                                     cfg["rms_eps"], cfg["rope_theta"])
+        batching = bench_continuous_batching(fa, be, dec, dcfg, max_active=batch)
+        log("continuous batching: %d requests, %d generated tokens in %.2f s -> %.0f generated tokens/s "
+            "(mean %.1f active rows)" % (batching["requests"], batching["generated_tokens"], batching["seconds"],
+                                         batching["generated_tokens_per_s"], batching["mean_active_rows"]))
     lib.fa_decoder_destroy(be._ctx, dec)
     for x in keep:
         x.free()
@@ -566,6 +605,8 @@ def main():
     extras = {"step_algorithmic_gb": bytes_step / 1e9, "step_hbm_frac": bytes_step / sec_per_step / 1e9 / HBM_PEAK_GBS}
     if prompt is not None:
         extras["prompt_prefill"] = prompt
+    if batching is not None:
+        extras["continuous_batching"] = batching
     if not a.no_extras:
         c3 = np.random.default_rng(0).integers(128, 4097, size=64).tolist()
         sec, nb = bench_attention(fa, be, 64, 32, 8, c3, 40000, 50, seed=3)

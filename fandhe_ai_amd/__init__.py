@@ -9,3 +9,4 @@ from .backend import *  # noqa: F401,F403
 from .paged_cache import BlockTable, PagedKvCache, PagedKvCacheConfig  # noqa: F401,E402
 from .decoder import Decoder  # noqa: F401,E402
 from . import safetensors_io  # noqa: F401,E402
+from . import scheduler  # noqa: F401,E402

@@ -471,6 +471,23 @@ class RocmBackendOps:
                                  generator._h if generator is not None else None, out._h))
         return out
 
+    def sample_rows_per_row(self, logits, table):
+        """Next tokens [rows] where row r follows record r of `table`, a U32 device buffer of 6 * rows elements
+        holding fa_row_sampling records (see ``row_sampling_table``); generator states advance in the table."""
+        rows, vocab = logits.shape
+        out = self.alloc_uninit((rows,), capi.I32)
+        check(lib.fa_sample_rows_per_row(self._ctx, logits._h, rows, vocab, table._h, out._h))
+        return out
+
+    def row_sampling_table(self, records):
+        """records: [(strategy, temperature, top_k, seed)] -> device table for ``sample_rows_per_row``."""
+        arr = (capi.RowSampling * len(records))()
+        for r, (strategy, temperature, top_k, seed) in zip(arr, records):
+            st = capi.u64()
+            check(lib.fa_rng_state_from_seed(seed, C.byref(st)))
+            r.rng_state, r.temperature, r.top_k, r.strategy = st.value, temperature, top_k, strategy
+        return self.upload(np.frombuffer(bytes(arr), dtype=np.uint32).copy(), capi.U32)
+
     def gather(self, table, idx):
         rows, cols = idx.shape[0], table.shape[1]
         out = self.alloc_uninit((rows, cols))

@@ -63,6 +63,12 @@ class PagedPlan(C.Structure):
     _fields_ = [("out_numel", u64), ("s_max", u64), ("query_rows", u64), ("workspace_elems", u64)]
 
 
+class RowSampling(C.Structure):
+    """fa_row_sampling: one request's strategy and generator state."""
+    _fields_ = [("rng_state", C.c_uint64), ("temperature", C.c_float), ("top_k", C.c_uint32),
+                ("strategy", C.c_int32), ("reserved", C.c_uint32)]
+
+
 class DecoderConfig(C.Structure):
     _fields_ = [("n_layers", C.c_uint32), ("d_model", C.c_uint32), ("n_heads", C.c_uint32),
                 ("n_kv_heads", C.c_uint32), ("head_dim", C.c_uint32), ("d_ffn", C.c_uint32),
@@ -128,6 +134,10 @@ SIGNATURES = {
     "fa_sample_rows": (C.c_int32, [ctx_p, buf_p, u64, u64, C.c_int32, C.c_float, u64, buf_p, buf_p]),
     "fa_rng_seed": (C.c_int32, [ctx_p, buf_p, u64]),
     "fa_decoder_set_sampling": (C.c_int32, [ctx_p, C.c_void_p, C.c_int32, C.c_float, u64, u64]),
+    "fa_rng_state_from_seed": (C.c_int32, [u64, C.POINTER(u64)]),
+    "fa_sample_rows_per_row": (C.c_int32, [ctx_p, buf_p, u64, u64, buf_p, buf_p]),
+    "fa_decoder_set_row_sampling": (C.c_int32, [ctx_p, C.c_void_p, C.POINTER(RowSampling)]),
+    "fa_decoder_read_row_sampling": (C.c_int32, [ctx_p, C.c_void_p, C.POINTER(RowSampling)]),
     "fa_decoder_prefill": (C.c_int32, [ctx_p, C.c_void_p, i32p, C.c_uint32]),
     "fa_probe_matrix_rate": (C.c_int32, [ctx_p, C.c_int32, buf_p, C.c_uint32, buf_p, C.POINTER(C.c_double)]),
     "fa_block_table_create": (C.c_int32, [C.POINTER(C.c_void_p)]),

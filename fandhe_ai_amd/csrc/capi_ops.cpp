@@ -12,7 +12,7 @@ using namespace fa;
 
 namespace fa {
 namespace k {
-extern int g_skinny_ntw, g_skinny_waves, g_skinny_astat, g_gemm_small_tiles, g_gemm_waves, g_gemm_ntb;
+extern int g_skinny_ntw, g_skinny_waves, g_skinny_astat, g_gemm_small_tiles, g_gemm_waves, g_gemm_ntb, g_gemm_split_fill;
 }
 int g_decode_waves = 0;
 int g_prefill_generic = 0;
@@ -79,6 +79,7 @@ fa_status fa_set_tuning(int32_t key, int32_t value) {
         case 6: k::g_gemm_waves = value; return FA_OK;
         case 7: k::g_gemm_ntb = value; return FA_OK;
         case 8: fa::g_prefill_generic = value; return FA_OK;
+        case 9: k::g_gemm_split_fill = value; return FA_OK;
     }
     return fail(FA_ERR_INVALID_ARGUMENT, "fa_set_tuning: unknown key");
 }
@@ -308,8 +309,11 @@ fa_status fa_linear_w8a8(fa_context *ctx, const fa_buffer *x, uint64_t m, const 
         if (fa_status s = xq.get(mk)) return s;
         k::quantize_rows_i8(x->ptr, x->dtype == FA_BF16, (int8_t *)xq.ptr, nullptr, (float *)sx.ptr, m, m, qw->k,
                             qw->k_pad, ctx->stream);
+        Scratch ws(ctx);
+        if (uint64_t wsb = k::gemm_w8a8_workspace_bytes(m, qw->n, qw->n_pad, qw->k_pad, ctx->props.multiProcessorCount))
+            if (fa_status s = ws.get(wsb)) return s;
         k::gemm_w8a8_mfma((const int8_t *)xq.ptr, (const int8_t *)qw->codes->ptr, m, qw->n, qw->n_pad, qw->k_pad, ep,
-                          ctx->props.multiProcessorCount, ctx->stream);
+                          ctx->props.multiProcessorCount, ctx->stream, ws.ptr, ws.bytes);
     }
     return after_launch(ctx, "linear_w8a8");
 }
@@ -336,8 +340,11 @@ fa_status fa_gemm_w8a8(fa_context *ctx, const fa_buffer *aq, const fa_buffer *sx
     ep.acc_out = acc_out ? (int32_t *)acc_out->ptr : nullptr;
     ep.out = out->ptr;
     ep.out_bf16 = out->dtype == FA_BF16;
+    Scratch ws(ctx);
+    if (uint64_t wsb = k::gemm_w8a8_workspace_bytes(m, qw->n, qw->n_pad, qw->k_pad, ctx->props.multiProcessorCount))
+        if (fa_status s = ws.get(wsb)) return s;
     k::gemm_w8a8_mfma((const int8_t *)aq->ptr, (const int8_t *)qw->codes->ptr, m, qw->n, qw->n_pad, qw->k_pad, ep,
-                      ctx->props.multiProcessorCount, ctx->stream);
+                      ctx->props.multiProcessorCount, ctx->stream, ws.ptr, ws.bytes);
     return after_launch(ctx, "gemm_w8a8_mfma");
 }
 
@@ -524,9 +531,33 @@ fa_status fa_sample_rows(fa_context *ctx, const fa_buffer *logits, uint64_t rows
 fa_status fa_rng_seed(fa_context *ctx, fa_buffer *rng, uint64_t seed) {
     if (fa_status s = check_ctx(ctx)) return s;
     if (fa_status s = check_buf_typed(ctx, rng, FA_U32, 2, "rng_seed: rng")) return s;
-    const uint64_t state = seed == 0 ? 0x9E3779B97F4A7C15ull : seed;
+    uint64_t state;
+    (void)fa_rng_state_from_seed(seed, &state);
     const uint32_t words[2] = {(uint32_t)state, (uint32_t)(state >> 32)};
     return fa_upload_into(ctx, words, 2, rng, 0);
+}
+
+fa_status fa_rng_state_from_seed(uint64_t seed, uint64_t *state) {
+    if (!state) return fail(FA_ERR_INVALID_ARGUMENT, "rng_state_from_seed: null state");
+    *state = seed == 0 ? 0x9E3779B97F4A7C15ull : seed;
+    return FA_OK;
+}
+
+fa_status fa_sample_rows_per_row(fa_context *ctx, const fa_buffer *logits, uint64_t rows, uint64_t vocab, fa_buffer *table,
+                                 fa_buffer *tokens) {
+    if (fa_status s = check_ctx(ctx)) return s;
+    uint64_t numel;
+    if (!mul3(rows, vocab, &numel)) return fail(FA_ERR_SHAPE_MISMATCH, "sample_rows_per_row: shape overflows");
+    if (fa_status s = check_buf_typed(ctx, logits, FA_F32, numel, "sample_rows_per_row: logits")) return s;
+    if (fa_status s = check_buf_typed(ctx, tokens, FA_I32, rows, "sample_rows_per_row: tokens")) return s;
+    if (vocab == 0 || vocab > (uint64_t)INT32_MAX)
+        return fail(FA_ERR_INVALID_ARGUMENT, "sample_rows_per_row: vocab must be in 1..=i32::MAX");
+    if (rows > 65535) return fail(FA_ERR_INVALID_ARGUMENT, "sample_rows_per_row: at most 65535 rows per call");
+    if (fa_status s = check_buf_typed(ctx, table, FA_U32, rows * 6, "sample_rows_per_row: table")) return s;
+    if (rows == 0) return FA_OK;
+    k::sample_rows_policy((const float *)logits->ptr, (int32_t *)tokens->ptr, (k::RowPolicy *)table->ptr, (uint32_t)rows,
+                          (uint32_t)vocab, ctx->stream);
+    return after_launch(ctx, "sample_rows_per_row");
 }
 
 fa_status fa_probe_matrix_rate(fa_context *ctx, int32_t kind, const fa_buffer *operands, uint32_t iters, fa_buffer *sink,

@@ -3,6 +3,7 @@
 // greedy argmax that the benchmark's full-step configuration names.  All
 // buffers are allocated when the decoder is created; a step only enqueues
 // kernels, so it can be captured once into a HIP graph and replayed.
+#include <map>
 #include <algorithm>
 #include <cmath>
 #include <exception>
@@ -37,14 +38,17 @@ struct fa_decoder {
     fa_buffer *tokens = nullptr, *tables = nullptr, *seq_lens = nullptr, *pos = nullptr, *slots = nullptr;
     fa_buffer *cos_sin = nullptr, *h = nullptr, *xq = nullptr, *sx = nullptr, *q_bf = nullptr;
     fa_buffer *attn = nullptr, *act = nullptr, *pmax = nullptr, *logits = nullptr;
-    fa_graph *graph = nullptr;
-    uint32_t graph_batch = 0;
+    // captured steps, one per batch size seen (a scheduler changes the batch as requests come and go)
+    std::map<uint32_t, fa_graph *> graphs;
     int graph_waves = 0;
     // how the step and the prompt pass pick the next token; rng holds the generator state on the device
     fa_sampling strategy = FA_SAMPLE_GREEDY;
     float temperature = 1.0f;
     uint32_t top_k = 0;
     fa_buffer *rng = nullptr;
+    // per-row sampling table (k::RowPolicy per row) and whether the pick uses it
+    fa_buffer *policy = nullptr;
+    bool per_row = false;
     // host mirror of the installed block tables and of the sequence lengths (advanced with every step and
     // prompt chunk), used to validate that a prompt fits before anything is queued
     std::vector<uint32_t> host_tables, host_lens;
@@ -55,6 +59,11 @@ namespace {
 constexpr uint32_t kDecMagic = 0xFA0DEC01u;
 
 uint64_t round_up(uint64_t v, uint64_t to) { return (v + to - 1) / to * to; }
+
+void drop_graphs(fa_decoder *d) {
+    for (auto &g : d->graphs) fa_graph_destroy(d->ctx, g.second);
+    d->graphs.clear();
+}
 
 fa_status check_dec(const fa_decoder *d) {
     if (!d || d->magic != kDecMagic) return fail(FA_ERR_INVALID_ARGUMENT, "decoder: not a decoder");
@@ -80,7 +89,7 @@ fa_status check_vec(const fa_decoder *d, const fa_buffer *b, uint64_t numel, con
 
 void free_all(fa_context *ctx, fa_decoder *d) {
     fa_buffer **bufs[] = {&d->tokens, &d->tables, &d->seq_lens, &d->pos, &d->slots, &d->cos_sin, &d->h, &d->xq,
-                          &d->sx,     &d->q_bf,     &d->attn, &d->act,  &d->pmax, &d->logits, &d->rng};
+                          &d->sx,     &d->q_bf,     &d->attn, &d->act,  &d->pmax, &d->logits, &d->rng, &d->policy};
     for (auto pb : bufs) {
         if (*pb) fa_buffer_free(ctx, *pb);
         *pb = nullptr;
@@ -94,7 +103,10 @@ void free_all(fa_context *ctx, fa_decoder *d) {
 
 // logits [batch, vocab] -> next tokens, by the decoder's sampling strategy
 void enqueue_pick(fa_decoder *d, hipStream_t s) {
-    if (d->strategy == FA_SAMPLE_GREEDY)
+    if (d->per_row)
+        k::sample_rows_policy((const float *)d->logits->ptr, (int32_t *)d->tokens->ptr, (k::RowPolicy *)d->policy->ptr,
+                              d->batch, d->cfg.vocab, s);
+    else if (d->strategy == FA_SAMPLE_GREEDY)
         k::argmax_rows_f32((const float *)d->logits->ptr, (int32_t *)d->tokens->ptr, d->batch, d->cfg.vocab, s);
     else
         k::sample_rows((const float *)d->logits->ptr, (int32_t *)d->tokens->ptr, (uint64_t *)d->rng->ptr, d->batch,
@@ -211,9 +223,9 @@ struct Temp {
 // that of the decode step (same quantizers, same dequantization, same RoPE and SwiGLU expressions), so
 // a prompt token leaves the same K / V rows in the cache as if it had been decoded.
 struct PrefillBuffers {
-    Temp tok, h, xq, sx, qkv, q_bf, attn, gu, slots, cos_sin, last_rows;
+    Temp tok, h, xq, sx, qkv, q_bf, attn, gu, slots, cos_sin, last_rows, splitk;
     explicit PrefillBuffers(fa_context *c)
-        : tok(c), h(c), xq(c), sx(c), qkv(c), q_bf(c), attn(c), gu(c), slots(c), cos_sin(c), last_rows(c) {}
+        : tok(c), h(c), xq(c), sx(c), qkv(c), q_bf(c), attn(c), gu(c), slots(c), cos_sin(c), last_rows(c), splitk(c) {}
 };
 
 fa_status enqueue_prefill_chunk(fa_context *ctx, fa_decoder *d, PrefillBuffers &t, uint32_t lc, bool last_chunk) {
@@ -254,7 +266,8 @@ fa_status enqueue_prefill_chunk(fa_context *ctx, fa_decoder *d, PrefillBuffers &
         ep.acc_out = nullptr;
         ep.out = out;
         ep.out_bf16 = 0;
-        k::gemm_w8a8_mfma(t.xq.as<int8_t>(), (const int8_t *)w->codes->ptr, M, w->n, w->n_pad, w->k_pad, ep, cus, s);
+        k::gemm_w8a8_mfma(t.xq.as<int8_t>(), (const int8_t *)w->codes->ptr, M, w->n, w->n_pad, w->k_pad, ep, cus, s,
+                          t.splitk.ptr, t.splitk.bytes);
     };
 
     for (uint32_t li = 0; li < c.n_layers; ++li) {
@@ -353,6 +366,7 @@ fa_status fa_decoder_create(fa_context *ctx, const fa_decoder_config *cfg, fa_de
     mk(FA_F32, B * std::max<uint64_t>(F / 16, c.n_heads), &d->pmax);
     mk(FA_F32, B * V, &d->logits);
     mk(FA_U32, 2, &d->rng);
+    mk(FA_U32, 6 * (uint64_t)c.max_batch, &d->policy);
     for (auto &l : d->layers) {
         mk(FA_BF16, layout.num_blocks * layout.block_size * layout.embed_dim, &l.k_pool);
         mk(FA_BF16, layout.num_blocks * layout.block_size * layout.embed_dim, &l.v_pool);
@@ -369,7 +383,7 @@ fa_status fa_decoder_create(fa_context *ctx, const fa_decoder_config *cfg, fa_de
 fa_status fa_decoder_destroy(fa_context *ctx, fa_decoder *d) {
     if (!d) return FA_OK;
     if (fa_status s = check_dec(d)) return s;
-    if (d->graph) fa_graph_destroy(ctx, d->graph);
+    drop_graphs(d);
     free_all(ctx, d);
     d->magic = 0;
     delete d;
@@ -396,10 +410,7 @@ fa_status fa_decoder_set_layer(fa_decoder *d, uint32_t layer, const fa_buffer *a
     L.wo = wo;
     L.wgu = wgu;
     L.wdown = wdown;
-    if (d->graph) {
-        fa_graph_destroy(d->ctx, d->graph);
-        d->graph = nullptr;
-    }
+    drop_graphs(d);
     return FA_OK;
 }
 
@@ -413,10 +424,7 @@ fa_status fa_decoder_set_head(fa_decoder *d, const fa_buffer *embed, const fa_bu
     d->embed = embed;
     d->final_norm = final_norm;
     d->lm_head = lm_head;
-    if (d->graph) {
-        fa_graph_destroy(d->ctx, d->graph);
-        d->graph = nullptr;
-    }
+    drop_graphs(d);
     return FA_OK;
 }
 
@@ -435,11 +443,42 @@ fa_status fa_decoder_set_sampling(fa_context *ctx, fa_decoder *d, fa_sampling st
     d->strategy = strategy;
     d->temperature = temperature;
     d->top_k = (uint32_t)top_k;
-    if (d->graph) {                                     // the captured step holds the old choice
-        fa_graph_destroy(ctx, d->graph);
-        d->graph = nullptr;
-    }
+    d->per_row = false;
+    drop_graphs(d);                                     // the captured steps hold the old choice
     return FA_OK;
+}
+
+static_assert(sizeof(fa_row_sampling) == sizeof(k::RowPolicy) && sizeof(fa_row_sampling) == 24, "row sampling layout");
+
+fa_status fa_decoder_set_row_sampling(fa_context *ctx, fa_decoder *d, const fa_row_sampling *rows) {
+    if (fa_status s = check_ctx(ctx)) return s;
+    if (fa_status s = check_dec(d)) return s;
+    if (d->ctx != ctx) return fail(FA_ERR_DEVICE_MISMATCH, "decoder_set_row_sampling: decoder belongs to another context");
+    if (d->batch == 0) return fail(FA_ERR_INVALID_ARGUMENT, "decoder_set_row_sampling: set the sequences first");
+    if (!rows) return fail(FA_ERR_INVALID_ARGUMENT, "decoder_set_row_sampling: null rows");
+    for (uint32_t b = 0; b < d->batch; ++b) {
+        const fa_row_sampling &r = rows[b];
+        const std::string where = "decoder_set_row_sampling: row " + std::to_string(b);
+        if (r.strategy != FA_SAMPLE_GREEDY && r.strategy != FA_SAMPLE_TEMPERATURE && r.strategy != FA_SAMPLE_TOP_K)
+            return fail(FA_ERR_INVALID_ARGUMENT, where + ": unknown strategy");
+        if (!(std::isfinite(r.temperature) && r.temperature > 0.0f))
+            return fail(FA_ERR_INVALID_ARGUMENT, where + ": temperature must be finite and positive");
+        if (r.strategy == FA_SAMPLE_TOP_K && (r.top_k == 0 || r.top_k > d->cfg.vocab))
+            return fail(FA_ERR_INVALID_ARGUMENT, where + ": top_k must be in 1..=vocab");
+        if (r.strategy != FA_SAMPLE_GREEDY && r.rng_state == 0)
+            return fail(FA_ERR_INVALID_ARGUMENT, where + ": a generator state is never zero (fa_rng_state_from_seed)");
+    }
+    if (fa_status s = fa_upload_into(ctx, rows, (uint64_t)d->batch * 6, d->policy, 0)) return s;
+    if (!d->per_row) drop_graphs(d);                    // the captured steps pick the other way
+    d->per_row = true;
+    return FA_OK;
+}
+
+fa_status fa_decoder_read_row_sampling(fa_context *ctx, fa_decoder *d, fa_row_sampling *rows) {
+    if (fa_status s = check_dec(d)) return s;
+    if (!rows) return fail(FA_ERR_INVALID_ARGUMENT, "decoder_read_row_sampling: null rows");
+    if (!d->per_row) return fail(FA_ERR_INVALID_ARGUMENT, "decoder_read_row_sampling: no per-row table installed");
+    return fa_download(ctx, d->policy, 0, rows, (uint64_t)d->batch * 6);
 }
 
 fa_status fa_decoder_kv_pools(fa_decoder *d, uint32_t layer, fa_buffer **k_pool, fa_buffer **v_pool) {
@@ -508,25 +547,34 @@ fa_status fa_decoder_step(fa_context *ctx, fa_decoder *d, int32_t use_graph) {
     if (fa_status s = ensure_workspace(ctx, k::paged_decode_workspace_bytes(ps, (uint32_t)g_decode_waves))) return s;
     for (auto &len : d->host_lens) len += 1;            // mirrors the device-side advance of this step
     if (!use_graph) return enqueue_step(ctx, d);
-    if (d->graph && (d->graph_batch != d->batch || d->graph_waves != g_decode_waves)) {
-        fa_graph_destroy(ctx, d->graph);
-        d->graph = nullptr;
-    }
-    if (!d->graph) {
-        if (fa_status s = fa_graph_capture_begin(ctx)) return s;
-        fa_status es = enqueue_step(ctx, d);
-        fa_graph *g = nullptr;
-        fa_status cs = fa_graph_capture_end(ctx, &g);
-        if (es != FA_OK) {
-            if (g) fa_graph_destroy(ctx, g);
-            return es;
+    if (d->graph_waves != g_decode_waves) drop_graphs(d);
+    auto it = d->graphs.find(d->batch);
+    if (it == d->graphs.end()) {
+        try {
+            it = d->graphs.emplace(d->batch, nullptr).first;
+        } catch (const std::exception &) {
+            return fail(FA_ERR_ALLOCATION_FAILED, "decoder_step: out of host memory");
         }
-        if (cs != FA_OK) return cs;
-        d->graph = g;
-        d->graph_batch = d->batch;
+        fa_status cs = fa_graph_capture_begin(ctx);
+        fa_graph *g = nullptr;
+        if (cs == FA_OK) {
+            fa_status es = enqueue_step(ctx, d);
+            cs = fa_graph_capture_end(ctx, &g);
+            if (es != FA_OK) {
+                if (g) fa_graph_destroy(ctx, g);
+                g = nullptr;
+                cs = es;
+            }
+        }
+        if (cs != FA_OK || !g) {
+            d->graphs.erase(it);
+            for (auto &len : d->host_lens) len -= 1;    // nothing ran
+            return cs != FA_OK ? cs : fail(FA_ERR_KERNEL_LAUNCH_FAILED, "decoder_step: capture produced no graph");
+        }
+        it->second = g;
         d->graph_waves = g_decode_waves;
     }
-    return fa_graph_launch(ctx, d->graph);
+    return fa_graph_launch(ctx, it->second);
 }
 
 fa_status fa_decoder_prefill(fa_context *ctx, fa_decoder *d, const int32_t *tokens, uint32_t l_new) {
@@ -577,6 +625,15 @@ fa_status fa_decoder_prefill(fa_context *ctx, fa_decoder *d, const int32_t *toke
     get(t.slots, M * 4);
     get(t.cos_sin, M * c.head_dim * 4);
     get(t.last_rows, (uint64_t)B * 4);
+    {
+        // short prompts leave the narrow projections too few tiles to fill the device: room for their k splits
+        uint64_t need = 0;
+        const int cus = ctx->props.multiProcessorCount;
+        for (const auto &l : d->layers)
+            for (const fa_qweight *w : {l.wqkv, l.wo, l.wgu, l.wdown})
+                need = std::max(need, k::gemm_w8a8_workspace_bytes(M, w->n, w->n_pad, w->k_pad, cus));
+        get(t.splitk, need);
+    }
     if (st != FA_OK) return st;
     k::PagedShape ps{};
     ps.batch = B;

@@ -6,6 +6,7 @@
 // are re-ordered into the same tile order on their way into LDS.  Both operand
 // tiles are double-buffered in LDS; every LDS read is a conflict-free 16-byte
 // read at lane * 16.
+#include <algorithm>
 #include <type_traits>
 
 #include "device_utils.hpp"
@@ -17,6 +18,7 @@ using namespace fa::dev;
 
 int g_gemm_small_tiles = 0;   // tuning: nonzero keeps the 128 x 128 kernel for every shape
 int g_gemm_waves = 0;
+int g_gemm_split_fill = 0;    // tuning: blocks per compute unit a split-k launch aims for (default 2)
 int g_gemm_ntb = 0;           // tuning: 14 or 16 fixes the column tiles per large-tile block         // tuning: 4 = four wavefronts per large-tile block instead of eight
 
 namespace {
@@ -48,7 +50,7 @@ struct Cfg {
 template <bool FP8, typename Epi>
 __global__ void __launch_bounds__(256)
     gemm_mfma_kernel(const uint8_t *__restrict__ aq, const uint8_t *__restrict__ w_tiles, uint32_t m, uint32_t n,
-                     uint32_t n_tiles, uint32_t k_tiles, Epi ep) {
+                     uint32_t n_tiles, uint32_t k_tiles, Epi ep, int32_t *__restrict__ partial) {
     using C = Cfg<FP8>;
     constexpr int TK = C::TK, CH = C::CH, TILE = C::TILE;
     constexpr int VPL = CH / 16;                    // 16-byte vectors per lane chunk
@@ -59,6 +61,10 @@ __global__ void __launch_bounds__(256)
     const int wm = wave / 2, wn = wave % 2;
     const uint32_t m0 = blockIdx.y * BM, nt0 = blockIdx.x * NT;
     const uint64_t k_bytes = (uint64_t)k_tiles * TK;
+    // split k: block z of gridDim.z covers k tiles [kt_lo, kt_hi) and leaves raw int32 sums in its own
+    // slice of `partial`; a second kernel adds the slices (exactly) and applies the epilogue
+    const uint32_t kt_lo = (uint32_t)((uint64_t)k_tiles * blockIdx.z / gridDim.z);
+    const uint32_t kt_hi = (uint32_t)((uint64_t)k_tiles * (blockIdx.z + 1) / gridDim.z);
 
     // global -> register staging: A has BM rows x TK bytes = MT*TILE bytes,
     // i.e. MT*64 lane chunks of CH bytes; thread t moves chunks t, t+256, ...
@@ -118,14 +124,14 @@ __global__ void __launch_bounds__(256)
             else acc[i][j] = v4i{0, 0, 0, 0};
         }
 
-    if (k_tiles > 0) {
-        load_stage(0);
+    if (kt_lo < kt_hi) {
+        load_stage(kt_lo);
         store_stage(0);
     }
     __syncthreads();
-    for (uint32_t kt = 0; kt < k_tiles; ++kt) {
-        int buf = kt & 1;
-        if (kt + 1 < k_tiles) load_stage(kt + 1);
+    for (uint32_t kt = kt_lo; kt < kt_hi; ++kt) {
+        int buf = (kt - kt_lo) & 1;
+        if (kt + 1 < kt_hi) load_stage(kt + 1);
         if constexpr (FP8) {
             v8i a[4], b[4];
 #pragma unroll
@@ -150,7 +156,7 @@ __global__ void __launch_bounds__(256)
                 for (int j = 0; j < 4; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[i], b[j], acc[i][j], 0, 0, 0);
         }
-        if (kt + 1 < k_tiles) store_stage(buf ^ 1);   // the other buffer was last read one iteration ago
+        if (kt + 1 < kt_hi) store_stage(buf ^ 1);     // the other buffer was last read one iteration ago
         __syncthreads();
     }
 
@@ -167,6 +173,12 @@ __global__ void __launch_bounds__(256)
                 if (row >= m || col >= n) continue;
                 uint64_t o = (uint64_t)row * n + col;
                 float v;
+                if constexpr (!FP8) {
+                    if (partial) {
+                        partial[(uint64_t)blockIdx.z * m * n + o] = acc[i][j][e];
+                        continue;
+                    }
+                }
                 if constexpr (FP8) {
                     v = __fmul_rn(acc[i][j][e], __fmul_rn(*ep.a_scale, *ep.w_scale));
                 } else {
@@ -180,6 +192,42 @@ __global__ void __launch_bounds__(256)
                 else
                     ((float *)ep.out)[o] = v;
             }
+}
+
+// Second half of a split-k int8 GEMM: adds the `splits` slices of raw sums (int32, exact in any order) and
+// applies the same epilogue arithmetic as the kernel above.  One thread per four consecutive columns.
+__global__ void __launch_bounds__(256)
+    splitk_epilogue_i8_kernel(const int32_t *__restrict__ partial, uint32_t splits, uint32_t m, uint32_t n, EpiI8 ep) {
+    const uint64_t quads_per_row = (n + 3) / 4, total = (uint64_t)m * quads_per_row;
+    for (uint64_t q = (uint64_t)blockIdx.x * 256 + threadIdx.x; q < total; q += (uint64_t)gridDim.x * 256) {
+        const uint32_t row = (uint32_t)(q / quads_per_row), c0 = (uint32_t)(q % quads_per_row) * 4;
+        const uint64_t o0 = (uint64_t)row * n + c0;
+        int32_t acc[4] = {0, 0, 0, 0};
+        const bool vec = (n % 4 == 0);                       // then o0 is a multiple of 4: 16-byte loads
+        for (uint32_t z = 0; z < splits; ++z) {
+            const int32_t *src = partial + (uint64_t)z * m * n + o0;
+            if (vec) {
+                v4i v = *(const v4i *)src;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[e] += v[e];
+            } else {
+                for (int e = 0; e < 4 && c0 + e < n; ++e) acc[e] += src[e];
+            }
+        }
+        const float sx = ep.sx[row];
+        for (int e = 0; e < 4 && c0 + e < n; ++e) {
+            const uint32_t col = c0 + e;
+            const uint64_t o = o0 + e;
+            if (ep.acc_out) ep.acc_out[o] = acc[e];
+            float v = __fmul_rn((float)acc[e], __fmul_rn(sx, ep.sw[col]));
+            if (ep.bias) v = __fadd_rn(v, ep.bias[col]);
+            if (ep.residual) v = __fadd_rn(ep.residual[o], v);
+            if (ep.out_bf16)
+                ((uint16_t *)ep.out)[o] = f32_to_bf16(v);
+            else
+                ((float *)ep.out)[o] = v;
+        }
+    }
 }
 
 // Matrix instructions with the accumulator pinned to the accumulation registers ("+a"): with 256
@@ -537,6 +585,9 @@ inline int pick_big_ntb(uint64_t m, uint64_t n_tiles, int num_cus) {
     if (m < 256 || n_tiles < 14) return 0;
     if (g_gemm_ntb == 14 || g_gemm_ntb == 16) return g_gemm_ntb;
     uint64_t mb = (m + 255) / 256;
+    // a few hundred rows against a narrow weight: too few large tiles to keep the compute units' L2 ports
+    // busy (each pulls operands at a fixed rate), the 128 x 128 kernel spreads the same bytes over more of them
+    if (mb * ((n_tiles + 13) / 14) * 2 <= (uint64_t)num_cus) return 0;
     int best = 0;
     double best_cost = 0;
     for (int ntb : {16, 14}) {
@@ -579,20 +630,58 @@ void launch_big(const uint8_t *aq, const uint8_t *w_tiles, uint64_t m, uint64_t 
 
 }  // namespace
 
+// How an int8 GEMM is launched.  ntb != 0: the large-tile kernel with that many column tiles per block,
+// ntb == 0: the 128 x 128 kernel; splits > 1 (128 x 128 kernel only): k is divided over that many blocks
+// per output tile, which leave int32 partial sums in a workspace that a second kernel adds (exactly) before
+// the epilogue.  A matrix with few output tiles (a prompt of a few hundred rows against a 4096-column
+// weight) occupies only a fraction of the compute units otherwise, and each of them pulls operands at a
+// fixed rate.  (The same split on the large-tile kernel measured no faster.)
+struct W8a8Plan {
+    int ntb;
+    uint32_t splits;
+};
+
+static W8a8Plan plan_w8a8(uint64_t m, uint64_t n_pad, uint64_t k_pad, int num_cus) {
+    const uint64_t n_tiles = n_pad / 16;
+    const uint64_t fill = (uint64_t)num_cus * (g_gemm_split_fill > 0 ? g_gemm_split_fill : 2);
+    const bool big_ok = !(g_gemm_small_tiles || k_pad % 128 || k_pad == 0) && n_tiles >= 14;
+    if (big_ok && m >= 256) {
+        if (int ntb = pick_big_ntb(m, n_tiles, num_cus)) return {ntb, 1};
+    }
+    const uint64_t blocks = ((n_tiles + NT - 1) / NT) * ((m + BM - 1) / BM);
+    if (blocks == 0 || blocks * 2 > fill) return {0, 1};
+    uint64_t s = std::min<uint64_t>(std::min<uint64_t>(16, fill / blocks), (k_pad / 64) / 4);
+    return {0, (uint32_t)std::max<uint64_t>(s, 1)};
+}
+
+uint64_t gemm_w8a8_workspace_bytes(uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad, int num_cus) {
+    const W8a8Plan p = plan_w8a8(m, n_pad, k_pad, num_cus);
+    return p.splits > 1 ? (uint64_t)p.splits * m * n * 4 : 0;
+}
+
 void gemm_w8a8_mfma(const int8_t *aq, const int8_t *w_tiles, uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad,
-                    const EpilogueI8 &ep, int num_cus, hipStream_t s) {
+                    const EpilogueI8 &ep, int num_cus, hipStream_t s, void *workspace, uint64_t workspace_bytes) {
     if (m == 0 || n == 0) return;
     EpiI8 e{ep.sx, ep.sw, ep.bias, ep.residual, ep.acc_out, ep.out, ep.out_bf16};
-    if (int ntb = (g_gemm_small_tiles || k_pad % 128 || k_pad == 0) ? 0 : pick_big_ntb(m, n_pad / 16, num_cus)) {
-        if (ntb == 16)
-            launch_big<false, 16, EpiI8>((const uint8_t *)aq, (const uint8_t *)w_tiles, m, n, n_pad / 16, k_pad / 128, e, s);
-        else
-            launch_big<false, 14, EpiI8>((const uint8_t *)aq, (const uint8_t *)w_tiles, m, n, n_pad / 16, k_pad / 128, e, s);
-        return;
+    W8a8Plan p = plan_w8a8(m, n_pad, k_pad, num_cus);
+    if (p.splits > 1 && (!workspace || workspace_bytes < (uint64_t)p.splits * m * n * 4))
+        p.splits = 1;                                 // no room for partial sums: one block per tile
+    int32_t *partial = p.splits > 1 ? (int32_t *)workspace : nullptr;
+    if (p.ntb == 16) {
+        launch_big<false, 16, EpiI8>((const uint8_t *)aq, (const uint8_t *)w_tiles, m, n, n_pad / 16, k_pad / 128, e, s);
+    } else if (p.ntb) {
+        launch_big<false, 14, EpiI8>((const uint8_t *)aq, (const uint8_t *)w_tiles, m, n, n_pad / 16, k_pad / 128, e, s);
+    } else {
+        dim3 grid((unsigned)((n_pad / 16 + NT - 1) / NT), (unsigned)((m + BM - 1) / BM), p.splits);
+        gemm_mfma_kernel<false, EpiI8><<<grid, 256, 0, s>>>((const uint8_t *)aq, (const uint8_t *)w_tiles, (uint32_t)m,
+                                                            (uint32_t)n, (uint32_t)(n_pad / 16), (uint32_t)(k_pad / 64), e,
+                                                            partial);
     }
-    dim3 grid((unsigned)((n_pad / 16 + NT - 1) / NT), (unsigned)((m + BM - 1) / BM));
-    gemm_mfma_kernel<false, EpiI8><<<grid, 256, 0, s>>>((const uint8_t *)aq, (const uint8_t *)w_tiles, (uint32_t)m,
-                                                        (uint32_t)n, (uint32_t)(n_pad / 16), (uint32_t)(k_pad / 64), e);
+    if (p.splits > 1) {
+        const uint64_t quads = m * ((n + 3) / 4);
+        const unsigned blocks = (unsigned)std::min<uint64_t>((quads + 255) / 256, (uint64_t)num_cus * 8);
+        splitk_epilogue_i8_kernel<<<blocks, 256, 0, s>>>((const int32_t *)workspace, p.splits, (uint32_t)m, (uint32_t)n, e);
+    }
 }
 
 void gemm_e4m3_mfma(const uint8_t *aq, const uint8_t *w_tiles, const float *a_scale, const float *w_scale, uint64_t m,
@@ -608,7 +697,7 @@ void gemm_e4m3_mfma(const uint8_t *aq, const uint8_t *w_tiles, const float *a_sc
     }
     dim3 grid((unsigned)((n_pad / 16 + NT - 1) / NT), (unsigned)((m + BM - 1) / BM));
     gemm_mfma_kernel<true, EpiF8><<<grid, 256, 0, s>>>(aq, w_tiles, (uint32_t)m, (uint32_t)n, (uint32_t)(n_pad / 16),
-                                                       (uint32_t)(k_pad / 128), e);
+                                                       (uint32_t)(k_pad / 128), e, nullptr);
 }
 
 }  // namespace k

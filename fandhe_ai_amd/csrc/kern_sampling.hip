@@ -5,6 +5,9 @@
 // cumulative weight exceeds u * total, u the next 53-bit uniform of an xorshift64* generator whose state
 // lives on the device; rows draw in row order from the one generator.  Only the order of the f64 sums
 // differs from the host loop (a block-wide tree instead of a sequential pass).
+// With a policy table every row has a strategy, temperature, k and generator of its own (one request per
+// row, each drawing from the generator its own seed started: crates/autodiff/src/generate/scheduler.rs:
+// 176-211, 553-562); a greedy row takes the first maximum and draws nothing.
 #include "device_utils.hpp"
 #include "kernels.hpp"
 
@@ -51,7 +54,7 @@ __device__ __forceinline__ T block_exclusive_scan(T v, T *buf, T *total) {
 
 __global__ void __launch_bounds__(kThreads)
     sample_rows_kernel(const float *__restrict__ logits, int32_t *__restrict__ tokens, const uint64_t *__restrict__ rng_state,
-                       uint32_t vocab, int top_k_mode, float temperature, uint32_t top_k) {
+                       RowPolicy *__restrict__ policy, uint32_t vocab, int top_k_mode, float temperature, uint32_t top_k) {
     __shared__ double s_d[kThreads];
     __shared__ uint32_t s_u[kThreads];
     __shared__ uint32_t hist[256];
@@ -60,6 +63,14 @@ __global__ void __launch_bounds__(kThreads)
     __shared__ double s_x;
     const uint32_t b = blockIdx.x, t = threadIdx.x;
     const float *row = logits + (uint64_t)b * vocab;
+    bool greedy = false;
+    if (policy) {                                        // uniform over the block
+        const RowPolicy pr = policy[b];
+        greedy = pr.strategy == 0;
+        top_k_mode = pr.strategy == 2;
+        temperature = pr.temperature;
+        top_k = pr.top_k < vocab ? pr.top_k : vocab;
+    }
     const uint32_t seg = (vocab + kThreads - 1) / kThreads;
     const uint32_t lo = t * seg < vocab ? t * seg : vocab, hi = lo + seg < vocab ? lo + seg : vocab;
 
@@ -83,6 +94,18 @@ __global__ void __launch_bounds__(kThreads)
     }
     mx = s_max[0];
     for (int w = 1; w < kThreads / 64; ++w) mx = fmaxf(mx, s_max[w]);
+    if (greedy) {                                        // first index holding the maximum
+        if (t == 0) s_sel[0] = 0xffffffffu;
+        __syncthreads();
+        for (uint32_t i = lo; i < hi; ++i)
+            if (row[i] == mx) {
+                atomicMin(&s_sel[0], i);
+                break;
+            }
+        __syncthreads();
+        if (t == 0) tokens[b] = (int32_t)s_sel[0];
+        return;
+    }
     const double dmax = (double)mx, dt = (double)temperature;
 
     // ---- top-k: key of the k-th largest value and how many elements with that key are kept (lowest indices)
@@ -163,9 +186,15 @@ __global__ void __launch_bounds__(kThreads)
     double total;
     const double before = block_exclusive_scan<double>(wsum, s_d, &total);
     if (t == 0) {
-        uint64_t st = rng_state[0];
         uint64_t bits = 0;
-        for (uint32_t r = 0; r <= b; ++r) bits = xorshift64star_next(st);     // row b takes the (b + 1)-th draw of the step
+        if (policy) {                            // the row's own generator: one draw, state kept for the next step
+            uint64_t st = policy[b].rng_state;
+            bits = xorshift64star_next(st);
+            policy[b].rng_state = st;
+        } else {
+            uint64_t st = rng_state[0];
+            for (uint32_t r = 0; r <= b; ++r) bits = xorshift64star_next(st);     // row b takes the (b + 1)-th draw of the step
+        }
         s_x = (double)(bits >> 11) / 9007199254740992.0 * total;
         s_sel[0] = 0xffffffffu;                 // first index whose cumulative weight exceeds x
         s_sel[1] = 0;                           // last index with a positive weight (+ 1)
@@ -206,8 +235,13 @@ __global__ void advance_rng_kernel(uint64_t *state, uint32_t draws) {
 void sample_rows(const float *logits, int32_t *tokens, uint64_t *rng_state, uint32_t rows, uint32_t vocab, int top_k_mode,
                  float temperature, uint32_t top_k, hipStream_t s) {
     if (rows == 0 || vocab == 0) return;
-    sample_rows_kernel<<<rows, kThreads, 0, s>>>(logits, tokens, rng_state, vocab, top_k_mode, temperature, top_k);
+    sample_rows_kernel<<<rows, kThreads, 0, s>>>(logits, tokens, rng_state, nullptr, vocab, top_k_mode, temperature, top_k);
     advance_rng_kernel<<<1, 1, 0, s>>>(rng_state, rows);
+}
+
+void sample_rows_policy(const float *logits, int32_t *tokens, RowPolicy *policy, uint32_t rows, uint32_t vocab, hipStream_t s) {
+    if (rows == 0 || vocab == 0) return;
+    sample_rows_kernel<<<rows, kThreads, 0, s>>>(logits, tokens, nullptr, policy, vocab, 0, 1.0f, 0);
 }
 
 }  // namespace k

@@ -121,9 +121,13 @@ void linear_w8a16_skinny(const uint16_t *a, const int8_t *w_tiles, const float *
                          int num_cus, hipStream_t s);
 
 // ---- prefill-shape MFMA GEMMs (kern_gemm_mfma.hip) -----------------------------
-// aq: int8 [m, k_pad] row-major.
+// aq: int8 [m, k_pad] row-major.  workspace (optional, gemm_w8a8_workspace_bytes): lets a matrix with too few
+// output tiles to occupy the device split k across blocks; the int32 partial sums meet there and are
+// added exactly, so the result does not depend on the split.
 void gemm_w8a8_mfma(const int8_t *aq, const int8_t *w_tiles, uint64_t m, uint64_t n, uint64_t n_pad,
-                    uint64_t k_pad, const EpilogueI8 &ep, int num_cus, hipStream_t s);
+                    uint64_t k_pad, const EpilogueI8 &ep, int num_cus, hipStream_t s, void *workspace = nullptr,
+                    uint64_t workspace_bytes = 0);
+uint64_t gemm_w8a8_workspace_bytes(uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad, int num_cus);
 // aq: e4m3 [m, k_pad] row-major; scales are device scalars.
 void gemm_e4m3_mfma(const uint8_t *aq, const uint8_t *w_tiles, const float *a_scale,
                     const float *w_scale, uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad,
@@ -170,11 +174,22 @@ void paged_attention_prefill_bf16(const uint16_t *q, const uint16_t *k_pool, con
                                   uint32_t waves_per_cu, void *workspace, void *out, int out_bf16, hipStream_t s);
 
 // ---- sampling (kern_sampling.hip) ------------------------------------------------
+// one row of a per-row sampling table (the layout of fa_row_sampling)
+struct RowPolicy {
+    uint64_t rng_state;
+    float temperature;
+    uint32_t top_k;
+    int32_t strategy;
+    uint32_t reserved;
+};
 // One token per row of logits [rows, vocab] by temperature (top_k_mode 0) or top-k (1) sampling with the
 // reference's arithmetic; row b takes the (b + 1)-th draw of the xorshift64* generator at rng_state, which is
 // advanced by `rows` draws afterwards.  A row with a non-finite logit gets token -1.
 void sample_rows(const float *logits, int32_t *tokens, uint64_t *rng_state, uint32_t rows, uint32_t vocab, int top_k_mode,
                  float temperature, uint32_t top_k, hipStream_t s);
+// The same with one RowPolicy per row (strategy 0 takes the first maximum and draws nothing; otherwise one
+// draw from the row's own state, which is advanced in place).
+void sample_rows_policy(const float *logits, int32_t *tokens, RowPolicy *policy, uint32_t rows, uint32_t vocab, hipStream_t s);
 
 // ---- measurement aid (kern_probe.hip) -------------------------------------------
 // Launches a register-only loop of one matrix instruction kind (0: i32_16x16x64_i8, 1: i32_32x32x32_i8,

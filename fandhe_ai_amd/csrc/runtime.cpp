@@ -236,14 +236,21 @@ fa_status ensure_workspace(fa_context *ctx, uint64_t bytes) {
     if (ctx->workspace_bytes >= bytes) return FA_OK;
     if (ctx->capturing)
         return fail(FA_ERR_CAPTURE_IN_PROGRESS, "workspace must be sized before graph capture");
-    uint64_t want = std::max<uint64_t>(bytes, 1ull << 20);
+    uint64_t want = std::max<uint64_t>(std::max<uint64_t>(bytes, 2 * ctx->workspace_bytes), 1ull << 20);
+    if (ctx->workspace) {
+        try {
+            ctx->retired_workspaces.reserve(ctx->retired_workspaces.size() + 1);
+        } catch (const std::exception &) {
+            return fail(FA_ERR_ALLOCATION_FAILED, "workspace: out of host memory");
+        }
+    }
     void *p = nullptr;
     hipError_t e = hipMalloc(&p, want);
     if (e != hipSuccess) {
         (void)hipGetLastError();
         return hip_fail(ctx, e, "hipMalloc(workspace)", FA_ERR_ALLOCATION_FAILED);
     }
-    if (ctx->workspace) (void)hipFree(ctx->workspace);   // waits for queued work
+    if (ctx->workspace) ctx->retired_workspaces.push_back(ctx->workspace);   // a captured graph may replay with it
     ctx->workspace = p;
     ctx->workspace_bytes = want;
     return FA_OK;
@@ -361,6 +368,7 @@ fa_status fa_context_destroy(fa_context *ctx) {
     while (ctx->pool.take_one_for_release(&ent)) (void)hipFree(ent.second);
     if (ctx->table_stage) (void)hipFree(ctx->table_stage);
     if (ctx->workspace) (void)hipFree(ctx->workspace);
+    for (void *w : ctx->retired_workspaces) (void)hipFree(w);
     (void)hipStreamDestroy(ctx->stream);
     (void)hipGetLastError();
     ctx->magic = 0;

@@ -72,6 +72,9 @@ struct fa_context {
     // scratch for split-KV attention partials and similar kernel workspaces
     void *workspace;
     uint64_t workspace_bytes;
+    // workspaces that were outgrown: captured graphs may still hold their addresses, so they stay
+    // allocated until the context is destroyed (growth is geometric, the total stays below twice the last)
+    std::vector<void *> retired_workspaces;
 };
 
 struct fa_buffer {

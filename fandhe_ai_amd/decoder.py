@@ -22,7 +22,17 @@ class Decoder:
         self._keep = []                                   # weights must outlive the decoder that points at them
         self.batch = 0
 
+    @classmethod
+    def from_handle(cls, ops, handle, cfg):
+        """Wraps an fa_decoder created elsewhere (not destroyed by ``close``)."""
+        d = cls.__new__(cls)
+        d._ops, d._h, d.cfg, d._keep, d.batch, d._borrowed = ops, handle, cfg, [], 0, True
+        return d
+
     def close(self):
+        if getattr(self, "_borrowed", False):
+            self._h = None
+            return
         h, self._h = getattr(self, "_h", None), None
         if h and self._ops._ctx:
             lib.fa_decoder_destroy(self._ops._ctx, h)
@@ -54,6 +64,17 @@ class Decoder:
 
     def set_sampling(self, strategy, temperature=1.0, top_k=0, seed=0):
         check(lib.fa_decoder_set_sampling(self._ops._ctx, self._h, strategy, temperature, top_k, seed))
+
+    def set_row_sampling(self, rows):
+        """rows: a ctypes array of ``capi.RowSampling``, one per installed sequence."""
+        if len(rows) != self.batch:
+            raise ValueError("one sampling record per installed sequence")
+        check(lib.fa_decoder_set_row_sampling(self._ops._ctx, self._h, rows))
+
+    def read_row_sampling(self):
+        rows = (capi.RowSampling * self.batch)()
+        check(lib.fa_decoder_read_row_sampling(self._ops._ctx, self._h, rows))
+        return rows
 
     def prefill(self, prompt):
         """prompt: int32 [batch, l_new]; leaves the next tokens resident like a step."""

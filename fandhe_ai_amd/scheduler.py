@@ -1,0 +1,423 @@
+"""Autoregressive generation and continuous batching on the resident decoder.
+
+Host-side mirror of the reference's generation layer (crates/autodiff/src/generate/mod.rs:101-215 config and
+validation, :500-640 ``generate``; crates/autodiff/src/generate/scheduler.rs:75-127 limits, :445-508 ``submit``,
+:521-562 admission, :571-590 ``step``, :712-720 ``take_*``) for a model whose state lives on the device: the KV
+pages of all requests share the decoder's pools, every request owns a block-table row, a sampling record with
+its own generator (seeded from its config, one draw per generated token) and its token list.  One ``step``
+admits queued requests while rows and pages are free, ingests the prompt of every newly admitted request
+(batch 1, the whole prompt in one pass) and advances all other active requests together by one decode step of
+the batch they currently form; requests finish when they reach ``max_length`` (there is no end-of-sequence
+stop, as in the reference) and leave the batch between steps.
+
+What differs from the reference, by construction: the decode step is batched on the device (the reference's
+opt-in ``step_batched``), so a request's tokens equal a stand-alone ``generate`` of the same request only as
+far as its logits are decisive (the attention reduction is split differently when the batch changes); a
+request that runs alone is identical to ``generate``.  Pages for the whole ``max_length`` are reserved at
+admission, so a request that is admitted can always finish; a request that needs more pages than are free
+waits at the head of the queue.
+"""
+import math
+from collections import deque
+
+import numpy as np
+
+from . import capi
+from .backend import SAMPLE_GREEDY as GREEDY
+from .backend import SAMPLE_TEMPERATURE as TEMPERATURE
+from .backend import SAMPLE_TOP_K as TOP_K
+from .backend import BackendError, check
+
+lib = capi.lib
+
+
+class InvalidArgument(ValueError):
+    """AutodiffError::InvalidArgument"""
+
+
+class RankMismatch(ValueError):
+    """AutodiffError::Shape(ShapeError::RankMismatch)"""
+
+
+class SamplingStrategy:
+    """``SamplingStrategy::{Greedy, TopK(k), Temperature(t)}`` (generate/mod.rs:101-113)."""
+
+    def __init__(self, kind, value=None):
+        self.kind, self.value = kind, value
+
+    @classmethod
+    def Greedy(cls):
+        return cls(GREEDY)
+
+    @classmethod
+    def TopK(cls, k):
+        return cls(TOP_K, k)
+
+    @classmethod
+    def Temperature(cls, t):
+        return cls(TEMPERATURE, t)
+
+    def __eq__(self, other):
+        return isinstance(other, SamplingStrategy) and (self.kind, self.value) == (other.kind, other.value)
+
+    def __repr__(self):
+        return {GREEDY: "Greedy", TOP_K: "TopK(%r)" % (self.value,), TEMPERATURE: "Temperature(%r)" % (self.value,)}[self.kind]
+
+
+class GenerateConfig:
+    """``GenerateConfig`` (generate/mod.rs:124-168): ``max_length`` counts the prompt; ``temperature`` and
+    ``top_k`` are derived from the strategy and may only be changed where the strategy allows it."""
+
+    def __init__(self, max_length, strategy, seed=0):
+        self.max_length, self.strategy, self.seed = max_length, strategy, seed
+        self.temperature = float(strategy.value) if strategy.kind == TEMPERATURE else 1.0
+        self.top_k = strategy.value if strategy.kind == TOP_K else None
+
+    new = classmethod(lambda cls, max_length, strategy: cls(max_length, strategy))
+
+    def with_temperature(self, temperature):
+        self.temperature = temperature
+        return self
+
+    def with_seed(self, seed):
+        self.seed = seed
+        return self
+
+    def clone(self):
+        c = GenerateConfig(self.max_length, SamplingStrategy(self.strategy.kind, self.strategy.value), self.seed)
+        c.temperature, c.top_k = self.temperature, self.top_k
+        return c
+
+    def validate(self):
+        """generate/mod.rs:170-229: contradictory or non-finite settings are rejected, never repaired."""
+        t = self.temperature
+        if not (isinstance(t, (int, float)) and math.isfinite(t) and t > 0):
+            raise InvalidArgument("GenerateConfig: temperature must be finite and positive (got %r)" % (t,))
+        s = self.strategy
+        if s.kind == GREEDY:
+            if t != 1.0 or self.top_k is not None:
+                raise InvalidArgument("GenerateConfig: Greedy requires temperature == 1.0 and top_k == None")
+        elif s.kind == TOP_K:
+            if self.top_k != s.value:
+                raise InvalidArgument("GenerateConfig: TopK(%r) requires top_k == %r" % (s.value, s.value))
+            if not isinstance(s.value, int) or s.value < 1:
+                raise InvalidArgument("GenerateConfig: TopK needs k >= 1")
+        elif s.kind == TEMPERATURE:
+            if self.top_k is not None:
+                raise InvalidArgument("GenerateConfig: Temperature requires top_k == None")
+            if t != s.value:
+                raise InvalidArgument("GenerateConfig: Temperature(%r) requires temperature == %r" % (s.value, s.value))
+        else:
+            raise InvalidArgument("GenerateConfig: unknown strategy")
+        if not (isinstance(self.seed, int) and 0 <= self.seed < 1 << 64):
+            raise InvalidArgument("GenerateConfig: seed must be a u64")
+
+    def validate_top_k_le_vocab(self, vocab):
+        """generate/mod.rs:236-248: k beyond the vocabulary is an error, not clamped."""
+        if self.strategy.kind == TOP_K and self.strategy.value > vocab:
+            raise InvalidArgument("GenerateConfig: TopK k (%d) exceeds vocab_size (%d)" % (self.strategy.value, vocab))
+
+
+_I32_BYTES_MAX = (1 << 63) - 1
+
+
+def _check_buffer_bytes(elems):
+    if elems * 4 > _I32_BYTES_MAX:
+        raise InvalidArgument("output of %d i32 elements exceeds the allocation limit" % elems)
+
+
+def _prompt_shape(input_ids, what):
+    ids = np.asarray(input_ids)
+    if ids.ndim == 1:
+        return ids.reshape(1, -1), 1, ids.shape[0], True
+    if ids.ndim == 2:
+        return ids, ids.shape[0], ids.shape[1], False
+    raise RankMismatch("%s: input_ids must be [T] or [B, T] (rank %d)" % (what, ids.ndim))
+
+
+def _pages_for(max_length, block_size):
+    # positions 0 .. max_length - 2 are written (the last generated token is never fed back)
+    return max(1, -(-(max_length - 1) // block_size))
+
+
+def generate(decoder, input_ids, config):
+    """``generate`` (generate/mod.rs:500-640) on a resident decoder: prompt pass, then one decode step per
+    token until every row holds ``max_length`` tokens.  input_ids [T] or [B, T] int32; returns an int32 array
+    of the same rank.  The B rows draw in row order from the one generator ``config.seed`` starts.  Uses
+    pages 0 .. of the decoder's pools and replaces whatever sequences were installed."""
+    config.validate()
+    ids, b, prompt_len, want_rank1 = _prompt_shape(input_ids, "generate")
+    if prompt_len == 0:
+        raise InvalidArgument("generate: the prompt is empty")
+    if b == 0:
+        raise InvalidArgument("generate: the batch is empty")
+    if config.max_length < prompt_len:
+        raise InvalidArgument("generate: max_length (%d) must be at least the prompt length (%d)" % (config.max_length, prompt_len))
+    _check_buffer_bytes(b * config.max_length)
+    if config.max_length == prompt_len:                    # nothing to generate, no forward pass
+        out = np.array(ids, dtype=np.int32)
+        return out[0] if want_rank1 else out
+    cfg = decoder.cfg
+    pages = _pages_for(config.max_length, cfg.block_size)
+    if b > cfg.max_batch or pages > cfg.max_blocks_per_seq or b * pages > cfg.num_blocks:
+        raise InvalidArgument("generate: %d rows of %d tokens do not fit the decoder's batch or page pool" % (b, config.max_length))
+    config.validate_top_k_le_vocab(cfg.vocab)
+    out = np.empty((b, config.max_length), dtype=np.int32)
+    out[:, :prompt_len] = ids
+    tables = np.full((b, cfg.max_blocks_per_seq), 0xFFFFFFFF, dtype=np.uint32)
+    tables[:, :pages] = np.arange(b * pages, dtype=np.uint32).reshape(b, pages)
+    decoder.set_sequences(tables, np.zeros(b, np.uint32))
+    decoder.set_sampling(config.strategy.kind, config.temperature, config.top_k or 0, config.seed)
+    decoder.prefill(ids.astype(np.int32))
+    for pos in range(prompt_len, config.max_length):
+        if pos > prompt_len:
+            decoder.step()
+        tok = decoder.tokens()
+        if (tok < 0).any():
+            raise InvalidArgument("generate: logits hold non-finite values")
+        out[:, pos] = tok
+    return out[0] if want_rank1 else out
+
+
+class SchedulerLimits:
+    """scheduler.rs:80-127: every limit is mandatory and at least 1."""
+
+    def __init__(self, max_active, max_queued, max_length):
+        if min(max_active, max_queued, max_length) < 1:
+            raise InvalidArgument("SchedulerLimits: every limit must be at least 1 (max_active=%d, max_queued=%d, max_length=%d)"
+                                  % (max_active, max_queued, max_length))
+        _check_buffer_bytes(max_length)
+        self.max_active, self.max_queued, self.max_length = max_active, max_queued, max_length
+
+
+class PageAllocator:
+    """Page ids of the shared pools: pages that were returned are handed out again last-in first-out, then
+    ids never used before in ascending order (the allocation order of the reference's block table,
+    crates/autodiff/src/nn/paged_kv.rs:147-191)."""
+
+    def __init__(self, num_blocks):
+        self.num_blocks, self._next, self._returned = num_blocks, 0, []
+
+    def free_pages(self):
+        return len(self._returned) + self.num_blocks - self._next
+
+    def take(self, n):
+        if n > self.free_pages():
+            raise InvalidArgument("page pool exhausted")
+        out = []
+        for _ in range(n):
+            if self._returned:
+                out.append(self._returned.pop())
+            else:
+                out.append(self._next)
+                self._next += 1
+        return out
+
+    def give_back(self, pages):
+        self._returned.extend(pages)
+
+
+class _Pending:
+    __slots__ = ("id", "prompt", "config", "want_rank1")
+
+    def __init__(self, rid, prompt, config, want_rank1):
+        self.id, self.prompt, self.config, self.want_rank1 = rid, prompt, config, want_rank1
+
+
+class _Active:
+    __slots__ = ("id", "tokens", "pages", "policy", "config", "want_rank1", "fresh")
+
+
+class BatchScheduler:
+    """``BatchScheduler`` (scheduler.rs:395-720) over a resident ``Decoder``."""
+
+    def __init__(self, decoder, limits):
+        cfg = decoder.cfg
+        if limits.max_active > cfg.max_batch:
+            raise InvalidArgument("scheduler: max_active (%d) exceeds the decoder's max_batch (%d)" % (limits.max_active, cfg.max_batch))
+        self._dec, self.limits = decoder, limits
+        self._queue, self._active, self._finished, self._failed = deque(), [], [], []
+        self._next_id = 0
+        self._pages = PageAllocator(cfg.num_blocks)
+        self._resident = None                              # ids whose decode state is installed on the device, in row order
+
+    def queued_len(self):
+        return len(self._queue)
+
+    def active_len(self):
+        return len(self._active)
+
+    def free_pages(self):
+        return self._pages.free_pages()
+
+    def submit(self, input_ids, config):
+        """Queues a request without touching the device; checks in the reference's order (config, rank, empty
+        prompt, batch of one, max_length against the prompt and the limit, queue room); on any error the
+        scheduler is unchanged.  Returns the request id (ascending)."""
+        config.validate()
+        ids, b, prompt_len, want_rank1 = _prompt_shape(input_ids, "scheduler")
+        if prompt_len == 0:
+            raise InvalidArgument("scheduler: the prompt is empty")
+        if b != 1:
+            raise InvalidArgument("scheduler: one sequence per request (got %d)" % b)
+        if config.max_length < prompt_len:
+            raise InvalidArgument("scheduler: max_length (%d) must be at least the prompt length (%d)" % (config.max_length, prompt_len))
+        if config.max_length > self.limits.max_length:
+            raise InvalidArgument("scheduler: max_length (%d) exceeds the limit (%d)" % (config.max_length, self.limits.max_length))
+        _check_buffer_bytes(config.max_length)
+        if len(self._queue) >= self.limits.max_queued:
+            raise InvalidArgument("scheduler: the queue is full (%d)" % self.limits.max_queued)
+        rid = self._next_id
+        self._next_id += 1
+        self._queue.append(_Pending(rid, [int(t) for t in ids[0]], config.clone(), want_rank1))
+        return rid
+
+    # ---- one iteration ------------------------------------------------------------------------------------
+
+    def step(self):
+        """Admits, ingests new prompts, advances everyone else by one token.  Returns how many requests
+        finished successfully in this call; failures of single requests go to ``take_failed``."""
+        completed = self._admit()
+        n_fin, n_fail = len(self._finished), len(self._failed)
+        fresh = [a for a in self._active if a.fresh]
+        old = [a for a in self._active if not a.fresh]
+        gone = set()
+        if fresh:
+            self._pull_resident_state()                    # the prompt passes overwrite the installed batch
+            for a in fresh:
+                try:
+                    self._ingest(a)
+                except (BackendError, InvalidArgument) as e:
+                    self._fail(a, e, gone)
+                    continue
+                completed += self._maybe_finish(a, gone)
+        if old:
+            try:
+                if self._resident != [a.id for a in old]:
+                    self._install(old)
+                self._dec.step()
+                picked = self._dec.tokens()
+            except BackendError as e:                      # a device failure takes the whole batch with it
+                for a in old:
+                    self._fail(a, e, gone)
+                self._resident = None
+            else:
+                for a, tok in zip(old, picked):
+                    if tok < 0:
+                        self._fail(a, InvalidArgument("generate: logits hold non-finite values"), gone)
+                        continue
+                    a.tokens.append(int(tok))
+                    completed += self._maybe_finish(a, gone)
+        if gone:
+            self._pull_resident_state(skip=gone)           # the rows move: keep the survivors' generator states
+            self._active = [a for a in self._active if a.id not in gone]
+        # within one iteration requests are reported in request order, as if they had been advanced one by one
+        self._finished[n_fin:] = sorted(self._finished[n_fin:], key=lambda e: e[0])
+        self._failed[n_fail:] = sorted(self._failed[n_fail:], key=lambda e: e[0])
+        return completed
+
+    def take_finished(self):
+        """[(request id, int32 tokens [max_length] or [1, max_length])] in completion order; drains."""
+        out, self._finished = self._finished, []
+        return out
+
+    def take_failed(self):
+        """[(request id, exception)]; drains."""
+        out, self._failed = self._failed, []
+        return out
+
+    # ---- internals ----------------------------------------------------------------------------------------
+
+    def _admit(self):
+        cfg, completed = self._dec.cfg, 0
+        while len(self._active) < self.limits.max_active and self._queue:
+            p = self._queue[0]
+            if p.config.max_length == len(p.prompt):       # nothing to generate: the prompt is the answer
+                self._queue.popleft()
+                self._finished.append((p.id, self._output(p.prompt, p.want_rank1)))
+                completed += 1
+                continue
+            need = _pages_for(p.config.max_length, cfg.block_size)
+            try:
+                p.config.validate_top_k_le_vocab(cfg.vocab)
+                if need > cfg.max_blocks_per_seq or need > cfg.num_blocks:
+                    raise InvalidArgument("scheduler: max_length (%d) needs %d pages, the decoder holds %d per sequence, %d in all"
+                                          % (p.config.max_length, need, cfg.max_blocks_per_seq, cfg.num_blocks))
+                if any(t < 0 or t >= cfg.vocab for t in p.prompt):
+                    raise InvalidArgument("scheduler: prompt token outside the vocabulary")
+            except InvalidArgument as e:
+                self._queue.popleft()
+                self._failed.append((p.id, e))
+                continue
+            if need > self._pages.free_pages():
+                break                                      # waits for pages, in order
+            self._queue.popleft()
+            a = _Active()
+            a.id, a.tokens, a.config, a.want_rank1, a.fresh = p.id, list(p.prompt), p.config, p.want_rank1, True
+            a.pages = self._pages.take(need)
+            state = capi.u64()
+            check(lib.fa_rng_state_from_seed(p.config.seed, state))
+            a.policy = (state.value, float(p.config.temperature), int(p.config.top_k or 0), int(p.config.strategy.kind))
+            self._active.append(a)
+        return completed
+
+    def _table_row(self, a):
+        row = np.full(self._dec.cfg.max_blocks_per_seq, 0xFFFFFFFF, dtype=np.uint32)
+        row[:len(a.pages)] = a.pages
+        return row
+
+    def _policy_rows(self, rows):
+        arr = (capi.RowSampling * len(rows))()
+        for r, a in zip(arr, rows):
+            r.rng_state, r.temperature, r.top_k, r.strategy = a.policy
+        return arr
+
+    def _install(self, rows):
+        self._pull_resident_state()
+        self._dec.set_sequences(np.stack([self._table_row(a) for a in rows]),
+                                np.array([len(a.tokens) - 1 for a in rows], dtype=np.uint32))
+        self._dec.set_tokens(np.array([a.tokens[-1] for a in rows], dtype=np.int32))
+        self._dec.set_row_sampling(self._policy_rows(rows))
+        self._resident = [a.id for a in rows]
+
+    def _pull_resident_state(self, skip=()):
+        """Generator states advance on the device; fetch them before the installed batch is replaced."""
+        if self._resident is None:
+            return
+        by_id = {a.id: a for a in self._active}
+        rows = self._dec.read_row_sampling()
+        for rid, r in zip(self._resident, rows):
+            a = by_id.get(rid)
+            if a is not None and rid not in skip:
+                a.policy = (r.rng_state, r.temperature, r.top_k, r.strategy)
+        self._resident = None
+
+    def _ingest(self, a):
+        self._dec.set_sequences(self._table_row(a)[None, :], np.zeros(1, np.uint32))
+        self._dec.set_row_sampling(self._policy_rows([a]))
+        self._dec.prefill(np.array([a.tokens], dtype=np.int32))
+        tok = int(self._dec.tokens()[0])
+        r = self._dec.read_row_sampling()[0]
+        a.policy = (r.rng_state, r.temperature, r.top_k, r.strategy)
+        a.fresh = False
+        if tok < 0:
+            raise InvalidArgument("generate: logits hold non-finite values")
+        a.tokens.append(tok)
+
+    def _maybe_finish(self, a, gone):
+        if len(a.tokens) < a.config.max_length:
+            return 0
+        self._finished.append((a.id, self._output(a.tokens, a.want_rank1)))
+        self._pages.give_back(a.pages)
+        gone.add(a.id)
+        return 1
+
+    def _fail(self, a, err, gone):
+        self._failed.append((a.id, err))
+        self._pages.give_back(a.pages)
+        gone.add(a.id)
+
+    @staticmethod
+    def _output(tokens, want_rank1):
+        out = np.array(tokens, dtype=np.int32)
+        return out if want_rank1 else out[None, :]

@@ -229,6 +229,25 @@ fa_status fa_sample_rows(fa_context *ctx, const fa_buffer *logits, uint64_t rows
                          fa_buffer *tokens);
 /* Generator::new(seed) (rng.rs:65-69, 684-689): seed 0 selects 0x9E3779B97F4A7C15. */
 fa_status fa_rng_seed(fa_context *ctx, fa_buffer *rng, uint64_t seed);
+/* The same rule as a plain host function: the generator state a seed starts. */
+fa_status fa_rng_state_from_seed(uint64_t seed, uint64_t *state);
+/* One row of a per-row sampling table: every row is a request with a
+ * GenerateConfig and a Generator of its own, as in the reference's continuous
+ * batching scheduler (crates/autodiff/src/generate/scheduler.rs:160-211: each
+ * active request owns its config and its rng, one draw per generated token).
+ * rng_state is advanced in place by one draw whenever a temperature / top-k row
+ * is sampled; a greedy row draws nothing. */
+typedef struct fa_row_sampling {
+    uint64_t rng_state;   /* xorshift64* state, never zero (fa_rng_state_from_seed) */
+    float temperature;    /* finite, > 0; 1 for greedy */
+    uint32_t top_k;       /* 1..=vocab for FA_SAMPLE_TOP_K, ignored otherwise */
+    int32_t strategy;     /* fa_sampling */
+    uint32_t reserved;
+} fa_row_sampling;
+/* fa_sample_rows with one fa_row_sampling per row: table is a U32 buffer of
+ * 6 * rows elements holding the rows' fa_row_sampling records. */
+fa_status fa_sample_rows_per_row(fa_context *ctx, const fa_buffer *logits, uint64_t rows, uint64_t vocab,
+                                 fa_buffer *table, fa_buffer *tokens);
 /* Measurement aid, not part of the reference's interface: queues a loop of one
  * matrix instruction kind with operands held in registers (kind 0:
  * v_mfma_i32_16x16x64_i8, 1: v_mfma_i32_32x32x32_i8, 2: the scaled
@@ -429,6 +448,14 @@ fa_status fa_decoder_step(fa_context *ctx, fa_decoder *dec, int32_t use_graph);
  * can be captured and replayed like a greedy one. */
 fa_status fa_decoder_set_sampling(fa_context *ctx, fa_decoder *dec, fa_sampling strategy, float temperature,
                                   uint64_t top_k, uint64_t seed);
+/* Per-request sampling for the installed sequences (rows [batch], host array):
+ * each row picks its next token by its own strategy from its own generator
+ * (scheduler.rs:160-211, 553-562).  The table stays on the device and its
+ * generator states advance there; read it back before the batch is rearranged
+ * and install the rearranged table after fa_decoder_set_sequences.
+ * fa_decoder_set_sampling returns to one strategy for all rows. */
+fa_status fa_decoder_set_row_sampling(fa_context *ctx, fa_decoder *dec, const fa_row_sampling *rows);
+fa_status fa_decoder_read_row_sampling(fa_context *ctx, fa_decoder *dec, fa_row_sampling *rows);
 /* Prompt ingestion: l_new tokens per installed sequence (tokens [batch, l_new],
  * host array), written behind what each sequence has cached, on the
  * prefill-shape GEMMs and the prefill form of the attention kernel, in chunks of
@@ -457,7 +484,9 @@ fa_status fa_decoder_read_seq_lens(fa_context *ctx, fa_decoder *dec, uint32_t *s
  * key 6: wavefronts per block of the large-tile prefill GEMMs (4 or 16; default 8);
  * key 7: column tiles of 16 per block of the large-tile prefill GEMMs (14 or 16);
  * key 8: nonzero sends attention with more than one new token per row to the generic
- *        kernel (the reference's summation order) instead of the streamed one. */
+ *        kernel (the reference's summation order) instead of the streamed one;
+ * key 9: blocks per compute unit that a split-k launch of the 128 x 128 int8 GEMM aims
+ *        for (default 2). */
 fa_status fa_set_tuning(int32_t key, int32_t value);
 /* A pair of HIP events recorded on the context's stream (the stream the
  * kernels run on); used by the benchmark to time launches. */

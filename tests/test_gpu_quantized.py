@@ -147,6 +147,34 @@ def test_w8a8_linear_row_sweep_bias_and_output_types(m):
     assert np.array_equal(out2, o.linear_w8a8(o.from_bf16(xb), wq, ws)[1])
 
 
+@pytest.mark.parametrize("m,k,n", [(33, 4096, 512), (100, 14336, 1030), (300, 2048, 768), (64, 1024, 4096), (200, 8192, 127)])
+def test_w8a8_split_k_gemm_is_bit_exact(m, k, n):
+    """A few hundred rows against a narrow weight: the GEMM splits k across blocks and adds the int32
+    partial sums afterwards; accumulators and outputs must not depend on it."""
+    fa = _fa()
+    be = ops()
+    rng = o.Rng(m + n)
+    x = rng.randn((m, k))
+    w = rng.randn((k, n), std=0.02)
+    bias = rng.randn((n,))
+    o.set_threads(8)
+    wq, ws = o.quantize_cols_i8(w)
+    want_acc, want = o.linear_w8a8(x, wq, ws, bias)
+    o.set_threads(1)
+    qw = be.import_quantized_weight(wq, ws)
+    dbias = fa.DeviceBufferView(be.upload(bias), 0, (n,))
+    out, acc = be.linear_w8a8(be.upload(x), qw, bias=dbias, want_acc=True)
+    assert np.array_equal(be.download_owned(acc), want_acc)
+    got = be.download_owned(out)
+    assert np.array_equal(got, want)
+    out_bf = be.linear_w8a8(be.upload(x), qw, bias=dbias, out_dtype=fa.capi.BF16)
+    assert_bf16_rounding_of("w8a8 split-k bf16", be.download_owned(out_bf), got)
+    # the pre-quantized entry point takes the same path
+    xq, sx = o.quantize_rows_i8(x)
+    got2 = be.download_owned(be.gemm_w8a8(be.upload(xq), be.upload(sx), qw, out_dtype=fa.capi.F32))
+    assert np.array_equal(got2, o.linear_w8a8(x, wq, ws)[1])
+
+
 def test_w8a8_ragged_shapes():
     be = ops()
     rng = o.Rng(13)

@@ -99,3 +99,35 @@ def test_decoder_steps_with_sampling_follow_the_oracle_generator():
         assert np.array_equal(dec.tokens(), o.argmax_rows(dec.logits()))
     finally:
         dec.close()
+
+
+@pytest.mark.parametrize("rows,vocab,kind", [(9, 1000, "normal"), (32, 32000, "ties"), (6, 17, "peaked"), (5, 300, "flat")])
+def test_per_row_policies_draw_from_their_own_generators(rows, vocab, kind):
+    """One request per row (fa_sample_rows_per_row): every row follows its own strategy, temperature, k and
+    generator; over consecutive calls each generator advances by exactly one draw per sampled token, a greedy
+    row draws nothing, and a row with a non-finite logit yields -1."""
+    fa = _fa()
+    be = ops()
+    rng = np.random.default_rng(rows + vocab)
+    menu = [(fa.SAMPLE_GREEDY, 1.0, 0), (fa.SAMPLE_TEMPERATURE, 0.7, 0), (fa.SAMPLE_TOP_K, 1.0, min(5, vocab)),
+            (fa.SAMPLE_TOP_K, 1.4, 1), (fa.SAMPLE_TEMPERATURE, 1.0, 0), (fa.SAMPLE_TOP_K, 0.5, vocab)]
+    records = [menu[r % len(menu)] + (0 if r == 1 else 1000 + 17 * r,) for r in range(rows)]
+    table = be.row_sampling_table(records)
+    refs = [os_.Generator(seed) for _, _, _, seed in records]
+    for step in range(4):
+        x = _logits(rng, rows, vocab, kind)
+        if step == 2:
+            x[rows - 1, vocab // 2] = np.inf
+        got = be.download_owned(be.sample_rows_per_row(be.upload(x), table))
+        for r, (strategy, temperature, k, _) in enumerate(records):
+            if not np.isfinite(x[r]).all():
+                assert got[r] == -1                        # and its generator did not move
+                continue
+            want = os_.sample_step(x[r:r + 1], strategy, temperature, k or None, refs[r])[0]
+            assert got[r] == want, (step, r, records[r], got[r], want)
+    words = be.download(table).reshape(rows, 6)
+    for r, (strategy, _, _, seed) in enumerate(records):
+        state = int(words[r, 1]) << 32 | int(words[r, 0])
+        assert state == refs[r].state
+        if strategy == fa.SAMPLE_GREEDY:
+            assert state == os_.Generator(seed).state
