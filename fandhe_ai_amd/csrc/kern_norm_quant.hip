@@ -221,32 +221,63 @@ __global__ void __launch_bounds__(kBlock)
 // SwiGLU of gu [m, 2 f] (gate columns first) followed by the per-token quantizer of the product, row-major:
 // pass 1 takes the row's absmax of silu(gate) * up, pass 2 recomputes the products (the row is in L2) and
 // writes their codes, so the f32 products never go to memory.  f a multiple of 16.
-__global__ void __launch_bounds__(kBlock)
+// ONE = true: 1024 threads and at most one 16-element chunk per thread (f <= 16384): the products stay in
+// registers between the two passes, so every element is loaded and its exponential taken once.
+template <bool ONE>
+__global__ void __launch_bounds__(ONE ? 1024 : kBlock)
     swiglu_quantize_rows_kernel(const float *__restrict__ gu, int8_t *__restrict__ xq_row, float *__restrict__ sx,
                                 uint64_t f) {
-    __shared__ float smem[kWaves];
+    constexpr int THREADS = ONE ? 1024 : kBlock;
+    __shared__ float smem[THREADS / 64];
     const uint64_t r = blockIdx.x;
     const float *gate = gu + r * 2 * f, *up = gate + f;
     float amax = 0.0f;
-    for (uint64_t c = threadIdx.x; c < f / 16; c += kBlock) {
-        float g[16], u[16];
-        load16<false>(gate, c * 16, g);
-        load16<false>(up, c * 16, u);
+    float prod[16];
+    if constexpr (ONE) {
+        const uint64_t c = threadIdx.x;
 #pragma unroll
-        for (int e = 0; e < 16; ++e) amax = fmaxf(amax, fabsf(silu_f32(g[e]) * u[e]));
+        for (int e = 0; e < 16; ++e) prod[e] = 0.0f;
+        if (c < f / 16) {
+            float g[16], u[16];
+            load16<false>(gate, c * 16, g);
+            load16<false>(up, c * 16, u);
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                prod[e] = silu_f32(g[e]) * u[e];
+                amax = fmaxf(amax, fabsf(prod[e]));
+            }
+        }
+    } else {
+        for (uint64_t c = threadIdx.x; c < f / 16; c += THREADS) {
+            float g[16], u[16];
+            load16<false>(gate, c * 16, g);
+            load16<false>(up, c * 16, u);
+#pragma unroll
+            for (int e = 0; e < 16; ++e) amax = fmaxf(amax, fabsf(silu_f32(g[e]) * u[e]));
+        }
     }
-    amax = block_max<kWaves>(amax, smem);
+    amax = block_max<THREADS / 64>(amax, smem);
     const float scale = __fdiv_rn(amax, 127.0f);
     if (threadIdx.x == 0) sx[r] = scale;
-    for (uint64_t c = threadIdx.x; c < f / 16; c += kBlock) {
-        float g[16], u[16];
-        load16<false>(gate, c * 16, g);
-        load16<false>(up, c * 16, u);
-        uint32_t words[4] = {0, 0, 0, 0};
+    if constexpr (ONE) {
+        const uint64_t c = threadIdx.x;
+        if (c < f / 16) {
+            uint32_t words[4] = {0, 0, 0, 0};
 #pragma unroll
-        for (int e = 0; e < 16; ++e)
-            words[e / 4] |= ((uint32_t)quant_i8(silu_f32(g[e]) * u[e], scale) & 0xffu) << (8 * (e % 4));
-        *(v4u *)(xq_row + r * f + c * 16) = v4u{words[0], words[1], words[2], words[3]};
+            for (int e = 0; e < 16; ++e) words[e / 4] |= ((uint32_t)quant_i8(prod[e], scale) & 0xffu) << (8 * (e % 4));
+            *(v4u *)(xq_row + r * f + c * 16) = v4u{words[0], words[1], words[2], words[3]};
+        }
+    } else {
+        for (uint64_t c = threadIdx.x; c < f / 16; c += THREADS) {
+            float g[16], u[16];
+            load16<false>(gate, c * 16, g);
+            load16<false>(up, c * 16, u);
+            uint32_t words[4] = {0, 0, 0, 0};
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+                words[e / 4] |= ((uint32_t)quant_i8(silu_f32(g[e]) * u[e], scale) & 0xffu) << (8 * (e % 4));
+            *(v4u *)(xq_row + r * f + c * 16) = v4u{words[0], words[1], words[2], words[3]};
+        }
     }
 }
 
@@ -359,7 +390,10 @@ void rmsnorm_quantize_rows_i8(const float *x, const float *w, float eps, int8_t 
 
 void swiglu_quantize_rows_i8(const float *gu, int8_t *xq_rowmajor, float *sx, uint64_t m, uint64_t f, hipStream_t s) {
     if (m == 0 || f == 0) return;
-    swiglu_quantize_rows_kernel<<<(unsigned)m, kBlock, 0, s>>>(gu, xq_rowmajor, sx, f);
+    if (f <= 16384)
+        swiglu_quantize_rows_kernel<true><<<(unsigned)m, 1024, 0, s>>>(gu, xq_rowmajor, sx, f);
+    else
+        swiglu_quantize_rows_kernel<false><<<(unsigned)m, kBlock, 0, s>>>(gu, xq_rowmajor, sx, f);
 }
 
 void quantize_rows_from_pmax(const void *x, bool in_bf16, const float *pmax, uint32_t parts, int8_t *xq_tiled,

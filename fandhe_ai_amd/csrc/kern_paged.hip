@@ -559,13 +559,17 @@ __global__ void __launch_bounds__(256) decode_stream_merge_kernel(StreamParams p
 }
 
 // Prefill: one block per (kv head, virtual sequence) merges the partial results of all its columns
-// (token tiles x tokens of a tile x heads of the group): two columns at a time, thread = (column parity, dim).
-__global__ void __launch_bounds__(256) prefill_stream_merge_kernel(StreamParams p, void *__restrict__ out, int out_bf16) {
-    __shared__ uint32_t s_tot[4], s_pre[4];
+// (token tiles x tokens of a tile x heads of the group): eight columns at a time, thread = (column slot, dim);
+// a column's partials are read one after the other, so the columns are what runs in parallel.
+constexpr int kPrefillMergeThreads = 1024;
+__global__ void __launch_bounds__(kPrefillMergeThreads)
+    prefill_stream_merge_kernel(StreamParams p, void *__restrict__ out, int out_bf16) {
+    constexpr int kW = kPrefillMergeThreads / 64, kSlots = kPrefillMergeThreads / 128;
+    __shared__ uint32_t s_tot[kW], s_pre[kW];
     const uint32_t kvh = blockIdx.x, vq = blockIdx.y, d = threadIdx.x % 128, part = threadIdx.x / 128;
     const uint32_t max_ctx = p.max_blocks_per_seq * kPage;
     uint32_t tot = 0, pre = 0;
-    for (uint32_t bb = threadIdx.x; bb < p.n_vseq; bb += 256) {
+    for (uint32_t bb = threadIdx.x; bb < p.n_vseq; bb += kPrefillMergeThreads) {
         uint32_t v = seq_pages<true>(p, bb, max_ctx);
         tot += v;
         if (bb < vq) pre += v;
@@ -577,14 +581,18 @@ __global__ void __launch_bounds__(256) prefill_stream_merge_kernel(StreamParams 
         s_pre[threadIdx.x / 64] = pre;
     }
     __syncthreads();
-    tot = s_tot[0] + s_tot[1] + s_tot[2] + s_tot[3];
-    pre = s_pre[0] + s_pre[1] + s_pre[2] + s_pre[3];
+    tot = pre = 0;
+#pragma unroll
+    for (int w = 0; w < kW; ++w) {
+        tot += s_tot[w];
+        pre += s_pre[w];
+    }
     const uint32_t npg = seq_pages<true>(p, vq, max_ctx);
     const uint32_t per = range_pages(p, tot);
     const uint32_t r_lo = npg ? pre / per : 1, r_hi = npg ? (pre + npg - 1) / per : 0;   // nothing streamed: no partials
     const uint32_t seq = vq / p.qt, tiles = p.tpv / p.tpt, cols = p.tpt * p.group;
     const bool violation = p.seq_lens[seq] < p.l_new;              // possible only with unvalidated device tables
-    for (uint32_t ci = part; ci < tiles * cols; ci += 2) {
+    for (uint32_t ci = part; ci < tiles * cols; ci += kSlots) {
         const uint32_t tile = ci / cols, col = ci % cols;
         const uint32_t t = p.t0 + (vq % p.qt) * p.tpv + tile * p.tpt + col / p.group;
         if (t >= p.l_new) continue;
@@ -897,7 +905,7 @@ void paged_attention_prefill_bf16(const uint16_t *q, const uint16_t *k_pool, con
             decode_stream_kernel<4, 4, 2, 1, true, kPrefillTT><<<(unsigned)((waves + 3) / 4), 256, 0, s>>>(sp);
         if (g_decode_partials_only) continue;
         dim3 grid2(ps.num_kv_heads, sp.n_vseq);
-        prefill_stream_merge_kernel<<<grid2, 256, 0, s>>>(sp, out, out_bf16);
+        prefill_stream_merge_kernel<<<grid2, kPrefillMergeThreads, 0, s>>>(sp, out, out_bf16);
     }
 }
 

@@ -81,6 +81,8 @@ PREFILL_SHAPES = [
     dict(n_layers=2, d_model=256, n_heads=4, n_kv_heads=2, d_ffn=512, vocab=1000, batch=4, ctxs=[0, 5, 16, 40], l_new=7),
     dict(n_layers=2, d_model=512, n_heads=8, n_kv_heads=2, d_ffn=768, vocab=500, batch=3, ctxs=[0, 1, 31], l_new=33),
     dict(n_layers=1, d_model=256, n_heads=2, n_kv_heads=2, d_ffn=256, vocab=300, batch=2, ctxs=[0, 100], l_new=1),
+    # d_ffn beyond 16384: the SwiGLU quantizer's two-pass form
+    dict(n_layers=1, d_model=256, n_heads=2, n_kv_heads=1, d_ffn=16448, vocab=300, batch=2, ctxs=[0, 5], l_new=9),
     # 8 x 600 rows: two chunks (512 + 88 tokens per sequence)
     dict(n_layers=1, d_model=256, n_heads=4, n_kv_heads=1, d_ffn=256, vocab=300, batch=8, ctxs=[0, 3, 9, 20, 0, 64, 7, 15],
          l_new=600),
