@@ -353,6 +353,29 @@ def bench_prompt_prefill(fa, be, dec, cfg, tables, batch=4, l_new=2048, reps=2):
     return dict(batch=batch, l_new=l_new, ms=ms, tokens_per_s=batch * l_new / (ms * 1e-3))
 
 
+def bench_short_prompts(fa, be, dec, cfg, tables, lengths=(64, 300, 1024), reps=3):
+    """One request's prompt pass (batch 1) on the resident model: what a scheduler runs when a request joins."""
+    lib = fa.capi.lib
+    row = int(np.argmax((tables != 0xFFFFFFFF).sum(axis=1)))           # the row with the most pages
+    tb = np.ascontiguousarray(tables[row:row + 1])
+    lens = np.zeros(1, dtype=np.uint32)
+    out = []
+    for l_new in lengths:
+        assert (l_new + 1 + cfg["block_size"] - 1) // cfg["block_size"] <= int((tb != 0xFFFFFFFF).sum())
+        prompt = np.random.default_rng(l_new).integers(0, cfg["vocab"], size=(1, l_new)).astype(np.int32)
+        best = None
+        for _ in range(reps + 1):
+            fa.check(lib.fa_decoder_set_sequences(be._ctx, dec, 1, tb.ctypes.data_as(fa.capi.u32p),
+                                                  lens.ctypes.data_as(fa.capi.u32p)))
+            t = Timer(fa, be)
+            t.start()
+            fa.check(lib.fa_decoder_prefill(be._ctx, dec, prompt.ctypes.data_as(fa.capi.i32p), l_new))
+            ms = t.stop_ms()
+            best = ms if best is None else min(best, ms)
+        out.append(dict(l_new=l_new, ms=best, tokens_per_s=l_new / (best * 1e-3)))
+    return out
+
+
 def bench_continuous_batching(fa, be, dec, dcfg, requests=96, max_active=32):
     """Continuous batching on the resident model: requests with prompts of 64..512 tokens that each generate
     64..192 tokens (greedy, temperature and top-k mixed) join and leave a batch of at most `max_active` rows;
@@ -485,12 +508,15 @@ def main():
     ap.add_argument("--layers", type=int, default=MODEL["n_layers"], help="debug only: fewer layers (invalidates the metric)")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-serving", action="store_true",
+                    help="skip the single-request prompt passes and the continuous-batching run (profiling aid: "
+                         "keeps the decode kernels of the trace at the benchmark's own shape)")
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--attn-waves", type=int, default=0,
                     help="tuning: wavefronts per compute unit of the decode attention (0 = built-in)")
     ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
                     help="tuning: raw fa_set_tuning key/value pairs (experiments)")
-    ap.add_argument("--only", choices=("attention", "copy", "linears", "prefill", "mfma"), default=None,
+    ap.add_argument("--only", choices=("attention", "copy", "linears", "prefill", "mfma", "prompt"), default=None,
                     help="profiling aid: run only the dominant kernel at the workload's shape, or a plain "
                          "copy kernel of known size (counter calibration), a few launches, no JSON line")
     a = ap.parse_args()
@@ -518,6 +544,14 @@ def main():
             for r in bench_prefill_attention(fa, be):
                 log("prefill attention 4 x 2048 new tokens, 32/8 heads, %s kernel: %.2f ms, %.1f TFLOP/s" %
                     (r["kernel"], r["ms"], r["tflops"]))
+            be.close()
+            return
+        if a.only == "prompt":
+            dec, keep, tables, _, _ = build_decoder(fa, be, cfg, batch, ctxs, 4)
+            for r in bench_short_prompts(fa, be, dec, cfg, tables):
+                log("one prompt of %d tokens through %d layers: %.2f ms, %.0f tokens/s" %
+                    (r["l_new"], cfg["n_layers"], r["ms"], r["tokens_per_s"]))
+            lib.fa_decoder_destroy(be._ctx, dec)
             be.close()
             return
         if a.only == "mfma":
@@ -576,8 +610,10 @@ def main():
             prompt = bench_prompt_prefill(fa, be, dec, cfg, np.ascontiguousarray(tables[order]))
             log("prompt prefill %d x %d tokens: %.1f ms, %.0f tokens/s" %
                 (prompt["batch"], prompt["l_new"], prompt["ms"], prompt["tokens_per_s"]))
-    batching = None
-    if not a.no_extras:
+    batching = short = None
+    if not a.no_extras and not a.no_serving:
+        short = bench_short_prompts(fa, be, dec, cfg, tables)
+        log("one prompt, batch 1: " + ", ".join("%d tokens %.2f ms" % (r["l_new"], r["ms"]) for r in short))
         dcfg = fa.capi.DecoderConfig(cfg["n_layers"], cfg["d_model"], cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"],
                                      cfg["d_ffn"], cfg["vocab"], cfg["block_size"], max_blocks, num_blocks, batch,
                                      cfg["rms_eps"], cfg["rope_theta"])
@@ -605,6 +641,8 @@ def main():
     extras = {"step_algorithmic_gb": bytes_step / 1e9, "step_hbm_frac": bytes_step / sec_per_step / 1e9 / HBM_PEAK_GBS}
     if prompt is not None:
         extras["prompt_prefill"] = prompt
+    if short is not None:
+        extras["prompt_pass_one_request"] = short
     if batching is not None:
         extras["continuous_batching"] = batching
     if not a.no_extras:
