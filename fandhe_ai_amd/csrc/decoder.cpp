@@ -224,11 +224,15 @@ struct Temp {
 // a prompt token leaves the same K / V rows in the cache as if it had been decoded.
 struct PrefillBuffers {
     Temp tok, h, xq, sx, qkv, q_bf, attn, gu, slots, cos_sin, last_rows, splitk;
+    // verification only: logits and greedy picks of every row
+    Temp all_logits, all_picked;
     explicit PrefillBuffers(fa_context *c)
-        : tok(c), h(c), xq(c), sx(c), qkv(c), q_bf(c), attn(c), gu(c), slots(c), cos_sin(c), last_rows(c), splitk(c) {}
+        : tok(c), h(c), xq(c), sx(c), qkv(c), q_bf(c), attn(c), gu(c), slots(c), cos_sin(c), last_rows(c), splitk(c),
+          all_logits(c), all_picked(c) {}
 };
 
-fa_status enqueue_prefill_chunk(fa_context *ctx, fa_decoder *d, PrefillBuffers &t, uint32_t lc, bool last_chunk) {
+fa_status enqueue_prefill_chunk(fa_context *ctx, fa_decoder *d, PrefillBuffers &t, uint32_t lc, bool last_chunk,
+                                bool every_row = false) {
     const fa_decoder_config &c = d->cfg;
     const uint32_t B = d->batch;
     const uint64_t M = (uint64_t)B * lc;
@@ -289,6 +293,13 @@ fa_status enqueue_prefill_chunk(fa_context *ctx, fa_decoder *d, PrefillBuffers &
         gemm(L.wgu, t.gu.as<float>(), nullptr);
         k::swiglu_quantize_rows_i8(t.gu.as<float>(), t.xq.as<int8_t>(), t.sx.as<float>(), M, F, s);
         gemm(L.wdown, t.h.as<float>(), t.h.as<float>());
+    }
+    if (every_row) {
+        // verification: the head over every row of the chunk (row b * lc + t is token t of sequence b)
+        k::rmsnorm_quantize_rows_i8(t.h.as<float>(), (const float *)d->final_norm->ptr, c.rms_eps, t.xq.as<int8_t>(),
+                                    t.sx.as<float>(), M, D, s);
+        gemm(d->lm_head, t.all_logits.as<float>(), nullptr);
+        k::argmax_rows_f32(t.all_logits.as<float>(), t.all_picked.as<int32_t>(), M, V, s);
     }
     if (last_chunk) {
         // logits of every sequence's last prompt token, and the greedy next token, as a decode step leaves them
@@ -577,7 +588,9 @@ fa_status fa_decoder_step(fa_context *ctx, fa_decoder *d, int32_t use_graph) {
     return fa_graph_launch(ctx, it->second);
 }
 
-fa_status fa_decoder_prefill(fa_context *ctx, fa_decoder *d, const int32_t *tokens, uint32_t l_new) {
+static fa_status prefill_impl(fa_context *ctx, fa_decoder *d, const int32_t *tokens, uint32_t l_new, int32_t *picked,
+                              float *logits) {
+    const bool verify = picked != nullptr;
     if (fa_status s = check_ctx(ctx)) return s;
     if (fa_status s = check_dec(d)) return s;
     if (d->ctx != ctx) return fail(FA_ERR_DEVICE_MISMATCH, "decoder_prefill: decoder belongs to another context");
@@ -605,6 +618,8 @@ fa_status fa_decoder_prefill(fa_context *ctx, fa_decoder *d, const int32_t *toke
     }
     // chunks of at most kRows rows per pass bound the activation memory (the widest is [rows, 2 d_ffn] f32)
     constexpr uint64_t kRows = 4096;
+    if (verify && (uint64_t)B * l_new > kRows)
+        return fail(FA_ERR_INVALID_ARGUMENT, "decoder_verify: at most 4096 rows (batch x tokens) per call");
     const uint32_t lc_max = (uint32_t)std::max<uint64_t>(1, std::min<uint64_t>(l_new, kRows / B));
     const uint64_t M = (uint64_t)B * lc_max;
     const uint64_t D = c.d_model, F = c.d_ffn, EQ = (uint64_t)c.n_heads * c.head_dim, EKV = (uint64_t)c.n_kv_heads * c.head_dim;
@@ -632,7 +647,13 @@ fa_status fa_decoder_prefill(fa_context *ctx, fa_decoder *d, const int32_t *toke
         for (const auto &l : d->layers)
             for (const fa_qweight *w : {l.wqkv, l.wo, l.wgu, l.wdown})
                 need = std::max(need, k::gemm_w8a8_workspace_bytes(M, w->n, w->n_pad, w->k_pad, cus));
+        if (verify)
+            need = std::max(need, k::gemm_w8a8_workspace_bytes(M, d->lm_head->n, d->lm_head->n_pad, d->lm_head->k_pad, cus));
         get(t.splitk, need);
+    }
+    if (verify) {
+        get(t.all_logits, M * c.vocab * 4);
+        get(t.all_picked, M * 4);
     }
     if (st != FA_OK) return st;
     k::PagedShape ps{};
@@ -657,9 +678,42 @@ fa_status fa_decoder_prefill(fa_context *ctx, fa_decoder *d, const int32_t *toke
         hipError_t e = hipMemcpyAsync(t.tok.ptr, stage.data(), (uint64_t)B * lc * 4, hipMemcpyHostToDevice, ctx->stream);
         if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
         if (e != hipSuccess) return hip_fail(ctx, e, "prompt token upload", FA_ERR_TRANSFER_FAILED);
-        if (fa_status s = enqueue_prefill_chunk(ctx, d, t, lc, t0 + lc == l_new)) return s;
+        if (fa_status s = enqueue_prefill_chunk(ctx, d, t, lc, t0 + lc == l_new, verify)) return s;
         for (auto &len : d->host_lens) len += lc;
     }
+    if (verify) {
+        // one chunk; the buffers go back to the pool when this call returns, so the copies finish here
+        hipError_t e = hipMemcpyAsync(picked, t.all_picked.ptr, (uint64_t)B * l_new * 4, hipMemcpyDeviceToHost, ctx->stream);
+        if (e == hipSuccess && logits)
+            e = hipMemcpyAsync(logits, t.all_logits.ptr, (uint64_t)B * l_new * c.vocab * 4, hipMemcpyDeviceToHost, ctx->stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+        if (e != hipSuccess) return hip_fail(ctx, e, "verification results download", FA_ERR_TRANSFER_FAILED);
+    }
+    return FA_OK;
+}
+
+fa_status fa_decoder_prefill(fa_context *ctx, fa_decoder *d, const int32_t *tokens, uint32_t l_new) {
+    return prefill_impl(ctx, d, tokens, l_new, nullptr, nullptr);
+}
+
+fa_status fa_decoder_verify(fa_context *ctx, fa_decoder *d, const int32_t *tokens, uint32_t l_new, int32_t *picked,
+                            float *logits) {
+    if (!picked) return fail(FA_ERR_INVALID_ARGUMENT, "decoder_verify: null picked");
+    return prefill_impl(ctx, d, tokens, l_new, picked, logits);
+}
+
+fa_status fa_decoder_rewind(fa_context *ctx, fa_decoder *d, const uint32_t *seq_lens) {
+    if (fa_status s = check_ctx(ctx)) return s;
+    if (fa_status s = check_dec(d)) return s;
+    if (d->ctx != ctx) return fail(FA_ERR_DEVICE_MISMATCH, "decoder_rewind: decoder belongs to another context");
+    if (ctx->capturing) return fail(FA_ERR_CAPTURE_IN_PROGRESS, "decoder_rewind during graph capture");
+    if (d->batch == 0 || !seq_lens) return fail(FA_ERR_INVALID_ARGUMENT, "decoder_rewind: no sequences or null lengths");
+    for (uint32_t b = 0; b < d->batch; ++b)
+        if (seq_lens[b] > d->host_lens[b])
+            return fail(FA_ERR_INVALID_ARGUMENT, "decoder_rewind: row " + std::to_string(b) + " cannot grow (" +
+                                                     std::to_string(seq_lens[b]) + " > " + std::to_string(d->host_lens[b]) + ")");
+    if (fa_status s = fa_upload_into(ctx, seq_lens, d->batch, d->seq_lens, 0)) return s;
+    std::copy(seq_lens, seq_lens + d->batch, d->host_lens.begin());
     return FA_OK;
 }
 

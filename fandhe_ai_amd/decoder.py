@@ -83,6 +83,26 @@ class Decoder:
             raise ValueError("prompt must be [batch, l_new]")
         check(lib.fa_decoder_prefill(self._ops._ctx, self._h, p.ctypes.data_as(capi.i32p), p.shape[1]))
 
+    def verify(self, tokens, want_logits=False):
+        """Speculative verification: feeds tokens [batch, l_new] like ``prefill`` and returns the greedy token
+        after every one of them, int32 [batch, l_new] (and the logits [batch, l_new, vocab] if asked)."""
+        p = np.ascontiguousarray(tokens, dtype=np.int32)
+        if p.ndim != 2 or p.shape[0] != self.batch:
+            raise ValueError("tokens must be [batch, l_new]")
+        picked = np.empty(p.shape, dtype=np.int32)
+        logits = np.empty(p.shape + (self.cfg.vocab,), dtype=np.float32) if want_logits else None
+        check(lib.fa_decoder_verify(self._ops._ctx, self._h, p.ctypes.data_as(capi.i32p), p.shape[1],
+                                    picked.ctypes.data_as(capi.i32p),
+                                    logits.ctypes.data_as(capi.f32p) if want_logits else None))
+        return (picked, logits) if want_logits else picked
+
+    def rewind(self, seq_lens):
+        """Shortens the installed sequences (no row may grow); the pages are kept."""
+        s = np.ascontiguousarray(seq_lens, dtype=np.uint32)
+        if s.size != self.batch:
+            raise ValueError("one length per installed sequence")
+        check(lib.fa_decoder_rewind(self._ops._ctx, self._h, s.ctypes.data_as(capi.u32p)))
+
     def step(self, use_graph=True):
         check(lib.fa_decoder_step(self._ops._ctx, self._h, 1 if use_graph else 0))
 

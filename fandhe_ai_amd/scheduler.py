@@ -179,6 +179,89 @@ def generate(decoder, input_ids, config):
     return out[0] if want_rank1 else out
 
 
+class Unsupported(ValueError):
+    """What the device path does not offer (the reference does)."""
+
+
+def generate_speculative(target, draft, input_ids, config, k):
+    """``generate_speculative`` (crates/autodiff/src/generate/speculative.rs:334-531), greedy form, on two
+    resident decoders: per round the draft decodes ``k_eff = min(k, remaining - 1)`` tokens, the target
+    consumes the pending token and those drafts in one verification pass (``Decoder.verify``), the longest
+    prefix of drafts that equals the target's own greedy tokens is kept and the target's token at the first
+    disagreement (or after the last draft) is appended.  Both caches are then cut back to the accepted
+    length with ``Decoder.rewind``: paged rows past a sequence's length are dead, so nothing is replayed
+    (the reference restores a snapshot and replays the accepted tokens, kv_rewind.rs:157-215).  One
+    sequence per call, as in the reference.  The output equals ``generate(target, ...)`` wherever the
+    target's greedy choice is decisive (the verification pass runs prompt-shape kernels, a decode step
+    the decode-shape ones; int32 accumulators are identical, attention sums are associated differently).
+    Returns (tokens, rounds, accepted drafts)."""
+    config.validate()
+    if not isinstance(k, int) or k < 1:
+        raise InvalidArgument("generate_speculative: k must be at least 1")
+    ids, b, prompt_len, want_rank1 = _prompt_shape(input_ids, "generate_speculative")
+    if prompt_len == 0:
+        raise InvalidArgument("generate_speculative: the prompt is empty")
+    if b != 1:
+        raise InvalidArgument("generate_speculative: one sequence only (got %d)" % b)
+    max_length = config.max_length
+    if max_length < prompt_len:
+        raise InvalidArgument("generate_speculative: max_length (%d) must be at least the prompt length (%d)" % (max_length, prompt_len))
+    _check_buffer_bytes(max_length)
+    if config.strategy.kind != GREEDY:
+        raise Unsupported("generate_speculative: only the greedy form runs on the device (sampled acceptance needs both "
+                          "models' probabilities on the host)")
+    row = [int(t) for t in ids[0]]
+    rounds = accepted = 0
+    if max_length > prompt_len:
+        if target.cfg.vocab != draft.cfg.vocab:
+            raise InvalidArgument("generate_speculative: the models disagree on the vocabulary (%d, %d)" % (draft.cfg.vocab, target.cfg.vocab))
+        for dec in (target, draft):
+            cfg = dec.cfg
+            pages = _pages_for(max_length + 1, cfg.block_size)     # the verification pass also writes the last draft
+            if pages > cfg.max_blocks_per_seq or pages > cfg.num_blocks:
+                raise InvalidArgument("generate_speculative: %d tokens do not fit the decoder's page pool" % max_length)
+            table = np.full((1, cfg.max_blocks_per_seq), 0xFFFFFFFF, dtype=np.uint32)
+            table[0, :pages] = np.arange(pages, dtype=np.uint32)
+            dec.set_sequences(table, np.zeros(1, np.uint32))
+            dec.set_sampling(GREEDY)
+            dec.prefill(ids.astype(np.int32))
+        row.append(int(target.tokens()[0]))
+        while len(row) < max_length:
+            cur, last = len(row), row[-1]
+            remaining = max_length - cur
+            if remaining == 1:
+                target.set_tokens([last])
+                target.step()
+                row.append(int(target.tokens()[0]))
+                break
+            k_eff = min(k, remaining - 1)
+            drafts, x = [], last
+            for _ in range(k_eff):                         # the draft's cache grows by last, d1 .. d_{k_eff - 1}
+                draft.set_tokens([x])
+                draft.step()
+                x = int(draft.tokens()[0])
+                drafts.append(x)
+            picked = target.verify(np.array([[last] + drafts], dtype=np.int32))[0]
+            n_acc = 0
+            while n_acc < k_eff and drafts[n_acc] == picked[n_acc]:
+                n_acc += 1
+            row.extend(drafts[:n_acc])
+            row.append(int(picked[n_acc]))
+            rounds += 1
+            accepted += n_acc
+            if len(row) >= max_length:
+                break
+            keep = cur + n_acc                             # tokens before the new pending one
+            target.rewind([keep])
+            if n_acc == k_eff:
+                draft.set_tokens([x])                      # the draft never consumed its own last token
+                draft.step()
+            else:
+                draft.rewind([keep])
+    out = np.array(row[:max_length], dtype=np.int32)
+    return (out if want_rank1 else out[None, :]), rounds, accepted
+
+
 class SchedulerLimits:
     """scheduler.rs:80-127: every limit is mandatory and at least 1."""
 

@@ -466,6 +466,22 @@ fa_status fa_decoder_read_row_sampling(fa_context *ctx, fa_decoder *dec, fa_row_
  * decoded.  Rejected before anything is queued if a row has no pages for its
  * prompt.  Asynchronous apart from the upload of the token ids. */
 fa_status fa_decoder_prefill(fa_context *ctx, fa_decoder *dec, const int32_t *tokens, uint32_t l_new);
+/* Speculative-decoding verification (crates/autodiff/src/generate/speculative.rs:
+ * 484-490: the target model consumes the pending token and the draft's k tokens
+ * in one forward pass and every position's logits decide): fa_decoder_prefill
+ * that also returns, for every row b * l_new + t, the greedy token after token t
+ * of sequence b (picked [batch, l_new], host array) and, if logits is not null,
+ * that row's logits ([batch * l_new, vocab] f32, host array).  At most 4096 rows;
+ * synchronous.  The sequence lengths advance by l_new as in a prompt pass; what
+ * was rejected is dropped with fa_decoder_rewind. */
+fa_status fa_decoder_verify(fa_context *ctx, fa_decoder *dec, const int32_t *tokens, uint32_t l_new,
+                            int32_t *picked, float *logits);
+/* Shortens the installed sequences to seq_lens [batch] (host array; a row may
+ * keep its length, none may grow).  The pages stay where they are and cached
+ * rows past the new length are simply overwritten by later tokens: the paged
+ * counterpart of the reference's snapshot / restore / replay
+ * (crates/autodiff/src/generate/kv_rewind.rs:60-215), without the replay. */
+fa_status fa_decoder_rewind(fa_context *ctx, fa_decoder *dec, const uint32_t *seq_lens);
 /* Host copies of the current tokens [batch] / logits [batch, vocab] /
  * sequence lengths [batch] (synchronize). */
 fa_status fa_decoder_read_tokens(fa_context *ctx, fa_decoder *dec, int32_t *tokens);

@@ -153,6 +153,20 @@ class GpuDecoder:
         self.fa.check(self.fa.capi.lib.fa_decoder_prefill(self.be._ctx, self.h, p.ctypes.data_as(self.fa.capi.i32p),
                                                           p.shape[1]))
 
+    def verify(self, tokens):
+        """tokens int32 [batch, l_new] -> (picked [batch, l_new], logits [batch, l_new, vocab])"""
+        p = np.ascontiguousarray(tokens, dtype=np.int32)
+        picked = np.empty(p.shape, dtype=np.int32)
+        logits = np.empty(p.shape + (self.m.cfg["vocab"],), dtype=np.float32)
+        self.fa.check(self.fa.capi.lib.fa_decoder_verify(self.be._ctx, self.h, p.ctypes.data_as(self.fa.capi.i32p), p.shape[1],
+                                                         picked.ctypes.data_as(self.fa.capi.i32p),
+                                                         logits.ctypes.data_as(self.fa.capi.f32p)))
+        return picked, logits
+
+    def rewind(self, seq_lens):
+        s = np.ascontiguousarray(seq_lens, dtype=np.uint32)
+        self.fa.check(self.fa.capi.lib.fa_decoder_rewind(self.be._ctx, self.h, s.ctypes.data_as(self.fa.capi.u32p)))
+
     def tokens(self):
         out = np.empty(self.m.batch, dtype=np.int32)
         self.fa.check(self.fa.capi.lib.fa_decoder_read_tokens(self.be._ctx, self.h, out.ctypes.data_as(self.fa.capi.i32p)))

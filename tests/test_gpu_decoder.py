@@ -135,6 +135,60 @@ def test_prompt_prefill_matches_the_oracle_decoding_the_prompt_token_by_token(sh
         dec.close()
 
 
+@pytest.mark.parametrize("shape", [
+    dict(n_layers=2, d_model=256, n_heads=4, n_kv_heads=2, d_ffn=512, vocab=1000, batch=3, ctxs=[0, 5, 40], l_new=6),
+    dict(n_layers=1, d_model=256, n_heads=2, n_kv_heads=1, d_ffn=256, vocab=300, batch=1, ctxs=[21], l_new=40),
+], ids=["B3_L6", "B1_L40"])
+def test_verification_pass_matches_the_oracle_at_every_position_and_rewind_drops_the_tail(shape):
+    """fa_decoder_verify returns the logits and the greedy token after every fed token: each row is held to
+    the oracle decoding the same tokens one by one (chained-step tolerance); the last row is the resident
+    result of the pass itself, bit for bit.  After a rewind the dropped positions are decoded again and
+    must reproduce the verification's logits for them."""
+    be = ops()
+    shape = dict(shape)
+    l_new = shape.pop("l_new")
+    B, V = shape["batch"], shape["vocab"]
+    m = build_model(seed=33, steps=l_new + 2, **shape)
+    dec = GpuDecoder(be, m)
+    try:
+        rng = o.Rng(8)
+        feed = rng.randint(0, V, B * l_new).astype(np.int32).reshape(B, l_new)
+        lens = m.seq_lens.copy()
+        want = []
+        for t in range(l_new):
+            want.append(oracle_step(m, lens, np.ascontiguousarray(feed[:, t])))
+        picked, logits = dec.verify(feed)
+        assert np.array_equal(dec.seq_lens(), m.seq_lens + l_new)
+        assert logits[:, -1].tobytes() == dec.logits().tobytes() and np.array_equal(picked[:, -1], dec.tokens())
+        worst = 0.0
+        for t, (want_next, want_logits) in enumerate(want):
+            spread = want_logits.max(axis=1, keepdims=True) - want_logits.min(axis=1, keepdims=True)
+            err = np.abs(logits[:, t] - want_logits) / spread
+            worst = max(worst, float(err.max()))
+            assert err.mean() < 2e-4 and err.max() < 2e-2, (t, err.mean(), err.max())
+            top2 = np.sort(want_logits, axis=1)[:, -2:]
+            decisive = (top2[:, 1] - top2[:, 0]) > 4e-2 * spread[:, 0]
+            assert np.array_equal(picked[decisive, t], want_next[decisive]), t
+            assert np.array_equal(picked[:, t], o.argmax_rows(np.ascontiguousarray(logits[:, t])))
+        print("VERIFY_PARITY\tB%d:L%d\tmax_err/range over all positions=%.3e" % (B, l_new, worst), flush=True)
+        # drop the last three tokens of every row and decode them again, one step at a time
+        keep = l_new - 3
+        dec.rewind(m.seq_lens + keep)
+        assert np.array_equal(dec.seq_lens(), m.seq_lens + keep)
+        for t in range(keep, l_new):
+            dec.set_state(m.seq_lens + t, feed[:, t])
+            dec.step(True)
+            got = dec.logits()
+            spread = logits[:, t].max(axis=1, keepdims=True) - logits[:, t].min(axis=1, keepdims=True)
+            err = np.abs(got - logits[:, t]) / spread
+            assert err.mean() < 2e-4 and err.max() < 2e-2, (t, err.mean(), err.max())
+        import fandhe_ai_amd as fa
+        with pytest.raises(fa.InvalidArgument):
+            dec.rewind(m.seq_lens + l_new + 1)                                # a rewind cannot grow a row
+    finally:
+        dec.close()
+
+
 def test_prefill_argument_errors():
     import fandhe_ai_amd as fa
     be = ops()

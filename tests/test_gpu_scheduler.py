@@ -225,3 +225,48 @@ def test_cached_step_graphs_survive_batch_changes_and_workspace_growth():
     for a, b, c in zip(eager, graph, again):
         assert np.isfinite(a).all() and a.tobytes() == b.tobytes() == c.tobytes()
     dec.close()
+
+
+def test_speculative_generation_equals_the_target_generating_alone():
+    """Greedy speculative decoding with (a) a draft that is the target's twin and (b) a different, smaller
+    draft: the tokens must be the target's own greedy tokens up to the first position where the target's
+    two best logits are closer than the chained-step bar allows to tell apart (verification runs the
+    prompt-shape kernels, plain generation the decode-shape ones)."""
+    import fandhe_ai_amd as fa
+    from fandhe_ai_amd.scheduler import SamplingStrategy, generate, generate_speculative
+    geometry = dict(max_blocks_per_seq=8, num_blocks=8, max_batch=1)
+    target = _recording(_decoder(**geometry))
+    twin = _decoder(**geometry)
+    other_ckpt = st_save(_checkpoint(77, 1, D, HEADS, KV, F, VOCAB))
+    other, store = fa.safetensors_io.load_decoder(ops(), other_ckpt, 1, HEADS, KV, **geometry)
+    store.free()
+    rng = np.random.default_rng(4)
+    total = matched = 0
+    for plen, max_length, k in ((5, 60, 4), (33, 80, 3), (1, 20, 7), (12, 14, 2)):
+        prompt = rng.integers(0, VOCAB, plen).astype(np.int32)
+        cfg = _cfg(max_length, SamplingStrategy.Greedy(), 0)
+        target.trace = []
+        want = generate(target, prompt, cfg)
+        margins = []
+        for _, _, logits, _ in target.trace:
+            top2 = np.sort(logits)[-2:]
+            margins.append(float(top2[1] - top2[0]) / float(logits.max() - logits.min()))
+        assert len(margins) == max_length - plen
+        for draft, name in ((twin, "twin"), (other, "other")):
+            got, rounds, accepted = generate_speculative(target, draft, prompt, cfg, k)
+            assert got.shape == want.shape and np.array_equal(got[:plen], prompt)
+            new = max_length - plen
+            agree = 0
+            while agree < new and got[plen + agree] == want[plen + agree]:
+                agree += 1
+            if agree < new:
+                assert margins[agree] < 4e-2, (name, plen, agree, margins[agree])     # only an indecisive pick may differ
+            total += new
+            matched += agree
+            if name == "twin":
+                assert accepted >= 0.5 * agree - k and rounds < new                   # most drafts are accepted
+            print("SPECULATIVE\t%s\tprompt %d, %d new tokens, k %d: %d rounds, %d drafts accepted, %d tokens equal"
+                  % (name, plen, new, k, rounds, accepted, agree), flush=True)
+    assert matched >= 0.9 * total
+    for d in (target, twin, other):
+        d.close()

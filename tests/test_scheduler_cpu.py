@@ -14,7 +14,7 @@ import sampling as osamp  # noqa: E402
 import fandhe_ai_amd as fa  # noqa: E402
 from fandhe_ai_amd import capi  # noqa: E402
 from fandhe_ai_amd.scheduler import (BatchScheduler, GenerateConfig, InvalidArgument, PageAllocator, RankMismatch,  # noqa: E402
-                                     SamplingStrategy, SchedulerLimits, generate)
+                                     SamplingStrategy, SchedulerLimits, Unsupported, generate, generate_speculative)
 
 VOCAB, BLOCK = 11, 16
 
@@ -25,9 +25,11 @@ class Cfg:
         self.block_size, self.vocab = BLOCK, VOCAB
 
 
-def toy_logits(history):
+def toy_logits(history, salt=0):
     """A table-like model: logits depend on every token seen so far and on the position."""
-    h = 0
+    if callable(salt):
+        salt = salt(len(history))
+    h = salt
     for i, t in enumerate(history):
         h = (h * 31 + (t + 1) * (i + 7)) % 1000003
     rng = np.random.default_rng(h)
@@ -37,8 +39,9 @@ def toy_logits(history):
 class ToyDecoder:
     """The surface of fandhe_ai_amd.Decoder that generation uses, on the host."""
 
-    def __init__(self, max_batch=4, num_blocks=8, max_blocks_per_seq=4):
+    def __init__(self, max_batch=4, num_blocks=8, max_blocks_per_seq=4, salt=0):
         self.cfg = Cfg(max_batch, num_blocks, max_blocks_per_seq)
+        self.salt = salt
         self.pool = np.full((num_blocks, BLOCK), -1, dtype=np.int64)
         self.calls = {"prefill": 0, "step": 0, "step_rows": 0}
         self.poison_token = None
@@ -82,7 +85,7 @@ class ToyDecoder:
         out = []
         for b in range(self.batch):
             hist = self._history(b)
-            logits = toy_logits(hist)
+            logits = toy_logits(hist, self.salt)
             if self.poison_token is not None and (hist[0], hist[-1]) == self.poison_token:
                 out.append(-1)                             # the device reports a non-finite row this way
                 continue
@@ -118,6 +121,23 @@ class ToyDecoder:
 
     def tokens(self):
         return np.array(self.cur, dtype=np.int32)
+
+    def verify(self, tokens):
+        self.calls["verify"] = self.calls.get("verify", 0) + 1
+        tokens = np.asarray(tokens)
+        picked = np.empty(tokens.shape, dtype=np.int32)
+        for b in range(self.batch):
+            for i, t in enumerate(tokens[b]):
+                self._write(b, int(self.lens[b]), int(t))
+                self.lens[b] += 1
+                picked[b, i] = osamp.greedy_argmax(toy_logits(self._history(b), self.salt))
+        self.cur = [int(p[-1]) for p in picked]
+        return picked
+
+    def rewind(self, lens):
+        lens = np.asarray(lens, dtype=np.int64)
+        assert (lens <= self.lens).all(), "a rewind cannot grow a sequence"
+        self.lens = lens.copy()
 
 
 def cfg(max_length, strategy, seed):
@@ -300,3 +320,45 @@ def test_rng_state_from_seed_is_the_generator_rule():
         assert capi.lib.fa_rng_state_from_seed(seed, st) == 0
         assert st.value == osamp.Generator(seed).state
     assert fa.scheduler.GREEDY == osamp.GREEDY and fa.scheduler.TOP_K == osamp.TOP_K
+
+
+def test_speculative_greedy_equals_plain_generation_whatever_the_draft_proposes():
+    # crates/autodiff/src/generate/speculative.rs tests: a draft that agrees, one that never does, one that
+    # agrees on two positions out of three
+    greedy = SamplingStrategy.Greedy()
+    drafts = {"same": 0, "wrong": 12345, "mixed": lambda n: 12345 if n % 3 == 0 else 0}
+    for prompt, max_length in (([3], 2), ([1, 2], 30), ([4] * 17, 40), ([5, 6, 7], 4), ([2], 3)):
+        want = generate(ToyDecoder(), prompt, cfg(max_length, greedy, 0))
+        for name, salt in drafts.items():
+            for k in (1, 2, 4, 7):
+                target, draft = ToyDecoder(num_blocks=4), ToyDecoder(num_blocks=4, salt=salt)
+                got, rounds, accepted = generate_speculative(target, draft, prompt, cfg(max_length, greedy, 0), k)
+                assert got.tolist() == want.tolist(), (prompt, max_length, name, k)
+                new = max_length - len(prompt)
+                if name == "same" and new > 2:
+                    assert accepted > 0 and target.calls["step"] <= 1      # the target only verifies
+                    assert rounds <= -(-new // (k + 1)) + 1
+                assert 0 <= accepted <= new and rounds <= max(new - 1, 0)
+    got, _, _ = generate_speculative(ToyDecoder(), ToyDecoder(), np.array([[1, 2]]), cfg(9, greedy, 0), 3)
+    assert got.shape == (1, 9)
+    got, rounds, _ = generate_speculative(ToyDecoder(), ToyDecoder(), [1, 2], cfg(2, greedy, 0), 3)
+    assert got.tolist() == [1, 2] and rounds == 0
+
+
+def test_speculative_argument_errors():
+    greedy = SamplingStrategy.Greedy()
+    T, D = ToyDecoder, ToyDecoder
+    with pytest.raises(InvalidArgument):
+        generate_speculative(T(), D(), [1], cfg(4, greedy, 0), 0)
+    with pytest.raises(InvalidArgument):
+        generate_speculative(T(), D(), np.array([[1], [2]]), cfg(4, greedy, 0), 2)
+    with pytest.raises(InvalidArgument):
+        generate_speculative(T(), D(), np.array([], dtype=np.int32), cfg(4, greedy, 0), 2)
+    with pytest.raises(InvalidArgument):
+        generate_speculative(T(), D(), [1, 2, 3], cfg(2, greedy, 0), 2)
+    with pytest.raises(RankMismatch):
+        generate_speculative(T(), D(), np.zeros((1, 1, 2), np.int32), cfg(4, greedy, 0), 2)
+    with pytest.raises(Unsupported):
+        generate_speculative(T(), D(), [1], cfg(4, SamplingStrategy.TopK(2), 0), 2)
+    with pytest.raises(InvalidArgument):                   # a sequence longer than the page table of one model
+        generate_speculative(T(), D(max_blocks_per_seq=1), [1], cfg(40, greedy, 0), 2)
