@@ -28,39 +28,52 @@ __global__ void add_kernel(const float *__restrict__ a, const float *__restrict_
 
 // First index of the maximum, NaN ignored, all-NaN row -> 0
 // (crates/autodiff/src/generate/mod.rs:333-343, crates/backend-rocm/src/ops.rs:991-995).
-__global__ void __launch_bounds__(256) argmax_rows_kernel(const float *__restrict__ x, int32_t *__restrict__ out,
-                                                          uint64_t cols) {
+__device__ __forceinline__ void argmax_take(float &mv, uint32_t &mi, float ov, uint32_t oi) {
+    const bool take = oi != 0xffffffffu && (mi == 0xffffffffu || ov > mv || (ov == mv && oi < mi));
+    mv = take ? ov : mv;
+    mi = take ? oi : mi;
+}
+
+constexpr int kArgmaxThreads = 1024;
+__global__ void __launch_bounds__(kArgmaxThreads)
+    argmax_rows_kernel(const float *__restrict__ x, int32_t *__restrict__ out, uint64_t cols) {
     const float *row = x + (uint64_t)blockIdx.x * cols;
     float best = -INFINITY;
     uint32_t best_i = 0xffffffffu;      // "nothing seen yet"
-    for (uint64_t i = threadIdx.x; i < cols; i += blockDim.x) {
-        float v = row[i];
-        if (v != v) continue;
-        if (best_i == 0xffffffffu || v > best) {
+    auto see = [&](float v, uint32_t i) {
+        if (v == v && (best_i == 0xffffffffu || v > best)) {      // ascending i per thread: the first maximum stays
             best = v;
-            best_i = (uint32_t)i;
+            best_i = i;
         }
+    };
+    if (cols % 4 == 0) {                                          // rows start on 16-byte boundaries
+        for (uint64_t q = threadIdx.x; q < cols / 4; q += kArgmaxThreads) {
+            const float4 v = *(const float4 *)(row + 4 * q);
+            see(v.x, (uint32_t)(4 * q));
+            see(v.y, (uint32_t)(4 * q + 1));
+            see(v.z, (uint32_t)(4 * q + 2));
+            see(v.w, (uint32_t)(4 * q + 3));
+        }
+    } else {
+        for (uint64_t i = threadIdx.x; i < cols; i += kArgmaxThreads) see(row[i], (uint32_t)i);
     }
-    __shared__ float s_val[256];
-    __shared__ uint32_t s_idx[256];
-    s_val[threadIdx.x] = best;
-    s_idx[threadIdx.x] = best_i;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(best, off);
+        const uint32_t oi = (uint32_t)__shfl_xor((int)best_i, off);
+        argmax_take(best, best_i, ov, oi);
+    }
+    __shared__ float s_val[kArgmaxThreads / 64];
+    __shared__ uint32_t s_idx[kArgmaxThreads / 64];
+    if (threadIdx.x % 64 == 0) {
+        s_val[threadIdx.x / 64] = best;
+        s_idx[threadIdx.x / 64] = best_i;
+    }
     __syncthreads();
-    for (int off = 128; off > 0; off >>= 1) {
-        if ((int)threadIdx.x < off) {
-            float ov = s_val[threadIdx.x + off];
-            uint32_t oi = s_idx[threadIdx.x + off];
-            float mv = s_val[threadIdx.x];
-            uint32_t mi = s_idx[threadIdx.x];
-            bool take = oi != 0xffffffffu && (mi == 0xffffffffu || ov > mv || (ov == mv && oi < mi));
-            if (take) {
-                s_val[threadIdx.x] = ov;
-                s_idx[threadIdx.x] = oi;
-            }
-        }
-        __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < kArgmaxThreads / 64; ++w) argmax_take(best, best_i, s_val[w], s_idx[w]);
+        out[blockIdx.x] = best_i == 0xffffffffu ? 0 : (int32_t)best_i;
     }
-    if (threadIdx.x == 0) out[blockIdx.x] = s_idx[0] == 0xffffffffu ? 0 : (int32_t)s_idx[0];
 }
 
 __global__ void gather_rows_kernel(const float *__restrict__ table, uint64_t table_rows, uint64_t cols,
@@ -158,7 +171,7 @@ void add_f32(const float *a, const float *b, float *out, uint64_t n, hipStream_t
 }
 void argmax_rows_f32(const float *x, int32_t *out, uint64_t rows, uint64_t cols, hipStream_t s) {
     if (rows == 0) return;
-    argmax_rows_kernel<<<(unsigned)rows, 256, 0, s>>>(x, out, cols);
+    argmax_rows_kernel<<<(unsigned)rows, kArgmaxThreads, 0, s>>>(x, out, cols);
 }
 void gather_rows_f32(const float *table, uint64_t table_rows, uint64_t cols, const int32_t *idx, float *out,
                      uint64_t rows, hipStream_t s) {

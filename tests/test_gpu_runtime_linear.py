@@ -174,6 +174,9 @@ def test_rope_and_elementwise_against_the_oracle():
     assert np.array_equal(got, o.argmax_rows(logits)) and got[3] == 100 and got[4] == 0
     small = np.array([[1.0, 3.0, 3.0, 2.0], [-1.0, -2.0, -0.5, -9.0]], np.float32)
     assert be.download_owned(be.argmax(be.upload(small))).tolist() == [1, 2]
+    for shape in ((7, 4099), (3, 50257), (5, 8192), (2, 3)):             # many ties; odd widths take the scalar loads
+        tied = np.round(rng.randn(shape) * 2).astype(np.float32)
+        assert np.array_equal(be.download_owned(be.argmax(be.upload(tied))), o.argmax_rows(tied)), shape
     table = rng.randn((50, 96))
     idx = np.array([3, 49, 0, 3], dtype=np.int32)
     assert np.array_equal(be.download_owned(be.gather(be.upload(table), be.upload(idx))), table[idx])
