@@ -224,6 +224,235 @@ __global__ void __launch_bounds__(kThreads)
     }
 }
 
+// exclusive prefix sums of one value per thread over the block (wavefront scan, then the wavefront totals
+// through LDS); *total receives the block total.  buf: one slot per wavefront.
+template <typename T>
+__device__ __forceinline__ T block_exclusive_scan_fast(T v, T *buf, T *total) {
+    const int lane = threadIdx.x % 64, w = threadIdx.x / 64;
+    T sc = v;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const T up = __shfl_up(sc, off);
+        if (lane >= off) sc += up;
+    }
+    __syncthreads();                                      // buf may still be read by an earlier scan
+    if (lane == 63) buf[w] = sc;
+    __syncthreads();
+    T before = (T)0, all = (T)0;
+    for (int i = 0; i < kThreads / 64; ++i) {
+        if (i == w) before = all;
+        all += buf[i];
+    }
+    *total = all;
+    return before + sc - v;
+}
+
+// The same sampler for rows of at most 1024 * SEG logits, with the row held in registers: thread t owns the
+// SEG consecutive logits from t * SEG on, loads them once (16 bytes at a time where the row's alignment
+// allows) and keeps first the logits, then their f64 exponentials, then the f32 weights in registers, so the
+// row is read from memory once and every exponential is taken once.  What depends on the index order (which
+// of several logits equal to the k-th largest are kept; the cumulative weights of the draw) goes through one
+// scan of per-thread totals each.
+template <int SEG>
+__global__ void __launch_bounds__(kThreads)
+    sample_rows_reg_kernel(const float *__restrict__ logits, int32_t *__restrict__ tokens, const uint64_t *__restrict__ rng_state,
+                           RowPolicy *__restrict__ policy, uint32_t vocab, int top_k_mode, float temperature, uint32_t top_k) {
+    constexpr int kW = kThreads / 64;
+    __shared__ double s_d[kW];
+    __shared__ uint32_t s_u[kW];
+    __shared__ uint32_t hist[256];
+    __shared__ float s_max[kW];
+    __shared__ uint32_t s_sel[4];
+    __shared__ double s_x;
+    const uint32_t b = blockIdx.x, t = threadIdx.x, lane = t % 64, w = t / 64;
+    const float *row = logits + (uint64_t)b * vocab;
+    const uint32_t base = t * SEG;
+    bool greedy = false;
+    if (policy) {
+        const RowPolicy pr = policy[b];
+        greedy = pr.strategy == 0;
+        top_k_mode = pr.strategy == 2;
+        temperature = pr.temperature;
+        top_k = pr.top_k < vocab ? pr.top_k : vocab;
+    }
+    float v[SEG];
+    const uint32_t n_own = base >= vocab ? 0u : (vocab - base < (uint32_t)SEG ? vocab - base : (uint32_t)SEG);
+    if (vocab % 4 == 0) {                                 // every row starts on a 16-byte boundary, and so does base
+#pragma unroll
+        for (int q = 0; q < SEG / 4; ++q) {
+            float4 x4 = float4{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+            if (base + 4 * q < vocab) x4 = *(const float4 *)(row + base + 4 * q);
+            v[4 * q] = x4.x;
+            v[4 * q + 1] = x4.y;
+            v[4 * q + 2] = x4.z;
+            v[4 * q + 3] = x4.w;
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < SEG; ++j) v[j] = (uint32_t)j < n_own ? row[base + j] : -INFINITY;
+    }
+    float mx = -INFINITY;
+    bool finite = true;
+#pragma unroll
+    for (int j = 0; j < SEG; ++j)
+        if ((uint32_t)j < n_own) {
+            finite = finite && (fabsf(v[j]) <= 3.402823466e38f);
+            mx = fmaxf(mx, v[j]);
+        }
+    if (t < 4) s_sel[t] = t == 0 ? 0xffffffffu : 0u;      // [0] smallest index found, [1] last positive + 1, [2] not finite
+    __syncthreads();
+    if (!finite) atomicOr(&s_sel[2], 1u);
+    mx = wave_max(mx);
+    if (lane == 0) s_max[w] = mx;
+    __syncthreads();
+    if (s_sel[2]) {
+        if (t == 0) tokens[b] = -1;
+        return;
+    }
+    mx = s_max[0];
+#pragma unroll
+    for (int i = 1; i < kW; ++i) mx = fmaxf(mx, s_max[i]);
+    if (greedy) {                                         // first index holding the maximum
+        uint32_t first = 0xffffffffu;
+#pragma unroll
+        for (int j = SEG - 1; j >= 0; --j)
+            if ((uint32_t)j < n_own && v[j] == mx) first = base + j;
+        if (first != 0xffffffffu) atomicMin(&s_sel[0], first);
+        __syncthreads();
+        if (t == 0) tokens[b] = (int32_t)s_sel[0];
+        return;
+    }
+    const double dmax = (double)mx, dt = (double)temperature;
+
+    uint32_t kept = n_own >= 32 ? 0xffffffffu : (1u << n_own) - 1u;      // bit j: logit j of this thread takes part
+    if (top_k_mode) {
+        uint32_t prefix = 0, mask = 0, remaining = top_k;
+        for (int pass = 0; pass < 4; ++pass) {
+            const int shift = 24 - 8 * pass;
+            if (t < 256) hist[t] = 0;
+            __syncthreads();
+#pragma unroll
+            for (int j = 0; j < SEG; ++j) {
+                const uint32_t key = order_key(v[j]);
+                if ((uint32_t)j < n_own && (key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
+            }
+            __syncthreads();
+            {
+                // the highest bin whose count together with all higher bins reaches `remaining`: suffix sums of
+                // the 256 bins over four wavefronts (a one-thread walk down the bins costs more than the pass)
+                const uint32_t c = t < 256 ? hist[t] : 0u;
+                uint32_t sfx = c;
+#pragma unroll
+                for (int off = 1; off < 64; off <<= 1) {
+                    const uint32_t dn = __shfl_down(sfx, off);
+                    if ((int)lane + off < 64) sfx += dn;
+                }
+                if (t < 256 && lane == 0) s_u[w] = sfx;
+                __syncthreads();
+                if (t < 256) {
+                    for (uint32_t i = w + 1; i < 4; ++i) sfx += s_u[i];
+                    const uint32_t above = sfx - c;               // count in the bins above this one
+                    if ((sfx >= remaining && above < remaining) || (t == 0 && sfx < remaining)) {
+                        s_sel[1] = prefix | (t << shift);
+                        s_sel[3] = remaining - above;
+                    }
+                }
+            }
+            __syncthreads();
+            prefix = s_sel[1];
+            remaining = s_sel[3];
+            mask |= 255u << shift;
+            __syncthreads();
+        }
+        if (t == 0) s_sel[1] = 0;
+        const uint32_t thr_key = prefix, keep_equal = remaining;
+        uint32_t eq = 0;
+#pragma unroll
+        for (int j = 0; j < SEG; ++j) eq += ((uint32_t)j < n_own && order_key(v[j]) == thr_key) ? 1u : 0u;
+        uint32_t eq_total;
+        uint32_t rank = block_exclusive_scan_fast<uint32_t>(eq, s_u, &eq_total);
+        uint32_t k2 = 0;
+#pragma unroll
+        for (int j = 0; j < SEG; ++j) {
+            const uint32_t key = order_key(v[j]);
+            bool ok = (uint32_t)j < n_own && key > thr_key;
+            if ((uint32_t)j < n_own && key == thr_key) {
+                ok = rank < keep_equal;
+                ++rank;
+            }
+            k2 |= (ok ? 1u : 0u) << j;
+        }
+        kept = k2;
+    }
+
+    // f64 exponentials of the kept logits and their sum
+    double ex[SEG], part = 0.0;
+#pragma unroll
+    for (int j = 0; j < SEG; ++j) {
+        ex[j] = ((kept >> j) & 1u) ? exp(((double)v[j] - dmax) / dt) : 0.0;
+        part += ex[j];
+        __builtin_amdgcn_sched_barrier(0);                // one exponential at a time: the row fills the registers
+    }
+    const double sum_exp = block_sum<double, kW>(part, s_d);
+    // f32 weights, their f64 sum in index order, the last positive one
+    double wsum = 0.0;
+    uint32_t last_pos = 0;
+#pragma unroll
+    for (int j = 0; j < SEG; ++j) {
+        const float wt = ((kept >> j) & 1u) ? (float)(ex[j] / sum_exp) : 0.0f;
+        v[j] = wt;
+        wsum += (double)wt;
+        if (wt > 0.0f) last_pos = base + j + 1;
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    if (last_pos) atomicMax(&s_sel[1], last_pos);
+    double total;
+    const double before = block_exclusive_scan_fast<double>(wsum, s_d, &total);
+    if (t == 0) {
+        uint64_t bits = 0;
+        if (policy) {
+            uint64_t st = policy[b].rng_state;
+            bits = xorshift64star_next(st);
+            policy[b].rng_state = st;
+        } else {
+            uint64_t st = rng_state[0];
+            for (uint32_t r = 0; r <= b; ++r) bits = xorshift64star_next(st);
+        }
+        s_x = (double)(bits >> 11) / 9007199254740992.0 * total;
+    }
+    __syncthreads();
+    const double x = s_x;
+    {
+        // as in the kernel above: the smallest first-crossing index over all threads is the crossing
+        double acc = before;
+        uint32_t found = 0xffffffffu;
+#pragma unroll
+        for (int j = 0; j < SEG; ++j) {
+            acc += (double)v[j];
+            if (found == 0xffffffffu && v[j] > 0.0f && acc > x) found = base + j;
+        }
+        if (found != 0xffffffffu) atomicMin(&s_sel[0], found);
+    }
+    __syncthreads();
+    if (t == 0) {
+        uint32_t idx = s_sel[0];
+        if (idx == 0xffffffffu) idx = s_sel[1] ? s_sel[1] - 1 : vocab - 1;
+        tokens[b] = (int32_t)idx;
+    }
+}
+
+template <typename... A>
+static void launch_sampler(uint32_t rows, uint32_t vocab, hipStream_t s, A... args) {
+    if (vocab <= kThreads * 8)
+        sample_rows_reg_kernel<8><<<rows, kThreads, 0, s>>>(args...);
+    else if (vocab <= kThreads * 16)
+        sample_rows_reg_kernel<16><<<rows, kThreads, 0, s>>>(args...);
+    else if (vocab <= kThreads * 32)
+        sample_rows_reg_kernel<32><<<rows, kThreads, 0, s>>>(args...);
+    else
+        sample_rows_kernel<<<rows, kThreads, 0, s>>>(args...);
+}
+
 __global__ void advance_rng_kernel(uint64_t *state, uint32_t draws) {
     uint64_t st = state[0];
     for (uint32_t i = 0; i < draws; ++i) (void)xorshift64star_next(st);
@@ -235,13 +464,14 @@ __global__ void advance_rng_kernel(uint64_t *state, uint32_t draws) {
 void sample_rows(const float *logits, int32_t *tokens, uint64_t *rng_state, uint32_t rows, uint32_t vocab, int top_k_mode,
                  float temperature, uint32_t top_k, hipStream_t s) {
     if (rows == 0 || vocab == 0) return;
-    sample_rows_kernel<<<rows, kThreads, 0, s>>>(logits, tokens, rng_state, nullptr, vocab, top_k_mode, temperature, top_k);
+    launch_sampler(rows, vocab, s, logits, tokens, (const uint64_t *)rng_state, (RowPolicy *)nullptr, vocab, top_k_mode,
+                   temperature, top_k);
     advance_rng_kernel<<<1, 1, 0, s>>>(rng_state, rows);
 }
 
 void sample_rows_policy(const float *logits, int32_t *tokens, RowPolicy *policy, uint32_t rows, uint32_t vocab, hipStream_t s) {
     if (rows == 0 || vocab == 0) return;
-    sample_rows_kernel<<<rows, kThreads, 0, s>>>(logits, tokens, nullptr, policy, vocab, 0, 1.0f, 0);
+    launch_sampler(rows, vocab, s, logits, tokens, (const uint64_t *)nullptr, policy, vocab, 0, 1.0f, 0u);
 }
 
 }  // namespace k
