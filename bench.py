@@ -376,6 +376,30 @@ def bench_short_prompts(fa, be, dec, cfg, tables, lengths=(64, 300, 1024), reps=
     return out
 
 
+def bench_single_stream(fa, be, dec, cfg, tables, prompt_len=128, steps=64):
+    """One sequence decoding by itself (graph-replayed steps after a short prompt): the latency floor a
+    speculative or interactive caller sees; dominated by streaming the weights once per token."""
+    lib = fa.capi.lib
+    row = int(np.argmax((tables != U32MAX).sum(axis=1)))
+    tb = np.ascontiguousarray(tables[row:row + 1])
+    lens = np.zeros(1, dtype=np.uint32)
+    prompt = np.random.default_rng(5).integers(0, cfg["vocab"], size=(1, prompt_len)).astype(np.int32)
+    fa.check(lib.fa_decoder_set_sequences(be._ctx, dec, 1, tb.ctypes.data_as(fa.capi.u32p), lens.ctypes.data_as(fa.capi.u32p)))
+    fa.check(lib.fa_decoder_prefill(be._ctx, dec, prompt.ctypes.data_as(fa.capi.i32p), prompt_len))
+    for _ in range(3):
+        fa.check(lib.fa_decoder_step(be._ctx, dec, 1))
+    t = Timer(fa, be)
+    t.start()
+    for _ in range(steps):
+        fa.check(lib.fa_decoder_step(be._ctx, dec, 1))
+    ms = t.stop_ms() / steps
+    weights = cfg["n_layers"] * (cfg["d_model"] * (cfg["n_heads"] + 2 * cfg["n_kv_heads"]) * cfg["head_dim"] +
+                                 cfg["n_heads"] * cfg["head_dim"] * cfg["d_model"] + 3 * cfg["d_model"] * cfg["d_ffn"]) + \
+        cfg["d_model"] * cfg["vocab"]
+    return dict(batch=1, context=prompt_len, ms_per_token=ms, tokens_per_s=1e3 / ms, weight_bytes=weights,
+                weight_stream_gbs=weights / (ms * 1e-3) / 1e9)
+
+
 def bench_continuous_batching(fa, be, dec, dcfg, requests=96, max_active=32):
     """Continuous batching on the resident model: requests with prompts of 64..512 tokens that each generate
     64..192 tokens (greedy, temperature and top-k mixed) join and leave a batch of at most `max_active` rows;
@@ -610,10 +634,13 @@ def main():
             prompt = bench_prompt_prefill(fa, be, dec, cfg, np.ascontiguousarray(tables[order]))
             log("prompt prefill %d x %d tokens: %.1f ms, %.0f tokens/s" %
                 (prompt["batch"], prompt["l_new"], prompt["ms"], prompt["tokens_per_s"]))
-    batching = short = None
+    batching = short = single = None
     if not a.no_extras and not a.no_serving:
         short = bench_short_prompts(fa, be, dec, cfg, tables)
         log("one prompt, batch 1: " + ", ".join("%d tokens %.2f ms" % (r["l_new"], r["ms"]) for r in short))
+        single = bench_single_stream(fa, be, dec, cfg, tables)
+        log("one sequence decoding alone: %.3f ms per token (%.0f tokens/s, weights streamed at %.0f GB/s)" %
+            (single["ms_per_token"], single["tokens_per_s"], single["weight_stream_gbs"]))
         dcfg = fa.capi.DecoderConfig(cfg["n_layers"], cfg["d_model"], cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"],
                                      cfg["d_ffn"], cfg["vocab"], cfg["block_size"], max_blocks, num_blocks, batch,
                                      cfg["rms_eps"], cfg["rope_theta"])
@@ -643,6 +670,7 @@ def main():
         extras["prompt_prefill"] = prompt
     if short is not None:
         extras["prompt_pass_one_request"] = short
+        extras["single_stream_decode"] = single
     if batching is not None:
         extras["continuous_batching"] = batching
     if not a.no_extras:

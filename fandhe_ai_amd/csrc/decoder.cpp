@@ -451,11 +451,14 @@ fa_status fa_decoder_set_sampling(fa_context *ctx, fa_decoder *d, fa_sampling st
     if (strategy == FA_SAMPLE_TOP_K && (top_k == 0 || top_k > d->cfg.vocab))
         return fail(FA_ERR_INVALID_ARGUMENT, "decoder_set_sampling: top_k must be in 1..=vocab");
     if (fa_status s = fa_rng_seed(ctx, d->rng, seed)) return s;
+    // the captured steps hold the choice (not the seed: the generator state is read from device memory)
+    const bool same = !d->per_row && d->strategy == strategy &&
+                      (strategy == FA_SAMPLE_GREEDY || (d->temperature == temperature && d->top_k == (uint32_t)top_k));
     d->strategy = strategy;
     d->temperature = temperature;
     d->top_k = (uint32_t)top_k;
     d->per_row = false;
-    drop_graphs(d);                                     // the captured steps hold the old choice
+    if (!same) drop_graphs(d);
     return FA_OK;
 }
 
