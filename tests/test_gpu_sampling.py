@@ -84,7 +84,7 @@ def test_decoder_steps_with_sampling_follow_the_oracle_generator():
     fa = _fa()
     be = ops()
     m = build_model(seed=4, n_layers=1, d_model=256, n_heads=2, n_kv_heads=1, d_ffn=256, vocab=700, batch=5,
-                    ctxs=[3, 20, 9, 33, 1], steps=8)
+                    ctxs=[3, 20, 9, 33, 1], steps=12)
     dec = GpuDecoder(be, m)
     try:
         for strategy, temperature, k, seed in ((fa.SAMPLE_TOP_K, 1.0, 40, 5), (fa.SAMPLE_TEMPERATURE, 0.9, 0, 0)):
@@ -94,6 +94,17 @@ def test_decoder_steps_with_sampling_follow_the_oracle_generator():
                 dec.step(use_graph=(step > 0))
                 want = os_.sample_step(dec.logits(), strategy, temperature, k or None, ref)
                 assert np.array_equal(dec.tokens(), want), (strategy, step)
+        # the same choice with another seed keeps the captured step and draws from the new generator
+        dec.set_sampling(fa.SAMPLE_TEMPERATURE, 0.9, 0, 77)
+        ref = os_.Generator(77)
+        for step in range(2):
+            dec.step(True)
+            assert np.array_equal(dec.tokens(), os_.sample_step(dec.logits(), fa.SAMPLE_TEMPERATURE, 0.9, None, ref)), step
+        # another temperature re-captures
+        dec.set_sampling(fa.SAMPLE_TEMPERATURE, 1.3, 0, 77)
+        ref = os_.Generator(77)
+        dec.step(True)
+        assert np.array_equal(dec.tokens(), os_.sample_step(dec.logits(), fa.SAMPLE_TEMPERATURE, 1.3, None, ref))
         dec.set_sampling(fa.SAMPLE_GREEDY)
         dec.step(False)
         assert np.array_equal(dec.tokens(), o.argmax_rows(dec.logits()))
