@@ -15,6 +15,7 @@ tensors (already quantized checkpoints), which the reference rejects (tests/st_t
 projections per output channel there.
 """
 import json
+import os
 import struct
 
 import numpy as np
@@ -133,7 +134,7 @@ def _parse_layout(buf):
         if dtype not in _WIRE_WIDTH_BITS:
             raise SafetensorsFormat("InvalidHeaderDeserialization: unknown dtype %r" % dtype)
         entries.append((name, dtype, shape, begin, end))
-    entries.sort(key=lambda e: (e[3], e[0]))
+    entries.sort(key=lambda e: (e[3], e[4], e[0]))          # by byte range, as the wire format validates it
     data_len = len(buf) - 8 - n
     cursor = 0
     for name, dtype, shape, begin, end in entries:
@@ -230,6 +231,95 @@ def require_keys(tensors, keys):
 
 
 require_keys_typed = require_keys
+
+
+# ---- saving (crates/onnx-interop/src/st_save.rs) -----------------------------------------------------------
+
+class SaveError(Exception):
+    """st_save.rs:77-81"""
+
+
+# the order in which the wire format's serializer lays tensors out: wider alignment first, then by name
+_DTYPE_RANK = {n: i for i, n in enumerate(("BOOL", "U8", "I8", "F8_E5M2", "F8_E4M3", "I16", "U16", "F16", "BF16", "I32",
+                                           "U32", "F32", "F64", "I64", "U64"))}
+_NUMPY_TAGS = {np.dtype(np.float32): "F32", np.dtype(np.float16): "F16", np.dtype(np.float64): "F64",
+               np.dtype(np.int32): "I32", np.dtype(np.int64): "I64", np.dtype(np.bool_): "BOOL"}
+
+
+def _as_typed(key, t):
+    if isinstance(t, TypedTensor):
+        if t.dtype not in _REFERENCE_DTYPES and t.dtype not in _QUANTIZED_DTYPES:
+            raise SaveError("%s: dtype %s cannot be written" % (key, t.dtype))
+        return t
+    a = np.asarray(t)
+    tag = _NUMPY_TAGS.get(a.dtype)
+    if tag is None:
+        raise SaveError("%s: numpy dtype %s has no safetensors tag here (wrap bf16 bits in a TypedTensor)" % (key, a.dtype))
+    return TypedTensor(tag, a.shape, a)
+
+
+def save_safetensors_typed_to_bytes(tensors, metadata=None):
+    """name -> TypedTensor (or a numpy array of a dtype the loader returns) -> file bytes, bit-identical to what
+    the wire format's own serializer writes for the same tensors (st_save.rs:246-288 hands the sorted tensors
+    to it): compact JSON header padded with spaces to a multiple of 8, tensors ordered by descending element
+    alignment and then by name, data little-endian.  Nothing is transposed or renamed.  The output is
+    deterministic.  metadata: optional str -> str map, written in sorted key order."""
+    typed = {k: _as_typed(k, t) for k, t in tensors.items()}
+    order = sorted(typed, key=lambda k: (-_DTYPE_RANK[typed[k].dtype], k))
+    header, chunks, off = {}, [], 0
+    if metadata:
+        if not all(isinstance(k, str) and isinstance(v, str) for k, v in metadata.items()):
+            raise SaveError("metadata must map strings to strings")
+        header["__metadata__"] = {k: metadata[k] for k in sorted(metadata)}
+    for k in order:
+        t = typed[k]
+        if k == "__metadata__":
+            raise SaveError("__metadata__ is not a tensor name")
+        width, npdt = (_REFERENCE_DTYPES.get(t.dtype) or _QUANTIZED_DTYPES[t.dtype])
+        data = np.ascontiguousarray(t.data)
+        if t.dtype == "BOOL":
+            data = data.astype(np.uint8)
+        if data.dtype.itemsize != width or int(np.prod(t.shape, dtype=np.int64)) != data.size:
+            raise SaveError("%s: %s data of shape %s does not hold %d-byte elements of shape %s"
+                            % (k, data.dtype, data.shape, width, t.shape))
+        raw = data.astype(data.dtype.newbyteorder("<"), copy=False).tobytes()
+        header[k] = {"dtype": t.dtype, "shape": [int(d) for d in t.shape], "data_offsets": [off, off + len(raw)]}
+        chunks.append(raw)
+        off += len(raw)
+    h = json.dumps(header, separators=(",", ":"), ensure_ascii=False).encode("utf-8")
+    h += b" " * (-len(h) % 8)
+    return struct.pack("<Q", len(h)) + h + b"".join(chunks)
+
+
+def save_safetensors_typed(path, tensors):
+    """Writes through a temporary file in the same directory and a rename (st_save.rs:290-296): the final
+    path never shows a partial file."""
+    data = save_safetensors_typed_to_bytes(tensors)
+    directory = os.path.dirname(os.path.abspath(path))
+    tmp = os.path.join(directory, ".%s.%d.tmp" % (os.path.basename(path), os.getpid()))
+    try:
+        with open(tmp, "wb") as f:
+            f.write(data)
+        os.replace(tmp, path)
+    except OSError as e:
+        try:
+            os.unlink(tmp)
+        except OSError:
+            pass
+        raise SaveError("io: %s" % e)
+
+
+def save_safetensors_f32_to_bytes(tensors):
+    """st_save.rs:118-190: float32 only."""
+    for k, a in tensors.items():
+        if np.asarray(a).dtype != np.float32:
+            raise SaveError("%s: not float32" % k)
+    return save_safetensors_typed_to_bytes(tensors)
+
+
+def save_safetensors_f32(path, tensors):
+    save_safetensors_f32_to_bytes(tensors)
+    save_safetensors_typed(path, tensors)
 
 
 class DeviceParamStore:

@@ -144,3 +144,47 @@ def test_llama_layout_transposes_explicitly_and_lists_every_missing_key():
     with pytest.raises(st.MissingKeys) as e:
         st.llama_decoder_tensors(typed, 1)
     assert sorted(e.value.keys) == sorted([p + "mlp.up_proj.weight", "model.norm.weight"])
+
+
+def test_writer_is_bit_identical_to_the_wire_formats_own_serializer_and_round_trips(tmp_path):
+    # st_save.rs hands its sorted tensors to the safetensors serializer; the library's writer is that serializer
+    rng = np.random.default_rng(3)
+    mixes = [
+        {"b": rng.standard_normal((2, 2)).astype(np.float32), "a": rng.integers(-5, 5, 3).astype(np.int64),
+         "c": np.array([True, False, True]), "d": rng.standard_normal(1).astype(np.float16),
+         "e": np.zeros((0, 3), np.float64), "aa": np.array([7], np.int32), "s": np.array(1.5, np.float32)},
+        {"only": rng.standard_normal((5, 7, 3)).astype(np.float32)},
+        {"w.%d" % i: rng.standard_normal((i + 1, 4)).astype(np.float32) for i in range(12)},
+        {},
+    ]
+    for t in mixes:
+        mine = st.save_safetensors_typed_to_bytes(t)
+        assert mine == st_lib_save(t)
+        assert mine == st.save_safetensors_typed_to_bytes(dict(reversed(list(t.items()))))       # deterministic
+        back = st.load_safetensors_typed_from_bytes(mine)
+        assert sorted(back) == sorted(t)
+        for k, a in t.items():
+            assert back[k].shape == a.shape and back[k].data.tobytes() == a.tobytes()
+        assert st.save_safetensors_typed_to_bytes(back) == mine                                 # save -> load -> save
+    # bf16 bits and special values survive (st_roundtrip.rs)
+    special = np.array([0x7FC00001, 0x80000000, 0x00000001, 0x7F800000, 0xFF800000], np.uint32).view(np.float32)
+    bf = st.TypedTensor("BF16", (3,), np.array([0x3F80, 0x7FC1, 0x8000], np.uint16))
+    data = st.save_safetensors_typed_to_bytes({"x": special, "h": bf})
+    back = st.load_safetensors_typed_from_bytes(data)
+    assert back["x"].data.view(np.uint32).tolist() == special.view(np.uint32).tolist()
+    assert back["h"].dtype == "BF16" and back["h"].data.tolist() == [0x3F80, 0x7FC1, 0x8000]
+    # files: through a temporary name; the float32 entry points refuse anything else
+    path = str(tmp_path / "ck.safetensors")
+    st.save_safetensors_f32(path, {"x": special})
+    assert st.load_safetensors_f32(path)["x"].view(np.uint32).tolist() == special.view(np.uint32).tolist()
+    assert [p.name for p in tmp_path.iterdir()] == ["ck.safetensors"]
+    with pytest.raises(st.SaveError):
+        st.save_safetensors_f32_to_bytes({"i": np.array([1], np.int32)})
+    with pytest.raises(st.SaveError):
+        st.save_safetensors_typed_to_bytes({"u": np.array([1], np.uint16)})
+    with pytest.raises(st.SaveError):
+        st.save_safetensors_typed_to_bytes({"t": st.TypedTensor("F32", (3,), np.zeros(2, np.float32))})
+    with pytest.raises(st.SaveError):
+        st.save_safetensors_typed(str(tmp_path / "no" / "such" / "dir.safetensors"), {"x": special})
+    meta = st.save_safetensors_typed_to_bytes({"x": special}, metadata={"format": "pt"})
+    assert meta == st_lib_save({"x": special}, metadata={"format": "pt"})
