@@ -362,3 +362,41 @@ def test_speculative_argument_errors():
         generate_speculative(T(), D(), [1], cfg(4, SamplingStrategy.TopK(2), 0), 2)
     with pytest.raises(InvalidArgument):                   # a sequence longer than the page table of one model
         generate_speculative(T(), D(max_blocks_per_seq=1), [1], cfg(40, greedy, 0), 2)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_arrivals_conserve_pages_and_match_single_generation(seed):
+    """Requests of random length and strategy arrive at random iterations into a small decoder (few rows, few
+    pages): whatever the interleaving, every request ends with exactly the tokens it gets alone, rows and pages
+    never exceed their limits, and every page is back at the end."""
+    rng = np.random.default_rng(100 + seed)
+    S = SamplingStrategy
+    max_active = int(rng.integers(1, 4))
+    m = ToyDecoder(max_batch=3, num_blocks=int(rng.integers(3, 7)), max_blocks_per_seq=3)
+    s = BatchScheduler(m, SchedulerLimits(max_active, 64, 48))
+    todo = []
+    for _ in range(int(rng.integers(5, 14))):
+        plen = int(rng.integers(1, 20))
+        max_length = plen + int(rng.integers(0, 28))
+        strategy = (S.Greedy(), S.Temperature(float(rng.uniform(0.3, 2.0))), S.TopK(int(rng.integers(1, VOCAB + 1))))[int(rng.integers(0, 3))]
+        c = cfg(max_length, strategy, int(rng.integers(0, 2 ** 63)))
+        if strategy.kind == fa.scheduler.TOP_K and rng.random() < 0.5:
+            c = c.with_temperature(float(rng.uniform(0.3, 2.0)))
+        todo.append((int(rng.integers(0, 25)), rng.integers(0, VOCAB, plen).astype(np.int32), c))
+    todo.sort(key=lambda e: e[0])
+    submitted, done = {}, {}
+    for it in range(600):
+        while todo and todo[0][0] <= it:
+            _, prompt, c = todo.pop(0)
+            submitted[s.submit(prompt, c)] = (prompt, c)
+        if not todo and s.active_len() == 0 and s.queued_len() == 0:
+            break
+        s.step()
+        assert s.active_len() <= max_active and 0 <= s.free_pages() <= m.cfg.num_blocks
+        used = [p for a in s._active for p in a.pages]
+        assert len(used) == len(set(used)) == m.cfg.num_blocks - s.free_pages()          # no page is shared or lost
+        done.update(dict(s.take_finished()))
+    assert s.take_failed() == [] and sorted(done) == sorted(submitted)
+    assert s.free_pages() == m.cfg.num_blocks
+    for rid, (prompt, c) in submitted.items():
+        assert done[rid].tolist() == generate(ToyDecoder(), prompt, c).tolist(), rid
