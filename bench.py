@@ -393,11 +393,27 @@ def bench_single_stream(fa, be, dec, cfg, tables, prompt_len=128, steps=64):
     for _ in range(steps):
         fa.check(lib.fa_decoder_step(be._ctx, dec, 1))
     ms = t.stop_ms() / steps
+    # speculative verification of a pending token and four drafts: one step whose five rows are five
+    # consecutive positions of the one sequence (same block table, lengths ctx .. ctx + 4)
+    ctx0 = prompt_len + 3 + steps
+    rows = 5
+    tb5 = np.ascontiguousarray(np.repeat(tb, rows, axis=0))
+    lens5 = np.arange(ctx0, ctx0 + rows, dtype=np.uint32)
+    toks5 = np.random.default_rng(6).integers(0, cfg["vocab"], size=rows).astype(np.int32)
+    verify_ms = None
+    for rep in range(3):
+        fa.check(lib.fa_decoder_set_sequences(be._ctx, dec, rows, tb5.ctypes.data_as(fa.capi.u32p),
+                                              lens5.ctypes.data_as(fa.capi.u32p)))
+        fa.check(lib.fa_decoder_set_tokens(be._ctx, dec, toks5.ctypes.data_as(fa.capi.i32p)))
+        t.start()
+        fa.check(lib.fa_decoder_step(be._ctx, dec, 1))
+        one = t.stop_ms()
+        verify_ms = one if rep == 1 else (min(verify_ms, one) if rep > 1 else None)
     weights = cfg["n_layers"] * (cfg["d_model"] * (cfg["n_heads"] + 2 * cfg["n_kv_heads"]) * cfg["head_dim"] +
                                  cfg["n_heads"] * cfg["head_dim"] * cfg["d_model"] + 3 * cfg["d_model"] * cfg["d_ffn"]) + \
         cfg["d_model"] * cfg["vocab"]
     return dict(batch=1, context=prompt_len, ms_per_token=ms, tokens_per_s=1e3 / ms, weight_bytes=weights,
-                weight_stream_gbs=weights / (ms * 1e-3) / 1e9)
+                weight_stream_gbs=weights / (ms * 1e-3) / 1e9, verify_5_positions_ms=verify_ms)
 
 
 def bench_continuous_batching(fa, be, dec, dcfg, requests=96, max_active=32):
@@ -639,8 +655,9 @@ def main():
         short = bench_short_prompts(fa, be, dec, cfg, tables)
         log("one prompt, batch 1: " + ", ".join("%d tokens %.2f ms" % (r["l_new"], r["ms"]) for r in short))
         single = bench_single_stream(fa, be, dec, cfg, tables)
-        log("one sequence decoding alone: %.3f ms per token (%.0f tokens/s, weights streamed at %.0f GB/s)" %
-            (single["ms_per_token"], single["tokens_per_s"], single["weight_stream_gbs"]))
+        log("one sequence decoding alone: %.3f ms per token (%.0f tokens/s, weights streamed at %.0f GB/s); "
+            "verifying 5 positions in one step: %.3f ms" %
+            (single["ms_per_token"], single["tokens_per_s"], single["weight_stream_gbs"], single["verify_5_positions_ms"]))
         dcfg = fa.capi.DecoderConfig(cfg["n_layers"], cfg["d_model"], cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"],
                                      cfg["d_ffn"], cfg["vocab"], cfg["block_size"], max_blocks, num_blocks, batch,
                                      cfg["rms_eps"], cfg["rope_theta"])

@@ -191,9 +191,13 @@ def generate_speculative(target, draft, input_ids, config, k):
     disagreement (or after the last draft) is appended.  Both caches are then cut back to the accepted
     length with ``Decoder.rewind``: paged rows past a sequence's length are dead, so nothing is replayed
     (the reference restores a snapshot and replays the accepted tokens, kv_rewind.rs:157-215).  One
-    sequence per call, as in the reference.  The output equals ``generate(target, ...)`` wherever the
-    target's greedy choice is decisive (the verification pass runs prompt-shape kernels, a decode step
-    the decode-shape ones; int32 accumulators are identical, attention sums are associated differently).
+    sequence per call, as in the reference.  When the pending token and the drafts fit the decoder's rows
+    (``k + 1 <= min(32, max_batch)``) the verification is one decode step whose rows are the k + 1 positions
+    of the one sequence (the same block table in every row, lengths ctx, ctx + 1, ...: every row appends its
+    own position and attends to its own prefix), which costs about what a single decode step costs; longer
+    look-aheads take the prompt-shape verification pass.  The output equals ``generate(target, ...)``
+    wherever the target's greedy choice is decisive (int32 accumulators are identical in every form,
+    attention sums are associated differently when the rows change).
     Returns (tokens, rounds, accepted drafts)."""
     config.validate()
     if not isinstance(k, int) or k < 1:
@@ -212,6 +216,8 @@ def generate_speculative(target, draft, input_ids, config, k):
                           "models' probabilities on the host)")
     row = [int(t) for t in ids[0]]
     rounds = accepted = 0
+    by_step = k + 1 <= min(32, target.cfg.max_batch)
+    target_table = None
     if max_length > prompt_len:
         if target.cfg.vocab != draft.cfg.vocab:
             raise InvalidArgument("generate_speculative: the models disagree on the vocabulary (%d, %d)" % (draft.cfg.vocab, target.cfg.vocab))
@@ -225,6 +231,8 @@ def generate_speculative(target, draft, input_ids, config, k):
             dec.set_sequences(table, np.zeros(1, np.uint32))
             dec.set_sampling(GREEDY)
             dec.prefill(ids.astype(np.int32))
+            if dec is target:
+                target_table = table
         row.append(int(target.tokens()[0]))
         while len(row) < max_length:
             cur, last = len(row), row[-1]
@@ -241,7 +249,16 @@ def generate_speculative(target, draft, input_ids, config, k):
                 draft.step()
                 x = int(draft.tokens()[0])
                 drafts.append(x)
-            picked = target.verify(np.array([[last] + drafts], dtype=np.int32))[0]
+            if by_step:
+                n = k_eff + 1
+                target.set_sequences(np.repeat(target_table, n, axis=0), np.arange(cur - 1, cur - 1 + n, dtype=np.uint32))
+                target.set_tokens([last] + drafts)
+                target.step()
+                picked = target.tokens()
+                if (picked < 0).any():
+                    raise InvalidArgument("generate_speculative: logits hold non-finite values")
+            else:
+                picked = target.verify(np.array([[last] + drafts], dtype=np.int32))[0]
             n_acc = 0
             while n_acc < k_eff and drafts[n_acc] == picked[n_acc]:
                 n_acc += 1
@@ -252,7 +269,10 @@ def generate_speculative(target, draft, input_ids, config, k):
             if len(row) >= max_length:
                 break
             keep = cur + n_acc                             # tokens before the new pending one
-            target.rewind([keep])
+            if by_step:
+                target.set_sequences(target_table, np.array([keep], dtype=np.uint32))
+            else:
+                target.rewind([keep])
             if n_acc == k_eff:
                 draft.set_tokens([x])                      # the draft never consumed its own last token
                 draft.step()

@@ -227,14 +227,15 @@ def test_cached_step_graphs_survive_batch_changes_and_workspace_growth():
     dec.close()
 
 
-def test_speculative_generation_equals_the_target_generating_alone():
+@pytest.mark.parametrize("rows", [1, 8], ids=["verify-by-prompt-pass", "verify-by-decode-step"])
+def test_speculative_generation_equals_the_target_generating_alone(rows):
     """Greedy speculative decoding with (a) a draft that is the target's twin and (b) a different, smaller
     draft: the tokens must be the target's own greedy tokens up to the first position where the target's
     two best logits are closer than the chained-step bar allows to tell apart (verification runs the
     prompt-shape kernels, plain generation the decode-shape ones)."""
     import fandhe_ai_amd as fa
     from fandhe_ai_amd.scheduler import SamplingStrategy, generate, generate_speculative
-    geometry = dict(max_blocks_per_seq=8, num_blocks=8, max_batch=1)
+    geometry = dict(max_blocks_per_seq=8, num_blocks=8, max_batch=rows)
     target = _recording(_decoder(**geometry))
     twin = _decoder(**geometry)
     other_ckpt = st_save(_checkpoint(77, 1, D, HEADS, KV, F, VOCAB))
@@ -248,7 +249,7 @@ def test_speculative_generation_equals_the_target_generating_alone():
         target.trace = []
         want = generate(target, prompt, cfg)
         margins = []
-        for _, _, logits, _ in target.trace:
+        for _, _, logits, _ in list(target.trace):
             top2 = np.sort(logits)[-2:]
             margins.append(float(top2[1] - top2[0]) / float(logits.max() - logits.min()))
         assert len(margins) == max_length - plen
