@@ -34,6 +34,7 @@ MFMA_PEAK_TOPS = 5000.0          # dense int8 and fp8 on MI355X
 # row-copy kernel of known size; the figures are in profiles/decode_stream_kernel_config5_pmc.txt).
 ATTENTION_TRAFFIC_BYTES = 627583562
 U32MAX = 0xFFFFFFFF
+SERVING_ROWS = 64          # rows of the continuous-batching run (the decoder's limit)
 
 MODEL = dict(n_layers=32, d_model=4096, n_heads=32, n_kv_heads=8, head_dim=128, d_ffn=14336, vocab=32000,
              block_size=16, rms_eps=1e-5, rope_theta=500000.0)
@@ -104,12 +105,12 @@ def make_tables(rng, ctxs, extra_tokens, bs, num_blocks=None):
 
 
 # ------------------------------------------------------------------ full step
-def build_decoder(fa, be, cfg, batch, ctxs, steps_total, seed=0):
+def build_decoder(fa, be, cfg, batch, ctxs, steps_total, seed=0, max_batch=None):
     lib = fa.capi.lib
     rng = np.random.default_rng(seed)
     tables, max_blocks, num_blocks = make_tables(rng, ctxs, steps_total + 1, cfg["block_size"])
     dcfg = fa.capi.DecoderConfig(cfg["n_layers"], cfg["d_model"], cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"],
-                                 cfg["d_ffn"], cfg["vocab"], cfg["block_size"], max_blocks, num_blocks, batch,
+                                 cfg["d_ffn"], cfg["vocab"], cfg["block_size"], max_blocks, num_blocks, max_batch or batch,
                                  cfg["rms_eps"], cfg["rope_theta"])
     dec = C.c_void_p()
     fa.check(lib.fa_decoder_create(be._ctx, C.byref(dcfg), C.byref(dec)))
@@ -616,7 +617,9 @@ def main():
         be.close()
         return
     t0 = time.time()
-    dec, keep, tables, max_blocks, num_blocks = build_decoder(fa, be, cfg, batch, ctxs, a.steps + a.warmup)
+    # rows for twice the benchmark's batch: the serving run below fills them; the timed steps use `batch`
+    dec, keep, tables, max_blocks, num_blocks = build_decoder(fa, be, cfg, batch, ctxs, a.steps + a.warmup,
+                                                              max_batch=SERVING_ROWS)
     log("model resident in %.1f s; sum ctx = %d" % (time.time() - t0, sum(ctxs)))
 
     use_graph = 0 if a.no_graph else 1
@@ -659,9 +662,9 @@ def main():
             "verifying 5 positions in one step: %.3f ms" %
             (single["ms_per_token"], single["tokens_per_s"], single["weight_stream_gbs"], single["verify_5_positions_ms"]))
         dcfg = fa.capi.DecoderConfig(cfg["n_layers"], cfg["d_model"], cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"],
-                                     cfg["d_ffn"], cfg["vocab"], cfg["block_size"], max_blocks, num_blocks, batch,
+                                     cfg["d_ffn"], cfg["vocab"], cfg["block_size"], max_blocks, num_blocks, SERVING_ROWS,
                                      cfg["rms_eps"], cfg["rope_theta"])
-        batching = bench_continuous_batching(fa, be, dec, dcfg, max_active=batch)
+        batching = bench_continuous_batching(fa, be, dec, dcfg, requests=3 * SERVING_ROWS, max_active=SERVING_ROWS)
         log("continuous batching: %d requests, %d generated tokens in %.2f s -> %.0f generated tokens/s "
             "(mean %.1f active rows)" % (batching["requests"], batching["generated_tokens"], batching["seconds"],
                                          batching["generated_tokens_per_s"], batching["mean_active_rows"]))

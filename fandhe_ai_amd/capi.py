@@ -138,6 +138,7 @@ SIGNATURES = {
     "fa_sample_rows_per_row": (C.c_int32, [ctx_p, buf_p, u64, u64, buf_p, buf_p]),
     "fa_decoder_set_row_sampling": (C.c_int32, [ctx_p, C.c_void_p, C.POINTER(RowSampling)]),
     "fa_decoder_read_row_sampling": (C.c_int32, [ctx_p, C.c_void_p, C.POINTER(RowSampling)]),
+    "fa_decoder_prefill_padded": (C.c_int32, [ctx_p, C.c_void_p, i32p, C.c_uint32, u32p]),
     "fa_decoder_verify": (C.c_int32, [ctx_p, C.c_void_p, i32p, C.c_uint32, i32p, f32p]),
     "fa_decoder_rewind": (C.c_int32, [ctx_p, C.c_void_p, u32p]),
     "fa_decoder_prefill": (C.c_int32, [ctx_p, C.c_void_p, i32p, C.c_uint32]),

@@ -297,7 +297,7 @@ fa_status fa_linear_w8a8(fa_context *ctx, const fa_buffer *x, uint64_t m, const 
     ep.acc_out = acc_out ? (int32_t *)acc_out->ptr : nullptr;
     ep.out = out->ptr;
     ep.out_bf16 = out->dtype == FA_BF16;
-    if (m <= 32) {
+    if (m <= 64) {
         uint64_t m_pad = round_up(m, 16);
         if (fa_status s = xq.get(m_pad * qw->k_pad)) return s;
         k::quantize_rows_i8(x->ptr, x->dtype == FA_BF16, nullptr, (int8_t *)xq.ptr, (float *)sx.ptr, m, m_pad, qw->k,
@@ -305,7 +305,7 @@ fa_status fa_linear_w8a8(fa_context *ctx, const fa_buffer *x, uint64_t m, const 
         k::linear_w8a8_skinny((const int8_t *)xq.ptr, (const int8_t *)qw->codes->ptr, m, qw->n, qw->n_pad, qw->k_pad,
                               ep, ctx->props.multiProcessorCount, ctx->stream);
     } else {
-        if (qw->k != qw->k_pad) return fail(FA_ERR_UNSUPPORTED, "linear_w8a8: m > 32 needs k to be a multiple of 64");
+        if (qw->k != qw->k_pad) return fail(FA_ERR_UNSUPPORTED, "linear_w8a8: m > 64 needs k to be a multiple of 64");
         if (fa_status s = xq.get(mk)) return s;
         k::quantize_rows_i8(x->ptr, x->dtype == FA_BF16, (int8_t *)xq.ptr, nullptr, (float *)sx.ptr, m, m, qw->k,
                             qw->k_pad, ctx->stream);

@@ -226,13 +226,15 @@ struct PrefillBuffers {
     Temp tok, h, xq, sx, qkv, q_bf, attn, gu, slots, cos_sin, last_rows, splitk;
     // verification only: logits and greedy picks of every row
     Temp all_logits, all_picked;
+    // padded pass only: the true prompt length of every row
+    Temp row_lens;
     explicit PrefillBuffers(fa_context *c)
         : tok(c), h(c), xq(c), sx(c), qkv(c), q_bf(c), attn(c), gu(c), slots(c), cos_sin(c), last_rows(c), splitk(c),
-          all_logits(c), all_picked(c) {}
+          all_logits(c), all_picked(c), row_lens(c) {}
 };
 
 fa_status enqueue_prefill_chunk(fa_context *ctx, fa_decoder *d, PrefillBuffers &t, uint32_t lc, bool last_chunk,
-                                bool every_row = false) {
+                                bool every_row = false, bool padded = false) {
     const fa_decoder_config &c = d->cfg;
     const uint32_t B = d->batch;
     const uint64_t M = (uint64_t)B * lc;
@@ -245,7 +247,8 @@ fa_status enqueue_prefill_chunk(fa_context *ctx, fa_decoder *d, PrefillBuffers &
     k::prefill_prepare((const uint32_t *)d->tables->ptr, (const uint32_t *)d->seq_lens->ptr, t.slots.as<uint32_t>(),
                        t.cos_sin.as<float>(), B, lc, c.block_size, c.max_blocks_per_seq, c.num_blocks, c.head_dim,
                        c.rope_theta, s);
-    k::advance_seq_lens((uint32_t *)d->seq_lens->ptr, t.last_rows.as<int32_t>(), B, lc, s);
+    k::advance_seq_lens((uint32_t *)d->seq_lens->ptr, t.last_rows.as<int32_t>(), B, lc,
+                        padded ? t.row_lens.as<uint32_t>() : nullptr, s);
     k::gather_rows_f32((const float *)d->embed->ptr, V, D, t.tok.as<int32_t>(), t.h.as<float>(), M, s);
 
     k::PagedShape ps;
@@ -294,6 +297,7 @@ fa_status enqueue_prefill_chunk(fa_context *ctx, fa_decoder *d, PrefillBuffers &
         k::swiglu_quantize_rows_i8(t.gu.as<float>(), t.xq.as<int8_t>(), t.sx.as<float>(), M, F, s);
         gemm(L.wdown, t.h.as<float>(), t.h.as<float>());
     }
+    if (padded) k::trim_seq_lens((uint32_t *)d->seq_lens->ptr, t.row_lens.as<uint32_t>(), B, lc, s);
     if (every_row) {
         // verification: the head over every row of the chunk (row b * lc + t is token t of sequence b)
         k::rmsnorm_quantize_rows_i8(t.h.as<float>(), (const float *)d->final_norm->ptr, c.rms_eps, t.xq.as<int8_t>(),
@@ -341,7 +345,7 @@ fa_status fa_decoder_create(fa_context *ctx, const fa_decoder_config *cfg, fa_de
     if (c.d_model % 64 != 0 || c.d_ffn % 64 != 0)
         return fail(FA_ERR_UNSUPPORTED, "decoder_create: d_model and d_ffn must be multiples of 64");
     if (c.d_model > 16384) return fail(FA_ERR_UNSUPPORTED, "decoder_create: d_model above 16384");
-    if (c.max_batch > 32) return fail(FA_ERR_UNSUPPORTED, "decoder_create: at most 32 sequences per step");
+    if (c.max_batch > 64) return fail(FA_ERR_UNSUPPORTED, "decoder_create: at most 64 sequences per step");
     if (!std::isfinite(c.rms_eps) || c.rms_eps < 0.0f) return fail(FA_ERR_INVALID_ARGUMENT, "decoder_create: bad rms_eps");
     if (!(c.rope_theta > 0.0)) return fail(FA_ERR_INVALID_ARGUMENT, "decoder_create: bad rope_theta");
     fa_paged_layout layout{c.num_blocks, c.block_size, (uint64_t)c.n_kv_heads * c.head_dim};
@@ -592,8 +596,8 @@ fa_status fa_decoder_step(fa_context *ctx, fa_decoder *d, int32_t use_graph) {
 }
 
 static fa_status prefill_impl(fa_context *ctx, fa_decoder *d, const int32_t *tokens, uint32_t l_new, int32_t *picked,
-                              float *logits) {
-    const bool verify = picked != nullptr;
+                              float *logits, const uint32_t *row_lens = nullptr) {
+    const bool verify = picked != nullptr, padded = row_lens != nullptr;
     if (fa_status s = check_ctx(ctx)) return s;
     if (fa_status s = check_dec(d)) return s;
     if (d->ctx != ctx) return fail(FA_ERR_DEVICE_MISMATCH, "decoder_prefill: decoder belongs to another context");
@@ -610,7 +614,12 @@ static fa_status prefill_impl(fa_context *ctx, fa_decoder *d, const int32_t *tok
             return fail(FA_ERR_INVALID_ARGUMENT, "decoder_prefill: token id outside the vocabulary");
     // every position the prompt writes must have a valid page
     for (uint32_t b = 0; b < B; ++b) {
-        const uint64_t end = (uint64_t)d->host_lens[b] + l_new;
+        if (padded && (row_lens[b] == 0 || row_lens[b] > l_new))
+            return fail(FA_ERR_INVALID_ARGUMENT, "decoder_prefill: row " + std::to_string(b) + " has a length outside 1..=l_max");
+        // the padding needs no pages, but its positions must stay inside the row of the block table
+        if ((uint64_t)d->host_lens[b] + l_new > (uint64_t)c.max_blocks_per_seq * c.block_size)
+            return fail(FA_ERR_INVALID_ARGUMENT, "paged_kv: row " + std::to_string(b) + " has no room for the prompt");
+        const uint64_t end = (uint64_t)d->host_lens[b] + (padded ? row_lens[b] : l_new);
         const uint64_t need = (end + c.block_size - 1) / c.block_size;
         if (need > c.max_blocks_per_seq)
             return fail(FA_ERR_INVALID_ARGUMENT, "paged_kv: row " + std::to_string(b) + " has no room for the prompt");
@@ -621,8 +630,8 @@ static fa_status prefill_impl(fa_context *ctx, fa_decoder *d, const int32_t *tok
     }
     // chunks of at most kRows rows per pass bound the activation memory (the widest is [rows, 2 d_ffn] f32)
     constexpr uint64_t kRows = 4096;
-    if (verify && (uint64_t)B * l_new > kRows)
-        return fail(FA_ERR_INVALID_ARGUMENT, "decoder_verify: at most 4096 rows (batch x tokens) per call");
+    if ((verify || padded) && (uint64_t)B * l_new > kRows)
+        return fail(FA_ERR_INVALID_ARGUMENT, "decoder: at most 4096 rows (batch x tokens) per verification or padded prompt pass");
     const uint32_t lc_max = (uint32_t)std::max<uint64_t>(1, std::min<uint64_t>(l_new, kRows / B));
     const uint64_t M = (uint64_t)B * lc_max;
     const uint64_t D = c.d_model, F = c.d_ffn, EQ = (uint64_t)c.n_heads * c.head_dim, EKV = (uint64_t)c.n_kv_heads * c.head_dim;
@@ -658,6 +667,7 @@ static fa_status prefill_impl(fa_context *ctx, fa_decoder *d, const int32_t *tok
         get(t.all_logits, M * c.vocab * 4);
         get(t.all_picked, M * 4);
     }
+    if (padded) get(t.row_lens, (uint64_t)B * 4);
     if (st != FA_OK) return st;
     k::PagedShape ps{};
     ps.batch = B;
@@ -681,8 +691,13 @@ static fa_status prefill_impl(fa_context *ctx, fa_decoder *d, const int32_t *tok
         hipError_t e = hipMemcpyAsync(t.tok.ptr, stage.data(), (uint64_t)B * lc * 4, hipMemcpyHostToDevice, ctx->stream);
         if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
         if (e != hipSuccess) return hip_fail(ctx, e, "prompt token upload", FA_ERR_TRANSFER_FAILED);
-        if (fa_status s = enqueue_prefill_chunk(ctx, d, t, lc, t0 + lc == l_new, verify)) return s;
-        for (auto &len : d->host_lens) len += lc;
+        if (padded) {
+            e = hipMemcpyAsync(t.row_lens.ptr, row_lens, (uint64_t)B * 4, hipMemcpyHostToDevice, ctx->stream);
+            if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+            if (e != hipSuccess) return hip_fail(ctx, e, "prompt lengths upload", FA_ERR_TRANSFER_FAILED);
+        }
+        if (fa_status s = enqueue_prefill_chunk(ctx, d, t, lc, t0 + lc == l_new, verify, padded)) return s;
+        for (uint32_t b = 0; b < B; ++b) d->host_lens[b] += padded ? row_lens[b] : lc;
     }
     if (verify) {
         // one chunk; the buffers go back to the pool when this call returns, so the copies finish here
@@ -697,6 +712,12 @@ static fa_status prefill_impl(fa_context *ctx, fa_decoder *d, const int32_t *tok
 
 fa_status fa_decoder_prefill(fa_context *ctx, fa_decoder *d, const int32_t *tokens, uint32_t l_new) {
     return prefill_impl(ctx, d, tokens, l_new, nullptr, nullptr);
+}
+
+fa_status fa_decoder_prefill_padded(fa_context *ctx, fa_decoder *d, const int32_t *tokens, uint32_t l_max,
+                                    const uint32_t *row_lens) {
+    if (!row_lens) return fail(FA_ERR_INVALID_ARGUMENT, "decoder_prefill_padded: null lengths");
+    return prefill_impl(ctx, d, tokens, l_max, nullptr, nullptr, row_lens);
 }
 
 fa_status fa_decoder_verify(fa_context *ctx, fa_decoder *d, const int32_t *tokens, uint32_t l_new, int32_t *picked,

@@ -69,13 +69,23 @@ __global__ void __launch_bounds__(64)
     }
 }
 
+// row_lens (optional): row b's prompt is only row_lens[b] <= l_chunk tokens long and the rest of its chunk
+// is padding; its last token is then row b * l_chunk + row_lens[b] - 1.  seq_lens advances by the whole chunk
+// either way (the attention of the pass places token t at seq_len - l_chunk + t); trim_lens_kernel takes the
+// padding off afterwards.
 __global__ void advance_lens_kernel(uint32_t *__restrict__ seq_lens, int32_t *__restrict__ last_rows, uint32_t batch,
-                                    uint32_t l_chunk) {
+                                    uint32_t l_chunk, const uint32_t *__restrict__ row_lens) {
     const uint32_t b = blockIdx.x * blockDim.x + threadIdx.x;
     if (b < batch) {
         seq_lens[b] += l_chunk;
-        last_rows[b] = (int32_t)(b * l_chunk + l_chunk - 1);
+        last_rows[b] = (int32_t)(b * l_chunk + (row_lens ? row_lens[b] : l_chunk) - 1);
     }
+}
+
+__global__ void trim_lens_kernel(uint32_t *__restrict__ seq_lens, const uint32_t *__restrict__ row_lens, uint32_t batch,
+                                 uint32_t l_chunk) {
+    const uint32_t b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b < batch) seq_lens[b] -= l_chunk - row_lens[b];
 }
 
 // qkv [rows, (heads + 2 kv_heads) head_dim] f32 -> q rotated, bf16 [rows, heads head_dim]; K rotated and V
@@ -125,9 +135,15 @@ void prefill_prepare(const uint32_t *tables, const uint32_t *seq_lens, uint32_t 
                                                               max_blocks_per_seq, num_blocks, head_dim, theta);
 }
 
-void advance_seq_lens(uint32_t *seq_lens, int32_t *last_rows, uint32_t batch, uint32_t l_chunk, hipStream_t s) {
+void advance_seq_lens(uint32_t *seq_lens, int32_t *last_rows, uint32_t batch, uint32_t l_chunk, const uint32_t *row_lens,
+                      hipStream_t s) {
     if (batch == 0) return;
-    advance_lens_kernel<<<(batch + 63) / 64, 64, 0, s>>>(seq_lens, last_rows, batch, l_chunk);
+    advance_lens_kernel<<<(batch + 63) / 64, 64, 0, s>>>(seq_lens, last_rows, batch, l_chunk, row_lens);
+}
+
+void trim_seq_lens(uint32_t *seq_lens, const uint32_t *row_lens, uint32_t batch, uint32_t l_chunk, hipStream_t s) {
+    if (batch == 0) return;
+    trim_lens_kernel<<<(batch + 63) / 64, 64, 0, s>>>(seq_lens, row_lens, batch, l_chunk);
 }
 
 void rope_append(const float *qkv, const float *cos_sin, const uint32_t *slots, uint16_t *q_out, uint16_t *k_pool,

@@ -1,10 +1,12 @@
-// Decode-shape ("skinny", m <= 32 tokens) quantized linears.  Both kernels are
+// Decode-shape ("skinny", m <= 64 tokens for int8 activations, m <= 32 for bf16) quantized linears.  Both kernels are
 // HBM-bound streams over the tile-ordered int8 weight: every wavefront load
 // is one contiguous 1 KiB tile that lands directly in the operand layout of
 // the matrix instruction, so the weight never passes through LDS.  The block
 // splits K over its wavefronts and reduces their partial tiles in LDS in a
 // fixed order (deterministic).
 #include <algorithm>
+
+#include <type_traits>
 
 #include "device_utils.hpp"
 #include "kernels.hpp"
@@ -576,18 +578,24 @@ inline bool astat_applies(uint64_t n_units, uint64_t k_tiles, int num_cus) {
     return n_units >= 3 * (uint64_t)num_cus;
 }
 
-template <int MT>
-void launch_w8a8(const int8_t *xq, const int8_t *wt, uint32_t m, uint32_t n, uint32_t n_tiles, uint32_t k_tiles,
-                 const EpiI8 &ep, int ntw, int waves, hipStream_t s) {
-    unsigned grid = (n_tiles + ntw - 1) / ntw;
-    if (ntw == 1 && waves == 8)
-        w8a8_skinny_kernel<MT, 1, 8, kEpiPlain><<<grid, 512, 0, s>>>(xq, wt, m, n, n_tiles, k_tiles, ep);
-    else if (ntw == 1)
-        w8a8_skinny_kernel<MT, 1, 4, kEpiPlain><<<grid, 256, 0, s>>>(xq, wt, m, n, n_tiles, k_tiles, ep);
-    else if (waves == 8)
-        w8a8_skinny_kernel<MT, 2, 8, kEpiPlain><<<grid, 512, 0, s>>>(xq, wt, m, n, n_tiles, k_tiles, ep);
+// Row tiles per block by the number of rows (16 each, at most 64 rows), 4 or 8 wavefronts.
+template <int NTW, int MODE, typename... A>
+void launch_w8a8_rows(uint64_t m, int waves, unsigned grid, hipStream_t s, A... args) {
+    auto go = [&](auto mt) {
+        constexpr int MT = decltype(mt)::value;
+        if (waves == 8)
+            w8a8_skinny_kernel<MT, NTW, 8, MODE><<<grid, 512, 0, s>>>(args...);
+        else
+            w8a8_skinny_kernel<MT, NTW, 4, MODE><<<grid, 256, 0, s>>>(args...);
+    };
+    if (m <= 16)
+        go(std::integral_constant<int, 1>{});
+    else if (m <= 32)
+        go(std::integral_constant<int, 2>{});
+    else if (m <= 48)
+        go(std::integral_constant<int, 3>{});
     else
-        w8a8_skinny_kernel<MT, 2, 4, kEpiPlain><<<grid, 256, 0, s>>>(xq, wt, m, n, n_tiles, k_tiles, ep);
+        go(std::integral_constant<int, 4>{});
 }
 
 template <int MT>
@@ -618,7 +626,7 @@ void linear_w8a8_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t 
     e.acc_out = ep.acc_out;
     e.out = ep.out;
     e.out_bf16 = ep.out_bf16;
-    if (astat_applies((n_tiles + 1) / 2, k_tiles, num_cus)) {
+    if (m <= 32 && astat_applies((n_tiles + 1) / 2, k_tiles, num_cus)) {
         unsigned n_units = (n_tiles + 1) / 2;
         unsigned blocks = (unsigned)std::min<uint64_t>(n_units, (uint64_t)num_cus);
         if (m <= 16)
@@ -629,10 +637,11 @@ void linear_w8a8_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t 
     }
     int ntw, waves;
     pick_config(n_tiles, k_tiles, num_cus, &ntw, &waves);
-    if (m <= 16)
-        launch_w8a8<1>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e, ntw, waves, s);
+    const unsigned grid = (n_tiles + ntw - 1) / ntw;
+    if (ntw == 1)
+        launch_w8a8_rows<1, kEpiPlain>(m, waves, grid, s, xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e);
     else
-        launch_w8a8<2>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e, ntw, waves, s);
+        launch_w8a8_rows<2, kEpiPlain>(m, waves, grid, s, xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e);
 }
 
 void linear_w8a8_swiglu_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, const float *sx, const float *sw,
@@ -646,7 +655,7 @@ void linear_w8a8_swiglu_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, co
     e.sw = sw;
     e.out = act;
     e.pmax = pmax;
-    if (astat_applies(n_tiles / 2, k_tiles, num_cus)) {
+    if (m <= 32 && astat_applies(n_tiles / 2, k_tiles, num_cus)) {
         unsigned blocks = (unsigned)std::min<uint64_t>(n_tiles / 2, (uint64_t)num_cus);
         if (m <= 16)
             w8a8_astat_kernel<1, 8, kEpiSwiglu><<<blocks, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, n_tiles / 2, e);
@@ -654,18 +663,7 @@ void linear_w8a8_swiglu_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, co
             w8a8_astat_kernel<2, 8, kEpiSwiglu><<<blocks, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, n_tiles / 2, e);
         return;
     }
-    unsigned grid = n_tiles / 2;
-    if (m <= 16) {
-        if (waves == 8)
-            w8a8_skinny_kernel<1, 2, 8, kEpiSwiglu><<<grid, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e);
-        else
-            w8a8_skinny_kernel<1, 2, 4, kEpiSwiglu><<<grid, 256, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e);
-    } else {
-        if (waves == 8)
-            w8a8_skinny_kernel<2, 2, 8, kEpiSwiglu><<<grid, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e);
-        else
-            w8a8_skinny_kernel<2, 2, 4, kEpiSwiglu><<<grid, 256, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e);
-    }
+    launch_w8a8_rows<2, kEpiSwiglu>(m, waves, n_tiles / 2, s, xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e);
 }
 
 void linear_w8a8_qkv_rope_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, const float *sx, const float *sw,
@@ -687,17 +685,7 @@ void linear_w8a8_qkv_rope_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, 
     e.pool_rows = t.pool_rows;
     unsigned grid = n / 32;                                  // one block per pair of 16-column tiles
     int waves = g_skinny_waves ? g_skinny_waves : 8;
-    if (m <= 16) {
-        if (waves == 8)
-            w8a8_skinny_kernel<1, 2, 8, kEpiRope><<<grid, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, n, n_tiles, k_tiles, e);
-        else
-            w8a8_skinny_kernel<1, 2, 4, kEpiRope><<<grid, 256, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, n, n_tiles, k_tiles, e);
-    } else {
-        if (waves == 8)
-            w8a8_skinny_kernel<2, 2, 8, kEpiRope><<<grid, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, n, n_tiles, k_tiles, e);
-        else
-            w8a8_skinny_kernel<2, 2, 4, kEpiRope><<<grid, 256, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, n, n_tiles, k_tiles, e);
-    }
+    launch_w8a8_rows<2, kEpiRope>(m, waves, grid, s, xq_tiled, w_tiles, (uint32_t)m, n, n_tiles, k_tiles, e);
 }
 
 void linear_w8a16_skinny(const uint16_t *a, const int8_t *w_tiles, const float *sw, uint64_t m, uint64_t n,

@@ -92,7 +92,7 @@ struct EpilogueI8 {
     void *out;            // [m, n] f32 or bf16
     int out_bf16;
 };
-// xq_tiled: activation tiles (see quantize_rows_i8); m <= 32.
+// xq_tiled: activation tiles (see quantize_rows_i8); m <= 64 (one to four row tiles of 16 per block).
 void linear_w8a8_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t m, uint64_t n,
                         uint64_t n_pad, uint64_t k_pad, const EpilogueI8 &ep, int num_cus,
                         hipStream_t s);
@@ -211,7 +211,10 @@ void prefill_prepare(const uint32_t *tables, const uint32_t *seq_lens, uint32_t 
                      uint32_t l_chunk, uint32_t block_size, uint32_t max_blocks_per_seq, uint32_t num_blocks,
                      uint32_t head_dim, double theta, hipStream_t s);
 // seq_lens[b] += l_chunk; last_rows[b] = row of the chunk's last token of sequence b
-void advance_seq_lens(uint32_t *seq_lens, int32_t *last_rows, uint32_t batch, uint32_t l_chunk, hipStream_t s);
+void advance_seq_lens(uint32_t *seq_lens, int32_t *last_rows, uint32_t batch, uint32_t l_chunk, const uint32_t *row_lens,
+                      hipStream_t s);
+// After a padded prompt pass: seq_lens[b] -= l_chunk - row_lens[b].
+void trim_seq_lens(uint32_t *seq_lens, const uint32_t *row_lens, uint32_t batch, uint32_t l_chunk, hipStream_t s);
 // RoPE on the q and k heads of qkv [rows, (heads + 2 kv_heads) head_dim] (f32), one rounding to bf16;
 // q to q_out [rows, heads head_dim], K / V to pool row slots[r].
 void rope_append(const float *qkv, const float *cos_sin, const uint32_t *slots, uint16_t *q_out, uint16_t *k_pool,

@@ -83,6 +83,18 @@ class Decoder:
             raise ValueError("prompt must be [batch, l_new]")
         check(lib.fa_decoder_prefill(self._ops._ctx, self._h, p.ctypes.data_as(capi.i32p), p.shape[1]))
 
+    def prefill_padded(self, prompts):
+        """prompts: one int32 sequence per installed row, of any lengths >= 1; they are padded to the longest
+        and ingested in one pass (batch * longest <= 4096).  Every row ends as after its own ``prefill``."""
+        if len(prompts) != self.batch:
+            raise ValueError("one prompt per installed sequence")
+        lens = np.array([len(p) for p in prompts], dtype=np.uint32)
+        padded = np.zeros((self.batch, int(lens.max()) if len(prompts) else 0), dtype=np.int32)
+        for b, p in enumerate(prompts):
+            padded[b, :len(p)] = p
+        check(lib.fa_decoder_prefill_padded(self._ops._ctx, self._h, padded.ctypes.data_as(capi.i32p), padded.shape[1],
+                                            lens.ctypes.data_as(capi.u32p)))
+
     def verify(self, tokens, want_logits=False):
         """Speculative verification: feeds tokens [batch, l_new] like ``prefill`` and returns the greedy token
         after every one of them, int32 [batch, l_new] (and the logits [batch, l_new, vocab] if asked)."""

@@ -5,9 +5,9 @@ validation, :500-640 ``generate``; crates/autodiff/src/generate/scheduler.rs:75-
 :521-562 admission, :571-590 ``step``, :712-720 ``take_*``) for a model whose state lives on the device: the KV
 pages of all requests share the decoder's pools, every request owns a block-table row, a sampling record with
 its own generator (seeded from its config, one draw per generated token) and its token list.  One ``step``
-admits queued requests while rows and pages are free, ingests the prompt of every newly admitted request
-(batch 1, the whole prompt in one pass) and advances all other active requests together by one decode step of
-the batch they currently form; requests finish when they reach ``max_length`` (there is no end-of-sequence
+admits queued requests while rows and pages are free, ingests the prompts of the newly admitted requests
+(whole prompts; requests that join together share padded passes) and advances all other active requests
+together by one decode step of the batch they currently form; requests finish when they reach ``max_length`` (there is no end-of-sequence
 stop, as in the reference) and leave the batch between steps.
 
 What differs from the reference, by construction: the decode step is batched on the device (the reference's
@@ -387,13 +387,18 @@ class BatchScheduler:
         gone = set()
         if fresh:
             self._pull_resident_state()                    # the prompt passes overwrite the installed batch
-            for a in fresh:
+            for group in self._prompt_groups(fresh):
                 try:
-                    self._ingest(a)
-                except (BackendError, InvalidArgument) as e:
-                    self._fail(a, e, gone)
+                    bad = self._ingest(group)
+                except BackendError as e:                  # a device failure takes the whole pass with it
+                    for a in group:
+                        self._fail(a, e, gone)
                     continue
-                completed += self._maybe_finish(a, gone)
+                for a in group:
+                    if a in bad:
+                        self._fail(a, InvalidArgument("generate: logits hold non-finite values"), gone)
+                    else:
+                        completed += self._maybe_finish(a, gone)
         if old:
             try:
                 if self._resident != [a.id for a in old]:
@@ -495,17 +500,43 @@ class BatchScheduler:
                 a.policy = (r.rng_state, r.temperature, r.top_k, r.strategy)
         self._resident = None
 
-    def _ingest(self, a):
-        self._dec.set_sequences(self._table_row(a)[None, :], np.zeros(1, np.uint32))
-        self._dec.set_row_sampling(self._policy_rows([a]))
-        self._dec.prefill(np.array([a.tokens], dtype=np.int32))
-        tok = int(self._dec.tokens()[0])
-        r = self._dec.read_row_sampling()[0]
-        a.policy = (r.rng_state, r.temperature, r.top_k, r.strategy)
-        a.fresh = False
-        if tok < 0:
-            raise InvalidArgument("generate: logits hold non-finite values")
-        a.tokens.append(tok)
+    MAX_PROMPT_ROWS = 4096                                  # rows (requests x longest prompt) of one padded pass
+
+    def _prompt_groups(self, fresh):
+        """Requests that join in the same iteration share prompt passes: sorted by prompt length and cut into
+        groups whose padded size stays within one pass and whose longest prompt is at most twice the
+        shortest (the padding is computed and thrown away)."""
+        groups, cur = [], []
+        for a in sorted(fresh, key=lambda a: (len(a.tokens), a.id)):
+            n = len(a.tokens)
+            if cur and ((len(cur) + 1) * n > self.MAX_PROMPT_ROWS or n > 2 * len(cur[0].tokens)
+                        or len(cur) >= self._dec.cfg.max_batch):
+                groups.append(cur)
+                cur = []
+            cur.append(a)
+        if cur:
+            groups.append(cur)
+        return groups
+
+    def _ingest(self, group):
+        """One prompt pass for the group; returns the requests whose logits were not finite."""
+        self._dec.set_sequences(np.stack([self._table_row(a) for a in group]), np.zeros(len(group), np.uint32))
+        self._dec.set_row_sampling(self._policy_rows(group))
+        if len(group) == 1:
+            self._dec.prefill(np.array([group[0].tokens], dtype=np.int32))
+        else:
+            self._dec.prefill_padded([np.array(a.tokens, dtype=np.int32) for a in group])
+        toks = self._dec.tokens()
+        rows = self._dec.read_row_sampling()
+        bad = []
+        for a, tok, r in zip(group, toks, rows):
+            a.policy = (r.rng_state, r.temperature, r.top_k, r.strategy)
+            a.fresh = False
+            if tok < 0:
+                bad.append(a)
+            else:
+                a.tokens.append(int(tok))
+        return bad
 
     def _maybe_finish(self, a, gone):
         if len(a.tokens) < a.config.max_length:

@@ -466,6 +466,18 @@ fa_status fa_decoder_read_row_sampling(fa_context *ctx, fa_decoder *dec, fa_row_
  * decoded.  Rejected before anything is queued if a row has no pages for its
  * prompt.  Asynchronous apart from the upload of the token ids. */
 fa_status fa_decoder_prefill(fa_context *ctx, fa_decoder *dec, const int32_t *tokens, uint32_t l_new);
+/* Prompts of different lengths in one pass: tokens [batch, l_max] holds row b's
+ * row_lens[b] prompt tokens followed by padding (any valid token id), row_lens
+ * [batch] is a host array with 1 <= row_lens[b] <= l_max, batch * l_max <= 4096.
+ * Every row ends as if it had been ingested alone with fa_decoder_prefill: its
+ * length advances by row_lens[b], the logits and the next token are those of
+ * its own last prompt token.  The padding is computed and thrown away: its
+ * cache rows land past the sequence's length (in pages the row owns, if any;
+ * positions without a page are skipped) and are overwritten by later tokens.
+ * What a scheduler uses when several requests join in the same iteration
+ * (crates/autodiff/src/generate/scheduler.rs:521-562 admits them one by one). */
+fa_status fa_decoder_prefill_padded(fa_context *ctx, fa_decoder *dec, const int32_t *tokens, uint32_t l_max,
+                                    const uint32_t *row_lens);
 /* Speculative-decoding verification (crates/autodiff/src/generate/speculative.rs:
  * 484-490: the target model consumes the pending token and the draft's k tokens
  * in one forward pass and every position's logits decide): fa_decoder_prefill

@@ -56,6 +56,9 @@ def _check_step(m, dec, lens, tokens, use_graph, tag):
     dict(n_layers=2, d_model=256, n_heads=4, n_kv_heads=2, d_ffn=512, vocab=1000, batch=4, ctxs=[1, 15, 16, 200]),
     dict(n_layers=1, d_model=512, n_heads=8, n_kv_heads=8, d_ffn=256, vocab=333, batch=17, ctxs=list(range(3, 20))),
     dict(n_layers=2, d_model=1024, n_heads=8, n_kv_heads=1, d_ffn=1536, vocab=4000, batch=32, ctxs=[40 + 9 * i for i in range(32)]),
+    # more than 32 rows: three and four row tiles per block in the decode-shape linears
+    dict(n_layers=2, d_model=512, n_heads=4, n_kv_heads=2, d_ffn=1024, vocab=2000, batch=41, ctxs=[1 + 7 * i for i in range(41)]),
+    dict(n_layers=1, d_model=1024, n_heads=8, n_kv_heads=2, d_ffn=1536, vocab=1500, batch=64, ctxs=[5 + 3 * i for i in range(64)]),
 ])
 @pytest.mark.parametrize("astat", [1, 2], ids=["block-per-tile", "activation-stationary"])
 def test_decode_steps_match_the_oracle_eager_and_graph(shape, astat):
@@ -240,7 +243,7 @@ def test_decoder_argument_errors():
     h = C.c_void_p()
     bad = fa.capi.DecoderConfig(1, 256, 4, 2, 64, 512, 100, 16, 8, 32, 4, 1e-5, 500000.0)       # head_dim 64
     assert lib.fa_decoder_create(be._ctx, C.byref(bad), C.byref(h)) == fa.capi.UNSUPPORTED
-    bad = fa.capi.DecoderConfig(1, 256, 4, 2, 128, 512, 100, 16, 8, 32, 64, 1e-5, 500000.0)     # batch 64
+    bad = fa.capi.DecoderConfig(1, 256, 4, 2, 128, 512, 100, 16, 8, 32, 65, 1e-5, 500000.0)     # batch 65
     assert lib.fa_decoder_create(be._ctx, C.byref(bad), C.byref(h)) == fa.capi.UNSUPPORTED
     m = build_model(seed=1, n_layers=1, d_model=128, n_heads=2, n_kv_heads=1, d_ffn=128, vocab=50, batch=2,
                     ctxs=[3, 4], steps=1)

@@ -120,12 +120,12 @@ def test_w8a8_linear_benchmark_configuration_is_bit_exact():
     assert np.abs(got_out - ref).max() < 0.03 * np.abs(ref).max()
 
 
-@pytest.mark.parametrize("m", [1, 8, 16, 17, 32, 33, 100, 300])
+@pytest.mark.parametrize("m", [1, 8, 16, 17, 32, 33, 48, 49, 64, 65, 100, 300])
 def test_w8a8_linear_row_sweep_bias_and_output_types(m):
     fa = _fa()
     be = ops()
     rng = o.Rng(100 + m)
-    k, n = (4096, 6144) if m <= 32 else (512, 200)
+    k, n = (4096, 6144) if m <= 64 else (512, 200)
     x = rng.randn((m, k))
     w = rng.randn((k, n), std=0.02)
     bias = rng.randn((n,))

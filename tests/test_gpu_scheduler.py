@@ -49,14 +49,20 @@ def _recording(dec):
             self.rows = [tuple(int(x) for x in r) for r in np.asarray(tables)]
             super().set_sequences(tables, lens)
 
-        def _record(self, kind):
+        def _record(self, kind, prompts=None):
             logits, toks = self.logits(), self.tokens()
             for r, row in enumerate(self.rows):
-                self.trace.append((kind, row, logits[r].copy(), int(toks[r])))
+                tag = kind if prompts is None else (kind, tuple(int(t) for t in prompts[r]))
+                self.trace.append((tag, row, logits[r].copy(), int(toks[r])))
 
         def prefill(self, prompt):
             super().prefill(prompt)
-            self._record("prefill")
+            self._record("prefill", list(np.asarray(prompt)))
+
+        def prefill_padded(self, prompts):
+            super().prefill_padded(prompts)
+            self.padded_passes = getattr(self, "padded_passes", 0) + 1
+            self._record("prefill", prompts)
 
         def step(self, use_graph=True):
             super().step(use_graph)
@@ -75,7 +81,7 @@ def _cfg(max_length, strategy, seed):
 def _requests():
     from fandhe_ai_amd.scheduler import SamplingStrategy as S
     rng = np.random.default_rng(77)
-    spec = [(1, 9, S.Greedy(), 0), (30, 60, S.TopK(5), 7), (3, 20, S.Temperature(0.8), 11), (17, 33, S.Greedy(), 0),
+    spec = [(1, 9, S.Greedy(), 0), (30, 60, S.TopK(5), 7), (2, 20, S.Temperature(0.8), 11), (17, 33, S.Greedy(), 0),
             (5, 48, S.TopK(40), 0), (12, 13, S.Temperature(1.5), 2 ** 63 + 5), (2, 2, S.Greedy(), 0), (8, 40, S.TopK(1), 3)]
     out = []
     for plen, max_length, strategy, seed in spec:
@@ -92,7 +98,7 @@ def _split_by_request(trace, reqs_by_prompt):
     owner, per = {}, {}
     for kind, row, logits, tok in trace:
         if kind[0] == "prefill":
-            owner[row] = kind[1]
+            owner[row] = reqs_by_prompt[kind[1]]
         per.setdefault(owner[row], []).append((logits, tok))
     return per
 
@@ -105,15 +111,7 @@ def test_scheduler_tokens_are_the_oracle_picks_and_logits_match_stand_alone_gene
     s = BatchScheduler(dec, SchedulerLimits(3, 16, 64))
     ids = [s.submit(p, c) for p, c in reqs]
 
-    # name each prompt pass by the request that is being ingested
-    real_prefill = dec.prefill
-
-    def prefill(prompt):
-        n = len(dec.trace)
-        real_prefill(prompt)
-        rid = next(i for i, (p, _) in zip(ids, reqs) if len(p) == prompt.shape[1] and (p == prompt[0]).all())
-        dec.trace[n:] = [(("prefill", rid),) + e[1:] for e in dec.trace[n:]]
-    dec.prefill = prefill
+    by_prompt = {tuple(int(t) for t in p): rid for rid, (p, _) in zip(ids, reqs)}      # the prompts are all different
 
     done, sizes = {}, []
     for _ in range(400):
@@ -124,7 +122,8 @@ def test_scheduler_tokens_are_the_oracle_picks_and_logits_match_stand_alone_gene
         done.update(dict(s.take_finished()))
     assert s.take_failed() == [] and sorted(done) == ids and s.free_pages() == 10
     assert max(sizes) == 3 and len(set(sizes)) > 2          # the batch really changed size while running
-    per = _split_by_request(dec.trace, None)
+    assert getattr(dec, "padded_passes", 0) >= 1            # requests that joined together shared a prompt pass
+    per = _split_by_request(dec.trace, by_prompt)
 
     # (1) tokens = oracle picks from the produced logits, own generator stream per request
     for rid, (prompt, cfg) in zip(ids, reqs):
@@ -149,8 +148,6 @@ def test_scheduler_tokens_are_the_oracle_picks_and_logits_match_stand_alone_gene
             spread = float(logits.max() - logits.min())
             err = np.abs(got_logits - logits) / spread
             assert err.mean() < 2e-4 and err.max() < 2e-2, (rid, i, err.mean(), err.max())
-            if i == 0:
-                assert got_logits.tobytes() == logits.tobytes() and got_tok == tok      # the prompt pass is the same launch
             compared += 1
             if got_tok != tok:
                 break                                      # an indecisive pick: the histories part here
@@ -271,3 +268,64 @@ def test_speculative_generation_equals_the_target_generating_alone(rows):
     assert matched >= 0.9 * total
     for d in (target, twin, other):
         d.close()
+
+
+def test_padded_prompt_pass_leaves_every_row_as_its_own_prompt_pass_would():
+    """Three prompts of different lengths in one padded pass against the same prompts ingested one by one:
+    logits of every row's last prompt token within the chained-step bar (the rows of a GEMM and the ranges of
+    the attention are cut differently), lengths exact, and decode steps continue from either state alike.
+    One row has pages for its own prompt only, so part of its padding has no page to land on."""
+    import fandhe_ai_amd as fa
+    geometry = dict(max_blocks_per_seq=4, num_blocks=12, max_batch=4)
+    dec = _decoder(**geometry)
+    rng = np.random.default_rng(8)
+    prompts = [rng.integers(0, VOCAB, n).astype(np.int32) for n in (5, 37, 16)]
+    tables = np.full((3, 4), 0xFFFFFFFF, dtype=np.uint32)
+    tables[0, :1] = [7]                                     # 5 tokens + a few steps fit one page; padding to 37 does not
+    tables[1, :3] = [0, 1, 2]
+    tables[2, :2] = [9, 4]
+    alone_logits, alone_tokens = [], []
+    for b in range(3):
+        dec.set_sequences(tables[b:b + 1], np.zeros(1, np.uint32))
+        dec.prefill(prompts[b][None, :])
+        alone_logits.append(dec.logits()[0].copy())
+        alone_tokens.append(int(dec.tokens()[0]))
+    dec.set_sequences(tables, np.zeros(3, np.uint32))
+    dec.prefill_padded(prompts)
+    assert dec.seq_lens().tolist() == [5, 37, 16]
+    got_logits, got_tokens = dec.logits(), dec.tokens()
+    for b in range(3):
+        spread = float(alone_logits[b].max() - alone_logits[b].min())
+        err = np.abs(got_logits[b] - alone_logits[b]) / spread
+        assert np.isfinite(got_logits[b]).all() and err.mean() < 2e-4 and err.max() < 2e-2, (b, err.mean(), err.max())
+        top2 = np.sort(alone_logits[b])[-2:]
+        if (top2[1] - top2[0]) / spread > 4e-2:
+            assert got_tokens[b] == alone_tokens[b]
+    # both states decode on: same logits within the bar for three more steps
+    after_padded = []
+    toks = got_tokens.copy()
+    for _ in range(3):
+        dec.step()
+        after_padded.append(dec.logits().copy())
+    fed = [toks] + [o.argmax(axis=1).astype(np.int32) for o in after_padded[:-1]]
+    for b in range(3):                                      # replay row b alone, feeding what the padded run fed
+        dec.set_sequences(tables[b:b + 1], np.zeros(1, np.uint32))
+        dec.prefill(prompts[b][None, :])
+        for s_i in range(3):
+            dec.set_tokens(fed[s_i][b:b + 1])
+            dec.step()
+            ref = dec.logits()[0]
+            spread = float(ref.max() - ref.min())
+            err = np.abs(after_padded[s_i][b] - ref) / spread
+            assert err.mean() < 2e-4 and err.max() < 2e-2, (b, s_i, err.mean(), err.max())
+    # argument checks
+    dec.set_sequences(tables, np.zeros(3, np.uint32))
+    with pytest.raises(fa.InvalidArgument):
+        dec.prefill_padded([prompts[0], prompts[1], np.zeros(70, np.int32)])          # beyond the row's block table
+    with pytest.raises(fa.InvalidArgument):
+        dec.prefill_padded([np.zeros(20, np.int32), prompts[1], prompts[2]])          # row 0 has one page
+    lens = np.array([5, 0, 3], np.uint32)
+    pad = np.zeros((3, 5), np.int32)
+    assert fa.capi.lib.fa_decoder_prefill_padded(ops()._ctx, dec._h, pad.ctypes.data_as(fa.capi.i32p), 5,
+                                                 lens.ctypes.data_as(fa.capi.u32p)) == fa.capi.INVALID_ARGUMENT
+    dec.close()

@@ -111,6 +111,16 @@ class ToyDecoder:
                 self.lens[b] += 1
         self._pick()
 
+    def prefill_padded(self, prompts):
+        self.calls["prefill"] += 1
+        self.calls["padded_rows"] = self.calls.get("padded_rows", 0) + len(prompts)
+        assert len(prompts) == self.batch and len(prompts) * max(len(p) for p in prompts) <= 4096
+        for b, p in enumerate(prompts):
+            for t in p:
+                self._write(b, int(self.lens[b]), int(t))
+                self.lens[b] += 1
+        self._pick()
+
     def step(self, use_graph=True):
         self.calls["step"] += 1
         self.calls["step_rows"] += self.batch
@@ -249,6 +259,7 @@ def test_interleaved_requests_match_single_generate():
         want = generate(ToyDecoder(), i, c)
         assert done[rid].shape == want.shape and done[rid].tolist() == want.tolist()
     assert m.calls["step_rows"] > m.calls["step"]          # decode steps really ran several requests at once
+    assert m.calls.get("padded_rows", 0) >= 2              # and requests that joined together shared a prompt pass
     assert s.free_pages() == 6                             # every page came back
 
 
