@@ -412,7 +412,7 @@ fa_status fa_graph_destroy(fa_context *ctx, fa_graph *graph);
 typedef struct {
     uint32_t n_layers, d_model, n_heads, n_kv_heads, head_dim, d_ffn, vocab;
     uint32_t block_size, max_blocks_per_seq, num_blocks;
-    uint32_t max_batch;
+    uint32_t max_batch;           /* rows of a step: 1..=64 */
     float rms_eps;
     double rope_theta;
 } fa_decoder_config;
