@@ -444,7 +444,8 @@ def bench_continuous_batching(fa, be, dec, dcfg, requests=96, max_active=32):
     sec = time.perf_counter() - t0
     assert done == requests and not s.take_failed() and len(s.take_finished()) == requests
     return dict(requests=requests, max_active=max_active, prompt_tokens=prompt_tokens, generated_tokens=new_tokens,
-                seconds=sec, generated_tokens_per_s=new_tokens / sec, iterations=steps, mean_active_rows=rows / steps)
+                seconds=sec, generated_tokens_per_s=new_tokens / sec, iterations=steps, mean_active_rows=rows / steps,
+                **s.stats)
 
 
 def bench_sampling(fa, be, rows=32, vocab=32000, iters=50):

@@ -343,6 +343,8 @@ class BatchScheduler:
         self._next_id = 0
         self._pages = PageAllocator(cfg.num_blocks)
         self._resident = None                              # ids whose decode state is installed on the device, in row order
+        # what the device was asked to do so far: prompt passes, their rows incl. padding, decode steps and their rows
+        self.stats = {"prompt_passes": 0, "prompt_rows": 0, "decode_steps": 0, "decode_rows": 0}
 
     def queued_len(self):
         return len(self._queue)
@@ -405,6 +407,8 @@ class BatchScheduler:
                     self._install(old)
                 self._dec.step()
                 picked = self._dec.tokens()
+                self.stats["decode_steps"] += 1
+                self.stats["decode_rows"] += len(old)
             except BackendError as e:                      # a device failure takes the whole batch with it
                 for a in old:
                     self._fail(a, e, gone)
@@ -522,6 +526,8 @@ class BatchScheduler:
         """One prompt pass for the group; returns the requests whose logits were not finite."""
         self._dec.set_sequences(np.stack([self._table_row(a) for a in group]), np.zeros(len(group), np.uint32))
         self._dec.set_row_sampling(self._policy_rows(group))
+        self.stats["prompt_passes"] += 1
+        self.stats["prompt_rows"] += len(group) * max(len(a.tokens) for a in group)
         if len(group) == 1:
             self._dec.prefill(np.array([group[0].tokens], dtype=np.int32))
         else:
