@@ -14,10 +14,24 @@ class Model:
 
 
 def build_model(seed, n_layers, d_model, n_heads, n_kv_heads, d_ffn, vocab, batch, ctxs, steps, num_blocks=None,
-                head_dim=128, block_size=16, quantize_on_host=True, threads=8):
+                head_dim=128, block_size=16, quantize_on_host=True, threads=8, numpy_fill=False):
     """Weights ~N(0, 0.02) quantized per output channel; norm weights ~1; KV pools pre-filled for the
-    given context lengths; block tables sized for `steps` more tokens."""
+    given context lengths; block tables sized for `steps` more tokens.  numpy_fill: the large tensors come
+    from numpy's generator instead of the reference's (for models of hundreds of millions of elements)."""
     rng = o.Rng(seed)
+    if numpy_fill:
+        class _Fast:
+            def __init__(self, base, seed):
+                self.base, self.np = base, np.random.default_rng(seed)
+
+            def randn(self, shape, std=1.0):
+                if int(np.prod(shape)) < 1 << 20:
+                    return self.base.randn(shape, std=std) if std != 1.0 else self.base.randn(shape)
+                return (self.np.standard_normal(shape, dtype=np.float32) * np.float32(std)).astype(np.float32)
+
+            def __getattr__(self, name):
+                return getattr(self.base, name)
+        rng = _Fast(rng, seed)
     m = Model()
     m.cfg = dict(n_layers=n_layers, d_model=d_model, n_heads=n_heads, n_kv_heads=n_kv_heads, head_dim=head_dim,
                  d_ffn=d_ffn, vocab=vocab, block_size=block_size, rms_eps=1e-5, rope_theta=500000.0)

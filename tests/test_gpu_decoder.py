@@ -80,6 +80,24 @@ def test_decode_steps_match_the_oracle_eager_and_graph(shape, astat):
         fa.check(fa.capi.lib.fa_set_tuning(5, 0))
 
 
+def test_decode_step_at_the_benchmark_width():
+    """One layer of the benchmark's decoder at its full width (d_model 4096, 32 / 8 heads, FFN 14336, vocab
+    32000), batch 32, contexts uniform in [1024, 8192]: the shapes at which the step's kernels are timed
+    (activation-stationary gate/up and lm_head, deep-k down projection, long ragged contexts), eager and graph."""
+    be = ops()
+    ctxs = np.random.default_rng(0).integers(1024, 8193, size=32).tolist()
+    m = build_model(seed=3, n_layers=1, d_model=4096, n_heads=32, n_kv_heads=8, d_ffn=14336, vocab=32000, batch=32,
+                    ctxs=ctxs, steps=3, numpy_fill=True)
+    dec = GpuDecoder(be, m)
+    try:
+        lens, tokens = m.seq_lens.copy(), m.tokens.copy()
+        for step in range(2):
+            tokens = _check_step(m, dec, lens, tokens, use_graph=(step > 0), tag="benchmark width:step%d" % step)
+            dec.set_state(lens, tokens)
+    finally:
+        dec.close()
+
+
 PREFILL_SHAPES = [
     dict(n_layers=2, d_model=256, n_heads=4, n_kv_heads=2, d_ffn=512, vocab=1000, batch=4, ctxs=[0, 5, 16, 40], l_new=7),
     dict(n_layers=2, d_model=512, n_heads=8, n_kv_heads=2, d_ffn=768, vocab=500, batch=3, ctxs=[0, 1, 31], l_new=33),
