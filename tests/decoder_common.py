@@ -214,3 +214,26 @@ class GpuDecoder:
         for x in self.keep:
             x.free()
         self.keep = []
+
+
+def llama_checkpoint(seed, n_layers, d, heads, kv, f, vocab, dh=128):
+    """Random float32 tensors under the names and [out, in] shapes of a Llama-style safetensors checkpoint."""
+    rng = np.random.default_rng(seed)
+
+    def w(*shape):
+        return (rng.standard_normal(shape) / np.sqrt(shape[-1])).astype(np.float32)
+
+    t = {"model.embed_tokens.weight": rng.standard_normal((vocab, d)).astype(np.float32),
+         "model.norm.weight": (1 + 0.1 * rng.standard_normal(d)).astype(np.float32), "lm_head.weight": w(vocab, d)}
+    for i in range(n_layers):
+        p = "model.layers.%d." % i
+        t[p + "input_layernorm.weight"] = (1 + 0.1 * rng.standard_normal(d)).astype(np.float32)
+        t[p + "post_attention_layernorm.weight"] = (1 + 0.1 * rng.standard_normal(d)).astype(np.float32)
+        t[p + "self_attn.q_proj.weight"] = w(heads * dh, d)
+        t[p + "self_attn.k_proj.weight"] = w(kv * dh, d)
+        t[p + "self_attn.v_proj.weight"] = w(kv * dh, d)
+        t[p + "self_attn.o_proj.weight"] = w(d, heads * dh)
+        t[p + "mlp.gate_proj.weight"] = w(f, d)
+        t[p + "mlp.up_proj.weight"] = w(f, d)
+        t[p + "mlp.down_proj.weight"] = w(d, f)
+    return t

@@ -8,31 +8,10 @@ import pytest
 from safetensors.numpy import save as st_save
 
 import oracle_lib as o
+from decoder_common import llama_checkpoint as _checkpoint
 from gpu_common import ops
 
 pytestmark = pytest.mark.gpu
-
-
-def _checkpoint(seed, n_layers, d, heads, kv, f, vocab, dh=128):
-    rng = np.random.default_rng(seed)
-
-    def w(*shape):
-        return (rng.standard_normal(shape) / np.sqrt(shape[-1])).astype(np.float32)
-
-    t = {"model.embed_tokens.weight": rng.standard_normal((vocab, d)).astype(np.float32),
-         "model.norm.weight": (1 + 0.1 * rng.standard_normal(d)).astype(np.float32), "lm_head.weight": w(vocab, d)}
-    for i in range(n_layers):
-        p = "model.layers.%d." % i
-        t[p + "input_layernorm.weight"] = (1 + 0.1 * rng.standard_normal(d)).astype(np.float32)
-        t[p + "post_attention_layernorm.weight"] = (1 + 0.1 * rng.standard_normal(d)).astype(np.float32)
-        t[p + "self_attn.q_proj.weight"] = w(heads * dh, d)
-        t[p + "self_attn.k_proj.weight"] = w(kv * dh, d)
-        t[p + "self_attn.v_proj.weight"] = w(kv * dh, d)
-        t[p + "self_attn.o_proj.weight"] = w(d, heads * dh)
-        t[p + "mlp.gate_proj.weight"] = w(f, d)
-        t[p + "mlp.up_proj.weight"] = w(f, d)
-        t[p + "mlp.down_proj.weight"] = w(d, f)
-    return t
 
 
 def test_loaded_decoder_equals_hand_built_decoder(tmp_path):

@@ -19,7 +19,7 @@ import pytest
 from safetensors.numpy import save as st_save
 
 from gpu_common import ops
-from test_gpu_checkpoint import _checkpoint
+from decoder_common import llama_checkpoint as _checkpoint
 
 sys.path.insert(0, os.path.join(os.path.dirname(__file__), "..", "oracle"))
 import sampling as osamp  # noqa: E402
