@@ -295,7 +295,8 @@ def bench_prefill(fa, be, iters):
 
 def bench_prefill_attention(fa, be, batch=4, l_new=2048, heads=32, kv_heads=8):
     """Causal attention of `l_new` new tokens per row over their own pages (empty cache before them), bf16,
-    page 16: the streamed matrix-core kernel, and the generic kernel (reference summation order) beside it."""
+    page 16: the block form (what this shape selects), the streamed form and the generic kernel (reference
+    summation order) beside it."""
     lib = fa.capi.lib
     rng = np.random.default_rng(5)
     tables, max_blocks, num_blocks = make_tables(rng, [l_new] * batch, 0, 16)
@@ -310,7 +311,8 @@ def bench_prefill_attention(fa, be, batch=4, l_new=2048, heads=32, kv_heads=8):
     d_tables, d_lens = be.upload(tables), be.upload(np.full(batch, l_new, np.uint32))
     flops = 4.0 * batch * heads * 128 * l_new * (l_new + 1) / 2          # QK^T and PV over the causal triangle
     res = []
-    for name, generic, reps in (("streamed", 0, 5), ("generic", 1, 1)):
+    for name, form, generic, reps in (("block", 0, 0, 5), ("streamed", 1, 0, 5), ("generic", 0, 1, 1)):
+        fa.check(lib.fa_set_tuning(10, form))
         fa.check(lib.fa_set_tuning(8, generic))
         fn = lambda: fa.check(lib.fa_paged_attention_forward_device(be._ctx, q._h, pools[0]._h, pools[1]._h, d_tables._h,
                                                                     d_lens._h, C.byref(args.c()), out._h))
@@ -323,6 +325,7 @@ def bench_prefill_attention(fa, be, batch=4, l_new=2048, heads=32, kv_heads=8):
         ms = t.stop_ms() / reps
         res.append(dict(kernel=name, ms=ms, tflops=flops / (ms * 1e-3) / 1e12))
     fa.check(lib.fa_set_tuning(8, 0))
+    fa.check(lib.fa_set_tuning(10, 0))
     for b in pools + [q, out, d_tables, d_lens]:
         b.free()
     return res

@@ -718,6 +718,287 @@ __global__ void __launch_bounds__(1024) decode_stream_merge_quantize_kernel(Stre
     *(uint32_t *)(xq_tiled + tiled_chunk_offset(b, col / 16, k_tiles) + col % 16) = word;
 }
 
+// ------------------------------------------------------- prefill, block form
+// Causal attention of many new tokens per row, one block per (row, kv head, tile of 256 / group new
+// tokens).  The block walks the cached positions once, 32 at a time: the K and V rows of a step are
+// staged in LDS (two stages; the loads of the next step are in flight while this one is multiplied)
+// and shared by the eight wavefronts, so K / V leave the L2 once per 256 / group new tokens.  Every
+// wavefront owns 32 columns (new token x head of the group, column = token * group + head):
+//   S^T = K Q^T on v_mfma_f32_16x16x32_bf16 as in the decode kernel (lane (g, c): positions 4g .. 4g+3
+//   of a 16-position tile for column c), two position tiles per step;
+//   O^T += V^T P^T on the same instruction with k = the 32 positions of the step: the operand slot
+//   8g + i of a lane is position 4g + i of the first tile (i < 4) or of the second (i >= 4), which is
+//   where the scores of that lane already are; V^T is read from the staged rows 4 bytes (two dims of
+//   one position) at a time and split into an even and an odd operand by byte permutes.  A weight is
+//   fed as two bf16 terms, the value rounded to nearest and the remainder rounded to nearest (relative
+//   error of a weight <= 2^-18, unbiased).
+// The running maximum is per column; accumulators are rescaled only on steps where some column's maximum
+// grew.  A step wholly past the causal limit of all the columns of a wavefront is skipped by it.  The
+// result is normalised and written by the block itself (no partial results, no merge pass).
+struct FlashParams {
+    const uint16_t *q, *k_pool, *v_pool;
+    const uint32_t *tables, *seq_lens;
+    void *out;
+    int out_bf16;
+    uint32_t num_blocks, e_kv, batch, num_heads, num_kv_heads, group, max_blocks_per_seq, l_new, tq, tiles;
+    float scale;
+};
+constexpr int kFlashWaves = 8, kFlashNQ = 2, kFlashKeys = 32;
+constexpr int kFlashCols = kFlashWaves * kFlashNQ * 16;
+
+// two f32 values rounded to nearest-even bf16, first value in the low half
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16_rne(float a, float b) {
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{a, b}, v2bf));
+}
+
+__global__ void __launch_bounds__(kFlashWaves * 64) prefill_flash_kernel(FlashParams p) {
+    __shared__ __attribute__((aligned(16))) uint16_t k_s[2][kFlashKeys * kVPitch];
+    __shared__ __attribute__((aligned(16))) uint16_t v_s[2][kFlashKeys * kVPitch];
+    __shared__ uint32_t s_bad;
+    const int tid = threadIdx.x, lane = tid % 64;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
+    const int g = lane / 16, c = lane % 16;
+    // longest tiles first
+    const uint32_t per_tile = p.batch * p.num_kv_heads;
+    const uint32_t tile = p.tiles - 1 - blockIdx.x / per_tile;
+    const uint32_t b = (blockIdx.x % per_tile) / p.num_kv_heads, kvh = blockIdx.x % p.num_kv_heads;
+    const uint32_t max_ctx = p.max_blocks_per_seq * kPage;
+    const uint32_t len = p.seq_lens[b];
+    const bool violation = len < p.l_new || len > max_ctx;     // possible only with unvalidated device tables
+    const uint32_t ctx = len > max_ctx ? max_ctx : len;
+    const uint32_t base = violation ? 0 : len - p.l_new;       // cached positions before the new tokens
+    const uint32_t t0 = tile * p.tq;
+    const uint32_t t_end = t0 + p.tq < p.l_new ? t0 + p.tq : p.l_new;
+    uint32_t kmax = violation ? 0 : base + t_end;              // positions the last token of the tile sees
+    if (kmax > ctx) kmax = ctx;
+    const uint32_t npages = (kmax + kPage - 1) / kPage, n_it = (kmax + kFlashKeys - 1) / kFlashKeys;
+    const uint32_t *tab = p.tables + (uint64_t)b * p.max_blocks_per_seq;
+
+    // first page of the walk whose id is outside the pool: columns that would read it give NaN
+    if (tid == 0) s_bad = 0xffffffffu;
+    __syncthreads();
+    for (uint32_t i = tid; i < npages; i += kFlashWaves * 64)
+        if (tab[i] >= p.num_blocks) atomicMin(&s_bad, i);
+    __syncthreads();
+    const uint32_t first_bad_tok = s_bad == 0xffffffffu ? 0xffffffffu : s_bad * kPage;
+
+    // Q^T operands and causal limits of this lane's columns
+    v8bf qb[kFlashNQ][4];
+    uint32_t lim[kFlashNQ];
+    bool valid[kFlashNQ];
+    uint64_t out_row[kFlashNQ];
+#pragma unroll
+    for (int qi = 0; qi < kFlashNQ; ++qi) {
+        const uint32_t col = (uint32_t)wave * (kFlashNQ * 16) + qi * 16 + c;
+        const uint32_t t = t0 + col / p.group, hc = col % p.group;
+        valid[qi] = t < p.l_new;
+        const uint32_t tc = valid[qi] ? t : 0;
+        out_row[qi] = (((uint64_t)b * p.l_new + tc) * p.num_heads + (uint64_t)kvh * p.group + hc) * kDh;
+        const uint16_t *qrow = p.q + out_row[qi] + 8 * g;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            v4u t4 = *(const v4u *)(qrow + 32 * s);
+            if (!valid[qi]) t4 = v4u{0, 0, 0, 0};
+            qb[qi][s] = __builtin_bit_cast(v8bf, t4);
+        }
+        const uint32_t l = base + t + 1;
+        lim[qi] = !valid[qi] || violation ? 0 : (l < ctx ? l : ctx);
+    }
+    uint32_t wmax = 0, wmin = 0xffffffffu;
+#pragma unroll
+    for (int qi = 0; qi < kFlashNQ; ++qi) {
+        wmax = lim[qi] > wmax ? lim[qi] : wmax;
+        wmin = lim[qi] < wmin ? lim[qi] : wmin;
+    }
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const uint32_t a = __shfl_xor(wmax, off, 64), i = __shfl_xor(wmin, off, 64);
+        wmax = a > wmax ? a : wmax;
+        wmin = i < wmin ? i : wmin;
+    }
+    wmax = __builtin_amdgcn_readfirstlane(wmax);
+    wmin = __builtin_amdgcn_readfirstlane(wmin);
+
+    // staging: thread (row r of the step, 16-byte piece c16)
+    const uint32_t r_st = tid / 16, c16 = tid % 16;
+    auto stage_src = [&](uint32_t it, uint32_t &pos) -> uint64_t {
+        pos = it * kFlashKeys + r_st;
+        uint32_t pg = pos / kPage;
+        if (pg >= npages) pg = npages - 1;                      // rows past the walk repeat its last page (masked)
+        uint32_t id = tab[pg];
+        if (id >= p.num_blocks) id = 0;
+        return ((uint64_t)id * kPage + pos % kPage) * p.e_kv + (uint64_t)kvh * kDh + 8 * c16;
+    };
+    v4u kreg = v4u{0, 0, 0, 0}, vreg = v4u{0, 0, 0, 0};
+    if (n_it > 0) {
+        uint32_t pos;
+        const uint64_t off = stage_src(0, pos);
+        kreg = *(const v4u *)(p.k_pool + off);
+        vreg = *(const v4u *)(p.v_pool + off);
+        if (pos >= ctx) vreg = v4u{0, 0, 0, 0};                 // the pool may hold anything past the sequence end
+        *(v4u *)(&k_s[0][r_st * kVPitch + 8 * c16]) = kreg;
+        *(v4u *)(&v_s[0][r_st * kVPitch + 8 * c16]) = vreg;
+    }
+    __syncthreads();
+
+    float m_run[kFlashNQ], l_run[kFlashNQ];
+    v4f o[kFlashNQ][8];
+#pragma unroll
+    for (int qi = 0; qi < kFlashNQ; ++qi) {
+        m_run[qi] = -INFINITY;
+        l_run[qi] = 0.0f;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) o[qi][t] = v4f{0.f, 0.f, 0.f, 0.f};
+    }
+    constexpr float kLog2e = 1.4426950408889634f;
+
+    for (uint32_t it = 0; it < n_it; ++it) {
+        const int st = it & 1;
+        const bool more = it + 1 < n_it;
+        uint32_t pos_next = 0;
+        if (more) {
+            const uint64_t off = stage_src(it + 1, pos_next);
+            kreg = *(const v4u *)(p.k_pool + off);
+            vreg = *(const v4u *)(p.v_pool + off);
+        }
+        const uint32_t key0 = it * kFlashKeys;
+        if (key0 < wmax) {
+            // ---- scores of the step: two tiles of 16 positions
+            float sc[kFlashNQ][8];
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt) {
+                v4u ka[4];
+#pragma unroll
+                for (int s = 0; s < 4; ++s) ka[s] = *(const v4u *)(&k_s[st][(kt * 16 + c) * kVPitch + 32 * s + 8 * g]);
+#pragma unroll
+                for (int qi = 0; qi < kFlashNQ; ++qi) {
+                    v4f acc = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int s = 0; s < 4; ++s)
+                        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, ka[s]), qb[qi][s], acc, 0, 0, 0);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) sc[qi][kt * 4 + j] = acc[j] * p.scale;
+                }
+            }
+            if (key0 + kFlashKeys > wmin) {
+#pragma unroll
+                for (int qi = 0; qi < kFlashNQ; ++qi)
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        const uint32_t tok = key0 + (i / 4) * 16 + 4 * g + (i % 4);
+                        sc[qi][i] = tok < lim[qi] ? sc[qi][i] : -INFINITY;
+                    }
+            }
+            // ---- running maximum per column (lanes with equal c hold one column)
+            float m_new[kFlashNQ], m_use[kFlashNQ];
+            bool grew = false;
+#pragma unroll
+            for (int qi = 0; qi < kFlashNQ; ++qi) {
+                float m = sc[qi][0];
+#pragma unroll
+                for (int i = 1; i < 8; ++i) m = fmaxf(m, sc[qi][i]);
+                m = fmaxf(m, __shfl_xor(m, 16, 64));
+                m = fmaxf(m, __shfl_xor(m, 32, 64));
+                m_new[qi] = fmaxf(m_run[qi], m);
+                grew = grew || m_new[qi] > m_run[qi];
+                // every score of a column can be masked so far: its maximum stays -inf and the exponentials
+                // are taken against 0
+                m_use[qi] = m_new[qi] == -INFINITY ? 0.0f : m_new[qi];
+            }
+            if (__ballot(grew) != 0) {
+#pragma unroll
+                for (int qi = 0; qi < kFlashNQ; ++qi) {
+                    const float alpha = exp2f((m_run[qi] - m_use[qi]) * kLog2e);   // first step: exp2(-inf) = 0
+                    l_run[qi] *= alpha;
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) o[qi][t] = o[qi][t] * alpha;
+                }
+            }
+            v8bf p_hi[kFlashNQ], p_lo[kFlashNQ];
+#pragma unroll
+            for (int qi = 0; qi < kFlashNQ; ++qi) {
+                m_run[qi] = m_new[qi];
+                const float mb = m_use[qi] * kLog2e;
+                float sum = 0.0f;
+                v4u ph, pl;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    // masked scores: exp2(-inf) = 0
+                    const float e0 = exp2f(__builtin_fmaf(sc[qi][2 * i], kLog2e, -mb));
+                    const float e1 = exp2f(__builtin_fmaf(sc[qi][2 * i + 1], kLog2e, -mb));
+                    sum += e0 + e1;
+                    ph[i] = pack_bf16_rne(e0, e1);
+                    pl[i] = pack_bf16_rne(e0 - __uint_as_float(ph[i] << 16), e1 - __uint_as_float(ph[i] & 0xffff0000u));
+                }
+                l_run[qi] += sum;
+                p_hi[qi] = __builtin_bit_cast(v8bf, ph);
+                p_lo[qi] = __builtin_bit_cast(v8bf, pl);
+            }
+            // ---- O^T += V^T P^T
+#pragma unroll
+            for (int bp = 0; bp < 4; ++bp) {
+                uint32_t w[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    w[i] = *(const uint32_t *)(&v_s[st][((i / 4) * 16 + 4 * g + (i % 4)) * kVPitch + 32 * bp + 2 * c]);
+                v4u ae, ao;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    ae[i] = __builtin_amdgcn_perm(w[2 * i + 1], w[2 * i], 0x05040100u);
+                    ao[i] = __builtin_amdgcn_perm(w[2 * i + 1], w[2 * i], 0x07060302u);
+                }
+                const v8bf a_even = __builtin_bit_cast(v8bf, ae), a_odd = __builtin_bit_cast(v8bf, ao);
+#pragma unroll
+                for (int qi = 0; qi < kFlashNQ; ++qi) {
+                    o[qi][2 * bp] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_even, p_lo[qi], o[qi][2 * bp], 0, 0, 0);
+                    o[qi][2 * bp + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_odd, p_lo[qi], o[qi][2 * bp + 1], 0, 0, 0);
+                    o[qi][2 * bp] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_even, p_hi[qi], o[qi][2 * bp], 0, 0, 0);
+                    o[qi][2 * bp + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_odd, p_hi[qi], o[qi][2 * bp + 1], 0, 0, 0);
+                }
+            }
+        }
+        if (more) {
+            if (pos_next >= ctx) vreg = v4u{0, 0, 0, 0};
+            *(v4u *)(&k_s[st ^ 1][r_st * kVPitch + 8 * c16]) = kreg;
+            *(v4u *)(&v_s[st ^ 1][r_st * kVPitch + 8 * c16]) = vreg;
+        }
+        __syncthreads();
+    }
+
+    // lane (g, c) holds, for column c: dims 32 bp + 8 g + {0..7} = {o[2bp][0], o[2bp+1][0], o[2bp][1], ...}
+#pragma unroll
+    for (int qi = 0; qi < kFlashNQ; ++qi) {
+        float l = l_run[qi];
+        l += __shfl_xor(l, 16, 64);
+        l += __shfl_xor(l, 32, 64);
+        if (!valid[qi]) continue;
+        const bool nan_out = violation || lim[qi] > first_bad_tok;
+#pragma unroll
+        for (int bp = 0; bp < 4; ++bp) {
+            float r8[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float acc = o[qi][2 * bp + (e & 1)][e / 2];
+                float res = l > 0.0f ? __fdiv_rn(acc, l) : 0.0f;
+                r8[e] = nan_out ? __uint_as_float(0x7fc00000u) : res;
+            }
+            const uint64_t oi = out_row[qi] + 32 * bp + 8 * g;
+            if (p.out_bf16) {
+                v4u pk;
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    pk[e] = (uint32_t)f32_to_bf16(r8[2 * e]) | ((uint32_t)f32_to_bf16(r8[2 * e + 1]) << 16);
+                *(v4u *)((uint16_t *)p.out + oi) = pk;
+            } else {
+                *(v4f *)((float *)p.out + oi) = v4f{r8[0], r8[1], r8[2], r8[3]};
+                *(v4f *)((float *)p.out + oi + 4) = v4f{r8[4], r8[5], r8[6], r8[7]};
+            }
+        }
+    }
+}
+
 inline int group_pad(uint32_t group) {
     int gp = 1;
     while ((uint32_t)gp < group) gp *= 2;
@@ -759,6 +1040,7 @@ void paged_attention_generic(const void *q, const void *k_pool, const void *v_po
 
 }  // namespace k
 int g_decode_partials_only = 0;   // profiling: launch only the streaming kernel (the output is not written)
+int g_prefill_block_form = 0;     // 0: by shape, 1: never, 2: whenever the group size allows
 namespace k {
 
 static uint32_t compute_units() {
@@ -863,10 +1145,46 @@ uint64_t paged_prefill_workspace_bytes(const PagedShape &ps, uint32_t waves_per_
     return items * (16 * kDh + 2 * 16) * sizeof(float);
 }
 
+// The block form pays when its tiles are reasonably full and there are enough of them to occupy the
+// device; few new tokens against a long cache stay on the streamed form, which splits the cache walk.
+static bool prefill_block_form(const PagedShape &ps) {
+    const uint32_t group = ps.num_heads / ps.num_kv_heads;
+    if (group == 0 || group > 16 || (group & (group - 1)) != 0) return false;
+    if (g_prefill_block_form == 1) return false;
+    if (g_prefill_block_form == 2) return true;
+    const uint32_t tq = kFlashCols / group;
+    const uint64_t blocks = (uint64_t)ps.batch * ps.num_kv_heads * ((ps.l_new + tq - 1) / tq);
+    return ps.l_new * 2 >= tq && blocks * 4 >= compute_units();
+}
+
 void paged_attention_prefill_bf16(const uint16_t *q, const uint16_t *k_pool, const uint16_t *v_pool,
                                   const uint32_t *tables, const uint32_t *seq_lens, const PagedShape &ps,
                                   uint32_t waves_per_cu, void *workspace, void *out, int out_bf16, hipStream_t s) {
     if (ps.batch == 0 || ps.l_new == 0) return;
+    if (prefill_block_form(ps)) {
+        FlashParams fp;
+        fp.q = q;
+        fp.k_pool = k_pool;
+        fp.v_pool = v_pool;
+        fp.tables = tables;
+        fp.seq_lens = seq_lens;
+        fp.out = out;
+        fp.out_bf16 = out_bf16;
+        fp.num_blocks = ps.num_blocks;
+        fp.e_kv = ps.e_kv;
+        fp.batch = ps.batch;
+        fp.num_heads = ps.num_heads;
+        fp.num_kv_heads = ps.num_kv_heads;
+        fp.group = ps.num_heads / ps.num_kv_heads;
+        fp.max_blocks_per_seq = ps.max_blocks_per_seq;
+        fp.l_new = ps.l_new;
+        fp.tq = kFlashCols / fp.group;
+        fp.tiles = (ps.l_new + fp.tq - 1) / fp.tq;
+        fp.scale = ps.scale;
+        const uint64_t blocks = (uint64_t)ps.batch * ps.num_kv_heads * fp.tiles;
+        prefill_flash_kernel<<<(unsigned)blocks, kFlashWaves * 64, 0, s>>>(fp);
+        return;
+    }
     StreamParams sp;
     sp.q = q;
     sp.k_pool = k_pool;

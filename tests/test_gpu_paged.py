@@ -248,6 +248,9 @@ PREFILL_CASES = [
     (32, 8, 16, [16, 17, 64]), (32, 8, 17, [17, 31, 200]), (32, 8, 37, [37, 38, 500]), (32, 8, 200, [200, 333, 777]),
     (8, 8, 19, [19, 40]), (8, 4, 9, [9, 100]), (16, 2, 11, [11, 64]), (16, 1, 6, [6, 90]), (6, 2, 13, [13, 70]),
     (5, 1, 7, [7, 40]),
+    # several tiles of the block form (256 / group new tokens per tile), ragged last tiles
+    (32, 8, 300, [300, 1000]), (8, 8, 600, [600, 700]), (16, 2, 100, [100, 250]), (16, 1, 50, [50, 51, 333]),
+    (4, 2, 129, [129, 640]),
 ]
 
 
@@ -277,6 +280,19 @@ def test_bf16_prefill_on_the_streaming_kernel_against_the_oracle(heads, kv_heads
         got = be.download_owned(be.paged_attention_forward(dq, dk, dv, tables, seq_lens, args, out_dtype=fa.capi.F32))
         assert_parity("PAGED_PREFILL_PARITY", f"H{heads}/{kv_heads}:L{l_new}:waves{waves}", got, want)
     fa.check(fa.capi.lib.fa_set_tuning(2, 0))
+    # the block form (one block per tile of 256 / group new tokens walks the cache once), forced for every
+    # group size it supports whatever the shape heuristics would choose
+    fa.check(fa.capi.lib.fa_set_tuning(10, 2))
+    blk = be.download_owned(be.paged_attention_forward(dq, dk, dv, tables, seq_lens, args, out_dtype=fa.capi.F32))
+    assert_parity("PAGED_PREFILL_PARITY", f"H{heads}/{kv_heads}:L{l_new}:block form", blk, want)
+    blk_bf = be.download_owned(be.paged_attention_forward(dq, dk, dv, tables, seq_lens, args))
+    assert_bf16_rounding_of("paged prefill bf16, block form", blk_bf, blk)
+    blk_dev = be.download_owned(be.paged_attention_forward_device(dq, dk, dv, be.upload(tables), be.upload(seq_lens), args))
+    assert np.array_equal(blk_dev, blk_bf)
+    for h in range(heads):
+        gq = h // (heads // kv_heads)
+        assert np.array_equal(blk_bf[0, 0, h * 128:(h + 1) * 128], vp[tables[0, 0], 0, gq * 128:(gq + 1) * 128])
+    fa.check(fa.capi.lib.fa_set_tuning(10, 1))
     got = be.download_owned(be.paged_attention_forward(dq, dk, dv, tables, seq_lens, args, out_dtype=fa.capi.F32))
     got_bf = be.download_owned(be.paged_attention_forward(dq, dk, dv, tables, seq_lens, args))
     assert_bf16_rounding_of("paged prefill bf16", got_bf, got)      # same launch shape: same f32 values
@@ -293,6 +309,8 @@ def test_bf16_prefill_on_the_streaming_kernel_against_the_oracle(heads, kv_heads
     dec = be.download_owned(be.paged_attention_forward(be.upload(q_last), dk, dv, tables, seq_lens, args1,
                                                        out_dtype=fa.capi.F32))
     assert_parity("PREFILL_LAST_VS_DECODE", f"H{heads}/{kv_heads}:L{l_new}", got[:, -1:, :], dec)
+    assert_parity("PREFILL_LAST_VS_DECODE", f"H{heads}/{kv_heads}:L{l_new}:block form", blk[:, -1:, :], dec)
+    fa.check(fa.capi.lib.fa_set_tuning(10, 0))
 
 
 def test_bf16_prefill_in_several_launches_matches_one_token_at_a_time():
@@ -310,21 +328,25 @@ def test_bf16_prefill_in_several_launches_matches_one_token_at_a_time():
     layout = fa.PagedKvLayout.new(num_blocks, 16, e_kv)
     args = fa.PagedAttentionArgs(layout, batch, l_new, heads, max_blocks, fa.default_scale(128), kv_heads)
     dq, dk, dv = be.upload(q), be.upload(kp), be.upload(vp)
-    got = be.download_owned(be.paged_attention_forward(dq, dk, dv, tables, seq_lens, args, out_dtype=fa.capi.F32))
-    assert np.all(np.isfinite(got))
-    args1 = fa.PagedAttentionArgs(layout, batch, 1, heads, max_blocks, fa.default_scale(128), kv_heads)
-    for t in (0, 1, 3, 4, 170, 171, 682, 683, 684, 799):
-        lens_t = (seq_lens - l_new + t + 1).astype(np.uint32)
-        dec = be.download_owned(be.paged_attention_forward(be.upload(np.ascontiguousarray(q[:, t:t + 1, :])), dk, dv,
-                                                           tables, lens_t, args1, out_dtype=fa.capi.F32))
-        assert_parity("PREFILL_VS_DECODE", f"t{t}", got[:, t:t + 1, :], dec)
     oargs = o.paged_args(num_blocks, 16, e_kv, 1, l_new, heads, max_blocks, args.scale, kv_heads)
     o.set_threads(8)
     rc, want = o.paged_attention_bf16(np.ascontiguousarray(q[4:5]), kp, vp, np.ascontiguousarray(tables[4:5]),
                                       np.ascontiguousarray(seq_lens[4:5]), oargs)
     o.set_threads(1)
     assert rc == 0
-    assert_parity("PAGED_PREFILL_PARITY", "row4 of 6 x 800", got[4:5], want)
+    args1 = fa.PagedAttentionArgs(layout, batch, 1, heads, max_blocks, fa.default_scale(128), kv_heads)
+    # 1: the streamed form in several launches; 0: what the shape selects by itself (the block form, 13 tiles a row)
+    for form in (1, 0):
+        fa.check(fa.capi.lib.fa_set_tuning(10, form))
+        got = be.download_owned(be.paged_attention_forward(dq, dk, dv, tables, seq_lens, args, out_dtype=fa.capi.F32))
+        assert np.all(np.isfinite(got))
+        for t in (0, 1, 3, 4, 63, 64, 170, 171, 682, 683, 684, 799):
+            lens_t = (seq_lens - l_new + t + 1).astype(np.uint32)
+            dec = be.download_owned(be.paged_attention_forward(be.upload(np.ascontiguousarray(q[:, t:t + 1, :])), dk, dv,
+                                                               tables, lens_t, args1, out_dtype=fa.capi.F32))
+            assert_parity("PREFILL_VS_DECODE", f"form{form}:t{t}", got[:, t:t + 1, :], dec)
+        assert_parity("PAGED_PREFILL_PARITY", f"form{form}:row4 of 6 x 800", got[4:5], want)
+    fa.check(fa.capi.lib.fa_set_tuning(10, 0))
 
 
 def test_bf16_generic_path_covers_shapes_outside_the_fast_path():
@@ -374,3 +396,34 @@ def test_device_tables_flag_violations_with_nan():
     be.paged_kv_append_device(be.upload(rows), be.upload(rows), kpool, vpool, be.upload(slots), layout)
     pool = be.download(kpool).reshape(-1, e_kv)
     assert np.array_equal(pool[5], rows[0]) and not np.delete(pool, 5, axis=0).any()
+
+
+def test_block_form_prefill_flags_violations_per_column():
+    """Device tables, 40 new tokens: a page id outside the pool gives NaN in exactly the columns whose causal
+    range reaches that page; a row whose length is below its new tokens is NaN throughout."""
+    fa = _fa()
+    be = ops()
+    rng = o.Rng(33)
+    heads, kv_heads, num_blocks, l_new = 8, 2, 64, 40
+    tables, lens, max_blocks, e_kv, e_q = _decode_case(rng, 3, heads, kv_heads, [100, 60, 60], num_blocks)
+    kp, vp = o.to_bf16(rng.randn((num_blocks, 16, e_kv))), o.to_bf16(rng.randn((num_blocks, 16, e_kv)))
+    q = o.to_bf16(rng.randn((3, l_new, e_q)))
+    layout = fa.PagedKvLayout.new(num_blocks, 16, e_kv)
+    args = fa.PagedAttentionArgs(layout, 3, l_new, heads, max_blocks, fa.default_scale(128), kv_heads)
+    oargs = o.paged_args(num_blocks, 16, e_kv, 3, l_new, heads, max_blocks, args.scale, kv_heads)
+    rc, want = o.paged_attention_bf16(q, kp, vp, tables, lens, oargs)
+    assert rc == 0
+    bad_t = tables.copy()
+    bad_t[1, 2] = num_blocks + 9                    # row 1: positions 32 .. 47 are unreachable
+    bad_l = lens.copy()
+    bad_l[2] = l_new - 1                            # row 2: fewer positions than new tokens
+    fa.check(fa.capi.lib.fa_set_tuning(10, 2))
+    try:
+        got = be.download_owned(be.paged_attention_forward_device(
+            be.upload(q), be.upload(kp), be.upload(vp), be.upload(bad_t), be.upload(bad_l), args, out_dtype=fa.capi.F32))
+    finally:
+        fa.check(fa.capi.lib.fa_set_tuning(10, 0))
+    assert_parity("PAGED_PREFILL_PARITY", "row 0 beside violations", got[0:1], want[0:1])
+    # row 1: 20 positions were cached, token t sees positions < 21 + t, so tokens 0 .. 11 stay below position 32
+    assert_parity("PAGED_PREFILL_PARITY", "row 1 before the bad page", got[1:2, :12], want[1:2, :12])
+    assert np.all(np.isnan(got[1, 12:])) and np.all(np.isnan(got[2]))
