@@ -52,8 +52,9 @@ bool stream_fast_path(const k::PagedShape &ps, const fa_buffer *q) {
 // shared tail of the two attention entry points: tables already on the device
 fa_status launch_attention(fa_context *ctx, const fa_buffer *q, const fa_buffer *k_pool, const fa_buffer *v_pool,
                            const uint32_t *d_tables, const uint32_t *d_lens, const fa_paged_args *args,
-                           uint64_t s_stride, fa_buffer *out) {
+                           uint64_t s_stride, uint32_t ctx_hint, fa_buffer *out) {
     k::PagedShape ps = make_shape(args);
+    ps.ctx_hint = ctx_hint;
     if (stream_fast_path(ps, q) && ps.l_new > 1 && !g_prefill_generic) {
         uint64_t need = k::paged_prefill_workspace_bytes(ps, (uint32_t)g_decode_waves);
         if (fa_status s = ensure_workspace(ctx, need)) return s;
@@ -175,8 +176,10 @@ fa_status fa_paged_attention_forward(fa_context *ctx, const fa_buffer *q, const 
         e = hipMemcpyAsync((char *)ctx->table_stage + lens_off, seq_lens, lb, hipMemcpyHostToDevice, ctx->stream);
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
     if (e != hipSuccess) return hip_fail(ctx, e, "block table upload", FA_ERR_TRANSFER_FAILED);
+    uint32_t longest = 0;
+    for (uint64_t i = 0; i < n_seq; ++i) longest = seq_lens[i] > longest ? seq_lens[i] : longest;
     return launch_attention(ctx, q, k_pool, v_pool, (const uint32_t *)ctx->table_stage,
-                            (const uint32_t *)((char *)ctx->table_stage + lens_off), args, plan.s_max, out);
+                            (const uint32_t *)((char *)ctx->table_stage + lens_off), args, plan.s_max, longest, out);
 }
 
 fa_status fa_paged_attention_forward_device(fa_context *ctx, const fa_buffer *q, const fa_buffer *k_pool,
@@ -202,7 +205,7 @@ fa_status fa_paged_attention_forward_device(fa_context *ctx, const fa_buffer *q,
     if (query_rows > (uint64_t)INT32_MAX) return fail(FA_ERR_INVALID_ARGUMENT, "paged_kv: B * H * L_new exceeds i32::MAX");
     uint64_t s_stride = args->max_blocks_per_seq * l->block_size;     // longest sequence the tables can describe
     return launch_attention(ctx, q, k_pool, v_pool, (const uint32_t *)block_tables->ptr,
-                            (const uint32_t *)seq_lens->ptr, args, s_stride, out);
+                            (const uint32_t *)seq_lens->ptr, args, s_stride, 0, out);
 }
 
 }  // extern "C"

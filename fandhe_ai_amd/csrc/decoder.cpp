@@ -262,6 +262,7 @@ fa_status enqueue_prefill_chunk(fa_context *ctx, fa_decoder *d, PrefillBuffers &
     ps.head_dim = c.head_dim;
     ps.max_blocks_per_seq = c.max_blocks_per_seq;
     ps.scale = 1.0f / std::sqrt((float)c.head_dim);
+    for (uint32_t b = 0; b < B; ++b) ps.ctx_hint = std::max(ps.ctx_hint, d->host_lens[b] + lc);
 
     // y = dequant(xq @ w) (+ residual) for the rows quantized into t.xq / t.sx just before
     auto gemm = [&](const fa_qweight *w, float *out, const float *residual) {

@@ -719,19 +719,18 @@ __global__ void __launch_bounds__(1024) decode_stream_merge_quantize_kernel(Stre
 }
 
 // ------------------------------------------------------- prefill, block form
-// Causal attention of many new tokens per row, one block per (row, kv head, tile of 256 / group new
-// tokens).  The block walks the cached positions once, 32 at a time: the K and V rows of a step are
-// staged in LDS (two stages; the loads of the next step are in flight while this one is multiplied)
-// and shared by the eight wavefronts, so K / V leave the L2 once per 256 / group new tokens.  Every
+// Causal attention of many new tokens per row, one block of NW wavefronts per (row, kv head, tile of
+// 32 NW / group new tokens).  The block walks the cached positions once, 32 at a time: the K and V rows
+// of a step are staged in LDS (two stages; the loads of the next three steps are in flight while this
+// one is multiplied) and shared by the wavefronts, so K / V leave the L2 once per tile.  Every
 // wavefront owns 32 columns (new token x head of the group, column = token * group + head):
 //   S^T = K Q^T on v_mfma_f32_16x16x32_bf16 as in the decode kernel (lane (g, c): positions 4g .. 4g+3
 //   of a 16-position tile for column c), two position tiles per step;
 //   O^T += V^T P^T on the same instruction with k = the 32 positions of the step: the operand slot
 //   8g + i of a lane is position 4g + i of the first tile (i < 4) or of the second (i >= 4), which is
 //   where the scores of that lane already are; V^T is read from the staged rows 4 bytes (two dims of
-//   one position) at a time and split into an even and an odd operand by byte permutes.  A weight is
-//   fed as two bf16 terms, the value rounded to nearest and the remainder rounded to nearest (relative
-//   error of a weight <= 2^-18, unbiased).
+//   one position) at a time and split into an even and an odd operand by byte permutes.  Every f32
+//   weight is fed as three bf16 terms that add up to it exactly, as in the decode kernel.
 // The running maximum is per column; accumulators are rescaled only on steps where some column's maximum
 // grew.  A step wholly past the causal limit of all the columns of a wavefront is skipped by it.  The
 // result is normalised and written by the block itself (no partial results, no merge pass).
@@ -743,17 +742,11 @@ struct FlashParams {
     uint32_t num_blocks, e_kv, batch, num_heads, num_kv_heads, group, max_blocks_per_seq, l_new, tq, tiles;
     float scale;
 };
-constexpr int kFlashWaves = 8, kFlashNQ = 2, kFlashKeys = 32;
-constexpr int kFlashCols = kFlashWaves * kFlashNQ * 16;
+constexpr int kFlashNQ = 2, kFlashKeys = 32;
 
-// two f32 values rounded to nearest-even bf16, first value in the low half
-typedef float v2f __attribute__((ext_vector_type(2)));
-typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ uint32_t pack_bf16_rne(float a, float b) {
-    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{a, b}, v2bf));
-}
-
-__global__ void __launch_bounds__(kFlashWaves * 64) prefill_flash_kernel(FlashParams p) {
+template <int NW>
+__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) prefill_flash_kernel(FlashParams p) {
+    constexpr int kRows = NW * 4, kPasses = kFlashKeys / kRows;   // staging: rows per pass of the block, passes per step
     __shared__ __attribute__((aligned(16))) uint16_t k_s[2][kFlashKeys * kVPitch];
     __shared__ __attribute__((aligned(16))) uint16_t v_s[2][kFlashKeys * kVPitch];
     __shared__ uint32_t s_bad;
@@ -779,7 +772,7 @@ __global__ void __launch_bounds__(kFlashWaves * 64) prefill_flash_kernel(FlashPa
     // first page of the walk whose id is outside the pool: columns that would read it give NaN
     if (tid == 0) s_bad = 0xffffffffu;
     __syncthreads();
-    for (uint32_t i = tid; i < npages; i += kFlashWaves * 64)
+    for (uint32_t i = tid; i < npages; i += NW * 64)
         if (tab[i] >= p.num_blocks) atomicMin(&s_bad, i);
     __syncthreads();
     const uint32_t first_bad_tok = s_bad == 0xffffffffu ? 0xffffffffu : s_bad * kPage;
@@ -821,25 +814,42 @@ __global__ void __launch_bounds__(kFlashWaves * 64) prefill_flash_kernel(FlashPa
     wmax = __builtin_amdgcn_readfirstlane(wmax);
     wmin = __builtin_amdgcn_readfirstlane(wmin);
 
-    // staging: thread (row r of the step, 16-byte piece c16)
-    const uint32_t r_st = tid / 16, c16 = tid % 16;
-    auto stage_src = [&](uint32_t it, uint32_t &pos) -> uint64_t {
-        pos = it * kFlashKeys + r_st;
-        uint32_t pg = pos / kPage;
-        if (pg >= npages) pg = npages - 1;                      // rows past the walk repeat its last page (masked)
-        uint32_t id = tab[pg];
-        if (id >= p.num_blocks) id = 0;
-        return ((uint64_t)id * kPage + pos % kPage) * p.e_kv + (uint64_t)kvh * kDh + 8 * c16;
+    // staging: thread (row r of the step, 16-byte piece c16).  Page ids are requested four steps and K / V
+    // rows three steps ahead of the step that multiplies them, so neither the id -> row dependence nor the
+    // row loads themselves are waited for; steps past the walk repeat its last page (never used).
+    const uint32_t r_st = tid / 16, c16 = tid % 16;           // pass ps stages row r_st + ps * kRows
+    auto load_id = [&](uint32_t it, int ps) -> uint32_t {
+        uint32_t pg = (it * kFlashKeys + ps * kRows + r_st) / kPage;
+        if (pg >= npages) pg = npages - 1;
+        return tab[pg];
     };
-    v4u kreg = v4u{0, 0, 0, 0}, vreg = v4u{0, 0, 0, 0};
+    auto row_off = [&](uint32_t it, int ps, uint32_t id) -> uint64_t {
+        if (id >= p.num_blocks) id = 0;
+        return ((uint64_t)id * kPage + (it * kFlashKeys + ps * kRows + r_st) % kPage) * p.e_kv + (uint64_t)kvh * kDh + 8 * c16;
+    };
+    v4u k_a[kPasses], v_a[kPasses], k_b[kPasses], v_b[kPasses];  // rows of step it + 1 (a) and it + 2 (b)
+    uint32_t id_c[kPasses];                                      // page ids of step it + 3
+#pragma unroll
+    for (int ps = 0; ps < kPasses; ++ps) {
+        k_a[ps] = v_a[ps] = k_b[ps] = v_b[ps] = v4u{0, 0, 0, 0};
+        id_c[ps] = 0;
+    }
     if (n_it > 0) {
-        uint32_t pos;
-        const uint64_t off = stage_src(0, pos);
-        kreg = *(const v4u *)(p.k_pool + off);
-        vreg = *(const v4u *)(p.v_pool + off);
-        if (pos >= ctx) vreg = v4u{0, 0, 0, 0};                 // the pool may hold anything past the sequence end
-        *(v4u *)(&k_s[0][r_st * kVPitch + 8 * c16]) = kreg;
-        *(v4u *)(&v_s[0][r_st * kVPitch + 8 * c16]) = vreg;
+#pragma unroll
+        for (int ps = 0; ps < kPasses; ++ps) {
+            const uint32_t id0 = load_id(0, ps), id1 = load_id(1, ps), id2 = load_id(2, ps);
+            id_c[ps] = load_id(3, ps);
+            const uint64_t off0 = row_off(0, ps, id0), off1 = row_off(1, ps, id1), off2 = row_off(2, ps, id2);
+            v4u k0 = *(const v4u *)(p.k_pool + off0), v0 = *(const v4u *)(p.v_pool + off0);
+            k_a[ps] = *(const v4u *)(p.k_pool + off1);
+            v_a[ps] = *(const v4u *)(p.v_pool + off1);
+            k_b[ps] = *(const v4u *)(p.k_pool + off2);
+            v_b[ps] = *(const v4u *)(p.v_pool + off2);
+            const uint32_t row = ps * kRows + r_st;
+            if (row >= ctx) v0 = v4u{0, 0, 0, 0};               // the pool may hold anything past the sequence end
+            *(v4u *)(&k_s[0][row * kVPitch + 8 * c16]) = k0;
+            *(v4u *)(&v_s[0][row * kVPitch + 8 * c16]) = v0;
+        }
     }
     __syncthreads();
 
@@ -856,12 +866,16 @@ __global__ void __launch_bounds__(kFlashWaves * 64) prefill_flash_kernel(FlashPa
 
     for (uint32_t it = 0; it < n_it; ++it) {
         const int st = it & 1;
-        const bool more = it + 1 < n_it;
-        uint32_t pos_next = 0;
-        if (more) {
-            const uint64_t off = stage_src(it + 1, pos_next);
-            kreg = *(const v4u *)(p.k_pool + off);
-            vreg = *(const v4u *)(p.v_pool + off);
+        // requests of this step: the rows of step it + 3 (their page id was requested one step ago) and the
+        // page id of step it + 4
+        v4u k_n[kPasses], v_n[kPasses];
+#pragma unroll
+        for (int ps = 0; ps < kPasses; ++ps) {
+            const uint32_t id_use = id_c[ps];
+            id_c[ps] = load_id(it + 4, ps);
+            const uint64_t off_n = row_off(it + 3, ps, id_use);
+            k_n[ps] = *(const v4u *)(p.k_pool + off_n);
+            v_n[ps] = *(const v4u *)(p.v_pool + off_n);
         }
         const uint32_t key0 = it * kFlashKeys;
         if (key0 < wmax) {
@@ -910,30 +924,41 @@ __global__ void __launch_bounds__(kFlashWaves * 64) prefill_flash_kernel(FlashPa
             if (__ballot(grew) != 0) {
 #pragma unroll
                 for (int qi = 0; qi < kFlashNQ; ++qi) {
-                    const float alpha = exp2f((m_run[qi] - m_use[qi]) * kLog2e);   // first step: exp2(-inf) = 0
+                    const float alpha = __builtin_amdgcn_exp2f((m_run[qi] - m_use[qi]) * kLog2e);   // first step: exp2(-inf) = 0
                     l_run[qi] *= alpha;
 #pragma unroll
                     for (int t = 0; t < 8; ++t) o[qi][t] = o[qi][t] * alpha;
                 }
             }
-            v8bf p_hi[kFlashNQ], p_lo[kFlashNQ];
+            // each f32 weight as three bf16 operands by repeated truncation: hi + mid + lo == weight exactly
+            v8bf p_hi[kFlashNQ], p_mid[kFlashNQ], p_lo[kFlashNQ];
 #pragma unroll
             for (int qi = 0; qi < kFlashNQ; ++qi) {
                 m_run[qi] = m_new[qi];
-                const float mb = m_use[qi] * kLog2e;
                 float sum = 0.0f;
-                v4u ph, pl;
+                v4u ph, pm, pl;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    // masked scores: exp2(-inf) = 0
-                    const float e0 = exp2f(__builtin_fmaf(sc[qi][2 * i], kLog2e, -mb));
-                    const float e1 = exp2f(__builtin_fmaf(sc[qi][2 * i + 1], kLog2e, -mb));
-                    sum += e0 + e1;
-                    ph[i] = pack_bf16_rne(e0, e1);
-                    pl[i] = pack_bf16_rne(e0 - __uint_as_float(ph[i] << 16), e1 - __uint_as_float(ph[i] & 0xffff0000u));
+                    float e[2];
+                    uint32_t hi[2], mid[2], lo[2];
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+                        // the difference is exact for scores near the maximum, which carry the weight;
+                        // masked scores: exp2(-inf) = 0
+                        e[h] = __builtin_amdgcn_exp2f((sc[qi][2 * i + h] - m_use[qi]) * kLog2e);
+                        hi[h] = __float_as_uint(e[h]) & 0xffff0000u;
+                        const float r1 = e[h] - __uint_as_float(hi[h]);
+                        mid[h] = __float_as_uint(r1) & 0xffff0000u;
+                        lo[h] = __float_as_uint(r1 - __uint_as_float(mid[h]));
+                    }
+                    sum += e[0] + e[1];
+                    ph[i] = __builtin_amdgcn_perm(hi[1], hi[0], 0x07060302u);
+                    pm[i] = __builtin_amdgcn_perm(mid[1], mid[0], 0x07060302u);
+                    pl[i] = __builtin_amdgcn_perm(lo[1], lo[0], 0x07060302u);
                 }
                 l_run[qi] += sum;
                 p_hi[qi] = __builtin_bit_cast(v8bf, ph);
+                p_mid[qi] = __builtin_bit_cast(v8bf, pm);
                 p_lo[qi] = __builtin_bit_cast(v8bf, pl);
             }
             // ---- O^T += V^T P^T
@@ -952,17 +977,27 @@ __global__ void __launch_bounds__(kFlashWaves * 64) prefill_flash_kernel(FlashPa
                 const v8bf a_even = __builtin_bit_cast(v8bf, ae), a_odd = __builtin_bit_cast(v8bf, ao);
 #pragma unroll
                 for (int qi = 0; qi < kFlashNQ; ++qi) {
+                    // smallest terms first
                     o[qi][2 * bp] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_even, p_lo[qi], o[qi][2 * bp], 0, 0, 0);
                     o[qi][2 * bp + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_odd, p_lo[qi], o[qi][2 * bp + 1], 0, 0, 0);
+                    o[qi][2 * bp] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_even, p_mid[qi], o[qi][2 * bp], 0, 0, 0);
+                    o[qi][2 * bp + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_odd, p_mid[qi], o[qi][2 * bp + 1], 0, 0, 0);
                     o[qi][2 * bp] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_even, p_hi[qi], o[qi][2 * bp], 0, 0, 0);
                     o[qi][2 * bp + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_odd, p_hi[qi], o[qi][2 * bp + 1], 0, 0, 0);
                 }
             }
         }
-        if (more) {
-            if (pos_next >= ctx) vreg = v4u{0, 0, 0, 0};
-            *(v4u *)(&k_s[st ^ 1][r_st * kVPitch + 8 * c16]) = kreg;
-            *(v4u *)(&v_s[st ^ 1][r_st * kVPitch + 8 * c16]) = vreg;
+        // rows of step it + 1 go to the other stage (its readers passed the barrier of the last step)
+#pragma unroll
+        for (int ps = 0; ps < kPasses; ++ps) {
+            const uint32_t row = ps * kRows + r_st;
+            if ((it + 1) * kFlashKeys + row >= ctx) v_a[ps] = v4u{0, 0, 0, 0};
+            *(v4u *)(&k_s[st ^ 1][row * kVPitch + 8 * c16]) = k_a[ps];
+            *(v4u *)(&v_s[st ^ 1][row * kVPitch + 8 * c16]) = v_a[ps];
+            k_a[ps] = k_b[ps];
+            v_a[ps] = v_b[ps];
+            k_b[ps] = k_n[ps];
+            v_b[ps] = v_n[ps];
         }
         __syncthreads();
     }
@@ -1041,6 +1076,7 @@ void paged_attention_generic(const void *q, const void *k_pool, const void *v_po
 }  // namespace k
 int g_decode_partials_only = 0;   // profiling: launch only the streaming kernel (the output is not written)
 int g_prefill_block_form = 0;     // 0: by shape, 1: never, 2: whenever the group size allows
+int g_prefill_block_waves = 0;    // wavefronts per block of the block form: 4 or 8, anything else by shape
 namespace k {
 
 static uint32_t compute_units() {
@@ -1145,23 +1181,49 @@ uint64_t paged_prefill_workspace_bytes(const PagedShape &ps, uint32_t waves_per_
     return items * (16 * kDh + 2 * 16) * sizeof(float);
 }
 
-// The block form pays when its tiles are reasonably full and there are enough of them to occupy the
-// device; few new tokens against a long cache stay on the streamed form, which splits the cache walk.
-static bool prefill_block_form(const PagedShape &ps) {
+// Which prefill form a shape takes.  The block form walks the cache once per tile of new tokens, so its time
+// is the longest walk (a lone block does a step of 32 positions in about 1.4 us) or, when blocks queue, the sum
+// of the walks over the compute units; the streamed form splits every walk over the whole device but reads
+// K / V once per 32 / group new tokens and merges partial results per new token.  The constants are measured
+// (32 / 8 heads): they only need to be right where the two forms are far apart, which is where it matters.
+struct BlockFormPlan {
+    bool use;
+    int waves;
+};
+static BlockFormPlan plan_block_form(const PagedShape &ps) {
     const uint32_t group = ps.num_heads / ps.num_kv_heads;
-    if (group == 0 || group > 16 || (group & (group - 1)) != 0) return false;
-    if (g_prefill_block_form == 1) return false;
-    if (g_prefill_block_form == 2) return true;
-    const uint32_t tq = kFlashCols / group;
-    const uint64_t blocks = (uint64_t)ps.batch * ps.num_kv_heads * ((ps.l_new + tq - 1) / tq);
-    return ps.l_new * 2 >= tq && blocks * 4 >= compute_units();
+    if (group == 0 || group > 16 || (group & (group - 1)) != 0 || g_prefill_block_form == 1) return {false, 0};
+    const uint32_t cus = compute_units();
+    const uint32_t bound = ps.max_blocks_per_seq * kPage;
+    uint32_t ctx = ps.ctx_hint != 0 && ps.ctx_hint < bound ? ps.ctx_hint : bound;
+    if (ctx < ps.l_new) ctx = ps.l_new;
+    const double cached = (double)(ctx - ps.l_new), l_new = (double)ps.l_new;
+    const uint64_t rows = (uint64_t)ps.batch * ps.num_kv_heads;
+    int waves = g_prefill_block_waves == 8 ? 8 : g_prefill_block_waves == 4 ? 4 : 0;
+    if (waves == 0) {
+        // eight wavefronts halve the K / V traffic of a block pair; they pay once the device is oversubscribed
+        const uint32_t tq8 = 256 / group;
+        waves = rows * ((ps.l_new + tq8 - 1) / tq8) >= 2ull * cus && ps.l_new >= 1024 ? 8 : 4;
+    }
+    if (g_prefill_block_form == 2) return {true, waves};
+    const uint32_t tq = (uint32_t)waves * kFlashNQ * 16 / group, tiles = (ps.l_new + tq - 1) / tq;
+    const double steps_longest = (cached + l_new) / kFlashKeys;
+    const double steps_all = (double)(rows * tiles) * (cached + (tiles > 1 ? 0.5 * l_new : l_new)) / kFlashKeys;
+    const double per_cu = waves == 8 ? 2.05 : 1.05;                       // us per step at two wavefronts per SIMD
+    const double a = steps_longest * 1.4, b = steps_all / cus * per_cu;
+    const double t_block = (a > b ? a : b) + 8.0;
+    const uint32_t tpt = 16 / group, tpv = ps.l_new > tpt ? 2 * tpt : tpt;
+    const double bytes = (double)rows * ((ps.l_new + tpv - 1) / tpv) * (cached + 0.5 * l_new) * (2.0 * kDh * 2);
+    const double t_stream = 35.0 + bytes / 4.9e6 + 0.035 * l_new * ps.batch;
+    return {t_block <= t_stream, waves};
 }
 
 void paged_attention_prefill_bf16(const uint16_t *q, const uint16_t *k_pool, const uint16_t *v_pool,
                                   const uint32_t *tables, const uint32_t *seq_lens, const PagedShape &ps,
                                   uint32_t waves_per_cu, void *workspace, void *out, int out_bf16, hipStream_t s) {
     if (ps.batch == 0 || ps.l_new == 0) return;
-    if (prefill_block_form(ps)) {
+    const BlockFormPlan plan = plan_block_form(ps);
+    if (plan.use) {
         FlashParams fp;
         fp.q = q;
         fp.k_pool = k_pool;
@@ -1178,11 +1240,14 @@ void paged_attention_prefill_bf16(const uint16_t *q, const uint16_t *k_pool, con
         fp.group = ps.num_heads / ps.num_kv_heads;
         fp.max_blocks_per_seq = ps.max_blocks_per_seq;
         fp.l_new = ps.l_new;
-        fp.tq = kFlashCols / fp.group;
+        fp.tq = (uint32_t)plan.waves * kFlashNQ * 16 / fp.group;
         fp.tiles = (ps.l_new + fp.tq - 1) / fp.tq;
         fp.scale = ps.scale;
         const uint64_t blocks = (uint64_t)ps.batch * ps.num_kv_heads * fp.tiles;
-        prefill_flash_kernel<<<(unsigned)blocks, kFlashWaves * 64, 0, s>>>(fp);
+        if (plan.waves == 8)
+            prefill_flash_kernel<8><<<(unsigned)blocks, 512, 0, s>>>(fp);
+        else
+            prefill_flash_kernel<4><<<(unsigned)blocks, 256, 0, s>>>(fp);
         return;
     }
     StreamParams sp;

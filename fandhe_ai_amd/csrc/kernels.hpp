@@ -138,6 +138,9 @@ struct PagedShape {
     uint32_t num_blocks, block_size, e_kv, batch, l_new, num_heads, num_kv_heads, head_dim,
         max_blocks_per_seq;
     float scale;
+    // upper bound the host knows for the positions any row holds after this call's new tokens (0: unknown,
+    // the table width is used); only steers the choice between the two prefill forms
+    uint32_t ctx_hint = 0;
 };
 // Row scatter; elem_bytes 2 or 4; slots bounds-checked against pool_rows.
 void paged_kv_append(const void *k_new, const void *v_new, void *k_pool, void *v_pool,

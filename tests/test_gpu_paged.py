@@ -283,15 +283,22 @@ def test_bf16_prefill_on_the_streaming_kernel_against_the_oracle(heads, kv_heads
     # the block form (one block per tile of 256 / group new tokens walks the cache once), forced for every
     # group size it supports whatever the shape heuristics would choose
     fa.check(fa.capi.lib.fa_set_tuning(10, 2))
-    blk = be.download_owned(be.paged_attention_forward(dq, dk, dv, tables, seq_lens, args, out_dtype=fa.capi.F32))
-    assert_parity("PAGED_PREFILL_PARITY", f"H{heads}/{kv_heads}:L{l_new}:block form", blk, want)
-    blk_bf = be.download_owned(be.paged_attention_forward(dq, dk, dv, tables, seq_lens, args))
-    assert_bf16_rounding_of("paged prefill bf16, block form", blk_bf, blk)
-    blk_dev = be.download_owned(be.paged_attention_forward_device(dq, dk, dv, be.upload(tables), be.upload(seq_lens), args))
-    assert np.array_equal(blk_dev, blk_bf)
-    for h in range(heads):
-        gq = h // (heads // kv_heads)
-        assert np.array_equal(blk_bf[0, 0, h * 128:(h + 1) * 128], vp[tables[0, 0], 0, gq * 128:(gq + 1) * 128])
+    for block_waves in (8, 4):        # tiles of 256 / group and of 128 / group new tokens
+        fa.check(fa.capi.lib.fa_set_tuning(11, block_waves))
+        blk = be.download_owned(be.paged_attention_forward(dq, dk, dv, tables, seq_lens, args, out_dtype=fa.capi.F32))
+        assert_parity("PAGED_PREFILL_PARITY", f"H{heads}/{kv_heads}:L{l_new}:block form, {block_waves} wavefronts", blk, want)
+        blk_bf = be.download_owned(be.paged_attention_forward(dq, dk, dv, tables, seq_lens, args))
+        assert_bf16_rounding_of("paged prefill bf16, block form", blk_bf, blk)
+        blk_dev = be.download_owned(be.paged_attention_forward_device(dq, dk, dv, be.upload(tables), be.upload(seq_lens), args))
+        assert np.array_equal(blk_dev, blk_bf)
+        for h in range(heads):
+            gq = h // (heads // kv_heads)
+            assert np.array_equal(blk_bf[0, 0, h * 128:(h + 1) * 128], vp[tables[0, 0], 0, gq * 128:(gq + 1) * 128])
+    fa.check(fa.capi.lib.fa_set_tuning(11, 0))
+    # whatever the shape selects by itself (host tables: the longest row is known; device tables: the table width)
+    fa.check(fa.capi.lib.fa_set_tuning(10, 0))
+    auto = be.download_owned(be.paged_attention_forward(dq, dk, dv, tables, seq_lens, args, out_dtype=fa.capi.F32))
+    assert_parity("PAGED_PREFILL_PARITY", f"H{heads}/{kv_heads}:L{l_new}:form by shape", auto, want)
     fa.check(fa.capi.lib.fa_set_tuning(10, 1))
     got = be.download_owned(be.paged_attention_forward(dq, dk, dv, tables, seq_lens, args, out_dtype=fa.capi.F32))
     got_bf = be.download_owned(be.paged_attention_forward(dq, dk, dv, tables, seq_lens, args))
@@ -419,11 +426,14 @@ def test_block_form_prefill_flags_violations_per_column():
     bad_l[2] = l_new - 1                            # row 2: fewer positions than new tokens
     fa.check(fa.capi.lib.fa_set_tuning(10, 2))
     try:
-        got = be.download_owned(be.paged_attention_forward_device(
-            be.upload(q), be.upload(kp), be.upload(vp), be.upload(bad_t), be.upload(bad_l), args, out_dtype=fa.capi.F32))
+        for block_waves in (4, 8):
+            fa.check(fa.capi.lib.fa_set_tuning(11, block_waves))
+            got = be.download_owned(be.paged_attention_forward_device(
+                be.upload(q), be.upload(kp), be.upload(vp), be.upload(bad_t), be.upload(bad_l), args, out_dtype=fa.capi.F32))
+            assert_parity("PAGED_PREFILL_PARITY", "row 0 beside violations", got[0:1], want[0:1])
+            # row 1: 20 positions were cached, token t sees positions < 21 + t: tokens 0 .. 11 stay below position 32
+            assert_parity("PAGED_PREFILL_PARITY", "row 1 before the bad page", got[1:2, :12], want[1:2, :12])
+            assert np.all(np.isnan(got[1, 12:])) and np.all(np.isnan(got[2]))
     finally:
         fa.check(fa.capi.lib.fa_set_tuning(10, 0))
-    assert_parity("PAGED_PREFILL_PARITY", "row 0 beside violations", got[0:1], want[0:1])
-    # row 1: 20 positions were cached, token t sees positions < 21 + t, so tokens 0 .. 11 stay below position 32
-    assert_parity("PAGED_PREFILL_PARITY", "row 1 before the bad page", got[1:2, :12], want[1:2, :12])
-    assert np.all(np.isnan(got[1, 12:])) and np.all(np.isnan(got[2]))
+        fa.check(fa.capi.lib.fa_set_tuning(11, 0))
