@@ -67,7 +67,8 @@ extern "C" {
 // key 0 = n-tiles per block of the skinny linears, 1 = wavefronts per block,
 // 2 = wavefronts per compute unit of the decode attention, 3 = decode attention launches its streaming
 // kernel only (timing aid), 4 = prefill GEMMs keep the 128 x 128 block tile for every shape,
-// 5 = activation-stationary decode linears (1 never, 2 whenever they can run).
+// 5 = activation-stationary decode linears (1 never, 2 whenever they can run); the remaining keys are
+// described beside the declaration.
 fa_status fa_set_tuning(int32_t key, int32_t value) {
     switch (key) {
         case 0: k::g_skinny_ntw = value; return FA_OK;
