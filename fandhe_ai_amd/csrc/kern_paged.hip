@@ -786,7 +786,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
     for (int qi = 0; qi < kFlashNQ; ++qi) {
         const uint32_t col = (uint32_t)wave * (kFlashNQ * 16) + qi * 16 + c;
         const uint32_t t = t0 + col / p.group, hc = col % p.group;
-        valid[qi] = t < p.l_new;
+        valid[qi] = col < p.tq * p.group && t < p.l_new;        // a group that does not divide the columns leaves some idle
         const uint32_t tc = valid[qi] ? t : 0;
         out_row[qi] = (((uint64_t)b * p.l_new + tc) * p.num_heads + (uint64_t)kvh * p.group + hc) * kDh;
         const uint16_t *qrow = p.q + out_row[qi] + 8 * g;
@@ -1192,7 +1192,7 @@ struct BlockFormPlan {
 };
 static BlockFormPlan plan_block_form(const PagedShape &ps) {
     const uint32_t group = ps.num_heads / ps.num_kv_heads;
-    if (group == 0 || group > 16 || (group & (group - 1)) != 0 || g_prefill_block_form == 1) return {false, 0};
+    if (group == 0 || group > 16 || g_prefill_block_form == 1) return {false, 0};
     const uint32_t cus = compute_units();
     const uint32_t bound = ps.max_blocks_per_seq * kPage;
     uint32_t ctx = ps.ctx_hint != 0 && ps.ctx_hint < bound ? ps.ctx_hint : bound;

@@ -516,8 +516,7 @@ fa_status fa_decoder_read_seq_lens(fa_context *ctx, fa_decoder *dec, uint32_t *s
  * key 9: blocks per compute unit that a split-k launch of the 128 x 128 int8 GEMM aims
  *        for (default 2);
  * key 10: form of the attention with more than one new token per row: 1 always the
- *        streamed form, 2 the block form whenever the group size is a power of two,
- *        0 by shape;
+ *        streamed form, 2 always the block form, 0 by shape;
  * key 11: wavefronts per block of that block form (4 or 8; 0 by shape). */
 fa_status fa_set_tuning(int32_t key, int32_t value);
 /* A pair of HIP events recorded on the context's stream (the stream the
