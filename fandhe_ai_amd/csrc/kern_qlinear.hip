@@ -81,9 +81,14 @@ __global__ void __launch_bounds__(NWAVES * 64)
             b[j] = nt < n_tiles ? *(const v4i *)(b_base + ((uint64_t)nt * k_tiles + kt) * 1024) : v4i{0, 0, 0, 0};
         }
     };
+    // lane l holds row l % 16 of a row tile: the rows at or past m are zeros in memory, and the lanes that
+    // would fetch them do not ask (a step of one to four rows then pulls a quarter of each activation tile)
+    const uint32_t a_row = (uint32_t)lane % 16;
     auto load_a = [&](uint32_t kt, v4i *a) {
 #pragma unroll
-        for (int i = 0; i < MT; ++i) a[i] = *(const v4i *)(a_base + ((uint64_t)i * k_tiles + kt) * 1024);
+        for (int i = 0; i < MT; ++i)
+            a[i] = (uint32_t)i * 16 + a_row < m ? *(const v4i *)(a_base + ((uint64_t)i * k_tiles + kt) * 1024)
+                                                : v4i{0, 0, 0, 0};
     };
     auto mma = [&](const v4i *a, const v4i *b) {
 #pragma unroll
