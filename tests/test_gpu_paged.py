@@ -437,3 +437,73 @@ def test_block_form_prefill_flags_violations_per_column():
     finally:
         fa.check(fa.capi.lib.fa_set_tuning(10, 0))
         fa.check(fa.capi.lib.fa_set_tuning(11, 0))
+
+
+def test_bf16_prefill_properties_at_prompt_size():
+    """4 rows x 2048 new tokens, 32 / 8 heads (the prompt pass of the benchmark): both block sizes of the block
+    form and the streamed form against each other and against one-token decode calls on sampled positions, plus
+    the invariances that hold at any size."""
+    fa = _fa()
+    be = ops()
+    rng = o.Rng(5)
+    batch, heads, kv_heads, l_new, num_blocks = 4, 32, 8, 2048, 700
+    lens = [2048, 2048 + 333, 2048 + 16, 2048 + 1]
+    tables, seq_lens, max_blocks, e_kv, e_q = _decode_case(rng, batch, heads, kv_heads, lens, num_blocks)
+    kp = o.to_bf16(rng.randn((num_blocks, 16, e_kv)))
+    vp = o.to_bf16(rng.randn((num_blocks, 16, e_kv)))
+    q = o.to_bf16(rng.randn((batch, l_new, e_q)))
+    layout = fa.PagedKvLayout.new(num_blocks, 16, e_kv)
+    args = fa.PagedAttentionArgs(layout, batch, l_new, heads, max_blocks, fa.default_scale(128), kv_heads)
+    args1 = fa.PagedAttentionArgs(layout, batch, 1, heads, max_blocks, fa.default_scale(128), kv_heads)
+    dq, dk, dv = be.upload(q), be.upload(kp), be.upload(vp)
+    lib = fa.capi.lib
+    outs = {}
+    try:
+        for name, form, waves in (("block8", 2, 8), ("block4", 2, 4), ("streamed", 1, 0), ("by shape", 0, 0)):
+            fa.check(lib.fa_set_tuning(10, form))
+            fa.check(lib.fa_set_tuning(11, waves))
+            outs[name] = be.download_owned(be.paged_attention_forward(dq, dk, dv, tables, seq_lens, args, out_dtype=fa.capi.F32))
+            assert np.all(np.isfinite(outs[name])), name
+        fa.check(lib.fa_set_tuning(10, 0))
+        fa.check(lib.fa_set_tuning(11, 0))
+        for name in ("block8", "block4", "by shape"):
+            assert_parity("PREFILL_FORMS", f"{name} vs streamed", outs[name], outs["streamed"])
+        # sampled positions against one-token decode calls over the same cache (tile edges of both block sizes)
+        for t in (0, 1, 31, 32, 63, 64, 1000, 2047):
+            lens_t = (seq_lens - l_new + t + 1).astype(np.uint32)
+            dec = be.download_owned(be.paged_attention_forward(be.upload(np.ascontiguousarray(q[:, t:t + 1, :])), dk, dv,
+                                                               tables, lens_t, args1, out_dtype=fa.capi.F32))
+            for name in ("block8", "block4"):
+                assert_parity("PREFILL_VS_DECODE", f"{name}:t{t}", outs[name][:, t:t + 1, :], dec)
+        # the oracle on the first 40 tokens of the row with the longest cache
+        oargs = o.paged_args(num_blocks, 16, e_kv, 1, 40, heads, max_blocks, args.scale, kv_heads)
+        o.set_threads(8)
+        rc, want = o.paged_attention_bf16(np.ascontiguousarray(q[1:2, :40]), kp, vp, np.ascontiguousarray(tables[1:2]),
+                                          np.array([lens[1] - l_new + 40], np.uint32), oargs)
+        o.set_threads(1)
+        assert rc == 0
+        assert_parity("PAGED_PREFILL_PARITY", "row 1, tokens 0..39", outs["block8"][1:2, :40], want)
+        got = outs["by shape"]
+        # every output is a convex combination of V rows of its kv head
+        used = tables[tables != U32MAX]
+        vmax = np.abs(o.from_bf16(vp[used])).reshape(-1, kv_heads, 128).max(axis=0)
+        bound = np.repeat(vmax, heads // kv_heads, axis=0)[None, None]
+        assert np.all(np.abs(got.reshape(batch, l_new, heads, 128)) <= bound + 1e-6)
+        # moving pages to other physical blocks changes no bit
+        perm2 = np.roll(np.arange(num_blocks), 11).astype(np.uint32)
+        kp2, vp2 = np.empty_like(kp), np.empty_like(vp)
+        kp2[perm2], vp2[perm2] = kp, vp
+        t2 = tables.copy()
+        msk = tables != U32MAX
+        t2[msk] = perm2[tables[msk]]
+        got2 = be.download_owned(be.paged_attention_forward(dq, be.upload(kp2), be.upload(vp2), t2, seq_lens, args,
+                                                            out_dtype=fa.capi.F32))
+        assert np.array_equal(got, got2)
+        # a constant V gives that constant back
+        ones = np.full_like(vp, o.to_bf16(np.array([1.5], np.float32))[0])
+        got3 = be.download_owned(be.paged_attention_forward(dq, dk, be.upload(ones), tables, seq_lens, args,
+                                                            out_dtype=fa.capi.F32))
+        assert np.allclose(got3, 1.5, rtol=1e-5, atol=0)
+    finally:
+        fa.check(lib.fa_set_tuning(10, 0))
+        fa.check(lib.fa_set_tuning(11, 0))
