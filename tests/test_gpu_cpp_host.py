@@ -1,0 +1,92 @@
+"""The C++ host layer on the device (tests/cpp/host_gpu_test.cpp) against the Python mirror: both build the same
+decoder from device-generated weights (same seeds, same order) through the same C ABI and must produce the same
+tokens from generate and from the continuous-batching scheduler."""
+import ctypes as C
+import json
+import subprocess
+
+import numpy as np
+import pytest
+
+from test_cpp_host_cpu import host_binary
+
+pytestmark = pytest.mark.gpu
+
+
+def _python_side():
+    import fandhe_ai_amd as fa
+    from fandhe_ai_amd import scheduler as sch
+    be = fa.tape_for(fa.Device.Rocm(0))
+    lib = fa.capi.lib
+    n_layers, d, heads, kv, dh, f, vocab = 2, 256, 4, 2, 128, 512, 1000
+    seed = [100]
+    keep = []
+
+    def filled(numel, mean, std):
+        b = be.alloc_uninit((numel,), fa.capi.F32)
+        fa.check(lib.fa_fill_normal(be._ctx, b._h, 0, numel, seed[0], mean, std))
+        seed[0] += 1
+        keep.append(b)
+        return b
+
+    def weight(k, n):
+        w = filled(k * n, 0.0, 0.05)
+        q = be.quantize_weight(fa.DeviceBufferView(w, 0, (k, n)))
+        keep.append(q)
+        return q
+
+    dec = fa.Decoder(be, n_layers, d, heads, kv, f, vocab, max_blocks_per_seq=8, num_blocks=48, max_batch=8,
+                     rms_eps=1e-5, rope_theta=10000.0)
+    eq, ekv = heads * dh, kv * dh
+    for l in range(n_layers):
+        an, fn = filled(d, 1.0, 0.1), filled(d, 1.0, 0.1)
+        dec.set_layer(l, an, fn, weight(d, eq + 2 * ekv), weight(eq, d), weight(d, 2 * f), weight(f, d))
+    embed, norm = filled(vocab * d, 0.0, 1.0), filled(d, 1.0, 0.1)
+    dec.set_head(embed, norm, weight(d, vocab))
+
+    G, K, T = sch.SamplingStrategy.Greedy, sch.SamplingStrategy.TopK, sch.SamplingStrategy.Temperature
+    out = {}
+    prompts = np.array([[5, 17, 900, 3, 44], [1, 2, 3, 4, 5]], np.int32)
+    out["generate_greedy"] = sch.generate(dec, prompts, sch.GenerateConfig(12, G())).tolist()
+    out["generate_top_k"] = sch.generate(dec, np.array([[8, 9, 10]], np.int32), sch.GenerateConfig(14, K(5), seed=7)).tolist()
+    out["generate_temperature"] = sch.generate(dec, prompts, sch.GenerateConfig(10, T(np.float32(0.8)), seed=3)).tolist()
+    requests = [([5, 17, 900, 3, 44], sch.GenerateConfig(12, G())),
+                ([11, 12], sch.GenerateConfig(20, K(5), seed=7)),
+                ([21, 22, 23, 24, 25, 26, 27], sch.GenerateConfig(16, T(np.float32(0.8)), seed=3)),
+                ([31], sch.GenerateConfig(9, G())),
+                ([41, 42, 43], sch.GenerateConfig(3, G())),
+                ([51, 52, 53, 54], sch.GenerateConfig(25, T(np.float32(1.3)), seed=11)),
+                ([61, 62], sch.GenerateConfig(30, K(50), seed=13))]
+    s = sch.BatchScheduler(dec, sch.SchedulerLimits(3, 16, 40))
+    for p, c in requests:
+        s.submit(np.array(p, np.int32), c)
+    done = {}
+    for _ in range(200):
+        if not (s.queued_len() or s.active_len()):
+            break
+        s.step()
+        for rid, toks in s.take_finished():
+            done[rid] = toks.tolist()
+    assert not s.take_failed() and len(done) == len(requests) and s.free_pages() == 48
+    out["scheduler"] = [done[i] for i in sorted(done)]
+    out["scheduler_prompt_passes"] = s.stats["prompt_passes"]
+    out["scheduler_decode_steps"] = s.stats["decode_steps"]
+    dec.close()
+    be.close()
+    return out
+
+
+def test_cpp_host_layer_matches_the_python_mirror_on_the_device():
+    r = subprocess.run([host_binary("host_gpu_test")], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout + r.stderr
+    cpp = json.loads(r.stdout)
+    assert cpp["gemm_device_bit_exact"] and cpp["scheduler_clean"] and cpp["bad_table_rejected"]
+    # a request that runs alone through the scheduler is generate of the same request
+    assert cpp["scheduler_alone"] == cpp["generate_same_request"]
+    assert cpp["scheduler"][4] == [41, 42, 43]                       # nothing to generate: the prompt is the answer
+    for row, n in zip(cpp["scheduler"], (12, 20, 16, 9, 3, 25, 30)):
+        assert len(row) == n and all(0 <= t < 1000 for t in row)
+    py = _python_side()
+    for key in ("generate_greedy", "generate_top_k", "generate_temperature", "scheduler", "scheduler_prompt_passes",
+                "scheduler_decode_steps"):
+        assert cpp[key] == py[key], key
