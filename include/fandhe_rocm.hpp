@@ -13,6 +13,8 @@
 //   SchedulerLimits, PageAllocator, BatchScheduler
 //                                  crates/autodiff/src/generate/scheduler.rs:75-127, 395-720;
 //                                  crates/autodiff/src/nn/paged_kv.rs:147-191 (allocation order)
+//   generate_speculative           crates/autodiff/src/generate/speculative.rs:334-531 (greedy form)
+//   BlockTable, PagedKvCache       crates/autodiff/src/nn/paged_kv.rs:147-363, paged_kv_device.rs:67-372
 //
 // Header only, C++17, no dependency besides the C header; every device call goes through the C ABI, so
 // nothing here computes on the host what the library computes on the device.
@@ -42,6 +44,11 @@ class BackendError : public std::runtime_error {
 };
 // AutodiffError::InvalidArgument: a request the host layer rejects before anything is queued.
 class InvalidArgument : public std::invalid_argument {
+  public:
+    using std::invalid_argument::invalid_argument;
+};
+// What the device path does not offer although the reference does.
+class Unsupported : public std::invalid_argument {
   public:
     using std::invalid_argument::invalid_argument;
 };
@@ -269,6 +276,104 @@ class RocmBackendOps {
     const Context &ctx_;
 };
 
+// ------------------------------------------------------------------------------------------- cache layer
+// BlockTable (crates/autodiff/src/nn/paged_kv.rs:147-363): page table with free-block bookkeeping; pure host
+// state.  Free blocks are the stack of returned ids (last in, first out), then the never-used ids ascending;
+// all rows have one length; every call either succeeds or leaves the table unchanged.
+class BlockTable {
+  public:
+    explicit BlockTable(uint64_t max_blocks, uint64_t block_size) : max_blocks_(max_blocks), block_size_(block_size) {
+        check(fa_block_table_create(&h_));
+    }
+    ~BlockTable() {
+        if (h_) fa_block_table_destroy(h_);
+    }
+    BlockTable(const BlockTable &o) : max_blocks_(o.max_blocks_), block_size_(o.block_size_) { check(fa_block_table_clone(o.h_, &h_)); }
+    BlockTable &operator=(const BlockTable &) = delete;
+    fa_block_table_state state() const {
+        fa_block_table_state st;
+        check(fa_block_table_state_get(h_, max_blocks_, &st));
+        return st;
+    }
+    uint64_t seq_len() const { return state().seq_len; }
+    uint64_t free_blocks() const { return state().free_blocks; }
+    std::optional<uint32_t> alloc() {
+        uint32_t id = 0;
+        int32_t got = 0;
+        check(fa_block_table_alloc(h_, max_blocks_, &id, &got));
+        return got ? std::optional<uint32_t>(id) : std::nullopt;
+    }
+    // slots of the b * l_new new tokens, rows first
+    std::vector<uint32_t> extend_for_append(uint64_t b, uint64_t l_new) {
+        std::vector<uint32_t> slots(b * l_new);
+        uint64_t n = 0;
+        check(fa_block_table_extend_for_append(h_, max_blocks_, block_size_, b, l_new, slots.data(), slots.size(), &n));
+        slots.resize(n);
+        return slots;
+    }
+    // [rows, max_blocks_per_seq], UINT32_MAX in unused entries
+    std::vector<uint32_t> flatten_tables(uint64_t max_blocks_per_seq) const {
+        std::vector<uint32_t> out(state().batch * max_blocks_per_seq);
+        uint64_t n = 0;
+        check(fa_block_table_flatten(h_, max_blocks_per_seq, out.data(), out.size(), &n));
+        out.resize(n);
+        return out;
+    }
+    void rewind_to(uint64_t new_len) { check(fa_block_table_rewind_to(h_, new_len, block_size_)); }
+    void reset() { check(fa_block_table_reset(h_)); }
+
+  private:
+    fa_block_table *h_ = nullptr;
+    uint64_t max_blocks_, block_size_;
+};
+
+// PagedKvCache (crates/autodiff/src/nn/paged_kv_device.rs:67-372): the one-layer device-resident cache.
+class PagedKvCache {
+  public:
+    PagedKvCache(const Context &ctx, uint64_t block_size, uint64_t max_blocks, uint64_t embed_dim, fa_dtype dtype = FA_F32)
+        : ctx_(ctx), embed_dim_(embed_dim), dtype_(dtype) {
+        check(fa_paged_cache_create(ctx.handle(), block_size, max_blocks, embed_dim, dtype, &h_));
+    }
+    ~PagedKvCache() {
+        if (h_) fa_paged_cache_destroy(ctx_.handle(), h_);
+    }
+    PagedKvCache(const PagedKvCache &) = delete;
+    PagedKvCache &operator=(const PagedKvCache &) = delete;
+    fa_block_table_state state(bool *poisoned = nullptr) const {
+        fa_block_table_state st;
+        int32_t p = 0;
+        check(fa_paged_cache_state_get(h_, &st, &p));
+        if (poisoned) *poisoned = p != 0;
+        return st;
+    }
+    uint64_t seq_len() const { return state().seq_len; }
+    uint64_t num_free_blocks() const { return state().free_blocks; }
+    bool is_poisoned() const {
+        bool p = false;
+        state(&p);
+        return p;
+    }
+    // k_new / v_new [b, l_new, embed_dim] of the pools' type
+    void append(const Buffer &k_new, const Buffer &v_new, uint64_t b, uint64_t l_new) {
+        check(fa_paged_cache_append(ctx_.handle(), h_, k_new.handle(), v_new.handle(), b, l_new));
+    }
+    // q / out [b, l_new, num_heads * head_dim]
+    Buffer attention(const Buffer &q, uint64_t b, uint64_t l_new, uint64_t num_heads, uint64_t num_kv_heads, float scale) const {
+        const uint64_t hkv = num_kv_heads ? num_kv_heads : num_heads;
+        Buffer out = Buffer::alloc_uninit(ctx_, dtype_, b * l_new * num_heads * (embed_dim_ / hkv));
+        check(fa_paged_cache_attention(ctx_.handle(), h_, q.handle(), b, l_new, num_heads, num_kv_heads, scale, out.handle()));
+        return out;
+    }
+    void rewind_to(uint64_t new_len) { check(fa_paged_cache_rewind_to(h_, new_len)); }
+    void clear() { check(fa_paged_cache_clear(h_)); }
+
+  private:
+    const Context &ctx_;
+    fa_paged_cache *h_ = nullptr;
+    uint64_t embed_dim_;
+    fa_dtype dtype_;
+};
+
 // ------------------------------------------------------------------------------------------------ decoder
 // The resident decoder: weights are borrowed (the caller keeps buffers and quantized weights alive).
 class Decoder {
@@ -475,6 +580,112 @@ std::vector<std::vector<int32_t>> generate(DecoderT &decoder, const std::vector<
             out[r].push_back(tok[r]);
         }
     }
+    return out;
+}
+
+// generate_speculative (crates/autodiff/src/generate/speculative.rs:334-531), greedy form, on two resident
+// decoders: per round the draft decodes k_eff = min(k, remaining - 1) tokens, the target consumes the pending
+// token and those drafts in one verification, the longest prefix of drafts that equals the target's own greedy
+// tokens is kept and the target's token at the first disagreement (or after the last draft) is appended.  Both
+// caches are then cut back to the accepted length: paged rows past a sequence's length are dead, so nothing is
+// replayed (the reference restores a snapshot and replays, kv_rewind.rs:157-215).  One sequence per call.  When
+// the pending token and the drafts fit the decoder's rows (k + 1 <= min(32, max_batch)) the verification is one
+// decode step whose rows are the k + 1 positions of the one sequence (the same block table in every row, lengths
+// ctx, ctx + 1, ...); longer look-aheads take the prompt-shape verification pass.
+struct SpeculativeOutput {
+    std::vector<int32_t> tokens;
+    uint64_t rounds = 0, accepted = 0;
+};
+template <typename DecoderT>
+SpeculativeOutput generate_speculative(DecoderT &target, DecoderT &draft, const std::vector<int32_t> &input_ids,
+                                       const GenerateConfig &config, uint64_t k) {
+    config.validate();
+    if (k < 1) throw InvalidArgument("generate_speculative: k must be at least 1");
+    if (input_ids.empty()) throw InvalidArgument("generate_speculative: the prompt is empty");
+    const uint64_t max_length = config.max_length, prompt_len = input_ids.size();
+    if (max_length < prompt_len) throw InvalidArgument("generate_speculative: max_length must be at least the prompt length");
+    detail::check_output_bytes(max_length);
+    if (config.strategy.kind != FA_SAMPLE_GREEDY)
+        throw Unsupported("generate_speculative: only the greedy form runs on the device (sampled acceptance needs both models' "
+                          "probabilities on the host)");
+    SpeculativeOutput out;
+    std::vector<int32_t> &row = out.tokens;
+    row = input_ids;
+    if (max_length == prompt_len) return out;
+    if (target.config().vocab != draft.config().vocab) throw InvalidArgument("generate_speculative: the models disagree on the vocabulary");
+    const bool by_step = k + 1 <= std::min<uint64_t>(32, target.config().max_batch);
+    std::vector<uint32_t> target_table;
+    for (DecoderT *dec : {&target, &draft}) {
+        const auto &cfg = dec->config();
+        const uint64_t pages = detail::pages_for(max_length + 1, cfg.block_size);   // the verification also writes the last draft
+        if (pages > cfg.max_blocks_per_seq || pages > cfg.num_blocks)
+            throw InvalidArgument("generate_speculative: the tokens do not fit the decoder's page pool");
+        std::vector<uint32_t> table(cfg.max_blocks_per_seq, UINT32_MAX);
+        for (uint64_t p = 0; p < pages; ++p) table[p] = (uint32_t)p;
+        dec->set_sequences(table, {0});
+        dec->set_sampling(FA_SAMPLE_GREEDY, 1.0f, 0, 0);
+        dec->prefill(input_ids, (uint32_t)prompt_len);
+        if (dec == &target) target_table = table;
+    }
+    row.push_back(target.tokens()[0]);
+    while (row.size() < max_length) {
+        const uint64_t cur = row.size();
+        const int32_t last = row.back();
+        const uint64_t remaining = max_length - cur;
+        if (remaining == 1) {
+            target.set_tokens({last});
+            target.step();
+            row.push_back(target.tokens()[0]);
+            break;
+        }
+        const uint64_t k_eff = std::min(k, remaining - 1);
+        std::vector<int32_t> drafts;
+        int32_t x = last;
+        for (uint64_t i = 0; i < k_eff; ++i) {                    // the draft's cache grows by last, d1 .. d_{k_eff - 1}
+            draft.set_tokens({x});
+            draft.step();
+            x = draft.tokens()[0];
+            drafts.push_back(x);
+        }
+        std::vector<int32_t> fed{last};
+        fed.insert(fed.end(), drafts.begin(), drafts.end());
+        std::vector<int32_t> picked;
+        if (by_step) {
+            const uint64_t n = k_eff + 1;
+            std::vector<uint32_t> tables, lens;
+            for (uint64_t r = 0; r < n; ++r) {
+                tables.insert(tables.end(), target_table.begin(), target_table.end());
+                lens.push_back((uint32_t)(cur - 1 + r));
+            }
+            target.set_sequences(tables, lens);
+            target.set_tokens(fed);
+            target.step();
+            picked = target.tokens();
+            for (int32_t t : picked)
+                if (t < 0) throw InvalidArgument("generate_speculative: logits hold non-finite values");
+        } else {
+            picked = target.verify(fed, (uint32_t)fed.size());
+        }
+        uint64_t n_acc = 0;
+        while (n_acc < k_eff && drafts[n_acc] == picked[n_acc]) ++n_acc;
+        row.insert(row.end(), drafts.begin(), drafts.begin() + n_acc);
+        row.push_back(picked[n_acc]);
+        out.rounds += 1;
+        out.accepted += n_acc;
+        if (row.size() >= max_length) break;
+        const uint32_t keep = (uint32_t)(cur + n_acc);            // tokens before the new pending one
+        if (by_step)
+            target.set_sequences(target_table, {keep});
+        else
+            target.rewind({keep});
+        if (n_acc == k_eff) {
+            draft.set_tokens({x});                                // the draft never consumed its own last token
+            draft.step();
+        } else {
+            draft.rewind({keep});
+        }
+    }
+    row.resize(std::min<uint64_t>(row.size(), max_length));
     return out;
 }
 

@@ -159,6 +159,37 @@ int main() {
         CHECK(throws_invalid([] { SchedulerLimits(1, 0, 1); }));
         CHECK(throws_invalid([] { SchedulerLimits(1, 1, 0); }));
     }
+    // ---- block table: slots follow the pages, rewinding returns pages, the last returned page is reused first
+    {
+        BlockTable bt(/*max_blocks=*/6, /*block_size=*/4);
+        const std::vector<uint32_t> slots = bt.extend_for_append(2, 5);
+        CHECK(slots.size() == 10 && std::set<uint32_t>(slots.begin(), slots.end()).size() == 10);
+        CHECK(bt.seq_len() == 5 && bt.state().used_blocks == 4 && bt.free_blocks() == 2);
+        const std::vector<uint32_t> tables = bt.flatten_tables(3);
+        CHECK(tables.size() == 6 && tables[2] == UINT32_MAX && tables[5] == UINT32_MAX);
+        for (uint32_t r = 0; r < 2; ++r)
+            for (uint32_t t = 0; t < 5; ++t) CHECK(slots[r * 5 + t] == tables[r * 3 + t / 4] * 4 + t % 4);
+        BlockTable saved(bt);                                    // a copy is a snapshot
+        bool refused = false;
+        try {
+            bt.extend_for_append(2, 8);                          // 13 positions need 4 pages a row, 8 > 6
+        } catch (const BackendError &) {
+            refused = true;
+        }
+        CHECK(refused && bt.seq_len() == 5 && bt.free_blocks() == 2);
+        bt.rewind_to(4);
+        CHECK(bt.seq_len() == 4 && bt.free_blocks() == 4);
+        const uint32_t dropped_last = tables[1 * 3 + 1];         // row 1 gave its second page back last
+        CHECK(bt.alloc().value() == dropped_last);
+        refused = false;
+        try {
+            bt.rewind_to(9);
+        } catch (const BackendError &) {
+            refused = true;
+        }
+        CHECK(refused);
+        CHECK(saved.seq_len() == 5 && saved.free_blocks() == 2);
+    }
     const ToyConfig tc{97, 4, 16, 40, 4};
     // ---- generate: rows of a batch share one generator and draw in row order
     {

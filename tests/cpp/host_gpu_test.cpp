@@ -45,17 +45,27 @@ int main() {
             qkeep.push_back(std::make_unique<QWeight>(QWeight::from_f32(ctx, BufferView{&w, 0}, k, n)));
             return *qkeep.back();
         };
-        Decoder dec(ctx, cfg);
+        struct LayerRefs {
+            const Buffer *an, *fn;
+            const QWeight *wqkv, *wo, *wgu, *wdown;
+        };
+        std::vector<LayerRefs> layers;
         for (uint32_t l = 0; l < cfg.n_layers; ++l) {
             const Buffer &an = filled(D, 1.0f, 0.1f), &fn = filled(D, 1.0f, 0.1f);
             const QWeight &wqkv = weight(D, EQ + 2 * EKV), &wo = weight(EQ, D), &wgu = weight(D, 2 * (uint64_t)cfg.d_ffn),
                           &wdown = weight(cfg.d_ffn, D);
-            dec.set_layer(l, an, fn, wqkv, wo, wgu, wdown);
+            layers.push_back({&an, &fn, &wqkv, &wo, &wgu, &wdown});
         }
-        {
-            const Buffer &embed = filled((uint64_t)cfg.vocab * D, 0.0f, 1.0f), &norm = filled(D, 1.0f, 0.1f);
-            dec.set_head(embed, norm, weight(D, cfg.vocab));
-        }
+        const Buffer &embed = filled((uint64_t)cfg.vocab * D, 0.0f, 1.0f), &final_norm = filled(D, 1.0f, 0.1f);
+        const QWeight &lm_head = weight(D, cfg.vocab);
+        auto wire = [&](Decoder &d) {                             // weights are borrowed: two decoders can share them
+            for (uint32_t l = 0; l < cfg.n_layers; ++l)
+                d.set_layer(l, *layers[l].an, *layers[l].fn, *layers[l].wqkv, *layers[l].wo, *layers[l].wgu, *layers[l].wdown);
+            d.set_head(embed, final_norm, lm_head);
+        };
+        Decoder dec(ctx, cfg), draft(ctx, cfg);
+        wire(dec);
+        wire(draft);
 
         std::printf("{\n");
         // f32 GEMM against the host loop of the reference (k ascending, one fused multiply-add per term)
@@ -113,6 +123,56 @@ int main() {
         }
         print_rows("scheduler_alone", alone);
         print_rows("generate_same_request", generate(dec, {requests[1].first}, requests[1].second));
+        // speculative decoding with a draft that is the target itself: every draft is accepted, in both verification forms
+        for (uint64_t k : {4, 9}) {
+            const SpeculativeOutput so = generate_speculative(dec, draft, prompts[0], GenerateConfig(24, SamplingStrategy::Greedy()), k);
+            std::printf("\"speculative_k%llu\": {\"tokens\": [", (unsigned long long)k);
+            for (size_t i = 0; i < so.tokens.size(); ++i) std::printf("%s%d", i ? ", " : "", so.tokens[i]);
+            std::printf("], \"rounds\": %llu, \"accepted\": %llu},\n", (unsigned long long)so.rounds, (unsigned long long)so.accepted);
+        }
+        print_rows("generate_greedy_24", generate(dec, {prompts[0]}, GenerateConfig(24, SamplingStrategy::Greedy())));
+        // the one-layer cache: two appends, then the last token of every row attends to its five positions
+        {
+            const uint64_t bs = 4, e = 8, heads = 2, dh = 4, b = 2;
+            PagedKvCache cache(ctx, bs, 8, e, FA_F32);
+            std::vector<float> k_all, v_all, q(b * e);
+            for (size_t i = 0; i < q.size(); ++i) q[i] = 0.25f * (float)((int)(i * 3 % 7) - 3);
+            auto chunk = [&](uint64_t l_new, uint64_t t0, std::vector<float> &all, float mul) {
+                std::vector<float> x(b * l_new * e);
+                for (uint64_t r = 0; r < b; ++r)
+                    for (uint64_t t = 0; t < l_new; ++t)
+                        for (uint64_t d = 0; d < e; ++d) x[(r * l_new + t) * e + d] = mul * (float)((int)((r * 31 + (t0 + t) * 7 + d * 3) % 11) - 5);
+                all.insert(all.end(), x.begin(), x.end());
+                return Buffer::upload(ctx, x);
+            };
+            std::vector<float> k1, v1, k2, v2;
+            cache.append(chunk(3, 0, k1, 0.125f), chunk(3, 0, v1, 0.5f), b, 3);
+            cache.append(chunk(2, 3, k2, 0.125f), chunk(2, 3, v2, 0.5f), b, 2);
+            auto at = [&](const std::vector<float> &c1, const std::vector<float> &c2, uint64_t r, uint64_t t, uint64_t d) {
+                return t < 3 ? c1[(r * 3 + t) * e + d] : c2[(r * 2 + (t - 3)) * e + d];
+            };
+            const std::vector<float> got = cache.attention(Buffer::upload(ctx, q), b, 1, heads, 0, 0.5f).download<float>();
+            double worst = 0.0;
+            for (uint64_t r = 0; r < b; ++r)
+                for (uint64_t h = 0; h < heads; ++h) {
+                    double sc[5], mx = -1e30, den = 0.0;
+                    for (uint64_t t = 0; t < 5; ++t) {
+                        double s = 0.0;
+                        for (uint64_t d = 0; d < dh; ++d) s += (double)q[r * e + h * dh + d] * at(k1, k2, r, t, h * dh + d);
+                        sc[t] = s * 0.5;
+                        mx = std::max(mx, sc[t]);
+                    }
+                    for (uint64_t t = 0; t < 5; ++t) den += (sc[t] = std::exp(sc[t] - mx));
+                    for (uint64_t d = 0; d < dh; ++d) {
+                        double o = 0.0;
+                        for (uint64_t t = 0; t < 5; ++t) o += sc[t] / den * at(v1, v2, r, t, h * dh + d);
+                        worst = std::max(worst, std::fabs(o - (double)got[r * e + h * dh + d]));
+                    }
+                }
+            cache.rewind_to(2);
+            const bool state_ok = cache.seq_len() == 2 && cache.num_free_blocks() == 8 - 2 && !cache.is_poisoned();
+            std::printf("\"paged_cache_max_abs_err\": %.3e, \"paged_cache_state_ok\": %s,\n", worst, state_ok ? "true" : "false");
+        }
         // error behaviour of the boundary reaches the caller as BackendError with the status of the call
         bool rejected = false;
         try {

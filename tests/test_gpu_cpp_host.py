@@ -35,14 +35,21 @@ def _python_side():
         keep.append(q)
         return q
 
-    dec = fa.Decoder(be, n_layers, d, heads, kv, f, vocab, max_blocks_per_seq=8, num_blocks=48, max_batch=8,
-                     rms_eps=1e-5, rope_theta=10000.0)
+    def decoder():
+        return fa.Decoder(be, n_layers, d, heads, kv, f, vocab, max_blocks_per_seq=8, num_blocks=48, max_batch=8,
+                          rms_eps=1e-5, rope_theta=10000.0)
+
+    dec, draft = decoder(), decoder()                       # weights are borrowed: the two share them
     eq, ekv = heads * dh, kv * dh
     for l in range(n_layers):
         an, fn = filled(d, 1.0, 0.1), filled(d, 1.0, 0.1)
-        dec.set_layer(l, an, fn, weight(d, eq + 2 * ekv), weight(eq, d), weight(d, 2 * f), weight(f, d))
+        ws = (weight(d, eq + 2 * ekv), weight(eq, d), weight(d, 2 * f), weight(f, d))
+        dec.set_layer(l, an, fn, *ws)
+        draft.set_layer(l, an, fn, *ws)
     embed, norm = filled(vocab * d, 0.0, 1.0), filled(d, 1.0, 0.1)
-    dec.set_head(embed, norm, weight(d, vocab))
+    head = weight(d, vocab)
+    dec.set_head(embed, norm, head)
+    draft.set_head(embed, norm, head)
 
     G, K, T = sch.SamplingStrategy.Greedy, sch.SamplingStrategy.TopK, sch.SamplingStrategy.Temperature
     out = {}
@@ -71,6 +78,10 @@ def _python_side():
     out["scheduler"] = [done[i] for i in sorted(done)]
     out["scheduler_prompt_passes"] = s.stats["prompt_passes"]
     out["scheduler_decode_steps"] = s.stats["decode_steps"]
+    for k in (4, 9):
+        toks, rounds, accepted = sch.generate_speculative(dec, draft, prompts[0], sch.GenerateConfig(24, G()), k)
+        out["speculative_k%d" % k] = {"tokens": toks.tolist(), "rounds": rounds, "accepted": accepted}
+    draft.close()
     dec.close()
     be.close()
     return out
@@ -86,7 +97,13 @@ def test_cpp_host_layer_matches_the_python_mirror_on_the_device():
     assert cpp["scheduler"][4] == [41, 42, 43]                       # nothing to generate: the prompt is the answer
     for row, n in zip(cpp["scheduler"], (12, 20, 16, 9, 3, 25, 30)):
         assert len(row) == n and all(0 <= t < 1000 for t in row)
+    # the draft is the target itself: all drafts are accepted and the tokens are plain greedy generation
+    for k in (4, 9):
+        sp = cpp["speculative_k%d" % k]
+        assert sp["tokens"] == cpp["generate_greedy_24"][0] and sp["accepted"] > 0 and sp["rounds"] < 24 - 5
+    # the one-layer cache against a double-precision host loop
+    assert cpp["paged_cache_max_abs_err"] < 1e-5 and cpp["paged_cache_state_ok"]
     py = _python_side()
     for key in ("generate_greedy", "generate_top_k", "generate_temperature", "scheduler", "scheduler_prompt_passes",
-                "scheduler_decode_steps"):
+                "scheduler_decode_steps", "speculative_k4", "speculative_k9"):
         assert cpp[key] == py[key], key
