@@ -5,7 +5,7 @@
 #include <map>
 #include <memory>
 
-#include "fandhe_rocm.hpp"
+#include "fandhe_safetensors.hpp"
 
 using namespace fandhe;
 
@@ -19,12 +19,33 @@ static void print_rows(const char *key, const std::vector<std::vector<int32_t>> 
     std::printf("]%s\n", last ? "" : ",");
 }
 
-int main() {
+// host_gpu_test <checkpoint> <n_layers> <n_heads> <n_kv_heads>: a resident decoder straight from a Llama-style
+// safetensors file, then greedy and top-k generation from two fixed prompts.
+static int from_checkpoint(int argc, char **argv) {
+    if (argc != 5) {
+        std::fprintf(stderr, "usage: host_gpu_test [checkpoint n_layers n_heads n_kv_heads]\n");
+        return 2;
+    }
+    Context ctx(0);
+    const std::vector<uint8_t> file = st::read_file(argv[1]);
+    st::LoadedDecoder m = st::load_decoder(ctx, file.data(), file.size(), (uint32_t)std::atoi(argv[2]), (uint32_t)std::atoi(argv[3]),
+                                           (uint32_t)std::atoi(argv[4]), /*max_blocks_per_seq=*/4, /*num_blocks=*/16, /*max_batch=*/4,
+                                           128, 16, 1e-5f, 10000.0);
+    const std::vector<std::vector<int32_t>> prompts{{3, 1, 4, 1, 5}, {2, 7, 1, 8, 2}};
+    std::printf("{\n");
+    print_rows("checkpoint_greedy", generate(*m.decoder, prompts, GenerateConfig(20, SamplingStrategy::Greedy())));
+    print_rows("checkpoint_top_k", generate(*m.decoder, {prompts[0]}, GenerateConfig(20, SamplingStrategy::TopK(8)).with_seed(21)), true);
+    std::printf("}\n");
+    return 0;
+}
+
+int main(int argc, char **argv) {
     try {
         if (Context::device_count() < 1) {
             std::fprintf(stderr, "host_gpu_test: no gfx950 device\n");
             return 2;
         }
+        if (argc > 1) return from_checkpoint(argc, argv);
         Context ctx(0);
         RocmBackendOps ops(ctx);
         fa_decoder_config cfg{};
