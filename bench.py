@@ -561,7 +561,7 @@ def main():
                     help="tuning: wavefronts per compute unit of the decode attention (0 = built-in)")
     ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
                     help="tuning: raw fa_set_tuning key/value pairs (experiments)")
-    ap.add_argument("--only", choices=("attention", "copy", "linears", "prefill", "mfma", "prompt"), default=None,
+    ap.add_argument("--only", choices=("attention", "copy", "linears", "prefill", "prefill-attention", "mfma", "prompt"), default=None,
                     help="profiling aid: run only the dominant kernel at the workload's shape, or a plain "
                          "copy kernel of known size (counter calibration), a few launches, no JSON line")
     a = ap.parse_args()
@@ -582,10 +582,11 @@ def main():
     ctxs = np.random.default_rng(0).integers(1024, 8193, size=batch).tolist()
     if a.only is not None:
         mid_ctx = [c + a.warmup + a.steps // 2 for c in ctxs]
-        if a.only == "prefill":
-            for r in bench_prefill(fa, be, 20):
-                log("%s m=%d k=%d n=%d: %.1f us, %.0f TOPS (%.1f %% of peak)" %
-                    (r["op"], r["m"], r["k"], r["n"], r["us"], r["tops"], 100 * r["frac"]))
+        if a.only in ("prefill", "prefill-attention"):
+            if a.only == "prefill":
+                for r in bench_prefill(fa, be, 20):
+                    log("%s m=%d k=%d n=%d: %.1f us, %.0f TOPS (%.1f %% of peak)" %
+                        (r["op"], r["m"], r["k"], r["n"], r["us"], r["tops"], 100 * r["frac"]))
             for r in bench_prefill_attention(fa, be):
                 log("prefill attention 4 x 2048 new tokens, 32/8 heads, %s kernel: %.2f ms, %.1f TFLOP/s" %
                     (r["kernel"], r["ms"], r["tflops"]))
