@@ -16,7 +16,7 @@ extern int g_skinny_ntw, g_skinny_waves, g_skinny_astat, g_gemm_small_tiles, g_g
 }
 int g_decode_waves = 0;
 int g_prefill_generic = 0;
-extern int g_decode_partials_only, g_prefill_block_form, g_prefill_block_waves;
+extern int g_decode_partials_only, g_prefill_block_form, g_prefill_block_waves, g_prefill_block_split;
 }  // namespace fa
 
 namespace {
@@ -83,6 +83,7 @@ fa_status fa_set_tuning(int32_t key, int32_t value) {
         case 9: k::g_gemm_split_fill = value; return FA_OK;
         case 10: fa::g_prefill_block_form = value; return FA_OK;
         case 11: fa::g_prefill_block_waves = value; return FA_OK;
+        case 12: fa::g_prefill_block_split = value; return FA_OK;
     }
     return fail(FA_ERR_INVALID_ARGUMENT, "fa_set_tuning: unknown key");
 }

@@ -741,6 +741,11 @@ struct FlashParams {
     int out_bf16;
     uint32_t num_blocks, e_kv, batch, num_heads, num_kv_heads, group, max_blocks_per_seq, l_new, tq, tiles;
     float scale;
+    // Split walk (few blocks against a long cache): gridDim.y blocks share a tile, block y walks the steps
+    // [y, y + 1) * ceil(steps / gridDim.y) and leaves its unnormalised sums, running maxima and denominators in
+    // part_o [tile block][y][column][128] / part_ml [tile block][y][2][columns]; flash_split_merge_kernel adds them.
+    uint32_t nsplit;
+    float *part_o, *part_ml;
 };
 constexpr int kFlashNQ = 2, kFlashKeys = 32;
 
@@ -766,8 +771,12 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
     const uint32_t t_end = t0 + p.tq < p.l_new ? t0 + p.tq : p.l_new;
     uint32_t kmax = violation ? 0 : base + t_end;              // positions the last token of the tile sees
     if (kmax > ctx) kmax = ctx;
-    const uint32_t npages = (kmax + kPage - 1) / kPage, n_it = (kmax + kFlashKeys - 1) / kFlashKeys;
+    const uint32_t npages = (kmax + kPage - 1) / kPage, n_all = (kmax + kFlashKeys - 1) / kFlashKeys;
     const uint32_t *tab = p.tables + (uint64_t)b * p.max_blocks_per_seq;
+    // this block's share of the walk: steps [it_lo, n_it)
+    const uint32_t per_split = (n_all + p.nsplit - 1) / p.nsplit;
+    const uint32_t it_lo = p.nsplit > 1 ? (blockIdx.y * per_split < n_all ? blockIdx.y * per_split : n_all) : 0;
+    const uint32_t n_it = p.nsplit > 1 ? (it_lo + per_split < n_all ? it_lo + per_split : n_all) : n_all;
 
     // first page of the walk whose id is outside the pool: columns that would read it give NaN
     if (tid == 0) s_bad = 0xffffffffu;
@@ -834,19 +843,19 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
         k_a[ps] = v_a[ps] = k_b[ps] = v_b[ps] = v4u{0, 0, 0, 0};
         id_c[ps] = 0;
     }
-    if (n_it > 0) {
+    if (n_it > it_lo) {
 #pragma unroll
         for (int ps = 0; ps < kPasses; ++ps) {
-            const uint32_t id0 = load_id(0, ps), id1 = load_id(1, ps), id2 = load_id(2, ps);
-            id_c[ps] = load_id(3, ps);
-            const uint64_t off0 = row_off(0, ps, id0), off1 = row_off(1, ps, id1), off2 = row_off(2, ps, id2);
+            const uint32_t id0 = load_id(it_lo, ps), id1 = load_id(it_lo + 1, ps), id2 = load_id(it_lo + 2, ps);
+            id_c[ps] = load_id(it_lo + 3, ps);
+            const uint64_t off0 = row_off(it_lo, ps, id0), off1 = row_off(it_lo + 1, ps, id1), off2 = row_off(it_lo + 2, ps, id2);
             v4u k0 = *(const v4u *)(p.k_pool + off0), v0 = *(const v4u *)(p.v_pool + off0);
             k_a[ps] = *(const v4u *)(p.k_pool + off1);
             v_a[ps] = *(const v4u *)(p.v_pool + off1);
             k_b[ps] = *(const v4u *)(p.k_pool + off2);
             v_b[ps] = *(const v4u *)(p.v_pool + off2);
             const uint32_t row = ps * kRows + r_st;
-            if (row >= ctx) v0 = v4u{0, 0, 0, 0};               // the pool may hold anything past the sequence end
+            if (it_lo * kFlashKeys + row >= ctx) v0 = v4u{0, 0, 0, 0};   // the pool may hold anything past the sequence end
             *(v4u *)(&k_s[0][row * kVPitch + 8 * c16]) = k0;
             *(v4u *)(&v_s[0][row * kVPitch + 8 * c16]) = v0;
         }
@@ -864,8 +873,8 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
     }
     constexpr float kLog2e = 1.4426950408889634f;
 
-    for (uint32_t it = 0; it < n_it; ++it) {
-        const int st = it & 1;
+    for (uint32_t it = it_lo; it < n_it; ++it) {
+        const int st = (it - it_lo) & 1;
         // requests of this step: the rows of step it + 3 (their page id was requested one step ago) and the
         // page id of step it + 4
         v4u k_n[kPasses], v_n[kPasses];
@@ -1010,6 +1019,22 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
         l += __shfl_xor(l, 32, 64);
         if (!valid[qi]) continue;
         const bool nan_out = violation || lim[qi] > first_bad_tok;
+        if (p.nsplit > 1) {
+            const uint32_t cols = NW * kFlashNQ * 16, col = (uint32_t)wave * (kFlashNQ * 16) + qi * 16 + c;
+            const uint64_t slot = (uint64_t)blockIdx.x * p.nsplit + blockIdx.y;
+            float *po = p.part_o + (slot * cols + col) * kDh + 8 * g;
+#pragma unroll
+            for (int bp = 0; bp < 4; ++bp) {
+                *(v4f *)(po + 32 * bp) = v4f{o[qi][2 * bp][0], o[qi][2 * bp + 1][0], o[qi][2 * bp][1], o[qi][2 * bp + 1][1]};
+                *(v4f *)(po + 32 * bp + 4) = v4f{o[qi][2 * bp][2], o[qi][2 * bp + 1][2], o[qi][2 * bp][3], o[qi][2 * bp + 1][3]};
+            }
+            if (g == 0) {
+                const float nanv = __uint_as_float(0x7fc00000u);
+                p.part_ml[slot * (2 * cols) + col] = nan_out ? nanv : m_run[qi];
+                p.part_ml[slot * (2 * cols) + cols + col] = nan_out ? nanv : l;
+            }
+            continue;
+        }
 #pragma unroll
         for (int bp = 0; bp < 4; ++bp) {
             float r8[8];
@@ -1032,6 +1057,56 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
             }
         }
     }
+}
+
+// Adds the shares of a split walk: one block per (tile block, eight columns), thread (column, dim).  The shares
+// of a column are read eight at a time, all loads of a batch before the first use (a chain of L2 round trips
+// otherwise); slots past the last share repeat it with weight zero.
+template <int NW>
+__global__ void __launch_bounds__(1024) flash_split_merge_kernel(FlashParams p) {
+    constexpr uint32_t kCols = NW * kFlashNQ * 16;
+    const uint32_t per_tile = p.batch * p.num_kv_heads;
+    const uint32_t tile = p.tiles - 1 - blockIdx.x / per_tile;
+    const uint32_t b = (blockIdx.x % per_tile) / p.num_kv_heads, kvh = blockIdx.x % p.num_kv_heads;
+    const uint32_t d = threadIdx.x % 128, col = blockIdx.y * 8 + threadIdx.x / 128;
+    const uint32_t t = tile * p.tq + col / p.group;
+    if (col >= p.tq * p.group || t >= p.l_new) return;
+    const float *ml = p.part_ml + (uint64_t)blockIdx.x * p.nsplit * (2 * kCols) + col;
+    const float *po = p.part_o + ((uint64_t)blockIdx.x * p.nsplit * kCols + col) * kDh + d;
+    const uint32_t last = p.nsplit - 1;
+    float mx = -INFINITY;
+    for (uint32_t z0 = 0; z0 < p.nsplit; z0 += 8) {
+        float m[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) m[u] = ml[(uint64_t)(z0 + u < p.nsplit ? z0 + u : last) * (2 * kCols)];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) mx = (m[u] != m[u] || mx != mx) ? __uint_as_float(0x7fc00000u) : fmaxf(mx, m[u]);   // NaN marks a violation
+    }
+    const float m_use = mx == -INFINITY ? 0.0f : mx;
+    float acc = 0.0f, den = 0.0f;
+    for (uint32_t z0 = 0; z0 < p.nsplit; z0 += 8) {
+        float m[8], l[8], o[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const uint64_t z = z0 + u < p.nsplit ? z0 + u : last;
+            m[u] = ml[z * (2 * kCols)];
+            l[u] = ml[z * (2 * kCols) + kCols];
+            o[u] = po[z * kCols * kDh];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const float w = z0 + u < p.nsplit ? expf(m[u] - m_use) : 0.0f;           // a share that saw nothing: exp(-inf) = 0
+            den = __builtin_fmaf(w, l[u], den);
+            acc = __builtin_fmaf(w, o[u], acc);
+        }
+    }
+    float res = den > 0.0f ? __fdiv_rn(acc, den) : 0.0f;
+    if (mx != mx) res = mx;
+    const uint64_t oi = (((uint64_t)b * p.l_new + t) * p.num_heads + (uint64_t)kvh * p.group + col % p.group) * kDh + d;
+    if (p.out_bf16)
+        ((uint16_t *)p.out)[oi] = f32_to_bf16(res);
+    else
+        ((float *)p.out)[oi] = res;
 }
 
 inline int group_pad(uint32_t group) {
@@ -1077,6 +1152,7 @@ void paged_attention_generic(const void *q, const void *k_pool, const void *v_po
 int g_decode_partials_only = 0;   // profiling: launch only the streaming kernel (the output is not written)
 int g_prefill_block_form = 0;     // 0: by shape, 1: never, 2: whenever the group size allows
 int g_prefill_block_waves = 0;    // wavefronts per block of the block form: 4 or 8, anything else by shape
+int g_prefill_block_split = 0;    // upper bound of the blocks that share one tile's walk (0: by shape)
 namespace k {
 
 static uint32_t compute_units() {
@@ -1175,10 +1251,16 @@ static uint32_t prefill_seqs_per_row(const PagedShape &ps) {           // virtua
     return all < cap ? all : cap;
 }
 
+// shares of a split walk that one launch may leave in the workspace (four-wavefront blocks, 128 columns each)
+static uint64_t flash_split_slots() { return 2ull * compute_units(); }
+constexpr uint64_t kFlashSplitCols = 4 * kFlashNQ * 16;
+
 uint64_t paged_prefill_workspace_bytes(const PagedShape &ps, uint32_t waves_per_cu) {
     uint64_t items = ((uint64_t)stream_ranges(ps, waves_per_cu) + (uint64_t)ps.batch * prefill_seqs_per_row(ps)) *
                      ps.num_kv_heads * prefill_tt(ps);
-    return items * (16 * kDh + 2 * 16) * sizeof(float);
+    const uint64_t streamed = items * (16 * kDh + 2 * 16) * sizeof(float);
+    const uint64_t split = flash_split_slots() * kFlashSplitCols * (kDh + 2) * sizeof(float);
+    return streamed > split ? streamed : split;
 }
 
 // Which prefill form a shape takes.  The block form walks the cache once per tile of new tokens, so its time
@@ -1189,10 +1271,11 @@ uint64_t paged_prefill_workspace_bytes(const PagedShape &ps, uint32_t waves_per_
 struct BlockFormPlan {
     bool use;
     int waves;
+    uint32_t nsplit;                    // blocks sharing a tile's walk (1: none)
 };
 static BlockFormPlan plan_block_form(const PagedShape &ps) {
     const uint32_t group = ps.num_heads / ps.num_kv_heads;
-    if (group == 0 || group > 16 || g_prefill_block_form == 1) return {false, 0};
+    if (group == 0 || group > 16 || g_prefill_block_form == 1) return {false, 0, 1};
     const uint32_t cus = compute_units();
     const uint32_t bound = ps.max_blocks_per_seq * kPage;
     uint32_t ctx = ps.ctx_hint != 0 && ps.ctx_hint < bound ? ps.ctx_hint : bound;
@@ -1205,17 +1288,28 @@ static BlockFormPlan plan_block_form(const PagedShape &ps) {
         const uint32_t tq8 = 256 / group;
         waves = rows * ((ps.l_new + tq8 - 1) / tq8) >= 2ull * cus && ps.l_new >= 1024 ? 8 : 4;
     }
-    if (g_prefill_block_form == 2) return {true, waves};
     const uint32_t tq = (uint32_t)waves * kFlashNQ * 16 / group, tiles = (ps.l_new + tq - 1) / tq;
     const double steps_longest = (cached + l_new) / kFlashKeys;
-    const double steps_all = (double)(rows * tiles) * (cached + (tiles > 1 ? 0.5 * l_new : l_new)) / kFlashKeys;
+    // few blocks against a long walk over what was cached before (the walks of all tiles are then about equally
+    // long): several blocks share a tile's walk (at least eight steps each, at most as many shares as the
+    // workspace holds) and a merge pass adds them
+    uint32_t nsplit = 1;
+    const uint64_t blocks = rows * tiles;
+    if (waves == 4 && blocks < cus && cached >= 2.0 * l_new) {
+        uint64_t want = flash_split_slots() / blocks, by_steps = (uint64_t)(steps_longest / 8.0);
+        if (g_prefill_block_split > 0) want = (uint64_t)g_prefill_block_split < want ? (uint64_t)g_prefill_block_split : want;
+        nsplit = (uint32_t)(want < by_steps ? want : by_steps);
+        if (nsplit < 1) nsplit = 1;
+    }
+    if (g_prefill_block_form == 2) return {true, waves, nsplit};
+    const double steps_all = (double)blocks * (cached + (tiles > 1 ? 0.5 * l_new : l_new)) / kFlashKeys;
     const double per_cu = waves == 8 ? 2.05 : 1.05;                       // us per step at two wavefronts per SIMD
-    const double a = steps_longest * 1.4, b = steps_all / cus * per_cu;
+    const double a = steps_longest / nsplit * 1.4 + (nsplit > 1 ? 9.0 : 0.0), b = steps_all / cus * per_cu;
     const double t_block = (a > b ? a : b) + 8.0;
     const uint32_t tpt = 16 / group, tpv = ps.l_new > tpt ? 2 * tpt : tpt;
     const double bytes = (double)rows * ((ps.l_new + tpv - 1) / tpv) * (cached + 0.5 * l_new) * (2.0 * kDh * 2);
     const double t_stream = 35.0 + bytes / 4.9e6 + 0.035 * l_new * ps.batch;
-    return {t_block <= t_stream, waves};
+    return {t_block <= t_stream, waves, nsplit};
 }
 
 void paged_attention_prefill_bf16(const uint16_t *q, const uint16_t *k_pool, const uint16_t *v_pool,
@@ -1244,10 +1338,16 @@ void paged_attention_prefill_bf16(const uint16_t *q, const uint16_t *k_pool, con
         fp.tiles = (ps.l_new + fp.tq - 1) / fp.tq;
         fp.scale = ps.scale;
         const uint64_t blocks = (uint64_t)ps.batch * ps.num_kv_heads * fp.tiles;
-        if (plan.waves == 8)
+        fp.nsplit = plan.nsplit;
+        fp.part_o = (float *)workspace;
+        fp.part_ml = fp.part_o + blocks * fp.nsplit * kFlashSplitCols * kDh;
+        if (plan.waves == 8) {
             prefill_flash_kernel<8><<<(unsigned)blocks, 512, 0, s>>>(fp);
-        else
-            prefill_flash_kernel<4><<<(unsigned)blocks, 256, 0, s>>>(fp);
+        } else {
+            prefill_flash_kernel<4><<<dim3((unsigned)blocks, fp.nsplit), 256, 0, s>>>(fp);
+            if (fp.nsplit > 1)
+                flash_split_merge_kernel<4><<<dim3((unsigned)blocks, (unsigned)((fp.tq * fp.group + 7) / 8)), 1024, 0, s>>>(fp);
+        }
         return;
     }
     StreamParams sp;

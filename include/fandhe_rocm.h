@@ -517,7 +517,9 @@ fa_status fa_decoder_read_seq_lens(fa_context *ctx, fa_decoder *dec, uint32_t *s
  *        for (default 2);
  * key 10: form of the attention with more than one new token per row: 1 always the
  *        streamed form, 2 always the block form, 0 by shape;
- * key 11: wavefronts per block of that block form (4 or 8; 0 by shape). */
+ * key 11: wavefronts per block of that block form (4 or 8; 0 by shape);
+ * key 12: upper bound of the blocks that share the cache walk of one tile of new tokens
+ *        in the block form (1: never split; 0 by shape). */
 fa_status fa_set_tuning(int32_t key, int32_t value);
 /* A pair of HIP events recorded on the context's stream (the stream the
  * kernels run on); used by the benchmark to time launches. */

@@ -283,18 +283,26 @@ def test_bf16_prefill_on_the_streaming_kernel_against_the_oracle(heads, kv_heads
     # the block form (one block per tile of 256 / group new tokens walks the cache once), forced for every
     # group size it supports whatever the shape heuristics would choose
     fa.check(fa.capi.lib.fa_set_tuning(10, 2))
-    for block_waves in (8, 4):        # tiles of 256 / group and of 128 / group new tokens
+    # tiles of 256 / group and of 128 / group new tokens; the smaller blocks also with the cache walk of a tile
+    # shared by several blocks (as many as the shape allows, or two) and a merge pass
+    for block_waves, split in ((8, 1), (4, 1), (4, 0), (4, 2)):
         fa.check(fa.capi.lib.fa_set_tuning(11, block_waves))
+        fa.check(fa.capi.lib.fa_set_tuning(12, split))
         blk = be.download_owned(be.paged_attention_forward(dq, dk, dv, tables, seq_lens, args, out_dtype=fa.capi.F32))
-        assert_parity("PAGED_PREFILL_PARITY", f"H{heads}/{kv_heads}:L{l_new}:block form, {block_waves} wavefronts", blk, want)
+        assert_parity("PAGED_PREFILL_PARITY", f"H{heads}/{kv_heads}:L{l_new}:block form, {block_waves} wavefronts, split {split}", blk, want)
         blk_bf = be.download_owned(be.paged_attention_forward(dq, dk, dv, tables, seq_lens, args))
         assert_bf16_rounding_of("paged prefill bf16, block form", blk_bf, blk)
-        blk_dev = be.download_owned(be.paged_attention_forward_device(dq, dk, dv, be.upload(tables), be.upload(seq_lens), args))
-        assert np.array_equal(blk_dev, blk_bf)
+        blk_dev = be.download_owned(be.paged_attention_forward_device(dq, dk, dv, be.upload(tables), be.upload(seq_lens), args,
+                                                                     out_dtype=fa.capi.F32))
+        if split == 1:                # one block a tile: the same launch with host or device tables
+            assert np.array_equal(blk_dev, blk)
+        else:                         # the share count follows the longest row the host knows of
+            assert_parity("PAGED_PREFILL_PARITY", f"H{heads}/{kv_heads}:L{l_new}:device tables, split {split}", blk_dev, want)
         for h in range(heads):
             gq = h // (heads // kv_heads)
             assert np.array_equal(blk_bf[0, 0, h * 128:(h + 1) * 128], vp[tables[0, 0], 0, gq * 128:(gq + 1) * 128])
     fa.check(fa.capi.lib.fa_set_tuning(11, 0))
+    fa.check(fa.capi.lib.fa_set_tuning(12, 0))
     # whatever the shape selects by itself (host tables: the longest row is known; device tables: the table width)
     fa.check(fa.capi.lib.fa_set_tuning(10, 0))
     auto = be.download_owned(be.paged_attention_forward(dq, dk, dv, tables, seq_lens, args, out_dtype=fa.capi.F32))
@@ -426,8 +434,9 @@ def test_block_form_prefill_flags_violations_per_column():
     bad_l[2] = l_new - 1                            # row 2: fewer positions than new tokens
     fa.check(fa.capi.lib.fa_set_tuning(10, 2))
     try:
-        for block_waves in (4, 8):
+        for block_waves, split in ((4, 1), (4, 0), (8, 1)):
             fa.check(fa.capi.lib.fa_set_tuning(11, block_waves))
+            fa.check(fa.capi.lib.fa_set_tuning(12, split))
             got = be.download_owned(be.paged_attention_forward_device(
                 be.upload(q), be.upload(kp), be.upload(vp), be.upload(bad_t), be.upload(bad_l), args, out_dtype=fa.capi.F32))
             assert_parity("PAGED_PREFILL_PARITY", "row 0 beside violations", got[0:1], want[0:1])
@@ -437,6 +446,7 @@ def test_block_form_prefill_flags_violations_per_column():
     finally:
         fa.check(fa.capi.lib.fa_set_tuning(10, 0))
         fa.check(fa.capi.lib.fa_set_tuning(11, 0))
+        fa.check(fa.capi.lib.fa_set_tuning(12, 0))
 
 
 def test_bf16_prefill_properties_at_prompt_size():
@@ -507,3 +517,48 @@ def test_bf16_prefill_properties_at_prompt_size():
     finally:
         fa.check(lib.fa_set_tuning(10, 0))
         fa.check(lib.fa_set_tuning(11, 0))
+
+
+def test_bf16_prefill_few_new_tokens_over_a_long_cache_share_the_walk():
+    """64 new tokens per row over some thousand cached positions (a conversation that continues): few tiles, long
+    walks.  The block form with shared walks, the block form without and the streamed form agree with each other
+    and with one-token decode calls; the shape's own choice is one of them."""
+    fa = _fa()
+    be = ops()
+    rng = o.Rng(9)
+    batch, heads, kv_heads, l_new, num_blocks = 2, 32, 8, 64, 600
+    lens = [4096 + 64, 1500 + 64]
+    tables, seq_lens, max_blocks, e_kv, e_q = _decode_case(rng, batch, heads, kv_heads, lens, num_blocks)
+    kp = o.to_bf16(rng.randn((num_blocks, 16, e_kv)))
+    vp = o.to_bf16(rng.randn((num_blocks, 16, e_kv)))
+    q = o.to_bf16(rng.randn((batch, l_new, e_q)))
+    layout = fa.PagedKvLayout.new(num_blocks, 16, e_kv)
+    args = fa.PagedAttentionArgs(layout, batch, l_new, heads, max_blocks, fa.default_scale(128), kv_heads)
+    args1 = fa.PagedAttentionArgs(layout, batch, 1, heads, max_blocks, fa.default_scale(128), kv_heads)
+    dq, dk, dv = be.upload(q), be.upload(kp), be.upload(vp)
+    lib = fa.capi.lib
+    outs = {}
+    try:
+        for name, form, split in (("shared walks", 2, 0), ("two shares", 2, 2), ("one block a tile", 2, 1), ("streamed", 1, 0), ("by shape", 0, 0)):
+            fa.check(lib.fa_set_tuning(10, form))
+            fa.check(lib.fa_set_tuning(12, split))
+            outs[name] = be.download_owned(be.paged_attention_forward(dq, dk, dv, tables, seq_lens, args, out_dtype=fa.capi.F32))
+            assert np.all(np.isfinite(outs[name])), name
+    finally:
+        fa.check(lib.fa_set_tuning(10, 0))
+        fa.check(lib.fa_set_tuning(12, 0))
+    for name in ("shared walks", "two shares", "one block a tile", "by shape"):
+        assert_parity("PREFILL_FORMS", f"{name} vs streamed", outs[name], outs["streamed"])
+    for t in (0, 31, 32, 63):
+        lens_t = (seq_lens - l_new + t + 1).astype(np.uint32)
+        dec = be.download_owned(be.paged_attention_forward(be.upload(np.ascontiguousarray(q[:, t:t + 1, :])), dk, dv,
+                                                           tables, lens_t, args1, out_dtype=fa.capi.F32))
+        assert_parity("PREFILL_VS_DECODE", f"shared walks:t{t}", outs["shared walks"][:, t:t + 1, :], dec)
+    # the oracle on the shorter row
+    oargs = o.paged_args(num_blocks, 16, e_kv, 1, l_new, heads, max_blocks, args.scale, kv_heads)
+    o.set_threads(8)
+    rc, want = o.paged_attention_bf16(np.ascontiguousarray(q[1:2]), kp, vp, np.ascontiguousarray(tables[1:2]),
+                                      np.ascontiguousarray(seq_lens[1:2]), oargs)
+    o.set_threads(1)
+    assert rc == 0
+    assert_parity("PAGED_PREFILL_PARITY", "row 1, shared walks", outs["shared walks"][1:2], want)
