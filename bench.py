@@ -357,15 +357,17 @@ def bench_prompt_prefill(fa, be, dec, cfg, tables, batch=4, l_new=2048, reps=2):
     return dict(batch=batch, l_new=l_new, ms=ms, tokens_per_s=batch * l_new / (ms * 1e-3))
 
 
-def bench_short_prompts(fa, be, dec, cfg, tables, lengths=(64, 300, 1024), reps=3):
-    """One request's prompt pass (batch 1) on the resident model: what a scheduler runs when a request joins."""
+def bench_short_prompts(fa, be, dec, cfg, tables, lengths=(64, 300, 1024, (64, 4096)), reps=3):
+    """One request's prompt pass (batch 1) on the resident model: what a scheduler runs when a request joins
+    (an empty cache) or a conversation continues (new tokens after cached positions)."""
     lib = fa.capi.lib
     row = int(np.argmax((tables != 0xFFFFFFFF).sum(axis=1)))           # the row with the most pages
     tb = np.ascontiguousarray(tables[row:row + 1])
-    lens = np.zeros(1, dtype=np.uint32)
     out = []
-    for l_new in lengths:
-        assert (l_new + 1 + cfg["block_size"] - 1) // cfg["block_size"] <= int((tb != 0xFFFFFFFF).sum())
+    for item in lengths:                                               # l_new, or (l_new, positions cached before)
+        l_new, cached = item if isinstance(item, tuple) else (item, 0)
+        lens = np.full(1, cached, dtype=np.uint32)                     # the synthetic pools already hold K / V there
+        assert (cached + l_new + 1 + cfg["block_size"] - 1) // cfg["block_size"] <= int((tb != 0xFFFFFFFF).sum())
         prompt = np.random.default_rng(l_new).integers(0, cfg["vocab"], size=(1, l_new)).astype(np.int32)
         best = None
         for _ in range(reps + 1):
@@ -376,7 +378,7 @@ def bench_short_prompts(fa, be, dec, cfg, tables, lengths=(64, 300, 1024), reps=
             fa.check(lib.fa_decoder_prefill(be._ctx, dec, prompt.ctypes.data_as(fa.capi.i32p), l_new))
             ms = t.stop_ms()
             best = ms if best is None else min(best, ms)
-        out.append(dict(l_new=l_new, ms=best, tokens_per_s=l_new / (best * 1e-3)))
+        out.append(dict(l_new=l_new, cached=cached, ms=best, tokens_per_s=l_new / (best * 1e-3)))
     return out
 
 
@@ -595,8 +597,8 @@ def main():
         if a.only == "prompt":
             dec, keep, tables, _, _ = build_decoder(fa, be, cfg, batch, ctxs, 4)
             for r in bench_short_prompts(fa, be, dec, cfg, tables):
-                log("one prompt of %d tokens through %d layers: %.2f ms, %.0f tokens/s" %
-                    (r["l_new"], cfg["n_layers"], r["ms"], r["tokens_per_s"]))
+                log("one prompt of %d tokens%s through %d layers: %.2f ms, %.0f tokens/s" %
+                    (r["l_new"], " after %d cached" % r["cached"] if r["cached"] else "", cfg["n_layers"], r["ms"], r["tokens_per_s"]))
             lib.fa_decoder_destroy(be._ctx, dec)
             be.close()
             return
@@ -661,7 +663,8 @@ def main():
     batching = short = single = None
     if not a.no_extras and not a.no_serving:
         short = bench_short_prompts(fa, be, dec, cfg, tables)
-        log("one prompt, batch 1: " + ", ".join("%d tokens %.2f ms" % (r["l_new"], r["ms"]) for r in short))
+        log("one prompt, batch 1: " + ", ".join("%d tokens%s %.2f ms" % (r["l_new"], " after %d cached" % r["cached"] if r["cached"] else "", r["ms"])
+                                                for r in short))
         single = bench_single_stream(fa, be, dec, cfg, tables)
         log("one sequence decoding alone: %.3f ms per token (%.0f tokens/s, weights streamed at %.0f GB/s); "
             "verifying 5 positions in one step: %.3f ms" %
