@@ -562,3 +562,36 @@ def test_bf16_prefill_few_new_tokens_over_a_long_cache_share_the_walk():
     o.set_threads(1)
     assert rc == 0
     assert_parity("PAGED_PREFILL_PARITY", "row 1, shared walks", outs["shared walks"][1:2], want)
+
+
+def test_shared_walks_flag_violations_per_column():
+    """Device tables, 64 new tokens over a long cache, the walk of each tile shared by several blocks: a page id
+    outside the pool gives NaN in exactly the columns whose causal range reaches that page, through the merge."""
+    fa = _fa()
+    be = ops()
+    rng = o.Rng(10)
+    batch, heads, kv_heads, l_new, num_blocks = 2, 8, 2, 64, 400
+    lens = [4096 + 64, 1500 + 64]
+    tables, seq_lens, max_blocks, e_kv, e_q = _decode_case(rng, batch, heads, kv_heads, lens, num_blocks)
+    kp = o.to_bf16(rng.randn((num_blocks, 16, e_kv)))
+    vp = o.to_bf16(rng.randn((num_blocks, 16, e_kv)))
+    q = o.to_bf16(rng.randn((batch, l_new, e_q)))
+    layout = fa.PagedKvLayout.new(num_blocks, 16, e_kv)
+    args = fa.PagedAttentionArgs(layout, batch, l_new, heads, max_blocks, fa.default_scale(128), kv_heads)
+    dq, dk, dv = be.upload(q), be.upload(kp), be.upload(vp)
+    bad = tables.copy()
+    bad[0, 259] = num_blocks + 1                    # row 0: its last page, positions 4144 .. 4159
+    bad[1, 10] = 0xFFFFFFF0                         # row 1: a page every new token sees
+    lib = fa.capi.lib
+    fa.check(lib.fa_set_tuning(10, 2))
+    try:
+        good = be.download_owned(be.paged_attention_forward_device(dq, dk, dv, be.upload(tables), be.upload(seq_lens), args,
+                                                                   out_dtype=fa.capi.F32))
+        got = be.download_owned(be.paged_attention_forward_device(dq, dk, dv, be.upload(bad), be.upload(seq_lens), args,
+                                                                  out_dtype=fa.capi.F32))
+    finally:
+        fa.check(lib.fa_set_tuning(10, 0))
+    assert np.all(np.isfinite(good))
+    # row 0: 4096 positions were cached, token t sees positions < 4097 + t: tokens 0 .. 47 stay below position 4144
+    assert np.array_equal(got[0, :48], good[0, :48]) and np.all(np.isnan(got[0, 48:]))
+    assert np.all(np.isnan(got[1]))
