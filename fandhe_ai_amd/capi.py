@@ -1,4 +1,5 @@
-"""ctypes declarations of the C ABI in include/fandhe_rocm.h.
+"""ctypes declarations of the C ABI in include/fandhe_rocm.h and of the
+measurement / test aids in include/fandhe_rocm_bench.h.
 
 Loads ``fandhe_ai_amd/lib/libfandhe_rocm.so`` (built by ``make -C
 fandhe_ai_amd/csrc`` / ``__graft_entry__.build()``).  There is no fallback: if
@@ -67,6 +68,11 @@ class RowSampling(C.Structure):
     """fa_row_sampling: one request's strategy and generator state."""
     _fields_ = [("rng_state", C.c_uint64), ("temperature", C.c_float), ("top_k", C.c_uint32),
                 ("strategy", C.c_int32), ("reserved", C.c_uint32)]
+
+
+class GemmPlan(C.Structure):
+    """fa_gemm_plan: the kernel a prefill-shape GEMM is launched with."""
+    _fields_ = [("big_ntb", C.c_int32), ("waves", C.c_int32), ("splits", C.c_uint32)]
 
 
 class DecoderConfig(C.Structure):
@@ -186,6 +192,8 @@ SIGNATURES = {
     "fa_timer_stop": (C.c_int32, [ctx_p, C.c_void_p]),
     "fa_timer_elapsed_ms": (C.c_int32, [ctx_p, C.c_void_p, f32p]),
     "fa_timer_destroy": (C.c_int32, [ctx_p, C.c_void_p]),
+    "fa_gemm_plan_query": (C.c_int32, [ctx_p, u64, qw_p, C.POINTER(GemmPlan)]),
+    "fa_graph_owned_blocks": (C.c_int32, [C.c_void_p, C.POINTER(C.c_void_p), u64, C.POINTER(u64)]),
 }
 
 for _name, (_res, _args) in SIGNATURES.items():

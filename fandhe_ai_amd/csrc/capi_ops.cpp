@@ -44,7 +44,9 @@ fa_status check_qw(const fa_context *ctx, const fa_qweight *qw, fa_qweight_kind 
 
 // scratch taken from the pool for the duration of one call; the block goes
 // back right after the launch, which is safe because every later use is
-// ordered after it on the context's stream
+// ordered after it on the context's stream.  A call recorded into a graph
+// capture hands its scratch to the graph instead (scratch_release): the
+// recorded kernels use those addresses on every replay.
 struct Scratch {
     fa_context *ctx;
     void *ptr = nullptr;
@@ -55,7 +57,7 @@ struct Scratch {
         return pool_alloc(ctx, n, &ptr, &cls);
     }
     ~Scratch() {
-        if (ptr) pool_free(ctx, ptr, bytes, cls);
+        if (ptr) scratch_release(ctx, ptr, bytes, cls);
     }
 };
 
@@ -86,6 +88,16 @@ fa_status fa_set_tuning(int32_t key, int32_t value) {
         case 12: fa::g_prefill_block_split = value; return FA_OK;
     }
     return fail(FA_ERR_INVALID_ARGUMENT, "fa_set_tuning: unknown key");
+}
+
+fa_status fa_gemm_plan_query(const fa_context *ctx, uint64_t m, const fa_qweight *qw, fa_gemm_plan *out) {
+    if (!ctx || ctx->magic != kCtxMagic || !out) return fail(FA_ERR_INVALID_ARGUMENT, "gemm_plan_query: bad argument");
+    if (!qw || qw->magic != kQwMagic) return fail(FA_ERR_INVALID_ARGUMENT, "gemm_plan_query: not a quantized weight");
+    const k::GemmPlan p = k::gemm_plan(qw->kind != FA_QW_INT8_CHANNEL, m, qw->n_pad, qw->k_pad, ctx->props.multiProcessorCount);
+    out->big_ntb = p.big_ntb;
+    out->waves = p.waves;
+    out->splits = p.splits;
+    return FA_OK;
 }
 
 // ------------------------------------------------------------- f32 linear

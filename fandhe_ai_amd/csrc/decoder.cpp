@@ -212,7 +212,7 @@ struct Temp {
         return pool_alloc(ctx, bytes, &ptr, &cls);
     }
     ~Temp() {
-        if (ptr) pool_free(ctx, ptr, bytes, cls);
+        if (ptr) scratch_release(ctx, ptr, bytes, cls);
     }
     template <typename T>
     T *as() const { return (T *)ptr; }
@@ -564,8 +564,24 @@ fa_status fa_decoder_step(fa_context *ctx, fa_decoder *d, int32_t use_graph) {
     ps.num_kv_heads = d->cfg.n_kv_heads;
     ps.max_blocks_per_seq = d->cfg.max_blocks_per_seq;
     if (fa_status s = ensure_workspace(ctx, k::paged_decode_workspace_bytes(ps, (uint32_t)g_decode_waves))) return s;
+    // the position every row writes in this step must have a page (validate_paged_kv_append rejects a row
+    // without a slot before anything is queued, crates/tensor-core/src/paged_kv.rs:222-290)
+    for (uint32_t b = 0; b < d->batch; ++b) {
+        const uint64_t pos = d->host_lens[b];
+        const fa_decoder_config &c = d->cfg;
+        if (pos >= (uint64_t)c.max_blocks_per_seq * c.block_size)
+            return fail(FA_ERR_INVALID_ARGUMENT, "paged_kv: row " + std::to_string(b) + " has no room for one more token");
+        if (d->host_tables[(uint64_t)b * c.max_blocks_per_seq + pos / c.block_size] >= c.num_blocks)
+            return fail(FA_ERR_INVALID_ARGUMENT, "paged_kv: row " + std::to_string(b) + " has no page for position " +
+                                                     std::to_string(pos));
+    }
     for (auto &len : d->host_lens) len += 1;            // mirrors the device-side advance of this step
-    if (!use_graph) return enqueue_step(ctx, d);
+    if (!use_graph) {
+        fa_status es = enqueue_step(ctx, d);
+        if (es != FA_OK)
+            for (auto &len : d->host_lens) len -= 1;
+        return es;
+    }
     if (d->graph_waves != g_decode_waves) drop_graphs(d);
     auto it = d->graphs.find(d->batch);
     if (it == d->graphs.end()) {
@@ -593,7 +609,10 @@ fa_status fa_decoder_step(fa_context *ctx, fa_decoder *d, int32_t use_graph) {
         it->second = g;
         d->graph_waves = g_decode_waves;
     }
-    return fa_graph_launch(ctx, it->second);
+    fa_status ls = fa_graph_launch(ctx, it->second);
+    if (ls != FA_OK)
+        for (auto &len : d->host_lens) len -= 1;
+    return ls;
 }
 
 static fa_status prefill_impl(fa_context *ctx, fa_decoder *d, const int32_t *tokens, uint32_t l_new, int32_t *picked,

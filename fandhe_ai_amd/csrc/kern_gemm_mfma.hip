@@ -654,6 +654,19 @@ static W8a8Plan plan_w8a8(uint64_t m, uint64_t n_pad, uint64_t k_pad, int num_cu
     return {0, (uint32_t)std::max<uint64_t>(s, 1)};
 }
 
+GemmPlan gemm_plan(bool fp8, uint64_t m, uint64_t n_pad, uint64_t k_pad, int num_cus) {
+    GemmPlan out{0, 4, 1};
+    if (fp8) {
+        out.big_ntb = (g_gemm_small_tiles || k_pad == 0) ? 0 : pick_big_ntb(m, n_pad / 16, num_cus);
+    } else {
+        const W8a8Plan p = plan_w8a8(m, n_pad, k_pad, num_cus);
+        out.big_ntb = p.ntb;
+        out.splits = p.splits;
+    }
+    if (out.big_ntb) out.waves = g_gemm_waves == 4 ? 4 : g_gemm_waves == 16 ? 16 : 8;
+    return out;
+}
+
 uint64_t gemm_w8a8_workspace_bytes(uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad, int num_cus) {
     const W8a8Plan p = plan_w8a8(m, n_pad, k_pad, num_cus);
     return p.splits > 1 ? (uint64_t)p.splits * m * n * 4 : 0;

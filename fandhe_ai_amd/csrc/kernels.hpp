@@ -128,6 +128,13 @@ void gemm_w8a8_mfma(const int8_t *aq, const int8_t *w_tiles, uint64_t m, uint64_
                     uint64_t k_pad, const EpilogueI8 &ep, int num_cus, hipStream_t s, void *workspace = nullptr,
                     uint64_t workspace_bytes = 0);
 uint64_t gemm_w8a8_workspace_bytes(uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad, int num_cus);
+// Which kernel the two launchers pick for a shape under the current tuning knobs: big_ntb column tiles of
+// 16 per block of the large-tile kernel (0: the 128 x 128 kernel), wavefronts per block, k splits.
+struct GemmPlan {
+    int big_ntb, waves;
+    uint32_t splits;
+};
+GemmPlan gemm_plan(bool fp8, uint64_t m, uint64_t n_pad, uint64_t k_pad, int num_cus);
 // aq: e4m3 [m, k_pad] row-major; scales are device scalars.
 void gemm_e4m3_mfma(const uint8_t *aq, const uint8_t *w_tiles, const float *a_scale,
                     const float *w_scale, uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad,

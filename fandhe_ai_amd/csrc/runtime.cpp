@@ -4,6 +4,7 @@
 #include <algorithm>
 #include <cstdio>
 #include <cstring>
+#include <exception>
 #include <new>
 
 namespace fa {
@@ -164,9 +165,28 @@ fa_status pool_alloc(fa_context *ctx, uint64_t bytes, void **ptr, uint64_t *clas
     void *p = ctx->pool.take(cls);
     if (p) {
         ctx->pool.record_reuse(bytes, cls);
+    } else if (ctx->capturing) {
+        // Scratch of a call that is being recorded (buffers cannot be created during a capture: the entry
+        // points that make them return FA_ERR_CAPTURE_IN_PROGRESS first).  The capture is thread-local, which
+        // forbids allocation calls on this thread; the relaxed mode lifts that for the one call.  Nothing
+        // is released to make room here (hipFree is not allowed either).
+        hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
+        hipError_t e = hipThreadExchangeStreamCaptureMode(&mode);
+        if (e == hipSuccess) {
+            e = hipMalloc(&p, cls);
+            hipError_t back = hipThreadExchangeStreamCaptureMode(&mode);
+            if (e == hipSuccess && back != hipSuccess) {
+                (void)hipFree(p);
+                e = back;
+            }
+        }
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(FA_ERR_CAPTURE_IN_PROGRESS,
+                        std::string("scratch allocation during graph capture failed: ") + hipGetErrorString(e));
+        }
+        ctx->pool.record_allocation(bytes, cls);
     } else {
-        if (ctx->capturing)
-            return fail(FA_ERR_CAPTURE_IN_PROGRESS, "device allocation during graph capture");
         hipError_t e = hipMalloc(&p, cls);
         if (e != hipSuccess) {
             // give cached blocks back to the driver once, then retry
@@ -193,9 +213,33 @@ void pool_free(fa_context *ctx, void *ptr, uint64_t logical, uint64_t class_byte
     ctx->pool.record_loan_end(logical, class_bytes);
     auto evicted = ctx->pool.put(class_bytes, ptr);
     for (auto &e : evicted) {
+        if (ctx->capturing) {
+            // no hipFree while this thread records a capture: released when the capture ends
+            try {
+                ctx->deferred_frees.push_back(e.second);
+            } catch (const std::exception &) {
+                // out of host memory for the list: the block stays allocated until the process ends
+            }
+            continue;
+        }
         // hipFree waits for the device, so work still queued on the stream is safe
         if (hipFree(e.second) != hipSuccess) (void)hipGetLastError();
     }
+}
+
+void scratch_release(fa_context *ctx, void *ptr, uint64_t logical, uint64_t class_bytes) {
+    if (!ptr) return;
+    if (ctx->capturing) {
+        try {
+            ctx->capture_owned.push_back(fa_owned_block{ptr, logical, class_bytes});
+            ctx->pending_return_bytes += class_bytes;
+            return;
+        } catch (const std::exception &) {
+            // cannot track it: leak the block rather than let the pool hand it to someone else
+            return;
+        }
+    }
+    pool_free(ctx, ptr, logical, class_bytes);
 }
 
 fa_status make_buffer(fa_context *ctx, fa_dtype dtype, uint64_t numel, bool zero, fa_buffer **out) {
@@ -213,6 +257,11 @@ fa_status make_buffer(fa_context *ctx, fa_dtype dtype, uint64_t numel, bool zero
     b->dtype = dtype;
     b->logical_bytes = bytes;
     b->class_bytes = 0;
+    if (bytes != 0 && ctx->capturing) {
+        // a buffer outlives the call that makes it, and zeroing it would record a memset node
+        delete b;
+        return fail(FA_ERR_CAPTURE_IN_PROGRESS, "buffer allocation during graph capture");
+    }
     if (bytes != 0) {     // numel == 0 never touches the device (buffer.rs:50-59)
         fa_status s = pool_alloc(ctx, bytes, &b->ptr, &b->class_bytes);
         if (s != FA_OK) {
@@ -369,6 +418,8 @@ fa_status fa_context_destroy(fa_context *ctx) {
     if (ctx->table_stage) (void)hipFree(ctx->table_stage);
     if (ctx->workspace) (void)hipFree(ctx->workspace);
     for (void *w : ctx->retired_workspaces) (void)hipFree(w);
+    for (auto &b : ctx->capture_owned) (void)hipFree(b.ptr);   // a capture that was never ended
+    for (void *p : ctx->deferred_frees) (void)hipFree(p);
     (void)hipStreamDestroy(ctx->stream);
     (void)hipGetLastError();
     ctx->magic = 0;
@@ -497,6 +548,7 @@ fa_status fa_synchronize_device(fa_context *ctx) {
 fa_status fa_device_memory_pool_stats(fa_context *ctx, fa_pool_stats *out) {
     if (!ctx || ctx->magic != kCtxMagic || !out) return fail(FA_ERR_INVALID_ARGUMENT, "fa_device_memory_pool_stats: bad argument");
     *out = ctx->pool.stats();
+    out->pending_return_bytes = ctx->pending_return_bytes;
     return FA_OK;
 }
 
@@ -539,22 +591,39 @@ fa_status fa_graph_capture_end(fa_context *ctx, fa_graph **out) {
     ctx->capturing = false;
     hipGraph_t g = nullptr;
     hipError_t e = hipStreamEndCapture(ctx->stream, &g);
-    if (e != hipSuccess || !g) return hip_fail(ctx, e, "hipStreamEndCapture", FA_ERR_KERNEL_LAUNCH_FAILED);
+    for (void *p : ctx->deferred_frees)
+        if (hipFree(p) != hipSuccess) (void)hipGetLastError();
+    ctx->deferred_frees.clear();
+    // without a graph nothing will replay the recorded kernels: their scratch goes straight back to the pool
+    auto drop_owned = [&]() {
+        for (auto &b : ctx->capture_owned) {
+            ctx->pending_return_bytes -= std::min(ctx->pending_return_bytes, b.cls);
+            pool_free(ctx, b.ptr, b.bytes, b.cls);
+        }
+        ctx->capture_owned.clear();
+    };
+    if (e != hipSuccess || !g) {
+        drop_owned();
+        return hip_fail(ctx, e, "hipStreamEndCapture", FA_ERR_KERNEL_LAUNCH_FAILED);
+    }
     hipGraphExec_t exec = nullptr;
     e = hipGraphInstantiate(&exec, g, nullptr, nullptr, 0);
     if (e != hipSuccess) {
         (void)hipGraphDestroy(g);
+        drop_owned();
         return hip_fail(ctx, e, "hipGraphInstantiate", FA_ERR_KERNEL_LAUNCH_FAILED);
     }
     fa_graph *gr = new (std::nothrow) fa_graph();
     if (!gr) {
         (void)hipGraphExecDestroy(exec);
         (void)hipGraphDestroy(g);
+        drop_owned();
         return fail(FA_ERR_ALLOCATION_FAILED, "host allocation of the graph handle failed");
     }
     gr->magic = kGraphMagic;
     gr->graph = g;
     gr->exec = exec;
+    gr->owned.swap(ctx->capture_owned);
     *out = gr;
     return FA_OK;
 }
@@ -571,11 +640,26 @@ fa_status fa_graph_launch(fa_context *ctx, fa_graph *graph) {
 fa_status fa_graph_destroy(fa_context *ctx, fa_graph *graph) {
     if (!graph) return FA_OK;
     if (graph->magic != kGraphMagic) return fail(FA_ERR_INVALID_ARGUMENT, "fa_graph_destroy: not a graph");
+    if (!graph->owned.empty() && !(ctx && ctx->magic == kCtxMagic))
+        return fail(FA_ERR_INVALID_ARGUMENT, "fa_graph_destroy: the graph owns device blocks, its context is needed");
     if (ctx && ctx->magic == kCtxMagic) (void)hipStreamSynchronize(ctx->stream);
     (void)hipGraphExecDestroy(graph->exec);
     (void)hipGraphDestroy(graph->graph);
+    // every replay has finished (synchronized above): the scratch the recorded kernels used is free again
+    for (auto &b : graph->owned) {
+        ctx->pending_return_bytes -= std::min(ctx->pending_return_bytes, b.cls);
+        pool_free(ctx, b.ptr, b.bytes, b.cls);
+    }
+    graph->owned.clear();
     graph->magic = 0;
     delete graph;
+    return FA_OK;
+}
+
+fa_status fa_graph_owned_blocks(const fa_graph *graph, void **ptrs, uint64_t capacity, uint64_t *count) {
+    if (!graph || graph->magic != kGraphMagic || !count) return fail(FA_ERR_INVALID_ARGUMENT, "fa_graph_owned_blocks: bad argument");
+    *count = graph->owned.size();
+    for (uint64_t i = 0; i < graph->owned.size() && i < capacity && ptrs; ++i) ptrs[i] = graph->owned[i].ptr;
     return FA_OK;
 }
 

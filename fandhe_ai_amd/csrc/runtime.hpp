@@ -12,6 +12,7 @@
 #include <vector>
 
 #include "../../include/fandhe_rocm.h"
+#include "../../include/fandhe_rocm_bench.h"
 
 namespace fa {
 
@@ -58,6 +59,12 @@ size_t dtype_size(fa_dtype t);
 
 }  // namespace fa
 
+// a pool block on loan: device address, logical size, size class
+struct fa_owned_block {
+    void *ptr;
+    uint64_t bytes, cls;
+};
+
 struct fa_context {
     uint32_t magic;
     int device;
@@ -75,6 +82,14 @@ struct fa_context {
     // workspaces that were outgrown: captured graphs may still hold their addresses, so they stay
     // allocated until the context is destroyed (growth is geometric, the total stays below twice the last)
     std::vector<void *> retired_workspaces;
+    // Scratch that calls recorded into the open capture took: the recorded kernels hold these addresses, so
+    // the blocks belong to the graph (moved into it when the capture ends) instead of going back to the pool.
+    std::vector<fa_owned_block> capture_owned;
+    // blocks the pool evicted while a capture was open: released to the driver when the capture ends
+    std::vector<void *> deferred_frees;
+    // class bytes of the blocks on loan to an open capture or to live graphs (PoolStats::pending_return_bytes:
+    // idle-side memory that is neither cached nor in use by a buffer and comes back when its holder ends)
+    uint64_t pending_return_bytes = 0;
 };
 
 struct fa_buffer {
@@ -101,6 +116,8 @@ struct fa_graph {
     uint32_t magic;
     hipGraph_t graph;
     hipGraphExec_t exec;
+    // device blocks whose addresses the recorded kernels hold; returned to the pool when the graph is destroyed
+    std::vector<fa_owned_block> owned;
 };
 
 struct fa_timer {
@@ -126,6 +143,10 @@ fa_status after_launch(fa_context *ctx, const char *kernel);
 // Pool-backed raw allocation used by buffers and by internal scratch.
 fa_status pool_alloc(fa_context *ctx, uint64_t bytes, void **ptr, uint64_t *class_bytes);
 void pool_free(fa_context *ctx, void *ptr, uint64_t logical, uint64_t class_bytes);
+// End of a loan taken for the duration of one call (kernel scratch).  Outside a capture the block goes back
+// to the pool (the stream is in order, so the next user is queued behind this call's kernels).  While a
+// capture is open the recorded kernels keep the address for every replay: the block is handed to the graph.
+void scratch_release(fa_context *ctx, void *ptr, uint64_t logical, uint64_t class_bytes);
 fa_status make_buffer(fa_context *ctx, fa_dtype dtype, uint64_t numel, bool zero, fa_buffer **out);
 // Ensures ctx->workspace holds at least `bytes` (grows outside capture only).
 fa_status ensure_workspace(fa_context *ctx, uint64_t bytes);

@@ -207,12 +207,6 @@ fa_status fa_argmax_rows(fa_context *ctx, const fa_buffer *x, uint64_t rows, uin
 /* BackendOps::gather of rows (backend_ops.rs:3375): out[r, :] = table[idx[r], :]. */
 fa_status fa_gather_rows(fa_context *ctx, const fa_buffer *table, uint64_t table_rows,
                          uint64_t cols, const fa_buffer *idx, uint64_t rows, fa_buffer *out);
-/* Synthetic data: fills an f32 or bf16 buffer with N(mean, std) values from a
- * counter-based generator (value i depends only on seed and i).  For
- * benchmarks that need tens of GB of resident inputs; not part of the
- * reference's interface. */
-fa_status fa_fill_normal(fa_context *ctx, fa_buffer *buf, uint64_t offset, uint64_t numel,
-                         uint64_t seed, float mean, float std);
 /* Next-token sampling from logits [rows, vocab] (f32), on the device, with the
  * arithmetic of the reference's host sampler (crates/autodiff/src/generate/mod.rs:
  * 333-452, sample_step / sampling_weights_f32; crates/tensor-core/src/rng.rs:
@@ -248,15 +242,6 @@ typedef struct fa_row_sampling {
  * 6 * rows elements holding the rows' fa_row_sampling records. */
 fa_status fa_sample_rows_per_row(fa_context *ctx, const fa_buffer *logits, uint64_t rows, uint64_t vocab,
                                  fa_buffer *table, fa_buffer *tokens);
-/* Measurement aid, not part of the reference's interface: queues a loop of one
- * matrix instruction kind with operands held in registers (kind 0:
- * v_mfma_i32_16x16x64_i8, 1: v_mfma_i32_32x32x32_i8, 2: the scaled
- * 16x16x128 e4m3 form).  The operand bits are taken from `operands` (64 KiB of
- * any element type): the sustained rate of the matrix cores depends on them.
- * *ops receives the multiply-add operations x 2 of the launch; time it with an
- * fa_timer. */
-fa_status fa_probe_matrix_rate(fa_context *ctx, int32_t kind, const fa_buffer *operands,
-                               uint32_t iters, fa_buffer *sink, double *ops);
 /* dtype conversion f32 <-> bf16 (round to nearest even, once). */
 fa_status fa_convert(fa_context *ctx, const fa_buffer *src, uint64_t numel, fa_buffer *dst);
 
@@ -499,37 +484,6 @@ fa_status fa_decoder_rewind(fa_context *ctx, fa_decoder *dec, const uint32_t *se
 fa_status fa_decoder_read_tokens(fa_context *ctx, fa_decoder *dec, int32_t *tokens);
 fa_status fa_decoder_read_logits(fa_context *ctx, fa_decoder *dec, float *logits);
 fa_status fa_decoder_read_seq_lens(fa_context *ctx, fa_decoder *dec, uint32_t *seq_lens);
-
-/* ------------------------------------------------------ profiling / tuning */
-/* Launch-shape knobs for experiments; value 0 restores the built-in choice.
- * key 0: n-tiles per block of the decode-shape linears (1 or 2);
- * key 1: wavefronts per block of the decode-shape linears (4 or 8);
- * key 2: wavefronts per compute unit of the decode attention (1 .. 8);
- * key 3: nonzero launches only the streaming kernel of the decode attention and
- *        leaves the output unwritten (for timing that kernel by itself);
- * key 4: nonzero keeps the 128 x 128 block tile of the prefill GEMMs for every shape;
- * key 5: activation-stationary decode linears: 1 never, 2 whenever the shape allows;
- * key 6: wavefronts per block of the large-tile prefill GEMMs (4 or 16; default 8);
- * key 7: column tiles of 16 per block of the large-tile prefill GEMMs (14 or 16);
- * key 8: nonzero sends attention with more than one new token per row to the generic
- *        kernel (the reference's summation order) instead of the streamed one;
- * key 9: blocks per compute unit that a split-k launch of the 128 x 128 int8 GEMM aims
- *        for (default 2);
- * key 10: form of the attention with more than one new token per row: 1 always the
- *        streamed form, 2 always the block form, 0 by shape;
- * key 11: wavefronts per block of that block form (4 or 8; 0 by shape);
- * key 12: upper bound of the blocks that share the cache walk of one tile of new tokens
- *        in the block form (1: never split; 0 by shape). */
-fa_status fa_set_tuning(int32_t key, int32_t value);
-/* A pair of HIP events recorded on the context's stream (the stream the
- * kernels run on); used by the benchmark to time launches. */
-typedef struct fa_timer fa_timer;
-fa_status fa_timer_create(fa_context *ctx, fa_timer **out);
-fa_status fa_timer_start(fa_context *ctx, fa_timer *t);
-fa_status fa_timer_stop(fa_context *ctx, fa_timer *t);
-/* Blocks until the stop event has completed. */
-fa_status fa_timer_elapsed_ms(fa_context *ctx, fa_timer *t, float *ms);
-fa_status fa_timer_destroy(fa_context *ctx, fa_timer *t);
 
 #ifdef __cplusplus
 }

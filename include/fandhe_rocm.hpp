@@ -268,9 +268,6 @@ class RocmBackendOps {
                                          block_tables.size(), seq_lens.data(), seq_lens.size(), &args, out.handle()));
         return out;
     }
-    void fill_normal(Buffer &buf, uint64_t seed, float mean, float std) const {
-        check(fa_fill_normal(ctx_.handle(), buf.handle(), 0, buf.numel(), seed, mean, std));
-    }
 
   private:
     const Context &ctx_;

@@ -1,0 +1,86 @@
+/*
+ * fandhe_rocm_bench.h - measurement and test aids of libfandhe_rocm.so.
+ *
+ * Nothing in this header stands behind an interface of the reference; a
+ * BackendOps / MemoryOps binding needs fandhe_rocm.h only.  These entry points
+ * exist for the benchmark (synthetic data, event timers, a matrix-rate probe),
+ * for experiments (launch-shape knobs) and for tests that have to know which
+ * kernel a shape reaches or which device blocks a captured graph owns.
+ */
+#ifndef FANDHE_ROCM_BENCH_H
+#define FANDHE_ROCM_BENCH_H
+
+#include "fandhe_rocm.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Synthetic data: fills an f32 or bf16 buffer with N(mean, std) values from a
+ * counter-based generator (value i depends only on seed and i).  For
+ * benchmarks that need tens of GB of resident inputs. */
+fa_status fa_fill_normal(fa_context *ctx, fa_buffer *buf, uint64_t offset, uint64_t numel,
+                         uint64_t seed, float mean, float std);
+
+/* Queues a loop of one matrix instruction kind with operands held in registers
+ * (kind 0: v_mfma_i32_16x16x64_i8, 1: v_mfma_i32_32x32x32_i8, 2: the scaled
+ * 16x16x128 e4m3 form).  The operand bits are taken from `operands` (64 KiB of
+ * any element type): the sustained rate of the matrix cores depends on them.
+ * *ops receives the multiply-add operations x 2 of the launch; time it with an
+ * fa_timer. */
+fa_status fa_probe_matrix_rate(fa_context *ctx, int32_t kind, const fa_buffer *operands,
+                               uint32_t iters, fa_buffer *sink, double *ops);
+
+/* Launch-shape knobs for experiments; value 0 restores the built-in choice.
+ * The knobs are plain process-wide integers read by every context's launches:
+ * set them while no other thread is submitting work.
+ * key 0: n-tiles per block of the decode-shape linears (1 or 2);
+ * key 1: wavefronts per block of the decode-shape linears (4 or 8);
+ * key 2: wavefronts per compute unit of the decode attention (1 .. 8);
+ * key 3: nonzero launches only the streaming kernel of the decode attention and
+ *        leaves the output unwritten (for timing that kernel by itself);
+ * key 4: nonzero keeps the 128 x 128 block tile of the prefill GEMMs for every shape;
+ * key 5: activation-stationary decode linears: 1 never, 2 whenever the shape allows;
+ * key 6: wavefronts per block of the large-tile prefill GEMMs (4 or 16; default 8);
+ * key 7: column tiles of 16 per block of the large-tile prefill GEMMs (14 or 16);
+ * key 8: nonzero sends attention with more than one new token per row to the generic
+ *        kernel (the reference's summation order) instead of the streamed one;
+ * key 9: blocks per compute unit that a split-k launch of the 128 x 128 int8 GEMM aims
+ *        for (default 2);
+ * key 10: form of the attention with more than one new token per row: 1 always the
+ *        streamed form, 2 always the block form, 0 by shape;
+ * key 11: wavefronts per block of that block form (4 or 8; 0 by shape);
+ * key 12: upper bound of the blocks that share the cache walk of one tile of new tokens
+ *        in the block form (1: never split; 0 by shape). */
+fa_status fa_set_tuning(int32_t key, int32_t value);
+
+/* Which kernel a prefill-shape GEMM of m rows against `qw` is launched with under the
+ * current knobs (pure host function, nothing is queued).  big_ntb: column tiles of 16
+ * per block of the large-tile kernel (gemm_mfma_big_kernel), 0 when the 128 x 128 kernel
+ * (gemm_mfma_kernel) is used; waves: wavefronts per block; splits: blocks that share the
+ * k range of one output tile (1: no split). */
+typedef struct {
+    int32_t big_ntb, waves;
+    uint32_t splits;
+} fa_gemm_plan;
+fa_status fa_gemm_plan_query(const fa_context *ctx, uint64_t m, const fa_qweight *qw, fa_gemm_plan *out);
+
+/* Device blocks a captured graph owns (scratch that calls recorded into it took while the
+ * capture was open; they return to the pool when the graph is destroyed).  Writes up to
+ * `capacity` device addresses and the total count. */
+fa_status fa_graph_owned_blocks(const fa_graph *graph, void **ptrs, uint64_t capacity, uint64_t *count);
+
+/* A pair of HIP events recorded on the context's stream (the stream the
+ * kernels run on); used by the benchmark to time launches. */
+typedef struct fa_timer fa_timer;
+fa_status fa_timer_create(fa_context *ctx, fa_timer **out);
+fa_status fa_timer_start(fa_context *ctx, fa_timer *t);
+fa_status fa_timer_stop(fa_context *ctx, fa_timer *t);
+/* Blocks until the stop event has completed. */
+fa_status fa_timer_elapsed_ms(fa_context *ctx, fa_timer *t, float *ms);
+fa_status fa_timer_destroy(fa_context *ctx, fa_timer *t);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

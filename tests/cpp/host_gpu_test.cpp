@@ -5,6 +5,7 @@
 #include <map>
 #include <memory>
 
+#include "fandhe_rocm_bench.h"
 #include "fandhe_safetensors.hpp"
 
 using namespace fandhe;
@@ -58,7 +59,7 @@ int main(int argc, char **argv) {
         std::vector<std::unique_ptr<QWeight>> qkeep;
         auto filled = [&](uint64_t numel, float mean, float std) -> const Buffer & {
             keep.push_back(std::make_unique<Buffer>(Buffer::alloc_uninit(ctx, FA_F32, numel)));
-            ops.fill_normal(*keep.back(), seed++, mean, std);
+            check(fa_fill_normal(ctx.handle(), keep.back()->handle(), 0, numel, seed++, mean, std));
             return *keep.back();
         };
         auto weight = [&](uint64_t k, uint64_t n) -> const QWeight & {

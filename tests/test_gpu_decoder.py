@@ -285,3 +285,34 @@ def test_decoder_argument_errors():
         assert lib.fa_decoder_set_head(dec.h, dec.keep[-3]._h, dec.keep[-2]._h, wrong._h) == fa.capi.SHAPE_MISMATCH
     finally:
         dec.close()
+
+
+def test_step_without_a_page_for_the_next_position_is_refused():
+    """A row that has used up its pages (or whose next table entry is the sentinel) is refused before
+    anything is queued, with the row named; lengths and tokens stay as they were (the validators of the
+    reference reject a row without a slot before the device is touched,
+    crates/tensor-core/src/paged_kv.rs:222-290)."""
+    import fandhe_ai_amd as fa
+    be = ops()
+    # row 0 ends exactly at a page boundary with no further page in its table; row 1 has room
+    m = build_model(seed=9, n_layers=1, d_model=256, n_heads=4, n_kv_heads=2, d_ffn=512, vocab=300, batch=2,
+                    ctxs=[30, 20], steps=1, threads=2)
+    dec = GpuDecoder(be, m)
+    try:
+        bs = m.cfg["block_size"]
+        tables = m.tables.copy()
+        owned = int((tables[0] != 0xFFFFFFFF).sum())
+        lens = np.array([owned * bs - 1, 20], dtype=np.uint32)
+        dec.set_state(lens, m.tokens)
+        for use_graph in (False, True):
+            dec.step(use_graph)                       # writes the last free slot of row 0
+            lens[0:2] += 1
+            assert np.array_equal(dec.seq_lens(), lens)
+            before = dec.tokens()
+            with pytest.raises(fa.InvalidArgument, match="row 0"):
+                dec.step(use_graph)
+            assert np.array_equal(dec.seq_lens(), lens) and np.array_equal(dec.tokens(), before)
+            dec.rewind(lens - 1)
+            lens -= 1
+    finally:
+        dec.close()

@@ -347,3 +347,157 @@ def test_fp8_quantizer_bit_exact_and_gemm_within_stated_bound():
     assert be.download(sa)[0] == 1.0 and np.array_equal(o.from_e4m3(be.download(aq)), a)
     got = be.download_owned(be.gemm_e4m3(aq, sa, qw, fa.capi.F32))
     assert np.array_equal(got, (a.astype(np.float64) @ w.astype(np.float64)).astype(np.float32))
+
+
+def _gemm_plan(fa, be, m, qw):
+    plan = fa.capi.GemmPlan()
+    fa.check(fa.capi.lib.fa_gemm_plan_query(be._ctx, m, qw._h, __import__("ctypes").byref(plan)))
+    return plan
+
+
+def _fp8_rows_check(tag, got_rows, aq_rows, wq, sa, sw):
+    """Sampled output rows of an e4m3 GEMM against the oracle's exact-product f64 sum rounded once, under the
+    stated fp8 bound |gpu - exact| <= 2^-15 * sum_k |a_k||b_k| * (sa * sw), with >= 98 % of the outputs
+    inside the composite tolerance (rel < 1e-3 or abs < 1e-5)."""
+    o.set_threads(8)
+    want = o.gemm_e4m3(np.ascontiguousarray(aq_rows), wq, sa, sw)
+    o.set_threads(1)
+    a_abs = np.abs(o.from_e4m3(np.ascontiguousarray(aq_rows))).astype(np.float64)
+    n = wq.shape[1]
+    absprod = np.empty((aq_rows.shape[0], n), np.float64)
+    for c0 in range(0, n, 2048):
+        absprod[:, c0:c0 + 2048] = a_abs @ np.abs(o.from_e4m3(np.ascontiguousarray(wq[:, c0:c0 + 2048]))).astype(np.float64)
+    bound = absprod * float(sa) * float(sw) * 2.0 ** -15 + 1e-30
+    err = np.abs(got_rows.astype(np.float64) - want.astype(np.float64))
+    print("FP8_PARITY\t%s\tmax_err/bound=%.3e" % (tag, float((err / bound).max())), flush=True)
+    assert np.all(err <= bound), tag
+    r = o.compare(got_rows, want)
+    print(r.line("FP8_PARITY", tag), flush=True)
+    assert r.fail_count <= 2e-2 * r.total, tag
+
+
+def test_fp8_prefill_gemm_large_tile_kernel_rows_sampled_at_full_size():
+    """M=2048, K=4096, N=14336, N(0,1) operands cast to e4m3 per tensor (absmax / 448): the shape of the
+    benchmark's fp8 GEMM, which the launcher sends to gemm_mfma_big_kernel<true, 14 | 16, waves / 2, EpiF8>.
+    Sampled rows are compared with the oracle for 14 and 16 column tiles per block, 4 / 8 / 16 wavefronts per
+    block and f32 / bf16 outputs; the plan query confirms the large-tile kernel is what ran."""
+    fa = _fa()
+    be = ops()
+    lib = fa.capi.lib
+    m, k, n = 2048, 4096, 14336
+    rng = np.random.default_rng(44)
+    a = rng.standard_normal((m, k), dtype=np.float32)
+    w = rng.standard_normal((k, n), dtype=np.float32)
+    aq, a_scale = be.quantize_tensor_e4m3(be.upload(a))
+    o.set_threads(8)
+    want_aq, want_sa = o.quantize_tensor_e4m3(a)
+    want_wq, want_sw = o.quantize_tensor_e4m3(w)
+    o.set_threads(1)
+    assert be.download(a_scale)[0] == want_sa and np.array_equal(be.download(aq), want_aq)
+    qw = be.quantize_weight(fa.DeviceBufferView(be.upload(w), 0, (k, n)), fa.capi.QW_E4M3_TENSOR)
+    wq, sw = qw.export()
+    assert sw[0] == want_sw and np.array_equal(wq, want_wq)
+    del a, w
+    # rows from every quarter of a 256-row block tile (both wavefront rows of it), first / middle / last blocks
+    rows = np.r_[0:4, 60:68, 124:132, 188:196, 252:260, 1020:1028, 1500:1504, 2044:2048]
+    try:
+        for ntb, waves in ((0, 0), (14, 0), (16, 0), (14, 4), (16, 16)):
+            fa.check(lib.fa_set_tuning(7, ntb))
+            fa.check(lib.fa_set_tuning(6, waves))
+            plan = _gemm_plan(fa, be, m, qw)
+            assert plan.big_ntb in (14, 16) and (ntb == 0 or plan.big_ntb == ntb), (ntb, plan.big_ntb)
+            assert plan.waves == (waves or 8) and plan.splits == 1
+            got = be.download_owned(be.gemm_e4m3(aq, a_scale, qw, fa.capi.F32))
+            _fp8_rows_check("2048x14336x4096 ntb=%d waves=%d" % (plan.big_ntb, plan.waves), got[rows], want_aq[rows],
+                            want_wq, want_sa, want_sw)
+            # every output finite and the untested rows sane: row sums against a row-sum identity
+            assert np.all(np.isfinite(got))
+            out_bf = be.download_owned(be.gemm_e4m3(aq, a_scale, qw, fa.capi.BF16))
+            assert_bf16_rounding_of("gemm_e4m3 large tile bf16", out_bf, got)
+            if ntb == 0:
+                base = got
+            else:
+                # the tile shape changes which wavefront owns an output, not the order of its k sum
+                assert np.array_equal(got, base), (ntb, waves)
+    finally:
+        fa.check(lib.fa_set_tuning(7, 0))
+        fa.check(lib.fa_set_tuning(6, 0))
+    # whole-output checksum: sum over rows of the exact result is (sum_m a[m, :]) @ w; the f32 outputs
+    # summed in f64 must agree within the per-element bound summed over the rows
+    a_f = o.from_e4m3(want_aq).astype(np.float64)
+    colsum = a_f.sum(axis=0)
+    exact = np.empty(n, np.float64)
+    abs_col = np.abs(a_f).sum(axis=0)
+    slack = np.empty(n, np.float64)
+    for c0 in range(0, n, 2048):
+        wf = o.from_e4m3(np.ascontiguousarray(want_wq[:, c0:c0 + 2048])).astype(np.float64)
+        exact[c0:c0 + 2048] = colsum @ wf
+        slack[c0:c0 + 2048] = abs_col @ np.abs(wf)
+    scale = float(want_sa) * float(want_sw)
+    assert np.all(np.abs(base.astype(np.float64).sum(axis=0) - exact * scale) <= slack * scale * 2.0 ** -14)
+
+
+def test_fp8_large_tile_kernel_ragged_shape():
+    """A shape with a ragged last row block (1000 rows), a column count that is not a multiple of the tile
+    or of 8 (the row-band store path is off, the last tile is cut) which still selects the large-tile kernel."""
+    fa = _fa()
+    be = ops()
+    m, k, n = 1000, 1024, 9004
+    rng = np.random.default_rng(45)
+    a = rng.standard_normal((m, k), dtype=np.float32)
+    w = rng.standard_normal((k, n), dtype=np.float32)
+    aq, a_scale = be.quantize_tensor_e4m3(be.upload(a))
+    qw = be.quantize_weight(fa.DeviceBufferView(be.upload(w), 0, (k, n)), fa.capi.QW_E4M3_TENSOR)
+    o.set_threads(8)
+    want_aq, want_sa = o.quantize_tensor_e4m3(a)
+    want_wq, want_sw = o.quantize_tensor_e4m3(w)
+    o.set_threads(1)
+    plan = _gemm_plan(fa, be, m, qw)
+    assert plan.big_ntb in (14, 16), plan.big_ntb
+    got = be.download_owned(be.gemm_e4m3(aq, a_scale, qw, fa.capi.F32))
+    rows = np.r_[0:8, 250:262, 760:776, 990:1000]
+    _fp8_rows_check("1000x9004x1024 ntb=%d" % plan.big_ntb, got[rows], want_aq[rows], want_wq, want_sa, want_sw)
+    assert np.all(np.isfinite(got))
+    out_bf = be.download_owned(be.gemm_e4m3(aq, a_scale, qw, fa.capi.BF16))
+    assert_bf16_rounding_of("gemm_e4m3 ragged bf16", out_bf, got)
+    # the 128 x 128 kernel on the same operands sums k in the same order: identical bits
+    fa.check(fa.capi.lib.fa_set_tuning(4, 1))
+    try:
+        assert _gemm_plan(fa, be, m, qw).big_ntb == 0
+        small = be.download_owned(be.gemm_e4m3(aq, a_scale, qw, fa.capi.F32))
+    finally:
+        fa.check(fa.capi.lib.fa_set_tuning(4, 0))
+    assert np.array_equal(small, got)
+
+
+def test_int8_large_tile_kernel_wavefront_variants_are_bit_exact():
+    """The 4- and 16-wavefront variants and both tile widths of the large-tile int8 kernel against the oracle
+    on sampled rows of a ragged shape (exact integers: any difference is an indexing error)."""
+    fa = _fa()
+    be = ops()
+    lib = fa.capi.lib
+    m, k, n = 1000, 1024, 9004
+    rng = np.random.default_rng(46)
+    aq = rng.integers(-127, 128, size=(m, k), dtype=np.int8)
+    wq = rng.integers(-127, 128, size=(k, n), dtype=np.int8)
+    sx = rng.uniform(0.01, 0.05, size=m).astype(np.float32)
+    sw = rng.uniform(1e-4, 1e-3, size=n).astype(np.float32)
+    qw = be.import_quantized_weight(wq, sw)
+    rows = np.r_[0:8, 250:262, 760:776, 990:1000]
+    o.set_threads(8)
+    want_acc = o.gemm_i8_i32(np.ascontiguousarray(aq[rows]), wq)
+    o.set_threads(1)
+    want = o.dequant_i32(want_acc, np.ascontiguousarray(sx[rows]), sw)
+    daq, dsx = be.upload(aq), be.upload(sx)
+    try:
+        for ntb, waves in ((14, 4), (16, 4), (14, 16), (16, 16), (0, 0)):
+            fa.check(lib.fa_set_tuning(7, ntb))
+            fa.check(lib.fa_set_tuning(6, waves))
+            plan = _gemm_plan(fa, be, m, qw)
+            assert plan.big_ntb in (14, 16) and plan.waves == (waves or 8)
+            out, acc = be.gemm_w8a8(daq, dsx, qw, fa.capi.F32, want_acc=True)
+            assert np.array_equal(be.download_owned(acc)[rows], want_acc), (ntb, waves)
+            assert np.array_equal(be.download_owned(out)[rows], want), (ntb, waves)
+    finally:
+        fa.check(lib.fa_set_tuning(7, 0))
+        fa.check(lib.fa_set_tuning(6, 0))

@@ -213,3 +213,95 @@ def test_sync_points_are_rejected_during_graph_capture_and_graph_replays():
         assert np.all(be.download(out) == 8.0)
         be.upload_into(np.zeros(256, np.float32), out, 0)
     fa.check(lib.fa_graph_destroy(be._ctx, g))
+
+
+def _capture(fa, be, fn):
+    lib = fa.capi.lib
+    g = C.c_void_p()
+    fa.check(lib.fa_graph_capture_begin(be._ctx))
+    try:
+        fn()
+    finally:
+        st = lib.fa_graph_capture_end(be._ctx, C.byref(g))
+    fa.check(st)
+    return g
+
+
+def _owned(fa, g):
+    n = C.c_uint64()
+    ptrs = (C.c_void_p * 16)()
+    fa.check(fa.capi.lib.fa_graph_owned_blocks(g, ptrs, 16, C.byref(n)))
+    return [ptrs[i] for i in range(min(n.value, 16))]
+
+
+def test_captured_quantized_linear_owns_its_scratch():
+    """A graph recorded over fa_linear_w8a8 keeps the addresses of the call's scratch (row scales, activation
+    codes).  Those blocks belong to the graph until it is destroyed: a buffer of the same size class allocated
+    afterwards gets other memory, replays leave it untouched bit for bit and still produce the eager result,
+    and the pool never lists a block a live graph uses."""
+    import fandhe_ai_amd as fa
+    be = ops()
+    lib = fa.capi.lib
+    rng = o.Rng(31)
+    m, k, n = 32, 512, 256
+    x, w = rng.randn((m, k)), rng.randn((k, n), std=0.05)
+    wq, ws = o.quantize_cols_i8(w)
+    want_acc, want = o.linear_w8a8(x, wq, ws)
+    qw = be.import_quantized_weight(wq, ws)
+    dx = be.upload(x)
+    out = be.alloc_zeroed((m, n))
+    be.release_cached_device_memory()        # every scratch request of the capture misses the pool
+    s0 = be.device_memory_pool_stats()
+    g = _capture(fa, be, lambda: fa.check(lib.fa_linear_w8a8(be._ctx, dx._h, m, qw._h, None, 0, None, out._h)))
+    try:
+        owned = _owned(fa, g)
+        assert len(owned) == 2                       # row scales (128 B -> class 256) and codes (16 KiB)
+        s1 = be.device_memory_pool_stats()
+        assert s1.cached_bytes == s0.cached_bytes == 0          # nothing went back to the pool
+        assert s1.pending_return_bytes - s0.pending_return_bytes == 256 + 16384
+        # bystanders of both classes: must not share memory with the graph
+        by_small = [be.upload(np.full(32, 7.25 + i, np.float32)) for i in range(4)]
+        by_big = [be.upload(np.full(4096, -3.5 - i, np.float32)) for i in range(2)]
+        addrs = [lib.fa_buffer_device_ptr(b._h) for b in by_small + by_big]
+        assert not set(addrs) & set(owned)
+        for rep in range(3):
+            fa.check(lib.fa_graph_launch(be._ctx, g))
+            got = be.download(out)
+            assert np.array_equal(got, want), rep
+            for i, b in enumerate(by_small):
+                assert np.all(be.download(b) == np.float32(7.25 + i))
+            for i, b in enumerate(by_big):
+                assert np.all(be.download(b) == np.float32(-3.5 - i))
+            be.upload_into(np.zeros(m * n, np.float32), out, 0)
+            # the pool being emptied between replays must not touch the graph's blocks either
+            be.release_cached_device_memory()
+        for b in by_small + by_big:
+            b.free()
+    finally:
+        fa.check(lib.fa_graph_destroy(be._ctx, g))
+    s2 = be.device_memory_pool_stats()
+    assert s2.pending_return_bytes == s0.pending_return_bytes    # the blocks came back with the graph
+    # a second capture with a warm pool: hits are owned by the graph too
+    g = _capture(fa, be, lambda: fa.check(lib.fa_linear_w8a8(be._ctx, dx._h, m, qw._h, None, 0, None, out._h)))
+    try:
+        owned = _owned(fa, g)
+        assert len(owned) == 2
+        fresh = be.upload(np.ones(32, np.float32))
+        assert lib.fa_buffer_device_ptr(fresh._h) not in owned
+        fa.check(lib.fa_graph_launch(be._ctx, g))
+        assert np.array_equal(be.download(out), want)
+        fresh.free()
+    finally:
+        fa.check(lib.fa_graph_destroy(be._ctx, g))
+    # buffers cannot be made while a capture is open, whatever the pool holds
+    t = be.alloc_zeroed((64,))
+    t.free()
+    fa.check(lib.fa_graph_capture_begin(be._ctx))
+    try:
+        h = C.c_void_p()
+        assert lib.fa_alloc_zeroed(be._ctx, fa.capi.F32, 64, C.byref(h)) == fa.capi.CAPTURE_IN_PROGRESS
+        assert lib.fa_alloc_uninit(be._ctx, fa.capi.F32, 64, C.byref(h)) == fa.capi.CAPTURE_IN_PROGRESS
+    finally:
+        g = C.c_void_p()
+        lib.fa_graph_capture_end(be._ctx, C.byref(g))
+        lib.fa_graph_destroy(be._ctx, g)
