@@ -323,10 +323,10 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
                 const int pp = (p4 - r / 2 - (FP8 ? 0 : 2 * x)) & 3;
                 a_src[i][x] = aq + (uint64_t)row * k_bytes + pp * 32 + x * 16;
             }
-            // a block of NTB = 14 has no tiles 14, 15: the wavefronts that would move them repeat their
-            // first tile instead (same bytes to the same place, served by the L1), which keeps the main
-            // loop free of branches
-            uint32_t t = nt0 + (wave + NWAVES * i < NTB ? wave + NWAVES * i : wave);
+            // a block of NTB = 14 has no tiles 14, 15: the wavefronts that would move them repeat tiles
+            // 0, 1 instead (same bytes to the same place, served by the L1), which keeps the main loop
+            // free of branches
+            uint32_t t = nt0 + (wave + NWAVES * i) % NTB;
             t = t < n_tiles ? t : n_tiles - 1;
             b_src[i] = w_tiles + (uint64_t)t * k_steps * TILE + lane * B_L;
         }
@@ -363,7 +363,7 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
     };
     auto issue_b = [&](uint32_t ks, int slot, int idx) {
         const int i = idx / 2, h = idx % 2;
-        const int t = wave + NWAVES * i < NTB ? wave + NWAVES * i : wave;
+        const int t = (wave + NWAVES * i) % NTB;
         __builtin_amdgcn_global_load_lds((gptr)(b_src[i] + (uint64_t)ks * TILE + h * B_H),
                                          (lptr)(lds_b0 + slot * B_STAGE + t * TILE + h * 1024), 16, 0, 0);
     };

@@ -401,7 +401,7 @@ def test_fp8_prefill_gemm_large_tile_kernel_rows_sampled_at_full_size():
     # rows from every quarter of a 256-row block tile (both wavefront rows of it), first / middle / last blocks
     rows = np.r_[0:4, 60:68, 124:132, 188:196, 252:260, 1020:1028, 1500:1504, 2044:2048]
     try:
-        for ntb, waves in ((0, 0), (14, 0), (16, 0), (14, 4), (16, 16)):
+        for ntb, waves in ((0, 0), (14, 0), (16, 0), (14, 4), (16, 16), (14, 16)):
             fa.check(lib.fa_set_tuning(7, ntb))
             fa.check(lib.fa_set_tuning(6, waves))
             plan = _gemm_plan(fa, be, m, qw)
