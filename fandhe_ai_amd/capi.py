@@ -137,6 +137,9 @@ SIGNATURES = {
     "fa_paged_kv_append_device": (C.c_int32, [ctx_p, buf_p, buf_p, buf_p, buf_p, buf_p, u64, C.POINTER(PagedLayout)]),
     "fa_paged_attention_forward_device": (C.c_int32, [ctx_p, buf_p, buf_p, buf_p, buf_p, buf_p,
                                                       C.POINTER(PagedArgs), buf_p]),
+    "fa_paged_attention_decode_static": (C.c_int32, [ctx_p, buf_p, buf_p, buf_p, buf_p, buf_p,
+                                                     C.POINTER(PagedArgs), buf_p]),
+    "fa_paged_attention_decode_static_max_bytes": (u64, []),
     "fa_sample_rows": (C.c_int32, [ctx_p, buf_p, u64, u64, C.c_int32, C.c_float, u64, buf_p, buf_p]),
     "fa_rng_seed": (C.c_int32, [ctx_p, buf_p, u64]),
     "fa_decoder_set_sampling": (C.c_int32, [ctx_p, C.c_void_p, C.c_int32, C.c_float, u64, u64]),

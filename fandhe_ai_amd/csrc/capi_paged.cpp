@@ -1,6 +1,7 @@
 // C ABI: paged KV append and paged attention (host-table and device-table
 // variants).  Host tables are validated completely before any launch
 // (crates/backend-rocm/src/ops/paged_kv.rs:11-13: no partial writes).
+#include <mutex>
 #include <string>
 
 #include "kernels.hpp"
@@ -13,7 +14,49 @@ namespace fa {
 extern int g_decode_waves, g_prefill_generic;
 }
 
+// ------------------------------------------------ scratch of the entry point that allocates nothing
+// Partial results of the decode attention for callers that cannot allocate (under a graph capture of their
+// own, in a serving loop that forbids it).  One array per GPU, held until the process ends; every call on a
+// GPU shares it, so calls that overlap on one GPU race.  `scratch` is a host-side stand-in for the symbol:
+// the device address is looked up once per device (scratch_address) and only that address is handed to
+// kernels.
+constexpr uint64_t kStaticScratchBytes = 16ull << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 namespace {
+
+constexpr int kMaxDevices = 64;
+void *g_scratch_addr[kMaxDevices];      // per device: each GPU holds its own copy of the array
+bool g_scratch_tried[kMaxDevices];
+std::mutex g_scratch_mu;
+
+}  // namespace
+
+namespace fa {
+// Called with `device` current (context creation).  The lookup may initialise the module on that device,
+// which is why it happens at set-up and not inside the entry point.
+void static_scratch_init(int device) {
+    if (device < 0 || device >= kMaxDevices) return;
+    std::lock_guard<std::mutex> g(g_scratch_mu);
+    if (g_scratch_tried[device]) return;
+    g_scratch_tried[device] = true;
+    void *ptr = nullptr;
+    hipError_t e = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return;                           // the entry point reports it
+    }
+    g_scratch_addr[device] = ptr;
+}
+}  // namespace fa
+
+namespace {
+
+void *scratch_address(int device) {
+    if (device < 0 || device >= kMaxDevices) return nullptr;
+    std::lock_guard<std::mutex> g(g_scratch_mu);
+    return g_scratch_addr[device];
+}
 
 fa_status same_storage(const fa_buffer *a, const fa_buffer *b, const char *what) {
     if (a->dtype != b->dtype) return fail(FA_ERR_INVALID_ARGUMENT, std::string(what) + ": element types differ");
@@ -182,9 +225,13 @@ fa_status fa_paged_attention_forward(fa_context *ctx, const fa_buffer *q, const 
                             (const uint32_t *)((char *)ctx->table_stage + lens_off), args, plan.s_max, longest, out);
 }
 
-fa_status fa_paged_attention_forward_device(fa_context *ctx, const fa_buffer *q, const fa_buffer *k_pool,
-                                            const fa_buffer *v_pool, const fa_buffer *block_tables,
-                                            const fa_buffer *seq_lens, const fa_paged_args *args, fa_buffer *out) {
+// argument checks shared by the two device-table entry points; *s_stride receives the longest sequence the
+// tables can describe, *done is set when there is nothing to compute
+static fa_status check_device_attention(fa_context *ctx, const fa_buffer *q, const fa_buffer *k_pool,
+                                        const fa_buffer *v_pool, const fa_buffer *block_tables,
+                                        const fa_buffer *seq_lens, const fa_paged_args *args, fa_buffer *out,
+                                        uint64_t *s_stride, bool *done) {
+    *done = false;
     if (fa_status s = check_ctx(ctx)) return s;
     if (fa_status s = paged_args_check(args)) return s;
     if (fa_status s = check_attention_buffers(ctx, q, k_pool, v_pool, out)) return s;
@@ -200,12 +247,57 @@ fa_status fa_paged_attention_forward_device(fa_context *ctx, const fa_buffer *q,
                                       "paged_attention: block_tables"))
         return s;
     if (fa_status s = check_buf_typed(ctx, seq_lens, FA_U32, args->batch, "paged_attention: seq_lens")) return s;
-    if (out_numel == 0) return FA_OK;
+    if (out_numel == 0) {
+        *done = true;
+        return FA_OK;
+    }
     uint64_t query_rows = args->batch * args->num_heads * args->l_new;
     if (query_rows > (uint64_t)INT32_MAX) return fail(FA_ERR_INVALID_ARGUMENT, "paged_kv: B * H * L_new exceeds i32::MAX");
-    uint64_t s_stride = args->max_blocks_per_seq * l->block_size;     // longest sequence the tables can describe
+    *s_stride = args->max_blocks_per_seq * l->block_size;
+    return FA_OK;
+}
+
+fa_status fa_paged_attention_forward_device(fa_context *ctx, const fa_buffer *q, const fa_buffer *k_pool,
+                                            const fa_buffer *v_pool, const fa_buffer *block_tables,
+                                            const fa_buffer *seq_lens, const fa_paged_args *args, fa_buffer *out) {
+    uint64_t s_stride = 0;
+    bool done = false;
+    if (fa_status s = check_device_attention(ctx, q, k_pool, v_pool, block_tables, seq_lens, args, out, &s_stride, &done))
+        return s;
+    if (done) return FA_OK;
     return launch_attention(ctx, q, k_pool, v_pool, (const uint32_t *)block_tables->ptr,
                             (const uint32_t *)seq_lens->ptr, args, s_stride, 0, out);
 }
+
+fa_status fa_paged_attention_decode_static(fa_context *ctx, const fa_buffer *q, const fa_buffer *k_pool,
+                                           const fa_buffer *v_pool, const fa_buffer *block_tables,
+                                           const fa_buffer *seq_lens, const fa_paged_args *args, fa_buffer *out) {
+    uint64_t s_stride = 0;
+    bool done = false;
+    if (fa_status s = check_device_attention(ctx, q, k_pool, v_pool, block_tables, seq_lens, args, out, &s_stride, &done))
+        return s;
+    if (done) return FA_OK;
+    const k::PagedShape ps = make_shape(args);
+    if (!(stream_fast_path(ps, q) && ps.l_new == 1))
+        return fail(FA_ERR_UNSUPPORTED,
+                    "paged_attention_decode_static: only the decode shape of the streamed kernel (bf16, head_dim 128, "
+                    "block_size 16, one new token per row, at most 16 query heads per kv head)");
+    const uint64_t need = k::paged_decode_workspace_bytes(ps, (uint32_t)g_decode_waves);
+    if (need > kStaticScratchBytes)
+        return fail(FA_ERR_INVALID_ARGUMENT,
+                    "paged_attention_decode_static: the partial results of this shape need " + std::to_string(need) +
+                        " bytes, the static scratch holds " + std::to_string(kStaticScratchBytes) +
+                        " (fewer rows or kv heads, or fa_paged_attention_forward_device)");
+    void *ws = scratch_address(ctx->device);
+    if (!ws)
+        return fail(FA_ERR_DEVICE_UNAVAILABLE, "paged_attention_decode_static: the address of the static scratch could not "
+                                               "be resolved when the context was created");
+    k::paged_attention_decode_bf16((const uint16_t *)q->ptr, (const uint16_t *)k_pool->ptr, (const uint16_t *)v_pool->ptr,
+                                   (const uint32_t *)block_tables->ptr, (const uint32_t *)seq_lens->ptr, ps,
+                                   (uint32_t)g_decode_waves, ws, out->ptr, out->dtype == FA_BF16, nullptr, ctx->stream);
+    return after_launch(ctx, "paged_attention_decode_static");
+}
+
+uint64_t fa_paged_attention_decode_static_max_bytes(void) { return kStaticScratchBytes; }
 
 }  // extern "C"

@@ -400,6 +400,7 @@ fa_status fa_context_create(int32_t ordinal, fa_context **out) {
     ctx->table_stage_bytes = 0;
     ctx->workspace = nullptr;
     ctx->workspace_bytes = 0;
+    static_scratch_init(ordinal);
     e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
     if (e != hipSuccess) {
         delete ctx;

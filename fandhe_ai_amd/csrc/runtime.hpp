@@ -151,5 +151,8 @@ fa_status make_buffer(fa_context *ctx, fa_dtype dtype, uint64_t numel, bool zero
 // Ensures ctx->workspace holds at least `bytes` (grows outside capture only).
 fa_status ensure_workspace(fa_context *ctx, uint64_t bytes);
 fa_status ensure_table_stage(fa_context *ctx, uint64_t bytes);
+// Resolves the device address of the static scratch of fa_paged_attention_decode_static on `device`, which
+// must be current; once per device.
+void static_scratch_init(int device);
 
 }  // namespace fa

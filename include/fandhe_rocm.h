@@ -306,6 +306,21 @@ fa_status fa_paged_attention_forward_device(fa_context *ctx, const fa_buffer *q,
                                             const fa_buffer *block_tables, const fa_buffer *seq_lens,
                                             const fa_paged_args *args, fa_buffer *out);
 
+/* No counterpart in the reference.  fa_paged_attention_forward_device for callers that cannot allocate:
+ * code under a HIP graph capture of its own, serving loops and harnesses that forbid hipMalloc.  The partial
+ * results of the streamed decode kernel live in a static device array of the library (16 MiB per GPU, held
+ * until the process ends) instead of the context's pooled workspace, and the call allocates and frees
+ * nothing.  Decode shape of the streamed kernel only (bf16, head_dim 128, block_size 16, l_new 1, at most 16
+ * query heads per kv head): FA_ERR_UNSUPPORTED otherwise; a shape whose partial results exceed the array
+ * ((ranges + batch) * kv heads * 520 floats * padded group / 4; a batch of 64 with 8 kv heads needs 3.2 MB)
+ * is FA_ERR_INVALID_ARGUMENT.  Same results, bit for bit, as fa_paged_attention_forward_device.  All calls
+ * on one GPU share the array: calls that overlap on one GPU (two contexts, two streams) race. */
+fa_status fa_paged_attention_decode_static(fa_context *ctx, const fa_buffer *q, const fa_buffer *k_pool,
+                                           const fa_buffer *v_pool, const fa_buffer *block_tables,
+                                           const fa_buffer *seq_lens, const fa_paged_args *args, fa_buffer *out);
+/* Size in bytes of that array. */
+uint64_t fa_paged_attention_decode_static_max_bytes(void);
+
 /* ---------------------------------------------------- paged KV cache (layer) */
 /* The caller side of the paged operators: page table with free-block
  * bookkeeping and the one-layer device-resident cache built on it.
