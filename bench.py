@@ -242,8 +242,8 @@ def bench_w8a8_decode(fa, be, cfg, m, iters):
     return res
 
 
-def bench_linears(fa, be, iters):
-    """Decode-shape int8-weight linears: bf16 activations (W8A16) and W8A8, Llama-7B layer shapes."""
+def bench_linears(fa, be, iters, ms=(1, 8, 32)):
+    """Decode-shape int8-weight linears with bf16 activations (W8A16), Llama-7B layer shapes."""
     lib = fa.capi.lib
     res = []
     for k, n in ((4096, 12288), (4096, 4096), (4096, 22016), (11008, 4096)):
@@ -251,7 +251,7 @@ def bench_linears(fa, be, iters):
         fa.check(lib.fa_fill_normal(be._ctx, w._h, 0, k * n, k + n, 0.0, 0.02))
         qw = be.quantize_weight(fa.DeviceBufferView(w, 0, (k, n)))
         w.free()
-        for m in (1, 8, 32):
+        for m in ms:
             a = be.alloc_uninit((m, k), fa.capi.BF16)
             fa.check(lib.fa_fill_normal(be._ctx, a._h, 0, m * k, 5, 0.0, 1.0))
             out = be.alloc_uninit((m, n), fa.capi.BF16)
@@ -563,7 +563,10 @@ def main():
                     help="tuning: wavefronts per compute unit of the decode attention (0 = built-in)")
     ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
                     help="tuning: raw fa_set_tuning key/value pairs (experiments)")
-    ap.add_argument("--only", choices=("attention", "copy", "linears", "prefill", "prefill-attention", "mfma", "prompt"), default=None,
+    ap.add_argument("--rows", type=int, default=0,
+                    help="with --only decode-linears: one row count of the sweep instead of 1, 8 and 32")
+    ap.add_argument("--only", choices=("attention", "copy", "linears", "decode-linears", "prefill", "prefill-attention", "mfma",
+                                       "prompt"), default=None,
                     help="profiling aid: run only the dominant kernel at the workload's shape, or a plain "
                          "copy kernel of known size (counter calibration), a few launches, no JSON line")
     a = ap.parse_args()
@@ -606,6 +609,12 @@ def main():
             for r in bench_matrix_rate(fa, be):
                 log("%-42s %-20s: %.2f ms, %.0f T op/s (%.1f %% of peak)" %
                     (r["instr"], r["fill"], r["ms"], r["tops"], 100 * r["tops"] / MFMA_PEAK_TOPS))
+            be.close()
+            return
+        if a.only == "decode-linears":
+            for r in bench_linears(fa, be, 20, (a.rows,) if a.rows else (1, 8, 32)):
+                log("w8a16 m=%d %5d->%5d: %.2f us, %.0f GB/s (%.1f %% of peak)" %
+                    (r["m"], r["k"], r["n"], r["us"], r["gbs"], 100 * r["frac"]))
             be.close()
             return
         if a.only == "linears":

@@ -69,52 +69,59 @@ __global__ void __launch_bounds__(NWAVES * 64)
 #pragma unroll
         for (int j = 0; j < NTW; ++j) acc[i][j] = v4i{0, 0, 0, 0};
 
-    const int8_t *a_base = xq_tiled + (uint64_t)lane * 16;
     const int8_t *b_base = w_tiles + (uint64_t)lane * 16;
-    // U k-tiles per trip: all their loads are issued before the first multiply
-    constexpr int U = (MT * NTW >= 4) ? 2 : 4;
+    // Wavefront w owns the k-tiles w, w + NWAVES, ...: `cnt` of them.  They are streamed through a ring of
+    // D register slots (one slot = the weight tiles and the activation tiles of one k-tile): the loads of a
+    // whole group of D k-tiles are in flight while the group before it is multiplied, and every multiply
+    // is followed at once by the load that refills its slot, so the memory pipe never drains between trips.
+    // (A weight tile comes from HBM and takes several times longer than an activation tile from L2; with
+    // few loads in flight the whole stream runs at in-flight bytes / HBM latency.)  Loads past the end are
+    // clamped to the wavefront's last k-tile instead of predicated, which keeps the number of outstanding
+    // loads the same on every path, so the waits the compiler inserts are exact.
+    constexpr int D = (MT * NTW >= 6) ? 4 : 8;
     const uint32_t cnt = k_tiles > (uint32_t)wave ? (k_tiles - wave + NWAVES - 1) / NWAVES : 0;
-    auto load_b = [&](uint32_t kt, v4i *b) {
+    // lane l holds row l % 16 of a row tile.  The lanes of rows at or past m fetch row 0 of their k-group
+    // instead (bytes that its own lane fetches anyway), so a step of one to four rows pulls a quarter of
+    // each activation tile; what they hold only reaches accumulator rows that are never stored.  (A load
+    // skipped by predicate would make the count of outstanding loads depend on m.)
+    uint32_t a_off[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) a_off[i] = ((uint32_t)i * 16 + (uint32_t)lane % 16 < m ? (uint32_t)lane : (uint32_t)lane & 48u) * 16;
+    v4i a[D][MT], b[D][NTW];
+    auto load_slot = [&](int s, uint32_t it) {
+        const uint32_t kt = wave + (it < cnt ? it : cnt - 1) * NWAVES;
 #pragma unroll
         for (int j = 0; j < NTW; ++j) {
             uint32_t nt = nt0 + j * nt_step;
-            b[j] = nt < n_tiles ? *(const v4i *)(b_base + ((uint64_t)nt * k_tiles + kt) * 1024) : v4i{0, 0, 0, 0};
+            nt = nt < n_tiles ? nt : n_tiles - 1;            // a tile past the edge is loaded clamped, never stored
+            b[s][j] = *(const v4i *)(b_base + ((uint64_t)nt * k_tiles + kt) * 1024);
         }
-    };
-    // lane l holds row l % 16 of a row tile: the rows at or past m are zeros in memory, and the lanes that
-    // would fetch them do not ask (a step of one to four rows then pulls a quarter of each activation tile)
-    const uint32_t a_row = (uint32_t)lane % 16;
-    auto load_a = [&](uint32_t kt, v4i *a) {
 #pragma unroll
-        for (int i = 0; i < MT; ++i)
-            a[i] = (uint32_t)i * 16 + a_row < m ? *(const v4i *)(a_base + ((uint64_t)i * k_tiles + kt) * 1024)
-                                                : v4i{0, 0, 0, 0};
+        for (int i = 0; i < MT; ++i) a[s][i] = *(const v4i *)(xq_tiled + ((uint64_t)i * k_tiles + kt) * 1024 + a_off[i]);
     };
-    auto mma = [&](const v4i *a, const v4i *b) {
+    auto mma_slot = [&](int s) {
 #pragma unroll
         for (int i = 0; i < MT; ++i)
 #pragma unroll
             for (int j = 0; j < NTW; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[i], b[j], acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[s][i], b[s][j], acc[i][j], 0, 0, 0);
     };
-    uint32_t it = 0;
-    for (; it + U <= cnt; it += U) {
-        v4i a[U][MT], b[U][NTW];
+    if (cnt != 0) {
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            uint32_t kt = wave + (it + u) * NWAVES;
-            load_b(kt, b[u]);
-            load_a(kt, a[u]);
+        for (int s = 0; s < D; ++s) load_slot(s, (uint32_t)s);
+        uint32_t it0 = 0;
+        for (; it0 + D < cnt; it0 += D) {                     // a further group exists: refill while multiplying
+#pragma unroll
+            for (int s = 0; s < D; ++s) {
+                mma_slot(s);
+                __builtin_amdgcn_sched_barrier(0);            // keep every refill right behind its consumer
+                load_slot(s, it0 + D + s);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
 #pragma unroll
-        for (int u = 0; u < U; ++u) mma(a[u], b[u]);
-    }
-    for (; it < cnt; ++it) {
-        v4i a[MT], b[NTW];
-        uint32_t kt = wave + it * NWAVES;
-        load_b(kt, b);
-        load_a(kt, a);
-        mma(a, b);
+        for (int s = 0; s < D; ++s)
+            if (it0 + s < cnt) mma_slot(s);
     }
 
 #pragma unroll
