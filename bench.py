@@ -495,6 +495,46 @@ def bench_matrix_rate(fa, be, iters=20000):
     return res
 
 
+def bench_stream_floor(fa, be, sizes, reps=30):
+    """Plain streaming read of `sizes` bytes (fa_probe_stream_read, 512 blocks of 512 threads), each launch on
+    a fresh window of a 4 GiB buffer so that nothing is served from the 256 MB memory-side cache: the best a
+    memory-bound kernel that must fetch that many bytes can do on this part, launch ramp and tail included."""
+    lib = fa.capi.lib
+    total = 4 << 30
+    buf = be.alloc_uninit((total // 4,))
+    fa.check(lib.fa_fill_normal(be._ctx, buf._h, 0, total // 4, 3, 0.0, 1.0))
+    sink = be.alloc_zeroed((1,), fa.capi.I32)
+    res = []
+    for name, nbytes in sizes:
+        nb = nbytes // (16 * 512) * (16 * 512)
+        win = (nb + 4095) // 4096 * 4096
+        nwin = total // win
+
+        def launch(i):
+            fa.check(lib.fa_probe_stream_read(be._ctx, buf._h, (i % nwin) * win, nb, 512, 512, sink._h))
+        for i in range(3):
+            launch(i)
+        be.synchronize_device()
+        t = Timer(fa, be)
+        t.start()
+        for i in range(reps):
+            launch(3 + i)
+        us = t.stop_ms() / reps * 1e3
+        res.append(dict(what=name, bytes=nb, us=us, gbs=nb / us / 1e3, frac=nb / us / 1e3 / HBM_PEAK_GBS))
+    buf.free()
+    sink.free()
+    return res
+
+
+def floor_sizes(cfg, att_bytes):
+    D, F, V = cfg["d_model"], cfg["d_ffn"], cfg["vocab"]
+    EQ, EKV = cfg["n_heads"] * cfg["head_dim"], cfg["n_kv_heads"] * cfg["head_dim"]
+    return [("o projection weight 4096x4096", EQ * D), ("qkv weight 4096x6144", D * (EQ + 2 * EKV)),
+            ("config-2 weight 4096x12288", 4096 * 12288), ("down weight 14336x4096", F * D),
+            ("config-2 weight 4096x22016", 4096 * 22016), ("gate/up weight 4096x28672", D * 2 * F),
+            ("lm_head weight 4096x32000", D * V), ("decode attention K/V of one layer", att_bytes)]
+
+
 # ---------------------------------------------------------------- CPU baseline
 def cpu_baseline(cfg, batch, ctxs, threads):
     """The CPU oracle (a restatement of the reference's backend-cpu algorithms; the Rust crate cannot be
@@ -566,7 +606,7 @@ def main():
     ap.add_argument("--rows", type=int, default=0,
                     help="with --only decode-linears: one row count of the sweep instead of 1, 8 and 32")
     ap.add_argument("--only", choices=("attention", "copy", "linears", "decode-linears", "prefill", "prefill-attention", "mfma",
-                                       "prompt"), default=None,
+                                       "prompt", "stream-floor"), default=None,
                     help="profiling aid: run only the dominant kernel at the workload's shape, or a plain "
                          "copy kernel of known size (counter calibration), a few launches, no JSON line")
     a = ap.parse_args()
@@ -609,6 +649,12 @@ def main():
             for r in bench_matrix_rate(fa, be):
                 log("%-42s %-20s: %.2f ms, %.0f T op/s (%.1f %% of peak)" %
                     (r["instr"], r["fill"], r["ms"], r["tops"], 100 * r["tops"] / MFMA_PEAK_TOPS))
+            be.close()
+            return
+        if a.only == "stream-floor":
+            for r in bench_stream_floor(fa, be, floor_sizes(cfg, attention_bytes(sum(mid_ctx), mid_ctx, cfg["n_heads"], cfg["n_kv_heads"]))):
+                log("plain read of %-36s %10d bytes: %7.2f us, %5.0f GB/s (%.1f %% of peak)" %
+                    (r["what"], r["bytes"], r["us"], r["gbs"], 100 * r["frac"]))
             be.close()
             return
         if a.only == "decode-linears":
@@ -718,6 +764,8 @@ def main():
         extras["decode_linears"] = bench_linears(fa, be, 100)
         extras["sampling_32x32000"] = bench_sampling(fa, be)
         extras["prefill_gemm"] = bench_prefill(fa, be, 20)
+        # what a plain streaming read of the same bytes reaches: the yardstick for the bandwidth-bound kernels
+        extras["stream_read_floor"] = bench_stream_floor(fa, be, floor_sizes(cfg, att_bytes))
     out = {
         "metric": METRIC, "value": batch / sec_per_step, "unit": "tokens/s", "n_gpus": 1, "steps": a.steps,
         "warmup": a.warmup, "ms_per_step": sec_per_step * 1e3, "higher_is_better": True, "scaling": "weak",

@@ -590,6 +590,23 @@ fa_status fa_probe_matrix_rate(fa_context *ctx, int32_t kind, const fa_buffer *o
     return after_launch(ctx, "matrix_rate_probe");
 }
 
+fa_status fa_probe_stream_read(fa_context *ctx, const fa_buffer *src, uint64_t offset_bytes, uint64_t bytes, int32_t blocks,
+                               int32_t threads, fa_buffer *sink) {
+    if (fa_status s = check_ctx(ctx)) return s;
+    if (fa_status s = check_buf(ctx, src, "probe_stream_read: src")) return s;
+    if (fa_status s = check_buf(ctx, sink, "probe_stream_read: sink")) return s;
+    if (blocks <= 0 || blocks > 65536 || (threads != 256 && threads != 512))
+        return fail(FA_ERR_INVALID_ARGUMENT, "probe_stream_read: blocks in 1..=65536, threads 256 or 512");
+    const uint64_t have = src->numel * dtype_size(src->dtype);
+    uint64_t end;
+    if (offset_bytes % 16 != 0 || __builtin_add_overflow(offset_bytes, bytes, &end) || end > have)
+        return fail(FA_ERR_INVALID_ARGUMENT, "probe_stream_read: range exceeds the buffer or is not 16-byte aligned");
+    if (sink->numel * dtype_size(sink->dtype) < 4) return fail(FA_ERR_SHAPE_MISMATCH, "probe_stream_read: sink too small");
+    if (bytes < 16ull * (uint64_t)blocks) return FA_OK;
+    k::stream_read_probe((const char *)src->ptr + offset_bytes, bytes, blocks, threads, (int *)sink->ptr, ctx->stream);
+    return after_launch(ctx, "stream_read_probe");
+}
+
 fa_status fa_convert(fa_context *ctx, const fa_buffer *src, uint64_t numel, fa_buffer *dst) {
     if (fa_status s = check_ctx(ctx)) return s;
     if (fa_status s = check_buf(ctx, src, "convert: src")) return s;

@@ -55,7 +55,31 @@ __global__ void __launch_bounds__(256) matrix_rate_kernel(const v4i *__restrict_
     if (s == 0x12345678) sink[0] = s;                 // keeps the loop alive; practically never taken
 }
 
+// Plain streaming read: every block reads its own contiguous share of [src, src + bytes) with 16-byte loads,
+// eight per thread in flight.  What a memory-bound kernel of this size can reach on this part at best
+// (launch ramp and tail included): the yardstick for the decode-shape linears and the decode attention.
+__global__ void __launch_bounds__(512) stream_read_kernel(const v4u *__restrict__ src, uint64_t vecs_per_block, int *sink) {
+    constexpr int U = 8;
+    const v4u *base = src + (uint64_t)blockIdx.x * vecs_per_block;
+    v4u acc = v4u{0, 0, 0, 0};
+    for (uint64_t i = threadIdx.x; i < vecs_per_block; i += (uint64_t)blockDim.x * U) {
+        v4u t[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint64_t idx = i + (uint64_t)u * blockDim.x;
+            t[u] = idx < vecs_per_block ? base[idx] : v4u{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) acc ^= t[u];
+    }
+    if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x12345678u) sink[0] = 1;   // keeps the loads alive
+}
+
 }  // namespace
+
+void stream_read_probe(const void *src, uint64_t bytes, int blocks, int threads, int *sink, hipStream_t s) {
+    stream_read_kernel<<<blocks, threads, 0, s>>>((const v4u *)src, bytes / 16 / (uint64_t)blocks, sink);
+}
 
 double matrix_rate_probe(int kind, const void *operands, uint32_t iters, int num_cus, int *sink, hipStream_t s) {
     const int blocks = 2 * num_cus;                   // two wavefronts per SIMD

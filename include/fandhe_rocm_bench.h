@@ -31,6 +31,13 @@ fa_status fa_fill_normal(fa_context *ctx, fa_buffer *buf, uint64_t offset, uint6
 fa_status fa_probe_matrix_rate(fa_context *ctx, int32_t kind, const fa_buffer *operands,
                                uint32_t iters, fa_buffer *sink, double *ops);
 
+/* Queues a plain streaming read of `bytes` starting `offset_bytes` into `src`: `blocks` blocks of `threads`
+ * (256 or 512) threads, each reading its own contiguous share with 16-byte loads, eight per thread in
+ * flight, nothing written.  The time of this launch is the floor for a memory-bound kernel that must
+ * fetch that many bytes; time it with an fa_timer. */
+fa_status fa_probe_stream_read(fa_context *ctx, const fa_buffer *src, uint64_t offset_bytes, uint64_t bytes,
+                               int32_t blocks, int32_t threads, fa_buffer *sink);
+
 /* Launch-shape knobs for experiments; value 0 restores the built-in choice.
  * The knobs are plain process-wide integers read by every context's launches:
  * set them while no other thread is submitting work.
