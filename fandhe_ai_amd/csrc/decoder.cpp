@@ -113,8 +113,12 @@ void enqueue_pick(fa_decoder *d, hipStream_t s) {
                        d->cfg.vocab, d->strategy == FA_SAMPLE_TOP_K, d->temperature, d->top_k, s);
 }
 
-// The kernels of one step, enqueued on the context's stream.
-fa_status enqueue_step(fa_context *ctx, fa_decoder *d) {
+// The kernels of one step, enqueued on the context's stream.  stop_after (test aid, -1 in normal use) ends the
+// step after the given stage: stage 0 is the per-step bookkeeping and the embedding gather, stage
+// 1 + 8 * layer + i (i = 0 .. 7) is the i-th launch of that layer (norm + quantizer, qkv projection with RoPE
+// and cache append, attention with merge + quantizer, o projection, norm + quantizer, gate / up with SwiGLU,
+// quantizer, down projection), and the three stages after the last layer are the final norm, the head and the pick.
+fa_status enqueue_step(fa_context *ctx, fa_decoder *d, int stop_after = -1) {
     const fa_decoder_config &c = d->cfg;
     const uint32_t B = d->batch;
     const uint64_t D = c.d_model, H = c.n_heads, HKV = c.n_kv_heads, DH = c.head_dim, F = c.d_ffn, V = c.vocab;
@@ -128,6 +132,9 @@ fa_status enqueue_step(fa_context *ctx, fa_decoder *d) {
                       (uint32_t *)d->slots->ptr, (float *)d->cos_sin->ptr, B, c.block_size, c.max_blocks_per_seq,
                       c.num_blocks, c.head_dim, c.rope_theta, s);
     k::gather_rows_f32((const float *)d->embed->ptr, V, D, (const int32_t *)d->tokens->ptr, (float *)d->h->ptr, B, s);
+    int stage = 0;
+    auto stop_here = [&]() { return stop_after >= 0 && stage++ == stop_after; };
+    if (stop_here()) return after_launch(ctx, "decoder step (partial)");
 
     k::PagedShape ps;
     ps.num_blocks = c.num_blocks;
@@ -161,6 +168,7 @@ fa_status enqueue_step(fa_context *ctx, fa_decoder *d) {
         const fa_decoder::Layer &L = d->layers[li];
         k::rmsnorm_quantize_i8((const float *)d->h->ptr, (const float *)L.attn_norm->ptr, c.rms_eps, nullptr,
                                (int8_t *)d->xq->ptr, (float *)d->sx->ptr, B, m_pad, D, s);
+        if (stop_here()) break;
         {
             k::QkvRopeTargets t{(const float *)d->cos_sin->ptr, (const uint32_t *)d->slots->ptr, (uint16_t *)d->q_bf->ptr,
                                 (uint16_t *)L.k_pool->ptr, (uint16_t *)L.v_pool->ptr, c.n_heads, c.n_kv_heads,
@@ -169,6 +177,7 @@ fa_status enqueue_step(fa_context *ctx, fa_decoder *d) {
                                            (const float *)d->sx->ptr, (const float *)L.wqkv->scales->ptr, B,
                                            L.wqkv->n_pad, L.wqkv->k_pad, t, s);
         }
+        if (stop_here()) break;
         if (c.n_heads <= 32) {
             k::paged_attention_decode_bf16((const uint16_t *)d->q_bf->ptr, (const uint16_t *)L.k_pool->ptr,
                                            (const uint16_t *)L.v_pool->ptr, (const uint32_t *)d->tables->ptr,
@@ -183,19 +192,28 @@ fa_status enqueue_step(fa_context *ctx, fa_decoder *d) {
             k::quantize_rows_from_pmax(d->attn->ptr, true, (const float *)d->pmax->ptr, c.n_heads, (int8_t *)d->xq->ptr,
                                        (float *)d->sx->ptr, B, m_pad, EQ, s);
         }
+        if (stop_here()) break;
         linear(L.wo, d->h->ptr, (const float *)d->h->ptr);
+        if (stop_here()) break;
         k::rmsnorm_quantize_i8((const float *)d->h->ptr, (const float *)L.ffn_norm->ptr, c.rms_eps, nullptr,
                                (int8_t *)d->xq->ptr, (float *)d->sx->ptr, B, m_pad, D, s);
+        if (stop_here()) break;
         k::linear_w8a8_swiglu_skinny((const int8_t *)d->xq->ptr, (const int8_t *)L.wgu->codes->ptr,
                                      (const float *)d->sx->ptr, (const float *)L.wgu->scales->ptr, B, L.wgu->n,
                                      L.wgu->n_pad, L.wgu->k_pad, (float *)d->act->ptr, (float *)d->pmax->ptr, 4, cus, s);
+        if (stop_here()) break;
         k::quantize_rows_from_pmax(d->act->ptr, false, (const float *)d->pmax->ptr, (uint32_t)(F / 16),
                                    (int8_t *)d->xq->ptr, (float *)d->sx->ptr, B, m_pad, F, s);
+        if (stop_here()) break;
         linear(L.wdown, d->h->ptr, (const float *)d->h->ptr);
+        if (stop_here()) break;
     }
+    if (stop_after >= 0 && stage > stop_after) return after_launch(ctx, "decoder step (partial)");
     k::rmsnorm_quantize_i8((const float *)d->h->ptr, (const float *)d->final_norm->ptr, c.rms_eps, nullptr,
                            (int8_t *)d->xq->ptr, (float *)d->sx->ptr, B, m_pad, D, s);
+    if (stop_here()) return after_launch(ctx, "decoder step (partial)");
     linear(d->lm_head, d->logits->ptr, nullptr);
+    if (stop_here()) return after_launch(ctx, "decoder step (partial)");
     enqueue_pick(d, s);
     return after_launch(ctx, "decoder step");
 }
@@ -758,6 +776,35 @@ fa_status fa_decoder_rewind(fa_context *ctx, fa_decoder *d, const uint32_t *seq_
                                                      std::to_string(seq_lens[b]) + " > " + std::to_string(d->host_lens[b]) + ")");
     if (fa_status s = fa_upload_into(ctx, seq_lens, d->batch, d->seq_lens, 0)) return s;
     std::copy(seq_lens, seq_lens + d->batch, d->host_lens.begin());
+    return FA_OK;
+}
+
+fa_status fa_decoder_debug_step_until(fa_context *ctx, fa_decoder *d, int32_t stop_after) {
+    if (fa_status s = check_ctx(ctx)) return s;
+    if (fa_status s = check_dec(d)) return s;
+    if (d->ctx != ctx) return fail(FA_ERR_DEVICE_MISMATCH, "decoder_debug_step_until: decoder belongs to another context");
+    if (ctx->capturing) return fail(FA_ERR_CAPTURE_IN_PROGRESS, "decoder_debug_step_until during graph capture");
+    if (d->batch == 0 || stop_after < 0) return fail(FA_ERR_INVALID_ARGUMENT, "decoder_debug_step_until: no sequences or negative stage");
+    if (!d->embed || !d->final_norm || !d->lm_head) return fail(FA_ERR_INVALID_ARGUMENT, "decoder_debug_step_until: head weights missing");
+    for (auto &l : d->layers)
+        if (!l.wqkv) return fail(FA_ERR_INVALID_ARGUMENT, "decoder_debug_step_until: layer weights missing");
+    k::PagedShape ps{};
+    ps.batch = d->batch;
+    ps.num_heads = d->cfg.n_heads;
+    ps.num_kv_heads = d->cfg.n_kv_heads;
+    ps.max_blocks_per_seq = d->cfg.max_blocks_per_seq;
+    if (fa_status s = ensure_workspace(ctx, k::paged_decode_workspace_bytes(ps, (uint32_t)g_decode_waves))) return s;
+    for (auto &len : d->host_lens) len += 1;            // the bookkeeping stage advances the lengths on the device
+    return enqueue_step(ctx, d, stop_after);
+}
+
+fa_status fa_decoder_debug_buffer(fa_decoder *d, int32_t which, fa_buffer **out) {
+    if (fa_status s = check_dec(d)) return s;
+    if (!out) return fail(FA_ERR_INVALID_ARGUMENT, "decoder_debug_buffer: null output");
+    fa_buffer *table[] = {d->h, d->xq, d->sx, d->q_bf, d->act, d->pmax, d->logits, d->cos_sin, d->slots, d->pos};
+    if (which < 0 || which >= (int32_t)(sizeof(table) / sizeof(table[0])))
+        return fail(FA_ERR_INVALID_ARGUMENT, "decoder_debug_buffer: unknown buffer");
+    *out = table[which];
     return FA_OK;
 }
 

@@ -77,6 +77,21 @@ fa_status fa_gemm_plan_query(const fa_context *ctx, uint64_t m, const fa_qweight
  * `capacity` device addresses and the total count. */
 fa_status fa_graph_owned_blocks(const fa_graph *graph, void **ptrs, uint64_t capacity, uint64_t *count);
 
+/* Test aids for the decode step: run the step's launches, eagerly, up to and including stage `stop_after` and
+ * stop, so that a test can read what each fused stage left behind and hold it against the matching operator of
+ * the oracle.  Stage 0: per-step bookkeeping (positions, slots, cos / sin, lengths + 1) and the embedding
+ * gather; stage 1 + 8 * layer + i, i = 0 .. 7: norm + quantizer, qkv projection with RoPE and cache append,
+ * attention with merge + quantizer, o projection (+ residual), norm + quantizer, gate / up with SwiGLU,
+ * quantizer, down projection (+ residual); then the final norm + quantizer, the head, the pick.  The sequence
+ * lengths advance as in a step: reinstall the sequences before the next call.
+ * fa_decoder_debug_buffer hands out the decoder's own resident buffers (not copies; do not free):
+ * 0 residual stream h f32 [batch, d_model]; 1 activation codes int8 in tile order (tiles [row tile][k tile] of
+ * 16 rows x 64 k, byte ((g * 16 + r) * 16 + j) = row r, k 16 g + j); 2 row scales f32; 3 q bf16 [batch, heads *
+ * head_dim]; 4 SwiGLU activation f32 [batch, d_ffn]; 5 partial row maxima f32; 6 logits f32; 7 cos / sin f32
+ * [batch, head_dim]; 8 cache slots u32 [batch]; 9 positions i32 [batch]. */
+fa_status fa_decoder_debug_step_until(fa_context *ctx, fa_decoder *dec, int32_t stop_after);
+fa_status fa_decoder_debug_buffer(fa_decoder *dec, int32_t which, fa_buffer **out);
+
 /* A pair of HIP events recorded on the context's stream (the stream the
  * kernels run on); used by the benchmark to time launches. */
 typedef struct fa_timer fa_timer;
