@@ -510,16 +510,13 @@ def bench_stream_floor(fa, be, sizes, reps=30):
         win = (nb + 4095) // 4096 * 4096
         nwin = total // win
 
-        def launch(i):
-            fa.check(lib.fa_probe_stream_read(be._ctx, buf._h, (i % nwin) * win, nb, 512, 512, sink._h))
-        for i in range(3):
-            launch(i)
-        be.synchronize_device()
-        t = Timer(fa, be)
-        t.start()
-        for i in range(reps):
-            launch(3 + i)
-        us = t.stop_ms() / reps * 1e3
+        counter = [0]
+
+        def launch():
+            # every launch of the replayed graph reads another window
+            fa.check(lib.fa_probe_stream_read(be._ctx, buf._h, (counter[0] % nwin) * win, nb, 512, 512, sink._h))
+            counter[0] += 1
+        us = time_launches(fa, be, launch, reps, warmup=3) * 1e6
         res.append(dict(what=name, bytes=nb, us=us, gbs=nb / us / 1e3, frac=nb / us / 1e3 / HBM_PEAK_GBS))
     buf.free()
     sink.free()
@@ -565,12 +562,13 @@ def cpu_baseline(cfg, batch, ctxs, threads):
                      k_pool=bf16_noise((num_blocks, 16, EKV)), v_pool=bf16_noise((num_blocks, 16, EKV)))]
     tokens = rng.integers(0, V, size=batch).astype(np.int32)
     oracle_step(m, np.asarray(ctxs, dtype=np.uint32).copy(), tokens, threads=threads)   # warm-up
-    reps, t_one = 2, 0.0
-    for _ in range(reps):
+    times = []
+    for _ in range(3):                                    # one iteration takes seconds: warm-up 1, 3 timed, median
         lens = np.asarray(ctxs, dtype=np.uint32).copy()
         t0 = time.perf_counter()
         oracle_step(m, lens, tokens, threads=threads)
-        t_one += (time.perf_counter() - t0) / reps
+        times.append(time.perf_counter() - t0)
+    t_one = float(np.median(times))
     # separate the lm_head share: time a zero-layer-equivalent by timing the head alone
     x = rng.standard_normal((batch, D), dtype=np.float32)
     o.set_threads(threads)
@@ -582,8 +580,112 @@ def cpu_baseline(cfg, batch, ctxs, threads):
     t_full = t_layer * cfg["n_layers"] + t_head
     return dict(value=batch / t_full, unit="tokens/s", cores=threads, kind="port",
                 sample="CPU oracle (C++ restatement of backend-cpu, not the Rust binary): 1 of %d layers + lm_head at "
-                       "batch %d, same contexts, %.2f s per layer measured, scaled to the full depth" %
-                       (cfg["n_layers"], batch, t_layer))
+                       "batch %d, same contexts, warm-up 1 + median of 3 timed passes, %.2f s per layer measured, scaled "
+                       "to the full depth" % (cfg["n_layers"], batch, t_layer))
+
+
+def _median_time(fn, min_iters, budget_s):
+    """Median seconds of fn after one warm-up: at least min_iters timed calls, more while the budget lasts (up to 20)."""
+    fn()
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < min_iters or (len(times) < 20 and time.perf_counter() - t_start < budget_s):
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    return float(np.median(times)), len(times)
+
+
+def cpu_operator_baselines(fa, be, threads):
+    """The CPU oracle beside the operator figures of `extras`, on the operands the GPU itself used (the codes and
+    scales are read back from the device), with the GPU result judged against the CPU result in the same run.
+    Each entry: CPU seconds (median, iterations stated), the GPU / CPU parity line, and what was sampled where one CPU
+    pass over the full operator would take minutes."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle_lib as o
+    lib = fa.capi.lib
+    o.set_threads(threads)
+    res = {"cores": threads, "kind": "port",
+           "note": "C++ restatement of backend-cpu (not the Rust binary), OpenMP over independent rows / columns"}
+    # decode-shape W8A16 sweep (config 2)
+    gemv = []
+    for k, n in ((4096, 12288), (4096, 4096), (4096, 22016), (11008, 4096)):
+        w = be.alloc_uninit((k, n))
+        fa.check(lib.fa_fill_normal(be._ctx, w._h, 0, k * n, k + n, 0.0, 0.02))
+        qw = be.quantize_weight(fa.DeviceBufferView(w, 0, (k, n)))
+        w.free()
+        codes, scales = qw.export()
+        for m in (1, 8, 32):
+            a = be.alloc_uninit((m, k), fa.capi.BF16)
+            fa.check(lib.fa_fill_normal(be._ctx, a._h, 0, m * k, 5, 0.0, 1.0))
+            out = be.alloc_uninit((m, n), fa.capi.F32)
+            fa.check(lib.fa_linear_w8a16(be._ctx, a._h, m, qw._h, out._h))
+            got, a_host = be.download(out), be.download(a)
+            want = o.linear_w8a16(a_host, codes, scales)
+            sec, iters = _median_time(lambda: o.linear_w8a16(a_host, codes, scales), 5, 0.5)
+            r = o.compare(got, want)
+            gemv.append(dict(op="w8a16", m=m, k=k, n=n, cpu_us=sec * 1e6, iters=iters, parity_fail=int(r.fail_count),
+                             parity=r.line("W8A16_PARITY", "%dx%dx%d" % (m, n, k))))
+            a.free(), out.free()
+        qw.free()
+    res["decode_linears"] = gemv
+    # paged attention, config 3
+    rng = np.random.default_rng(3)
+    c3 = np.random.default_rng(0).integers(128, 4097, size=64).tolist()
+    tables, max_blocks, num_blocks = make_tables(rng, c3, 0, 16, 40000)
+    kp = be.alloc_uninit((num_blocks, 16, 1024), fa.capi.BF16)
+    vp = be.alloc_uninit((num_blocks, 16, 1024), fa.capi.BF16)
+    q = be.alloc_uninit((64, 1, 4096), fa.capi.BF16)
+    for b, sd in ((kp, 31), (vp, 32), (q, 33)):
+        fa.check(lib.fa_fill_normal(be._ctx, b._h, 0, b.numel(), sd, 0.0, 1.0))
+    lens = np.asarray(c3, dtype=np.uint32)
+    layout = fa.PagedKvLayout.new(num_blocks, 16, 1024)
+    args = fa.PagedAttentionArgs(layout, 64, 1, 32, max_blocks, fa.default_scale(128), 8)
+    got = be.download(be.paged_attention_forward(q, kp, vp, tables, lens, args, out_dtype=fa.capi.F32))
+    kph, vph, qh = be.download(kp), be.download(vp), be.download(q)
+    oargs = o.paged_args(num_blocks, 16, 1024, 64, 1, 32, max_blocks, args.scale, 8)
+    rc, want = o.paged_attention_bf16(qh, kph, vph, tables, lens, oargs)
+    sec, iters = _median_time(lambda: o.paged_attention_bf16(qh, kph, vph, tables, lens, oargs), 3, 3.0)
+    r = o.compare(got, want)
+    res["paged_attention_bs64"] = dict(cpu_us=sec * 1e6, iters=iters, parity_fail=int(r.fail_count),
+                                       parity=r.line("PAGED_DECODE_PARITY", "bs64"))
+    for b in (kp, vp, q):
+        b.free()
+    # prefill GEMMs, config 4: the CPU takes a sample of the rows (all columns, full k) and is scaled
+    m, k, n, rows = 2048, 4096, 14336, 32
+    w = be.alloc_uninit((k, n))
+    x = be.alloc_uninit((m, k))
+    fa.check(lib.fa_fill_normal(be._ctx, w._h, 0, k * n, 11, 0.0, 1.0))
+    fa.check(lib.fa_fill_normal(be._ctx, x._h, 0, m * k, 12, 0.0, 1.0))
+    sel = np.linspace(0, m - 1, rows).astype(np.int64)
+    gemm = []
+    qw = be.quantize_weight(fa.DeviceBufferView(w, 0, (k, n)))
+    xq, sx = be.quantize_rows_i8(x)
+    out, acc = be.gemm_w8a8(xq, sx, qw, fa.capi.F32, want_acc=True)
+    codes, scales = qw.export()
+    a_rows = np.ascontiguousarray(be.download(xq)[sel])
+    sec, iters = _median_time(lambda: o.gemm_i8_i32(a_rows, codes), 3, 2.0)
+    want_acc = o.gemm_i8_i32(a_rows, codes)
+    mism = int((be.download(acc)[sel] != want_acc).sum())
+    gemm.append(dict(op="gemm_w8a8", m=m, k=k, n=n, cpu_ms_full=sec * m / rows * 1e3, sampled_rows=rows, iters=iters,
+                     acc_bit_mismatch=mism))
+    for b in (qw, xq, sx, out, acc):
+        b.free()
+    qw = be.quantize_weight(fa.DeviceBufferView(w, 0, (k, n)), fa.capi.QW_E4M3_TENSOR)
+    xq, xs = be.quantize_tensor_e4m3(x)
+    got = be.download(be.gemm_e4m3(xq, xs, qw, fa.capi.F32))[sel]
+    codes, wscale = qw.export()
+    a_rows = np.ascontiguousarray(be.download(xq)[sel])
+    sa, sw = np.float32(be.download(xs)[0]), np.float32(wscale[0])
+    sec, iters = _median_time(lambda: o.gemm_e4m3(a_rows, codes, sa, sw), 3, 2.0)
+    r = o.compare(got, o.gemm_e4m3(a_rows, codes, sa, sw))
+    gemm.append(dict(op="gemm_e4m3", m=m, k=k, n=n, cpu_ms_full=sec * m / rows * 1e3, sampled_rows=rows, iters=iters,
+                     parity_fail=int(r.fail_count), parity=r.line("FP8_PARITY", "%dx%dx%d" % (m, n, k))))
+    for b in (qw, xq, xs, w, x):
+        b.free()
+    res["prefill_gemm"] = gemm
+    o.set_threads(1)
+    return res
 
 
 # ------------------------------------------------------------------------ main
@@ -778,7 +880,10 @@ def main():
         "roofline": roofline, "extras": extras,
     }
     if not a.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(cfg, batch, ctxs, min(16, os.cpu_count() or 1))
+        threads = min(16, os.cpu_count() or 1)
+        out["cpu_baseline"] = cpu_baseline(cfg, batch, ctxs, threads)
+        if not a.no_extras:
+            extras["cpu_operator_baselines"] = cpu_operator_baselines(fa, be, threads)
     else:
         out["cpu_baseline"] = None
     be.close()
