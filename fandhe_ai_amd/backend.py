@@ -177,14 +177,14 @@ class DeviceBufferView:
 
 
 class QuantizedWeight:
-    """int8 per-channel or e4m3 per-tensor weight in the kernels' tile order."""
+    """int8 per-channel, e4m3 per-tensor or e4m3 per-channel weight in the kernels' tile order."""
 
     def __init__(self, ops, handle, k, n, kind):
         self._ops, self._h, self.k, self.n, self.kind = ops, handle, k, n, kind
 
     def export(self):
         codes = np.empty((self.k, self.n), dtype=np.int8 if self.kind == capi.QW_INT8_CHANNEL else np.uint8)
-        scales = np.empty(self.n if self.kind == capi.QW_INT8_CHANNEL else 1, dtype=np.float32)
+        scales = np.empty(1 if self.kind == capi.QW_E4M3_TENSOR else self.n, dtype=np.float32)
         check(lib.fa_qweight_export(self._ops._ctx, self._h, codes.ctypes.data,
                                     scales.ctypes.data_as(capi.f32p)))
         return codes, scales
@@ -416,6 +416,27 @@ class RocmBackendOps:
         m = aq.shape[0]
         out = self.alloc_uninit((m, qw.n), out_dtype)
         check(lib.fa_gemm_e4m3(self._ctx, aq._h, a_scale._h, m, qw._h, out._h))
+        return out
+
+    def quantize_rows_e4m3(self, x):
+        m, k = x.shape
+        xq, sx = self.alloc_uninit((m, k), capi.E4M3), self.alloc_uninit((m,), capi.F32)
+        check(lib.fa_quantize_rows_e4m3(self._ctx, x._h, m, k, xq._h, sx._h))
+        return xq, sx
+
+    def linear_e4m3(self, x, qw, bias=None, out_dtype=capi.F32):
+        """Per-token x per-channel fp8 linear: x f32 / bf16 [m, k], qw of kind QW_E4M3_CHANNEL."""
+        m = x.shape[0]
+        out = self.alloc_uninit((m, qw.n), out_dtype)
+        check(lib.fa_linear_e4m3(self._ctx, x._h, m, qw._h, bias.buffer._h if bias is not None else None,
+                                 bias.offset if bias is not None else 0, out._h))
+        return out
+
+    def gemm_e4m3_rows(self, aq, sx, qw, bias=None, out_dtype=capi.F32):
+        m = aq.shape[0]
+        out = self.alloc_uninit((m, qw.n), out_dtype)
+        check(lib.fa_gemm_e4m3_rows(self._ctx, aq._h, sx._h, m, qw._h, bias.buffer._h if bias is not None else None,
+                                    bias.offset if bias is not None else 0, out._h))
         return out
 
     # -- norms / elementwise (backend_ops.rs:5113, 2276-2390, 3375) -------------

@@ -23,7 +23,7 @@ OK, INVALID_ARGUMENT, SHAPE_MISMATCH, DEVICE_MISMATCH, ALLOCATION_FAILED, KERNEL
     DEVICE_UNAVAILABLE, TRANSFER_FAILED, UNSUPPORTED, CONTEXT_POISONED, CAPTURE_IN_PROGRESS, STORE_POISONED = range(12)
 
 F32, BF16, I8, E4M3, I32, U32 = range(6)
-QW_INT8_CHANNEL, QW_E4M3_TENSOR = 0, 1
+QW_INT8_CHANNEL, QW_E4M3_TENSOR, QW_E4M3_CHANNEL = 0, 1, 2
 ACT_NONE, ACT_RELU = 0, 1
 
 ctx_p = C.c_void_p
@@ -119,6 +119,9 @@ SIGNATURES = {
     "fa_linear_w8a16": (C.c_int32, [ctx_p, buf_p, u64, qw_p, buf_p]),
     "fa_quantize_tensor_e4m3": (C.c_int32, [ctx_p, buf_p, u64, buf_p, buf_p]),
     "fa_gemm_e4m3": (C.c_int32, [ctx_p, buf_p, buf_p, u64, qw_p, buf_p]),
+    "fa_quantize_rows_e4m3": (C.c_int32, [ctx_p, buf_p, u64, u64, buf_p, buf_p]),
+    "fa_linear_e4m3": (C.c_int32, [ctx_p, buf_p, u64, qw_p, buf_p, u64, buf_p]),
+    "fa_gemm_e4m3_rows": (C.c_int32, [ctx_p, buf_p, buf_p, u64, qw_p, buf_p, u64, buf_p]),
     "fa_gemm_w8a8": (C.c_int32, [ctx_p, buf_p, buf_p, u64, qw_p, buf_p, buf_p]),
     "fa_rmsnorm": (C.c_int32, [ctx_p, buf_p, buf_p, C.c_float, u64, u64, buf_p]),
     "fa_rope": (C.c_int32, [ctx_p, buf_p, buf_p, u64, u64, u64, C.c_double, buf_p]),

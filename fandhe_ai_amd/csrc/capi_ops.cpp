@@ -141,7 +141,7 @@ fa_status fa_linear_forward_device(fa_context *ctx, const fa_buffer *a, uint64_t
 
 // ------------------------------------------------------- quantized weights
 static fa_status qweight_alloc(fa_context *ctx, uint64_t kdim, uint64_t n, fa_qweight_kind kind, fa_qweight **out) {
-    if (kind != FA_QW_INT8_CHANNEL && kind != FA_QW_E4M3_TENSOR)
+    if (kind != FA_QW_INT8_CHANNEL && kind != FA_QW_E4M3_TENSOR && kind != FA_QW_E4M3_CHANNEL)
         return fail(FA_ERR_INVALID_ARGUMENT, "qweight: unknown kind");
     if (kdim == 0 || n == 0) return fail(FA_ERR_INVALID_ARGUMENT, "qweight: k and n must be positive");
     if (kdim > (1ull << 31) || n > (1ull << 31)) return fail(FA_ERR_INVALID_ARGUMENT, "qweight: dimension too large");
@@ -158,7 +158,7 @@ static fa_status qweight_alloc(fa_context *ctx, uint64_t kdim, uint64_t n, fa_qw
     qw->codes = nullptr;
     qw->scales = nullptr;
     fa_status s = make_buffer(ctx, kind == FA_QW_INT8_CHANNEL ? FA_I8 : FA_E4M3, qw->k_pad * qw->n_pad, false, &qw->codes);
-    if (s == FA_OK) s = make_buffer(ctx, FA_F32, kind == FA_QW_INT8_CHANNEL ? qw->n_pad : 1, true, &qw->scales);
+    if (s == FA_OK) s = make_buffer(ctx, FA_F32, kind == FA_QW_E4M3_TENSOR ? 1 : qw->n_pad, true, &qw->scales);
     if (s != FA_OK) {
         if (qw->codes) fa_buffer_free(ctx, qw->codes);
         delete qw;
@@ -183,6 +183,10 @@ fa_status fa_qweight_from_f32(fa_context *ctx, const fa_buffer *w, uint64_t w_of
         k::weight_col_scales_i8(wp, kdim, n, qw->n_pad, (float *)qw->scales->ptr, ctx->stream);
         k::weight_quantize_pack_i8(wp, (const float *)qw->scales->ptr, kdim, n, qw->k_pad, qw->n_pad,
                                    (int8_t *)qw->codes->ptr, ctx->stream);
+    } else if (kind == FA_QW_E4M3_CHANNEL) {
+        k::weight_col_scales(wp, kdim, n, qw->n_pad, 448.0f, (float *)qw->scales->ptr, ctx->stream);
+        k::weight_quantize_pack_e4m3_cols(wp, (const float *)qw->scales->ptr, kdim, n, qw->k_pad, qw->n_pad,
+                                          (uint8_t *)qw->codes->ptr, ctx->stream);
     } else {
         Scratch am(ctx);
         if (fa_status s = am.get(4)) {
@@ -213,7 +217,7 @@ fa_status fa_qweight_from_codes(fa_context *ctx, const void *codes, const float 
     if (fa_status s = qweight_alloc(ctx, kdim, n, kind, &qw)) return s;
     fa_buffer *tmp = nullptr;
     fa_status s = fa_upload(ctx, FA_I8, codes, kn, &tmp);
-    if (s == FA_OK) s = fa_upload_into(ctx, scales, kind == FA_QW_INT8_CHANNEL ? n : 1, qw->scales, 0);
+    if (s == FA_OK) s = fa_upload_into(ctx, scales, kind == FA_QW_E4M3_TENSOR ? 1 : n, qw->scales, 0);
     if (s == FA_OK) {
         k::weight_pack_codes((const uint8_t *)tmp->ptr, kdim, n, qw->k_pad, qw->n_pad,
                              kind == FA_QW_INT8_CHANNEL ? 64 : 128, (uint8_t *)qw->codes->ptr, ctx->stream);
@@ -243,7 +247,7 @@ fa_status fa_qweight_export(fa_context *ctx, const fa_qweight *qw, void *codes, 
         fa_buffer_free(ctx, tmp);
         if (s != FA_OK) return s;
     }
-    if (scales) return fa_download(ctx, qw->scales, 0, scales, qw->kind == FA_QW_INT8_CHANNEL ? qw->n : 1);
+    if (scales) return fa_download(ctx, qw->scales, 0, scales, qw->kind == FA_QW_E4M3_TENSOR ? 1 : qw->n);
     return FA_OK;
 }
 
@@ -408,6 +412,76 @@ fa_status fa_gemm_e4m3(fa_context *ctx, const fa_buffer *aq, const fa_buffer *a_
                       (const float *)qw->scales->ptr, m, qw->n, qw->n_pad, qw->k_pad, out->ptr, out->dtype == FA_BF16,
                       ctx->props.multiProcessorCount, ctx->stream);
     return after_launch(ctx, "gemm_e4m3_mfma");
+}
+
+fa_status fa_quantize_rows_e4m3(fa_context *ctx, const fa_buffer *x, uint64_t m, uint64_t kdim, fa_buffer *xq,
+                                fa_buffer *sx) {
+    if (fa_status s = check_ctx(ctx)) return s;
+    uint64_t mk;
+    if (!mul3(m, kdim, &mk)) return fail(FA_ERR_SHAPE_MISMATCH, "quantize_rows_e4m3: shape overflows");
+    if (fa_status s = check_buf(ctx, x, "quantize_rows_e4m3: x")) return s;
+    if (x->dtype != FA_F32 && x->dtype != FA_BF16) return fail(FA_ERR_INVALID_ARGUMENT, "quantize_rows_e4m3: x must be f32 or bf16");
+    if (x->numel < mk) return fail(FA_ERR_SHAPE_MISMATCH, "quantize_rows_e4m3: x is smaller than [m, k]");
+    if (fa_status s = check_buf_typed(ctx, xq, FA_E4M3, mk, "quantize_rows_e4m3: xq")) return s;
+    if (fa_status s = check_buf_typed(ctx, sx, FA_F32, m, "quantize_rows_e4m3: sx")) return s;
+    if (mk == 0) return FA_OK;
+    if (m > (1ull << 31) - 1) return fail(FA_ERR_INVALID_ARGUMENT, "quantize_rows_e4m3: too many rows");
+    k::quantize_rows_e4m3(x->ptr, x->dtype == FA_BF16, (uint8_t *)xq->ptr, (float *)sx->ptr, m, kdim, kdim, ctx->stream);
+    return after_launch(ctx, "quantize_rows_e4m3");
+}
+
+// shared tail of the two per-token x per-channel fp8 entry points: aq row-major e4m3 [m, k_pad]
+static fa_status launch_e4m3_rows(fa_context *ctx, const uint8_t *aq, const float *sx, uint64_t m, const fa_qweight *qw,
+                                  const fa_buffer *bias, uint64_t bias_offset, fa_buffer *out) {
+    const float *bp = bias ? (const float *)bias->ptr + bias_offset : nullptr;
+    if (m <= 64)
+        k::linear_e4m3_skinny(aq, (const uint8_t *)qw->codes->ptr, sx, (const float *)qw->scales->ptr, bp, m, qw->n, qw->n_pad,
+                              qw->k_pad, out->ptr, out->dtype == FA_BF16, ctx->stream);
+    else
+        k::gemm_e4m3_rows_mfma(aq, (const uint8_t *)qw->codes->ptr, sx, (const float *)qw->scales->ptr, bp, m, qw->n,
+                               qw->n_pad, qw->k_pad, out->ptr, out->dtype == FA_BF16, ctx->props.multiProcessorCount,
+                               ctx->stream);
+    return after_launch(ctx, "linear_e4m3");
+}
+
+fa_status fa_gemm_e4m3_rows(fa_context *ctx, const fa_buffer *aq, const fa_buffer *sx, uint64_t m, const fa_qweight *qw,
+                            const fa_buffer *bias, uint64_t bias_offset, fa_buffer *out) {
+    if (fa_status s = check_ctx(ctx)) return s;
+    if (fa_status s = check_qw(ctx, qw, FA_QW_E4M3_CHANNEL, "gemm_e4m3_rows: weight")) return s;
+    if (qw->k != qw->k_pad) return fail(FA_ERR_UNSUPPORTED, "gemm_e4m3_rows: k must be a multiple of 128");
+    uint64_t mk, mn;
+    if (!mul3(m, qw->k, &mk) || !mul3(m, qw->n, &mn)) return fail(FA_ERR_SHAPE_MISMATCH, "gemm_e4m3_rows: shape overflows");
+    if (fa_status s = check_buf_typed(ctx, aq, FA_E4M3, mk, "gemm_e4m3_rows: aq")) return s;
+    if (fa_status s = check_buf_typed(ctx, sx, FA_F32, m, "gemm_e4m3_rows: sx")) return s;
+    if (bias)
+        if (fa_status s = check_view(ctx, bias, bias_offset, qw->n, FA_F32, "gemm_e4m3_rows: bias")) return s;
+    if (fa_status s = check_out_f32_or_bf16(ctx, out, mn, "gemm_e4m3_rows: out")) return s;
+    if (mn == 0) return FA_OK;
+    if (m > (1ull << 22)) return fail(FA_ERR_INVALID_ARGUMENT, "gemm_e4m3_rows: m too large for one launch");
+    return launch_e4m3_rows(ctx, (const uint8_t *)aq->ptr, (const float *)sx->ptr, m, qw, bias, bias_offset, out);
+}
+
+fa_status fa_linear_e4m3(fa_context *ctx, const fa_buffer *x, uint64_t m, const fa_qweight *qw, const fa_buffer *bias,
+                         uint64_t bias_offset, fa_buffer *out) {
+    if (fa_status s = check_ctx(ctx)) return s;
+    if (fa_status s = check_qw(ctx, qw, FA_QW_E4M3_CHANNEL, "linear_e4m3: weight")) return s;
+    uint64_t mk, mn, mkp;
+    if (!mul3(m, qw->k, &mk) || !mul3(m, qw->n, &mn) || !mul3(m, qw->k_pad, &mkp))
+        return fail(FA_ERR_SHAPE_MISMATCH, "linear_e4m3: shape overflows");
+    if (fa_status s = check_buf(ctx, x, "linear_e4m3: x")) return s;
+    if (x->dtype != FA_F32 && x->dtype != FA_BF16) return fail(FA_ERR_INVALID_ARGUMENT, "linear_e4m3: x must be f32 or bf16");
+    if (x->numel != mk) return fail(FA_ERR_SHAPE_MISMATCH, "linear_e4m3: x is not [m, k]");
+    if (bias)
+        if (fa_status s = check_view(ctx, bias, bias_offset, qw->n, FA_F32, "linear_e4m3: bias")) return s;
+    if (fa_status s = check_out_f32_or_bf16(ctx, out, mn, "linear_e4m3: out")) return s;
+    if (mn == 0) return FA_OK;
+    if (m > (1ull << 22)) return fail(FA_ERR_INVALID_ARGUMENT, "linear_e4m3: m too large for one launch");
+    Scratch sx(ctx), xq(ctx);
+    if (fa_status s = sx.get(m * 4)) return s;
+    if (fa_status s = xq.get(mkp)) return s;
+    // rows padded to the weight's k tiles with zero codes, so that any k is accepted
+    k::quantize_rows_e4m3(x->ptr, x->dtype == FA_BF16, (uint8_t *)xq.ptr, (float *)sx.ptr, m, qw->k, qw->k_pad, ctx->stream);
+    return launch_e4m3_rows(ctx, (const uint8_t *)xq.ptr, (const float *)sx.ptr, m, qw, bias, bias_offset, out);
 }
 
 // ------------------------------------------------------------------ norms

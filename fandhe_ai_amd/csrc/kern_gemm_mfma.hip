@@ -30,9 +30,10 @@ struct EpiI8 {
     int out_bf16;
 };
 struct EpiF8 {
-    const float *a_scale, *w_scale;
+    const float *a_scale, *w_scale;   // one scale each (per-tensor form) ...
     void *out;
     int out_bf16;
+    const float *sx, *sw, *bias;      // ... or, when sx is set, one per row and one per column (+ optional bias)
 };
 
 constexpr int BM = 128, BN = 128;      // block tile; 4 wavefronts in 2 x 2, 64 x 64 each
@@ -180,7 +181,12 @@ __global__ void __launch_bounds__(256)
                     }
                 }
                 if constexpr (FP8) {
-                    v = __fmul_rn(acc[i][j][e], __fmul_rn(*ep.a_scale, *ep.w_scale));
+                    if (ep.sx) {
+                        v = __fmul_rn(acc[i][j][e], __fmul_rn(ep.sx[row], ep.sw[col]));
+                        if (ep.bias) v = __fadd_rn(v, ep.bias[col]);
+                    } else {
+                        v = __fmul_rn(acc[i][j][e], __fmul_rn(*ep.a_scale, *ep.w_scale));
+                    }
                 } else {
                     if (ep.acc_out) ep.acc_out[o] = acc[i][j][e];
                     v = __fmul_rn((float)acc[i][j][e], __fmul_rn(ep.sx[row], ep.sw[col]));
@@ -484,8 +490,14 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
     float fscale = 0.0f;
     bool extras = false;
     const bool out_bf16 = ep.out_bf16 != 0;
-    if constexpr (FP8) fscale = __fmul_rn(*ep.a_scale, *ep.w_scale);
-    else extras = ep.acc_out != nullptr || ep.bias != nullptr || ep.residual != nullptr;
+    bool f8_rows = false;
+    if constexpr (FP8) {
+        f8_rows = ep.sx != nullptr;
+        if (!f8_rows) fscale = __fmul_rn(*ep.a_scale, *ep.w_scale);
+        extras = f8_rows && ep.bias != nullptr;
+    } else {
+        extras = ep.acc_out != nullptr || ep.bias != nullptr || ep.residual != nullptr;
+    }
     const uint32_t col0 = (nt0 + wn * WNT) * 16;      // first column of this wavefront
     const bool full_cols = nt0 + wn * WNT + WNT <= n_tiles && col0 + WNT * 16 <= n;
     if (!extras && full_cols && n % 8 == 0) {
@@ -497,7 +509,7 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
         constexpr int PITCH = COLS * 4 + 16;          // bytes; also enough for bf16
         uint8_t *band = lds + wave * (16 * PITCH);
         float swc[WNT];
-        if constexpr (!FP8) {
+        if (!FP8 || f8_rows) {
 #pragma unroll
             for (int j = 0; j < WNT; ++j) swc[j] = ep.sw[col0 + j * 16 + c];
         }
@@ -505,7 +517,7 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
         for (int i = 0; i < AI; ++i) {
             const uint32_t row_base = m0 + (wm * AI + i) * 16;
             float sxr[4];
-            if constexpr (!FP8) {
+            if (!FP8 || f8_rows) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     uint32_t row = row_base + 4 * g + e;
@@ -517,7 +529,7 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     float v;
-                    if constexpr (FP8) v = __fmul_rn(acc[i][j][e], fscale);
+                    if constexpr (FP8) v = __fmul_rn(acc[i][j][e], f8_rows ? __fmul_rn(sxr[e], swc[j]) : fscale);
                     else v = __fmul_rn((float)acc[i][j][e], __fmul_rn(sxr[e], swc[j]));
                     uint8_t *dst = band + (4 * g + e) * PITCH;
                     if (out_bf16)
@@ -550,7 +562,7 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
         const uint32_t col = (nt0 + wn * WNT + j) * 16 + c;
         const bool col_ok = col < n && nt0 + wn * WNT + j < n_tiles;
         float swc = 0.0f;
-        if constexpr (!FP8) swc = col_ok ? ep.sw[col] : 0.0f;
+        if (!FP8 || f8_rows) swc = col_ok ? ep.sw[col] : 0.0f;
 #pragma unroll
         for (int i = 0; i < AI; ++i) {
 #pragma unroll
@@ -560,7 +572,8 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
                     const uint64_t o = (uint64_t)row * n + col;
                     float v;
                     if constexpr (FP8) {
-                        v = __fmul_rn(acc[i][j][e], fscale);
+                        v = __fmul_rn(acc[i][j][e], f8_rows ? __fmul_rn(ep.sx[row], swc) : fscale);
+                        if (extras) v = __fadd_rn(v, ep.bias[col]);
                     } else {
                         v = __fmul_rn((float)acc[i][j][e], __fmul_rn(ep.sx[row], swc));
                         if (extras) {                  // uniform: raw accumulators, bias, residual
@@ -697,10 +710,24 @@ void gemm_w8a8_mfma(const int8_t *aq, const int8_t *w_tiles, uint64_t m, uint64_
     }
 }
 
+static void launch_e4m3(const uint8_t *aq, const uint8_t *w_tiles, const EpiF8 &e, uint64_t m, uint64_t n, uint64_t n_pad,
+                        uint64_t k_pad, int num_cus, hipStream_t s);
+
 void gemm_e4m3_mfma(const uint8_t *aq, const uint8_t *w_tiles, const float *a_scale, const float *w_scale, uint64_t m,
                     uint64_t n, uint64_t n_pad, uint64_t k_pad, void *out, int out_bf16, int num_cus, hipStream_t s) {
     if (m == 0 || n == 0) return;
-    EpiF8 e{a_scale, w_scale, out, out_bf16};
+    launch_e4m3(aq, w_tiles, EpiF8{a_scale, w_scale, out, out_bf16, nullptr, nullptr, nullptr}, m, n, n_pad, k_pad, num_cus, s);
+}
+
+void gemm_e4m3_rows_mfma(const uint8_t *aq, const uint8_t *w_tiles, const float *sx, const float *sw, const float *bias,
+                         uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad, void *out, int out_bf16, int num_cus,
+                         hipStream_t s) {
+    if (m == 0 || n == 0) return;
+    launch_e4m3(aq, w_tiles, EpiF8{nullptr, nullptr, out, out_bf16, sx, sw, bias}, m, n, n_pad, k_pad, num_cus, s);
+}
+
+static void launch_e4m3(const uint8_t *aq, const uint8_t *w_tiles, const EpiF8 &e, uint64_t m, uint64_t n, uint64_t n_pad,
+                        uint64_t k_pad, int num_cus, hipStream_t s) {
     if (int ntb = (g_gemm_small_tiles || k_pad == 0) ? 0 : pick_big_ntb(m, n_pad / 16, num_cus)) {
         if (ntb == 16)
             launch_big<true, 16, EpiF8>(aq, w_tiles, m, n, n_pad / 16, k_pad / 128, e, s);

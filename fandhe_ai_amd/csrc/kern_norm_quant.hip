@@ -337,6 +337,23 @@ __global__ void __launch_bounds__(kBlock) quantize_e4m3_kernel(const float *__re
     for (; i < n; i += stride) q[i] = scale == 0.0f ? 0 : (uint8_t)f32_to_e4m3(__fdiv_rn(x[i], scale));
 }
 
+// Per-token e4m3: one block per row, scale = absmax / 448, code = e4m3(x / scale), row-major codes with the
+// row padded to k_pad by zeros.
+template <bool IN_BF16>
+__global__ void __launch_bounds__(kBlock)
+    quantize_rows_e4m3_kernel(const void *__restrict__ x, uint8_t *__restrict__ xq, float *__restrict__ sx, uint64_t k,
+                              uint64_t k_pad) {
+    __shared__ float smem[kWaves];
+    const uint64_t r = blockIdx.x, base = r * k;
+    float amax = 0.0f;
+    for (uint64_t i = threadIdx.x; i < k; i += kBlock) amax = fmaxf(amax, fabsf(load_in<IN_BF16>(x, base + i)));
+    amax = block_max<kWaves>(amax, smem);
+    const float scale = __fdiv_rn(amax, 448.0f);
+    if (threadIdx.x == 0) sx[r] = scale;
+    for (uint64_t i = threadIdx.x; i < k_pad; i += kBlock)
+        xq[r * k_pad + i] = (i < k && scale != 0.0f) ? (uint8_t)f32_to_e4m3(__fdiv_rn(load_in<IN_BF16>(x, base + i), scale)) : 0;
+}
+
 __global__ void zero_f32_kernel(float *p) {
     if (threadIdx.x == 0 && blockIdx.x == 0) *p = 0.0f;
 }
@@ -404,6 +421,15 @@ void quantize_rows_from_pmax(const void *x, bool in_bf16, const float *pmax, uin
         quantize_from_pmax_kernel<true><<<grid, kBlock, 0, s>>>(x, pmax, parts, xq_tiled, sx, m, k);
     else
         quantize_from_pmax_kernel<false><<<grid, kBlock, 0, s>>>(x, pmax, parts, xq_tiled, sx, m, k);
+}
+
+void quantize_rows_e4m3(const void *x, bool in_bf16, uint8_t *xq_rowmajor, float *sx, uint64_t m, uint64_t k,
+                        uint64_t k_pad, hipStream_t s) {
+    if (m == 0 || k_pad == 0) return;
+    if (in_bf16)
+        quantize_rows_e4m3_kernel<true><<<(unsigned)m, kBlock, 0, s>>>(x, xq_rowmajor, sx, k, k_pad);
+    else
+        quantize_rows_e4m3_kernel<false><<<(unsigned)m, kBlock, 0, s>>>(x, xq_rowmajor, sx, k, k_pad);
 }
 
 void tensor_absmax_f32(const float *x, uint64_t n, float *absmax, hipStream_t s) {

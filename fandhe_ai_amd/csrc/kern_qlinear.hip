@@ -567,6 +567,98 @@ __global__ void __launch_bounds__(512)
     }
 }
 
+// ------------------------------------------------------------------ e4m3 x e4m3, decode shape
+// out[m, n] = (sum_k a[m, k] * w[k, n]) * (sx[m] * sw[n]) (+ bias[n]) on the scaled 16x16x128 fp8 matrix
+// instruction with unit block scales.  The weight is in tiles of 16 columns x 128 k (2 KiB, 32 bytes per lane:
+// column l % 16, k-group l / 16); the activations are row-major e4m3 [m, k_pad], and a lane fetches the 32 bytes
+// of row l % 16, k-group l / 16 of the k-tile directly (lanes of rows at or past m fetch the row tile's first
+// row: their accumulator rows are never stored).  One block per column tile, k split over the wavefronts, the
+// k-tiles of a wavefront streamed through a ring of D register slots as in the int8 kernel above; the partial
+// tiles are added in LDS in wavefront order.
+template <int MT, int NWAVES>
+__global__ void __launch_bounds__(NWAVES * 64)
+    e4m3_skinny_kernel(const uint8_t *__restrict__ aq, const uint8_t *__restrict__ w_tiles, const float *__restrict__ sx,
+                       const float *__restrict__ sw, const float *__restrict__ bias, uint32_t m, uint32_t n,
+                       uint32_t k_tiles, void *__restrict__ out, int out_bf16) {
+    constexpr int NACC = MT * 4, D = MT >= 3 ? 2 : 4;
+    __shared__ float red[NWAVES][NACC][64];
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+    const uint32_t nt = blockIdx.x;
+    const uint64_t k_bytes = (uint64_t)k_tiles * 128;
+    v4f acc[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) acc[i] = v4f{0.f, 0.f, 0.f, 0.f};
+    const uint8_t *b_base = w_tiles + (uint64_t)nt * k_tiles * 2048 + (uint64_t)lane * 32;
+    const uint8_t *a_base[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+        uint32_t row = (uint32_t)i * 16 + (uint32_t)lane % 16;
+        row = row < m ? row : (uint32_t)i * 16;
+        a_base[i] = aq + (uint64_t)row * k_bytes + (uint64_t)(lane / 16) * 32;
+    }
+    const uint32_t cnt = k_tiles > (uint32_t)wave ? (k_tiles - wave + NWAVES - 1) / NWAVES : 0;
+    v4i a[D][MT][2], b[D][2];
+    auto load_slot = [&](int s, uint32_t it) {
+        const uint32_t kt = wave + (it < cnt ? it : cnt - 1) * NWAVES;
+        const v4i *bp = (const v4i *)(b_base + (uint64_t)kt * 2048);
+        b[s][0] = bp[0];
+        b[s][1] = bp[1];
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            const v4i *ap = (const v4i *)(a_base[i] + (uint64_t)kt * 128);
+            a[s][i][0] = ap[0];
+            a[s][i][1] = ap[1];
+        }
+    };
+    auto mma_slot = [&](int s) {
+        const v8i y{b[s][0][0], b[s][0][1], b[s][0][2], b[s][0][3], b[s][1][0], b[s][1][1], b[s][1][2], b[s][1][3]};
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            const v8i x{a[s][i][0][0], a[s][i][0][1], a[s][i][0][2], a[s][i][0][3],
+                        a[s][i][1][0], a[s][i][1][1], a[s][i][1][2], a[s][i][1][3]};
+            acc[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(x, y, acc[i], 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
+        }
+    };
+    if (cnt != 0) {
+#pragma unroll
+        for (int s = 0; s < D; ++s) load_slot(s, (uint32_t)s);
+        uint32_t it0 = 0;
+        for (; it0 + D < cnt; it0 += D) {
+#pragma unroll
+            for (int s = 0; s < D; ++s) {
+                mma_slot(s);
+                __builtin_amdgcn_sched_barrier(0);
+                load_slot(s, it0 + D + s);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < D; ++s)
+            if (it0 + s < cnt) mma_slot(s);
+    }
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) red[wave][i * 4 + e][lane] = acc[i][e];
+    __syncthreads();
+    for (int idx = wave; idx < NACC; idx += NWAVES) {
+        float sum = red[0][idx][lane];
+#pragma unroll
+        for (int w = 1; w < NWAVES; ++w) sum = __fadd_rn(sum, red[w][idx][lane]);
+        const int e = idx % 4, i = idx / 4;
+        const uint32_t row = i * 16 + 4 * (lane / 16) + e, col = nt * 16 + lane % 16;
+        if (row < m && col < n) {
+            float v = __fmul_rn(sum, __fmul_rn(sx[row], sw[col]));
+            if (bias) v = __fadd_rn(v, bias[col]);
+            const uint64_t o = (uint64_t)row * n + col;
+            if (out_bf16)
+                ((uint16_t *)out)[o] = f32_to_bf16(v);
+            else
+                ((float *)out)[o] = v;
+        }
+    }
+}
+
 // Picks n-tiles per block and wavefronts per block so that the whole grid is
 // resident at once with about 8-16 wavefronts per compute unit.
 inline void pick_config(uint64_t n_tiles, uint64_t k_tiles, int num_cus, int *ntw, int *waves) {
@@ -698,6 +790,27 @@ void linear_w8a8_qkv_rope_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, 
     unsigned grid = n / 32;                                  // one block per pair of 16-column tiles
     int waves = g_skinny_waves ? g_skinny_waves : 8;
     launch_w8a8_rows<2, kEpiRope>(m, waves, grid, s, xq_tiled, w_tiles, (uint32_t)m, n, n_tiles, k_tiles, e);
+}
+
+void linear_e4m3_skinny(const uint8_t *aq, const uint8_t *w_tiles, const float *sx, const float *sw, const float *bias,
+                        uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad, void *out, int out_bf16, hipStream_t s) {
+    if (m == 0 || n == 0) return;
+    const uint32_t n_tiles = (uint32_t)(n_pad / 16), k_tiles = (uint32_t)(k_pad / 128);
+    auto go = [&](auto mt) {
+        constexpr int MT = decltype(mt)::value;
+        if (k_tiles >= 16)
+            e4m3_skinny_kernel<MT, 8><<<n_tiles, 512, 0, s>>>(aq, w_tiles, sx, sw, bias, (uint32_t)m, (uint32_t)n, k_tiles, out, out_bf16);
+        else
+            e4m3_skinny_kernel<MT, 4><<<n_tiles, 256, 0, s>>>(aq, w_tiles, sx, sw, bias, (uint32_t)m, (uint32_t)n, k_tiles, out, out_bf16);
+    };
+    if (m <= 16)
+        go(std::integral_constant<int, 1>{});
+    else if (m <= 32)
+        go(std::integral_constant<int, 2>{});
+    else if (m <= 48)
+        go(std::integral_constant<int, 3>{});
+    else
+        go(std::integral_constant<int, 4>{});
 }
 
 void linear_w8a16_skinny(const uint16_t *a, const int8_t *w_tiles, const float *sw, uint64_t m, uint64_t n,

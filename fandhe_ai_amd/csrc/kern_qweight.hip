@@ -23,10 +23,11 @@ __global__ void __launch_bounds__(256) col_absmax_kernel(const float *__restrict
     atomicMax(&absmax_bits[col], __float_as_uint(a));
 }
 
-__global__ void __launch_bounds__(256) absmax_to_scale_kernel(float *__restrict__ scales, uint64_t n, uint64_t n_pad) {
+__global__ void __launch_bounds__(256) absmax_to_scale_kernel(float *__restrict__ scales, uint64_t n, uint64_t n_pad,
+                                                              float divisor) {
     uint64_t col = (uint64_t)blockIdx.x * 256 + threadIdx.x;
     if (col >= n_pad) return;
-    scales[col] = col < n ? __fdiv_rn(scales[col], 127.0f) : 0.0f;
+    scales[col] = col < n ? __fdiv_rn(scales[col], divisor) : 0.0f;
 }
 
 // One thread per 16-byte (TILE_K 64) or 32-byte (TILE_K 128) lane chunk.
@@ -73,6 +74,19 @@ __global__ void __launch_bounds__(256)
     });
 }
 
+// per-column scales (scale_cols != 0) instead of one scale for the tensor
+__global__ void __launch_bounds__(256)
+    quantize_pack_e4m3_cols_kernel(const float *__restrict__ w, const float *__restrict__ scales, uint64_t k, uint64_t n,
+                                   uint64_t k_tiles, uint64_t n_chunks, uint8_t *__restrict__ tiles) {
+    uint64_t chunk = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (chunk >= n_chunks) return;
+    pack_chunk<128>(chunk, k_tiles, tiles, [&](uint64_t kk, uint64_t col) -> uint32_t {
+        if (kk >= k || col >= n) return 0u;
+        const float scale = scales[col];
+        return scale == 0.0f ? 0u : f32_to_e4m3(__fdiv_rn(w[kk * n + col], scale));
+    });
+}
+
 template <int TILE_K>
 __global__ void __launch_bounds__(256) pack_codes_kernel(const uint8_t *__restrict__ codes, uint64_t k, uint64_t n,
                                                          uint64_t k_tiles, uint64_t n_chunks, uint8_t *__restrict__ tiles) {
@@ -98,6 +112,18 @@ __global__ void __launch_bounds__(256) unpack_codes_kernel(const uint8_t *__rest
 }  // namespace
 
 void weight_col_scales_i8(const float *w, uint64_t k, uint64_t n, uint64_t n_pad, float *scales, hipStream_t s) {
+    weight_col_scales(w, k, n, n_pad, 127.0f, scales, s);
+}
+
+void weight_quantize_pack_e4m3_cols(const float *w, const float *scales, uint64_t k, uint64_t n, uint64_t k_pad,
+                                    uint64_t n_pad, uint8_t *tiles, hipStream_t s) {
+    uint64_t n_chunks = (k_pad / 128) * (n_pad / 16) * 64;
+    if (n_chunks == 0) return;
+    quantize_pack_e4m3_cols_kernel<<<(unsigned)((n_chunks + 255) / 256), 256, 0, s>>>(w, scales, k, n, k_pad / 128,
+                                                                                       n_chunks, tiles);
+}
+
+void weight_col_scales(const float *w, uint64_t k, uint64_t n, uint64_t n_pad, float divisor, float *scales, hipStream_t s) {
     if (n_pad == 0) return;
     fill_u32((uint32_t *)scales, 0u, n_pad, s);
     if (k != 0 && n != 0) {
@@ -106,7 +132,7 @@ void weight_col_scales_i8(const float *w, uint64_t k, uint64_t n, uint64_t n_pad
         dim3 grid((unsigned)((n + 255) / 256), (unsigned)slices);
         col_absmax_kernel<<<grid, 256, 0, s>>>(w, k, n, rows_per_slice, (unsigned int *)scales);
     }
-    absmax_to_scale_kernel<<<(unsigned)((n_pad + 255) / 256), 256, 0, s>>>(scales, n, n_pad);
+    absmax_to_scale_kernel<<<(unsigned)((n_pad + 255) / 256), 256, 0, s>>>(scales, n, n_pad, divisor);
 }
 
 void weight_quantize_pack_i8(const float *w, const float *scales, uint64_t k, uint64_t n, uint64_t k_pad,

@@ -62,10 +62,18 @@ void swiglu_quantize_rows_i8(const float *gu, int8_t *xq_rowmajor, float *sx, ui
 void quantize_tensor_e4m3(const float *x, uint8_t *q, float *scale, float *absmax_scratch, uint64_t n,
                           hipStream_t s);
 
+// Per-token e4m3 (scale = row absmax / 448): row-major codes [m, k_pad], rows zero-padded to k_pad, scales sx[m].
+void quantize_rows_e4m3(const void *x, bool in_bf16, uint8_t *xq_rowmajor, float *sx, uint64_t m, uint64_t k,
+                        uint64_t k_pad, hipStream_t s);
+
 // ---- weights (kern_qweight.hip) ----------------------------------------------
 // Column absmax / 127 of w[k, n] (f32, row-major) -> scales[n_pad] (padding 0)
 void weight_col_scales_i8(const float *w, uint64_t k, uint64_t n, uint64_t n_pad, float *scales,
                           hipStream_t s);
+// The same with scale = column absmax / divisor (448 for e4m3 weights with one scale per output channel).
+void weight_col_scales(const float *w, uint64_t k, uint64_t n, uint64_t n_pad, float divisor, float *scales, hipStream_t s);
+void weight_quantize_pack_e4m3_cols(const float *w, const float *scales, uint64_t k, uint64_t n, uint64_t k_pad,
+                                    uint64_t n_pad, uint8_t *tiles, hipStream_t s);
 void weight_quantize_pack_i8(const float *w, const float *scales, uint64_t k, uint64_t n,
                              uint64_t k_pad, uint64_t n_pad, int8_t *tiles, hipStream_t s);
 // Pack row-major codes [k, n] (1 byte each) into tile order; tile_k = 64 or 128.
@@ -139,6 +147,15 @@ GemmPlan gemm_plan(bool fp8, uint64_t m, uint64_t n_pad, uint64_t k_pad, int num
 void gemm_e4m3_mfma(const uint8_t *aq, const uint8_t *w_tiles, const float *a_scale,
                     const float *w_scale, uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad,
                     void *out, int out_bf16, int num_cus, hipStream_t s);
+// The same with one scale per row of aq (sx[m]) and one per output column (sw[n_pad]):
+// out = acc * (sx[row] * sw[col]) (+ bias[col]).
+void gemm_e4m3_rows_mfma(const uint8_t *aq, const uint8_t *w_tiles, const float *sx, const float *sw, const float *bias,
+                         uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad, void *out, int out_bf16, int num_cus,
+                         hipStream_t s);
+// Decode shape (m <= 64) of the same operator: a weight-streaming kernel, one block per 16-column tile, k split
+// over the block's wavefronts.
+void linear_e4m3_skinny(const uint8_t *aq, const uint8_t *w_tiles, const float *sx, const float *sw, const float *bias,
+                        uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad, void *out, int out_bf16, hipStream_t s);
 
 // ---- paged KV (kern_paged.hip) ---------------------------------------------------
 struct PagedShape {

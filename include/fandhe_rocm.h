@@ -135,14 +135,15 @@ fa_status fa_linear_forward_device(fa_context *ctx, const fa_buffer *a, uint64_t
  * A quantized weight is an opaque object: int8 (or e4m3) codes in an
  * MFMA-friendly tile order plus f32 scales. */
 typedef struct fa_qweight fa_qweight;
-typedef enum { FA_QW_INT8_CHANNEL = 0, FA_QW_E4M3_TENSOR = 1 } fa_qweight_kind;
+typedef enum { FA_QW_INT8_CHANNEL = 0, FA_QW_E4M3_TENSOR = 1, FA_QW_E4M3_CHANNEL = 2 } fa_qweight_kind;
 /* Quantize an f32 weight view w[k, n] (the layout of linear_forward_device)
- * on the device.  INT8_CHANNEL: one scale per output column.
- * E4M3_TENSOR: one scale (absmax / 448). */
+ * on the device.  INT8_CHANNEL: one scale per output column (absmax / 127).
+ * E4M3_TENSOR: one scale (absmax / 448).  E4M3_CHANNEL: e4m3 codes with one
+ * scale per output column (column absmax / 448). */
 fa_status fa_qweight_from_f32(fa_context *ctx, const fa_buffer *w, uint64_t w_offset, uint64_t k,
                               uint64_t n, fa_qweight_kind kind, fa_qweight **out);
 /* Import host codes q[k, n] (int8 or e4m3 bytes) with their scales
- * (n scales for INT8_CHANNEL, 1 for E4M3_TENSOR). */
+ * (n scales for INT8_CHANNEL and E4M3_CHANNEL, 1 for E4M3_TENSOR). */
 fa_status fa_qweight_from_codes(fa_context *ctx, const void *codes, const float *scales,
                                 uint64_t k, uint64_t n, fa_qweight_kind kind, fa_qweight **out);
 /* Read back codes as [k, n] and scales (test / export path; synchronizes). */
@@ -174,6 +175,24 @@ fa_status fa_quantize_tensor_e4m3(fa_context *ctx, const fa_buffer *x, uint64_t 
  * accumulation; qw of kind E4M3_TENSOR; out f32 or bf16. */
 fa_status fa_gemm_e4m3(fa_context *ctx, const fa_buffer *aq, const fa_buffer *a_scale, uint64_t m,
                        const fa_qweight *qw, fa_buffer *out);
+/* fp8 linear with per-token activation and per-channel weight scales (the
+ * e4m3 counterpart of fa_linear_w8a8; design record
+ * docs/spec-proposal-fp8-int8-quant-gemm.md:95-97): dynamic per-token
+ * quantization of x[m, k] (f32 or bf16) to e4m3, scale = row absmax / 448;
+ * writes row-major codes xq[m, k] and scales sx[m]. */
+fa_status fa_quantize_rows_e4m3(fa_context *ctx, const fa_buffer *x, uint64_t m, uint64_t k,
+                                fa_buffer *xq, fa_buffer *sx);
+/* out[m, n] = (xq @ W) * (sx[m] * sw[n]) (+ bias[n]) with f32 accumulation on
+ * the fp8 matrix cores and the dequantization fused into the epilogue; qw of
+ * kind E4M3_CHANNEL, x f32 or bf16 (quantized per token inside the call), out
+ * f32 or bf16.  Rows up to 64 take a weight-streaming kernel (decode shape),
+ * more rows the tiled GEMM kernels (k must then be a multiple of 128). */
+fa_status fa_linear_e4m3(fa_context *ctx, const fa_buffer *x, uint64_t m, const fa_qweight *qw,
+                         const fa_buffer *bias, uint64_t bias_offset, fa_buffer *out);
+/* The same on activations quantized beforehand (fa_quantize_rows_e4m3). */
+fa_status fa_gemm_e4m3_rows(fa_context *ctx, const fa_buffer *aq, const fa_buffer *sx, uint64_t m,
+                            const fa_qweight *qw, const fa_buffer *bias, uint64_t bias_offset,
+                            fa_buffer *out);
 /* int8 GEMM on pre-quantized row-major activations aq[m, k] with scales
  * sx[m] (prefill shape); same epilogue as fa_linear_w8a8. */
 fa_status fa_gemm_w8a8(fa_context *ctx, const fa_buffer *aq, const fa_buffer *sx, uint64_t m,

@@ -123,6 +123,17 @@ void orc_linear_w8a8(const float *x, const int8_t *wq, const float *sw, const fl
  * acc = fma over k ascending of a[m,k] * (float)wq[k,n]; out = acc * sw[n]. */
 void orc_linear_w8a16(const uint16_t *a_bf16, const int8_t *wq, const float *sw,
                       float *out_f32, size_t m, size_t n, size_t k);
+/* Per-token / per-channel fp8 (the e4m3 counterpart of the int8 quantizers above; build-defined like them,
+ * BASELINE.json north_star "fp8-e4m3 quantized linear (per-token activation and per-channel weight scales)"):
+ * scale = absmax / 448 over the row (rows) or the column (cols) of x[rows, cols], code = e4m3(x / scale), a zero
+ * row / column has scale 0 and codes 0.  Pinned by closed forms (the absmax element maps to +-448 = 0x7E / 0xFE,
+ * |x - decode(code) * scale| <= 2^-4 |x| + scale * 2^-10) in tests/test_oracle_pins.py. */
+void orc_quantize_rows_e4m3(const float *x, size_t rows, size_t cols, uint8_t *q, float *scale);
+void orc_quantize_cols_e4m3(const float *w, size_t k, size_t n, uint8_t *q, float *scale);
+/* out[i, j] = (float)(sum_k a[i,k] * b[k,j] summed exactly in double) * (sa[i] * sb[j]) (+ bias[j]); the scale
+ * product is formed once in f32, as in orc_dequant_i32.  Pinned by the double GEMM of the dequantized operands. */
+void orc_linear_e4m3_rows(const uint8_t *a, const uint8_t *b, const float *sa, const float *sb,
+                          const float *bias /*nullable*/, float *out, size_t m, size_t n, size_t k);
 /* Per-tensor fp8: scale = absmax / 448, code = e4m3(x / scale). */
 float orc_quantize_tensor_e4m3(const float *x, size_t n, uint8_t *q);
 /* out = (sum_k a*b accumulated in f64, rounded once to f32) * (sa * sb);

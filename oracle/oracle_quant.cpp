@@ -120,6 +120,54 @@ extern "C" float orc_quantize_tensor_e4m3(const float *x, size_t n, uint8_t *q) 
     return s;
 }
 
+extern "C" void orc_quantize_rows_e4m3(const float *x, size_t rows, size_t cols, uint8_t *q, float *scale) {
+    int nt = orc_get_threads();
+#pragma omp parallel for num_threads(nt) schedule(static) if (nt > 1)
+    for (size_t r = 0; r < rows; ++r) {
+        float amax = 0.0f;
+        for (size_t c = 0; c < cols; ++c) amax = std::fmax(amax, std::fabs(x[r * cols + c]));
+        float s = amax / 448.0f;
+        scale[r] = s;
+        for (size_t c = 0; c < cols; ++c) q[r * cols + c] = s == 0.0f ? 0 : orc_f32_to_e4m3(x[r * cols + c] / s);
+    }
+}
+
+extern "C" void orc_quantize_cols_e4m3(const float *w, size_t k, size_t n, uint8_t *q, float *scale) {
+    int nt = orc_get_threads();
+#pragma omp parallel for num_threads(nt) schedule(static) if (nt > 1)
+    for (size_t c = 0; c < n; ++c) {
+        float amax = 0.0f;
+        for (size_t r = 0; r < k; ++r) amax = std::fmax(amax, std::fabs(w[r * n + c]));
+        float s = amax / 448.0f;
+        scale[c] = s;
+        for (size_t r = 0; r < k; ++r) q[r * n + c] = s == 0.0f ? 0 : orc_f32_to_e4m3(w[r * n + c] / s);
+    }
+}
+
+extern "C" void orc_linear_e4m3_rows(const uint8_t *a, const uint8_t *b, const float *sa, const float *sb,
+                                     const float *bias, float *out, size_t m, size_t n, size_t k) {
+    float lut[256];
+    for (int i = 0; i < 256; ++i) lut[i] = orc_e4m3_to_f32((uint8_t)i);
+    int nt = orc_get_threads();
+#pragma omp parallel num_threads(nt) if (nt > 1)
+    {
+        std::vector<double> acc(n);
+#pragma omp for schedule(static)
+        for (size_t i = 0; i < m; ++i) {
+            std::fill(acc.begin(), acc.end(), 0.0);
+            for (size_t p = 0; p < k; ++p) {
+                double av = (double)lut[a[i * k + p]];
+                const uint8_t *b_row = b + p * n;
+                for (size_t j = 0; j < n; ++j) acc[j] += av * (double)lut[b_row[j]];
+            }
+            for (size_t j = 0; j < n; ++j) {
+                float v = (float)acc[j] * (sa[i] * sb[j]);
+                out[i * n + j] = bias ? v + bias[j] : v;
+            }
+        }
+    }
+}
+
 extern "C" void orc_gemm_e4m3(const uint8_t *a, const uint8_t *b, float sa, float sb, float *out,
                               size_t m, size_t n, size_t k) {
     float lut[256];

@@ -135,6 +135,9 @@ lib.orc_linear_w8a16.argtypes = [u16p, i8p, f32p, f32p, C.c_size_t, C.c_size_t, 
 lib.orc_quantize_tensor_e4m3.restype = C.c_float
 lib.orc_quantize_tensor_e4m3.argtypes = [f32p, C.c_size_t, u8p]
 lib.orc_gemm_e4m3.argtypes = [u8p, u8p, C.c_float, C.c_float, f32p, C.c_size_t, C.c_size_t, C.c_size_t]
+lib.orc_quantize_rows_e4m3.argtypes = [f32p, C.c_size_t, C.c_size_t, u8p, f32p]
+lib.orc_quantize_cols_e4m3.argtypes = [f32p, C.c_size_t, C.c_size_t, u8p, f32p]
+lib.orc_linear_e4m3_rows.argtypes = [u8p, u8p, f32p, f32p, f32p, f32p, C.c_size_t, C.c_size_t, C.c_size_t]
 lib.orc_rmsnorm_f32.argtypes = [f32p, f32p, C.c_size_t, C.c_float, C.c_size_t, C.c_size_t, C.c_size_t, f32p]
 lib.orc_rope_f32.argtypes = [f32p, i32p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_double, f32p]
 lib.orc_silu_f32.restype = C.c_float
@@ -302,6 +305,30 @@ def quantize_tensor_e4m3(x):
     q = np.empty(x.shape, dtype=np.uint8)
     s = lib.orc_quantize_tensor_e4m3(ptr(x, f32p), x.size, ptr(q, u8p))
     return q, np.float32(s)
+
+
+def quantize_rows_e4m3(x):
+    rows, cols = x.shape
+    q = np.empty((rows, cols), dtype=np.uint8)
+    s = np.empty(rows, dtype=np.float32)
+    lib.orc_quantize_rows_e4m3(ptr(x, f32p), rows, cols, ptr(q, u8p), ptr(s, f32p))
+    return q, s
+
+
+def quantize_cols_e4m3(w):
+    k, n = w.shape
+    q = np.empty((k, n), dtype=np.uint8)
+    s = np.empty(n, dtype=np.float32)
+    lib.orc_quantize_cols_e4m3(ptr(w, f32p), k, n, ptr(q, u8p), ptr(s, f32p))
+    return q, s
+
+
+def linear_e4m3_rows(a, b, sa, sb, bias=None):
+    m, k = a.shape
+    n = b.shape[1]
+    out = np.empty((m, n), dtype=np.float32)
+    lib.orc_linear_e4m3_rows(ptr(a, u8p), ptr(b, u8p), ptr(sa, f32p), ptr(sb, f32p), ptr(bias, f32p), ptr(out, f32p), m, n, k)
+    return out
 
 
 def gemm_e4m3(a, b, sa, sb):

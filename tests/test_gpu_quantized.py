@@ -501,3 +501,73 @@ def test_int8_large_tile_kernel_wavefront_variants_are_bit_exact():
     finally:
         fa.check(lib.fa_set_tuning(7, 0))
         fa.check(lib.fa_set_tuning(6, 0))
+
+
+def _fp8_rows_bound_check(tag, got, qa, qb, sa, sb, bias=None):
+    """Stated fp8 bound for the per-token x per-channel linear: |gpu - exact| <= 2^-15 * sum_k |a_k||b_k| * sa[m] * sb[n]
+    (+ one rounding of the bias add), and >= 98 % of the outputs inside the composite tolerance."""
+    o.set_threads(8)
+    want = o.linear_e4m3_rows(qa, qb, sa, sb, bias)
+    o.set_threads(1)
+    absprod = np.abs(o.from_e4m3(qa)).astype(np.float64) @ np.abs(o.from_e4m3(qb)).astype(np.float64)
+    bound = absprod * sa[:, None].astype(np.float64) * sb[None, :].astype(np.float64) * 2.0 ** -15 + 1e-30
+    if bias is not None:
+        bound = bound + np.abs(want) * 2.0 ** -23
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    print("FP8_ROWS_PARITY\t%s\tmax_err/bound=%.3e" % (tag, float((err / bound).max())), flush=True)
+    assert np.all(err <= bound), tag
+    r = o.compare(got, want)
+    print(r.line("FP8_ROWS_PARITY", tag), flush=True)
+    assert r.fail_count <= 2e-2 * r.total, tag
+    return want
+
+
+@pytest.mark.parametrize("m,k,n", [(1, 4096, 6144), (8, 4096, 4096), (32, 4096, 6144), (33, 1024, 528), (64, 11008, 512),
+                                   (17, 200, 70), (300, 1024, 520), (1000, 1024, 9004)])
+def test_fp8_per_token_per_channel_linear(m, k, n):
+    """fa_linear_e4m3: per-token e4m3 activations (row absmax / 448) against per-channel e4m3 weights (column
+    absmax / 448), dequantization fused.  Rows up to 64 take the weight-streaming kernel, 300 rows the 128 x 128
+    GEMM, 1000 x 9004 the large-tile GEMM; (17, 200, 70) has a k that is no multiple of the 128-wide tile."""
+    fa = _fa()
+    be = ops()
+    rng = np.random.default_rng(m * 7 + n)
+    x = rng.standard_normal((m, k), dtype=np.float32) * rng.uniform(0.1, 10.0, size=(m, 1)).astype(np.float32)
+    w = rng.standard_normal((k, n), dtype=np.float32) * rng.uniform(0.005, 0.05, size=(1, n)).astype(np.float32)
+    bias = rng.standard_normal(n, dtype=np.float32)
+    o.set_threads(8)
+    want_xq, want_sx = o.quantize_rows_e4m3(x)
+    want_wq, want_sw = o.quantize_cols_e4m3(w)
+    o.set_threads(1)
+    dx = be.upload(x)
+    xq, sx = be.quantize_rows_e4m3(dx)
+    assert np.array_equal(be.download(sx), want_sx) and np.array_equal(be.download(xq), want_xq)
+    qw = be.quantize_weight(fa.DeviceBufferView(be.upload(w), 0, (k, n)), fa.capi.QW_E4M3_CHANNEL)
+    codes, scales = qw.export()
+    assert np.array_equal(scales, want_sw) and np.array_equal(codes, want_wq)
+    qw2 = be.import_quantized_weight(want_wq, want_sw, fa.capi.QW_E4M3_CHANNEL)
+    c2, s2 = qw2.export()
+    assert np.array_equal(c2, want_wq) and np.array_equal(s2, want_sw)
+    if m > 64:
+        plan = _gemm_plan(fa, be, m, qw)
+        assert (plan.big_ntb != 0) == (m == 1000)
+    dbias = fa.DeviceBufferView(be.upload(bias), 0, (n,))
+    got = be.download_owned(be.linear_e4m3(dx, qw, out_dtype=fa.capi.F32))
+    _fp8_rows_bound_check("%dx%dx%d" % (m, n, k), got, want_xq, want_wq, want_sx, want_sw)
+    got_b = be.download_owned(be.linear_e4m3(dx, qw, bias=dbias, out_dtype=fa.capi.F32))
+    _fp8_rows_bound_check("%dx%dx%d+bias" % (m, n, k), got_b, want_xq, want_wq, want_sx, want_sw, bias)
+    assert_bf16_rounding_of("linear_e4m3 bf16", be.download_owned(be.linear_e4m3(dx, qw, bias=dbias, out_dtype=fa.capi.BF16)),
+                            got_b)
+    # bf16 activations are promoted exactly before the quantizer
+    xb = o.to_bf16(x)
+    o.set_threads(8)
+    qb16, sb16 = o.quantize_rows_e4m3(o.from_bf16(xb))
+    o.set_threads(1)
+    got16 = be.download_owned(be.linear_e4m3(be.upload(xb), qw, out_dtype=fa.capi.F32))
+    _fp8_rows_bound_check("%dx%dx%d:bf16 in" % (m, n, k), got16, qb16, want_wq, sb16, want_sw)
+    if k % 128 == 0:
+        # the pre-quantized entry point takes the same path: identical bits
+        again = be.download_owned(be.gemm_e4m3_rows(xq, sx, qw, out_dtype=fa.capi.F32))
+        assert np.array_equal(again, got)
+    # a weight of another kind is refused
+    with pytest.raises(fa.InvalidArgument):
+        be.linear_e4m3(dx, be.quantize_weight(fa.DeviceBufferView(be.upload(w), 0, (k, n)), fa.capi.QW_E4M3_TENSOR))

@@ -354,6 +354,53 @@ def test_fp8_quantize_and_gemm():
     assert np.abs(got - ref).max() < 0.1 * np.abs(ref).max()
 
 
+def test_fp8_per_token_and_per_channel_quantizers_and_linear():
+    """Closed forms for the per-row / per-column e4m3 quantizers and the double GEMM of the dequantized operands
+    for the linear built on them."""
+    rng = np.random.default_rng(18)
+    x = rng.normal(size=(6, 96)).astype(np.float32) * np.array([[1e-3], [1.0], [50.0], [0.0], [3.0], [1e4]], np.float32)
+    q, s = o.quantize_rows_e4m3(x)
+    amax = np.abs(x).max(axis=1)
+    assert np.array_equal(s, amax / np.float32(448.0))
+    dec = o.from_e4m3(q)
+    for r in range(6):
+        if amax[r] == 0:
+            assert s[r] == 0 and not q[r].any()                       # a zero row: scale 0, codes 0
+            continue
+        j = int(np.abs(x[r]).argmax())
+        assert q[r, j] == (0x7E if x[r, j] > 0 else 0xFE)             # the absmax element is +-448
+        assert np.abs(dec[r]).max() == 448.0
+        # three mantissa bits: half an ulp is 2^-4 relative for normal codes; below 2^-6 the spacing is 2^-9
+        err = np.abs(dec[r].astype(np.float64) * float(s[r]) - x[r].astype(np.float64))
+        assert np.all(err <= np.abs(x[r]) * 2.0 ** -4 + float(s[r]) * 2.0 ** -10 + 1e-30)
+        # every code is the nearest representable value of x / s (ties aside): re-encoding the scaled input agrees
+        assert np.array_equal(q[r], o.to_e4m3((x[r] / s[r]).astype(np.float32)))
+        # order is preserved
+        order = np.argsort(x[r], kind="stable")
+        assert np.all(np.diff(dec[r][order]) >= 0)
+    # columns: the transpose of the row quantizer
+    w = np.ascontiguousarray(x.T)
+    qc, sc = o.quantize_cols_e4m3(w)
+    assert np.array_equal(qc, q.T) and np.array_equal(sc, s)
+    # linear: exact double sum of the decoded codes, one f32 scale product per output, bias added last
+    a = rng.normal(size=(7, 128)).astype(np.float32)
+    b = (rng.normal(size=(128, 9)) * np.linspace(0.01, 3.0, 9)).astype(np.float32)
+    bias = rng.normal(size=9).astype(np.float32)
+    qa, sa = o.quantize_rows_e4m3(a)
+    qb, sb = o.quantize_cols_e4m3(b)
+    got = o.linear_e4m3_rows(qa, qb, sa, sb, bias)
+    exact = o.from_e4m3(qa).astype(np.float64) @ o.from_e4m3(qb).astype(np.float64)
+    want = exact.astype(np.float32) * (sa[:, None] * sb[None, :]) + bias[None, :]
+    assert np.array_equal(got, want.astype(np.float32))
+    assert np.array_equal(o.linear_e4m3_rows(qa, qb, sa, sb), (exact.astype(np.float32) * (sa[:, None] * sb[None, :])))
+    # with all scales equal it reduces to the per-tensor GEMM
+    ones_a, ones_b = np.full(7, 0.5, np.float32), np.full(9, 0.25, np.float32)
+    assert np.array_equal(o.linear_e4m3_rows(qa, qb, ones_a, ones_b), o.gemm_e4m3(qa, qb, np.float32(0.5), np.float32(0.25)))
+    # and the quantized linear tracks the real one (per-channel scales keep the small columns accurate)
+    ref = a.astype(np.float64) @ b.astype(np.float64)
+    assert np.all(np.abs(o.linear_e4m3_rows(qa, qb, sa, sb) - ref).max(axis=0) < 0.12 * np.abs(ref).max(axis=0))
+
+
 # ----------------------------------------------------------------- RMSNorm
 def test_rmsnorm_reference_fixtures():
     # crates/backend-cpu/src/rmsnorm.rs:433-441: [1,2,3,4], eps 0 -> x / sqrt(7.5)
