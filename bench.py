@@ -242,11 +242,14 @@ def bench_w8a8_decode(fa, be, cfg, m, iters):
     return res
 
 
-def bench_linears(fa, be, iters, ms=(1, 8, 32)):
+LINEAR_SHAPES = ((4096, 12288), (4096, 4096), (4096, 22016), (11008, 4096))
+
+
+def bench_linears(fa, be, iters, ms=(1, 8, 32), shapes=LINEAR_SHAPES):
     """Decode-shape int8-weight linears with bf16 activations (W8A16), Llama-7B layer shapes."""
     lib = fa.capi.lib
     res = []
-    for k, n in ((4096, 12288), (4096, 4096), (4096, 22016), (11008, 4096)):
+    for k, n in shapes:
         w = be.alloc_uninit((k, n))
         fa.check(lib.fa_fill_normal(be._ctx, w._h, 0, k * n, k + n, 0.0, 0.02))
         qw = be.quantize_weight(fa.DeviceBufferView(w, 0, (k, n)))
@@ -707,6 +710,9 @@ def main():
                     help="tuning: raw fa_set_tuning key/value pairs (experiments)")
     ap.add_argument("--rows", type=int, default=0,
                     help="with --only decode-linears: one row count of the sweep instead of 1, 8 and 32")
+    ap.add_argument("--shape", type=int, default=-1,
+                    help="with --only decode-linears: one of the four layer shapes (0 .. 3) instead of all, so that "
+                         "a counter run sees launches of one shape only")
     ap.add_argument("--only", choices=("attention", "copy", "linears", "decode-linears", "prefill", "prefill-attention", "mfma",
                                        "prompt", "stream-floor"), default=None,
                     help="profiling aid: run only the dominant kernel at the workload's shape, or a plain "
@@ -760,7 +766,8 @@ def main():
             be.close()
             return
         if a.only == "decode-linears":
-            for r in bench_linears(fa, be, 20, (a.rows,) if a.rows else (1, 8, 32)):
+            shapes = LINEAR_SHAPES if a.shape < 0 else LINEAR_SHAPES[a.shape:a.shape + 1]
+            for r in bench_linears(fa, be, 20, (a.rows,) if a.rows else (1, 8, 32), shapes):
                 log("w8a16 m=%d %5d->%5d: %.2f us, %.0f GB/s (%.1f %% of peak)" %
                     (r["m"], r["k"], r["n"], r["us"], r["gbs"], 100 * r["frac"]))
             be.close()

@@ -316,16 +316,40 @@ class RocmBackendOps:
         return out.reshape(buffer.shape) if (offset == 0 and numel is None) else out
 
     def download_owned(self, buffer):
-        out = self.download(buffer)
-        buffer.free()
-        return out
+        out = np.empty(buffer.numel(), dtype=_NP[buffer.dtype])
+        h, buffer._h = buffer._h, None  # the library frees the handle whether or not the copy succeeds
+        check(lib.fa_download_owned(self._ctx, h, out.ctypes.data, out.size))
+        return out.reshape(buffer.shape)
 
     def upload_into(self, tensor, dst, dst_offset):
         a = np.ascontiguousarray(tensor, dtype=_NP[dst.dtype])
         check(lib.fa_upload_into(self._ctx, a.ctypes.data, a.size, dst._h, dst_offset))
 
     def with_host_view(self, buffer, f):
-        f(self.download(buffer).ravel())
+        dt = _NP[buffer.dtype]
+        raised = []
+
+        def thunk(_user, data, numel):
+            try:
+                if numel == 0:
+                    f(np.empty(0, dtype=dt))
+                else:
+                    raw = (C.c_ubyte * (numel * np.dtype(dt).itemsize)).from_address(data)
+                    view = np.frombuffer(raw, dtype=dt)
+                    view.flags.writeable = False
+                    f(view)
+            except BaseException as e:  # an exception must not unwind through the C frame
+                raised.append(e)
+
+        cb = capi.HOST_VIEW_FN(thunk)
+        check(lib.fa_with_host_view(self._ctx, buffer._h, C.cast(cb, C.c_void_p), None))
+        if raised:
+            raise raised[0]
+
+    def is_poisoned(self):
+        flag = C.c_int32()
+        check(lib.fa_context_poisoned(self._ctx, C.byref(flag)))
+        return bool(flag.value)
 
     def synchronize_device(self):
         check(lib.fa_synchronize_device(self._ctx))

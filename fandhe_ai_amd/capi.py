@@ -35,6 +35,9 @@ f32p = C.POINTER(C.c_float)
 u64 = C.c_uint64
 
 
+HOST_VIEW_FN = C.CFUNCTYPE(None, C.c_void_p, C.c_void_p, C.c_uint64)
+
+
 class DeviceInfo(C.Structure):
     _fields_ = [("ordinal", C.c_int32), ("compute_units", C.c_int32), ("clock_khz", C.c_int32),
                 ("wavefront_size", C.c_int32), ("total_memory_bytes", C.c_uint64),
@@ -97,6 +100,9 @@ SIGNATURES = {
     "fa_upload": (C.c_int32, [ctx_p, C.c_int, C.c_void_p, u64, C.POINTER(buf_p)]),
     "fa_upload_into": (C.c_int32, [ctx_p, C.c_void_p, u64, buf_p, u64]),
     "fa_download": (C.c_int32, [ctx_p, buf_p, u64, C.c_void_p, u64]),
+    "fa_context_poisoned": (C.c_int32, [ctx_p, C.POINTER(C.c_int32)]),
+    "fa_download_owned": (C.c_int32, [ctx_p, buf_p, C.c_void_p, u64]),
+    "fa_with_host_view": (C.c_int32, [ctx_p, buf_p, C.c_void_p, C.c_void_p]),
     "fa_buffer_free": (C.c_int32, [ctx_p, buf_p]),
     "fa_buffer_numel": (u64, [buf_p]),
     "fa_buffer_dtype": (C.c_int, [buf_p]),

@@ -523,6 +523,36 @@ fa_status fa_download(fa_context *ctx, const fa_buffer *src, uint64_t src_offset
     return FA_OK;
 }
 
+fa_status fa_download_owned(fa_context *ctx, fa_buffer *src, void *host, uint64_t numel) {
+    fa_status s = fa_download(ctx, src, 0, host, numel);
+    // consumed either way; a handle that is not a buffer of this context was reported by the download
+    if (src && ctx && ctx->magic == kCtxMagic && src->magic == kBufMagic && src->ctx == ctx) {
+        const std::string msg = fa_last_error_message();
+        (void)fa_buffer_free(ctx, src);
+        if (s != FA_OK) set_error(msg);
+    }
+    return s;
+}
+
+fa_status fa_with_host_view(fa_context *ctx, const fa_buffer *src, fa_host_view_fn f, void *user) {
+    if (fa_status s = check_ctx(ctx)) return s;
+    if (fa_status s = check_buf(ctx, src, "fa_with_host_view: src")) return s;
+    if (!f) return fail(FA_ERR_INVALID_ARGUMENT, "fa_with_host_view: null callback");
+    if (src->numel == 0) {
+        f(user, nullptr, 0);
+        return FA_OK;
+    }
+    std::vector<unsigned char> host;
+    try {
+        host.resize(src->logical_bytes);
+    } catch (const std::exception &) {
+        return fail(FA_ERR_ALLOCATION_FAILED, "fa_with_host_view: out of host memory");
+    }
+    if (fa_status s = fa_download(ctx, src, 0, host.data(), src->numel)) return s;
+    f(user, host.data(), src->numel);
+    return FA_OK;
+}
+
 fa_status fa_buffer_free(fa_context *ctx, fa_buffer *buf) {
     if (!buf) return FA_OK;
     if (!ctx || ctx->magic != kCtxMagic) return fail(FA_ERR_INVALID_ARGUMENT, "fa_buffer_free: not a context");
@@ -543,6 +573,12 @@ fa_status fa_synchronize_device(fa_context *ctx) {
     if (fa_status s = reject_in_capture(ctx, "fa_synchronize_device")) return s;
     hipError_t e = hipStreamSynchronize(ctx->stream);
     if (e != hipSuccess) return hip_fail(ctx, e, "hipStreamSynchronize", FA_ERR_KERNEL_LAUNCH_FAILED);
+    return FA_OK;
+}
+
+fa_status fa_context_poisoned(const fa_context *ctx, int32_t *poisoned) {
+    if (!ctx || ctx->magic != kCtxMagic || !poisoned) return fail(FA_ERR_INVALID_ARGUMENT, "fa_context_poisoned: bad argument");
+    *poisoned = ctx->poisoned ? 1 : 0;
     return FA_OK;
 }
 

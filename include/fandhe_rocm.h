@@ -90,6 +90,13 @@ fa_status fa_upload_into(fa_context *ctx, const void *host, uint64_t numel, fa_b
  * synchronization point).  src_offset / numel in elements. */
 fa_status fa_download(fa_context *ctx, const fa_buffer *src, uint64_t src_offset, void *host,
                       uint64_t numel);
+/* MemoryOps::download_owned (buffer.rs:414-430): the caller gives the buffer up; host data is final on return
+ * and the handle is freed whether or not the copy succeeded (it is consumed either way, as in the trait). */
+fa_status fa_download_owned(fa_context *ctx, fa_buffer *src, void *host, uint64_t numel);
+/* MemoryOps::with_host_view (buffer.rs:486-521): calls f(user, data, numel) once with a host copy of the whole
+ * buffer that is valid only during the call (numel == 0: an empty view, no device access). */
+typedef void (*fa_host_view_fn)(void *user, const void *data, uint64_t numel);
+fa_status fa_with_host_view(fa_context *ctx, const fa_buffer *src, fa_host_view_fn f, void *user);
 /* Drop of the handle (buffer.rs:40-48): returns the block to the pool. */
 fa_status fa_buffer_free(fa_context *ctx, fa_buffer *buf);
 uint64_t fa_buffer_numel(const fa_buffer *buf);
@@ -98,6 +105,11 @@ void *fa_buffer_device_ptr(const fa_buffer *buf);
 
 /* BackendOps::synchronize_device (backend_ops.rs:4897). */
 fa_status fa_synchronize_device(fa_context *ctx);
+/* Whether an earlier device failure poisoned the context (1) or not (0); never fails on a live context and
+ * does not touch the device.  With all work ordered on one stream this is what a caller re-checks after a
+ * download where a batching backend would re-check a DispatchFailureCell (dispatch_failure.rs:1-40;
+ * backend_ops.rs:4724-4726: a stream-ordered backend poisons the ordinal and keeps the *_tracked defaults). */
+fa_status fa_context_poisoned(const fa_context *ctx, int32_t *poisoned);
 /* The HIP stream (hipStream_t) every call of this context is ordered on. */
 void *fa_context_stream(fa_context *ctx);
 

@@ -28,7 +28,7 @@ def test_memory_ops_round_trip_views_and_pool():
     be = ops()
     x = np.arange(1000, dtype=np.float32).reshape(10, 100)
     b = be.upload(x)
-    assert np.array_equal(be.download(b), x)
+    assert np.array_equal(be.download(b), x) and not be.is_poisoned()
     z = be.alloc_zeroed((7, 5))
     assert not be.download(z).any()
     be.upload_into(np.array([1, 2, 3], np.float32), z, 4)
@@ -41,9 +41,20 @@ def test_memory_ops_round_trip_views_and_pool():
     seen = []
     be.with_host_view(b, lambda s: seen.append(float(s.sum())))
     assert seen == [float(x.sum())]
+    # the view is read-only and dies with the call; an exception of the closure comes back to the caller
+    with pytest.raises(ValueError):
+        be.with_host_view(b, lambda s: s.__setitem__(0, 1.0))
+    with pytest.raises(KeyError):
+        be.with_host_view(b, lambda s: {}["x"])
+    # download_owned consumes the handle (crates/tensor-core/src/buffer.rs:414-430)
+    c = be.upload(x)
+    assert np.array_equal(be.download_owned(c), x) and c._h is None
+    c.free()                                # a second release of a consumed buffer is a no-op
     # numel == 0 never touches the device (crates/tensor-core/src/buffer.rs:50-59)
     e = be.alloc_zeroed((0, 4))
     assert be.download(e).size == 0
+    be.with_host_view(e, lambda s: seen.append(s.size))
+    assert seen[-1] == 0
     # pool: a freed block is reused for the same size class, stats follow pool_core.rs:122-139
     s0 = be.device_memory_pool_stats()
     t = be.alloc_zeroed((1000,))            # 4000 B -> class 4096
