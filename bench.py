@@ -32,7 +32,7 @@ MFMA_PEAK_TOPS = 5000.0          # dense int8 and fp8 on MI355X
 # HBM bytes per launch of decode_stream_kernel at this benchmark's shape, from hardware counters
 # (rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE, each scaled by the same counter's reading for a plain
 # row-copy kernel of known size; the figures are in profiles/decode_stream_kernel_config5_pmc.txt).
-ATTENTION_TRAFFIC_BYTES = 627583562
+ATTENTION_TRAFFIC_BYTES = 627514974
 U32MAX = 0xFFFFFFFF
 SERVING_ROWS = 64          # rows of the continuous-batching run (the decoder's limit)
 
@@ -530,7 +530,8 @@ def floor_sizes(cfg, att_bytes):
     D, F, V = cfg["d_model"], cfg["d_ffn"], cfg["vocab"]
     EQ, EKV = cfg["n_heads"] * cfg["head_dim"], cfg["n_kv_heads"] * cfg["head_dim"]
     return [("o projection weight 4096x4096", EQ * D), ("qkv weight 4096x6144", D * (EQ + 2 * EKV)),
-            ("config-2 weight 4096x12288", 4096 * 12288), ("down weight 14336x4096", F * D),
+            ("config-2 weight 11008x4096", 11008 * 4096), ("config-2 weight 4096x12288", 4096 * 12288),
+            ("down weight 14336x4096", F * D),
             ("config-2 weight 4096x22016", 4096 * 22016), ("gate/up weight 4096x28672", D * 2 * F),
             ("lm_head weight 4096x32000", D * V), ("decode attention K/V of one layer", att_bytes)]
 
@@ -681,9 +682,17 @@ def cpu_operator_baselines(fa, be, threads):
     a_rows = np.ascontiguousarray(be.download(xq)[sel])
     sa, sw = np.float32(be.download(xs)[0]), np.float32(wscale[0])
     sec, iters = _median_time(lambda: o.gemm_e4m3(a_rows, codes, sa, sw), 3, 2.0)
-    r = o.compare(got, o.gemm_e4m3(a_rows, codes, sa, sw))
+    want = o.gemm_e4m3(a_rows, codes, sa, sw)
+    r = o.compare(got, want)
+    # the fp8 bar: every output within 2^-15 * sum_k |a_k||b_k| * (sa * sw) of the exact-product f64 sum (the f32
+    # accumulation of the matrix cores), and at least 98 % of them inside rel < 1e-3 or abs < 1e-5 as well
+    absprod = np.abs(o.from_e4m3(a_rows)).astype(np.float64) @ np.abs(o.from_e4m3(codes)).astype(np.float64)
+    bound = absprod * float(sa) * float(sw) * 2.0 ** -15 + 1e-30
+    over = int((np.abs(got.astype(np.float64) - want.astype(np.float64)) > bound).sum())
     gemm.append(dict(op="gemm_e4m3", m=m, k=k, n=n, cpu_ms_full=sec * m / rows * 1e3, sampled_rows=rows, iters=iters,
-                     parity_fail=int(r.fail_count), parity=r.line("FP8_PARITY", "%dx%dx%d" % (m, n, k))))
+                     parity_fail=over + (int(r.fail_count) if r.fail_count > 2e-2 * r.total else 0),
+                     outside_fp8_bound=over, outside_composite=int(r.fail_count), total=int(r.total),
+                     parity=r.line("FP8_PARITY", "%dx%dx%d" % (m, n, k))))
     for b in (qw, xq, xs, w, x):
         b.free()
     res["prefill_gemm"] = gemm
