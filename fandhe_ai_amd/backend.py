@@ -516,6 +516,21 @@ class RocmBackendOps:
                                  generator._h if generator is not None else None, out._h))
         return out
 
+    def sampling_weights(self, logits, rows, vocab, strategy, temperature, top_k, weights, status, logits_row=0, weights_row=0):
+        """``sampling_weights_f32`` (crates/autodiff/src/generate/mod.rs:432-452) of `rows` rows of `logits` from row
+        `logits_row` on, into rows `weights_row` .. of `weights`; `logits` may be a raw buffer handle."""
+        check(lib.fa_sampling_weights(self._ctx, getattr(logits, "_h", logits), logits_row * vocab, rows, vocab, strategy,
+                                      temperature, top_k, weights._h, weights_row * vocab, status._h))
+
+    def speculative_accept(self, p_weights, q_weights, drafts, vocab, generator, result, p_row=0, q_row=0):
+        """``verify_sampling`` (crates/autodiff/src/generate/speculative.rs:246-279) on the device; no drafts: one
+        draw from row `p_row` of p_weights.  Returns (accepted drafts, next token, status) after a download."""
+        d = np.ascontiguousarray(drafts, dtype=np.int32)
+        check(lib.fa_speculative_accept(self._ctx, p_weights._h, p_row * vocab, q_weights._h if d.size else None, q_row * vocab,
+                                        d.ctypes.data_as(capi.i32p) if d.size else None, d.size, vocab, generator._h, result._h))
+        n_acc, token, status, _ = (int(v) for v in self.download(result))
+        return n_acc, token, status
+
     def sample_rows_per_row(self, logits, table):
         """Next tokens [rows] where row r follows record r of `table`, a U32 device buffer of 6 * rows elements
         holding fa_row_sampling records (see ``row_sampling_table``); generator states advance in the table."""

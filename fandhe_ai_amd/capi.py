@@ -150,6 +150,8 @@ SIGNATURES = {
                                                      C.POINTER(PagedArgs), buf_p]),
     "fa_paged_attention_decode_static_max_bytes": (u64, []),
     "fa_sample_rows": (C.c_int32, [ctx_p, buf_p, u64, u64, C.c_int32, C.c_float, u64, buf_p, buf_p]),
+    "fa_sampling_weights": (C.c_int32, [ctx_p, buf_p, u64, u64, u64, C.c_int32, C.c_float, u64, buf_p, u64, buf_p]),
+    "fa_speculative_accept": (C.c_int32, [ctx_p, buf_p, u64, buf_p, u64, i32p, u64, u64, buf_p, buf_p]),
     "fa_rng_seed": (C.c_int32, [ctx_p, buf_p, u64]),
     "fa_decoder_set_sampling": (C.c_int32, [ctx_p, C.c_void_p, C.c_int32, C.c_float, u64, u64]),
     "fa_rng_state_from_seed": (C.c_int32, [u64, C.POINTER(u64)]),
@@ -197,6 +199,7 @@ SIGNATURES = {
     "fa_decoder_step": (C.c_int32, [ctx_p, C.c_void_p, C.c_int32]),
     "fa_decoder_read_tokens": (C.c_int32, [ctx_p, C.c_void_p, i32p]),
     "fa_decoder_read_logits": (C.c_int32, [ctx_p, C.c_void_p, f32p]),
+    "fa_decoder_logits_buffer": (C.c_int32, [C.c_void_p, C.POINTER(buf_p)]),
     "fa_decoder_read_seq_lens": (C.c_int32, [ctx_p, C.c_void_p, u32p]),
     "fa_set_tuning": (C.c_int32, [C.c_int32, C.c_int32]),
     "fa_timer_create": (C.c_int32, [ctx_p, C.POINTER(C.c_void_p)]),

@@ -618,6 +618,59 @@ fa_status fa_sample_rows(fa_context *ctx, const fa_buffer *logits, uint64_t rows
     return after_launch(ctx, "sample_rows");
 }
 
+fa_status fa_sampling_weights(fa_context *ctx, const fa_buffer *logits, uint64_t logits_offset, uint64_t rows, uint64_t vocab,
+                              fa_sampling strategy, float temperature, uint64_t top_k, fa_buffer *weights,
+                              uint64_t weights_offset, fa_buffer *status) {
+    if (fa_status s = check_ctx(ctx)) return s;
+    uint64_t numel, end;
+    if (!mul3(rows, vocab, &numel) || __builtin_add_overflow(numel, logits_offset, &end))
+        return fail(FA_ERR_SHAPE_MISMATCH, "sampling_weights: shape overflows");
+    if (fa_status s = check_buf_typed(ctx, logits, FA_F32, end, "sampling_weights: logits")) return s;
+    if (__builtin_add_overflow(numel, weights_offset, &end)) return fail(FA_ERR_SHAPE_MISMATCH, "sampling_weights: shape overflows");
+    if (fa_status s = check_buf_typed(ctx, weights, FA_F32, end, "sampling_weights: weights")) return s;
+    if (fa_status s = check_buf_typed(ctx, status, FA_I32, rows, "sampling_weights: status")) return s;
+    if (vocab == 0 || vocab > (uint64_t)INT32_MAX)
+        return fail(FA_ERR_INVALID_ARGUMENT, "sampling_weights: vocab must be in 1..=i32::MAX");
+    if (rows > 65535) return fail(FA_ERR_INVALID_ARGUMENT, "sampling_weights: at most 65535 rows per call");
+    if (fa_status s = check_sampling(strategy, temperature, top_k, vocab)) return s;
+    if (rows == 0) return FA_OK;
+    const int mode = strategy == FA_SAMPLE_GREEDY ? 2 : (strategy == FA_SAMPLE_TOP_K ? 1 : 0);
+    k::sampling_weights((const float *)logits->ptr + logits_offset, (float *)weights->ptr + weights_offset, (int32_t *)status->ptr,
+                        (uint32_t)rows, (uint32_t)vocab, mode, temperature, (uint32_t)top_k, ctx->stream);
+    return after_launch(ctx, "sampling_weights");
+}
+
+fa_status fa_speculative_accept(fa_context *ctx, const fa_buffer *p_weights, uint64_t p_offset, const fa_buffer *q_weights,
+                                uint64_t q_offset, const int32_t *drafts, uint64_t k, uint64_t vocab, fa_buffer *rng,
+                                fa_buffer *result) {
+    if (fa_status s = check_ctx(ctx)) return s;
+    if (k > k::kMaxDraftTokens) return fail(FA_ERR_INVALID_ARGUMENT, "speculative_accept: at most 32 draft tokens per call");
+    if (vocab == 0 || vocab > (uint64_t)INT32_MAX)
+        return fail(FA_ERR_INVALID_ARGUMENT, "speculative_accept: vocab must be in 1..=i32::MAX");
+    uint64_t numel, end;
+    if (!mul3(k + 1, vocab, &numel) || __builtin_add_overflow(numel, p_offset, &end))
+        return fail(FA_ERR_SHAPE_MISMATCH, "speculative_accept: shape overflows");
+    if (fa_status s = check_buf_typed(ctx, p_weights, FA_F32, end, "speculative_accept: p_weights")) return s;
+    k::DraftTokens d{};
+    if (k > 0) {
+        if (!drafts) return fail(FA_ERR_INVALID_ARGUMENT, "speculative_accept: null drafts");
+        if (!mul3(k, vocab, &numel) || __builtin_add_overflow(numel, q_offset, &end))
+            return fail(FA_ERR_SHAPE_MISMATCH, "speculative_accept: shape overflows");
+        if (fa_status s = check_buf_typed(ctx, q_weights, FA_F32, end, "speculative_accept: q_weights")) return s;
+        for (uint64_t i = 0; i < k; ++i) {
+            if (drafts[i] < 0 || (uint64_t)drafts[i] >= vocab)
+                return fail(FA_ERR_INVALID_ARGUMENT, "speculative_accept: draft " + std::to_string(i) + " (" +
+                                                         std::to_string(drafts[i]) + ") is outside the vocabulary");
+            d.d[i] = drafts[i];
+        }
+    }
+    if (fa_status s = check_buf_typed(ctx, rng, FA_U32, 2, "speculative_accept: rng")) return s;
+    if (fa_status s = check_buf_typed(ctx, result, FA_I32, 4, "speculative_accept: result")) return s;
+    k::speculative_accept((const float *)p_weights->ptr + p_offset, k ? (const float *)q_weights->ptr + q_offset : nullptr, d,
+                          (uint32_t)k, (uint32_t)vocab, (uint64_t *)rng->ptr, (int32_t *)result->ptr, ctx->stream);
+    return after_launch(ctx, "speculative_accept");
+}
+
 fa_status fa_rng_seed(fa_context *ctx, fa_buffer *rng, uint64_t seed) {
     if (fa_status s = check_ctx(ctx)) return s;
     if (fa_status s = check_buf_typed(ctx, rng, FA_U32, 2, "rng_seed: rng")) return s;

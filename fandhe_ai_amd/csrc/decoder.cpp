@@ -816,6 +816,12 @@ fa_status fa_decoder_read_logits(fa_context *ctx, fa_decoder *d, float *logits) 
     if (fa_status s = check_dec(d)) return s;
     return fa_download(ctx, d->logits, 0, logits, (uint64_t)d->batch * d->cfg.vocab);
 }
+fa_status fa_decoder_logits_buffer(fa_decoder *d, fa_buffer **out) {
+    if (fa_status s = check_dec(d)) return s;
+    if (!out) return fail(FA_ERR_INVALID_ARGUMENT, "decoder_logits_buffer: null out");
+    *out = d->logits;
+    return FA_OK;
+}
 fa_status fa_decoder_read_seq_lens(fa_context *ctx, fa_decoder *d, uint32_t *seq_lens) {
     if (fa_status s = check_dec(d)) return s;
     return fa_download(ctx, d->seq_lens, 0, seq_lens, d->batch);

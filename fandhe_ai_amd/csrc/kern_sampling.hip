@@ -52,9 +52,13 @@ __device__ __forceinline__ T block_exclusive_scan(T v, T *buf, T *total) {
     return incl - v;
 }
 
+// WEIGHTS: the draw is left out and the row's f32 sampling weights are stored instead (one-hot at the first
+// maximum for a greedy row; NaN throughout, and status 1, when a logit is not finite).
+template <bool WEIGHTS>
 __global__ void __launch_bounds__(kThreads)
     sample_rows_kernel(const float *__restrict__ logits, int32_t *__restrict__ tokens, const uint64_t *__restrict__ rng_state,
-                       RowPolicy *__restrict__ policy, uint32_t vocab, int top_k_mode, float temperature, uint32_t top_k) {
+                       RowPolicy *__restrict__ policy, uint32_t vocab, int top_k_mode, float temperature, uint32_t top_k,
+                       float *__restrict__ weights_out, int32_t *__restrict__ status, int greedy_weights) {
     __shared__ double s_d[kThreads];
     __shared__ uint32_t s_u[kThreads];
     __shared__ uint32_t hist[256];
@@ -63,7 +67,8 @@ __global__ void __launch_bounds__(kThreads)
     __shared__ double s_x;
     const uint32_t b = blockIdx.x, t = threadIdx.x;
     const float *row = logits + (uint64_t)b * vocab;
-    bool greedy = false;
+    bool greedy = WEIGHTS && greedy_weights != 0;
+    float *wrow = WEIGHTS ? weights_out + (uint64_t)b * vocab : nullptr;
     if (policy) {                                        // uniform over the block
         const RowPolicy pr = policy[b];
         greedy = pr.strategy == 0;
@@ -89,9 +94,15 @@ __global__ void __launch_bounds__(kThreads)
     if (t % 64 == 0) s_max[t / 64] = mx;
     __syncthreads();
     if (s_sel[2]) {
-        if (t == 0) tokens[b] = -1;
+        if constexpr (WEIGHTS) {
+            for (uint32_t i = lo; i < hi; ++i) wrow[i] = __uint_as_float(0x7fc00000u);
+            if (t == 0) status[b] = 1;
+        } else {
+            if (t == 0) tokens[b] = -1;
+        }
         return;
     }
+    if (WEIGHTS && t == 0) status[b] = 0;
     mx = s_max[0];
     for (int w = 1; w < kThreads / 64; ++w) mx = fmaxf(mx, s_max[w]);
     if (greedy) {                                        // first index holding the maximum
@@ -103,7 +114,11 @@ __global__ void __launch_bounds__(kThreads)
                 break;
             }
         __syncthreads();
-        if (t == 0) tokens[b] = (int32_t)s_sel[0];
+        if constexpr (WEIGHTS) {
+            for (uint32_t i = lo; i < hi; ++i) wrow[i] = i == s_sel[0] ? 1.0f : 0.0f;
+        } else {
+            if (t == 0) tokens[b] = (int32_t)s_sel[0];
+        }
         return;
     }
     const double dmax = (double)mx, dt = (double)temperature;
@@ -172,6 +187,10 @@ __global__ void __launch_bounds__(kThreads)
 
     // ---- f32 weights, their f64 cumulative sums, and the draw
     auto weight = [&](float v, bool kept) -> float { return kept ? (float)(exp(((double)v - dmax) / dt) / sum_exp) : 0.0f; };
+    if constexpr (WEIGHTS) {
+        for_each_kept([&](uint32_t i, float v, bool kept) { wrow[i] = weight(v, kept); });
+        return;
+    }
     double wsum = 0.0;
     uint32_t last_pos = 0;
     bool any_pos = false;
@@ -450,7 +469,127 @@ static void launch_sampler(uint32_t rows, uint32_t vocab, hipStream_t s, A... ar
     else if (vocab <= kThreads * 32)
         sample_rows_reg_kernel<32><<<rows, kThreads, 0, s>>>(args...);
     else
-        sample_rows_kernel<<<rows, kThreads, 0, s>>>(args...);
+        sample_rows_kernel<false><<<rows, kThreads, 0, s>>>(args..., (float *)nullptr, (int32_t *)nullptr, 0);
+}
+
+// Acceptance step of sampled speculative decoding for one sequence (crates/autodiff/src/generate/
+// speculative.rs:111-189, 246-279), one block: for draft i, p and q are the f32 weight rows of the target and
+// of the draft normalised in f64; the draft is accepted when the next uniform u < (f32)min(1, p[d] / q[d]);
+// at the first refusal one token is drawn from max(0, p - q) / sum (cast to f32, drawn like every multinomial
+// here) and the kernel stops; if all k drafts are accepted one token is drawn from row k of the target's
+// weights.  k = 0 is a plain draw from a weight row.  result: accepted drafts, token, status (0 ok; 2 q(d) not
+// positive or a probability not finite; 3 a weight row negative, not finite or summing to zero; 4 the
+// residual sums to zero; 5 a draft outside the vocabulary).  The generator state is read once and stored
+// back with the draws this call consumed.  The f64 sums are block-wide trees instead of sequential passes.
+__global__ void __launch_bounds__(kThreads)
+    speculative_accept_kernel(const float *__restrict__ p_w, const float *__restrict__ q_w, DraftTokens drafts, uint32_t k,
+                              uint32_t vocab, uint64_t *__restrict__ rng_state, int32_t *__restrict__ result) {
+    constexpr int kW = kThreads / 64;
+    __shared__ double s_d[kW];
+    __shared__ uint32_t s_sel[2];
+    __shared__ double s_x;
+    __shared__ int s_flag;
+    const uint32_t t = threadIdx.x;
+    const uint32_t seg = (vocab + kThreads - 1) / kThreads;
+    const uint32_t lo = t * seg < vocab ? t * seg : vocab, hi = lo + seg < vocab ? lo + seg : vocab;
+    uint64_t st = rng_state[0];                          // only thread 0 advances and stores it
+    auto finish = [&](uint32_t n_acc, int32_t token, int32_t status) {
+        if (t == 0) {
+            result[0] = (int32_t)n_acc;
+            result[1] = token;
+            result[2] = status;
+            rng_state[0] = st;
+        }
+    };
+    // f64 sum of a weight row; ok = every weight finite and not negative
+    auto row_sum = [&](const float *w, bool *ok) -> double {
+        double part = 0.0;
+        int good = 1;
+        for (uint32_t i = lo; i < hi; ++i) {
+            const float v = w[i];
+            good &= (v >= 0.0f && v <= 3.402823466e38f) ? 1 : 0;
+            part += (double)v;
+        }
+        double total;
+        (void)block_exclusive_scan_fast<double>(part, s_d, &total);
+        *ok = __syncthreads_and(good) != 0;
+        return total;
+    };
+    // one multinomial draw from weights given by index; -1 (and nothing drawn) when they sum to zero
+    auto draw = [&](auto &&weight_at) -> int32_t {
+        double wsum = 0.0;
+        uint32_t last_pos = 0;
+        for (uint32_t i = lo; i < hi; ++i) {
+            const float w = weight_at(i);
+            wsum += (double)w;
+            if (w > 0.0f) last_pos = i + 1;
+        }
+        double total;
+        const double before = block_exclusive_scan_fast<double>(wsum, s_d, &total);
+        if (!(total > 0.0)) return -1;                   // uniform over the block
+        if (t == 0) {
+            const uint64_t bits = xorshift64star_next(st);
+            s_x = (double)(bits >> 11) / 9007199254740992.0 * total;
+            s_sel[0] = 0xffffffffu;
+            s_sel[1] = 0;
+        }
+        __syncthreads();
+        const double x = s_x;
+        if (last_pos) atomicMax(&s_sel[1], last_pos);
+        double acc = before;
+        uint32_t found = 0xffffffffu;
+        for (uint32_t i = lo; i < hi; ++i) {
+            const float w = weight_at(i);
+            acc += (double)w;
+            if (found == 0xffffffffu && w > 0.0f && acc > x) found = i;
+        }
+        if (found != 0xffffffffu) atomicMin(&s_sel[0], found);
+        __syncthreads();
+        uint32_t idx = s_sel[0];
+        if (idx == 0xffffffffu) idx = s_sel[1] ? s_sel[1] - 1 : vocab - 1;
+        __syncthreads();
+        return (int32_t)idx;
+    };
+    for (uint32_t i = 0; i < k; ++i) {
+        const float *pr = p_w + (uint64_t)i * vocab, *qr = q_w + (uint64_t)i * vocab;
+        bool okp, okq;
+        const double sp = row_sum(pr, &okp);
+        const double sq = row_sum(qr, &okq);
+        if (!okp || !okq || !(sp > 0.0 && sp <= 1.7976931348623157e308) || !(sq > 0.0 && sq <= 1.7976931348623157e308))
+            return finish(i, -1, 3);
+        const int32_t d = drafts.d[i];
+        if (d < 0 || (uint32_t)d >= vocab) return finish(i, -1, 5);
+        const double px = (double)pr[d] / sp, qx = (double)qr[d] / sq;
+        if (!(qx > 0.0 && qx <= 1.7976931348623157e308) || !(px >= 0.0 && px <= 1.7976931348623157e308)) return finish(i, -1, 2);
+        double ratio = px / qx;
+        ratio = ratio > 1.0 ? 1.0 : ratio;
+        const float a = (float)ratio;
+        if (t == 0) {
+            const uint64_t bits = xorshift64star_next(st);
+            s_flag = (double)(bits >> 11) / 9007199254740992.0 < (double)a ? 1 : 0;
+        }
+        __syncthreads();
+        const bool accepted = s_flag != 0;
+        __syncthreads();
+        if (accepted) continue;
+        auto residual = [&](uint32_t j) -> double {
+            const double r = (double)pr[j] / sp - (double)qr[j] / sq;
+            return r > 0.0 ? r : 0.0;
+        };
+        double part = 0.0;
+        for (uint32_t j = lo; j < hi; ++j) part += residual(j);
+        double sr;
+        (void)block_exclusive_scan_fast<double>(part, s_d, &sr);
+        if (!(sr > 0.0 && sr <= 1.7976931348623157e308)) return finish(i, -1, 4);
+        const int32_t tok = draw([&](uint32_t j) -> float { return (float)(residual(j) / sr); });
+        return finish(i, tok, tok < 0 ? 3 : 0);
+    }
+    const float *br = p_w + (uint64_t)k * vocab;
+    bool ok;
+    const double sb = row_sum(br, &ok);
+    if (!ok || !(sb > 0.0 && sb <= 1.7976931348623157e308)) return finish(k, -1, 3);
+    const int32_t tok = draw([&](uint32_t j) -> float { return br[j]; });
+    finish(k, tok, tok < 0 ? 3 : 0);
 }
 
 __global__ void advance_rng_kernel(uint64_t *state, uint32_t draws) {
@@ -467,6 +606,18 @@ void sample_rows(const float *logits, int32_t *tokens, uint64_t *rng_state, uint
     launch_sampler(rows, vocab, s, logits, tokens, (const uint64_t *)rng_state, (RowPolicy *)nullptr, vocab, top_k_mode,
                    temperature, top_k);
     advance_rng_kernel<<<1, 1, 0, s>>>(rng_state, rows);
+}
+
+void sampling_weights(const float *logits, float *weights, int32_t *status, uint32_t rows, uint32_t vocab, int mode,
+                      float temperature, uint32_t top_k, hipStream_t s) {
+    if (rows == 0 || vocab == 0) return;
+    sample_rows_kernel<true><<<rows, kThreads, 0, s>>>(logits, (int32_t *)nullptr, (const uint64_t *)nullptr, (RowPolicy *)nullptr,
+                                                       vocab, mode == 1, temperature, top_k, weights, status, mode == 2);
+}
+
+void speculative_accept(const float *p_weights, const float *q_weights, const DraftTokens &drafts, uint32_t k, uint32_t vocab,
+                        uint64_t *rng_state, int32_t *result, hipStream_t s) {
+    speculative_accept_kernel<<<1, kThreads, 0, s>>>(p_weights, q_weights, drafts, k, vocab, rng_state, result);
 }
 
 void sample_rows_policy(const float *logits, int32_t *tokens, RowPolicy *policy, uint32_t rows, uint32_t vocab, hipStream_t s) {

@@ -214,6 +214,19 @@ struct RowPolicy {
 // advanced by `rows` draws afterwards.  A row with a non-finite logit gets token -1.
 void sample_rows(const float *logits, int32_t *tokens, uint64_t *rng_state, uint32_t rows, uint32_t vocab, int top_k_mode,
                  float temperature, uint32_t top_k, hipStream_t s);
+// The f32 sampling weights of every row instead of a draw (mode 0 temperature, 1 top-k, 2 greedy: one-hot at the
+// first maximum); status[row] = 1 and a NaN row where a logit is not finite, else 0.
+void sampling_weights(const float *logits, float *weights, int32_t *status, uint32_t rows, uint32_t vocab, int mode,
+                      float temperature, uint32_t top_k, hipStream_t s);
+// Acceptance step of sampled speculative decoding for one sequence: p_weights [k + 1, vocab] (target), q_weights
+// [k, vocab] (draft; unused when k == 0), the k draft tokens by value; result[0 .. 2] = accepted drafts, the token
+// that follows them, status.  Draws from, and advances, the generator state.
+constexpr uint32_t kMaxDraftTokens = 32;
+struct DraftTokens {
+    int32_t d[kMaxDraftTokens];
+};
+void speculative_accept(const float *p_weights, const float *q_weights, const DraftTokens &drafts, uint32_t k, uint32_t vocab,
+                        uint64_t *rng_state, int32_t *result, hipStream_t s);
 // The same with one RowPolicy per row (strategy 0 takes the first maximum and draws nothing; otherwise one
 // draw from the row's own state, which is advanced in place).
 void sample_rows_policy(const float *logits, int32_t *tokens, RowPolicy *policy, uint32_t rows, uint32_t vocab, hipStream_t s);

@@ -128,6 +128,12 @@ class Decoder:
         check(lib.fa_decoder_read_logits(self._ops._ctx, self._h, out.ctypes.data_as(capi.f32p)))
         return out
 
+    def logits_buffer(self):
+        """Raw handle of the resident logits [max_batch, vocab] (owned by the decoder)."""
+        h = capi.buf_p()
+        check(lib.fa_decoder_logits_buffer(self._h, C.byref(h)))
+        return h
+
     def seq_lens(self):
         out = np.empty(self.batch, dtype=np.uint32)
         check(lib.fa_decoder_read_seq_lens(self._ops._ctx, self._h, out.ctypes.data_as(capi.u32p)))

@@ -179,25 +179,69 @@ def generate(decoder, input_ids, config):
     return out[0] if want_rank1 else out
 
 
-class Unsupported(ValueError):
-    """What the device path does not offer (the reference does)."""
+class _DeviceAcceptance:
+    """The probabilities of sampled speculative decoding, kept on the device: the f32 weight rows of the target
+    (k + 1) and of the draft (k), one generator for every draw of the call (speculative.rs:438-447), and the
+    acceptance kernel behind ``fa_speculative_accept``.  Only (accepted, token, status) come back to the host."""
+
+    _WHY = {2: "q(x) is not positive, or a probability is not finite", 3: "probability weights are negative, not finite or sum to zero",
+            4: "the residual distribution sums to zero", 5: "a draft token lies outside the vocabulary"}
+
+    def __init__(self, be, config, vocab, k):
+        self.be, self.vocab = be, vocab
+        self.kind, self.temperature, self.top_k = config.strategy.kind, config.temperature, config.top_k or 0
+        self.gen = be.new_generator(config.seed)
+        self.pw, self.qw = be.alloc_uninit((k + 1, vocab)), be.alloc_uninit((k, vocab))
+        self.status, self.result = be.alloc_zeroed((k + 1,), capi.I32), be.alloc_zeroed((4,), capi.I32)
+
+    def close(self):
+        for b in (self.gen, self.pw, self.qw, self.status, self.result):
+            b.free()
+
+    def _raise_unless_ok(self, status, rows):
+        if status == 0:
+            return
+        if status == 3 and self.be.download(self.status)[:rows].any():
+            raise InvalidArgument("generate_speculative: logits hold non-finite values")
+        raise InvalidArgument("generate_speculative: " + self._WHY.get(status, "acceptance failed (status %d)" % status))
+
+    def draw(self, logits, row=0, keep_as_q=None):
+        """One token from row `row` of `logits` (``sample_from`` over ``sampling_weights_f32``); the weights stay
+        behind as draft row `keep_as_q` for the acceptance step when asked."""
+        dst, dst_row = (self.pw, 0) if keep_as_q is None else (self.qw, keep_as_q)
+        self.be.sampling_weights(logits, 1, self.vocab, self.kind, self.temperature, self.top_k, dst, self.status, row, dst_row)
+        _, token, status = self.be.speculative_accept(dst, None, [], self.vocab, self.gen, self.result, p_row=dst_row)
+        self._raise_unless_ok(status, 1)
+        return token
+
+    def verify(self, logits, drafts):
+        """``verify_sampling``: rows 0 .. len(drafts) of `logits` are the verification pass."""
+        rows = len(drafts) + 1
+        self.be.sampling_weights(logits, rows, self.vocab, self.kind, self.temperature, self.top_k, self.pw, self.status)
+        n_acc, token, status = self.be.speculative_accept(self.pw, self.qw, drafts, self.vocab, self.gen, self.result)
+        self._raise_unless_ok(status, rows)
+        return n_acc, token
 
 
 def generate_speculative(target, draft, input_ids, config, k):
-    """``generate_speculative`` (crates/autodiff/src/generate/speculative.rs:334-531), greedy form, on two
-    resident decoders: per round the draft decodes ``k_eff = min(k, remaining - 1)`` tokens, the target
-    consumes the pending token and those drafts in one verification pass (``Decoder.verify``), the longest
-    prefix of drafts that equals the target's own greedy tokens is kept and the target's token at the first
-    disagreement (or after the last draft) is appended.  Both caches are then cut back to the accepted
-    length with ``Decoder.rewind``: paged rows past a sequence's length are dead, so nothing is replayed
-    (the reference restores a snapshot and replays the accepted tokens, kv_rewind.rs:157-215).  One
-    sequence per call, as in the reference.  When the pending token and the drafts fit the decoder's rows
-    (``k + 1 <= min(32, max_batch)``) the verification is one decode step whose rows are the k + 1 positions
-    of the one sequence (the same block table in every row, lengths ctx, ctx + 1, ...: every row appends its
-    own position and attends to its own prefix), which costs about what a single decode step costs; longer
-    look-aheads take the prompt-shape verification pass.  The output equals ``generate(target, ...)``
-    wherever the target's greedy choice is decisive (int32 accumulators are identical in every form,
-    attention sums are associated differently when the rows change).
+    """``generate_speculative`` (crates/autodiff/src/generate/speculative.rs:334-531) on two resident decoders:
+    per round the draft decodes ``k_eff = min(k, remaining - 1)`` tokens, the target consumes the pending token
+    and those drafts in one verification pass, a prefix of the drafts is kept and one more token from the
+    target's own distribution is appended.  Greedy: the longest prefix that equals the target's greedy tokens,
+    then the target's token at the first disagreement (or after the last draft).  Temperature / top-k:
+    standard speculative sampling (draft i is kept with probability min(1, p / q), the first refused one is
+    replaced by a draw from max(0, p - q), a fully accepted round ends with a bonus draw), with one generator
+    seeded from ``config.seed`` for every draw of the call in the reference's order and all probabilities on
+    the device (``fa_sampling_weights`` + ``fa_speculative_accept`` on the decoders' resident logits).
+    Both caches are then cut back to the accepted length with ``Decoder.rewind``: paged rows past a sequence's
+    length are dead, so nothing is replayed (the reference restores a snapshot and replays the accepted
+    tokens, kv_rewind.rs:157-215).  One sequence per call, as in the reference.  When the pending token and
+    the drafts fit the decoder's rows (``k + 1 <= min(32, max_batch)``) the verification is one decode step
+    whose rows are the k + 1 positions of the one sequence (the same block table in every row, lengths ctx,
+    ctx + 1, ...: every row appends its own position and attends to its own prefix), which costs about what a
+    single decode step costs; longer look-aheads take the prompt-shape verification pass.  The greedy output
+    equals ``generate(target, ...)`` wherever the target's greedy choice is decisive (int32 accumulators are
+    identical in every form, attention sums are associated differently when the rows change).
     Returns (tokens, rounds, accepted drafts)."""
     config.validate()
     if not isinstance(k, int) or k < 1:
@@ -211,73 +255,110 @@ def generate_speculative(target, draft, input_ids, config, k):
     if max_length < prompt_len:
         raise InvalidArgument("generate_speculative: max_length (%d) must be at least the prompt length (%d)" % (max_length, prompt_len))
     _check_buffer_bytes(max_length)
-    if config.strategy.kind != GREEDY:
-        raise Unsupported("generate_speculative: only the greedy form runs on the device (sampled acceptance needs both "
-                          "models' probabilities on the host)")
+    sampled = config.strategy.kind != GREEDY
     row = [int(t) for t in ids[0]]
     rounds = accepted = 0
     by_step = k + 1 <= min(32, target.cfg.max_batch)
     target_table = None
+    acc = None
     if max_length > prompt_len:
         if target.cfg.vocab != draft.cfg.vocab:
             raise InvalidArgument("generate_speculative: the models disagree on the vocabulary (%d, %d)" % (draft.cfg.vocab, target.cfg.vocab))
+        vocab = target.cfg.vocab
+        config.validate_top_k_le_vocab(vocab)
+        if sampled and k > 32:
+            raise InvalidArgument("generate_speculative: the sampled form verifies at most 32 drafts per round (got %d)" % k)
         for dec in (target, draft):
             cfg = dec.cfg
             pages = _pages_for(max_length + 1, cfg.block_size)     # the verification pass also writes the last draft
             if pages > cfg.max_blocks_per_seq or pages > cfg.num_blocks:
                 raise InvalidArgument("generate_speculative: %d tokens do not fit the decoder's page pool" % max_length)
-            table = np.full((1, cfg.max_blocks_per_seq), 0xFFFFFFFF, dtype=np.uint32)
-            table[0, :pages] = np.arange(pages, dtype=np.uint32)
-            dec.set_sequences(table, np.zeros(1, np.uint32))
-            dec.set_sampling(GREEDY)
-            dec.prefill(ids.astype(np.int32))
-            if dec is target:
-                target_table = table
-        row.append(int(target.tokens()[0]))
-        while len(row) < max_length:
-            cur, last = len(row), row[-1]
-            remaining = max_length - cur
-            if remaining == 1:
-                target.set_tokens([last])
-                target.step()
-                row.append(int(target.tokens()[0]))
-                break
-            k_eff = min(k, remaining - 1)
-            drafts, x = [], last
-            for _ in range(k_eff):                         # the draft's cache grows by last, d1 .. d_{k_eff - 1}
-                draft.set_tokens([x])
-                draft.step()
-                x = int(draft.tokens()[0])
-                drafts.append(x)
-            if by_step:
-                n = k_eff + 1
-                target.set_sequences(np.repeat(target_table, n, axis=0), np.arange(cur - 1, cur - 1 + n, dtype=np.uint32))
-                target.set_tokens([last] + drafts)
-                target.step()
-                picked = target.tokens()
-                if (picked < 0).any():
+        try:
+            if sampled:
+                acc = _DeviceAcceptance(target._ops, config, vocab, k)
+            for dec in (target, draft):
+                cfg = dec.cfg
+                pages = _pages_for(max_length + 1, cfg.block_size)
+                table = np.full((1, cfg.max_blocks_per_seq), 0xFFFFFFFF, dtype=np.uint32)
+                table[0, :pages] = np.arange(pages, dtype=np.uint32)
+                dec.set_sequences(table, np.zeros(1, np.uint32))
+                dec.set_sampling(GREEDY)                           # the decoders' own picks are not used when sampling
+                dec.prefill(ids.astype(np.int32))
+                if dec is target:
+                    target_table = table
+
+            def pick(dec):
+                """The next token from row 0 of a decoder's logits."""
+                if sampled:
+                    return acc.draw(dec.logits_buffer())
+                tok = int(dec.tokens()[0])
+                if tok < 0:
                     raise InvalidArgument("generate_speculative: logits hold non-finite values")
-            else:
-                picked = target.verify(np.array([[last] + drafts], dtype=np.int32))[0]
-            n_acc = 0
-            while n_acc < k_eff and drafts[n_acc] == picked[n_acc]:
-                n_acc += 1
-            row.extend(drafts[:n_acc])
-            row.append(int(picked[n_acc]))
-            rounds += 1
-            accepted += n_acc
-            if len(row) >= max_length:
-                break
-            keep = cur + n_acc                             # tokens before the new pending one
-            if by_step:
-                target.set_sequences(target_table, np.array([keep], dtype=np.uint32))
-            else:
-                target.rewind([keep])
-            if n_acc == k_eff:
-                draft.set_tokens([x])                      # the draft never consumed its own last token
-                draft.step()
-            else:
-                draft.rewind([keep])
+                return tok
+
+            row.append(pick(target))
+            while len(row) < max_length:
+                cur, last = len(row), row[-1]
+                remaining = max_length - cur
+                if remaining == 1:
+                    target.set_tokens([last])
+                    target.step()
+                    row.append(pick(target))
+                    break
+                k_eff = min(k, remaining - 1)
+                drafts, x = [], last
+                for i in range(k_eff):                         # the draft's cache grows by last, d1 .. d_{k_eff - 1}
+                    draft.set_tokens([x])
+                    draft.step()
+                    x = acc.draw(draft.logits_buffer(), 0, keep_as_q=i) if sampled else pick(draft)
+                    drafts.append(x)
+                picked = staged = None
+                if by_step:
+                    n = k_eff + 1
+                    target.set_sequences(np.repeat(target_table, n, axis=0), np.arange(cur - 1, cur - 1 + n, dtype=np.uint32))
+                    target.set_tokens([last] + drafts)
+                    target.step()
+                    if sampled:
+                        logits = target.logits_buffer()
+                    else:
+                        picked = target.tokens()
+                        if (picked < 0).any():
+                            raise InvalidArgument("generate_speculative: logits hold non-finite values")
+                elif sampled:
+                    _, host_logits = target.verify(np.array([[last] + drafts], dtype=np.int32), want_logits=True)
+                    logits = staged = target._ops.upload(host_logits[0])
+                else:
+                    picked = target.verify(np.array([[last] + drafts], dtype=np.int32))[0]
+                if sampled:
+                    try:
+                        n_acc, correction = acc.verify(logits, drafts)
+                    finally:
+                        if staged is not None:
+                            staged.free()
+                else:
+                    n_acc = 0
+                    while n_acc < k_eff and drafts[n_acc] == picked[n_acc]:
+                        n_acc += 1
+                    correction = int(picked[n_acc])
+                row.extend(drafts[:n_acc])
+                row.append(correction)
+                rounds += 1
+                accepted += n_acc
+                if len(row) >= max_length:
+                    break
+                keep = cur + n_acc                             # tokens before the new pending one
+                if by_step:
+                    target.set_sequences(target_table, np.array([keep], dtype=np.uint32))
+                else:
+                    target.rewind([keep])
+                if n_acc == k_eff:
+                    draft.set_tokens([x])                      # the draft never consumed its own last token
+                    draft.step()
+                else:
+                    draft.rewind([keep])
+        finally:
+            if acc is not None:
+                acc.close()
     out = np.array(row[:max_length], dtype=np.int32)
     return (out if want_rank1 else out[None, :]), rounds, accepted
 

@@ -256,6 +256,27 @@ fa_status fa_sample_rows(fa_context *ctx, const fa_buffer *logits, uint64_t rows
 fa_status fa_rng_seed(fa_context *ctx, fa_buffer *rng, uint64_t seed);
 /* The same rule as a plain host function: the generator state a seed starts. */
 fa_status fa_rng_state_from_seed(uint64_t seed, uint64_t *state);
+/* sampling_weights_f32 (crates/autodiff/src/generate/mod.rs:432-452) of `rows` rows of logits that start
+ * `logits_offset` elements into `logits`: the f32 weights the sampler draws from, stored from `weights_offset` on
+ * (greedy: one-hot at the first maximum).  status (I32 [rows]): 0, or 1 where a logit is not finite (that row of
+ * weights is NaN; the reference rejects the step there). */
+fa_status fa_sampling_weights(fa_context *ctx, const fa_buffer *logits, uint64_t logits_offset, uint64_t rows, uint64_t vocab,
+                              fa_sampling strategy, float temperature, uint64_t top_k, fa_buffer *weights,
+                              uint64_t weights_offset, fa_buffer *status);
+/* Acceptance step of sampled speculative decoding for one sequence, on the device (verify_sampling,
+ * crates/autodiff/src/generate/speculative.rs:246-279, with normalize_f64 / acceptance_prob_f32 /
+ * residual_weights_f32 / accept_draw / sample_from, :111-189): p_weights holds the target's k + 1 weight rows of
+ * the verification pass, q_weights the k rows every draft was drawn from, drafts the k draft tokens (host array,
+ * k <= 32).  Draft i is accepted when the next uniform of `rng` is below (f32) min(1, p(d) / q(d)); at the first
+ * refusal one token is drawn from max(0, p - q) and the call stops; when every draft is accepted one token is
+ * drawn from row k of p_weights.  k == 0 is one multinomial draw from row 0 of p_weights (sample_from).
+ * result (I32 [4]): accepted drafts, the token that follows them, status (0 ok; 2 q(d) <= 0 or a probability not
+ * finite; 3 a weight row negative, not finite or summing to zero; 4 the residual sums to zero), unused.  The
+ * generator advances by the draws the call consumed.  Nothing is read back: download `result`. */
+fa_status fa_speculative_accept(fa_context *ctx, const fa_buffer *p_weights, uint64_t p_offset, const fa_buffer *q_weights,
+                                uint64_t q_offset, const int32_t *drafts, uint64_t k, uint64_t vocab, fa_buffer *rng,
+                                fa_buffer *result);
+
 /* One row of a per-row sampling table: every row is a request with a
  * GenerateConfig and a Generator of its own, as in the reference's continuous
  * batching scheduler (crates/autodiff/src/generate/scheduler.rs:160-211: each
@@ -530,6 +551,10 @@ fa_status fa_decoder_rewind(fa_context *ctx, fa_decoder *dec, const uint32_t *se
 fa_status fa_decoder_read_tokens(fa_context *ctx, fa_decoder *dec, int32_t *tokens);
 fa_status fa_decoder_read_logits(fa_context *ctx, fa_decoder *dec, float *logits);
 fa_status fa_decoder_read_seq_lens(fa_context *ctx, fa_decoder *dec, uint32_t *seq_lens);
+/* The decoder's resident logits, f32 [max_batch, vocab] (rows of the last step, prompt pass or verification by
+ * step; not a copy, do not free): what fa_sampling_weights reads when the sampled form of speculative decoding
+ * (speculative.rs:334-531) keeps the probabilities on the device. */
+fa_status fa_decoder_logits_buffer(fa_decoder *dec, fa_buffer **out);
 
 #ifdef __cplusplus
 }

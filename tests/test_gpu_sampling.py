@@ -142,3 +142,119 @@ def test_per_row_policies_draw_from_their_own_generators(rows, vocab, kind):
         assert state == refs[r].state
         if strategy == fa.SAMPLE_GREEDY:
             assert state == os_.Generator(seed).state
+
+
+# ---------------------------------------------------------------- sampled speculative decoding
+def _ulp_apart(a, b):
+    ia, ib = a.view(np.int32).astype(np.int64), b.view(np.int32).astype(np.int64)
+    return np.abs(ia - ib)
+
+
+@pytest.mark.parametrize("rows,vocab,kind", [(1, 17, "normal"), (5, 1000, "ties"), (6, 32000, "normal"), (2, 50257, "peaked"),
+                                             (3, 129, "flat"), (2, 1, "normal")])
+def test_sampling_weights_equal_the_oracle(rows, vocab, kind):
+    """fa_sampling_weights against sampling_weights_f32 of the oracle: the same f32 weights (a weight may differ
+    by one unit in the last place where the block-wide f64 sum of exponentials rounds differently from the
+    sequential one; zeros and the kept set of a top-k row are exact), at an offset into a larger buffer."""
+    fa = _fa()
+    be = ops()
+    rng = np.random.default_rng(vocab + rows)
+    x = _logits(rng, rows + 1, vocab, kind)
+    dx = be.upload(x)
+    w = be.alloc_zeroed((rows + 2, vocab))
+    st = be.alloc_zeroed((rows,), fa.capi.I32)
+    for strategy, temperature, k in ((fa.SAMPLE_TEMPERATURE, 1.0, 0), (fa.SAMPLE_TEMPERATURE, 0.6, 0), (fa.SAMPLE_TOP_K, 1.0, 1),
+                                     (fa.SAMPLE_TOP_K, 0.8, min(50, vocab)), (fa.SAMPLE_TOP_K, 1.3, vocab), (fa.SAMPLE_GREEDY, 1.0, 0)):
+        be.sampling_weights(dx, rows, vocab, strategy, temperature, k, w, st, logits_row=1, weights_row=2)
+        got = be.download(w)
+        assert not got[:2].any() and not be.download(st).any()
+        want = np.stack([os_.sampling_weights_f32(x[1 + r], strategy, temperature, k or None) for r in range(rows)])
+        assert np.array_equal(got[2:] == 0, want == 0), (strategy, temperature, k)
+        apart = _ulp_apart(got[2:], want)
+        assert apart.max() <= 1 and (apart != 0).sum() <= max(1, int(1e-4 * want.size)), (strategy, temperature, k, apart.max())
+    bad = x.copy()
+    bad[rows, vocab // 2] = np.nan                           # the last of the rows that are read
+    be.sampling_weights(be.upload(bad), rows, vocab, fa.SAMPLE_TEMPERATURE, 1.0, 0, w, st, logits_row=1, weights_row=2)
+    status, got = be.download(st), be.download(w)
+    assert status[rows - 1] == 1 and np.isnan(got[rows + 1]).all()
+    assert not status[:rows - 1].any() and np.isfinite(got[2:rows + 1]).all()
+    with pytest.raises(fa.ShapeMismatch):
+        be.sampling_weights(dx, rows + 1, vocab, fa.SAMPLE_TEMPERATURE, 1.0, 0, w, st, logits_row=1)      # past the logits
+    with pytest.raises(fa.InvalidArgument):
+        be.sampling_weights(dx, rows, vocab, fa.SAMPLE_TOP_K, 1.0, vocab + 1, w, st)
+
+
+ACCEPT_CASES = [(17, 1, 0.3), (1000, 4, 0.5), (32000, 3, 0.2), (50257, 7, 1.0), (129, 32, 0.1), (2, 2, 2.0), (1, 3, 0.0)]
+
+
+@pytest.mark.parametrize("vocab,k,spread", ACCEPT_CASES, ids=["v%d_k%d" % c[:2] for c in ACCEPT_CASES])
+def test_speculative_acceptance_equals_the_oracle(vocab, k, spread):
+    """fa_speculative_accept against verify_sampling of the oracle over many rounds with one running generator:
+    drafts drawn on the device from the draft's weights (k = 0 calls), then the acceptance step; accepted count,
+    token and generator state must all equal the oracle's, for drafts close to and far from the target."""
+    fa = _fa()
+    be = ops()
+    rng = np.random.default_rng(vocab * 31 + k)
+    pw, qw = be.alloc_uninit((k + 1, vocab)), be.alloc_uninit((k, vocab))
+    st, res = be.alloc_zeroed((k + 1,), fa.capi.I32), be.alloc_zeroed((4,), fa.capi.I32)
+    seen = np.zeros(k + 1, np.int64)
+    for strategy, temperature, top_k, seed in ((fa.SAMPLE_TEMPERATURE, 0.8, 0, 11), (fa.SAMPLE_TOP_K, 1.0, min(5, vocab), 7),
+                                               (fa.SAMPLE_TEMPERATURE, 1.5, 0, 0)):
+        gen, ref = be.new_generator(seed), os_.Generator(seed)
+        for rnd in range(6 if vocab > 5000 else 12):
+            lp = _logits(rng, k + 1, vocab, "normal")
+            lq = (lp[:k] + spread * rng.standard_normal((k, vocab))).astype(np.float32)
+            dq = be.upload(lq)
+            drafts, q_ws = [], []
+            for i in range(k):
+                be.sampling_weights(dq, 1, vocab, strategy, temperature, top_k, qw, st, logits_row=i, weights_row=i)
+                n0, tok, status = be.speculative_accept(qw, None, [], vocab, gen, res, p_row=i)
+                w = os_.sampling_weights_f32(lq[i], strategy, temperature, top_k or None)
+                assert (n0, status) == (0, 0) and tok == os_.sample_from(ref, w), (rnd, i)
+                drafts.append(tok)
+                q_ws.append(w)
+            be.sampling_weights(be.upload(lp), k + 1, vocab, strategy, temperature, top_k, pw, st)
+            got = be.speculative_accept(pw, qw, drafts, vocab, gen, res)
+            want = os_.verify_sampling(ref, lp, drafts, q_ws, strategy, temperature, top_k or None)
+            assert got == (want[0], want[1], 0), (strategy, rnd, got, want)
+            seen[want[0]] += 1
+            state = be.download(gen)
+            assert (int(state[1]) << 32 | int(state[0])) == ref.state
+            dq.free()
+        gen.free()
+    print("SPECULATIVE_ACCEPT\tvocab %d k %d spread %.1f\taccepted-count histogram %s" % (vocab, k, spread, seen.tolist()), flush=True)
+    if vocab > 1 and k > 1 and spread > 0:
+        assert seen[0] > 0 and seen[1:].sum() > 0            # both outcomes were exercised
+
+
+def test_speculative_acceptance_fails_closed():
+    """speculative.rs:1117-1150: a draft the draft model could not have drawn (q(d) = 0), weights that are not
+    finite, and arguments outside the contract."""
+    fa = _fa()
+    be = ops()
+    vocab = 64
+    rng = np.random.default_rng(2)
+    lp = _logits(rng, 2, vocab, "normal")
+    lq = _logits(rng, 1, vocab, "normal")
+    pw, qw = be.alloc_uninit((2, vocab)), be.alloc_uninit((1, vocab))
+    st, res, gen = be.alloc_zeroed((2,), fa.capi.I32), be.alloc_zeroed((4,), fa.capi.I32), be.new_generator(3)
+    be.sampling_weights(be.upload(lp), 2, vocab, fa.SAMPLE_TOP_K, 1.0, 4, pw, st)
+    be.sampling_weights(be.upload(lq), 1, vocab, fa.SAMPLE_TOP_K, 1.0, 4, qw, st)
+    outside = int(np.argmin(lq[0]))                          # not among the draft's four kept tokens: q = 0
+    before = be.download(gen).copy()
+    n_acc, tok, status = be.speculative_accept(pw, qw, [outside], vocab, gen, res)
+    assert (n_acc, tok, status) == (0, -1, 2) and np.array_equal(be.download(gen), before)   # refused before any draw
+    with pytest.raises(os_.SamplingError):
+        os_.verify_sampling(os_.Generator(3), lp, [outside], [os_.sampling_weights_f32(lq[0], os_.TOP_K, 1.0, 4)], os_.TOP_K, 1.0, 4)
+    bad = lp.copy()
+    bad[0, 5] = np.inf
+    be.sampling_weights(be.upload(bad), 2, vocab, fa.SAMPLE_TEMPERATURE, 1.0, 0, pw, st)
+    assert be.download(st).tolist() == [1, 0]
+    assert be.speculative_accept(pw, qw, [int(np.argmax(lq[0]))], vocab, gen, res)[2] == 3
+    for drafts in ([vocab], [-1]):
+        with pytest.raises(fa.InvalidArgument):
+            be.speculative_accept(pw, qw, drafts, vocab, gen, res)
+    with pytest.raises(fa.ShapeMismatch):
+        be.speculative_accept(pw, qw, [1, 2], vocab, gen, res)                                # q holds one row only
+    with pytest.raises(fa.InvalidArgument):
+        be.speculative_accept(pw, qw, [0] * 33, vocab, gen, res)

@@ -270,6 +270,112 @@ def test_speculative_generation_equals_the_target_generating_alone(rows):
         d.close()
 
 
+def _feeding(dec):
+    """Wraps a decoder so that every prompt pass, step and verification pass leaves (kind, token ids fed, logits)."""
+    import fandhe_ai_amd as fa
+
+    class Feeding(fa.Decoder):
+        def set_tokens(self, tokens):
+            self.fed = [int(t) for t in tokens]
+            super().set_tokens(tokens)
+
+        def prefill(self, prompt):
+            super().prefill(prompt)
+            self.trace.append(("prefill", [int(t) for t in np.asarray(prompt)[0]], self.logits()[:1].copy()))
+
+        def step(self, use_graph=True):
+            super().step(use_graph)
+            self.trace.append(("step", list(self.fed), self.logits()[:len(self.fed)].copy()))
+
+        def verify(self, tokens, want_logits=False):
+            picked, logits = super().verify(tokens, want_logits=True)
+            self.trace.append(("step", [int(t) for t in np.asarray(tokens)[0]], logits[0].copy()))
+            return (picked, logits) if want_logits else picked
+
+    dec.__class__ = Feeding
+    dec.trace, dec.fed = [], []
+    return dec
+
+
+class _Replay:
+    """A model of the oracle's speculative loop that hands out the logits the device produced, call by call, and
+    insists on being fed what the device was fed.  The oracle cuts a cache back by restoring a snapshot and
+    replaying the accepted tokens (as the reference does); the device only shortens the sequence, so the one
+    forward call after a ``truncate`` has no counterpart in the trace."""
+
+    def __init__(self, trace):
+        self.trace, self.len, self.replaying = list(trace), 0, False
+
+    def forward_step(self, ids):
+        ids = [int(t) for t in ids]
+        self.len += len(ids)
+        if self.replaying:
+            self.replaying = False
+            return np.zeros((len(ids), VOCAB), np.float32)
+        kind, fed, logits = self.trace.pop(0)
+        assert fed == ids, (kind, fed, ids)
+        if kind == "prefill":
+            out = np.zeros((len(ids), VOCAB), np.float32)
+            out[-1] = logits[0]
+            return out
+        return logits
+
+    def seq_len(self):
+        return self.len
+
+    def truncate(self, n):
+        assert n <= self.len
+        self.len, self.replaying = n, True
+
+
+@pytest.mark.parametrize("rows", [1, 8], ids=["verify-by-prompt-pass", "verify-by-decode-step"])
+def test_sampled_speculative_generation_takes_the_oracle_decisions(rows):
+    """Temperature / top-k speculative decoding on the device (weights, acceptance, residual and bonus draws in
+    fa_sampling_weights / fa_speculative_accept; rounds, rewinds and the draft's catch-up step in
+    scheduler.generate_speculative) against the oracle's restatement of the reference loop run on the very
+    logits the two decoders produced: the same tokens, the same sequence of forward calls with the same inputs."""
+    import fandhe_ai_amd as fa
+    from fandhe_ai_amd.scheduler import SamplingStrategy as S, generate_speculative
+    geometry = dict(max_blocks_per_seq=8, num_blocks=8, max_batch=rows)
+    target = _feeding(_decoder(**geometry))
+    twin = _feeding(_decoder(**geometry))
+    other_ckpt = st_save(_checkpoint(77, 1, D, HEADS, KV, F, VOCAB))
+    other, store = fa.safetensors_io.load_decoder(ops(), other_ckpt, 1, HEADS, KV, **geometry)
+    store.free()
+    other = _feeding(other)
+    rng = np.random.default_rng(9)
+    drafted = {"twin": [0, 0], "other": [0, 0]}
+    for plen, max_length, k, strategy, seed in ((5, 40, 4, S.Temperature(0.8), 11), (33, 60, 3, S.TopK(5), 7), (1, 20, 7, S.Temperature(1.4), 0),
+                                                (12, 14, 2, S.TopK(40), 3), (3, 4, 5, S.Temperature(1.0), 5), (6, 30, 1, S.TopK(2), 2 ** 63 + 1)):
+        prompt = rng.integers(0, VOCAB, plen).astype(np.int32)
+        cfg = _cfg(max_length, strategy, seed)
+        for draft, name in ((twin, "twin"), (other, "other")):
+            target.trace, draft.trace = [], []
+            got, rounds, accepted = generate_speculative(target, draft, prompt, cfg, k)
+            assert got.shape == (max_length,) and np.array_equal(got[:plen], prompt)
+            t_model, d_model = _Replay(target.trace), _Replay(draft.trace)
+            want = osamp.generate_speculative(t_model, d_model, prompt, max_length, strategy.kind, cfg.temperature, cfg.top_k,
+                                              seed, k)
+            assert got.tolist() == want, (name, plen, max_length, k, strategy)
+            assert not t_model.trace and not d_model.trace               # every device call was one the oracle makes
+            drafted[name][0] += accepted
+            drafted[name][1] += sum(len(fed) - 1 for kind, fed, _ in target.trace if kind == "step" and len(fed) > 1)
+            again, r2, a2 = generate_speculative(target, draft, prompt, cfg, k)        # speculative.rs:1041-1062
+            assert np.array_equal(again, got) and (r2, a2) == (rounds, accepted)
+            print("SPECULATIVE_SAMPLED\t%s\t%s\tprompt %d, %d new tokens, k %d: %d rounds, %d drafts accepted"
+                  % (name, strategy, plen, max_length - plen, k, rounds, accepted), flush=True)
+    # a draft with the target's own weights is accepted almost always (its logits differ only by the rounding of
+    # another batch shape); an unrelated one-layer draft is refused often
+    assert drafted["twin"][0] >= 0.9 * drafted["twin"][1] and drafted["other"][0] < 0.9 * drafted["other"][1], drafted
+    # speculative.rs:1097-1115: top-k 1 draws from one-hot weights and is the greedy sequence
+    prompt = rng.integers(0, VOCAB, 7).astype(np.int32)
+    greedy, _, _ = generate_speculative(target, other, prompt, _cfg(30, S.Greedy(), 0), 3)
+    top1, _, _ = generate_speculative(target, other, prompt, _cfg(30, S.TopK(1), 9), 3)
+    assert np.array_equal(greedy, top1)
+    for d in (target, twin, other):
+        d.close()
+
+
 def test_padded_prompt_pass_leaves_every_row_as_its_own_prompt_pass_would():
     """Three prompts of different lengths in one padded pass against the same prompts ingested one by one:
     logits of every row's last prompt token within the chained-step bar (the rows of a GEMM and the ranges of

@@ -14,7 +14,7 @@ import sampling as osamp  # noqa: E402
 import fandhe_ai_amd as fa  # noqa: E402
 from fandhe_ai_amd import capi  # noqa: E402
 from fandhe_ai_amd.scheduler import (BatchScheduler, GenerateConfig, InvalidArgument, PageAllocator, RankMismatch,  # noqa: E402
-                                     SamplingStrategy, SchedulerLimits, Unsupported, generate, generate_speculative)
+                                     SamplingStrategy, SchedulerLimits, generate, generate_speculative)
 
 VOCAB, BLOCK = 11, 16
 
@@ -373,8 +373,10 @@ def test_speculative_argument_errors():
         generate_speculative(T(), D(), [1, 2, 3], cfg(2, greedy, 0), 2)
     with pytest.raises(RankMismatch):
         generate_speculative(T(), D(), np.zeros((1, 1, 2), np.int32), cfg(4, greedy, 0), 2)
-    with pytest.raises(Unsupported):
-        generate_speculative(T(), D(), [1], cfg(4, SamplingStrategy.TopK(2), 0), 2)
+    with pytest.raises(InvalidArgument):                   # the sampled form: k beyond what one acceptance call takes
+        generate_speculative(T(), D(), [1], cfg(4, SamplingStrategy.TopK(2), 0), 33)
+    with pytest.raises(InvalidArgument):                   # speculative.rs:1117-1131: top-k beyond the vocabulary
+        generate_speculative(T(), D(), [1], cfg(4, SamplingStrategy.TopK(VOCAB + 1), 0), 2)
     with pytest.raises(InvalidArgument):                   # a sequence longer than the page table of one model
         generate_speculative(T(), D(max_blocks_per_seq=1), [1], cfg(40, greedy, 0), 2)
 
