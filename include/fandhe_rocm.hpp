@@ -13,7 +13,7 @@
 //   SchedulerLimits, PageAllocator, BatchScheduler
 //                                  crates/autodiff/src/generate/scheduler.rs:75-127, 395-720;
 //                                  crates/autodiff/src/nn/paged_kv.rs:147-191 (allocation order)
-//   generate_speculative           crates/autodiff/src/generate/speculative.rs:334-531 (greedy form)
+//   generate_speculative           crates/autodiff/src/generate/speculative.rs:334-531 (greedy and sampled forms)
 //   BlockTable, PagedKvCache       crates/autodiff/src/nn/paged_kv.rs:147-363, paged_kv_device.rs:67-372
 //
 // Header only, C++17, no dependency besides the C header; every device call goes through the C ABI, so
@@ -28,6 +28,7 @@
 #include <set>
 #include <stdexcept>
 #include <string>
+#include <tuple>
 #include <utility>
 #include <vector>
 
@@ -44,11 +45,6 @@ class BackendError : public std::runtime_error {
 };
 // AutodiffError::InvalidArgument: a request the host layer rejects before anything is queued.
 class InvalidArgument : public std::invalid_argument {
-  public:
-    using std::invalid_argument::invalid_argument;
-};
-// What the device path does not offer although the reference does.
-class Unsupported : public std::invalid_argument {
   public:
     using std::invalid_argument::invalid_argument;
 };
@@ -463,6 +459,13 @@ class Decoder {
         check(fa_decoder_read_seq_lens(ctx_.handle(), h_, out.data()));
         return out;
     }
+    // the resident logits [max_batch, vocab] (owned by the decoder)
+    fa_buffer *logits_buffer() const {
+        fa_buffer *b = nullptr;
+        check(fa_decoder_logits_buffer(h_, &b));
+        return b;
+    }
+    const Context &context() const { return ctx_; }
 
   private:
     const Context &ctx_;
@@ -580,15 +583,75 @@ std::vector<std::vector<int32_t>> generate(DecoderT &decoder, const std::vector<
     return out;
 }
 
-// generate_speculative (crates/autodiff/src/generate/speculative.rs:334-531), greedy form, on two resident
-// decoders: per round the draft decodes k_eff = min(k, remaining - 1) tokens, the target consumes the pending
-// token and those drafts in one verification, the longest prefix of drafts that equals the target's own greedy
-// tokens is kept and the target's token at the first disagreement (or after the last draft) is appended.  Both
-// caches are then cut back to the accepted length: paged rows past a sequence's length are dead, so nothing is
-// replayed (the reference restores a snapshot and replays, kv_rewind.rs:157-215).  One sequence per call.  When
-// the pending token and the drafts fit the decoder's rows (k + 1 <= min(32, max_batch)) the verification is one
-// decode step whose rows are the k + 1 positions of the one sequence (the same block table in every row, lengths
-// ctx, ctx + 1, ...); longer look-aheads take the prompt-shape verification pass.
+namespace detail {
+// The probabilities of sampled speculative decoding, kept on the device: the f32 weight rows of the target
+// (k + 1) and of the draft (k), one generator for every draw of the call (speculative.rs:438-447) and the
+// acceptance kernel behind fa_speculative_accept.  Only (accepted, token, status) come back to the host.
+class DeviceAcceptance {
+  public:
+    DeviceAcceptance(const Context &ctx, const GenerateConfig &config, uint64_t vocab, uint64_t k)
+        : ctx_(ctx), vocab_(vocab), kind_(config.strategy.kind), temperature_(config.temperature), top_k_(config.top_k.value_or(0)),
+          gen_(Buffer::alloc_zeroed(ctx, FA_U32, 2)), pw_(Buffer::alloc_uninit(ctx, FA_F32, (k + 1) * vocab)),
+          qw_(Buffer::alloc_uninit(ctx, FA_F32, k * vocab)), status_(Buffer::alloc_zeroed(ctx, FA_I32, k + 1)),
+          result_(Buffer::alloc_zeroed(ctx, FA_I32, 4)) {
+        check(fa_rng_seed(ctx.handle(), gen_.handle(), config.seed));
+    }
+    // one token from row `row` of `logits` (sample_from over sampling_weights_f32); the weights stay behind as
+    // draft row keep_as_q for the acceptance step when keep_as_q >= 0
+    int32_t draw(const fa_buffer *logits, uint64_t row, int64_t keep_as_q = -1) {
+        Buffer &dst = keep_as_q < 0 ? pw_ : qw_;
+        const uint64_t dst_row = keep_as_q < 0 ? 0 : (uint64_t)keep_as_q;
+        check(fa_sampling_weights(ctx_.handle(), logits, row * vocab_, 1, vocab_, kind_, temperature_, top_k_, dst.handle(),
+                                  dst_row * vocab_, status_.handle()));
+        check(fa_speculative_accept(ctx_.handle(), dst.handle(), dst_row * vocab_, nullptr, 0, nullptr, 0, vocab_, gen_.handle(),
+                                    result_.handle()));
+        return finish(1).second;
+    }
+    // verify_sampling: rows 0 .. drafts.size() of `logits` are the verification pass
+    std::pair<uint64_t, int32_t> verify(const fa_buffer *logits, const std::vector<int32_t> &drafts) {
+        const uint64_t rows = drafts.size() + 1;
+        check(fa_sampling_weights(ctx_.handle(), logits, 0, rows, vocab_, kind_, temperature_, top_k_, pw_.handle(), 0, status_.handle()));
+        check(fa_speculative_accept(ctx_.handle(), pw_.handle(), 0, qw_.handle(), 0, drafts.data(), drafts.size(), vocab_, gen_.handle(),
+                                    result_.handle()));
+        return finish(rows);
+    }
+
+  private:
+    std::pair<uint64_t, int32_t> finish(uint64_t rows) {
+        const std::vector<int32_t> r = result_.download<int32_t>();
+        if (r[2] == 0) return {(uint64_t)r[0], r[1]};
+        if (r[2] == 3) {
+            const std::vector<int32_t> st = status_.download<int32_t>(0, rows);
+            if (std::any_of(st.begin(), st.end(), [](int32_t v) { return v != 0; }))
+                throw InvalidArgument("generate_speculative: logits hold non-finite values");
+        }
+        static const char *why[] = {"", "", "q(x) is not positive, or a probability is not finite",
+                                    "probability weights are negative, not finite or sum to zero", "the residual distribution sums to zero",
+                                    "a draft token lies outside the vocabulary"};
+        throw InvalidArgument(std::string("generate_speculative: ") + (r[2] >= 2 && r[2] <= 5 ? why[r[2]] : "acceptance failed"));
+    }
+    const Context &ctx_;
+    uint64_t vocab_;
+    fa_sampling kind_;
+    float temperature_;
+    uint64_t top_k_;
+    Buffer gen_, pw_, qw_, status_, result_;
+};
+}  // namespace detail
+
+// generate_speculative (crates/autodiff/src/generate/speculative.rs:334-531) on two resident decoders: per round
+// the draft decodes k_eff = min(k, remaining - 1) tokens, the target consumes the pending token and those drafts
+// in one verification, a prefix of the drafts is kept and one more token from the target's own distribution is
+// appended.  Greedy: the longest prefix that equals the target's greedy tokens, then the target's token at the
+// first disagreement (or after the last draft).  Temperature / top-k: standard speculative sampling (draft i is
+// kept with probability min(1, p / q), the first refused one is replaced by a draw from max(0, p - q), a fully
+// accepted round ends with a bonus draw) with one generator seeded from config.seed for every draw of the call in
+// the reference's order and all probabilities on the device (detail::DeviceAcceptance).  Both caches are then cut
+// back to the accepted length: paged rows past a sequence's length are dead, so nothing is replayed (the
+// reference restores a snapshot and replays, kv_rewind.rs:157-215).  One sequence per call.  When the pending
+// token and the drafts fit the decoder's rows (k + 1 <= min(32, max_batch)) the verification is one decode step
+// whose rows are the k + 1 positions of the one sequence (the same block table in every row, lengths ctx,
+// ctx + 1, ...); longer look-aheads take the prompt-shape verification pass.
 struct SpeculativeOutput {
     std::vector<int32_t> tokens;
     uint64_t rounds = 0, accepted = 0;
@@ -602,29 +665,42 @@ SpeculativeOutput generate_speculative(DecoderT &target, DecoderT &draft, const 
     const uint64_t max_length = config.max_length, prompt_len = input_ids.size();
     if (max_length < prompt_len) throw InvalidArgument("generate_speculative: max_length must be at least the prompt length");
     detail::check_output_bytes(max_length);
-    if (config.strategy.kind != FA_SAMPLE_GREEDY)
-        throw Unsupported("generate_speculative: only the greedy form runs on the device (sampled acceptance needs both models' "
-                          "probabilities on the host)");
+    const bool sampled = config.strategy.kind != FA_SAMPLE_GREEDY;
     SpeculativeOutput out;
     std::vector<int32_t> &row = out.tokens;
     row = input_ids;
     if (max_length == prompt_len) return out;
     if (target.config().vocab != draft.config().vocab) throw InvalidArgument("generate_speculative: the models disagree on the vocabulary");
+    const uint64_t vocab = target.config().vocab;
+    config.validate_top_k_le_vocab(vocab);
+    if (sampled && k > 32) throw InvalidArgument("generate_speculative: the sampled form verifies at most 32 drafts per round");
     const bool by_step = k + 1 <= std::min<uint64_t>(32, target.config().max_batch);
-    std::vector<uint32_t> target_table;
     for (DecoderT *dec : {&target, &draft}) {
         const auto &cfg = dec->config();
         const uint64_t pages = detail::pages_for(max_length + 1, cfg.block_size);   // the verification also writes the last draft
         if (pages > cfg.max_blocks_per_seq || pages > cfg.num_blocks)
             throw InvalidArgument("generate_speculative: the tokens do not fit the decoder's page pool");
+    }
+    std::optional<detail::DeviceAcceptance> acc;
+    if (sampled) acc.emplace(target.context(), config, vocab, k);
+    std::vector<uint32_t> target_table;
+    for (DecoderT *dec : {&target, &draft}) {
+        const auto &cfg = dec->config();
+        const uint64_t pages = detail::pages_for(max_length + 1, cfg.block_size);
         std::vector<uint32_t> table(cfg.max_blocks_per_seq, UINT32_MAX);
         for (uint64_t p = 0; p < pages; ++p) table[p] = (uint32_t)p;
         dec->set_sequences(table, {0});
-        dec->set_sampling(FA_SAMPLE_GREEDY, 1.0f, 0, 0);
+        dec->set_sampling(FA_SAMPLE_GREEDY, 1.0f, 0, 0);          // the decoders' own picks are not used when sampling
         dec->prefill(input_ids, (uint32_t)prompt_len);
         if (dec == &target) target_table = table;
     }
-    row.push_back(target.tokens()[0]);
+    auto pick = [&](DecoderT &dec) -> int32_t {                   // the next token from row 0 of a decoder's logits
+        if (sampled) return acc->draw(dec.logits_buffer(), 0);
+        const int32_t tok = dec.tokens()[0];
+        if (tok < 0) throw InvalidArgument("generate_speculative: logits hold non-finite values");
+        return tok;
+    };
+    row.push_back(pick(target));
     while (row.size() < max_length) {
         const uint64_t cur = row.size();
         const int32_t last = row.back();
@@ -632,7 +708,7 @@ SpeculativeOutput generate_speculative(DecoderT &target, DecoderT &draft, const 
         if (remaining == 1) {
             target.set_tokens({last});
             target.step();
-            row.push_back(target.tokens()[0]);
+            row.push_back(pick(target));
             break;
         }
         const uint64_t k_eff = std::min(k, remaining - 1);
@@ -641,12 +717,14 @@ SpeculativeOutput generate_speculative(DecoderT &target, DecoderT &draft, const 
         for (uint64_t i = 0; i < k_eff; ++i) {                    // the draft's cache grows by last, d1 .. d_{k_eff - 1}
             draft.set_tokens({x});
             draft.step();
-            x = draft.tokens()[0];
+            x = sampled ? acc->draw(draft.logits_buffer(), 0, (int64_t)i) : pick(draft);
             drafts.push_back(x);
         }
         std::vector<int32_t> fed{last};
         fed.insert(fed.end(), drafts.begin(), drafts.end());
         std::vector<int32_t> picked;
+        uint64_t n_acc = 0;
+        int32_t correction = 0;
         if (by_step) {
             const uint64_t n = k_eff + 1;
             std::vector<uint32_t> tables, lens;
@@ -657,16 +735,27 @@ SpeculativeOutput generate_speculative(DecoderT &target, DecoderT &draft, const 
             target.set_sequences(tables, lens);
             target.set_tokens(fed);
             target.step();
-            picked = target.tokens();
-            for (int32_t t : picked)
-                if (t < 0) throw InvalidArgument("generate_speculative: logits hold non-finite values");
+            if (sampled) {
+                std::tie(n_acc, correction) = acc->verify(target.logits_buffer(), drafts);
+            } else {
+                picked = target.tokens();
+                for (int32_t t : picked)
+                    if (t < 0) throw InvalidArgument("generate_speculative: logits hold non-finite values");
+            }
+        } else if (sampled) {
+            std::vector<float> host_logits;
+            (void)target.verify(fed, (uint32_t)fed.size(), &host_logits);
+            const Buffer staged = Buffer::upload(target.context(), host_logits);
+            std::tie(n_acc, correction) = acc->verify(staged.handle(), drafts);
         } else {
             picked = target.verify(fed, (uint32_t)fed.size());
         }
-        uint64_t n_acc = 0;
-        while (n_acc < k_eff && drafts[n_acc] == picked[n_acc]) ++n_acc;
+        if (!sampled) {
+            while (n_acc < k_eff && drafts[n_acc] == picked[n_acc]) ++n_acc;
+            correction = picked[n_acc];
+        }
         row.insert(row.end(), drafts.begin(), drafts.begin() + n_acc);
-        row.push_back(picked[n_acc]);
+        row.push_back(correction);
         out.rounds += 1;
         out.accepted += n_acc;
         if (row.size() >= max_length) break;

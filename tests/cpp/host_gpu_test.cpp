@@ -153,6 +153,19 @@ int main(int argc, char **argv) {
             std::printf("], \"rounds\": %llu, \"accepted\": %llu},\n", (unsigned long long)so.rounds, (unsigned long long)so.accepted);
         }
         print_rows("generate_greedy_24", generate(dec, {prompts[0]}, GenerateConfig(24, SamplingStrategy::Greedy())));
+        // the sampled form (acceptance on the device), in both verification forms, temperature and top-k
+        {
+            const std::pair<const char *, GenerateConfig> sampled[] = {
+                {"speculative_temperature", GenerateConfig(28, SamplingStrategy::Temperature(0.8f)).with_seed(11)},
+                {"speculative_top_k", GenerateConfig(28, SamplingStrategy::TopK(5)).with_seed(7)}};
+            for (const auto &sc : sampled)
+                for (uint64_t k : {3, 9}) {
+                    const SpeculativeOutput so = generate_speculative(dec, draft, prompts[1], sc.second, k);
+                    std::printf("\"%s_k%llu\": {\"tokens\": [", sc.first, (unsigned long long)k);
+                    for (size_t i = 0; i < so.tokens.size(); ++i) std::printf("%s%d", i ? ", " : "", so.tokens[i]);
+                    std::printf("], \"rounds\": %llu, \"accepted\": %llu},\n", (unsigned long long)so.rounds, (unsigned long long)so.accepted);
+                }
+        }
         // the one-layer cache: two appends, then the last token of every row attends to its five positions
         {
             const uint64_t bs = 4, e = 8, heads = 2, dh = 4, b = 2;

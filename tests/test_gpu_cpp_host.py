@@ -81,6 +81,11 @@ def _python_side():
     for k in (4, 9):
         toks, rounds, accepted = sch.generate_speculative(dec, draft, prompts[0], sch.GenerateConfig(24, G()), k)
         out["speculative_k%d" % k] = {"tokens": toks.tolist(), "rounds": rounds, "accepted": accepted}
+    for name, c in (("speculative_temperature", sch.GenerateConfig(28, sch.SamplingStrategy.Temperature(0.8)).with_seed(11)),
+                    ("speculative_top_k", sch.GenerateConfig(28, sch.SamplingStrategy.TopK(5)).with_seed(7))):
+        for k in (3, 9):
+            toks, rounds, accepted = sch.generate_speculative(dec, draft, prompts[1], c, k)
+            out["%s_k%d" % (name, k)] = {"tokens": toks.tolist(), "rounds": rounds, "accepted": accepted}
     draft.close()
     dec.close()
     be.close()
@@ -105,7 +110,8 @@ def test_cpp_host_layer_matches_the_python_mirror_on_the_device():
     assert cpp["paged_cache_max_abs_err"] < 1e-5 and cpp["paged_cache_state_ok"]
     py = _python_side()
     for key in ("generate_greedy", "generate_top_k", "generate_temperature", "scheduler", "scheduler_prompt_passes",
-                "scheduler_decode_steps", "speculative_k4", "speculative_k9"):
+                "scheduler_decode_steps", "speculative_k4", "speculative_k9", "speculative_temperature_k3",
+                "speculative_temperature_k9", "speculative_top_k_k3", "speculative_top_k_k9"):
         assert cpp[key] == py[key], key
 
 
