@@ -296,6 +296,27 @@ def bench_prefill(fa, be, iters):
     return res
 
 
+F32_PEAK_TFLOPS = 157.3         # dense f32 matrix rate of MI355X
+
+
+def bench_gemm_f32(fa, be, iters):
+    """The order-fixed f32 GEMM (gemm_device / linear_forward_device: one fused multiply-add per k, k ascending)
+    at a prompt shape and at a decode shape."""
+    lib = fa.capi.lib
+    res = []
+    for m, k, n in ((2048, 4096, 4096), (32, 4096, 4096)):
+        a, b, out = be.alloc_uninit((m, k)), be.alloc_uninit((k, n)), be.alloc_uninit((m, n))
+        fa.check(lib.fa_fill_normal(be._ctx, a._h, 0, m * k, 21, 0.0, 1.0))
+        fa.check(lib.fa_fill_normal(be._ctx, b._h, 0, k * n, 22, 0.0, 0.02))
+        sec = time_launches(fa, be, lambda: fa.check(lib.fa_gemm_device(be._ctx, a._h, b._h, m, n, k, out._h)), iters)
+        flops = 2.0 * m * k * n
+        res.append(dict(op="gemm_device_f32", m=m, k=k, n=n, us=sec * 1e6, tflops=flops / sec / 1e12,
+                        frac=flops / sec / 1e12 / F32_PEAK_TFLOPS))
+        for x in (a, b, out):
+            x.free()
+    return res
+
+
 def bench_prefill_attention(fa, be, batch=4, l_new=2048, heads=32, kv_heads=8):
     """Causal attention of `l_new` new tokens per row over their own pages (empty cache before them), bf16,
     page 16: the block form (what this shape selects), the streamed form and the generic kernel (reference
@@ -723,7 +744,7 @@ def main():
                     help="with --only decode-linears: one of the four layer shapes (0 .. 3) instead of all, so that "
                          "a counter run sees launches of one shape only")
     ap.add_argument("--only", choices=("attention", "copy", "linears", "decode-linears", "prefill", "prefill-attention", "mfma",
-                                       "prompt", "stream-floor"), default=None,
+                                       "prompt", "stream-floor", "gemm-f32"), default=None,
                     help="profiling aid: run only the dominant kernel at the workload's shape, or a plain "
                          "copy kernel of known size (counter calibration), a few launches, no JSON line")
     a = ap.parse_args()
@@ -760,6 +781,12 @@ def main():
                 log("one prompt of %d tokens%s through %d layers: %.2f ms, %.0f tokens/s" %
                     (r["l_new"], " after %d cached" % r["cached"] if r["cached"] else "", cfg["n_layers"], r["ms"], r["tokens_per_s"]))
             lib.fa_decoder_destroy(be._ctx, dec)
+            be.close()
+            return
+        if a.only == "gemm-f32":
+            for r in bench_gemm_f32(fa, be, 10):
+                log("f32 gemm_device m=%d k=%d n=%d: %.1f us, %.1f TFLOP/s (%.1f %% of the f32 matrix peak)" %
+                    (r["m"], r["k"], r["n"], r["us"], r["tflops"], 100 * r["frac"]))
             be.close()
             return
         if a.only == "mfma":
@@ -882,6 +909,10 @@ def main():
         extras["decode_linears"] = bench_linears(fa, be, 100)
         extras["sampling_32x32000"] = bench_sampling(fa, be)
         extras["prefill_gemm"] = bench_prefill(fa, be, 20)
+        extras["gemm_device_f32"] = bench_gemm_f32(fa, be, 10)
+        for r in extras["gemm_device_f32"]:
+            log("f32 gemm_device m=%d k=%d n=%d: %.1f us, %.1f TFLOP/s (%.1f %% of the f32 matrix peak)" %
+                (r["m"], r["k"], r["n"], r["us"], r["tflops"], 100 * r["frac"]))
         # what a plain streaming read of the same bytes reaches: the yardstick for the bandwidth-bound kernels
         extras["stream_read_floor"] = bench_stream_floor(fa, be, floor_sizes(cfg, att_bytes))
     out = {

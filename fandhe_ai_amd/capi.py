@@ -210,6 +210,7 @@ SIGNATURES = {
     "fa_decoder_debug_step_until": (C.c_int32, [ctx_p, C.c_void_p, C.c_int32]),
     "fa_decoder_debug_buffer": (C.c_int32, [C.c_void_p, C.c_int32, C.POINTER(buf_p)]),
     "fa_probe_stream_read": (C.c_int32, [ctx_p, buf_p, u64, u64, C.c_int32, C.c_int32, buf_p]),
+    "fa_gemm_f32_form_query": (C.c_int32, [u64, u64, u64, C.POINTER(C.c_int32)]),
     "fa_gemm_plan_query": (C.c_int32, [ctx_p, u64, qw_p, C.POINTER(GemmPlan)]),
     "fa_graph_owned_blocks": (C.c_int32, [C.c_void_p, C.POINTER(C.c_void_p), u64, C.POINTER(u64)]),
 }

@@ -12,6 +12,7 @@ using namespace fa;
 
 namespace fa {
 namespace k {
+extern int g_gemm_f32_form;
 extern int g_skinny_ntw, g_skinny_waves, g_skinny_astat, g_gemm_small_tiles, g_gemm_waves, g_gemm_ntb, g_gemm_split_fill;
 }
 int g_decode_waves = 0;
@@ -86,8 +87,15 @@ fa_status fa_set_tuning(int32_t key, int32_t value) {
         case 10: fa::g_prefill_block_form = value; return FA_OK;
         case 11: fa::g_prefill_block_waves = value; return FA_OK;
         case 12: fa::g_prefill_block_split = value; return FA_OK;
+        case 13: k::g_gemm_f32_form = value; return FA_OK;
     }
     return fail(FA_ERR_INVALID_ARGUMENT, "fa_set_tuning: unknown key");
+}
+
+fa_status fa_gemm_f32_form_query(uint64_t m, uint64_t n, uint64_t k, int32_t *form) {
+    if (!form) return fail(FA_ERR_INVALID_ARGUMENT, "gemm_f32_form_query: null out");
+    *form = k::gemm_f32_form(m, n, k);
+    return FA_OK;
 }
 
 fa_status fa_gemm_plan_query(const fa_context *ctx, uint64_t m, const fa_qweight *qw, fa_gemm_plan *out) {

@@ -89,6 +89,8 @@ void scale_from_absmax(const float *absmax, float divisor, float *scale, hipStre
 // ---- f32 GEMM with the reference's summation order (kern_gemm_f32.hip) -------
 void gemm_f32(const float *a, const float *b, const float *bias, float *out, uint64_t m, uint64_t n,
               uint64_t k, int relu, hipStream_t s);
+// Which kernel that call launches: 1 the few-rows vector kernel, 2 the matrix-core kernel.
+int gemm_f32_form(uint64_t m, uint64_t n, uint64_t k);
 
 // ---- skinny (decode-shape) quantized linears (kern_qlinear.hip) ---------------
 struct EpilogueI8 {

@@ -58,7 +58,9 @@ fa_status fa_probe_stream_read(fa_context *ctx, const fa_buffer *src, uint64_t o
  *        streamed form, 2 always the block form, 0 by shape;
  * key 11: wavefronts per block of that block form (4 or 8; 0 by shape);
  * key 12: upper bound of the blocks that share the cache walk of one tile of new tokens
- *        in the block form (1: never split; 0 by shape). */
+ *        in the block form (1: never split; 0 by shape);
+ * key 13: kernel of the order-fixed f32 GEMM (gemm_device / linear_forward_device): 1 the few-rows vector
+ *        kernel, 2 the matrix-core kernel, 0 by shape. */
 fa_status fa_set_tuning(int32_t key, int32_t value);
 
 /* Which kernel a prefill-shape GEMM of m rows against `qw` is launched with under the
@@ -71,6 +73,10 @@ typedef struct {
     uint32_t splits;
 } fa_gemm_plan;
 fa_status fa_gemm_plan_query(const fa_context *ctx, uint64_t m, const fa_qweight *qw, fa_gemm_plan *out);
+
+/* Which kernel fa_gemm_device / fa_linear_forward_device launch for an m x k by k x n product under the current
+ * knobs: 1 the few-rows vector kernel (gemm_f32_rows_kernel), 2 the matrix-core kernel (gemm_f32_mfma_kernel). */
+fa_status fa_gemm_f32_form_query(uint64_t m, uint64_t n, uint64_t k, int32_t *form);
 
 /* Device blocks a captured graph owns (scratch that calls recorded into it took while the
  * capture was open; they return to the pool when the graph is destroyed).  Writes up to

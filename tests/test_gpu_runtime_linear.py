@@ -94,17 +94,72 @@ def _data(n, seed):
     return out
 
 
+def _gemm_form(fa, m, n, k):
+    form = C.c_int32()
+    fa.check(fa.capi.lib.fa_gemm_f32_form_query(m, n, k, C.byref(form)))
+    return form.value
+
+
+# shapes that take the matrix-core kernel by themselves: whole 128 x 128 tiles, ragged edges with k % 4 != 0
+# (scalar slab loads), one tile row only
+GEMM_SHAPES_WIDE = [(512, 4096, 33), (515, 4099, 70), (640, 3968, 16), (1024, 2048, 5)]
+
+
 def test_gemm_device_is_bit_identical_to_the_fma_reference():
+    """Both kernels of the order-fixed GEMM (a chain of v_fma_f32 on the vector ALUs; a chain of one-product
+    matrix instructions) against the oracle's k-ascending fused multiply-add loop, bit for bit, on every shape."""
+    import fandhe_ai_amd as fa
     be = ops()
     o.set_threads(8)
-    for i, (m, n, k) in enumerate(GEMM_SHAPES):
-        a = _data(m * k, 1 + i).reshape(m, k)
-        b = _data(k * n, 100 + i).reshape(k, n)
-        want = o.gemm_f32(a, b)
-        got = be.download_owned(be.gemm_device(be.upload(a), be.upload(b)))
-        r = assert_parity("ROCM_PARITY", f"{m}x{n}x{k}", got, want)
-        assert r.bit_mismatch == 0
-    o.set_threads(1)
+    try:
+        for i, (m, n, k) in enumerate(GEMM_SHAPES + GEMM_SHAPES_WIDE):
+            a = _data(m * k, 1 + i).reshape(m, k)
+            b = _data(k * n, 100 + i).reshape(k, n)
+            want = o.gemm_f32(a, b)
+            da, db = be.upload(a), be.upload(b)
+            if (m, n, k) in GEMM_SHAPES_WIDE:
+                assert _gemm_form(fa, m, n, k) == 2
+            for form in (0, 1, 2):
+                fa.check(fa.capi.lib.fa_set_tuning(13, form))
+                if form and k and m and n:
+                    assert _gemm_form(fa, m, n, k) == form
+                got = be.download_owned(be.gemm_device(da, db))
+                r = assert_parity("ROCM_PARITY", f"{m}x{n}x{k} form {form}", got, want)
+                assert r.bit_mismatch == 0
+            da.free(), db.free()
+    finally:
+        fa.check(fa.capi.lib.fa_set_tuning(13, 0))
+        o.set_threads(1)
+
+
+def test_gemm_device_keeps_the_chain_on_special_values():
+    """Subnormal inputs and products, cancellation, overflow to infinity and NaNs: one rounding per step on
+    both kernels, as in the oracle's loop."""
+    import fandhe_ai_amd as fa
+    be = ops()
+    rng = np.random.default_rng(7)
+    m, n, k = 130, 192, 96
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    b = rng.standard_normal((k, n)).astype(np.float32)
+    a[:, 0:16] *= np.float32(2.0 ** -80)                     # products near 2^-150: subnormal partial sums
+    b[0:16, :] *= np.float32(2.0 ** -70)
+    a[:, 16:32] *= np.float32(2.0 ** 70)                     # overflow to +-inf in some chains
+    b[16:32, :] *= np.float32(2.0 ** 60)
+    b[40, 5] = np.float32(np.nan)
+    a[7, 50] = np.float32(np.inf)
+    b[60:70, :] = -b[50:60, :]                               # exact cancellation against a[:, 50:60] below
+    a[:, 60:70] = a[:, 50:60]
+    want = o.gemm_f32(a, b)
+    da, db = be.upload(a), be.upload(b)
+    try:
+        for form in (1, 2):
+            fa.check(fa.capi.lib.fa_set_tuning(13, form))
+            got = be.download_owned(be.gemm_device(da, db))
+            same = (got.view(np.uint32) == want.view(np.uint32)) | (np.isnan(got) & np.isnan(want))
+            assert same.all(), (form, int((~same).sum()))
+    finally:
+        fa.check(fa.capi.lib.fa_set_tuning(13, 0))
+    assert np.isinf(want).any() and np.isnan(want).any()
 
 
 def test_linear_forward_device_views_bias_relu():
