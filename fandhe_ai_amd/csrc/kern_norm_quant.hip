@@ -294,6 +294,11 @@ __global__ void __launch_bounds__(kBlock)
         if (c < n_chunks) *(v4i *)(xq_tiled + tiled_chunk_offset(r, c, k_tiles)) = v4i{0, 0, 0, 0};
         return;
     }
+    // the chunk's values are requested before the partial maxima are reduced: one memory round trip, not two
+    float xv[16];
+    const uint64_t cc = c < n_chunks ? c : n_chunks - 1;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) xv[e] = load_in<IN_BF16>(x, r * k + cc * 16 + e);
     float amax = 0.0f;
     for (uint32_t i = threadIdx.x; i < parts; i += kBlock) amax = fmaxf(amax, pmax[r * parts + i]);
     amax = block_max<kWaves>(amax, smem);
@@ -305,8 +310,7 @@ __global__ void __launch_bounds__(kBlock)
     for (int wd = 0; wd < 4; ++wd) {
         uint32_t word = 0;
 #pragma unroll
-        for (int b = 0; b < 4; ++b)
-            word |= ((uint32_t)quant_i8(load_in<IN_BF16>(x, r * k + c * 16 + wd * 4 + b), scale) & 0xffu) << (8 * b);
+        for (int b = 0; b < 4; ++b) word |= ((uint32_t)quant_i8(xv[wd * 4 + b], scale) & 0xffu) << (8 * b);
         words[wd] = word;
     }
     *(v4u *)(xq_tiled + tiled_chunk_offset(r, c, k_tiles)) = v4u{words[0], words[1], words[2], words[3]};

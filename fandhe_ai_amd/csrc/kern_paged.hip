@@ -517,12 +517,44 @@ __global__ void __launch_bounds__(256) decode_stream_merge_kernel(StreamParams p
     const uint32_t per = range_pages(p, tot);
     const uint32_t r_lo = npg ? pre / per : 1, r_hi = npg ? (pre + npg - 1) / per : 0;   // empty sequence: no partials
     float mx = -INFINITY;
-    for (uint32_t r = r_lo; r <= r_hi; ++r) {
+    float acc = 0.0f, den = 0.0f;
+    constexpr int kOneTrip = 8;
+    const bool one_trip = npg == 0 || r_hi - r_lo < (uint32_t)kOneTrip;
+    if (one_trip) {
+        // up to eight partial results: all maxima and this thread's every second (l, o) are requested at once,
+        // one memory round trip instead of two; the arithmetic and its order are those of the loops below
+        float m[kOneTrip], l[kOneTrip / 2], o[kOneTrip / 2];
+#pragma unroll
+        for (int u = 0; u < kOneTrip; ++u) {
+            const uint64_t r = r_lo + u <= r_hi ? r_lo + u : r_hi;
+            m[u] = p.part_ml[((r + b) * p.num_kv_heads + kvh) * (2 * p.g_pad) + hg];
+        }
+#pragma unroll
+        for (int u = 0; u < kOneTrip / 2; ++u) {
+            const uint64_t r = r_lo + part + 2 * u <= r_hi ? r_lo + part + 2 * u : r_hi;
+            const uint64_t item = (r + b) * p.num_kv_heads + kvh;
+            l[u] = p.part_ml[item * (2 * p.g_pad) + p.g_pad + hg];
+            o[u] = p.part_o[(item * p.g_pad + hg) * kDh + d];
+        }
+#pragma unroll
+        for (int u = 0; u < kOneTrip; ++u)
+            if (r_lo + u <= r_hi) mx = (m[u] != m[u] || mx != mx) ? __uint_as_float(0x7fc00000u) : fmaxf(mx, m[u]);
+#pragma unroll
+        for (int u = 0; u < kOneTrip / 2; ++u) {
+            if (r_lo + part + 2 * u <= r_hi) {
+                // m of partial part + 2 u: a static index for either value of part
+                const float mu = part ? m[2 * u + 1] : m[2 * u];
+                const float w = expf(mu - mx);
+                den = __builtin_fmaf(w, l[u], den);
+                acc = __builtin_fmaf(w, o[u], acc);
+            }
+        }
+    }
+    for (uint32_t r = r_lo; !one_trip && r <= r_hi; ++r) {
         float m = p.part_ml[((uint64_t)(r + b) * p.num_kv_heads + kvh) * (2 * p.g_pad) + hg];
         mx = (m != m || mx != mx) ? __uint_as_float(0x7fc00000u) : fmaxf(mx, m);   // NaN marks a violation
     }
-    float acc = 0.0f, den = 0.0f;
-    for (uint32_t r = r_lo + part; r <= r_hi; r += 2) {
+    for (uint32_t r = r_lo + part; !one_trip && r <= r_hi; r += 2) {
         const uint64_t item = (uint64_t)(r + b) * p.num_kv_heads + kvh;
         float m = p.part_ml[item * (2 * p.g_pad) + hg];
         float l = p.part_ml[item * (2 * p.g_pad) + p.g_pad + hg];
@@ -669,7 +701,36 @@ __global__ void __launch_bounds__(1024) decode_stream_merge_quantize_kernel(Stre
     const float *po = p.part_o + (((uint64_t)b * p.num_kv_heads + kvh) * p.g_pad + hg) * kDh + d4;
     const uint64_t ml_step = (uint64_t)p.num_kv_heads * (2 * p.g_pad), po_step = (uint64_t)p.num_kv_heads * p.g_pad * kDh;
     float mx = -INFINITY;
-    for (uint32_t r0 = r_lo; r0 <= r_hi; r0 += 4) {
+    v4f acc = v4f{0.f, 0.f, 0.f, 0.f};
+    float den = 0.0f;
+    constexpr int kOneTrip = 8;
+    const bool one_trip = npg == 0 || r_hi - r_lo < (uint32_t)kOneTrip;
+    if (one_trip) {
+        // up to eight partial results: everything is requested at once and the maximum is taken from registers,
+        // one memory round trip instead of two; the arithmetic and its order are those of the loops below
+        float m[kOneTrip], l[kOneTrip];
+        v4f o[kOneTrip];
+#pragma unroll
+        for (int u = 0; u < kOneTrip; ++u) {
+            const uint64_t r = r_lo + u <= r_hi ? r_lo + u : r_hi;
+            m[u] = ml[r * ml_step];
+            l[u] = ml[r * ml_step + p.g_pad];
+            o[u] = *(const v4f *)(po + r * po_step);
+        }
+#pragma unroll
+        for (int u = 0; u < kOneTrip; ++u)
+            if (r_lo + u <= r_hi) mx = (m[u] != m[u] || mx != mx) ? __uint_as_float(0x7fc00000u) : fmaxf(mx, m[u]);
+#pragma unroll
+        for (int u = 0; u < kOneTrip; ++u) {
+            if (r_lo + u <= r_hi) {
+                const float w = expf(m[u] - mx);
+                den = __builtin_fmaf(w, l[u], den);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[e] = __builtin_fmaf(w, o[u][e], acc[e]);
+            }
+        }
+    }
+    for (uint32_t r0 = r_lo; !one_trip && r0 <= r_hi; r0 += 4) {
         float m[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) m[u] = ml[(uint64_t)(r0 + u <= r_hi ? r0 + u : r_hi) * ml_step];
@@ -677,9 +738,7 @@ __global__ void __launch_bounds__(1024) decode_stream_merge_quantize_kernel(Stre
         for (int u = 0; u < 4; ++u)
             mx = (m[u] != m[u] || mx != mx) ? __uint_as_float(0x7fc00000u) : fmaxf(mx, m[u]);   // NaN marks a violation
     }
-    v4f acc = v4f{0.f, 0.f, 0.f, 0.f};
-    float den = 0.0f;
-    for (uint32_t r0 = r_lo; r0 <= r_hi; r0 += 4) {
+    for (uint32_t r0 = r_lo; !one_trip && r0 <= r_hi; r0 += 4) {
         float m[4], l[4];
         v4f o[4];
 #pragma unroll
