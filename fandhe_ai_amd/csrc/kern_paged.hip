@@ -656,16 +656,21 @@ __global__ void __launch_bounds__(kPrefillMergeThreads)
 // projection that consumes the attention output: thread (head, 4 dims) merges its partial results,
 // rounds once to bf16 (the attention output's type), the block takes the row's absmax, and the row
 // leaves as int8 activation tiles plus its scale.  Rows at or past the batch are written as zeros.
+// QUANT = false: the same merge without the quantizer, the row stored as the operator's output (bf16 or
+// f32) with, when asked, the absmax of every head's slice; used whenever the heads fit one block.
+template <bool QUANT>
 __global__ void __launch_bounds__(1024) decode_stream_merge_quantize_kernel(StreamParams p, int8_t *__restrict__ xq_tiled,
-                                                                           float *__restrict__ sx) {
+                                                                           float *__restrict__ sx, void *__restrict__ out,
+                                                                           int out_bf16, float *__restrict__ pmax) {
     __shared__ uint32_t s_tot[16], s_pre[16];
     __shared__ float s_max[16];
     const uint32_t b = blockIdx.x;
     const uint32_t e_q = p.num_heads * kDh, k_tiles = e_q / 64;
     const int wave = threadIdx.x / 64, n_waves = blockDim.x / 64;
     if (b >= p.batch) {
-        for (uint32_t c = threadIdx.x; c < e_q / 16; c += blockDim.x)
-            *(v4u *)(xq_tiled + tiled_chunk_offset(b, c, k_tiles)) = v4u{0, 0, 0, 0};
+        if constexpr (QUANT)
+            for (uint32_t c = threadIdx.x; c < e_q / 16; c += blockDim.x)
+                *(v4u *)(xq_tiled + tiled_chunk_offset(b, c, k_tiles)) = v4u{0, 0, 0, 0};
         return;
     }
     const uint32_t max_ctx = p.max_blocks_per_seq * kPage;
@@ -757,6 +762,29 @@ __global__ void __launch_bounds__(1024) decode_stream_merge_quantize_kernel(Stre
         }
     }
     float v[4], amax = 0.0f;
+    if constexpr (!QUANT) {
+        const uint64_t oi = ((uint64_t)b * p.num_heads + h) * kDh + d4;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            float res = npg == 0 ? 0.0f : __fdiv_rn(acc[e], den);
+            if (out_bf16) res = bf16_to_f32(f32_to_bf16(res));
+            v[e] = res;
+            amax = fmaxf(amax, fabsf(res));
+        }
+        if (out_bf16) {
+            const uint32_t lo = (uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16);
+            const uint32_t hi = (uint32_t)f32_to_bf16(v[2]) | ((uint32_t)f32_to_bf16(v[3]) << 16);
+            *(v2u *)((uint16_t *)out + oi) = v2u{lo, hi};
+        } else {
+            *(v4f *)((float *)out + oi) = v4f{v[0], v[1], v[2], v[3]};
+        }
+        if (pmax) {                                    // absmax of the stored head slice: the 32 threads of a head
+#pragma unroll
+            for (int off = 1; off < 32; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+            if (threadIdx.x % 32 == 0) pmax[(uint64_t)b * p.num_heads + h] = amax;
+        }
+        return;
+    }
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         float res = npg == 0 ? 0.0f : __fdiv_rn(acc[e], den);
@@ -1285,7 +1313,11 @@ void paged_attention_decode_bf16(const uint16_t *q, const uint16_t *k_pool, cons
     if (g_decode_partials_only) return;
     if (xq_tiled != nullptr && ps.num_heads <= 32) {
         // fused merge + per-token quantizer (the bf16 output itself is not written)
-        decode_stream_merge_quantize_kernel<<<m_pad, ps.num_heads * 32, 0, s>>>(sp, xq_tiled, sx);
+        decode_stream_merge_quantize_kernel<true><<<m_pad, ps.num_heads * 32, 0, s>>>(sp, xq_tiled, sx, nullptr, 0, nullptr);
+        return;
+    }
+    if (ps.num_heads <= 32 && ps.num_heads % 2 == 0) {    // a row per block (whole wavefronts): one launch of batch blocks
+        decode_stream_merge_quantize_kernel<false><<<ps.batch, ps.num_heads * 32, 0, s>>>(sp, nullptr, nullptr, out, out_bf16, pmax);
         return;
     }
     dim3 grid2(ps.num_heads, ps.batch);
