@@ -19,6 +19,9 @@ using namespace fa;
 
 namespace fa {
 extern int g_decode_waves;
+namespace k {
+extern int g_weight_prefetch;
+}
 }
 
 struct fa_decoder {
@@ -164,15 +167,27 @@ fa_status enqueue_step(fa_context *ctx, fa_decoder *d, int stop_after = -1) {
                               epilogue(w, out, residual), cus, s);
     };
 
+    // The row kernels in front of the two small projections pull those projections' weights into L2 while they wait
+    // on their own memory round trips (k::WeightPrefetch): all of the o projection (16.8 MB at the benchmark's width)
+    // under the merge + quantizer, half of q | k | v under the norm + quantizer.  Measured in the step's kernel trace:
+    // the o projection 6.7 -> about 4.5 us, q | k | v 9.1 -> 7.9 us, their row kernels + 0.6 and + 0.3 us.  The same
+    // for the wide projections (gate / up, down, the head) lengthens the row kernel by what the projection gains.
+    const uint64_t pull_scale = k::g_weight_prefetch >= 2 ? (uint64_t)k::g_weight_prefetch : 12;
+    const uint64_t kPullQkv = pull_scale << 20, kPullO = (2 * pull_scale) << 20;
+    auto pull_plain = [&](const fa_qweight *w, uint64_t budget) {
+        return k::prefetch_for_linear_w8a8_skinny((const int8_t *)w->codes->ptr, B, w->n_pad, w->k_pad, cus, budget);
+    };
     for (uint32_t li = 0; li < c.n_layers; ++li) {
         const fa_decoder::Layer &L = d->layers[li];
+        const k::QkvRopeTargets t{(const float *)d->cos_sin->ptr, (const uint32_t *)d->slots->ptr, (uint16_t *)d->q_bf->ptr,
+                                  (uint16_t *)L.k_pool->ptr, (uint16_t *)L.v_pool->ptr, c.n_heads, c.n_kv_heads,
+                                  c.head_dim, pool_rows};
         k::rmsnorm_quantize_i8((const float *)d->h->ptr, (const float *)L.attn_norm->ptr, c.rms_eps, nullptr,
-                               (int8_t *)d->xq->ptr, (float *)d->sx->ptr, B, m_pad, D, s);
+                               (int8_t *)d->xq->ptr, (float *)d->sx->ptr, B, m_pad, D, s,
+                               k::prefetch_for_linear_w8a8_qkv_rope_skinny((const int8_t *)L.wqkv->codes->ptr, B, L.wqkv->n_pad,
+                                                                           L.wqkv->k_pad, t, kPullQkv));
         if (stop_here()) break;
         {
-            k::QkvRopeTargets t{(const float *)d->cos_sin->ptr, (const uint32_t *)d->slots->ptr, (uint16_t *)d->q_bf->ptr,
-                                (uint16_t *)L.k_pool->ptr, (uint16_t *)L.v_pool->ptr, c.n_heads, c.n_kv_heads,
-                                c.head_dim, pool_rows};
             k::linear_w8a8_qkv_rope_skinny((const int8_t *)d->xq->ptr, (const int8_t *)L.wqkv->codes->ptr,
                                            (const float *)d->sx->ptr, (const float *)L.wqkv->scales->ptr, B,
                                            L.wqkv->n_pad, L.wqkv->k_pad, t, s);
@@ -183,14 +198,14 @@ fa_status enqueue_step(fa_context *ctx, fa_decoder *d, int stop_after = -1) {
                                            (const uint16_t *)L.v_pool->ptr, (const uint32_t *)d->tables->ptr,
                                            (const uint32_t *)d->seq_lens->ptr, ps, (uint32_t)g_decode_waves, ctx->workspace,
                                            nullptr, 1, nullptr, (int8_t *)d->xq->ptr, (float *)d->sx->ptr, (uint32_t)m_pad,
-                                           s);
+                                           s, pull_plain(L.wo, kPullO));
         } else {
             k::paged_attention_decode_bf16((const uint16_t *)d->q_bf->ptr, (const uint16_t *)L.k_pool->ptr,
                                            (const uint16_t *)L.v_pool->ptr, (const uint32_t *)d->tables->ptr,
                                            (const uint32_t *)d->seq_lens->ptr, ps, (uint32_t)g_decode_waves, ctx->workspace,
                                            d->attn->ptr, 1, (float *)d->pmax->ptr, s);
             k::quantize_rows_from_pmax(d->attn->ptr, true, (const float *)d->pmax->ptr, c.n_heads, (int8_t *)d->xq->ptr,
-                                       (float *)d->sx->ptr, B, m_pad, EQ, s);
+                                       (float *)d->sx->ptr, B, m_pad, EQ, s, pull_plain(L.wo, kPullO));
         }
         if (stop_here()) break;
         linear(L.wo, d->h->ptr, (const float *)d->h->ptr);

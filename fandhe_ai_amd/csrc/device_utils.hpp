@@ -114,5 +114,36 @@ __device__ __forceinline__ uint32_t f32_to_e4m3(float v) {
     return sign | (e << 3) | m;
 }
 
+
+// Weight bytes of the linear that runs next, pulled into the L2 of the XCD whose compute units will read them.
+// The small row kernels between two linears (norm + quantizer, merge + quantizer, quantizer) are chains of
+// memory round trips on 32 blocks; HBM idles for their whole duration.  Appended blocks of the same launch
+// stream the first bytes of the next linear's weight tiles meanwhile.  Workgroups go to the XCDs round-robin by
+// their linear id, so when the number of blocks in front of them is a multiple of eight, appended block j lands
+// on the XCD of block j of the next launch and reads exactly what that block will read first; L2 keeps clean
+// lines across the kernel boundary, and the linear then finds them there (a 25 MB weight read: 6.2 us cold,
+// 2.6 us after such a pull, 5.0 us when the pull ran on other XCDs).  Nothing is written.
+// PF: fa::k::WeightPrefetch (declared with the launchers)
+template <typename PF>
+__device__ __forceinline__ void prefetch_weights(const PF &pf, uint32_t j) {
+    if (j >= pf.blocks) return;
+    const uint32_t t0 = pf.half_tiles ? (j / pf.half_tiles) * 2 * pf.half_tiles + j % pf.half_tiles : j * pf.tile_stride;
+    const uint32_t vecs = pf.bytes / 16, nt = blockDim.x;
+    v4u acc = v4u{0, 0, 0, 0};
+    for (uint32_t r = 0; r < (pf.pair_step ? 2u : 1u); ++r) {
+        uint32_t tile = t0 + r * pf.pair_step;
+        tile = tile < pf.n_tiles ? tile : pf.n_tiles - 1;
+        const v4u *p = (const v4u *)(pf.w + (uint64_t)tile * pf.k_tiles * 1024);
+        for (uint32_t i = threadIdx.x; i < vecs; i += nt * 4) {
+            v4u t[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) t[u] = p[i + u * nt < vecs ? i + u * nt : i];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) acc ^= t[u];
+        }
+    }
+    asm volatile("" ::"v"(acc[0] ^ acc[1] ^ acc[2] ^ acc[3]));      // the loads are the point; keep them
+}
+
 }  // namespace dev
 }  // namespace fa

@@ -152,9 +152,13 @@ template <int NCH, bool ROW = false>
 __global__ void __launch_bounds__(kBlock)
     rmsnorm_quantize_kernel(const float *__restrict__ x, const float *__restrict__ w, float eps, float inv_n,
                             float *__restrict__ out_f32, int8_t *__restrict__ xq_tiled, float *__restrict__ sx,
-                            uint64_t m, uint64_t hidden) {
+                            uint64_t m, uint64_t hidden, uint32_t row_blocks, WeightPrefetch pull) {
     __shared__ double smem_d[kWaves];
     __shared__ float smem_f[kWaves];
+    if (blockIdx.x >= row_blocks) {                      // appended blocks: weights of the linear that follows
+        prefetch_weights(pull, blockIdx.x - row_blocks);
+        return;
+    }
     const uint64_t r = blockIdx.x;
     const uint64_t k_tiles = hidden / 64, n_chunks = hidden / 16;
     if (r >= m) {
@@ -286,8 +290,13 @@ __global__ void __launch_bounds__(ONE ? 1024 : kBlock)
 template <bool IN_BF16>
 __global__ void __launch_bounds__(kBlock)
     quantize_from_pmax_kernel(const void *__restrict__ x, const float *__restrict__ pmax, uint32_t parts,
-                              int8_t *__restrict__ xq_tiled, float *__restrict__ sx, uint64_t m, uint64_t k) {
+                              int8_t *__restrict__ xq_tiled, float *__restrict__ sx, uint64_t m, uint64_t k,
+                              uint32_t row_blocks, WeightPrefetch pull) {
     __shared__ float smem[kWaves];
+    if (blockIdx.y >= row_blocks) {                      // appended rows of blocks: weights of the linear that follows
+        prefetch_weights(pull, (blockIdx.y - row_blocks) * gridDim.x + blockIdx.x);
+        return;
+    }
     const uint64_t r = blockIdx.y, k_tiles = k / 64, n_chunks = k / 16;
     const uint64_t c = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
     if (r >= m) {
@@ -382,17 +391,20 @@ void quantize_rows_i8(const void *x, bool in_bf16, int8_t *xq_rowmajor, int8_t *
 }
 
 void rmsnorm_quantize_i8(const float *x, const float *w, float eps, float *out_f32, int8_t *xq_tiled, float *sx,
-                         uint64_t m, uint64_t m_pad, uint64_t hidden, hipStream_t s) {
+                         uint64_t m, uint64_t m_pad, uint64_t hidden, hipStream_t s, const WeightPrefetch &pull) {
     if (m_pad == 0 || hidden == 0) return;
     float inv_n = 1.0f / (float)hidden;
     uint64_t per_thread = (hidden / 16 + kBlock - 1) / kBlock;       // 16-element chunks per thread
-    unsigned grid = (unsigned)m_pad;
+    const uint32_t rows = (uint32_t)m_pad;
+    // the appended blocks only meet the next launch's blocks on their XCD when a multiple of eight blocks precedes them
+    const WeightPrefetch pf = (pull.w && rows % 8 == 0) ? pull : WeightPrefetch{};
+    unsigned grid = rows + pf.blocks;
     if (per_thread <= 1)
-        rmsnorm_quantize_kernel<1><<<grid, kBlock, 0, s>>>(x, w, eps, inv_n, out_f32, xq_tiled, sx, m, hidden);
+        rmsnorm_quantize_kernel<1><<<grid, kBlock, 0, s>>>(x, w, eps, inv_n, out_f32, xq_tiled, sx, m, hidden, rows, pf);
     else if (per_thread <= 2)
-        rmsnorm_quantize_kernel<2><<<grid, kBlock, 0, s>>>(x, w, eps, inv_n, out_f32, xq_tiled, sx, m, hidden);
+        rmsnorm_quantize_kernel<2><<<grid, kBlock, 0, s>>>(x, w, eps, inv_n, out_f32, xq_tiled, sx, m, hidden, rows, pf);
     else
-        rmsnorm_quantize_kernel<4><<<grid, kBlock, 0, s>>>(x, w, eps, inv_n, out_f32, xq_tiled, sx, m, hidden);
+        rmsnorm_quantize_kernel<4><<<grid, kBlock, 0, s>>>(x, w, eps, inv_n, out_f32, xq_tiled, sx, m, hidden, rows, pf);
 }
 
 void rmsnorm_quantize_rows_i8(const float *x, const float *w, float eps, int8_t *xq_rowmajor, float *sx, uint64_t m,
@@ -402,11 +414,11 @@ void rmsnorm_quantize_rows_i8(const float *x, const float *w, float eps, int8_t 
     uint64_t per_thread = (hidden / 16 + kBlock - 1) / kBlock;
     unsigned grid = (unsigned)m;
     if (per_thread <= 1)
-        rmsnorm_quantize_kernel<1, true><<<grid, kBlock, 0, s>>>(x, w, eps, inv_n, nullptr, xq_rowmajor, sx, m, hidden);
+        rmsnorm_quantize_kernel<1, true><<<grid, kBlock, 0, s>>>(x, w, eps, inv_n, nullptr, xq_rowmajor, sx, m, hidden, grid, WeightPrefetch{});
     else if (per_thread <= 2)
-        rmsnorm_quantize_kernel<2, true><<<grid, kBlock, 0, s>>>(x, w, eps, inv_n, nullptr, xq_rowmajor, sx, m, hidden);
+        rmsnorm_quantize_kernel<2, true><<<grid, kBlock, 0, s>>>(x, w, eps, inv_n, nullptr, xq_rowmajor, sx, m, hidden, grid, WeightPrefetch{});
     else
-        rmsnorm_quantize_kernel<4, true><<<grid, kBlock, 0, s>>>(x, w, eps, inv_n, nullptr, xq_rowmajor, sx, m, hidden);
+        rmsnorm_quantize_kernel<4, true><<<grid, kBlock, 0, s>>>(x, w, eps, inv_n, nullptr, xq_rowmajor, sx, m, hidden, grid, WeightPrefetch{});
 }
 
 void swiglu_quantize_rows_i8(const float *gu, int8_t *xq_rowmajor, float *sx, uint64_t m, uint64_t f, hipStream_t s) {
@@ -418,13 +430,17 @@ void swiglu_quantize_rows_i8(const float *gu, int8_t *xq_rowmajor, float *sx, ui
 }
 
 void quantize_rows_from_pmax(const void *x, bool in_bf16, const float *pmax, uint32_t parts, int8_t *xq_tiled,
-                             float *sx, uint64_t m, uint64_t m_pad, uint64_t k, hipStream_t s) {
+                             float *sx, uint64_t m, uint64_t m_pad, uint64_t k, hipStream_t s, const WeightPrefetch &pull) {
     if (m_pad == 0 || k == 0) return;
-    dim3 grid((unsigned)((k / 16 + kBlock - 1) / kBlock), (unsigned)m_pad);
+    const unsigned gx = (unsigned)((k / 16 + kBlock - 1) / kBlock), rows = (unsigned)m_pad;
+    // appended block (y, x) has linear id rows * gx + its index: it meets block `index` of the next launch on its XCD
+    // when rows * gx is a multiple of eight
+    const WeightPrefetch pf = (pull.w && ((uint64_t)rows * gx) % 8 == 0) ? pull : WeightPrefetch{};
+    dim3 grid(gx, rows + (pf.blocks + gx - 1) / gx);
     if (in_bf16)
-        quantize_from_pmax_kernel<true><<<grid, kBlock, 0, s>>>(x, pmax, parts, xq_tiled, sx, m, k);
+        quantize_from_pmax_kernel<true><<<grid, kBlock, 0, s>>>(x, pmax, parts, xq_tiled, sx, m, k, rows, pf);
     else
-        quantize_from_pmax_kernel<false><<<grid, kBlock, 0, s>>>(x, pmax, parts, xq_tiled, sx, m, k);
+        quantize_from_pmax_kernel<false><<<grid, kBlock, 0, s>>>(x, pmax, parts, xq_tiled, sx, m, k, rows, pf);
 }
 
 void quantize_rows_e4m3(const void *x, bool in_bf16, uint8_t *xq_rowmajor, float *sx, uint64_t m, uint64_t k,

@@ -661,9 +661,14 @@ __global__ void __launch_bounds__(kPrefillMergeThreads)
 template <bool QUANT>
 __global__ void __launch_bounds__(1024) decode_stream_merge_quantize_kernel(StreamParams p, int8_t *__restrict__ xq_tiled,
                                                                            float *__restrict__ sx, void *__restrict__ out,
-                                                                           int out_bf16, float *__restrict__ pmax) {
+                                                                           int out_bf16, float *__restrict__ pmax,
+                                                                           uint32_t row_blocks, WeightPrefetch pull) {
     __shared__ uint32_t s_tot[16], s_pre[16];
     __shared__ float s_max[16];
+    if (blockIdx.x >= row_blocks) {                      // appended blocks: weights of the linear that follows
+        prefetch_weights(pull, blockIdx.x - row_blocks);
+        return;
+    }
     const uint32_t b = blockIdx.x;
     const uint32_t e_q = p.num_heads * kDh, k_tiles = e_q / 64;
     const int wave = threadIdx.x / 64, n_waves = blockDim.x / 64;
@@ -1283,7 +1288,7 @@ void paged_attention_decode_bf16(const uint16_t *q, const uint16_t *k_pool, cons
 void paged_attention_decode_bf16(const uint16_t *q, const uint16_t *k_pool, const uint16_t *v_pool,
                                  const uint32_t *tables, const uint32_t *seq_lens, const PagedShape &ps,
                                  uint32_t waves_per_cu, void *workspace, void *out, int out_bf16, float *pmax,
-                                 int8_t *xq_tiled, float *sx, uint32_t m_pad, hipStream_t s) {
+                                 int8_t *xq_tiled, float *sx, uint32_t m_pad, hipStream_t s, const WeightPrefetch &pull) {
     if (ps.batch == 0) return;
     StreamParams sp;
     sp.q = q;
@@ -1313,11 +1318,14 @@ void paged_attention_decode_bf16(const uint16_t *q, const uint16_t *k_pool, cons
     if (g_decode_partials_only) return;
     if (xq_tiled != nullptr && ps.num_heads <= 32) {
         // fused merge + per-token quantizer (the bf16 output itself is not written)
-        decode_stream_merge_quantize_kernel<true><<<m_pad, ps.num_heads * 32, 0, s>>>(sp, xq_tiled, sx, nullptr, 0, nullptr);
+        const WeightPrefetch pf = (pull.w && m_pad % 8 == 0) ? pull : WeightPrefetch{};
+        decode_stream_merge_quantize_kernel<true><<<m_pad + pf.blocks, ps.num_heads * 32, 0, s>>>(sp, xq_tiled, sx, nullptr, 0, nullptr,
+                                                                                                 m_pad, pf);
         return;
     }
     if (ps.num_heads <= 32 && ps.num_heads % 2 == 0) {    // a row per block (whole wavefronts): one launch of batch blocks
-        decode_stream_merge_quantize_kernel<false><<<ps.batch, ps.num_heads * 32, 0, s>>>(sp, nullptr, nullptr, out, out_bf16, pmax);
+        decode_stream_merge_quantize_kernel<false><<<ps.batch, ps.num_heads * 32, 0, s>>>(sp, nullptr, nullptr, out, out_bf16, pmax, ps.batch,
+                                                                                         WeightPrefetch{});
         return;
     }
     dim3 grid2(ps.num_heads, ps.batch);

@@ -17,6 +17,7 @@ using namespace fa::dev;
 
 int g_skinny_ntw = 0;      // tuning overrides (0 = heuristic)
 int g_skinny_waves = 0;
+int g_weight_prefetch = 0;   // 1: row kernels pull nothing for the linear that follows them
 int g_skinny_astat = 0;     // activation-stationary kernel: 0 by shape, 1 never, 2 whenever it can run
 
 namespace {
@@ -717,6 +718,52 @@ void launch_w8a16(const uint16_t *a, const int8_t *wt, const float *sw, uint32_t
 }
 
 }  // namespace
+
+// Which weight bytes the blocks of the launches below read first, for the row kernel in front of them to pull
+// (WeightPrefetch): the block -> tile mapping of every form is restated here beside the launch that uses it.
+// `budget` bounds the bytes of one pull (what HBM delivers while a row kernel waits on its own round trips).
+namespace {
+WeightPrefetch make_prefetch(const int8_t *w_tiles, uint32_t blocks, uint32_t n_tiles, uint32_t k_tiles, uint32_t half_tiles,
+                             uint32_t tile_stride, uint32_t pair_step, uint64_t budget) {
+    WeightPrefetch pf;
+    if (g_weight_prefetch == 1 || blocks == 0 || k_tiles == 0 || n_tiles == 0) return pf;
+    const uint64_t regions = (uint64_t)blocks * (pair_step ? 2 : 1);
+    uint64_t per = budget / regions / 1024 * 1024;
+    if (per > (uint64_t)k_tiles * 1024) per = (uint64_t)k_tiles * 1024;
+    if (per == 0) return pf;
+    pf.w = w_tiles;
+    pf.blocks = blocks;
+    pf.n_tiles = n_tiles;
+    pf.k_tiles = k_tiles;
+    pf.half_tiles = half_tiles;
+    pf.tile_stride = tile_stride;
+    pf.pair_step = pair_step;
+    pf.bytes = (uint32_t)per;
+    return pf;
+}
+}  // namespace
+
+WeightPrefetch prefetch_for_linear_w8a8_skinny(const int8_t *w_tiles, uint64_t m, uint64_t n_pad, uint64_t k_pad, int num_cus,
+                                               uint64_t budget) {
+    const uint32_t n_tiles = (uint32_t)(n_pad / 16), k_tiles = (uint32_t)(k_pad / 64);
+    if (m == 0 || n_tiles == 0) return WeightPrefetch{};
+    if (m <= 32 && astat_applies((n_tiles + 1) / 2, k_tiles, num_cus)) {      // block b starts with unit b = tiles 2 b, 2 b + 1
+        const uint32_t n_units = (n_tiles + 1) / 2;
+        return make_prefetch(w_tiles, (uint32_t)std::min<uint64_t>(n_units, (uint64_t)num_cus), n_tiles, k_tiles, 0, 2, n_tiles > 1 ? 1 : 0, budget);
+    }
+    int ntw, waves;
+    pick_config(n_tiles, k_tiles, num_cus, &ntw, &waves);
+    const uint32_t grid = (n_tiles + ntw - 1) / ntw;
+    return make_prefetch(w_tiles, grid, n_tiles, k_tiles, 0, (uint32_t)ntw, ntw == 2 && n_tiles > 1 ? 1 : 0, budget);
+}
+
+WeightPrefetch prefetch_for_linear_w8a8_qkv_rope_skinny(const int8_t *w_tiles, uint64_t m, uint64_t n_pad, uint64_t k_pad,
+                                                        const QkvRopeTargets &t, uint64_t budget) {
+    if (m == 0) return WeightPrefetch{};
+    const uint32_t n = (t.heads + 2 * t.kv_heads) * t.head_dim, half_tiles = t.head_dim / 32;
+    // block b: tile (b / half) * 2 * half + b % half and the tile half_tiles further on
+    return make_prefetch(w_tiles, n / 32, (uint32_t)(n_pad / 16), (uint32_t)(k_pad / 64), half_tiles, 1, half_tiles, budget);
+}
 
 void linear_w8a8_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t m, uint64_t n, uint64_t n_pad,
                         uint64_t k_pad, const EpilogueI8 &ep, int num_cus, hipStream_t s) {

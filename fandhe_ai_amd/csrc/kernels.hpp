@@ -10,6 +10,20 @@
 namespace fa {
 namespace k {
 
+// What a row kernel pulls into L2 for the linear that follows it (dev::prefetch_weights): the first `bytes` of the
+// weight tiles each block of that launch starts with.
+struct WeightPrefetch {
+    const int8_t *w = nullptr;   // tile-ordered codes of the next linear; null: nothing to pull
+    uint32_t blocks = 0;         // blocks of the next launch (one appended block each)
+    uint32_t n_tiles = 0;        // column tiles of the weight (tile indices are clamped to it, as the kernels do)
+    uint32_t k_tiles = 0;        // KiB per column tile
+    uint32_t half_tiles = 0;     // != 0: block j starts at tile (j / half) * 2 * half + j % half (the q | k | v pairing)
+    uint32_t tile_stride = 1;    // otherwise block j starts at tile j * tile_stride
+    uint32_t pair_step = 0;      // != 0: the block also reads tile first + pair_step
+    uint32_t bytes = 0;          // bytes pulled from the start of each tile (multiple of 16)
+};
+
+
 // ---- weight tile order ---------------------------------------------------
 // int8 weights W[k, n] are stored as tiles of 16 columns x 64 k-values, one
 // tile = 1 KiB laid out in the order one wavefront loads it for the int8
@@ -47,10 +61,12 @@ void quantize_rows_i8(const void *x, bool in_bf16, int8_t *xq_rowmajor, int8_t *
 // Per-token quantization when the row absmax is already known as `parts` partial maxima per row
 // (pmax[m, parts]): x f32 or bf16 [m, k] -> activation tiles + sx[m].  k a multiple of 64.
 void quantize_rows_from_pmax(const void *x, bool in_bf16, const float *pmax, uint32_t parts, int8_t *xq_tiled,
-                             float *sx, uint64_t m, uint64_t m_pad, uint64_t k, hipStream_t s);
+                             float *sx, uint64_t m, uint64_t m_pad, uint64_t k, hipStream_t s,
+                             const WeightPrefetch &pull = WeightPrefetch{});
 // RMSNorm fused with the quantizer (f32 in): out_f32 nullable.
 void rmsnorm_quantize_i8(const float *x, const float *w, float eps, float *out_f32, int8_t *xq_tiled,
-                         float *sx, uint64_t m, uint64_t m_pad, uint64_t hidden, hipStream_t s);
+                         float *sx, uint64_t m, uint64_t m_pad, uint64_t hidden, hipStream_t s,
+                         const WeightPrefetch &pull = WeightPrefetch{});
 // The same fused pair with row-major codes [m, hidden] (operand layout of the prefill GEMMs); hidden a
 // multiple of 16 and at most 16384.
 void rmsnorm_quantize_rows_i8(const float *x, const float *w, float eps, int8_t *xq_rowmajor, float *sx, uint64_t m,
@@ -102,6 +118,13 @@ struct EpilogueI8 {
     void *out;            // [m, n] f32 or bf16
     int out_bf16;
 };
+// What the row kernel in front of each of the launches below should pull (see WeightPrefetch); same arguments as
+// the launch itself, `budget` = bytes of one pull.
+struct QkvRopeTargets;
+WeightPrefetch prefetch_for_linear_w8a8_skinny(const int8_t *w_tiles, uint64_t m, uint64_t n_pad, uint64_t k_pad, int num_cus,
+                                               uint64_t budget);
+WeightPrefetch prefetch_for_linear_w8a8_qkv_rope_skinny(const int8_t *w_tiles, uint64_t m, uint64_t n_pad, uint64_t k_pad,
+                                                        const QkvRopeTargets &t, uint64_t budget);
 // xq_tiled: activation tiles (see quantize_rows_i8); m <= 64 (one to four row tiles of 16 per block).
 void linear_w8a8_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t m, uint64_t n,
                         uint64_t n_pad, uint64_t k_pad, const EpilogueI8 &ep, int num_cus,
@@ -193,7 +216,8 @@ void paged_attention_decode_bf16(const uint16_t *q, const uint16_t *k_pool, cons
 void paged_attention_decode_bf16(const uint16_t *q, const uint16_t *k_pool, const uint16_t *v_pool,
                                  const uint32_t *tables, const uint32_t *seq_lens, const PagedShape &ps,
                                  uint32_t waves_per_cu, void *workspace, void *out, int out_bf16, float *pmax,
-                                 int8_t *xq_tiled, float *sx, uint32_t m_pad, hipStream_t s);
+                                 int8_t *xq_tiled, float *sx, uint32_t m_pad, hipStream_t s,
+                                 const WeightPrefetch &pull = WeightPrefetch{});
 
 // Prefill fast path: bf16, head_dim 128, block_size 16, l_new > 1, group <= 16.  Causal over the cached
 // positions: new token t of a row sees positions below seq_len - l_new + t + 1.
