@@ -170,8 +170,8 @@ fa_status enqueue_step(fa_context *ctx, fa_decoder *d, int stop_after = -1) {
     // The row kernels in front of the two small projections pull those projections' weights into L2 while they wait
     // on their own memory round trips (k::WeightPrefetch): all of the o projection (16.8 MB at the benchmark's width)
     // under the merge + quantizer, half of q | k | v under the norm + quantizer.  Measured in the step's kernel trace:
-    // the o projection 6.7 -> about 4.5 us, q | k | v 9.1 -> 7.9 us, their row kernels + 0.6 and + 0.3 us.  The same
-    // for the wide projections (gate / up, down, the head) lengthens the row kernel by what the projection gains.
+    // the o projection 6.7 -> 5.2 us, q | k | v 9.1 -> 8.0 us, their row kernels + 0.7 and + 0.3 us.  The same for
+    // the wide projections (gate / up, down, the head) lengthens the row kernel by what the projection gains.
     const uint64_t pull_scale = k::g_weight_prefetch >= 2 ? (uint64_t)k::g_weight_prefetch : 12;
     const uint64_t kPullQkv = pull_scale << 20, kPullO = (2 * pull_scale) << 20;
     auto pull_plain = [&](const fa_qweight *w, uint64_t budget) {
