@@ -261,6 +261,38 @@ def test_graph_replay_is_bit_identical_to_eager():
     assert runs[0][-1][2].tolist() == [c + 5 for c in shape["ctxs"]]
 
 
+def test_weight_pull_of_the_row_kernels_changes_no_bit():
+    """The blocks appended to the row kernels only read the next projection's weights (an L2 warm-up): with the
+    pull off, at its default and at a size that covers whole weights, every step leaves the same logits, tokens
+    and lengths, eagerly and replayed; shapes with a ragged last q | k | v tile pair and a single row tile."""
+    import fandhe_ai_amd as fa
+    be = ops()
+    for shape in (dict(n_layers=2, d_model=256, n_heads=4, n_kv_heads=2, d_ffn=512, vocab=1000, batch=8,
+                       ctxs=[7, 33, 64, 100, 5, 18, 250, 31]),
+                  dict(n_layers=1, d_model=384, n_heads=3, n_kv_heads=1, d_ffn=640, vocab=517, batch=3, ctxs=[1, 40, 17]),
+                  dict(n_layers=1, d_model=256, n_heads=2, n_kv_heads=2, d_ffn=256, vocab=300, batch=19, ctxs=list(range(1, 20)))):
+        runs = []
+        try:
+            for pull in (1, 0, 64):
+                fa.check(fa.capi.lib.fa_set_tuning(14, pull))
+                m = build_model(seed=6, steps=5, **shape)
+                dec = GpuDecoder(be, m)
+                try:
+                    outs = []
+                    for step in range(4):
+                        dec.step(step >= 2)
+                        be.synchronize_device()
+                        outs.append((dec.logits().copy(), dec.tokens().copy(), dec.seq_lens().copy()))
+                    runs.append(outs)
+                finally:
+                    dec.close()
+        finally:
+            fa.check(fa.capi.lib.fa_set_tuning(14, 0))
+        for other in runs[1:]:
+            for (l0, t0, s0), (l1, t1, s1) in zip(runs[0], other):
+                assert np.array_equal(l0, l1) and np.array_equal(t0, t1) and np.array_equal(s0, s1)
+
+
 def test_decoder_argument_errors():
     import ctypes as C
     import fandhe_ai_amd as fa
