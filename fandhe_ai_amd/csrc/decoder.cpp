@@ -205,7 +205,7 @@ fa_status enqueue_step(fa_context *ctx, fa_decoder *d, int stop_after = -1) {
                                            (const uint32_t *)d->seq_lens->ptr, ps, (uint32_t)g_decode_waves, ctx->workspace,
                                            d->attn->ptr, 1, (float *)d->pmax->ptr, s);
             k::quantize_rows_from_pmax(d->attn->ptr, true, (const float *)d->pmax->ptr, c.n_heads, (int8_t *)d->xq->ptr,
-                                       (float *)d->sx->ptr, B, m_pad, EQ, s, pull_plain(L.wo, kPullO));
+                                       (float *)d->sx->ptr, B, m_pad, EQ, s);
         }
         if (stop_here()) break;
         linear(L.wo, d->h->ptr, (const float *)d->h->ptr);

@@ -290,13 +290,8 @@ __global__ void __launch_bounds__(ONE ? 1024 : kBlock)
 template <bool IN_BF16>
 __global__ void __launch_bounds__(kBlock)
     quantize_from_pmax_kernel(const void *__restrict__ x, const float *__restrict__ pmax, uint32_t parts,
-                              int8_t *__restrict__ xq_tiled, float *__restrict__ sx, uint64_t m, uint64_t k,
-                              uint32_t row_blocks, WeightPrefetch pull) {
+                              int8_t *__restrict__ xq_tiled, float *__restrict__ sx, uint64_t m, uint64_t k) {
     __shared__ float smem[kWaves];
-    if (blockIdx.y >= row_blocks) {                      // appended rows of blocks: weights of the linear that follows
-        prefetch_weights(pull, (blockIdx.y - row_blocks) * gridDim.x + blockIdx.x);
-        return;
-    }
     const uint64_t r = blockIdx.y, k_tiles = k / 64, n_chunks = k / 16;
     const uint64_t c = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
     if (r >= m) {
@@ -430,17 +425,13 @@ void swiglu_quantize_rows_i8(const float *gu, int8_t *xq_rowmajor, float *sx, ui
 }
 
 void quantize_rows_from_pmax(const void *x, bool in_bf16, const float *pmax, uint32_t parts, int8_t *xq_tiled,
-                             float *sx, uint64_t m, uint64_t m_pad, uint64_t k, hipStream_t s, const WeightPrefetch &pull) {
+                             float *sx, uint64_t m, uint64_t m_pad, uint64_t k, hipStream_t s) {
     if (m_pad == 0 || k == 0) return;
-    const unsigned gx = (unsigned)((k / 16 + kBlock - 1) / kBlock), rows = (unsigned)m_pad;
-    // appended block (y, x) has linear id rows * gx + its index: it meets block `index` of the next launch on its XCD
-    // when rows * gx is a multiple of eight
-    const WeightPrefetch pf = (pull.w && ((uint64_t)rows * gx) % 8 == 0) ? pull : WeightPrefetch{};
-    dim3 grid(gx, rows + (pf.blocks + gx - 1) / gx);
+    dim3 grid((unsigned)((k / 16 + kBlock - 1) / kBlock), (unsigned)m_pad);
     if (in_bf16)
-        quantize_from_pmax_kernel<true><<<grid, kBlock, 0, s>>>(x, pmax, parts, xq_tiled, sx, m, k, rows, pf);
+        quantize_from_pmax_kernel<true><<<grid, kBlock, 0, s>>>(x, pmax, parts, xq_tiled, sx, m, k);
     else
-        quantize_from_pmax_kernel<false><<<grid, kBlock, 0, s>>>(x, pmax, parts, xq_tiled, sx, m, k, rows, pf);
+        quantize_from_pmax_kernel<false><<<grid, kBlock, 0, s>>>(x, pmax, parts, xq_tiled, sx, m, k);
 }
 
 void quantize_rows_e4m3(const void *x, bool in_bf16, uint8_t *xq_rowmajor, float *sx, uint64_t m, uint64_t k,

@@ -61,8 +61,7 @@ void quantize_rows_i8(const void *x, bool in_bf16, int8_t *xq_rowmajor, int8_t *
 // Per-token quantization when the row absmax is already known as `parts` partial maxima per row
 // (pmax[m, parts]): x f32 or bf16 [m, k] -> activation tiles + sx[m].  k a multiple of 64.
 void quantize_rows_from_pmax(const void *x, bool in_bf16, const float *pmax, uint32_t parts, int8_t *xq_tiled,
-                             float *sx, uint64_t m, uint64_t m_pad, uint64_t k, hipStream_t s,
-                             const WeightPrefetch &pull = WeightPrefetch{});
+                             float *sx, uint64_t m, uint64_t m_pad, uint64_t k, hipStream_t s);
 // RMSNorm fused with the quantizer (f32 in): out_f32 nullable.
 void rmsnorm_quantize_i8(const float *x, const float *w, float eps, float *out_f32, int8_t *xq_tiled,
                          float *sx, uint64_t m, uint64_t m_pad, uint64_t hidden, hipStream_t s,
