@@ -8,7 +8,7 @@
 // vector ALUs: a wavefront owns a 64 x 64 tile as two instructions per k (the 64 rows as the instruction's two
 // 32-row blocks against columns 0..31 and 32..63, each column operand repeated in both halves of the
 // wavefront) and needs one A value and two B values per lane per k, which LDS supplies at a tenth of its rate.
-// Block = 4 wavefronts = 128 x 128 outputs; k advances in slabs of 16 that travel global -> registers -> LDS,
+// Block = 4 wavefronts = 128 x 128 outputs; k advances in slabs of 32 that travel global -> registers -> LDS,
 // the next slab's loads in flight while the current one is multiplied (two LDS buffers, one barrier per
 // slab).  Edges: rows / columns past the matrix are loaded as zeros and never stored; k needs no padding,
 // the last slab simply runs fewer steps, so no accumulator ever sees a product the contract does not have.
@@ -20,7 +20,7 @@ namespace k {
 
 namespace {
 
-constexpr int BM = 128, BN = 128, BK = 16;
+constexpr int BM = 128, BN = 128, BK = 32;
 constexpr int A_PITCH = BK + 4;          // floats per A row in LDS (80 B: 16-byte reads of 64 rows spread over the banks)
 constexpr int B_PITCH = BN + 4;
 
@@ -39,14 +39,15 @@ __global__ void __launch_bounds__(256)
     const uint64_t row0 = (uint64_t)(blockIdx.x / tiles_n) * BM, col0 = (uint64_t)(blockIdx.x % tiles_n) * BN;
     const int wr = (wave / 2) * 64, wc = (wave % 2) * 64;       // this wavefront's 64 x 64 tile inside the block tile
 
-    // slab staging: A 128 rows x 16 k = 512 float4, B 16 k x 128 cols = 512 float4; two of each per thread
-    float4 ra[2], rb[2];
+    // slab staging: A 128 rows x BK k and B BK k x 128 cols, BK / 8 float4 of each per thread
+    constexpr int NLD = BK / 8, A4 = BK / 4;
+    float4 ra[NLD], rb[NLD];
     auto load_slab = [&](uint64_t k0) {
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
+        for (int t = 0; t < NLD; ++t) {
             const int e = tid + 256 * t;
             {
-                const int r = e / 4, c4 = (e % 4) * 4;
+                const int r = e / A4, c4 = (e % A4) * 4;
                 const uint64_t gr = row0 + r, gc = k0 + c4;
                 float4 v = float4{0.f, 0.f, 0.f, 0.f};
                 if (gr < m) {
@@ -83,9 +84,9 @@ __global__ void __launch_bounds__(256)
     };
     auto store_slab = [&](int buf) {
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
+        for (int t = 0; t < NLD; ++t) {
             const int e = tid + 256 * t;
-            *(float4 *)&As[buf][(e / 4) * A_PITCH + (e % 4) * 4] = ra[t];
+            *(float4 *)&As[buf][(e / A4) * A_PITCH + (e % A4) * 4] = ra[t];
             *(float4 *)&Bs[buf][(e / 32) * B_PITCH + (e % 32) * 4] = rb[t];
         }
     };
