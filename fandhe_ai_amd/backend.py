@@ -97,11 +97,22 @@ class Device:
     def Rocm(ordinal=0):
         return Device("rocm", ordinal)
 
+    @staticmethod
+    def Cuda(ordinal=0):
+        """Another backend's device: this provider refuses it."""
+        return Device("cuda", ordinal)
+
     def __eq__(self, other):
         return isinstance(other, Device) and (self.kind, self.ordinal) == (other.kind, other.ordinal)
 
+    def __hash__(self):
+        return hash((self.kind, self.ordinal))
+
     def __repr__(self):
-        return "Device::%s(%d)" % (self.kind.capitalize(), self.ordinal)
+        return "Device::Cpu" if self.kind == "cpu" else "Device::%s(%r)" % (self.kind.capitalize(), self.ordinal)
+
+
+Device.Cpu = Device("cpu", 0)
 
 
 class RocmDeviceProvider:
@@ -120,9 +131,14 @@ class RocmDeviceProvider:
         return [Device.Rocm(i) for i in range(n.value)]
 
     def select(self, device):
-        if device.kind != "rocm":
-            raise DeviceUnavailable("RocmDeviceProvider cannot provide %r" % (device,))
-        return RocmBackendOps(device.ordinal)
+        # decided before HIP is touched (crates/backend-rocm/src/device.rs:52-63): another backend's device, or an
+        # ordinal that is no device id at all
+        if not isinstance(device, Device) or device.kind != "rocm":
+            raise DeviceUnavailable("RocmDeviceProvider cannot select a non-ROCm device: %r" % (device,))
+        n = device.ordinal
+        if isinstance(n, bool) or not isinstance(n, int) or not 0 <= n < 2 ** 31:
+            raise DeviceUnavailable("Device::Rocm ordinal %r is not a HIP device id" % (n,))
+        return RocmBackendOps(n)
 
 
 def tape_for(device):

@@ -144,3 +144,28 @@ def test_typed_errors_without_a_device_or_with_bad_handles():
     assert lib.fa_buffer_free(None, None) == 0
     assert lib.fa_context_destroy(None) == fa.capi.INVALID_ARGUMENT
     assert lib.fa_set_tuning(99, 1) == fa.capi.INVALID_ARGUMENT
+
+
+def test_device_provider_is_consistent_on_any_host():
+    """crates/backend-rocm/tests/device_provider_absent.rs:9-58: the provider's name, enumerate / is_available /
+    select agree with each other on any host, and devices that are not an existing ROCm ordinal are
+    DeviceUnavailable before HIP is asked (this container has no device, a GPU host has one)."""
+    fa = _fa()
+    p = fa.RocmDeviceProvider()
+    assert p.backend_name() == "rocm"
+    listed = p.enumerate()                                   # never an error: an empty list without HIP
+    assert p.is_available() == (len(listed) > 0)
+    n = len(listed)
+    for d in (fa.Device.Rocm(n), fa.Device.Rocm(2 ** 64 - 1), fa.Device.Rocm(-1), fa.Device.Rocm(True),
+              fa.Device.Rocm(1.0), fa.Device.Cpu, fa.Device.Cuda(0), "rocm:0"):
+        with pytest.raises(fa.DeviceUnavailable):
+            p.select(d)
+    assert fa.Device.Rocm(0) == fa.Device.Rocm(0) != fa.Device.Cuda(0) and repr(fa.Device.Cpu) == "Device::Cpu"
+    if not listed:
+        with pytest.raises(fa.DeviceUnavailable):
+            p.select(fa.Device.Rocm(0))
+    else:
+        assert listed[0] == fa.Device.Rocm(0)
+        ops = p.select(listed[0])
+        assert ops.device() == fa.Device.Rocm(0)
+        ops.close()
