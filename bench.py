@@ -246,25 +246,36 @@ LINEAR_SHAPES = ((4096, 12288), (4096, 4096), (4096, 22016), (11008, 4096))
 
 
 def bench_linears(fa, be, iters, ms=(1, 8, 32), shapes=LINEAR_SHAPES):
-    """Decode-shape int8-weight linears with bf16 activations (W8A16), Llama-7B layer shapes."""
+    """Decode-shape int8-weight linears with bf16 activations (W8A16), Llama-7B layer shapes.  Consecutive
+    launches walk over copies of the weight that together exceed the caches (32 MB of L2, 256 MB memory-side),
+    as the layers of a model do: a launch that found its own weight of the previous launch still cached
+    would be timed on traffic that a decode step never sees."""
     lib = fa.capi.lib
     res = []
     for k, n in shapes:
         w = be.alloc_uninit((k, n))
         fa.check(lib.fa_fill_normal(be._ctx, w._h, 0, k * n, k + n, 0.0, 0.02))
-        qw = be.quantize_weight(fa.DeviceBufferView(w, 0, (k, n)))
+        copies = max(2, -(-(640 << 20) // (k * n)))
+        qws = [be.quantize_weight(fa.DeviceBufferView(w, 0, (k, n))) for _ in range(copies)]
         w.free()
         for m in ms:
             a = be.alloc_uninit((m, k), fa.capi.BF16)
             fa.check(lib.fa_fill_normal(be._ctx, a._h, 0, m * k, 5, 0.0, 1.0))
             out = be.alloc_uninit((m, n), fa.capi.BF16)
-            sec = time_launches(fa, be, lambda: fa.check(lib.fa_linear_w8a16(be._ctx, a._h, m, qw._h, out._h)), iters)
+            counter = [0]
+
+            def launch():
+                qw = qws[counter[0] % copies]
+                counter[0] += 1
+                fa.check(lib.fa_linear_w8a16(be._ctx, a._h, m, qw._h, out._h))
+            sec = time_launches(fa, be, launch, iters)
             nbytes = k * n + 4 * n + 2 * m * k + 2 * m * n
             res.append(dict(op="w8a16", m=m, k=k, n=n, us=sec * 1e6, gbs=nbytes / sec / 1e9,
-                            frac=nbytes / sec / 1e9 / HBM_PEAK_GBS))
+                            frac=nbytes / sec / 1e9 / HBM_PEAK_GBS, weight_copies=copies))
             a.free()
             out.free()
-        qw.free()
+        for qw in qws:
+            qw.free()
     return res
 
 
@@ -520,9 +531,11 @@ def bench_matrix_rate(fa, be, iters=20000):
 
 
 def bench_stream_floor(fa, be, sizes, reps=30):
-    """Plain streaming read of `sizes` bytes (fa_probe_stream_read, 512 blocks of 512 threads), each launch on
-    a fresh window of a 4 GiB buffer so that nothing is served from the 256 MB memory-side cache: the best a
-    memory-bound kernel that must fetch that many bytes can do on this part, launch ramp and tail included."""
+    """Streaming read of `sizes` bytes (fa_probe_stream_read, 512 blocks of 512 threads, the non-temporal
+    16-byte loads the kernels use for read-once data), each launch on a fresh window of a 4 GiB buffer so that
+    nothing is served from the 256 MB memory-side cache: the best a memory-bound kernel that must fetch that
+    many bytes can do on this part, launch ramp and tail included.  us_ordinary_loads: the same read with
+    ordinary loads."""
     lib = fa.capi.lib
     total = 4 << 30
     buf = be.alloc_uninit((total // 4,))
@@ -541,7 +554,13 @@ def bench_stream_floor(fa, be, sizes, reps=30):
             fa.check(lib.fa_probe_stream_read(be._ctx, buf._h, (counter[0] % nwin) * win, nb, 512, 512, sink._h))
             counter[0] += 1
         us = time_launches(fa, be, launch, reps, warmup=3) * 1e6
-        res.append(dict(what=name, bytes=nb, us=us, gbs=nb / us / 1e3, frac=nb / us / 1e3 / HBM_PEAK_GBS))
+        fa.check(lib.fa_set_tuning(15, 1))
+        try:
+            us_plain = time_launches(fa, be, launch, reps, warmup=3) * 1e6
+        finally:
+            fa.check(lib.fa_set_tuning(15, 0))
+        res.append(dict(what=name, bytes=nb, us=us, gbs=nb / us / 1e3, frac=nb / us / 1e3 / HBM_PEAK_GBS,
+                        us_ordinary_loads=us_plain))
     buf.free()
     sink.free()
     return res
@@ -797,8 +816,8 @@ def main():
             return
         if a.only == "stream-floor":
             for r in bench_stream_floor(fa, be, floor_sizes(cfg, attention_bytes(sum(mid_ctx), mid_ctx, cfg["n_heads"], cfg["n_kv_heads"]))):
-                log("plain read of %-36s %10d bytes: %7.2f us, %5.0f GB/s (%.1f %% of peak)" %
-                    (r["what"], r["bytes"], r["us"], r["gbs"], 100 * r["frac"]))
+                log("streaming read of %-36s %10d bytes: %7.2f us, %5.0f GB/s (%.1f %% of peak); ordinary loads %7.2f us" %
+                    (r["what"], r["bytes"], r["us"], r["gbs"], 100 * r["frac"], r["us_ordinary_loads"]))
             be.close()
             return
         if a.only == "decode-linears":

@@ -12,7 +12,7 @@ using namespace fa;
 
 namespace fa {
 namespace k {
-extern int g_gemm_f32_form, g_weight_prefetch;
+extern int g_gemm_f32_form, g_weight_prefetch, g_probe_plain_loads;
 extern int g_skinny_ntw, g_skinny_waves, g_skinny_astat, g_gemm_small_tiles, g_gemm_waves, g_gemm_ntb, g_gemm_split_fill;
 }
 int g_decode_waves = 0;
@@ -89,6 +89,7 @@ fa_status fa_set_tuning(int32_t key, int32_t value) {
         case 12: fa::g_prefill_block_split = value; return FA_OK;
         case 13: k::g_gemm_f32_form = value; return FA_OK;
         case 14: k::g_weight_prefetch = value; return FA_OK;
+        case 15: k::g_probe_plain_loads = value; return FA_OK;
     }
     return fail(FA_ERR_INVALID_ARGUMENT, "fa_set_tuning: unknown key");
 }

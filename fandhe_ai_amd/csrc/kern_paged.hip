@@ -303,12 +303,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, W
             auto load_k = [&](uint32_t i, v4u *dst) {
                 const uint16_t *src_p = p.k_pool + (uint64_t)page_id(i) * page_elems + k_lane;
 #pragma unroll
-                for (int s = 0; s < 4; ++s) dst[s] = *(const v4u *)(src_p + 32 * s);
+                for (int s = 0; s < 4; ++s) dst[s] = stream_load<!PF>((const v4u *)(src_p + 32 * s));
             };
             auto load_v = [&](uint32_t i, v4u *dst) {
                 const uint16_t *src_p = p.v_pool + (uint64_t)page_id(i) * page_elems + v_lane;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) dst[j] = *(const v4u *)(src_p + (uint64_t)j * p.e_kv);
+                for (int j = 0; j < 4; ++j) dst[j] = stream_load<!PF>((const v4u *)(src_p + (uint64_t)j * p.e_kv));
             };
 
             // the first requests go out in the order the loop consumes them (oldest first), so that the wait

@@ -55,9 +55,11 @@ __global__ void __launch_bounds__(256) matrix_rate_kernel(const v4i *__restrict_
     if (s == 0x12345678) sink[0] = s;                 // keeps the loop alive; practically never taken
 }
 
-// Plain streaming read: every block reads its own contiguous share of [src, src + bytes) with 16-byte loads,
-// eight per thread in flight.  What a memory-bound kernel of this size can reach on this part at best
-// (launch ramp and tail included): the yardstick for the decode-shape linears and the decode attention.
+// Streaming read: every block reads its own contiguous share of [src, src + bytes) with 16-byte loads, eight per
+// thread in flight.  What a memory-bound kernel of this size can reach on this part at best (launch ramp and
+// tail included): the yardstick for the decode-shape linears and the decode attention.  ONCE: the non-temporal
+// loads those kernels use for weights and K / V pages; ordinary loads for comparison.
+template <bool ONCE>
 __global__ void __launch_bounds__(512) stream_read_kernel(const v4u *__restrict__ src, uint64_t vecs_per_block, int *sink) {
     constexpr int U = 8;
     const v4u *base = src + (uint64_t)blockIdx.x * vecs_per_block;
@@ -67,7 +69,7 @@ __global__ void __launch_bounds__(512) stream_read_kernel(const v4u *__restrict_
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const uint64_t idx = i + (uint64_t)u * blockDim.x;
-            t[u] = idx < vecs_per_block ? base[idx] : v4u{0, 0, 0, 0};
+            t[u] = stream_load<ONCE>(base + (idx < vecs_per_block ? idx : vecs_per_block - 1));
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) acc ^= t[u];
@@ -77,8 +79,15 @@ __global__ void __launch_bounds__(512) stream_read_kernel(const v4u *__restrict_
 
 }  // namespace
 
+int g_probe_plain_loads = 0;
+
 void stream_read_probe(const void *src, uint64_t bytes, int blocks, int threads, int *sink, hipStream_t s) {
-    stream_read_kernel<<<blocks, threads, 0, s>>>((const v4u *)src, bytes / 16 / (uint64_t)blocks, sink);
+    const uint64_t vecs = bytes / 16 / (uint64_t)blocks;
+    if (vecs == 0) return;
+    if (g_probe_plain_loads)
+        stream_read_kernel<false><<<blocks, threads, 0, s>>>((const v4u *)src, vecs, sink);
+    else
+        stream_read_kernel<true><<<blocks, threads, 0, s>>>((const v4u *)src, vecs, sink);
 }
 
 double matrix_rate_probe(int kind, const void *operands, uint32_t iters, int num_cus, int *sink, hipStream_t s) {

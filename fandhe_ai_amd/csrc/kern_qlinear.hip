@@ -88,6 +88,48 @@ __global__ void __launch_bounds__(NWAVES * 64)
     uint32_t a_off[MT];
 #pragma unroll
     for (int i = 0; i < MT; ++i) a_off[i] = ((uint32_t)i * 16 + (uint32_t)lane % 16 < m ? (uint32_t)lane : (uint32_t)lane & 48u) * 16;
+    // What the epilogue needs from memory (scales, bias, residual, rotation, cache slot) is requested here,
+    // ahead of the weight stream: asked for after the reduction it would cost the kernel one more memory
+    // round trip with nothing else in flight.  Item q of this wavefront is accumulator wave + q * NWAVES
+    // (plain) or row group wave + q * NWAVES of both tiles (fused epilogues).
+    constexpr int NE = ((MODE == kEpiPlain ? NACC : MT * 4) + NWAVES - 1) / NWAVES;
+    float p_sx[NE], p_sw0[NE], p_sw1[NE], p_x0[NE], p_x1[NE];
+    uint32_t p_slot[NE];
+#pragma unroll
+    for (int q = 0; q < NE; ++q) {
+        p_sx[q] = p_sw0[q] = p_sw1[q] = p_x0[q] = p_x1[q] = 0.0f;
+        p_slot[q] = 0xffffffffu;
+        const int idx = wave + q * NWAVES;
+        if constexpr (MODE == kEpiPlain) {
+            const int e = idx % 4, j = (idx / 4) % NTW, i = idx / (4 * NTW);
+            const uint32_t row = i * 16 + 4 * (lane / 16) + e, col = (nt0 + j) * 16 + lane % 16;
+            if (idx < NACC && row < m && col < n) {
+                p_sx[q] = ep.sx[row];
+                p_sw0[q] = ep.sw[col];
+                if (ep.bias) p_x0[q] = ep.bias[col];
+                if (ep.residual) p_x1[q] = ep.residual[(uint64_t)row * n + col];
+            }
+        } else {
+            const int i = idx / 4, e = idx % 4;
+            const uint32_t row = i * 16 + 4 * (lane / 16) + e, col = nt0 * 16 + lane % 16;
+            const uint32_t pair = SWIGLU ? n / 2 : ep.head_dim / 2;      // distance to the partner column
+            if (idx < MT * 4 && row < m && col + pair < n) {
+                p_sx[q] = ep.sx[row];
+                p_sw0[q] = ep.sw[col];
+                p_sw1[q] = ep.sw[col + pair];
+                if constexpr (ROPE) {
+                    const uint32_t h = col / ep.head_dim, d = col % ep.head_dim;
+                    if (h < ep.heads + ep.kv_heads) {
+                        p_x0[q] = ep.cos_sin[(uint64_t)row * ep.head_dim + d];
+                        p_x1[q] = ep.cos_sin[(uint64_t)row * ep.head_dim + pair + d];
+                    }
+                    if (h >= ep.heads) p_slot[q] = ep.slots[row];
+                }
+            }
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
     v4i a[D][MT], b[D][NTW];
     auto load_slot = [&](int s, uint32_t it) {
         const uint32_t kt = wave + (it < cnt ? it : cnt - 1) * NWAVES;
@@ -95,7 +137,7 @@ __global__ void __launch_bounds__(NWAVES * 64)
         for (int j = 0; j < NTW; ++j) {
             uint32_t nt = nt0 + j * nt_step;
             nt = nt < n_tiles ? nt : n_tiles - 1;            // a tile past the edge is loaded clamped, never stored
-            b[s][j] = *(const v4i *)(b_base + ((uint64_t)nt * k_tiles + kt) * 1024);
+            b[s][j] = stream_load<true>((const v4i *)(b_base + ((uint64_t)nt * k_tiles + kt) * 1024));
         }
 #pragma unroll
         for (int i = 0; i < MT; ++i) a[s][i] = *(const v4i *)(xq_tiled + ((uint64_t)i * k_tiles + kt) * 1024 + a_off[i]);
@@ -135,7 +177,10 @@ __global__ void __launch_bounds__(NWAVES * 64)
 
     if constexpr (SWIGLU) {
         const uint32_t f = n / 2;
-        for (int q = wave; q < MT * 4; q += NWAVES) {
+#pragma unroll
+        for (int pq = 0; pq < NE; ++pq) {
+            const int q = wave + pq * NWAVES;
+            if (q >= MT * 4) break;
             int i = q / 4, e = q % 4;
             int sg = 0, su = 0;
 #pragma unroll
@@ -147,8 +192,8 @@ __global__ void __launch_bounds__(NWAVES * 64)
             uint32_t col = nt0 * 16 + lane % 16;
             float a = 0.0f;
             if (row < m && col < f) {
-                float vg = __fmul_rn((float)sg, __fmul_rn(ep.sx[row], ep.sw[col]));
-                float vu = __fmul_rn((float)su, __fmul_rn(ep.sx[row], ep.sw[col + f]));
+                float vg = __fmul_rn((float)sg, __fmul_rn(p_sx[pq], p_sw0[pq]));
+                float vu = __fmul_rn((float)su, __fmul_rn(p_sx[pq], p_sw1[pq]));
                 float act = silu_f32(vg) * vu;
                 ((float *)ep.out)[(uint64_t)row * f + col] = act;
                 a = fabsf(act);
@@ -163,7 +208,10 @@ __global__ void __launch_bounds__(NWAVES * 64)
     if constexpr (ROPE) {
         const uint32_t half = ep.head_dim / 2;
         const uint32_t eq = ep.heads * ep.head_dim, ekv = ep.kv_heads * ep.head_dim;
-        for (int q = wave; q < MT * 4; q += NWAVES) {
+#pragma unroll
+        for (int pq = 0; pq < NE; ++pq) {
+            const int q = wave + pq * NWAVES;
+            if (q >= MT * 4) break;
             int i = q / 4, e = q % 4;
             int s0 = 0, s1 = 0;
 #pragma unroll
@@ -174,14 +222,14 @@ __global__ void __launch_bounds__(NWAVES * 64)
             const uint32_t row = i * 16 + 4 * (lane / 16) + e;
             const uint32_t col = nt0 * 16 + lane % 16;             // first half of the head; partner at col + half
             if (row < m && col + half < n) {
-                float x0 = __fmul_rn((float)s0, __fmul_rn(ep.sx[row], ep.sw[col]));
-                float x1 = __fmul_rn((float)s1, __fmul_rn(ep.sx[row], ep.sw[col + half]));
+                float x0 = __fmul_rn((float)s0, __fmul_rn(p_sx[pq], p_sw0[pq]));
+                float x1 = __fmul_rn((float)s1, __fmul_rn(p_sx[pq], p_sw1[pq]));
                 const uint32_t h = col / ep.head_dim, d = col % ep.head_dim;
                 uint16_t *dst = nullptr;
                 if (h < ep.heads) {
                     dst = ep.q_out + (uint64_t)row * eq + (uint64_t)h * ep.head_dim + d;
                 } else {
-                    const uint64_t slot = ep.slots[row];
+                    const uint64_t slot = p_slot[pq];
                     if (slot < ep.pool_rows) {
                         const uint32_t hk = h - ep.heads;
                         dst = (hk < ep.kv_heads ? ep.k_pool + slot * ekv + (uint64_t)hk * ep.head_dim
@@ -189,8 +237,7 @@ __global__ void __launch_bounds__(NWAVES * 64)
                     }
                 }
                 if (h < ep.heads + ep.kv_heads) {
-                    const float c = ep.cos_sin[(uint64_t)row * ep.head_dim + d];
-                    const float sn = ep.cos_sin[(uint64_t)row * ep.head_dim + half + d];
+                    const float c = p_x0[pq], sn = p_x1[pq];
                     const float r0 = __fsub_rn(__fmul_rn(x0, c), __fmul_rn(x1, sn));
                     const float r1 = __fadd_rn(__fmul_rn(x1, c), __fmul_rn(x0, sn));
                     x0 = r0;
@@ -204,7 +251,10 @@ __global__ void __launch_bounds__(NWAVES * 64)
         }
         return;
     }
-    for (int idx = wave; idx < NACC; idx += NWAVES) {
+#pragma unroll
+    for (int pq = 0; pq < NE; ++pq) {
+        const int idx = wave + pq * NWAVES;
+        if (idx >= NACC) break;
         int sum = 0;
 #pragma unroll
         for (int w = 0; w < NWAVES; ++w) sum += red[w][idx][lane];
@@ -214,10 +264,10 @@ __global__ void __launch_bounds__(NWAVES * 64)
         if (row < m && col < n) {
             uint64_t o = (uint64_t)row * n + col;
             if (ep.acc_out) ep.acc_out[o] = sum;
-            float s = __fmul_rn(ep.sx[row], ep.sw[col]);
+            float s = __fmul_rn(p_sx[pq], p_sw0[pq]);
             float v = __fmul_rn((float)sum, s);
-            if (ep.bias) v = __fadd_rn(v, ep.bias[col]);
-            if (ep.residual) v = __fadd_rn(ep.residual[o], v);
+            if (ep.bias) v = __fadd_rn(v, p_x0[pq]);
+            if (ep.residual) v = __fadd_rn(p_x1[pq], v);
             if (ep.out_bf16)
                 ((uint16_t *)ep.out)[o] = f32_to_bf16(v);
             else
@@ -263,8 +313,30 @@ __global__ void __launch_bounds__(512)
         uint32_t nt = SWIGLU ? u + j * (n_tiles / 2) : 2 * u + j;
         return nt < last_tile ? nt : last_tile;
     };
-    auto load_unit = [&](uint32_t u, v4i (&b)[KTW][2]) {
+    // What the epilogue of a unit needs from memory travels with the unit's weights (requested first, so it
+    // is there before them): asked for after the reduction, these loads would queue behind the next unit's
+    // weight tiles, which are already in flight then, and the epilogue would wait for all of them.
+    // Wavefront w < 4 MT finishes rows 4 (l / 16) + w % 4 of row tile w / 4: its activation scale is fixed.
+    struct UnitEpi {
+        float sw[2], bias[2], res[2];
+    };
+    const uint32_t e_row = (wave / 4) * 16 + 4 * (lane / 16) + wave % 4;
+    const bool e_wave = wave < MT * 4 && e_row < m;
+    const float e_sx = e_wave ? ep.sx[e_row] : 0.0f;
+    auto load_unit = [&](uint32_t u, v4i (&b)[KTW][2], UnitEpi &ue) {
         u = u < n_units ? u : n_units - 1;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            ue.sw[j] = ue.bias[j] = ue.res[j] = 0.0f;
+            const uint32_t col = SWIGLU ? u * 16 + lane % 16 + j * (n / 2) : (2 * u + j) * 16 + lane % 16;
+            if (e_wave && col < n) {
+                ue.sw[j] = ep.sw[col];
+                if constexpr (!SWIGLU) {
+                    if (ep.bias) ue.bias[j] = ep.bias[col];
+                    if (ep.residual) ue.res[j] = ep.residual[(uint64_t)e_row * n + col];
+                }
+            }
+        }
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const int8_t *base = w_tiles + (uint64_t)tile_of(u, j) * k_tiles * 1024 + (uint64_t)lane * 16;
@@ -272,11 +344,11 @@ __global__ void __launch_bounds__(512)
             for (int t = 0; t < KTW; ++t) {
                 uint32_t kt = wave + NW * t;
                 kt = kt < k_tiles ? kt : last_kt;
-                b[t][j] = *(const v4i *)(base + (uint64_t)kt * 1024);
+                b[t][j] = stream_load<true>((const v4i *)(base + (uint64_t)kt * 1024));
             }
         }
     };
-    auto finish_unit = [&](uint32_t u, const v4i (&b)[KTW][2], int buf) {
+    auto finish_unit = [&](uint32_t u, const v4i (&b)[KTW][2], const UnitEpi &ue, int buf) {
         v4i acc[MT][2];
 #pragma unroll
         for (int i = 0; i < MT; ++i)
@@ -312,8 +384,8 @@ __global__ void __launch_bounds__(512)
                 const uint32_t f = n / 2, col = u * 16 + lane % 16;
                 float av = 0.0f;
                 if (row < m && col < f) {
-                    float vg = __fmul_rn((float)s0, __fmul_rn(ep.sx[row], ep.sw[col]));
-                    float vu = __fmul_rn((float)s1, __fmul_rn(ep.sx[row], ep.sw[col + f]));
+                    float vg = __fmul_rn((float)s0, __fmul_rn(e_sx, ue.sw[0]));
+                    float vu = __fmul_rn((float)s1, __fmul_rn(e_sx, ue.sw[1]));
                     float act = silu_f32(vg) * vu;
                     ((float *)ep.out)[(uint64_t)row * f + col] = act;
                     av = fabsf(act);
@@ -329,9 +401,9 @@ __global__ void __launch_bounds__(512)
                     if (row < m && col < n) {
                         uint64_t o = (uint64_t)row * n + col;
                         if (ep.acc_out) ep.acc_out[o] = sum;
-                        float v = __fmul_rn((float)sum, __fmul_rn(ep.sx[row], ep.sw[col]));
-                        if (ep.bias) v = __fadd_rn(v, ep.bias[col]);
-                        if (ep.residual) v = __fadd_rn(ep.residual[o], v);
+                        float v = __fmul_rn((float)sum, __fmul_rn(e_sx, ue.sw[j]));
+                        if (ep.bias) v = __fadd_rn(v, ue.bias[j]);
+                        if (ep.residual) v = __fadd_rn(ue.res[j], v);
                         if (ep.out_bf16)
                             ((uint16_t *)ep.out)[o] = f32_to_bf16(v);
                         else
@@ -345,14 +417,15 @@ __global__ void __launch_bounds__(512)
     // two units per trip so that the two weight register sets have fixed names; buffer u % 2 of `red` is
     // rewritten two units later, after the barrier of the unit in between
     v4i b0[KTW][2], b1[KTW][2];
+    UnitEpi ue0, ue1;
     uint32_t u = blockIdx.x;
-    load_unit(u, b0);
+    load_unit(u, b0, ue0);
     for (; u < n_units; u += 2 * gridDim.x) {
-        load_unit(u + gridDim.x, b1);
-        finish_unit(u, b0, 0);
+        load_unit(u + gridDim.x, b1, ue1);
+        finish_unit(u, b0, ue0, 0);
         if (u + gridDim.x >= n_units) break;
-        load_unit(u + 2 * gridDim.x, b0);
-        finish_unit(u + gridDim.x, b1, 1);
+        load_unit(u + 2 * gridDim.x, b0, ue0);
+        finish_unit(u + gridDim.x, b1, ue1, 1);
     }
 }
 
@@ -376,7 +449,11 @@ __device__ __forceinline__ void cvt_i8x8_bf16(uint32_t w0, uint32_t w1, v8bf *ou
 // A lane's 16 weight bytes are k = 64*kt + 16*g + 0..15; the first eight feed
 // one instruction, the last eight the next, and the activation operand uses the
 // same split, so the two instructions together cover the tile's 64 k-values.
-template <int MT, int NTW, int NWAVES>
+// RING: the k-tiles go through a ring of register slots (below); otherwise groups of D k-tiles are loaded,
+// waited for and multiplied in turn.  The ring is the faster form while a wavefront's share of k fits a few
+// groups (k = 4096: 10.4 against 11.2 us at 12288 columns and one row); with a deep k and eight or more rows
+// the group form is (k = 11008, 32 rows: 24.1 against 25.6 us), so the launcher picks by k.
+template <int MT, int NTW, int NWAVES, bool RING>
 __global__ void __launch_bounds__(NWAVES * 64)
     w8a16_skinny_kernel(const uint16_t *__restrict__ a, const int8_t *__restrict__ w_tiles,
                         const float *__restrict__ sw, uint32_t m, uint32_t n, uint32_t n_tiles, uint32_t k_tiles,
@@ -395,59 +472,119 @@ __global__ void __launch_bounds__(NWAVES * 64)
         for (int j = 0; j < NTW; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
 
     const int8_t *b_base = w_tiles + (uint64_t)lane * 16;
-    constexpr int U = (MT * NTW >= 4) ? 2 : 4;
     const uint32_t cnt = k_tiles > (uint32_t)wave ? (k_tiles - wave + NWAVES - 1) / NWAVES : 0;
-    auto load_b = [&](uint32_t kt, v4u *braw) {
+    // the channel scales of the epilogue are requested ahead of the weight stream (see w8a8_skinny_kernel)
+    constexpr int NE = (NACC + NWAVES - 1) / NWAVES;
+    float p_sw[NE];
+#pragma unroll
+    for (int q = 0; q < NE; ++q) {
+        const int idx = wave + q * NWAVES;
+        const uint32_t col = (nt0 + (idx / 4) % NTW) * 16 + r;
+        p_sw[q] = idx < NACC && col < n ? sw[col] : 0.0f;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // A ring of D register slots (the weight tiles and the activation tiles of one k-tile each), refilled
+    // behind every multiply, as in w8a8_skinny_kernel: the loads of D k-tiles stay in flight throughout.
+    // Loads past the wavefront's last k-tile repeat it (never multiplied) and column tiles past the edge repeat
+    // the last one (never stored), so the count of outstanding loads is the same on every path; lanes of rows
+    // at or past m read row 0 of their k-group, bytes that its own lane fetches anyway.
+    // (D = 8 only where the slots leave the kernel at 128 registers, i.e. two blocks per compute unit)
+    constexpr int D = (MT * NTW >= 2) ? 4 : 8;
+    const uint32_t last_tile = n_tiles - 1;
+    uint32_t a_row[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) a_row[i] = (uint32_t)i * 16 + r < m ? (uint32_t)i * 16 + r : 0u;
+    v4u braw[D][NTW], lo[D][MT], hi[D][MT];
+    auto load_slot = [&](int s_, uint32_t it) {
+        const uint32_t kt = wave + (it < cnt ? it : cnt - 1) * NWAVES;
 #pragma unroll
         for (int j = 0; j < NTW; ++j) {
             uint32_t nt = nt0 + j;
-            braw[j] = nt < n_tiles ? *(const v4u *)(b_base + ((uint64_t)nt * k_tiles + kt) * 1024) : v4u{0, 0, 0, 0};
+            nt = nt < last_tile ? nt : last_tile;
+            braw[s_][j] = stream_load<true>((const v4u *)(b_base + ((uint64_t)nt * k_tiles + kt) * 1024));
         }
-    };
-    auto load_a = [&](uint32_t kt, v4u *lo, v4u *hi) {
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
-            uint32_t row = i * 16 + r;
-            lo[i] = v4u{0, 0, 0, 0};
-            hi[i] = v4u{0, 0, 0, 0};
-            if (row < m) {
-                const v4u *p = (const v4u *)(a + (uint64_t)row * k + (uint64_t)kt * 64 + g * 16);
-                lo[i] = p[0];
-                hi[i] = p[1];
-            }
+            const v4u *p = (const v4u *)(a + (uint64_t)a_row[i] * k + (uint64_t)kt * 64 + g * 16);
+            lo[s_][i] = p[0];
+            hi[s_][i] = p[1];
         }
     };
-    auto mma = [&](const v4u *lo, const v4u *hi, const v4u *braw) {
+    auto mma_slot = [&](int s_) {
 #pragma unroll
         for (int j = 0; j < NTW; ++j) {
             v8bf blo, bhi;
-            cvt_i8x8_bf16(braw[j][0], braw[j][1], &blo);
-            cvt_i8x8_bf16(braw[j][2], braw[j][3], &bhi);
+            cvt_i8x8_bf16(braw[s_][j][0], braw[s_][j][1], &blo);
+            cvt_i8x8_bf16(braw[s_][j][2], braw[s_][j][3], &bhi);
 #pragma unroll
             for (int i = 0; i < MT; ++i) {
-                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, lo[i]), blo, acc[i][j], 0, 0, 0);
-                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, hi[i]), bhi, acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, lo[s_][i]), blo, acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, hi[s_][i]), bhi, acc[i][j], 0, 0, 0);
             }
         }
     };
-    uint32_t it = 0;
-    for (; it + U <= cnt; it += U) {
-        v4u braw[U][NTW], lo[U][MT], hi[U][MT];
+    if (cnt != 0 && RING) {
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            uint32_t kt = wave + (it + u) * NWAVES;
-            load_b(kt, braw[u]);
-            load_a(kt, lo[u], hi[u]);
+        for (int s_ = 0; s_ < D; ++s_) load_slot(s_, (uint32_t)s_);
+        uint32_t it0 = 0;
+        for (; it0 + D < cnt; it0 += D) {
+#pragma unroll
+            for (int s_ = 0; s_ < D; ++s_) {
+                mma_slot(s_);
+                __builtin_amdgcn_sched_barrier(0);
+                load_slot(s_, it0 + D + s_);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
 #pragma unroll
-        for (int u = 0; u < U; ++u) mma(lo[u], hi[u], braw[u]);
-    }
-    for (; it < cnt; ++it) {
-        v4u braw[NTW], lo[MT], hi[MT];
-        uint32_t kt = wave + it * NWAVES;
-        load_b(kt, braw);
-        load_a(kt, lo, hi);
-        mma(lo, hi, braw);
+        for (int s_ = 0; s_ < D; ++s_)
+            if (it0 + s_ < cnt) mma_slot(s_);
+    } else if (cnt != 0) {
+        constexpr int U = (MT * NTW >= 4) ? 2 : 4;
+        auto load_group = [&](uint32_t kt, v4u *bw, v4u *l, v4u *h) {
+#pragma unroll
+            for (int j = 0; j < NTW; ++j) {
+                const uint32_t nt = nt0 + j;
+                bw[j] = nt < n_tiles ? stream_load<true>((const v4u *)(b_base + ((uint64_t)nt * k_tiles + kt) * 1024)) : v4u{0, 0, 0, 0};
+            }
+#pragma unroll
+            for (int i = 0; i < MT; ++i) {
+                const uint32_t row = i * 16 + r;
+                l[i] = v4u{0, 0, 0, 0};
+                h[i] = v4u{0, 0, 0, 0};
+                if (row < m) {
+                    const v4u *p = (const v4u *)(a + (uint64_t)row * k + (uint64_t)kt * 64 + g * 16);
+                    l[i] = p[0];
+                    h[i] = p[1];
+                }
+            }
+        };
+        auto mma_group = [&](const v4u *l, const v4u *h, const v4u *bw) {
+#pragma unroll
+            for (int j = 0; j < NTW; ++j) {
+                v8bf blo, bhi;
+                cvt_i8x8_bf16(bw[j][0], bw[j][1], &blo);
+                cvt_i8x8_bf16(bw[j][2], bw[j][3], &bhi);
+#pragma unroll
+                for (int i = 0; i < MT; ++i) {
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, l[i]), blo, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, h[i]), bhi, acc[i][j], 0, 0, 0);
+                }
+            }
+        };
+        uint32_t it = 0;
+        for (; it + U <= cnt; it += U) {
+            v4u bw[U][NTW], l[U][MT], h[U][MT];
+#pragma unroll
+            for (int u = 0; u < U; ++u) load_group(wave + (it + u) * NWAVES, bw[u], l[u], h[u]);
+#pragma unroll
+            for (int u = 0; u < U; ++u) mma_group(l[u], h[u], bw[u]);
+        }
+        for (; it < cnt; ++it) {
+            v4u bw[NTW], l[MT], h[MT];
+            load_group(wave + it * NWAVES, bw, l, h);
+            mma_group(l, h, bw);
+        }
     }
 
 #pragma unroll
@@ -458,7 +595,10 @@ __global__ void __launch_bounds__(NWAVES * 64)
             for (int e = 0; e < 4; ++e) red[wave][(i * NTW + j) * 4 + e][lane] = acc[i][j][e];
     __syncthreads();
 
-    for (int idx = wave; idx < NACC; idx += NWAVES) {
+#pragma unroll
+    for (int pq = 0; pq < NE; ++pq) {
+        const int idx = wave + pq * NWAVES;
+        if (idx >= NACC) break;
         float sum = red[0][idx][lane];
 #pragma unroll
         for (int w = 1; w < NWAVES; ++w) sum = __fadd_rn(sum, red[w][idx][lane]);
@@ -466,7 +606,7 @@ __global__ void __launch_bounds__(NWAVES * 64)
         uint32_t row = i * 16 + 4 * g + e;
         uint32_t col = (nt0 + j) * 16 + r;
         if (row < m && col < n) {
-            float v = __fmul_rn(sum, sw[col]);
+            float v = __fmul_rn(sum, p_sw[pq]);
             uint64_t o = (uint64_t)row * n + col;
             if (out_bf16)
                 ((uint16_t *)out)[o] = f32_to_bf16(v);
@@ -508,17 +648,19 @@ __global__ void __launch_bounds__(512)
             hi[t][i] = p[1];
         }
     }
-    auto load_tile = [&](uint32_t nt, v4u (&b)[KTW]) {
+    // the channel scale of a tile travels with its weights (see w8a8_astat_kernel)
+    auto load_tile = [&](uint32_t nt, v4u (&b)[KTW], float &scale) {
         nt = nt < n_tiles ? nt : n_tiles - 1;
+        scale = wave < NACC && nt * 16 + r < n ? sw[nt * 16 + r] : 0.0f;
         const int8_t *base = w_tiles + (uint64_t)nt * k_tiles * 1024 + (uint64_t)lane * 16;
 #pragma unroll
         for (int t = 0; t < KTW; ++t) {
             uint32_t kt = wave + NW * t;
             kt = kt < k_tiles ? kt : last_kt;
-            b[t] = *(const v4u *)(base + (uint64_t)kt * 1024);
+            b[t] = stream_load<true>((const v4u *)(base + (uint64_t)kt * 1024));
         }
     };
-    auto finish_tile = [&](uint32_t nt, const v4u (&b)[KTW], int buf) {
+    auto finish_tile = [&](uint32_t nt, const v4u (&b)[KTW], float scale, int buf) {
         v4f acc[MT];
 #pragma unroll
         for (int i = 0; i < MT; ++i) acc[i] = v4f{0.f, 0.f, 0.f, 0.f};
@@ -547,7 +689,7 @@ __global__ void __launch_bounds__(512)
             const int i = wave / 4, e = wave % 4;
             const uint32_t row = i * 16 + 4 * g + e, col = nt * 16 + r;
             if (row < m && col < n) {
-                float v = __fmul_rn(sum, sw[col]);
+                float v = __fmul_rn(sum, scale);
                 uint64_t o = (uint64_t)row * n + col;
                 if (out_bf16)
                     ((uint16_t *)out)[o] = f32_to_bf16(v);
@@ -557,14 +699,15 @@ __global__ void __launch_bounds__(512)
         }
     };
     v4u b0[KTW], b1[KTW];
+    float sc0, sc1;
     uint32_t nt = blockIdx.x;
-    load_tile(nt, b0);
+    load_tile(nt, b0, sc0);
     for (; nt < n_tiles; nt += 2 * gridDim.x) {
-        load_tile(nt + gridDim.x, b1);
-        finish_tile(nt, b0, 0);
+        load_tile(nt + gridDim.x, b1, sc1);
+        finish_tile(nt, b0, sc0, 0);
         if (nt + gridDim.x >= n_tiles) break;
-        load_tile(nt + 2 * gridDim.x, b0);
-        finish_tile(nt + gridDim.x, b1, 1);
+        load_tile(nt + 2 * gridDim.x, b0, sc0);
+        finish_tile(nt + gridDim.x, b1, sc1, 1);
     }
 }
 
@@ -598,12 +741,25 @@ __global__ void __launch_bounds__(NWAVES * 64)
         a_base[i] = aq + (uint64_t)row * k_bytes + (uint64_t)(lane / 16) * 32;
     }
     const uint32_t cnt = k_tiles > (uint32_t)wave ? (k_tiles - wave + NWAVES - 1) / NWAVES : 0;
+    // scales and bias of the epilogue, requested ahead of the weight stream (see w8a8_skinny_kernel)
+    constexpr int NE = (NACC + NWAVES - 1) / NWAVES;
+    float p_sx[NE], p_sw[NE], p_bias[NE];
+#pragma unroll
+    for (int q = 0; q < NE; ++q) {
+        const int idx = wave + q * NWAVES;
+        const uint32_t row = (idx / 4) * 16 + 4 * (lane / 16) + idx % 4, col = nt * 16 + lane % 16;
+        const bool live = idx < NACC && row < m && col < n;
+        p_sx[q] = live ? sx[row] : 0.0f;
+        p_sw[q] = live ? sw[col] : 0.0f;
+        p_bias[q] = live && bias ? bias[col] : 0.0f;
+    }
+    __builtin_amdgcn_sched_barrier(0);
     v4i a[D][MT][2], b[D][2];
     auto load_slot = [&](int s, uint32_t it) {
         const uint32_t kt = wave + (it < cnt ? it : cnt - 1) * NWAVES;
         const v4i *bp = (const v4i *)(b_base + (uint64_t)kt * 2048);
-        b[s][0] = bp[0];
-        b[s][1] = bp[1];
+        b[s][0] = stream_load<true>(bp);
+        b[s][1] = stream_load<true>(bp + 1);
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
             const v4i *ap = (const v4i *)(a_base[i] + (uint64_t)kt * 128);
@@ -642,15 +798,18 @@ __global__ void __launch_bounds__(NWAVES * 64)
 #pragma unroll
         for (int e = 0; e < 4; ++e) red[wave][i * 4 + e][lane] = acc[i][e];
     __syncthreads();
-    for (int idx = wave; idx < NACC; idx += NWAVES) {
+#pragma unroll
+    for (int pq = 0; pq < NE; ++pq) {
+        const int idx = wave + pq * NWAVES;
+        if (idx >= NACC) break;
         float sum = red[0][idx][lane];
 #pragma unroll
         for (int w = 1; w < NWAVES; ++w) sum = __fadd_rn(sum, red[w][idx][lane]);
         const int e = idx % 4, i = idx / 4;
         const uint32_t row = i * 16 + 4 * (lane / 16) + e, col = nt * 16 + lane % 16;
         if (row < m && col < n) {
-            float v = __fmul_rn(sum, __fmul_rn(sx[row], sw[col]));
-            if (bias) v = __fadd_rn(v, bias[col]);
+            float v = __fmul_rn(sum, __fmul_rn(p_sx[pq], p_sw[pq]));
+            if (bias) v = __fadd_rn(v, p_bias[pq]);
             const uint64_t o = (uint64_t)row * n + col;
             if (out_bf16)
                 ((uint16_t *)out)[o] = f32_to_bf16(v);
@@ -703,18 +862,27 @@ void launch_w8a8_rows(uint64_t m, int waves, unsigned grid, hipStream_t s, A... 
         go(std::integral_constant<int, 4>{});
 }
 
+template <int MT, bool RING>
+void launch_w8a16_form(const uint16_t *a, const int8_t *wt, const float *sw, uint32_t m, uint32_t n, uint32_t n_tiles,
+                       uint32_t k_tiles, void *out, int out_bf16, int ntw, int waves, hipStream_t s) {
+    unsigned grid = (n_tiles + ntw - 1) / ntw;
+    if (ntw == 1 && waves == 8)
+        w8a16_skinny_kernel<MT, 1, 8, RING><<<grid, 512, 0, s>>>(a, wt, sw, m, n, n_tiles, k_tiles, out, out_bf16);
+    else if (ntw == 1)
+        w8a16_skinny_kernel<MT, 1, 4, RING><<<grid, 256, 0, s>>>(a, wt, sw, m, n, n_tiles, k_tiles, out, out_bf16);
+    else if (waves == 8)
+        w8a16_skinny_kernel<MT, 2, 8, RING><<<grid, 512, 0, s>>>(a, wt, sw, m, n, n_tiles, k_tiles, out, out_bf16);
+    else
+        w8a16_skinny_kernel<MT, 2, 4, RING><<<grid, 256, 0, s>>>(a, wt, sw, m, n, n_tiles, k_tiles, out, out_bf16);
+}
+
 template <int MT>
 void launch_w8a16(const uint16_t *a, const int8_t *wt, const float *sw, uint32_t m, uint32_t n, uint32_t n_tiles,
                   uint32_t k_tiles, void *out, int out_bf16, int ntw, int waves, hipStream_t s) {
-    unsigned grid = (n_tiles + ntw - 1) / ntw;
-    if (ntw == 1 && waves == 8)
-        w8a16_skinny_kernel<MT, 1, 8><<<grid, 512, 0, s>>>(a, wt, sw, m, n, n_tiles, k_tiles, out, out_bf16);
-    else if (ntw == 1)
-        w8a16_skinny_kernel<MT, 1, 4><<<grid, 256, 0, s>>>(a, wt, sw, m, n, n_tiles, k_tiles, out, out_bf16);
-    else if (waves == 8)
-        w8a16_skinny_kernel<MT, 2, 8><<<grid, 512, 0, s>>>(a, wt, sw, m, n, n_tiles, k_tiles, out, out_bf16);
+    if (k_tiles <= 64 || m == 1)
+        launch_w8a16_form<MT, true>(a, wt, sw, m, n, n_tiles, k_tiles, out, out_bf16, ntw, waves, s);
     else
-        w8a16_skinny_kernel<MT, 2, 4><<<grid, 256, 0, s>>>(a, wt, sw, m, n, n_tiles, k_tiles, out, out_bf16);
+        launch_w8a16_form<MT, false>(a, wt, sw, m, n, n_tiles, k_tiles, out, out_bf16, ntw, waves, s);
 }
 
 }  // namespace

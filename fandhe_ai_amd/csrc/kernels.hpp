@@ -260,7 +260,8 @@ void sample_rows_policy(const float *logits, int32_t *tokens, RowPolicy *policy,
 // Launches a register-only loop of one matrix instruction kind (0: i32_16x16x64_i8, 1: i32_32x32x32_i8,
 // 2: scaled f32_16x16x128 on e4m3) whose operand bits come from `operands` (64 KiB); returns the number
 // of multiply-add operations x 2 the launch performs.  sink: one int, never written in practice.
-// Plain streaming read of `bytes` (a multiple of 16 * blocks) by `blocks` blocks of `threads` threads.
+// Streaming read of `bytes` (a multiple of 16 * blocks) by `blocks` blocks of `threads` threads (non-temporal
+// loads unless tuning key 15 asks for ordinary ones).
 void stream_read_probe(const void *src, uint64_t bytes, int blocks, int threads, int *sink, hipStream_t s);
 double matrix_rate_probe(int kind, const void *operands, uint32_t iters, int num_cus, int *sink, hipStream_t s);
 

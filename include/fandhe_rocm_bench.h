@@ -63,7 +63,9 @@ fa_status fa_probe_stream_read(fa_context *ctx, const fa_buffer *src, uint64_t o
  *        kernel, 2 the matrix-core kernel, 0 by shape;
  * key 14: weights that the row kernels of the decode step pull into L2 for the projection that follows them: 1 none,
  *        n >= 2: n MiB of q | k | v and 2 n MiB of the o projection (0: 12 / 24); takes effect when a step is
- *        recorded, so set it before the first step of a batch size. */
+ *        recorded, so set it before the first step of a batch size;
+ * key 15: loads of fa_probe_stream_read: 1 ordinary loads, 0 the non-temporal loads that the kernels use for
+ *        data they read once. */
 fa_status fa_set_tuning(int32_t key, int32_t value);
 
 /* Which kernel a prefill-shape GEMM of m rows against `qw` is launched with under the
