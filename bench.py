@@ -32,7 +32,7 @@ MFMA_PEAK_TOPS = 5000.0          # dense int8 and fp8 on MI355X
 # HBM bytes per launch of decode_stream_kernel at this benchmark's shape, from hardware counters
 # (rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE, each scaled by the same counter's reading for a plain
 # row-copy kernel of known size; the figures are in profiles/decode_stream_kernel_config5_pmc.txt).
-ATTENTION_TRAFFIC_BYTES = 627567353
+ATTENTION_TRAFFIC_BYTES = 635879260
 U32MAX = 0xFFFFFFFF
 SERVING_ROWS = 64          # rows of the continuous-batching run (the decoder's limit)
 
