@@ -31,10 +31,11 @@ fa_status fa_fill_normal(fa_context *ctx, fa_buffer *buf, uint64_t offset, uint6
 fa_status fa_probe_matrix_rate(fa_context *ctx, int32_t kind, const fa_buffer *operands,
                                uint32_t iters, fa_buffer *sink, double *ops);
 
-/* Queues a plain streaming read of `bytes` starting `offset_bytes` into `src`: `blocks` blocks of `threads`
+/* Queues a streaming read of `bytes` starting `offset_bytes` into `src`: `blocks` blocks of `threads`
  * (256 or 512) threads, each reading its own contiguous share with 16-byte loads, eight per thread in
- * flight, nothing written.  The time of this launch is the floor for a memory-bound kernel that must
- * fetch that many bytes; time it with an fa_timer. */
+ * flight, nothing written; the loads are the non-temporal ones the kernels use for read-once data unless
+ * tuning key 15 asks for ordinary loads.  The time of this launch is the floor for a memory-bound kernel
+ * that must fetch that many bytes; time it with an fa_timer. */
 fa_status fa_probe_stream_read(fa_context *ctx, const fa_buffer *src, uint64_t offset_bytes, uint64_t bytes,
                                int32_t blocks, int32_t threads, fa_buffer *sink);
 

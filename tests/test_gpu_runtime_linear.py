@@ -371,3 +371,30 @@ def test_captured_quantized_linear_owns_its_scratch():
         g = C.c_void_p()
         lib.fa_graph_capture_end(be._ctx, C.byref(g))
         lib.fa_graph_destroy(be._ctx, g)
+
+
+def test_stream_read_probe_runs_with_both_load_kinds_and_checks_its_range():
+    """The read-floor probe of the benchmark (non-temporal and ordinary loads) reads only what it is given and
+    writes nothing; ranges past the buffer, misaligned offsets and bad launch shapes are argument errors."""
+    import fandhe_ai_amd as fa
+    be = ops()
+    lib = fa.capi.lib
+    n = 1 << 20
+    host = np.random.default_rng(5).standard_normal(n).astype(np.float32)
+    src = be.upload(host)
+    sink = be.alloc_zeroed((1,), fa.capi.I32)
+    try:
+        for plain in (0, 1):
+            fa.check(lib.fa_set_tuning(15, plain))
+            for blocks, threads, off, nbytes in ((512, 512, 0, 4 * n), (256, 256, 4096, 4 * n - 4096), (7, 512, 16, 16 * 7 * 513),
+                                                 (64, 256, 0, 16 * 63), (1, 256, 4 * n - 16, 16)):
+                fa.check(lib.fa_probe_stream_read(be._ctx, src._h, off, nbytes, blocks, threads, sink._h))
+        be.synchronize_device()
+        assert int(be.download(sink)[0]) == 0 and np.array_equal(be.download(src), host)
+        for blocks, threads, off, nbytes in ((512, 512, 0, 4 * n + 16), (512, 512, 8, 1024), (0, 512, 0, 1024), (512, 128, 0, 1024),
+                                             (70000, 512, 0, 1024), (512, 512, 4 * n, 16)):
+            assert lib.fa_probe_stream_read(be._ctx, src._h, off, nbytes, blocks, threads, sink._h) == fa.capi.INVALID_ARGUMENT
+    finally:
+        fa.check(lib.fa_set_tuning(15, 0))
+        src.free()
+        sink.free()
