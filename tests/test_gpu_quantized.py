@@ -176,16 +176,33 @@ def test_w8a8_split_k_gemm_is_bit_exact(m, k, n):
 
 
 def test_w8a8_ragged_shapes():
+    """Shapes off every tile size, with and without a bias, under one and two column tiles per block and four and
+    eight wavefronts (wavefronts without a k-tile, fewer k-tiles than ring slots, a clamped last column tile): the
+    epilogue's operands are fetched ahead of the stream by index, so every edge has to agree with the tail's."""
+    fa = _fa()
     be = ops()
+    lib = fa.capi.lib
     rng = o.Rng(13)
-    for m, k, n in ((3, 100, 37), (16, 64, 16), (32, 130, 70), (7, 4097, 33)):
-        x = rng.randn((m, k))
-        w = rng.randn((k, n), std=0.05)
-        wq, ws = o.quantize_cols_i8(w)
-        want_acc, want = o.linear_w8a8(x, wq, ws)
-        out, acc = be.linear_w8a8(be.upload(x), be.import_quantized_weight(wq, ws), want_acc=True)
-        assert np.array_equal(be.download_owned(acc), want_acc), (m, k, n)
-        assert np.array_equal(be.download_owned(out), want), (m, k, n)
+    try:
+        for m, k, n in ((3, 100, 37), (16, 64, 16), (32, 130, 70), (7, 4097, 33), (1, 64, 1), (64, 1000, 250), (33, 14336, 24)):
+            x = rng.randn((m, k))
+            w = rng.randn((k, n), std=0.05)
+            bias = rng.randn((n,))
+            wq, ws = o.quantize_cols_i8(w)
+            qw = be.import_quantized_weight(wq, ws)
+            dx = be.upload(x)
+            dbias = fa.DeviceBufferView(be.upload(bias), 0, (n,))
+            for with_bias in (False, True):
+                want_acc, want = o.linear_w8a8(x, wq, ws, bias if with_bias else None)
+                for ntw, waves in ((0, 0), (1, 4), (1, 8), (2, 4), (2, 8)):
+                    fa.check(lib.fa_set_tuning(0, ntw))
+                    fa.check(lib.fa_set_tuning(1, waves))
+                    out, acc = be.linear_w8a8(dx, qw, bias=dbias if with_bias else None, want_acc=True)
+                    assert np.array_equal(be.download_owned(acc), want_acc), (m, k, n, with_bias, ntw, waves)
+                    assert np.array_equal(be.download_owned(out), want), (m, k, n, with_bias, ntw, waves)
+    finally:
+        fa.check(lib.fa_set_tuning(0, 0))
+        fa.check(lib.fa_set_tuning(1, 0))
 
 
 def test_w8a8_activation_stationary_kernel_is_bit_exact():
@@ -259,6 +276,36 @@ def test_w8a16_rejects_shapes_outside_its_contract():
         be.linear_w8a16(be.upload(np.zeros((33, 128), np.uint16)), qw)
     with pytest.raises(fa.ShapeMismatch):
         be.linear_w8a16(be.upload(np.zeros((2, 64), np.uint16)), qw)
+
+
+def test_w8a16_ragged_shapes_under_every_launch_shape():
+    """Row counts off the tile size, column counts that leave a half-filled last tile or an odd number of
+    tiles, k of one to 172 tiles (wavefronts without a k-tile of their own, fewer k-tiles than ring slots,
+    the deep-k loop form), under one and two column tiles per block and four and eight wavefronts."""
+    fa = _fa()
+    be = ops()
+    lib = fa.capi.lib
+    o.set_threads(8)
+    try:
+        for m, k, n in ((3, 128, 40), (17, 192, 16), (32, 4096, 1000), (5, 11008, 48), (16, 64, 8), (1, 320, 33),
+                        (9, 1024, 272), (32, 11008, 100)):
+            rng = o.Rng(m * 7 + k + n)
+            wq, ws = o.quantize_cols_i8(rng.randn((k, n), std=0.02))
+            qw = be.import_quantized_weight(wq, ws)
+            a = o.to_bf16(rng.randn((m, k)))
+            want = o.linear_w8a16(a, wq, ws)
+            da = be.upload(a)
+            for ntw in (1, 2):
+                for waves in (4, 8):
+                    fa.check(lib.fa_set_tuning(0, ntw))
+                    fa.check(lib.fa_set_tuning(1, waves))
+                    got = be.download_owned(be.linear_w8a16(da, qw, fa.capi.F32))
+                    assert got.shape == (m, n)
+                    assert_parity("W8A16_PARITY", f"{m}x{n}x{k}:ntw{ntw}:w{waves}", got, want)
+    finally:
+        fa.check(lib.fa_set_tuning(0, 0))
+        fa.check(lib.fa_set_tuning(1, 0))
+        o.set_threads(1)
 
 
 def test_w8a16_one_hot_rows_pick_weight_rows_exactly():
