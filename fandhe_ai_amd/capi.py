@@ -213,6 +213,7 @@ SIGNATURES = {
     "fa_gemm_f32_form_query": (C.c_int32, [u64, u64, u64, C.POINTER(C.c_int32)]),
     "fa_gemm_plan_query": (C.c_int32, [ctx_p, u64, qw_p, C.POINTER(GemmPlan)]),
     "fa_graph_owned_blocks": (C.c_int32, [C.c_void_p, C.POINTER(C.c_void_p), u64, C.POINTER(u64)]),
+    "fa_topology_query": (C.c_int32, [ctx_p, i32p, i32p]),
 }
 
 for _name, (_res, _args) in SIGNATURES.items():

@@ -12,7 +12,8 @@ using namespace fa;
 
 namespace fa {
 namespace k {
-extern int g_gemm_f32_form, g_weight_prefetch, g_probe_plain_loads;
+extern int g_gemm_f32_form, g_weight_prefetch, g_probe_plain_loads, g_rows_wide;
+extern int g_skinny_ksplit, g_skinny_ksplit_s;
 extern int g_skinny_ntw, g_skinny_waves, g_skinny_astat, g_gemm_small_tiles, g_gemm_waves, g_gemm_ntb, g_gemm_split_fill;
 }
 int g_decode_waves = 0;
@@ -90,6 +91,9 @@ fa_status fa_set_tuning(int32_t key, int32_t value) {
         case 13: k::g_gemm_f32_form = value; return FA_OK;
         case 14: k::g_weight_prefetch = value; return FA_OK;
         case 15: k::g_probe_plain_loads = value; return FA_OK;
+        case 16: k::g_skinny_ksplit = value; return FA_OK;
+        case 17: k::g_skinny_ksplit_s = value; return FA_OK;
+        case 18: k::g_rows_wide = value; return FA_OK;
     }
     return fail(FA_ERR_INVALID_ARGUMENT, "fa_set_tuning: unknown key");
 }
@@ -333,7 +337,7 @@ fa_status fa_linear_w8a8(fa_context *ctx, const fa_buffer *x, uint64_t m, const 
         k::quantize_rows_i8(x->ptr, x->dtype == FA_BF16, nullptr, (int8_t *)xq.ptr, (float *)sx.ptr, m, m_pad, qw->k,
                             qw->k_pad, ctx->stream);
         k::linear_w8a8_skinny((const int8_t *)xq.ptr, (const int8_t *)qw->codes->ptr, m, qw->n, qw->n_pad, qw->k_pad,
-                              ep, ctx->props.multiProcessorCount, ctx->stream);
+                              ep, ctx->props.multiProcessorCount, ctx->stream, &ctx->splitk);
     } else {
         if (qw->k != qw->k_pad) return fail(FA_ERR_UNSUPPORTED, "linear_w8a8: m > 64 needs k to be a multiple of 64");
         if (fa_status s = xq.get(mk)) return s;
@@ -390,7 +394,7 @@ fa_status fa_linear_w8a16(fa_context *ctx, const fa_buffer *a, uint64_t m, const
     if (mn == 0) return FA_OK;
     k::linear_w8a16_skinny((const uint16_t *)a->ptr, (const int8_t *)qw->codes->ptr, (const float *)qw->scales->ptr, m,
                            qw->n, qw->n_pad, qw->k_pad, out->ptr, out->dtype == FA_BF16,
-                           ctx->props.multiProcessorCount, ctx->stream);
+                           ctx->props.multiProcessorCount, ctx->stream, &ctx->splitk);
     return after_launch(ctx, "linear_w8a16_skinny");
 }
 

@@ -164,7 +164,7 @@ fa_status enqueue_step(fa_context *ctx, fa_decoder *d, int stop_after = -1) {
     };
     auto linear = [&](const fa_qweight *w, void *out, const float *residual) {
         k::linear_w8a8_skinny((const int8_t *)d->xq->ptr, (const int8_t *)w->codes->ptr, B, w->n, w->n_pad, w->k_pad,
-                              epilogue(w, out, residual), cus, s);
+                              epilogue(w, out, residual), cus, s, &ctx->splitk);
     };
 
     // The row kernels in front of the two small projections pull those projections' weights into L2 while they wait
@@ -175,7 +175,7 @@ fa_status enqueue_step(fa_context *ctx, fa_decoder *d, int stop_after = -1) {
     const uint64_t pull_scale = k::g_weight_prefetch >= 2 ? (uint64_t)k::g_weight_prefetch : 12;
     const uint64_t kPullQkv = pull_scale << 20, kPullO = (2 * pull_scale) << 20;
     auto pull_plain = [&](const fa_qweight *w, uint64_t budget) {
-        return k::prefetch_for_linear_w8a8_skinny((const int8_t *)w->codes->ptr, B, w->n_pad, w->k_pad, cus, budget);
+        return k::prefetch_for_linear_w8a8_skinny((const int8_t *)w->codes->ptr, B, w->n_pad, w->k_pad, cus, budget, &ctx->splitk);
     };
     for (uint32_t li = 0; li < c.n_layers; ++li) {
         const fa_decoder::Layer &L = d->layers[li];

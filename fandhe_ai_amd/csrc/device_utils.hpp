@@ -54,12 +54,70 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
-// Block-wide reductions for blocks of NWAVES wavefronts; `smem` needs NWAVES slots.
-template <typename T, int NWAVES>
+// The same reductions on the DPP data path.  A __shfl_xor compiles to ds_bpermute_b32, one LDS round trip per step
+// and two per step for a double: the six steps of a wavefront reduction are a dependent chain of about a hundred
+// clocks each, which is most of the running time of a kernel that handles one row per block.  Here four DPP steps
+// (lane ^ 1, lane ^ 2, mirror within 8, mirror within 16: a few clocks each) leave every lane with the result of its
+// row of 16 lanes, and the four rows meet through v_readlane.  Sums are therefore associated differently from
+// wave_sum (pairs, quads, eights, rows, then row 0 + row 1 + row 2 + row 3); every lane gets the same value.
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_u32(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, false);
+}
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) { return __uint_as_float(dpp_u32<CTRL>(__float_as_uint(v))); }
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_move(uint32_t v) { return dpp_u32<CTRL>(v); }
+template <int CTRL>
+__device__ __forceinline__ double dpp_move(double v) {
+    const uint64_t u = (uint64_t)__double_as_longlong(v);
+    const uint32_t lo = dpp_u32<CTRL>((uint32_t)u), hi = dpp_u32<CTRL>((uint32_t)(u >> 32));
+    return __longlong_as_double((long long)(((uint64_t)hi << 32) | lo));
+}
+__device__ __forceinline__ float lane_value(float v, int lane) { return __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(v), lane)); }
+__device__ __forceinline__ uint32_t lane_value(uint32_t v, int lane) { return (uint32_t)__builtin_amdgcn_readlane((int)v, lane); }
+__device__ __forceinline__ double lane_value(double v, int lane) {
+    const uint64_t u = (uint64_t)__double_as_longlong(v);
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)u, lane);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(u >> 32), lane);
+    return __longlong_as_double((long long)(((uint64_t)hi << 32) | lo));
+}
+constexpr int kDppXor1 = 0xB1, kDppXor2 = 0x4E, kDppHalfMirror = 0x141, kDppMirror = 0x140;
+
+// every lane: the sum / maximum over its row of 16 lanes
+template <typename T>
+__device__ __forceinline__ T row16_sum(T v) {
+    v += dpp_move<kDppXor1>(v);
+    v += dpp_move<kDppXor2>(v);
+    v += dpp_move<kDppHalfMirror>(v);
+    v += dpp_move<kDppMirror>(v);
+    return v;
+}
+__device__ __forceinline__ float row16_max(float v) {
+    v = fmaxf(v, dpp_move<kDppXor1>(v));
+    v = fmaxf(v, dpp_move<kDppXor2>(v));
+    v = fmaxf(v, dpp_move<kDppHalfMirror>(v));
+    v = fmaxf(v, dpp_move<kDppMirror>(v));
+    return v;
+}
+template <typename T>
+__device__ __forceinline__ T wave_sum_dpp(T v) {
+    v = row16_sum(v);
+    return (lane_value(v, 0) + lane_value(v, 16)) + (lane_value(v, 32) + lane_value(v, 48));
+}
+__device__ __forceinline__ float wave_max_dpp(float v) {
+    v = row16_max(v);
+    return fmaxf(fmaxf(lane_value(v, 0), lane_value(v, 16)), fmaxf(lane_value(v, 32), lane_value(v, 48)));
+}
+
+// Block-wide reductions for blocks of NWAVES wavefronts; `smem` needs NWAVES slots.  DPP selects the wavefront
+// step above (a different association of the sum).  FRESH: nobody has read `smem` since the block's last barrier,
+// so the barrier that protects earlier readers is left out.
+template <typename T, int NWAVES, bool DPP = false, bool FRESH = false>
 __device__ __forceinline__ T block_sum(T v, T *smem) {
-    v = wave_sum(v);
+    v = DPP ? wave_sum_dpp(v) : wave_sum(v);
     int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-    __syncthreads();
+    if (!FRESH) __syncthreads();
     if (lane == 0) smem[wave] = v;
     __syncthreads();
     T r = smem[0];
@@ -67,11 +125,11 @@ __device__ __forceinline__ T block_sum(T v, T *smem) {
     for (int i = 1; i < NWAVES; ++i) r += smem[i];
     return r;
 }
-template <int NWAVES>
+template <int NWAVES, bool DPP = false, bool FRESH = false>
 __device__ __forceinline__ float block_max(float v, float *smem) {
-    v = wave_max(v);
+    v = DPP ? wave_max_dpp(v) : wave_max(v);
     int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-    __syncthreads();
+    if (!FRESH) __syncthreads();
     if (lane == 0) smem[wave] = v;
     __syncthreads();
     float r = smem[0];
@@ -139,13 +197,25 @@ __device__ __forceinline__ uint32_t f32_to_e4m3(float v) {
 template <typename PF>
 __device__ __forceinline__ void prefetch_weights(const PF &pf, uint32_t j) {
     if (j >= pf.blocks) return;
-    const uint32_t t0 = pf.half_tiles ? (j / pf.half_tiles) * 2 * pf.half_tiles + j % pf.half_tiles : j * pf.tile_stride;
+    uint32_t t0, reps, step;
+    uint64_t start = 0;                               // byte offset of the pull inside each tile
+    if (pf.ksplit) {                                  // split-k launch: group (q / S) * 8 + xcd, member q % S
+        const uint32_t S = pf.ksplit, xcd = j % 8, q = j / 8, member = q % S;
+        t0 = ((q / S) * 8 + xcd) * S;
+        reps = S;
+        step = 1;
+        start = ((uint64_t)pf.k_tiles * member / S) * 1024;
+    } else {
+        t0 = pf.half_tiles ? (j / pf.half_tiles) * 2 * pf.half_tiles + j % pf.half_tiles : j * pf.tile_stride;
+        reps = pf.pair_step ? 2u : 1u;
+        step = pf.pair_step;
+    }
     const uint32_t vecs = pf.bytes / 16, nt = blockDim.x;
     v4u acc = v4u{0, 0, 0, 0};
-    for (uint32_t r = 0; r < (pf.pair_step ? 2u : 1u); ++r) {
-        uint32_t tile = t0 + r * pf.pair_step;
+    for (uint32_t r = 0; r < reps; ++r) {
+        uint32_t tile = t0 + r * step;
         tile = tile < pf.n_tiles ? tile : pf.n_tiles - 1;
-        const v4u *p = (const v4u *)(pf.w + (uint64_t)tile * pf.k_tiles * 1024);
+        const v4u *p = (const v4u *)(pf.w + (uint64_t)tile * pf.k_tiles * 1024 + start);
         for (uint32_t i = threadIdx.x; i < vecs; i += nt * 4) {
             v4u t[4];
 #pragma unroll

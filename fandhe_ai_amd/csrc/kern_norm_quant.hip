@@ -1,11 +1,15 @@
 // RMSNorm (reference contract), dynamic per-token int8 quantization, their
 // fusion, and per-tensor e4m3 quantization.
+#include <type_traits>
+
 #include "device_utils.hpp"
 #include "kernels.hpp"
 
 namespace fa {
 namespace k {
 using namespace fa::dev;
+
+int g_rows_wide = 0;        // tuning: 1 keeps the 256-thread row kernels for every row count
 
 namespace {
 
@@ -222,6 +226,163 @@ __global__ void __launch_bounds__(kBlock)
     }
 }
 
+// The same for few rows (a decode step: 32 rows on 32 compute units), where the kernel's time is its chain of
+// dependent steps and not its bytes: a block of THREADS threads per row, thread t owning the four-element groups
+// t, t + THREADS, ... (VPT of them), so that at 4096 columns a thread converts, squares, scales and divides four
+// elements instead of sixteen and the row's bytes are requested by sixteen wavefronts at once.  Same arithmetic
+// per element; the f64 sum of squares is split over more threads (only its order differs, as above).
+template <int THREADS, int VPT, bool ROW>
+__global__ void __launch_bounds__(THREADS)
+    rmsnorm_quantize_wide_kernel(const float *__restrict__ x, const float *__restrict__ w, float eps, float inv_n,
+                                 float *__restrict__ out_f32, int8_t *__restrict__ xq, float *__restrict__ sx, uint64_t m,
+                                 uint64_t hidden, uint32_t row_blocks, WeightPrefetch pull) {
+    constexpr int NW = THREADS / kWave;
+    __shared__ double smem_d[NW];
+    __shared__ float smem_f[NW];
+    if (blockIdx.x >= row_blocks) {                      // appended blocks: weights of the linear that follows
+        prefetch_weights(pull, blockIdx.x - row_blocks);
+        return;
+    }
+    const uint64_t r = blockIdx.x;
+    const uint64_t k_tiles = hidden / 64, n_vec = hidden / 4;
+    if (r >= m) {
+        if (!ROW)
+            for (uint64_t c = threadIdx.x; c < hidden / 16; c += THREADS)
+                *(v4i *)(xq + tiled_chunk_offset(r, c, k_tiles)) = v4i{0, 0, 0, 0};
+        return;
+    }
+    const float *row = x + r * hidden;
+    v4f xv[VPT], wv[VPT];
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const uint64_t j = threadIdx.x + (uint64_t)i * THREADS;
+        xv[i] = j < n_vec ? *(const v4f *)(row + j * 4) : v4f{0.f, 0.f, 0.f, 0.f};
+        wv[i] = j < n_vec ? *(const v4f *)(w + j * 4) : v4f{0.f, 0.f, 0.f, 0.f};
+    }
+    double acc = 0.0;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const double d = (double)xv[i][e];
+            acc = fma(d, d, acc);
+        }
+    acc = block_sum<double, NW, true, true>(acc, smem_d);
+    const float rstd = (float)(1.0 / sqrt(fma(acc, (double)inv_n, (double)eps)));
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float y = __fmul_rn(__fmul_rn(xv[i][e], rstd), wv[i][e]);
+            xv[i][e] = y;
+            amax = fmaxf(amax, fabsf(y));
+        }
+    amax = block_max<NW, true, true>(amax, smem_f);
+    const float scale = __fdiv_rn(amax, 127.0f);
+    if (threadIdx.x == 0) sx[r] = scale;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const uint64_t j = threadIdx.x + (uint64_t)i * THREADS;
+        if (j >= n_vec) continue;
+        uint32_t word = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) word |= ((uint32_t)quant_i8(xv[i][e], scale) & 0xffu) << (8 * e);
+        if (out_f32) *(v4f *)(out_f32 + r * hidden + j * 4) = xv[i];
+        int8_t *dst = ROW ? xq + r * hidden + j * 4 : xq + tiled_chunk_offset(r, j / 4, k_tiles) + (j % 4) * 4;
+        *(uint32_t *)dst = word;
+    }
+}
+
+// RMSNorm alone and the per-token quantizer alone in the same few-rows form (the row stays in registers, so it is
+// read once).  hidden / k a multiple of 4 (rmsnorm) or of 16 with k == k_pad a multiple of 64 for tiles (quantizer).
+template <int THREADS, int VPT>
+__global__ void __launch_bounds__(THREADS)
+    rmsnorm_wide_kernel(const float *__restrict__ x, const float *__restrict__ w, float *__restrict__ out, uint64_t hidden,
+                        float inv_n, float eps) {
+    constexpr int NW = THREADS / kWave;
+    __shared__ double smem_d[NW];
+    const uint64_t r = blockIdx.x, n_vec = hidden / 4;
+    const float *row = x + r * hidden;
+    v4f xv[VPT], wv[VPT];
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const uint64_t j = threadIdx.x + (uint64_t)i * THREADS;
+        xv[i] = j < n_vec ? *(const v4f *)(row + j * 4) : v4f{0.f, 0.f, 0.f, 0.f};
+        wv[i] = (w && j < n_vec) ? *(const v4f *)(w + j * 4) : v4f{0.f, 0.f, 0.f, 0.f};
+    }
+    double acc = 0.0;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const double d = (double)xv[i][e];
+            acc = fma(d, d, acc);
+        }
+    acc = block_sum<double, NW, true, true>(acc, smem_d);
+    const float rstd = (float)(1.0 / sqrt(fma(acc, (double)inv_n, (double)eps)));
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const uint64_t j = threadIdx.x + (uint64_t)i * THREADS;
+        if (j >= n_vec) continue;
+        v4f y;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) y[e] = w ? __fmul_rn(__fmul_rn(xv[i][e], rstd), wv[i][e]) : __fmul_rn(xv[i][e], rstd);
+        *(v4f *)(out + r * hidden + j * 4) = y;
+    }
+}
+
+template <int THREADS, int VPT, bool IN_BF16>
+__global__ void __launch_bounds__(THREADS)
+    quantize_rows_wide_kernel(const void *__restrict__ x, int8_t *__restrict__ xq_row, int8_t *__restrict__ xq_tiled,
+                              float *__restrict__ sx, uint64_t m, uint64_t k) {
+    constexpr int NW = THREADS / kWave;
+    __shared__ float smem[NW];
+    const uint64_t r = blockIdx.x, k_tiles = k / 64, n_vec = k / 4;
+    if (r >= m) {                                     // padding row of the tiled layout
+        if (xq_tiled)
+            for (uint64_t c = threadIdx.x; c < k / 16; c += THREADS)
+                *(v4i *)(xq_tiled + tiled_chunk_offset(r, c, k_tiles)) = v4i{0, 0, 0, 0};
+        return;
+    }
+    float xv[VPT][4];
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const uint64_t j = threadIdx.x + (uint64_t)i * THREADS;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) xv[i][e] = 0.0f;
+        if (j < n_vec) {
+            if constexpr (IN_BF16) {
+                const v2u t = *(const v2u *)((const uint16_t *)x + r * k + j * 4);
+                xv[i][0] = bf16_lo(t[0]);
+                xv[i][1] = bf16_hi(t[0]);
+                xv[i][2] = bf16_lo(t[1]);
+                xv[i][3] = bf16_hi(t[1]);
+            } else {
+                const v4f t = *(const v4f *)((const float *)x + r * k + j * 4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) xv[i][e] = t[e];
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) amax = fmaxf(amax, fabsf(xv[i][e]));
+    }
+    amax = block_max<NW, true, true>(amax, smem);
+    const float scale = __fdiv_rn(amax, 127.0f);
+    if (threadIdx.x == 0) sx[r] = scale;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const uint64_t j = threadIdx.x + (uint64_t)i * THREADS;
+        if (j >= n_vec) continue;
+        uint32_t word = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) word |= ((uint32_t)quant_i8(xv[i][e], scale) & 0xffu) << (8 * e);
+        if (xq_tiled) *(uint32_t *)(xq_tiled + tiled_chunk_offset(r, j / 4, k_tiles) + (j % 4) * 4) = word;
+        if (xq_row) *(uint32_t *)(xq_row + r * k + j * 4) = word;
+    }
+}
+
 // SwiGLU of gu [m, 2 f] (gate columns first) followed by the per-token quantizer of the product, row-major:
 // pass 1 takes the row's absmax of silu(gate) * up, pass 2 recomputes the products (the row is in L2) and
 // writes their codes, so the f32 products never go to memory.  f a multiple of 16.
@@ -286,38 +447,44 @@ __global__ void __launch_bounds__(ONE ? 1024 : kBlock)
 }
 
 // Quantizer for rows whose absmax is already known as `parts` partial maxima: every block first
-// reduces its row's partials (cheap, L2-resident), then quantizes a slab of 256 chunks.
+// reduces its row's partials (cheap, L2-resident), then quantizes a slab of 256 groups of four elements (a thread
+// takes one 16-byte load of f32, or 8 bytes of bf16, and leaves four codes: with few rows the kernel's time is one
+// thread's chain of loads, divisions and stores, so the elements are spread over as many threads as there are).
 template <bool IN_BF16>
 __global__ void __launch_bounds__(kBlock)
     quantize_from_pmax_kernel(const void *__restrict__ x, const float *__restrict__ pmax, uint32_t parts,
                               int8_t *__restrict__ xq_tiled, float *__restrict__ sx, uint64_t m, uint64_t k) {
     __shared__ float smem[kWaves];
-    const uint64_t r = blockIdx.y, k_tiles = k / 64, n_chunks = k / 16;
-    const uint64_t c = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    const uint64_t r = blockIdx.y, k_tiles = k / 64, n_vec = k / 4;
+    const uint64_t j = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
     if (r >= m) {
-        if (c < n_chunks) *(v4i *)(xq_tiled + tiled_chunk_offset(r, c, k_tiles)) = v4i{0, 0, 0, 0};
+        if (j < n_vec) *(uint32_t *)(xq_tiled + tiled_chunk_offset(r, j / 4, k_tiles) + (j % 4) * 4) = 0u;
         return;
     }
-    // the chunk's values are requested before the partial maxima are reduced: one memory round trip, not two
-    float xv[16];
-    const uint64_t cc = c < n_chunks ? c : n_chunks - 1;
+    // the group's values are requested before the partial maxima are reduced: one memory round trip, not two
+    float xv[4];
+    const uint64_t jj = j < n_vec ? j : n_vec - 1;
+    if constexpr (IN_BF16) {
+        const v2u t = *(const v2u *)((const uint16_t *)x + r * k + jj * 4);
+        xv[0] = bf16_lo(t[0]);
+        xv[1] = bf16_hi(t[0]);
+        xv[2] = bf16_lo(t[1]);
+        xv[3] = bf16_hi(t[1]);
+    } else {
+        const v4f t = *(const v4f *)((const float *)x + r * k + jj * 4);
 #pragma unroll
-    for (int e = 0; e < 16; ++e) xv[e] = load_in<IN_BF16>(x, r * k + cc * 16 + e);
+        for (int e = 0; e < 4; ++e) xv[e] = t[e];
+    }
     float amax = 0.0f;
     for (uint32_t i = threadIdx.x; i < parts; i += kBlock) amax = fmaxf(amax, pmax[r * parts + i]);
-    amax = block_max<kWaves>(amax, smem);
+    amax = block_max<kWaves, true, true>(amax, smem);
     const float scale = __fdiv_rn(amax, 127.0f);
     if (blockIdx.x == 0 && threadIdx.x == 0) sx[r] = scale;
-    if (c >= n_chunks) return;
-    uint32_t words[4];
+    if (j >= n_vec) return;
+    uint32_t word = 0;
 #pragma unroll
-    for (int wd = 0; wd < 4; ++wd) {
-        uint32_t word = 0;
-#pragma unroll
-        for (int b = 0; b < 4; ++b) word |= ((uint32_t)quant_i8(xv[wd * 4 + b], scale) & 0xffu) << (8 * b);
-        words[wd] = word;
-    }
-    *(v4u *)(xq_tiled + tiled_chunk_offset(r, c, k_tiles)) = v4u{words[0], words[1], words[2], words[3]};
+    for (int b = 0; b < 4; ++b) word |= ((uint32_t)quant_i8(xv[b], scale) & 0xffu) << (8 * b);
+    *(uint32_t *)(xq_tiled + tiled_chunk_offset(r, j / 4, k_tiles) + (j % 4) * 4) = word;
 }
 
 // absmax over a tensor: block maxima merged with an integer max on the bit
@@ -372,6 +539,18 @@ void rmsnorm_f32(const float *x, const float *w, float *out, uint64_t rows, uint
                  hipStream_t s) {
     if (rows == 0 || hidden == 0) return;
     float inv_n = 1.0f / (float)hidden;
+    // few rows: the row in registers, up to 1024 threads on it (the kernel's time is its chain of round trips)
+    if (g_rows_wide != 1 && rows <= 256 && hidden % 4 == 0 && hidden <= 16384) {
+        if (hidden <= 1024)
+            rmsnorm_wide_kernel<256, 1><<<(unsigned)rows, 256, 0, s>>>(x, w, out, hidden, inv_n, eps);
+        else if (hidden <= 4096)
+            rmsnorm_wide_kernel<1024, 1><<<(unsigned)rows, 1024, 0, s>>>(x, w, out, hidden, inv_n, eps);
+        else if (hidden <= 8192)
+            rmsnorm_wide_kernel<1024, 2><<<(unsigned)rows, 1024, 0, s>>>(x, w, out, hidden, inv_n, eps);
+        else
+            rmsnorm_wide_kernel<1024, 4><<<(unsigned)rows, 1024, 0, s>>>(x, w, out, hidden, inv_n, eps);
+        return;
+    }
     rmsnorm_kernel<<<(unsigned)rows, kBlock, 0, s>>>(x, w, out, hidden, inv_n, eps);
 }
 
@@ -379,11 +558,48 @@ void quantize_rows_i8(const void *x, bool in_bf16, int8_t *xq_rowmajor, int8_t *
                       uint64_t m_pad, uint64_t k, uint64_t k_pad, hipStream_t s) {
     uint64_t rows = xq_tiled ? m_pad : m;
     if (rows == 0 || k_pad == 0) return;
+    if (g_rows_wide != 1 && rows <= 256 && k == k_pad && k % 64 == 0 && k <= 16384) {
+        auto go = [&](auto threads, auto vpt) {
+            constexpr int T = decltype(threads)::value, V = decltype(vpt)::value;
+            if (in_bf16)
+                quantize_rows_wide_kernel<T, V, true><<<(unsigned)rows, T, 0, s>>>(x, xq_rowmajor, xq_tiled, sx, m, k);
+            else
+                quantize_rows_wide_kernel<T, V, false><<<(unsigned)rows, T, 0, s>>>(x, xq_rowmajor, xq_tiled, sx, m, k);
+        };
+        if (k <= 1024)
+            go(std::integral_constant<int, 256>{}, std::integral_constant<int, 1>{});
+        else if (k <= 4096)
+            go(std::integral_constant<int, 1024>{}, std::integral_constant<int, 1>{});
+        else if (k <= 8192)
+            go(std::integral_constant<int, 1024>{}, std::integral_constant<int, 2>{});
+        else
+            go(std::integral_constant<int, 1024>{}, std::integral_constant<int, 4>{});
+        return;
+    }
     if (in_bf16)
         quantize_rows_kernel<true><<<(unsigned)rows, kBlock, 0, s>>>(x, xq_rowmajor, xq_tiled, sx, m, k, k_pad);
     else
         quantize_rows_kernel<false><<<(unsigned)rows, kBlock, 0, s>>>(x, xq_rowmajor, xq_tiled, sx, m, k, k_pad);
 }
+
+namespace {
+// Few rows (at most one block per compute unit): the wide form.  Returns false when the shape is not its case.
+template <bool ROW>
+bool launch_rmsnorm_quantize_wide(const float *x, const float *w, float eps, float inv_n, float *out_f32, int8_t *xq, float *sx,
+                                  uint64_t m, uint64_t hidden, uint32_t rows, unsigned grid, const WeightPrefetch &pf,
+                                  hipStream_t s) {
+    if (g_rows_wide == 1 || rows > 256 || hidden > 16384 || hidden % 16 != 0) return false;
+    if (hidden <= 1024)
+        rmsnorm_quantize_wide_kernel<256, 1, ROW><<<grid, 256, 0, s>>>(x, w, eps, inv_n, out_f32, xq, sx, m, hidden, rows, pf);
+    else if (hidden <= 4096)
+        rmsnorm_quantize_wide_kernel<1024, 1, ROW><<<grid, 1024, 0, s>>>(x, w, eps, inv_n, out_f32, xq, sx, m, hidden, rows, pf);
+    else if (hidden <= 8192)
+        rmsnorm_quantize_wide_kernel<1024, 2, ROW><<<grid, 1024, 0, s>>>(x, w, eps, inv_n, out_f32, xq, sx, m, hidden, rows, pf);
+    else
+        rmsnorm_quantize_wide_kernel<1024, 4, ROW><<<grid, 1024, 0, s>>>(x, w, eps, inv_n, out_f32, xq, sx, m, hidden, rows, pf);
+    return true;
+}
+}  // namespace
 
 void rmsnorm_quantize_i8(const float *x, const float *w, float eps, float *out_f32, int8_t *xq_tiled, float *sx,
                          uint64_t m, uint64_t m_pad, uint64_t hidden, hipStream_t s, const WeightPrefetch &pull) {
@@ -394,6 +610,7 @@ void rmsnorm_quantize_i8(const float *x, const float *w, float eps, float *out_f
     // the appended blocks only meet the next launch's blocks on their XCD when a multiple of eight blocks precedes them
     const WeightPrefetch pf = (pull.w && rows % 8 == 0) ? pull : WeightPrefetch{};
     unsigned grid = rows + pf.blocks;
+    if (launch_rmsnorm_quantize_wide<false>(x, w, eps, inv_n, out_f32, xq_tiled, sx, m, hidden, rows, grid, pf, s)) return;
     if (per_thread <= 1)
         rmsnorm_quantize_kernel<1><<<grid, kBlock, 0, s>>>(x, w, eps, inv_n, out_f32, xq_tiled, sx, m, hidden, rows, pf);
     else if (per_thread <= 2)
@@ -408,6 +625,7 @@ void rmsnorm_quantize_rows_i8(const float *x, const float *w, float eps, int8_t 
     float inv_n = 1.0f / (float)hidden;
     uint64_t per_thread = (hidden / 16 + kBlock - 1) / kBlock;
     unsigned grid = (unsigned)m;
+    if (launch_rmsnorm_quantize_wide<true>(x, w, eps, inv_n, nullptr, xq_rowmajor, sx, m, hidden, grid, grid, WeightPrefetch{}, s)) return;
     if (per_thread <= 1)
         rmsnorm_quantize_kernel<1, true><<<grid, kBlock, 0, s>>>(x, w, eps, inv_n, nullptr, xq_rowmajor, sx, m, hidden, grid, WeightPrefetch{});
     else if (per_thread <= 2)
@@ -427,7 +645,7 @@ void swiglu_quantize_rows_i8(const float *gu, int8_t *xq_rowmajor, float *sx, ui
 void quantize_rows_from_pmax(const void *x, bool in_bf16, const float *pmax, uint32_t parts, int8_t *xq_tiled,
                              float *sx, uint64_t m, uint64_t m_pad, uint64_t k, hipStream_t s) {
     if (m_pad == 0 || k == 0) return;
-    dim3 grid((unsigned)((k / 16 + kBlock - 1) / kBlock), (unsigned)m_pad);
+    dim3 grid((unsigned)((k / 4 + kBlock - 1) / kBlock), (unsigned)m_pad);
     if (in_bf16)
         quantize_from_pmax_kernel<true><<<grid, kBlock, 0, s>>>(x, pmax, parts, xq_tiled, sx, m, k);
     else

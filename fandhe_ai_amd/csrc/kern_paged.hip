@@ -208,7 +208,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, W
     const uint32_t nv = PF ? p.n_vseq : p.batch;
     uint32_t total = 0;
     for (uint32_t b = lane; b < nv; b += 64) total += seq_pages<PF>(p, b, max_ctx);
-    total = __builtin_amdgcn_readfirstlane(wave_sum<uint32_t>(total));
+    total = __builtin_amdgcn_readfirstlane(wave_sum_dpp<uint32_t>(total));
     const uint32_t per = range_pages(p, total);
     const uint64_t rlo64 = (uint64_t)r * per;
     if (rlo64 >= total) return;
@@ -685,8 +685,8 @@ __global__ void __launch_bounds__(1024) decode_stream_merge_quantize_kernel(Stre
         tot += v;
         if (bb < b) pre += v;
     }
-    tot = wave_sum<uint32_t>(tot);
-    pre = wave_sum<uint32_t>(pre);
+    tot = wave_sum_dpp<uint32_t>(tot);
+    pre = wave_sum_dpp<uint32_t>(pre);
     if (threadIdx.x % 64 == 0) {
         s_tot[wave] = tot;
         s_pre[wave] = pre;
@@ -796,7 +796,7 @@ __global__ void __launch_bounds__(1024) decode_stream_merge_quantize_kernel(Stre
         v[e] = bf16_to_f32(f32_to_bf16(res));         // the attention output is bf16: round once, then quantize
         amax = fmaxf(amax, fabsf(v[e]));
     }
-    amax = wave_max(amax);
+    amax = wave_max_dpp(amax);
     if (threadIdx.x % 64 == 0) s_max[wave] = amax;
     __syncthreads();
     amax = 0.0f;

@@ -19,6 +19,9 @@ int g_skinny_ntw = 0;      // tuning overrides (0 = heuristic)
 int g_skinny_waves = 0;
 int g_weight_prefetch = 0;   // 1: row kernels pull nothing for the linear that follows them
 int g_skinny_astat = 0;     // activation-stationary kernel: 0 by shape, 1 never, 2 whenever it can run
+int g_skinny_ksplit = 0;    // split k over the blocks of an XCD: 0 by shape, 1 never, 2 whenever it can run (agent-scope
+                            // meeting), 3 whenever it can run (meeting in the XCD's L2), 4 by shape but agent scope
+int g_skinny_ksplit_s = 0;  // members per group of the split (0 by shape, 2 or 4)
 
 namespace {
 
@@ -711,6 +714,321 @@ __global__ void __launch_bounds__(512)
     }
 }
 
+// ------------------------------------------------- split k across the blocks of one XCD
+// With few column tiles (n = 4096: 256 tiles, one per compute unit) every block of the kernels above pulls the whole
+// activation matrix through L2: 2 x (int8) or 4 x (bf16) the bytes of its weight tile at 32 rows, and with a deep k
+// no register file holds it.  Here a group of S blocks owns S column tiles and each member streams 1 / S of k for
+// all of them, so a compute unit fetches 1 / S of the activations.  The members' partial tiles meet in a workspace:
+// every member stores its sums, waits until the stores are acknowledged, and takes a ticket from the group's
+// counter; the member that draws the last ticket adds the S partial tiles in member order (a fixed order: the f32
+// sums do not depend on who arrives last) and runs the epilogue.  Nobody waits for anybody.
+// Workgroups are dealt to the eight XCDs round-robin by their linear id, so the members of a group are the blocks
+// x + 8 (S q + r), r = 0 .. S - 1: they share one L2.  LOCAL = true relies on that (probed once per context by
+// the caller): stores, ticket and loads are ordinary L2 accesses.  LOCAL = false uses agent-scope accesses that
+// are coherent between XCDs wherever the blocks run.  The ticket is relaxed; what orders it behind the stores is
+// the wait for their acknowledgement, not a fence (an agent-scope release writes back a whole L2).
+template <bool LOCAL, typename T>
+__device__ __forceinline__ void meet_store(T *p, T v) {
+    if constexpr (LOCAL)
+        __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    else
+        __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+template <bool LOCAL, typename T>
+__device__ __forceinline__ T meet_load(const T *p) {
+    if constexpr (LOCAL)
+        return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    else
+        return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Ticket of this block in its group (0 .. S - 1), the same value in every thread.  `slot` is one LDS word that
+// nobody else uses between the two barriers.  Call with all of the block's partial stores issued.
+template <bool LOCAL>
+__device__ __forceinline__ uint32_t meet_ticket(uint32_t *counter, uint32_t *slot) {
+    __builtin_amdgcn_s_waitcnt(0);                   // this thread's partial stores are acknowledged by L2 / memory
+    __syncthreads();                                 // ... and so are everybody's
+    if (threadIdx.x == 0) {
+        uint32_t t;
+        if constexpr (LOCAL)
+            t = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        else
+            t = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *slot = t;
+    }
+    __syncthreads();
+    return *slot;
+}
+
+// block -> (group, member) of a split-k launch: see above
+template <int S>
+__device__ __forceinline__ void ksplit_ids(uint32_t *group, uint32_t *member) {
+    const uint32_t xcd = blockIdx.x % 8, q = blockIdx.x / 8;
+    *group = (q / S) * 8 + xcd;
+    *member = q % S;
+}
+
+// W8A8, plain epilogue.  Item idx = (i * S + j) * 4 + e of a block is accumulator element e of row tile i, column
+// tile j of the group; wavefront w finishes the items w, w + 8, ...
+template <int MT, int S, int D, bool LOCAL>
+__global__ void __launch_bounds__(512)
+    w8a8_ksplit_kernel(const int8_t *__restrict__ xq_tiled, const int8_t *__restrict__ w_tiles, uint32_t m, uint32_t n,
+                       uint32_t n_tiles, uint32_t k_tiles, uint32_t n_groups, EpiI8 ep, int32_t *partial, uint32_t *counters) {
+    constexpr int NW = 8, NACC = MT * S * 4, NE = NACC / NW;
+    static_assert(NACC % NW == 0, "items divide over the wavefronts");
+    __shared__ int red[NW][NACC][64];
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+    uint32_t group, member;
+    ksplit_ids<S>(&group, &member);
+    if (group >= n_groups) return;                   // the same for every member of the group
+    const uint32_t nt0 = group * S;
+    const uint32_t kt_lo = (uint32_t)((uint64_t)k_tiles * member / S), kt_hi = (uint32_t)((uint64_t)k_tiles * (member + 1) / S);
+    const uint32_t len = kt_hi - kt_lo;
+    const uint32_t cnt = len > (uint32_t)wave ? (len - wave + NW - 1) / NW : 0;
+
+    v4i acc[MT][S];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < S; ++j) acc[i][j] = v4i{0, 0, 0, 0};
+    uint32_t a_off[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) a_off[i] = ((uint32_t)i * 16 + (uint32_t)lane % 16 < m ? (uint32_t)lane : (uint32_t)lane & 48u) * 16;
+    // epilogue operands, requested ahead of the weight stream by every member (only the last one uses them)
+    float p_sx[NE], p_sw[NE], p_bias[NE], p_res[NE];
+#pragma unroll
+    for (int q = 0; q < NE; ++q) {
+        p_sx[q] = p_sw[q] = p_bias[q] = p_res[q] = 0.0f;
+        const int idx = wave + q * NW;
+        const int e = idx % 4, j = (idx / 4) % S, i = idx / (4 * S);
+        const uint32_t row = i * 16 + 4 * (lane / 16) + e, col = (nt0 + j) * 16 + lane % 16;
+        if (row < m && col < n) {
+            p_sx[q] = ep.sx[row];
+            p_sw[q] = ep.sw[col];
+            if (ep.bias) p_bias[q] = ep.bias[col];
+            if (ep.residual) p_res[q] = ep.residual[(uint64_t)row * n + col];
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    const int8_t *b_base = w_tiles + (uint64_t)lane * 16;
+    v4i a[D][MT], b[D][S];
+    auto load_slot = [&](int s, uint32_t it) {
+        const uint32_t kt = kt_lo + wave + (it < cnt ? it : cnt - 1) * NW;
+#pragma unroll
+        for (int j = 0; j < S; ++j) {
+            uint32_t nt = nt0 + j;
+            nt = nt < n_tiles ? nt : n_tiles - 1;            // a tile past the edge is loaded clamped, never stored
+            b[s][j] = stream_load<true>((const v4i *)(b_base + ((uint64_t)nt * k_tiles + kt) * 1024));
+        }
+#pragma unroll
+        for (int i = 0; i < MT; ++i) a[s][i] = *(const v4i *)(xq_tiled + ((uint64_t)i * k_tiles + kt) * 1024 + a_off[i]);
+    };
+    auto mma_slot = [&](int s) {
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int j = 0; j < S; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[s][i], b[s][j], acc[i][j], 0, 0, 0);
+    };
+    if (cnt != 0) {
+#pragma unroll
+        for (int s = 0; s < D; ++s) load_slot(s, (uint32_t)s);
+        uint32_t it0 = 0;
+        for (; it0 + D < cnt; it0 += D) {
+#pragma unroll
+            for (int s = 0; s < D; ++s) {
+                mma_slot(s);
+                __builtin_amdgcn_sched_barrier(0);
+                load_slot(s, it0 + D + s);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < D; ++s)
+            if (it0 + s < cnt) mma_slot(s);
+    }
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < S; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) red[wave][(i * S + j) * 4 + e][lane] = acc[i][j][e];
+    __syncthreads();
+    int own[NE];
+    int32_t *mine = partial + ((uint64_t)group * S + member) * (NACC * 64);
+#pragma unroll
+    for (int q = 0; q < NE; ++q) {
+        const int idx = wave + q * NW;
+        int sum = 0;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) sum += red[w][idx][lane];
+        own[q] = sum;
+        meet_store<LOCAL>(mine + idx * 64 + lane, sum);
+    }
+    const uint32_t ticket = meet_ticket<LOCAL>(counters + group, (uint32_t *)&red[0][0][0]);
+    if (ticket != S - 1) return;
+    if (threadIdx.x == 0) meet_store<LOCAL>(counters + group, 0u);      // for the next launch
+    int other[NE][S];
+#pragma unroll
+    for (int q = 0; q < NE; ++q)
+#pragma unroll
+        for (int r = 0; r < S; ++r)
+            other[q][r] = meet_load<LOCAL>(partial + ((uint64_t)group * S + r) * (NACC * 64) + (wave + q * NW) * 64 + lane);
+#pragma unroll
+    for (int q = 0; q < NE; ++q) {
+        const int idx = wave + q * NW;
+        int sum = 0;
+#pragma unroll
+        for (int r = 0; r < S; ++r) sum += (uint32_t)r == member ? own[q] : other[q][r];
+        const int e = idx % 4, j = (idx / 4) % S, i = idx / (4 * S);
+        const uint32_t row = i * 16 + 4 * (lane / 16) + e, col = (nt0 + j) * 16 + lane % 16;
+        if (row < m && col < n) {
+            const uint64_t o = (uint64_t)row * n + col;
+            if (ep.acc_out) ep.acc_out[o] = sum;
+            float v = __fmul_rn((float)sum, __fmul_rn(p_sx[q], p_sw[q]));
+            if (ep.bias) v = __fadd_rn(v, p_bias[q]);
+            if (ep.residual) v = __fadd_rn(p_res[q], v);
+            if (ep.out_bf16)
+                ((uint16_t *)ep.out)[o] = f32_to_bf16(v);
+            else
+                ((float *)ep.out)[o] = v;
+        }
+    }
+}
+
+// W8A16: the same with bf16 activations, weights converted in registers, f32 partial tiles added in member order.
+template <int MT, int S, int D, bool LOCAL>
+__global__ void __launch_bounds__(512)
+    w8a16_ksplit_kernel(const uint16_t *__restrict__ a, const int8_t *__restrict__ w_tiles, const float *__restrict__ sw,
+                        uint32_t m, uint32_t n, uint32_t n_tiles, uint32_t k_tiles, uint32_t n_groups, void *__restrict__ out,
+                        int out_bf16, float *partial, uint32_t *counters) {
+    constexpr int NW = 8, NACC = MT * S * 4, NE = NACC / NW;
+    static_assert(NACC % NW == 0, "items divide over the wavefronts");
+    __shared__ float red[NW][NACC][64];
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+    const int g = lane / 16, r = lane % 16;
+    uint32_t group, member;
+    ksplit_ids<S>(&group, &member);
+    if (group >= n_groups) return;
+    const uint32_t nt0 = group * S;
+    const uint64_t k = (uint64_t)k_tiles * 64;
+    const uint32_t kt_lo = (uint32_t)((uint64_t)k_tiles * member / S), kt_hi = (uint32_t)((uint64_t)k_tiles * (member + 1) / S);
+    const uint32_t len = kt_hi - kt_lo;
+    const uint32_t cnt = len > (uint32_t)wave ? (len - wave + NW - 1) / NW : 0;
+
+    v4f acc[MT][S];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < S; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+    float p_sw[NE];
+#pragma unroll
+    for (int q = 0; q < NE; ++q) {
+        const int idx = wave + q * NW;
+        const uint32_t col = (nt0 + (idx / 4) % S) * 16 + r;
+        p_sw[q] = col < n ? sw[col] : 0.0f;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    const int8_t *b_base = w_tiles + (uint64_t)lane * 16;
+    const uint32_t last_tile = n_tiles - 1;
+    uint32_t a_row[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) a_row[i] = (uint32_t)i * 16 + r < m ? (uint32_t)i * 16 + r : 0u;
+    v4u braw[D][S], lo[D][MT], hi[D][MT];
+    auto load_slot = [&](int s_, uint32_t it) {
+        const uint32_t kt = kt_lo + wave + (it < cnt ? it : cnt - 1) * NW;
+#pragma unroll
+        for (int j = 0; j < S; ++j) {
+            uint32_t nt = nt0 + j;
+            nt = nt < last_tile ? nt : last_tile;
+            braw[s_][j] = stream_load<true>((const v4u *)(b_base + ((uint64_t)nt * k_tiles + kt) * 1024));
+        }
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            const v4u *p = (const v4u *)(a + (uint64_t)a_row[i] * k + (uint64_t)kt * 64 + g * 16);
+            lo[s_][i] = p[0];
+            hi[s_][i] = p[1];
+        }
+    };
+    auto mma_slot = [&](int s_) {
+#pragma unroll
+        for (int j = 0; j < S; ++j) {
+            v8bf blo, bhi;
+            cvt_i8x8_bf16(braw[s_][j][0], braw[s_][j][1], &blo);
+            cvt_i8x8_bf16(braw[s_][j][2], braw[s_][j][3], &bhi);
+#pragma unroll
+            for (int i = 0; i < MT; ++i) {
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, lo[s_][i]), blo, acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, hi[s_][i]), bhi, acc[i][j], 0, 0, 0);
+            }
+        }
+    };
+    if (cnt != 0) {
+#pragma unroll
+        for (int s_ = 0; s_ < D; ++s_) load_slot(s_, (uint32_t)s_);
+        uint32_t it0 = 0;
+        for (; it0 + D < cnt; it0 += D) {
+#pragma unroll
+            for (int s_ = 0; s_ < D; ++s_) {
+                mma_slot(s_);
+                __builtin_amdgcn_sched_barrier(0);
+                load_slot(s_, it0 + D + s_);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+#pragma unroll
+        for (int s_ = 0; s_ < D; ++s_)
+            if (it0 + s_ < cnt) mma_slot(s_);
+    }
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < S; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) red[wave][(i * S + j) * 4 + e][lane] = acc[i][j][e];
+    __syncthreads();
+    float own[NE];
+    float *mine = partial + ((uint64_t)group * S + member) * (NACC * 64);
+#pragma unroll
+    for (int q = 0; q < NE; ++q) {
+        const int idx = wave + q * NW;
+        float sum = red[0][idx][lane];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) sum = __fadd_rn(sum, red[w][idx][lane]);
+        own[q] = sum;
+        meet_store<LOCAL>(mine + idx * 64 + lane, sum);
+    }
+    const uint32_t ticket = meet_ticket<LOCAL>(counters + group, (uint32_t *)&red[0][0][0]);
+    if (ticket != S - 1) return;
+    if (threadIdx.x == 0) meet_store<LOCAL>(counters + group, 0u);
+    float other[NE][S];
+#pragma unroll
+    for (int q = 0; q < NE; ++q)
+#pragma unroll
+        for (int r2 = 0; r2 < S; ++r2)
+            other[q][r2] = meet_load<LOCAL>(partial + ((uint64_t)group * S + r2) * (NACC * 64) + (wave + q * NW) * 64 + lane);
+#pragma unroll
+    for (int q = 0; q < NE; ++q) {
+        const int idx = wave + q * NW;
+        float sum = 0.0f;
+#pragma unroll
+        for (int r2 = 0; r2 < S; ++r2) {
+            const float t = (uint32_t)r2 == member ? own[q] : other[q][r2];
+            sum = r2 == 0 ? t : __fadd_rn(sum, t);
+        }
+        const int e = idx % 4, j = (idx / 4) % S, i = idx / (4 * S);
+        const uint32_t row = i * 16 + 4 * g + e, col = (nt0 + j) * 16 + r;
+        if (row < m && col < n) {
+            const float v = __fmul_rn(sum, p_sw[q]);
+            const uint64_t o = (uint64_t)row * n + col;
+            if (out_bf16)
+                ((uint16_t *)out)[o] = f32_to_bf16(v);
+            else
+                ((float *)out)[o] = v;
+        }
+    }
+}
+
 // ------------------------------------------------------------------ e4m3 x e4m3, decode shape
 // out[m, n] = (sum_k a[m, k] * w[k, n]) * (sx[m] * sw[n]) (+ bias[n]) on the scaled 16x16x128 fp8 matrix
 // instruction with unit block scales.  The weight is in tiles of 16 columns x 128 k (2 KiB, 32 bytes per lane:
@@ -885,7 +1203,78 @@ void launch_w8a16(const uint16_t *a, const int8_t *wt, const float *sw, uint32_t
         launch_w8a16_form<MT, false>(a, wt, sw, m, n, n_tiles, k_tiles, out, out_bf16, ntw, waves, s);
 }
 
+
+// Whether a decode-shape linear goes out in the split-k form (w8a8_ksplit_kernel), and how: members per group,
+// depth of the register ring, where the partial tiles meet.
+struct KsplitPlan {
+    int s, d;
+    bool local;
+    uint32_t n_groups, blocks;
+};
+inline bool ksplit_plan(uint64_t m, uint32_t n_tiles, uint32_t k_tiles, int num_cus, const SplitKArea *sk, int act_bytes,
+                        KsplitPlan *p) {
+    if (!sk || !sk->partial || !sk->counters || g_skinny_ksplit == 1 || m == 0 || m > 32 || n_tiles == 0) return false;
+    const bool forced = g_skinny_ksplit == 2 || g_skinny_ksplit == 3;
+    // By shape: the projections with about one column tile per compute unit whose blocks would each pull 256 KiB of
+    // activations or more (measured in a decode step's kernel trace at 32 rows: 14336 -> 4096 int8 17.3 -> 14.6 us,
+    // while 4096 -> 4096 int8, 128 KiB per block, loses 0.7 us to the meeting); wider weights keep their activations
+    // in registers (w8a8_astat_kernel).
+    const uint64_t a_bytes = (uint64_t)(m <= 16 ? 16 : 32) * k_tiles * 64 * (uint64_t)act_bytes;
+    if (!forced && ((uint64_t)n_tiles > 2 * (uint64_t)num_cus || a_bytes < (256u << 10))) return false;
+    int s = g_skinny_ksplit_s ? g_skinny_ksplit_s : (k_tiles >= 128 ? 4 : 2);
+    if (s != 2 && s != 4) return false;
+    if (k_tiles / (uint32_t)s < 16) return false;              // two k-tiles per wavefront at least
+    const int mt = m <= 16 ? 1 : 2;
+    const uint32_t n_groups = (n_tiles + s - 1) / s;
+    const uint64_t bytes = (uint64_t)n_groups * s * ((uint64_t)mt * s * 4 * 64 * 4);
+    if (n_groups > sk->n_counters || bytes > sk->partial_bytes) return false;
+    p->s = s;
+    p->d = k_tiles / (uint32_t)s >= 32 ? 4 : 2;
+    p->local = g_skinny_ksplit == 3 || ((g_skinny_ksplit == 0) && sk->xcd_local);
+    p->n_groups = n_groups;
+    p->blocks = 8u * (uint32_t)s * ((n_groups + 7) / 8);       // whole groups on every XCD; surplus groups return at once
+    return true;
+}
+
+// Calls go(MT, S, D, LOCAL) with the plan's values as integral constants.
+template <typename F>
+void ksplit_dispatch(uint64_t m, const KsplitPlan &p, F &&go) {
+    auto with_local = [&](auto mt, auto s, auto d) {
+        if (p.local)
+            go(mt, s, d, std::true_type{});
+        else
+            go(mt, s, d, std::false_type{});
+    };
+    auto with_d = [&](auto mt, auto s) {
+        if (p.d == 4)
+            with_local(mt, s, std::integral_constant<int, 4>{});
+        else
+            with_local(mt, s, std::integral_constant<int, 2>{});
+    };
+    auto with_s = [&](auto mt) {
+        if (p.s == 4)
+            with_d(mt, std::integral_constant<int, 4>{});
+        else
+            with_d(mt, std::integral_constant<int, 2>{});
+    };
+    if (m <= 16)
+        with_s(std::integral_constant<int, 1>{});
+    else
+        with_s(std::integral_constant<int, 2>{});
+}
+
 }  // namespace
+
+// out[b] = id of the XCD that workgroup b of this launch runs on (what ksplit_ids assumes is b % 8 up to a
+// renaming of the XCDs; the caller checks)
+namespace {
+__global__ void __launch_bounds__(64) xcc_id_probe_kernel(uint32_t *out) {
+    uint32_t id;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(id));
+    if (threadIdx.x == 0) out[blockIdx.x] = id & 15u;
+}
+}  // namespace
+void xcc_id_probe(uint32_t *out, uint32_t blocks, hipStream_t s) { xcc_id_probe_kernel<<<blocks, 64, 0, s>>>(out); }
 
 // Which weight bytes the blocks of the launches below read first, for the row kernel in front of them to pull
 // (WeightPrefetch): the block -> tile mapping of every form is restated here beside the launch that uses it.
@@ -912,9 +1301,24 @@ WeightPrefetch make_prefetch(const int8_t *w_tiles, uint32_t blocks, uint32_t n_
 }  // namespace
 
 WeightPrefetch prefetch_for_linear_w8a8_skinny(const int8_t *w_tiles, uint64_t m, uint64_t n_pad, uint64_t k_pad, int num_cus,
-                                               uint64_t budget) {
+                                               uint64_t budget, const SplitKArea *sk) {
     const uint32_t n_tiles = (uint32_t)(n_pad / 16), k_tiles = (uint32_t)(k_pad / 64);
     if (m == 0 || n_tiles == 0) return WeightPrefetch{};
+    KsplitPlan kp;
+    if (ksplit_plan(m, n_tiles, k_tiles, num_cus, sk, 1, &kp)) {     // block -> (group, member) as in ksplit_ids
+        if (g_weight_prefetch == 1 || k_tiles == 0) return WeightPrefetch{};
+        WeightPrefetch pf;
+        uint64_t per = budget / ((uint64_t)kp.blocks * kp.s) / 1024 * 1024;
+        per = std::min<uint64_t>(per, (uint64_t)(k_tiles / kp.s) * 1024);
+        if (per == 0) return pf;
+        pf.w = w_tiles;
+        pf.blocks = kp.blocks;
+        pf.n_tiles = n_tiles;
+        pf.k_tiles = k_tiles;
+        pf.bytes = (uint32_t)per;
+        pf.ksplit = (uint32_t)kp.s;
+        return pf;
+    }
     if (m <= 32 && astat_applies((n_tiles + 1) / 2, k_tiles, num_cus)) {      // block b starts with unit b = tiles 2 b, 2 b + 1
         const uint32_t n_units = (n_tiles + 1) / 2;
         return make_prefetch(w_tiles, (uint32_t)std::min<uint64_t>(n_units, (uint64_t)num_cus), n_tiles, k_tiles, 0, 2, n_tiles > 1 ? 1 : 0, budget);
@@ -934,7 +1338,7 @@ WeightPrefetch prefetch_for_linear_w8a8_qkv_rope_skinny(const int8_t *w_tiles, u
 }
 
 void linear_w8a8_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t m, uint64_t n, uint64_t n_pad,
-                        uint64_t k_pad, const EpilogueI8 &ep, int num_cus, hipStream_t s) {
+                        uint64_t k_pad, const EpilogueI8 &ep, int num_cus, hipStream_t s, const SplitKArea *sk) {
     if (m == 0 || n == 0) return;
     uint32_t n_tiles = (uint32_t)(n_pad / 16), k_tiles = (uint32_t)(k_pad / 64);
     EpiI8 e{};
@@ -945,6 +1349,15 @@ void linear_w8a8_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t 
     e.acc_out = ep.acc_out;
     e.out = ep.out;
     e.out_bf16 = ep.out_bf16;
+    KsplitPlan kp;
+    if (ksplit_plan(m, n_tiles, k_tiles, num_cus, sk, 1, &kp)) {
+        ksplit_dispatch(m, kp, [&](auto mt, auto ss, auto d, auto local) {
+            w8a8_ksplit_kernel<decltype(mt)::value, decltype(ss)::value, decltype(d)::value, decltype(local)::value>
+                <<<kp.blocks, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, kp.n_groups, e,
+                                           (int32_t *)sk->partial, sk->counters);
+        });
+        return;
+    }
     if (m <= 32 && astat_applies((n_tiles + 1) / 2, k_tiles, num_cus)) {
         unsigned n_units = (n_tiles + 1) / 2;
         unsigned blocks = (unsigned)std::min<uint64_t>(n_units, (uint64_t)num_cus);
@@ -1029,9 +1442,19 @@ void linear_e4m3_skinny(const uint8_t *aq, const uint8_t *w_tiles, const float *
 }
 
 void linear_w8a16_skinny(const uint16_t *a, const int8_t *w_tiles, const float *sw, uint64_t m, uint64_t n,
-                         uint64_t n_pad, uint64_t k_pad, void *out, int out_bf16, int num_cus, hipStream_t s) {
+                         uint64_t n_pad, uint64_t k_pad, void *out, int out_bf16, int num_cus, hipStream_t s,
+                         const SplitKArea *sk) {
     if (m == 0 || n == 0) return;
     uint32_t n_tiles = (uint32_t)(n_pad / 16), k_tiles = (uint32_t)(k_pad / 64);
+    KsplitPlan kp;
+    if (m > 4 && ksplit_plan(m, n_tiles, k_tiles, num_cus, sk, 2, &kp)) {
+        ksplit_dispatch(m, kp, [&](auto mt, auto ss, auto d, auto local) {
+            w8a16_ksplit_kernel<decltype(mt)::value, decltype(ss)::value, decltype(d)::value, decltype(local)::value>
+                <<<kp.blocks, 512, 0, s>>>(a, w_tiles, sw, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, kp.n_groups, out, out_bf16,
+                                           (float *)sk->partial, sk->counters);
+        });
+        return;
+    }
     // by shape only above 16 rows: with one row tile the activations are as small as the weight tile
     // and the block-per-tile kernel, which spreads over more wavefronts, measured faster
     if (astat_applies(n_tiles, k_tiles, num_cus) && !(g_skinny_ntw || g_skinny_waves) && (m > 16 || g_skinny_astat == 2)) {

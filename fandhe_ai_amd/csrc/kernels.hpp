@@ -21,6 +21,8 @@ struct WeightPrefetch {
     uint32_t tile_stride = 1;    // otherwise block j starts at tile j * tile_stride
     uint32_t pair_step = 0;      // != 0: the block also reads tile first + pair_step
     uint32_t bytes = 0;          // bytes pulled from the start of each tile (multiple of 16)
+    uint32_t ksplit = 0;         // != 0: the next launch is the split-k form with this many blocks per group; block j
+                                 // reads tiles group * ksplit .. + ksplit - 1 from its member's share of k onwards
 };
 
 
@@ -120,14 +122,27 @@ struct EpilogueI8 {
 // What the row kernel in front of each of the launches below should pull (see WeightPrefetch); same arguments as
 // the launch itself, `budget` = bytes of one pull.
 struct QkvRopeTargets;
+struct SplitKArea;
 WeightPrefetch prefetch_for_linear_w8a8_skinny(const int8_t *w_tiles, uint64_t m, uint64_t n_pad, uint64_t k_pad, int num_cus,
-                                               uint64_t budget);
+                                               uint64_t budget, const SplitKArea *sk = nullptr);
 WeightPrefetch prefetch_for_linear_w8a8_qkv_rope_skinny(const int8_t *w_tiles, uint64_t m, uint64_t n_pad, uint64_t k_pad,
                                                         const QkvRopeTargets &t, uint64_t budget);
+// Where the blocks of a split-k decode linear leave their partial tiles and take their tickets: one area per
+// context (launches that use it are ordered by the context's stream).  The counters are zero between launches.
+struct SplitKArea {
+    void *partial = nullptr;
+    uint64_t partial_bytes = 0;
+    uint32_t *counters = nullptr;
+    uint32_t n_counters = 0;
+    int xcd_local = 0;          // probed: workgroups b and b + 8 of a launch run on the same XCD (share an L2)
+};
+// out[b] = hardware id of the XCD workgroup b of the probe launch ran on (b < blocks)
+void xcc_id_probe(uint32_t *out, uint32_t blocks, hipStream_t s);
 // xq_tiled: activation tiles (see quantize_rows_i8); m <= 64 (one to four row tiles of 16 per block).
+// sk (optional): lets narrow weights split k over groups of blocks (m <= 32).
 void linear_w8a8_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t m, uint64_t n,
                         uint64_t n_pad, uint64_t k_pad, const EpilogueI8 &ep, int num_cus,
-                        hipStream_t s);
+                        hipStream_t s, const SplitKArea *sk = nullptr);
 // gate_up projection fused with SwiGLU: the weight is [k, n] with gate columns [0, n/2) and up columns
 // [n/2, n), n/2 a multiple of 16; act[m, n/2] = silu(gate) * up (f32) and pmax[m, n/32] receives the
 // absmax of every 16-column block of act (consumed by quantize_rows_from_pmax).
@@ -150,7 +165,7 @@ void linear_w8a8_qkv_rope_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, 
 // a: bf16 [m, k] row-major (k == k_pad required), m <= 32.
 void linear_w8a16_skinny(const uint16_t *a, const int8_t *w_tiles, const float *sw, uint64_t m,
                          uint64_t n, uint64_t n_pad, uint64_t k_pad, void *out, int out_bf16,
-                         int num_cus, hipStream_t s);
+                         int num_cus, hipStream_t s, const SplitKArea *sk = nullptr);
 
 // ---- prefill-shape MFMA GEMMs (kern_gemm_mfma.hip) -----------------------------
 // aq: int8 [m, k_pad] row-major.  workspace (optional, gemm_w8a8_workspace_bytes): lets a matrix with too few

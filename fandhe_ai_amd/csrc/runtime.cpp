@@ -406,7 +406,54 @@ fa_status fa_context_create(int32_t ordinal, fa_context **out) {
         delete ctx;
         return fail(FA_ERR_DEVICE_UNAVAILABLE, std::string("hipStreamCreate: ") + hipGetErrorString(e));
     }
+    // Meeting area of the split-k decode linears: 16 MiB of partial tiles, 4096 arrival counters.  Whether the
+    // workgroups b and b + 8 of a launch share an XCD (and with it an L2) is read off the hardware once: 2048
+    // workgroups report the XCD they run on.  Without that property the partial tiles meet in memory instead.
+    {
+        constexpr uint64_t kPartial = 16ull << 20;
+        constexpr uint32_t kCounters = 4096, kProbe = 2048;
+        void *area = nullptr;
+        if (hipMalloc(&area, kPartial + kCounters * 4) == hipSuccess) {
+            uint32_t *counters = (uint32_t *)((uint8_t *)area + kPartial);
+            std::vector<uint32_t> ids(kProbe, 0xffu);
+            fa::k::xcc_id_probe(counters, kProbe, ctx->stream);
+            bool ok = hipGetLastError() == hipSuccess &&
+                      hipMemcpyAsync(ids.data(), counters, kProbe * 4, hipMemcpyDeviceToHost, ctx->stream) == hipSuccess &&
+                      hipStreamSynchronize(ctx->stream) == hipSuccess;
+            bool round_robin = ok;
+            for (uint32_t b = 0; round_robin && b < kProbe; ++b) round_robin = ids[b] == ids[b % 8];
+            for (uint32_t b = 0; round_robin && b < 8; ++b)
+                for (uint32_t c = 0; c < b; ++c) round_robin = round_robin && ids[b] != ids[c];
+            if (ok) {
+                bool seen[16] = {};
+                for (uint32_t b = 0; b < kProbe; ++b) seen[ids[b] & 15u] = true;
+                for (bool x : seen) ctx->xcd_count += x ? 1 : 0;
+            }
+            ok = ok && hipMemsetAsync(area, 0, kPartial + kCounters * 4, ctx->stream) == hipSuccess &&
+                 hipStreamSynchronize(ctx->stream) == hipSuccess;
+            if (ok) {
+                ctx->splitk.partial = area;
+                ctx->splitk.partial_bytes = kPartial;
+                ctx->splitk.counters = counters;
+                ctx->splitk.n_counters = kCounters;
+                ctx->splitk.xcd_local = round_robin ? 1 : 0;
+            } else {
+                (void)hipGetLastError();
+                (void)hipFree(area);                 // the linears then keep to their unsplit forms
+            }
+        } else {
+            (void)hipGetLastError();
+        }
+    }
     *out = ctx;
+    return FA_OK;
+}
+
+fa_status fa_topology_query(const fa_context *ctx, int32_t *xcd_local, int32_t *xcd_count) {
+    if (!ctx || ctx->magic != kCtxMagic || !xcd_local || !xcd_count)
+        return fail(FA_ERR_INVALID_ARGUMENT, "fa_topology_query: bad argument");
+    *xcd_local = ctx->splitk.xcd_local;
+    *xcd_count = ctx->xcd_count;
     return FA_OK;
 }
 
@@ -418,6 +465,7 @@ fa_status fa_context_destroy(fa_context *ctx) {
     while (ctx->pool.take_one_for_release(&ent)) (void)hipFree(ent.second);
     if (ctx->table_stage) (void)hipFree(ctx->table_stage);
     if (ctx->workspace) (void)hipFree(ctx->workspace);
+    if (ctx->splitk.partial) (void)hipFree(ctx->splitk.partial);
     for (void *w : ctx->retired_workspaces) (void)hipFree(w);
     for (auto &b : ctx->capture_owned) (void)hipFree(b.ptr);   // a capture that was never ended
     for (void *p : ctx->deferred_frees) (void)hipFree(p);

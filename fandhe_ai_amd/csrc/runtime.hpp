@@ -13,6 +13,7 @@
 
 #include "../../include/fandhe_rocm.h"
 #include "../../include/fandhe_rocm_bench.h"
+#include "kernels.hpp"
 
 namespace fa {
 
@@ -90,6 +91,10 @@ struct fa_context {
     // class bytes of the blocks on loan to an open capture or to live graphs (PoolStats::pending_return_bytes:
     // idle-side memory that is neither cached nor in use by a buffer and comes back when its holder ends)
     uint64_t pending_return_bytes = 0;
+    // where the blocks of a split-k decode linear meet (allocated with the context, outside the pool; the counters
+    // are zero whenever no such launch is running)
+    fa::k::SplitKArea splitk;
+    int xcd_count = 0;            // distinct XCDs seen by the probe launch at creation
 };
 
 struct fa_buffer {

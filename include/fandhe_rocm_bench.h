@@ -66,8 +66,20 @@ fa_status fa_probe_stream_read(fa_context *ctx, const fa_buffer *src, uint64_t o
  *        n >= 2: n MiB of q | k | v and 2 n MiB of the o projection (0: 12 / 24); takes effect when a step is
  *        recorded, so set it before the first step of a batch size;
  * key 15: loads of fa_probe_stream_read: 1 ordinary loads, 0 the non-temporal loads that the kernels use for
- *        data they read once. */
+ *        data they read once;
+ * key 16: split-k form of the decode-shape linears (groups of blocks that share an XCD divide k and add their
+ *        partial tiles through a workspace): 0 by shape, 1 never, 2 whenever the shape allows it with the partial
+ *        tiles meeting in memory (agent-scope accesses), 3 whenever the shape allows it with the partial tiles
+ *        meeting in the XCD's L2, 4 by shape but meeting in memory;
+ * key 17: blocks per group of that form: 0 by shape, 2 or 4;
+ * key 18: 1 keeps the 256-thread form of the row kernels (norm, quantizer, norm + quantizer) for every row count
+ *        instead of the up-to-1024-thread form used for at most 256 rows. */
 fa_status fa_set_tuning(int32_t key, int32_t value);
+
+/* What the context found when it was created: xcd_local = 1 when workgroups b and b + 8 of a launch were seen to
+ * run on the same XCD (the split-k linears then let their partial tiles meet in that XCD's L2), xcd_count = the
+ * number of distinct XCDs the probe launch saw. */
+fa_status fa_topology_query(const fa_context *ctx, int32_t *xcd_local, int32_t *xcd_count);
 
 /* Which kernel a prefill-shape GEMM of m rows against `qw` is launched with under the
  * current knobs (pure host function, nothing is queued).  big_ntb: column tiles of 16

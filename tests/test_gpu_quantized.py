@@ -308,6 +308,68 @@ def test_w8a16_ragged_shapes_under_every_launch_shape():
         o.set_threads(1)
 
 
+def _topology(fa, be):
+    import ctypes as C
+    local, count = C.c_int32(), C.c_int32()
+    fa.check(fa.capi.lib.fa_topology_query(be._ctx, C.byref(local), C.byref(count)))
+    return local.value, count.value
+
+
+def test_split_k_decode_linears_match_the_oracle():
+    """The form of the decode-shape linears in which groups of two or four blocks divide k and add their partial
+    tiles through a workspace, forced for every shape it accepts: partial tiles meeting in memory (key 16 = 2) and,
+    where the device deals workgroups b and b + 8 to one XCD, in that XCD's L2 (key 16 = 3).  W8A8 accumulators and
+    outputs bit-exact, W8A16 within the tolerance; every call three times in a row (the arrival counters must be
+    back at zero) and on shapes with ragged rows, a clamped last column tile, groups past the last tile, k ranges
+    that do not divide evenly and wavefronts with one k-tile more than others."""
+    fa = _fa()
+    be = ops()
+    lib = fa.capi.lib
+    local, count = _topology(fa, be)
+    print("xcd_local", local, "xcd_count", count, flush=True)
+    assert count >= 1
+    modes = (2, 3) if local else (2,)
+    o.set_threads(8)
+    try:
+        for m, k, n in ((32, 4096, 4096), (32, 14336, 4096), (7, 2048, 33), (17, 4160, 1000), (32, 11008, 100), (1, 4096, 16),
+                        (20, 2112, 4112), (16, 8192, 528)):
+            rng = o.Rng(m + k + n)
+            x = rng.randn((m, k))
+            w = rng.randn((k, n), std=0.05)
+            bias = rng.randn((n,))
+            wq, ws = o.quantize_cols_i8(w)
+            qw = be.import_quantized_weight(wq, ws)
+            dx = be.upload(x)
+            dbias = fa.DeviceBufferView(be.upload(bias), 0, (n,))
+            want_acc, want = o.linear_w8a8(x, wq, ws, bias)
+            a16 = o.to_bf16(rng.randn((m, k))) if k % 64 == 0 else None
+            want16 = o.linear_w8a16(a16, wq, ws) if a16 is not None else None
+            da16 = be.upload(a16) if a16 is not None else None
+            for mode in modes:
+                for s in (2, 4):
+                    if (k + 63) // 64 // s < 16:
+                        continue
+                    fa.check(lib.fa_set_tuning(16, mode))
+                    fa.check(lib.fa_set_tuning(17, s))
+                    for rep in range(3):
+                        out, acc = be.linear_w8a8(dx, qw, bias=dbias, want_acc=True)
+                        assert np.array_equal(be.download_owned(acc), want_acc), (m, k, n, mode, s, rep)
+                        assert np.array_equal(be.download_owned(out), want), (m, k, n, mode, s, rep)
+                    if a16 is not None and m > 4:
+                        first = None
+                        for rep in range(3):
+                            got = be.download_owned(be.linear_w8a16(da16, qw, fa.capi.F32))
+                            assert_parity("W8A16_PARITY", f"{m}x{n}x{k}:ksplit{s}:mode{mode}", got, want16)
+                            if first is None:
+                                first = got
+                            assert np.array_equal(got, first), "split-k f32 sums depend on the arrival order"
+                        assert_bf16_rounding_of("w8a16 split-k bf16", be.download_owned(be.linear_w8a16(da16, qw, fa.capi.BF16)), first)
+    finally:
+        fa.check(lib.fa_set_tuning(16, 0))
+        fa.check(lib.fa_set_tuning(17, 0))
+        o.set_threads(1)
+
+
 def test_w8a16_one_hot_rows_pick_weight_rows_exactly():
     fa = _fa()
     be = ops()
