@@ -566,6 +566,49 @@ def bench_stream_floor(fa, be, sizes, reps=30):
     return res
 
 
+def bench_l2_path(fa, be, reps=20):
+    """The path from L2 to the compute units (fa_probe_l2_path).  (1) A 1 MiB region that every block reads over and
+    over (L2 hits after the first touch) at 2, 8 and 16 wavefronts per compute unit: what a compute unit can pull
+    from L2.  (2) A 58.7 MB stream from memory no launch has touched (fresh windows of a 4 GiB buffer), 256 blocks
+    of 512 threads as the decode linears launch, alone and with two L2-hit loads mixed in per streamed load, at 8
+    and 16 streamed loads per thread in flight: what operand re-reads that hit in L2 cost an HBM stream."""
+    lib = fa.capi.lib
+    cus = be.info().compute_units
+    total = 4 << 30
+    cold = be.alloc_uninit((total // 4,))
+    fa.check(lib.fa_fill_normal(be._ctx, cold._h, 0, total // 4, 3, 0.0, 1.0))
+    hot = be.alloc_uninit(((1 << 20) // 4,))
+    fa.check(lib.fa_fill_normal(be._ctx, hot._h, 0, (1 << 20) // 4, 4, 0.0, 1.0))
+    sink = be.alloc_zeroed((1,), fa.capi.I32)
+    res = []
+    hot_bytes, passes = 1 << 20, 16
+    for waves, blocks, threads in ((2, cus, 128), (8, cus, 512), (16, 2 * cus, 512)):
+        def launch():
+            fa.check(lib.fa_probe_l2_path(be._ctx, cold._h, 0, 0, hot._h, hot_bytes, passes, 8, 0, blocks, threads, sink._h))
+        us = time_launches(fa, be, launch, reps, warmup=3) * 1e6
+        nbytes = blocks * hot_bytes * passes
+        res.append(dict(what="L2-resident region, %d wavefronts per compute unit" % waves, blocks=blocks, threads=threads,
+                        us=us, gbs=nbytes / us / 1e3, gbs_per_cu=nbytes / us / 1e3 / cus))
+    nb = 58720256
+    win = (nb + 4095) // 4096 * 4096
+    nwin = total // win
+    for in_flight, ratio in ((8, 0), (16, 0), (8, 2), (16, 2)):
+        counter = [0]
+
+        def launch():
+            fa.check(lib.fa_probe_l2_path(be._ctx, cold._h, (counter[0] % nwin) * win, nb, hot._h, 256 << 10, 0, in_flight, ratio,
+                                          cus, 512, sink._h))
+            counter[0] += 1
+        us = time_launches(fa, be, launch, reps, warmup=3) * 1e6
+        res.append(dict(what="58.7 MB from HBM, %d loads in flight per thread, %s" %
+                             (in_flight, "alone" if ratio == 0 else "%d L2-hit loads per streamed load" % ratio),
+                        blocks=cus, threads=512, us=us, gbs=nb / us / 1e3, gbs_per_cu=nb / us / 1e3 / cus,
+                        l2_hit_gbs=ratio * nb / us / 1e3))
+    for b in (cold, hot, sink):
+        b.free()
+    return res
+
+
 def floor_sizes(cfg, att_bytes):
     D, F, V = cfg["d_model"], cfg["d_ffn"], cfg["vocab"]
     EQ, EKV = cfg["n_heads"] * cfg["head_dim"], cfg["n_kv_heads"] * cfg["head_dim"]
@@ -763,7 +806,7 @@ def main():
                     help="with --only decode-linears: one of the four layer shapes (0 .. 3) instead of all, so that "
                          "a counter run sees launches of one shape only")
     ap.add_argument("--only", choices=("attention", "copy", "linears", "decode-linears", "prefill", "prefill-attention", "mfma",
-                                       "prompt", "stream-floor", "gemm-f32"), default=None,
+                                       "prompt", "stream-floor", "gemm-f32", "l2-path"), default=None,
                     help="profiling aid: run only the dominant kernel at the workload's shape, or a plain "
                          "copy kernel of known size (counter calibration), a few launches, no JSON line")
     a = ap.parse_args()
@@ -812,6 +855,13 @@ def main():
             for r in bench_matrix_rate(fa, be):
                 log("%-42s %-20s: %.2f ms, %.0f T op/s (%.1f %% of peak)" %
                     (r["instr"], r["fill"], r["ms"], r["tops"], 100 * r["tops"] / MFMA_PEAK_TOPS))
+            be.close()
+            return
+        if a.only == "l2-path":
+            for r in bench_l2_path(fa, be):
+                log("%-78s %4d x %3d threads: %8.2f us, %7.0f GB/s (%5.1f GB/s per compute unit)%s" %
+                    (r["what"], r["blocks"], r["threads"], r["us"], r["gbs"], r["gbs_per_cu"],
+                     ", L2 hits %.0f GB/s" % r["l2_hit_gbs"] if r.get("l2_hit_gbs") else ""))
             be.close()
             return
         if a.only == "stream-floor":

@@ -214,6 +214,8 @@ SIGNATURES = {
     "fa_gemm_plan_query": (C.c_int32, [ctx_p, u64, qw_p, C.POINTER(GemmPlan)]),
     "fa_graph_owned_blocks": (C.c_int32, [C.c_void_p, C.POINTER(C.c_void_p), u64, C.POINTER(u64)]),
     "fa_topology_query": (C.c_int32, [ctx_p, i32p, i32p]),
+    "fa_probe_l2_path": (C.c_int32, [ctx_p, buf_p, u64, u64, buf_p, C.c_uint32, C.c_uint32, C.c_int32, C.c_int32, C.c_int32,
+                                     C.c_int32, buf_p]),
 }
 
 for _name, (_res, _args) in SIGNATURES.items():

@@ -748,6 +748,30 @@ fa_status fa_probe_stream_read(fa_context *ctx, const fa_buffer *src, uint64_t o
     return after_launch(ctx, "stream_read_probe");
 }
 
+fa_status fa_probe_l2_path(fa_context *ctx, const fa_buffer *cold, uint64_t cold_offset_bytes, uint64_t cold_bytes,
+                           const fa_buffer *hot, uint32_t hot_bytes, uint32_t hot_passes, int32_t in_flight,
+                           int32_t hot_per_cold, int32_t blocks, int32_t threads, fa_buffer *sink) {
+    if (fa_status s = check_ctx(ctx)) return s;
+    if (fa_status s = check_buf(ctx, cold, "probe_l2_path: cold")) return s;
+    if (fa_status s = check_buf(ctx, hot, "probe_l2_path: hot")) return s;
+    if (fa_status s = check_buf(ctx, sink, "probe_l2_path: sink")) return s;
+    if (blocks <= 0 || blocks > 65536 || threads < 64 || threads > 512 || threads % 64 != 0)
+        return fail(FA_ERR_INVALID_ARGUMENT, "probe_l2_path: blocks in 1..=65536, threads a multiple of 64 up to 512");
+    const uint64_t have = cold->numel * dtype_size(cold->dtype);
+    uint64_t end;
+    if (cold_offset_bytes % 16 != 0 || __builtin_add_overflow(cold_offset_bytes, cold_bytes, &end) || end > have)
+        return fail(FA_ERR_INVALID_ARGUMENT, "probe_l2_path: cold range exceeds the buffer or is not 16-byte aligned");
+    if (hot_bytes < 16u * 512u || hot_bytes % 16 != 0 || hot_bytes > hot->numel * dtype_size(hot->dtype))
+        return fail(FA_ERR_INVALID_ARGUMENT, "probe_l2_path: hot region must hold 8 KiB .. its buffer, a multiple of 16 bytes");
+    if (sink->numel * dtype_size(sink->dtype) < 4) return fail(FA_ERR_SHAPE_MISMATCH, "probe_l2_path: sink too small");
+    if (cold_bytes == 0 && hot_passes == 0) return FA_OK;
+    if (cold_bytes != 0 && cold_bytes < 16ull * (uint64_t)blocks) return FA_OK;
+    if (!k::l2_path_probe((const char *)cold->ptr + cold_offset_bytes, cold_bytes, hot->ptr, hot_bytes, hot_passes, in_flight,
+                          hot_per_cold, blocks, threads, (int *)sink->ptr, ctx->stream))
+        return fail(FA_ERR_INVALID_ARGUMENT, "probe_l2_path: in_flight must be 8 or 16 and hot_per_cold 0 or 2");
+    return after_launch(ctx, "l2_path_probe");
+}
+
 fa_status fa_convert(fa_context *ctx, const fa_buffer *src, uint64_t numel, fa_buffer *dst) {
     if (fa_status s = check_ctx(ctx)) return s;
     if (fa_status s = check_buf(ctx, src, "convert: src")) return s;

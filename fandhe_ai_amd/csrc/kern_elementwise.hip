@@ -89,7 +89,9 @@ __global__ void gather_rows_kernel(const float *__restrict__ table, uint64_t tab
 __global__ void f32_to_bf16_kernel(const float *__restrict__ in, uint16_t *__restrict__ out, uint64_t n) {
     uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
     uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
-    for (; i < n; i += stride) out[i] = f32_to_bf16(in[i]);
+    // pairs go through the hardware converter, which the GEMM epilogues use too (an odd tail takes the integer form)
+    for (; 2 * i + 1 < n; i += stride) ((uint32_t *)out)[i] = f32x2_to_bf16x2(in[2 * i], in[2 * i + 1]);
+    if (n % 2 == 1 && blockIdx.x == 0 && threadIdx.x == 0) out[n - 1] = f32_to_bf16(in[n - 1]);
 }
 __global__ void bf16_to_f32_kernel(const uint16_t *__restrict__ in, float *__restrict__ out, uint64_t n) {
     uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;

@@ -453,8 +453,9 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
 #pragma unroll
                 for (int i = 0; i < AI; ++i) {
                     const v4i &x0 = a[i][0], &x1 = a[i][1], &y0 = b[cur][0], &y1 = b[cur][1];
-                    mfma_acc(acc[i][j], v8i{x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]},
-                             v8i{y0[0], y0[1], y0[2], y0[3], y1[0], y1[1], y1[2], y1[3]});
+                    // weight fragment first: the accumulator tile comes out transposed (see the epilogue)
+                    mfma_acc(acc[i][j], v8i{y0[0], y0[1], y0[2], y0[3], y1[0], y1[1], y1[2], y1[3]},
+                             v8i{x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]});
                     if (tail) {
                         a[i][0] = *(const v4i *)(la + i * TILE + a_off[0]);
                         a[i][1] = *(const v4i *)(la + i * TILE + a_off[1]);
@@ -467,7 +468,7 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
                 for (int h = 0; h < 2; ++h)
 #pragma unroll
                     for (int i = 0; i < AI; ++i) {
-                        mfma_acc(acc[i][j], a[i][h], b[cur][h]);
+                        mfma_acc(acc[i][j], b[cur][h], a[i][h]);
                         if (tail) a[i][h] = *(const v4i *)(la + i * TILE + a_off[h]);
                     }
             }
@@ -485,8 +486,12 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
     for (int i = 0; i < AI; ++i) drain_row(acc[i]);
     __builtin_amdgcn_s_waitcnt(0x0F70);               // the repeated loads of the tail have landed too
 
-    // epilogue: lane l holds column l % 16 and rows 4 * (l / 16) + e of each 16 x 16 tile
-    const int g = lane / 16, c = lane % 16;
+    // Epilogue.  The matrix instructions took the weight fragment as their first operand, so an accumulator tile is
+    // the transpose of the usual one: lane l holds row l % 16 of the output tile and its columns 4 (l / 16) + e,
+    // e = 0 .. 3: four consecutive outputs of one row, which leave as one 8-byte (bf16) or 16-byte (f32) store
+    // without passing through LDS, the activation scale is one value per lane and row tile, and the channel scales
+    // of a tile are one 16-byte load.  Two bf16 roundings are one v_cvt_pk_bf16_f32.
+    const int g = lane / 16, r = lane % 16;
     float fscale = 0.0f;
     bool extras = false;
     const bool out_bf16 = ep.out_bf16 != 0;
@@ -500,74 +505,47 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
     }
     const uint32_t col0 = (nt0 + wn * WNT) * 16;      // first column of this wavefront
     const bool full_cols = nt0 + wn * WNT + WNT <= n_tiles && col0 + WNT * 16 <= n;
+    const bool row_scales = !FP8 || f8_rows;
     if (!extras && full_cols && n % 8 == 0) {
-        // Fast path: a lane's values of one 16-row band are 2 or 4 bytes each, 16 lanes per 32 / 64 byte
-        // piece of a row; they are transposed through LDS (free now) so that the band leaves as whole
-        // rows of WNT * 16 columns in 16-byte stores.
-        __syncthreads();                              // every wavefront is done with the operand stages
-        constexpr int COLS = WNT * 16;
-        constexpr int PITCH = COLS * 4 + 16;          // bytes; also enough for bf16
-        uint8_t *band = lds + wave * (16 * PITCH);
-        float swc[WNT];
-        if (!FP8 || f8_rows) {
+        v4f swc[WNT];
+        if (row_scales) {
 #pragma unroll
-            for (int j = 0; j < WNT; ++j) swc[j] = ep.sw[col0 + j * 16 + c];
+            for (int j = 0; j < WNT; ++j) swc[j] = *(const v4f *)(ep.sw + col0 + j * 16 + 4 * g);
         }
 #pragma unroll
         for (int i = 0; i < AI; ++i) {
-            const uint32_t row_base = m0 + (wm * AI + i) * 16;
-            float sxr[4];
-            if (!FP8 || f8_rows) {
+            const uint32_t row = m0 + (wm * AI + i) * 16 + r;
+            const bool row_ok = row < m;
+            const float sxr = row_scales ? ep.sx[row_ok ? row : m - 1] : 0.0f;
+            uint8_t *orow = (uint8_t *)ep.out + ((uint64_t)(row_ok ? row : m - 1) * n + col0 + 4 * g) * (out_bf16 ? 2 : 4);
+#pragma unroll
+            for (int j = 0; j < WNT; ++j) {
+                float v[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    uint32_t row = row_base + 4 * g + e;
-                    sxr[e] = ep.sx[row < m ? row : m - 1];
+                    if constexpr (FP8) v[e] = __fmul_rn(acc[i][j][e], f8_rows ? __fmul_rn(sxr, swc[j][e]) : fscale);
+                    else v[e] = __fmul_rn((float)acc[i][j][e], __fmul_rn(sxr, swc[j][e]));
                 }
+                if (!row_ok) continue;
+                if (out_bf16)
+                    *(v2u *)(orow + j * 32) = v2u{f32x2_to_bf16x2(v[0], v[1]), f32x2_to_bf16x2(v[2], v[3])};
+                else
+                    *(v4f *)(orow + j * 64) = v4f{v[0], v[1], v[2], v[3]};
             }
-#pragma unroll
-            for (int j = 0; j < WNT; ++j)
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    float v;
-                    if constexpr (FP8) v = __fmul_rn(acc[i][j][e], f8_rows ? __fmul_rn(sxr[e], swc[j]) : fscale);
-                    else v = __fmul_rn((float)acc[i][j][e], __fmul_rn(sxr[e], swc[j]));
-                    uint8_t *dst = band + (4 * g + e) * PITCH;
-                    if (out_bf16)
-                        *(uint16_t *)(dst + (j * 16 + c) * 2) = f32_to_bf16(v);
-                    else
-                        *(float *)(dst + (j * 16 + c) * 4) = v;
-                }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-            const int row_bytes = out_bf16 ? COLS * 2 : COLS * 4;
-            const int vec_per_row = row_bytes / 16;
-            for (int t = lane; t < 16 * vec_per_row; t += 64) {
-                const int r = t / vec_per_row, vcol = t % vec_per_row;
-                const uint32_t row = row_base + r;
-                if (row < m) {
-                    v4u val = *(const v4u *)(band + r * PITCH + vcol * 16);
-                    uint8_t *o = (uint8_t *)ep.out + ((uint64_t)row * n + col0) * (out_bf16 ? 2 : 4) + vcol * 16;
-                    *(v4u *)o = val;
-                }
-            }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         }
         return;
     }
 #pragma unroll
     for (int j = 0; j < WNT; ++j) {
-        const uint32_t col = (nt0 + wn * WNT + j) * 16 + c;
-        const bool col_ok = col < n && nt0 + wn * WNT + j < n_tiles;
-        float swc = 0.0f;
-        if (!FP8 || f8_rows) swc = col_ok ? ep.sw[col] : 0.0f;
 #pragma unroll
-        for (int i = 0; i < AI; ++i) {
+        for (int e = 0; e < 4; ++e) {
+            const uint32_t col = (nt0 + wn * WNT + j) * 16 + 4 * g + e;
+            const bool col_ok = col < n && nt0 + wn * WNT + j < n_tiles;
+            float swc = 0.0f;
+            if (row_scales) swc = col_ok ? ep.sw[col] : 0.0f;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const uint32_t row = m0 + (wm * AI + i) * 16 + 4 * g + e;
+            for (int i = 0; i < AI; ++i) {
+                const uint32_t row = m0 + (wm * AI + i) * 16 + r;
                 if (col_ok && row < m) {
                     const uint64_t o = (uint64_t)row * n + col;
                     float v;

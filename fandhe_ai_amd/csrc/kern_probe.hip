@@ -2,6 +2,8 @@
 // limits them (operands stay in registers, no memory traffic inside the loop).  The operand bits come
 // from a caller-supplied buffer, because the sustained rate of this part depends on them: with
 // all-zero operands the cores run at the published peak, with random bits the clock is held lower.
+#include <type_traits>
+
 #include "device_utils.hpp"
 #include "kernels.hpp"
 
@@ -77,9 +79,82 @@ __global__ void __launch_bounds__(512) stream_read_kernel(const v4u *__restrict_
     if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x12345678u) sink[0] = 1;   // keeps the loads alive
 }
 
+// The path from L2 to a compute unit, two measurements in one kernel.  Every block streams its own share of `cold`
+// (memory nobody has touched: HBM) with G 16-byte loads per thread in flight and, with every cold load, R ordinary
+// loads of a small region `hot` that all blocks share and that therefore sits in every XCD's L2 after the first
+// touch.  cold_vecs_per_block == 0: the hot region alone, `hot_passes` times per block (G loads in flight): what a
+// compute unit can pull from L2 at the launch's number of wavefronts.  R == 0: the cold stream alone.  Otherwise:
+// what L2 hits mixed R : 1 into an HBM stream cost that stream.
+template <int G, int R>
+__global__ void __launch_bounds__(512) l2_path_kernel(const v4u *__restrict__ cold, uint64_t cold_vecs_per_block,
+                                                      const v4u *__restrict__ hot, uint32_t hot_vecs, uint32_t hot_passes,
+                                                      int *sink) {
+    const uint32_t tid = threadIdx.x, nt = blockDim.x;
+    v4u acc = v4u{0, 0, 0, 0};
+    uint32_t hpos = (tid + blockIdx.x * 64u) % hot_vecs;           // blocks start at different lines of the region
+    if (cold_vecs_per_block == 0) {
+        const uint32_t trips = (uint32_t)(((uint64_t)hot_vecs * hot_passes + (uint64_t)nt * G - 1) / ((uint64_t)nt * G));
+        for (uint32_t t = 0; t < trips; ++t) {
+            v4u h[G];
+#pragma unroll
+            for (int u = 0; u < G; ++u) {
+                h[u] = hot[hpos];
+                hpos += nt;
+                hpos = hpos >= hot_vecs ? hpos - hot_vecs : hpos;
+            }
+#pragma unroll
+            for (int u = 0; u < G; ++u) acc ^= h[u];
+        }
+    } else {
+        const v4u *cb = cold + (uint64_t)blockIdx.x * cold_vecs_per_block;
+        for (uint64_t i = tid; i < cold_vecs_per_block; i += (uint64_t)nt * G) {
+            v4u c[G], h[G * (R ? R : 1)];
+#pragma unroll
+            for (int u = 0; u < G; ++u) {
+                const uint64_t idx = i + (uint64_t)u * nt;
+                c[u] = stream_load<true>(cb + (idx < cold_vecs_per_block ? idx : cold_vecs_per_block - 1));
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    h[u * R + r] = hot[hpos];
+                    hpos += nt;
+                    hpos = hpos >= hot_vecs ? hpos - hot_vecs : hpos;
+                }
+                __builtin_amdgcn_sched_barrier(0);               // keep the two kinds of loads interleaved as written
+            }
+#pragma unroll
+            for (int u = 0; u < G; ++u) acc ^= c[u];
+            if (R) {
+#pragma unroll
+                for (int u = 0; u < G * R; ++u) acc ^= h[u];
+            }
+        }
+    }
+    if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x12345678u) sink[0] = 1;   // keeps the loads alive
+}
+
 }  // namespace
 
 int g_probe_plain_loads = 0;
+
+bool l2_path_probe(const void *cold, uint64_t cold_bytes, const void *hot, uint32_t hot_bytes, uint32_t hot_passes, int in_flight,
+                   int hot_per_cold, int blocks, int threads, int *sink, hipStream_t s) {
+    const uint64_t cvb = cold_bytes / 16 / (uint64_t)blocks;
+    const uint32_t hv = hot_bytes / 16;
+    auto go = [&](auto g, auto r) {
+        l2_path_kernel<decltype(g)::value, decltype(r)::value><<<blocks, threads, 0, s>>>((const v4u *)cold, cvb, (const v4u *)hot, hv,
+                                                                                         hot_passes, sink);
+    };
+    using I8 = std::integral_constant<int, 8>;
+    using I16 = std::integral_constant<int, 16>;
+    using R0 = std::integral_constant<int, 0>;
+    using R2 = std::integral_constant<int, 2>;
+    if (in_flight == 8 && hot_per_cold == 0) go(I8{}, R0{});
+    else if (in_flight == 16 && hot_per_cold == 0) go(I16{}, R0{});
+    else if (in_flight == 8 && hot_per_cold == 2) go(I8{}, R2{});
+    else if (in_flight == 16 && hot_per_cold == 2) go(I16{}, R2{});
+    else return false;
+    return true;
+}
 
 void stream_read_probe(const void *src, uint64_t bytes, int blocks, int threads, int *sink, hipStream_t s) {
     const uint64_t vecs = bytes / 16 / (uint64_t)blocks;

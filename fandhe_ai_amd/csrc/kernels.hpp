@@ -278,6 +278,10 @@ void sample_rows_policy(const float *logits, int32_t *tokens, RowPolicy *policy,
 // Streaming read of `bytes` (a multiple of 16 * blocks) by `blocks` blocks of `threads` threads (non-temporal
 // loads unless tuning key 15 asks for ordinary ones).
 void stream_read_probe(const void *src, uint64_t bytes, int blocks, int threads, int *sink, hipStream_t s);
+// The L2 -> compute unit path (l2_path_kernel): cold_bytes == 0 reads the hot region alone; in_flight 8 or 16,
+// hot_per_cold 0 or 2; false for any other combination.
+bool l2_path_probe(const void *cold, uint64_t cold_bytes, const void *hot, uint32_t hot_bytes, uint32_t hot_passes, int in_flight,
+                   int hot_per_cold, int blocks, int threads, int *sink, hipStream_t s);
 double matrix_rate_probe(int kind, const void *operands, uint32_t iters, int num_cus, int *sink, hipStream_t s);
 
 // ---- decode-step glue (kern_decoder.hip) --------------------------------------

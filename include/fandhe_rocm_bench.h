@@ -39,6 +39,16 @@ fa_status fa_probe_matrix_rate(fa_context *ctx, int32_t kind, const fa_buffer *o
 fa_status fa_probe_stream_read(fa_context *ctx, const fa_buffer *src, uint64_t offset_bytes, uint64_t bytes,
                                int32_t blocks, int32_t threads, fa_buffer *sink);
 
+/* Queues the probe of the path from L2 to the compute units: `blocks` blocks of `threads` threads (64 .. 512, a
+ * multiple of 64).  cold_bytes > 0: every block streams its own share of cold_bytes starting cold_offset_bytes into
+ * `cold` with non-temporal 16-byte loads, in_flight (8 or 16) per thread, and with every one of them hot_per_cold
+ * (0 or 2) ordinary loads of the first hot_bytes of `hot`, a region all blocks share (L2 hits).  cold_bytes == 0:
+ * every block reads the hot region alone hot_passes times, in_flight loads per thread in flight.  Nothing is
+ * written; time the launch with an fa_timer. */
+fa_status fa_probe_l2_path(fa_context *ctx, const fa_buffer *cold, uint64_t cold_offset_bytes, uint64_t cold_bytes,
+                           const fa_buffer *hot, uint32_t hot_bytes, uint32_t hot_passes, int32_t in_flight,
+                           int32_t hot_per_cold, int32_t blocks, int32_t threads, fa_buffer *sink);
+
 /* Launch-shape knobs for experiments; value 0 restores the built-in choice.
  * The knobs are plain process-wide integers read by every context's launches:
  * set them while no other thread is submitting work.

@@ -253,6 +253,22 @@ def test_rope_and_elementwise_against_the_oracle():
     assert np.array_equal(be.download_owned(be.convert(be.upload(bf), fa.capi.F32)), o.from_bf16(bf))
 
 
+def test_bf16_conversion_equals_round_to_nearest_even_on_every_upper_half():
+    """The device's f32 -> bf16 conversion (pairs on the hardware converter, an odd tail on the integer form) against
+    the oracle's round-to-nearest-even on every 16-bit upper half combined with a zero, a below-tie, a tie, an
+    above-tie and an all-ones lower half: normal numbers, subnormals, signed zeros, infinities, and every NaN pattern
+    (a NaN must stay a NaN with its quiet bit set, as the integer form leaves it)."""
+    import fandhe_ai_amd as fa
+    be = ops()
+    hi = np.arange(1 << 16, dtype=np.uint32) << 16
+    bits = np.concatenate([hi | lo for lo in (0x0000, 0x0001, 0x7FFF, 0x8000, 0x8001, 0xFFFF)] + [hi[:1]]).astype(np.uint32)
+    v = bits.view(np.float32)                      # an odd count: the last element takes the scalar path
+    got = be.download_owned(be.convert(be.upload(v), fa.capi.BF16))
+    want = o.to_bf16(v)
+    bad = np.nonzero(got != want)[0]
+    assert bad.size == 0, [(hex(int(bits[i])), hex(int(got[i])), hex(int(want[i]))) for i in bad[:8]]
+
+
 def test_sync_points_are_rejected_during_graph_capture_and_graph_replays():
     import fandhe_ai_amd as fa
     be = ops()
