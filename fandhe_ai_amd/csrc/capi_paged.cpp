@@ -27,7 +27,7 @@ namespace {
 
 constexpr int kMaxDevices = 64;
 void *g_scratch_addr[kMaxDevices];      // per device: each GPU holds its own copy of the array
-bool g_scratch_tried[kMaxDevices];
+std::string g_scratch_error[kMaxDevices];   // what the last failed lookup on the device reported
 std::mutex g_scratch_mu;
 
 }  // namespace
@@ -35,26 +35,34 @@ std::mutex g_scratch_mu;
 namespace fa {
 // Called with `device` current (context creation).  The lookup may initialise the module on that device,
 // which is why it happens at set-up and not inside the entry point.
+// A lookup that fails is tried again by the next context created on the device (only a success is remembered);
+// the entry point reports the last failure's text.
 void static_scratch_init(int device) {
     if (device < 0 || device >= kMaxDevices) return;
     std::lock_guard<std::mutex> g(g_scratch_mu);
-    if (g_scratch_tried[device]) return;
-    g_scratch_tried[device] = true;
+    if (g_scratch_addr[device]) return;
     void *ptr = nullptr;
     hipError_t e = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch));
-    if (e != hipSuccess) {
+    if (e != hipSuccess || !ptr) {
+        g_scratch_error[device] = e != hipSuccess ? hipGetErrorString(e) : "hipGetSymbolAddress returned a null address";
         (void)hipGetLastError();
-        return;                           // the entry point reports it
+        return;
     }
+    g_scratch_error[device].clear();
     g_scratch_addr[device] = ptr;
 }
 }  // namespace fa
 
 namespace {
 
-void *scratch_address(int device) {
-    if (device < 0 || device >= kMaxDevices) return nullptr;
+// Device address of the array on `device`, or null with the reason in *why.
+void *scratch_address(int device, std::string *why) {
+    if (device < 0 || device >= kMaxDevices) {
+        *why = "device ordinal " + std::to_string(device) + " is outside the " + std::to_string(kMaxDevices) + " devices this entry point keeps an address for";
+        return nullptr;
+    }
     std::lock_guard<std::mutex> g(g_scratch_mu);
+    if (!g_scratch_addr[device]) *why = g_scratch_error[device].empty() ? "no context has been created on the device" : g_scratch_error[device];
     return g_scratch_addr[device];
 }
 
@@ -288,10 +296,11 @@ fa_status fa_paged_attention_decode_static(fa_context *ctx, const fa_buffer *q, 
                     "paged_attention_decode_static: the partial results of this shape need " + std::to_string(need) +
                         " bytes, the static scratch holds " + std::to_string(kStaticScratchBytes) +
                         " (fewer rows or kv heads, or fa_paged_attention_forward_device)");
-    void *ws = scratch_address(ctx->device);
+    std::string why;
+    void *ws = scratch_address(ctx->device, &why);
     if (!ws)
         return fail(FA_ERR_DEVICE_UNAVAILABLE, "paged_attention_decode_static: the address of the static scratch could not "
-                                               "be resolved when the context was created");
+                                               "be resolved when the context was created (" + why + ")");
     k::paged_attention_decode_bf16((const uint16_t *)q->ptr, (const uint16_t *)k_pool->ptr, (const uint16_t *)v_pool->ptr,
                                    (const uint32_t *)block_tables->ptr, (const uint32_t *)seq_lens->ptr, ps,
                                    (uint32_t)g_decode_waves, ws, out->ptr, out->dtype == FA_BF16, nullptr, ctx->stream);

@@ -582,6 +582,22 @@ fa_status fa_decoder_set_tokens(fa_context *ctx, fa_decoder *d, const int32_t *t
     return fa_upload_into(ctx, tokens, d->batch, d->tokens, 0);
 }
 
+// The position every row writes in a decode step must have a page (validate_paged_kv_append rejects a row
+// without a slot before anything is queued, crates/tensor-core/src/paged_kv.rs:222-290); checked on the host
+// mirror of the installed tables by every entry point that runs the step's launches.
+static fa_status check_step_room(const fa_decoder *d) {
+    const fa_decoder_config &c = d->cfg;
+    for (uint32_t b = 0; b < d->batch; ++b) {
+        const uint64_t pos = d->host_lens[b];
+        if (pos >= (uint64_t)c.max_blocks_per_seq * c.block_size)
+            return fail(FA_ERR_INVALID_ARGUMENT, "paged_kv: row " + std::to_string(b) + " has no room for one more token");
+        if (d->host_tables[(uint64_t)b * c.max_blocks_per_seq + pos / c.block_size] >= c.num_blocks)
+            return fail(FA_ERR_INVALID_ARGUMENT, "paged_kv: row " + std::to_string(b) + " has no page for position " +
+                                                     std::to_string(pos));
+    }
+    return FA_OK;
+}
+
 fa_status fa_decoder_step(fa_context *ctx, fa_decoder *d, int32_t use_graph) {
     if (fa_status s = check_ctx(ctx)) return s;
     if (fa_status s = check_dec(d)) return s;
@@ -597,22 +613,16 @@ fa_status fa_decoder_step(fa_context *ctx, fa_decoder *d, int32_t use_graph) {
     ps.num_kv_heads = d->cfg.n_kv_heads;
     ps.max_blocks_per_seq = d->cfg.max_blocks_per_seq;
     if (fa_status s = ensure_workspace(ctx, k::paged_decode_workspace_bytes(ps, (uint32_t)g_decode_waves))) return s;
-    // the position every row writes in this step must have a page (validate_paged_kv_append rejects a row
-    // without a slot before anything is queued, crates/tensor-core/src/paged_kv.rs:222-290)
-    for (uint32_t b = 0; b < d->batch; ++b) {
-        const uint64_t pos = d->host_lens[b];
-        const fa_decoder_config &c = d->cfg;
-        if (pos >= (uint64_t)c.max_blocks_per_seq * c.block_size)
-            return fail(FA_ERR_INVALID_ARGUMENT, "paged_kv: row " + std::to_string(b) + " has no room for one more token");
-        if (d->host_tables[(uint64_t)b * c.max_blocks_per_seq + pos / c.block_size] >= c.num_blocks)
-            return fail(FA_ERR_INVALID_ARGUMENT, "paged_kv: row " + std::to_string(b) + " has no page for position " +
-                                                     std::to_string(pos));
-    }
-    for (auto &len : d->host_lens) len += 1;            // mirrors the device-side advance of this step
+    if (fa_status s = check_step_room(d)) return s;
+    // The host mirror of the lengths follows the device-side advance of this step; every return below that has
+    // queued nothing takes the advance back.
+    auto advance = [&](int by) {
+        for (auto &len : d->host_lens) len += by;
+    };
     if (!use_graph) {
+        advance(1);
         fa_status es = enqueue_step(ctx, d);
-        if (es != FA_OK)
-            for (auto &len : d->host_lens) len -= 1;
+        if (es != FA_OK) advance(-1);
         return es;
     }
     if (d->graph_waves != g_decode_waves) drop_graphs(d);
@@ -621,8 +631,11 @@ fa_status fa_decoder_step(fa_context *ctx, fa_decoder *d, int32_t use_graph) {
         try {
             it = d->graphs.emplace(d->batch, nullptr).first;
         } catch (const std::exception &) {
-            return fail(FA_ERR_ALLOCATION_FAILED, "decoder_step: out of host memory");
+            return fail(FA_ERR_ALLOCATION_FAILED, "decoder_step: out of host memory");      // lengths not advanced yet
         }
+    }
+    advance(1);
+    if (it->second == nullptr) {
         fa_status cs = fa_graph_capture_begin(ctx);
         fa_graph *g = nullptr;
         if (cs == FA_OK) {
@@ -636,15 +649,14 @@ fa_status fa_decoder_step(fa_context *ctx, fa_decoder *d, int32_t use_graph) {
         }
         if (cs != FA_OK || !g) {
             d->graphs.erase(it);
-            for (auto &len : d->host_lens) len -= 1;    // nothing ran
+            advance(-1);                                // nothing ran
             return cs != FA_OK ? cs : fail(FA_ERR_KERNEL_LAUNCH_FAILED, "decoder_step: capture produced no graph");
         }
         it->second = g;
         d->graph_waves = g_decode_waves;
     }
     fa_status ls = fa_graph_launch(ctx, it->second);
-    if (ls != FA_OK)
-        for (auto &len : d->host_lens) len -= 1;
+    if (ls != FA_OK) advance(-1);
     return ls;
 }
 
@@ -809,8 +821,12 @@ fa_status fa_decoder_debug_step_until(fa_context *ctx, fa_decoder *d, int32_t st
     ps.num_kv_heads = d->cfg.n_kv_heads;
     ps.max_blocks_per_seq = d->cfg.max_blocks_per_seq;
     if (fa_status s = ensure_workspace(ctx, k::paged_decode_workspace_bytes(ps, (uint32_t)g_decode_waves))) return s;
+    if (fa_status s = check_step_room(d)) return s;
     for (auto &len : d->host_lens) len += 1;            // the bookkeeping stage advances the lengths on the device
-    return enqueue_step(ctx, d, stop_after);
+    fa_status es = enqueue_step(ctx, d, stop_after);
+    if (es != FA_OK)
+        for (auto &len : d->host_lens) len -= 1;
+    return es;
 }
 
 fa_status fa_decoder_debug_buffer(fa_decoder *d, int32_t which, fa_buffer **out) {

@@ -1,0 +1,131 @@
+// Index arithmetic of the kernels whose addressing is easy to get wrong, as plain functions that compile for the
+// device and for the host: the kernels call them, and a host program (tests/cpp/host_index_model_test.cpp) walks
+// every block, wavefront, lane and stage of every instantiation through the same functions and checks that each
+// LDS and global offset is in bounds, that a stage's bytes land where the fragment reads expect them, and that every
+// output element is written exactly once.  (The reference keeps such host models beside its own kernels:
+// crates/backend-rocm/src/gemm_model.rs, paged_kv_model.rs, norm_model.rs.)
+#pragma once
+
+#include <cstdint>
+
+#if defined(__HIPCC__)
+#define FA_HD __host__ __device__ __forceinline__ constexpr
+#else
+#define FA_HD inline constexpr
+#endif
+
+namespace fa {
+namespace ixm {
+
+// ------------------------------------------------------------------ large-tile GEMM (gemm_mfma_big_kernel)
+// Block tile 256 rows x NTB * 16 columns, NWAVES = 2 WM wavefronts (WM along m, 2 along n).  One stage is 128 bytes
+// of k: 16 A tiles and NTB B tiles of 2 KiB, each moved as two 1 KiB slices by direct global -> LDS loads that
+// write 16 bytes per lane at slice base + lane * 16.
+constexpr int kBigTk = 128, kBigTile = 2048, kBigRows = 256;
+constexpr int kBigStagesA = 3, kBigStagesB = 2;
+
+template <int NTB>
+struct BigLds {
+    static constexpr int a_stage = 16 * kBigTile, b_stage = NTB * kBigTile;
+    static constexpr int b_base = kBigStagesA * a_stage;
+    static constexpr int bytes = b_base + kBigStagesB * b_stage;
+};
+
+// Blocks of one XCD (the hardware deals consecutive ids round-robin over 8 XCDs) take consecutive tiles, m fastest.
+FA_HD void big_block_tile(uint32_t bid, uint32_t m_blocks, uint32_t n_blocks, uint32_t *mb, uint32_t *nb) {
+    const uint32_t total = m_blocks * n_blocks;
+    if (total % 8 == 0) bid = (bid % 8) * (total / 8) + bid / 8;
+    *mb = bid % m_blocks;
+    *nb = bid / m_blocks;
+}
+
+// A tile (of 16 rows) that wavefront `wave` moves with its load pair i, and the tile-local row of lane `lane`.
+template <int NWAVES>
+FA_HD int big_a_tile(int wave, int i) { return wave + NWAVES * i; }
+FA_HD int big_a_row(int lane) { return lane / 4; }
+// Byte offset inside the row's 128 stage bytes that lane `lane` fetches with load x (0 or 1) of a pair: the
+// 16-byte piece q = 2 ((p - rot) mod 4) + x, p = lane % 4, rot = r / 2 (e4m3) or r / 2 + 2 x (int8), r = lane / 4.
+template <bool FP8>
+FA_HD int big_a_src_byte(int lane, int x) {
+    const int r = lane / 4, p4 = lane % 4;
+    const int pp = (p4 - r / 2 - (FP8 ? 0 : 2 * x)) & 3;
+    return pp * 32 + x * 16;
+}
+// LDS byte offset of the slice that load (tile, h) of stage slot `slot` fills (the lane's 16 bytes go to + lane * 16).
+template <int NTB>
+FA_HD int big_a_lds_slice(int slot, int tile, int h) { return slot * BigLds<NTB>::a_stage + tile * kBigTile + h * 1024; }
+// Byte offsets, inside an A tile of a stage, of the two 16-byte operand reads of lane `lane`: e4m3 reads k bytes
+// 32 g .. 32 g + 15 (sub 0) and 32 g + 16 .. + 31 (sub 1) of row r; int8 reads k bytes 64 sub + 16 g .. + 15
+// (k-step `sub` of the stage), g = lane / 16, r = lane % 16.
+template <bool FP8>
+FA_HD int big_a_frag_off(int lane, int sub) {
+    const int g = lane / 16, r = lane % 16;
+    if (FP8) return sub * 1024 + (4 * r + ((g + r / 2) & 3)) * 16;
+    const int q = 4 * sub + g, x = q & 1;
+    return x * 1024 + (4 * r + (((q >> 1) + r / 2 + 2 * x) & 3)) * 16;
+}
+
+// B tile (block-local column tile) that wavefront `wave` moves with load pair i: a block of 14 tiles has no tiles
+// 14, 15, the wavefronts that would move them repeat tiles 0, 1.
+template <int NTB, int NWAVES>
+FA_HD int big_b_tile(int wave, int i) { return (wave + NWAVES * i) % NTB; }
+// Byte offset, inside the 2 KiB weight tile of a stage in memory, of lane `lane`'s 16 bytes of slice h: e4m3 tiles
+// hold 32 bytes per lane (slice h = its half h), int8 stages are two adjacent 1 KiB tiles of 16 bytes per lane.
+template <bool FP8>
+FA_HD int big_b_src_byte(int lane, int h) { return FP8 ? lane * 32 + h * 16 : h * 1024 + lane * 16; }
+template <int NTB>
+FA_HD int big_b_lds_slice(int slot, int tile, int h) {
+    return BigLds<NTB>::b_base + slot * BigLds<NTB>::b_stage + tile * kBigTile + h * 1024;
+}
+// First byte, inside a stage's B region, of the fragment (tile j of wavefront column wn, slice h) of lane `lane`.
+template <int NTB>
+FA_HD int big_b_frag_off(int wn, int j, int h, int lane) { return (wn * (NTB / 2) + j) * kBigTile + h * 1024 + lane * 16; }
+
+// Output element e (0 .. 3) of accumulator tile (i, j) of wavefront (wm, wn) in lane `lane`, block-local: the matrix
+// instructions take the weight fragment first, so a lane holds row lane % 16 and columns 4 (lane / 16) + e.
+template <int NTB, int WM>
+FA_HD void big_out_elem(int wm, int wn, int i, int j, int e, int lane, int *row, int *col) {
+    *row = (wm * (16 / WM) + i) * 16 + lane % 16;
+    *col = (wn * (NTB / 2) + j) * 16 + 4 * (lane / 16) + e;
+}
+
+// ------------------------------------------------------------------ streamed paged attention (decode_stream_kernel)
+// The pages of all sequences, laid end to end, are cut into ranges of `per` pages; range r owns pages
+// [r per, (r + 1) per) of that axis and leaves one partial result per sequence it touches, in slot r + b.
+FA_HD uint32_t stream_range_pages(uint32_t total_pages, uint32_t n_ranges, uint32_t min_pages) {
+    const uint32_t per = (total_pages + n_ranges - 1) / n_ranges;
+    return per < min_pages ? min_pages : per;
+}
+// Pages [lo, hi) of a sequence (in its own numbering) that range [rlo, rhi) covers; the sequence occupies [sb, eb)
+// of the axis and overlaps the range.
+FA_HD void stream_segment(uint32_t rlo, uint32_t rhi, uint32_t sb, uint32_t eb, uint32_t *lo, uint32_t *hi) {
+    *lo = (rlo > sb ? rlo : sb) - sb;
+    *hi = (rhi < eb ? rhi : eb) - sb;
+}
+FA_HD uint32_t stream_slot(uint32_t r, uint32_t b) { return r + b; }
+// Ranges whose partial results the merge of a sequence adds: the sequence starts at page `pre` of the axis and
+// holds npg pages.  An empty sequence has none (lo > hi).
+FA_HD void stream_merge_ranges(uint32_t pre, uint32_t npg, uint32_t per, uint32_t *r_lo, uint32_t *r_hi) {
+    *r_lo = npg ? pre / per : 1;
+    *r_hi = npg ? (pre + npg - 1) / per : 0;
+}
+
+// ------------------------------------------------------------------ split-k decode linears (w8a8 / w8a16_ksplit_kernel)
+// Block `bid` of a launch with S members per group: the members of a group are S blocks that differ by multiples
+// of 8 (one XCD).  A launch has 8 S ceil(n_groups / 8) blocks; groups at or past n_groups return at once.
+FA_HD void ksplit_block(uint32_t bid, uint32_t s, uint32_t *group, uint32_t *member) {
+    const uint32_t xcd = bid % 8, q = bid / 8;
+    *group = (q / s) * 8 + xcd;
+    *member = q % s;
+}
+FA_HD void ksplit_k_range(uint32_t k_tiles, uint32_t member, uint32_t s, uint32_t *lo, uint32_t *hi) {
+    *lo = (uint32_t)((uint64_t)k_tiles * member / s);
+    *hi = (uint32_t)((uint64_t)k_tiles * (member + 1) / s);
+}
+// First element of the partial tile set of (group, member) in the workspace; nacc = row tiles x S x 4 items of 64 lanes.
+FA_HD uint64_t ksplit_partial_base(uint32_t group, uint32_t member, uint32_t s, uint32_t nacc) {
+    return ((uint64_t)group * s + member) * ((uint64_t)nacc * 64);
+}
+
+}  // namespace ixm
+}  // namespace fa

@@ -10,6 +10,7 @@
 #include <type_traits>
 
 #include "device_utils.hpp"
+#include "index_models.hpp"
 #include "kernels.hpp"
 
 namespace fa {
@@ -293,10 +294,8 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
     const int tid = threadIdx.x, lane = tid % 64;
     const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
     const int wm = wave / 2, wn = wave % 2;
-    uint32_t bid = blockIdx.x;
-    const uint32_t total = m_blocks * n_blocks;
-    if (total % 8 == 0) bid = (bid % 8) * (total / 8) + bid / 8;
-    const uint32_t mb = bid % m_blocks, nb = bid / m_blocks;
+    uint32_t mb, nb;
+    ixm::big_block_tile(blockIdx.x, m_blocks, n_blocks, &mb, &nb);
     const uint32_t m0 = mb * 256, nt0 = nb * NTB;
     const uint64_t k_bytes = (uint64_t)k_steps * TK;
 
@@ -315,43 +314,26 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
     // slot 4 r + (g + r / 2) mod 4 of both slices; rot = r / 2 + 2 x for int8, whose k-group g of k-step s
     // is the single piece q = 4 s + g in slice q % 2, slot 4 r + (q / 2 + rot) mod 4 (without the 2 x
     // term the lanes of k-groups g and g + 1 would read the same banks of the two slices).
-    constexpr int B_L = FP8 ? 32 : 16, B_H = FP8 ? 16 : 1024;    // byte offsets of lane l and slice h in a tile
+    constexpr int B_H = FP8 ? 16 : 1024;             // byte offset of slice h in a stage's weight tile in memory
+    static_assert(ixm::big_b_src_byte<FP8>(0, 1) == B_H && ixm::kBigTk == TK && ixm::kBigTile == TILE, "index model out of step");
     const uint8_t *a_src[TPW][2];
     const uint8_t *b_src[TPW];
-    {
-        const int r = lane / 4, p4 = lane % 4;
+    // (the index expressions live in index_models.hpp, where a host program checks them for every instantiation)
 #pragma unroll
-        for (int i = 0; i < TPW; ++i) {
-            uint32_t row = m0 + (wave + NWAVES * i) * 16 + r;
-            row = row < m ? row : m - 1;
+    for (int i = 0; i < TPW; ++i) {
+        uint32_t row = m0 + ixm::big_a_tile<NWAVES>(wave, i) * 16 + ixm::big_a_row(lane);
+        row = row < m ? row : m - 1;
 #pragma unroll
-            for (int x = 0; x < 2; ++x) {
-                const int pp = (p4 - r / 2 - (FP8 ? 0 : 2 * x)) & 3;
-                a_src[i][x] = aq + (uint64_t)row * k_bytes + pp * 32 + x * 16;
-            }
-            // a block of NTB = 14 has no tiles 14, 15: the wavefronts that would move them repeat tiles
-            // 0, 1 instead (same bytes to the same place, served by the L1), which keeps the main loop
-            // free of branches
-            uint32_t t = nt0 + (wave + NWAVES * i) % NTB;
-            t = t < n_tiles ? t : n_tiles - 1;
-            b_src[i] = w_tiles + (uint64_t)t * k_steps * TILE + lane * B_L;
-        }
+        for (int x = 0; x < 2; ++x) a_src[i][x] = aq + (uint64_t)row * k_bytes + ixm::big_a_src_byte<FP8>(lane, x);
+        // a block of NTB = 14 has no tiles 14, 15: the wavefronts that would move them repeat tiles
+        // 0, 1 instead (same bytes to the same place, served by the L1), which keeps the main loop
+        // free of branches
+        uint32_t t = nt0 + ixm::big_b_tile<NTB, NWAVES>(wave, i);
+        t = t < n_tiles ? t : n_tiles - 1;
+        b_src[i] = w_tiles + (uint64_t)t * k_steps * TILE + ixm::big_b_src_byte<FP8>(lane, 0);
     }
     // byte offsets of this lane's two A operand reads inside a tile
-    int a_off[2];
-    {
-        const int g = lane / 16, r = lane % 16;
-        if constexpr (FP8) {
-            a_off[0] = (4 * r + ((g + r / 2) & 3)) * 16;
-            a_off[1] = a_off[0] + 1024;
-        } else {
-#pragma unroll
-            for (int sub = 0; sub < 2; ++sub) {
-                const int q = 4 * sub + g, x = q & 1;
-                a_off[sub] = x * 1024 + (4 * r + (((q >> 1) + r / 2 + 2 * x) & 3)) * 16;
-            }
-        }
-    }
+    const int a_off[2] = {ixm::big_a_frag_off<FP8>(lane, 0), ixm::big_a_frag_off<FP8>(lane, 1)};
     // LDS holds three stages of A and two of B: A runs two stages ahead of the multiplies, B one, so that
     // requests stay in flight across the wait at the top of a stage (with both operands one stage ahead
     // the path from L2 runs dry there; a third stage of both does not fit).
@@ -365,13 +347,12 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
     auto issue_a = [&](uint32_t ks, int slot, int idx) {
         const int i = idx / 2, h = idx % 2;
         __builtin_amdgcn_global_load_lds((gptr)(a_src[i][h] + (uint64_t)ks * TK),
-                                         (lptr)(lds + slot * A_STAGE + (wave + NWAVES * i) * TILE + h * 1024), 16, 0, 0);
+                                         (lptr)(lds + ixm::big_a_lds_slice<NTB>(slot, ixm::big_a_tile<NWAVES>(wave, i), h)), 16, 0, 0);
     };
     auto issue_b = [&](uint32_t ks, int slot, int idx) {
         const int i = idx / 2, h = idx % 2;
-        const int t = (wave + NWAVES * i) % NTB;
         __builtin_amdgcn_global_load_lds((gptr)(b_src[i] + (uint64_t)ks * TILE + h * B_H),
-                                         (lptr)(lds_b0 + slot * B_STAGE + t * TILE + h * 1024), 16, 0, 0);
+                                         (lptr)(lds + ixm::big_b_lds_slice<NTB>(slot, ixm::big_b_tile<NTB, NWAVES>(wave, i), h)), 16, 0, 0);
     };
 
     typedef typename std::conditional<FP8, v4f, v4i>::type acc_t;
@@ -407,7 +388,7 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
     // stage ks, which a wavefront reaches only after all its reads of stage ks - 1 have completed.
     int slot_a = 0;
     const uint8_t *la = lds + (wm * AI) * TILE;
-    const uint8_t *lb = lds_b0 + (wn * WNT) * TILE + lane * 16;
+    const uint8_t *lb = lds_b0 + ixm::big_b_frag_off<NTB>(wn, 0, 0, lane);      // fragment j, slice h at + j * TILE + h * 1024
     __builtin_amdgcn_s_waitcnt(0x0F70 | NLD);         // stage 0 of this wavefront has landed (A of stage 1 may not)
     __builtin_amdgcn_s_barrier();                     // a bare barrier: __syncthreads would add a fence on top
     v4i a[AI][2], b[2][2];                            // [..][slice]
@@ -446,7 +427,7 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
                 __builtin_amdgcn_s_barrier();         // stage ks + 1 visible to all; stage ks no longer read
                 slot_a = slot_a == 2 ? 0 : slot_a + 1;
                 la = lds + slot_a * A_STAGE + (wm * AI) * TILE;
-                lb = lds_b0 + (buf ^ 1) * B_STAGE + (wn * WNT) * TILE + lane * 16;
+                lb = lds_b0 + (buf ^ 1) * B_STAGE + ixm::big_b_frag_off<NTB>(wn, 0, 0, lane);
             }
             const bool tail = j + 1 == WNT;           // past the last stage the reads fetch stale, unused data
             if constexpr (FP8) {
@@ -491,7 +472,9 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
     // e = 0 .. 3: four consecutive outputs of one row, which leave as one 8-byte (bf16) or 16-byte (f32) store
     // without passing through LDS, the activation scale is one value per lane and row tile, and the channel scales
     // of a tile are one 16-byte load.  Two bf16 roundings are one v_cvt_pk_bf16_f32.
-    const int g = lane / 16, r = lane % 16;
+    int row_l0, col_l0;                               // block-local row of this lane in row tile 0, first column in tile 0
+    ixm::big_out_elem<NTB, WM>(wm, wn, 0, 0, 0, lane, &row_l0, &col_l0);
+    const int g = lane / 16;
     float fscale = 0.0f;
     bool extras = false;
     const bool out_bf16 = ep.out_bf16 != 0;
@@ -514,10 +497,10 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
         }
 #pragma unroll
         for (int i = 0; i < AI; ++i) {
-            const uint32_t row = m0 + (wm * AI + i) * 16 + r;
+            const uint32_t row = m0 + row_l0 + i * 16;
             const bool row_ok = row < m;
             const float sxr = row_scales ? ep.sx[row_ok ? row : m - 1] : 0.0f;
-            uint8_t *orow = (uint8_t *)ep.out + ((uint64_t)(row_ok ? row : m - 1) * n + col0 + 4 * g) * (out_bf16 ? 2 : 4);
+            uint8_t *orow = (uint8_t *)ep.out + ((uint64_t)(row_ok ? row : m - 1) * n + nt0 * 16 + col_l0) * (out_bf16 ? 2 : 4);
 #pragma unroll
             for (int j = 0; j < WNT; ++j) {
                 float v[4];
@@ -545,7 +528,7 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
             if (row_scales) swc = col_ok ? ep.sw[col] : 0.0f;
 #pragma unroll
             for (int i = 0; i < AI; ++i) {
-                const uint32_t row = m0 + (wm * AI + i) * 16 + r;
+                const uint32_t row = m0 + row_l0 + i * 16;
                 if (col_ok && row < m) {
                     const uint64_t o = (uint64_t)row * n + col;
                     float v;

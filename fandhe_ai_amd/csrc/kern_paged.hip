@@ -2,6 +2,7 @@
 // that keeps the reference's per-row summation order, and the decode fast
 // path (bf16, head_dim 128, 16-token pages, one query token, grouped-query).
 #include "device_utils.hpp"
+#include "index_models.hpp"
 #include "kernels.hpp"
 
 namespace fa {
@@ -189,8 +190,7 @@ __device__ __forceinline__ uint32_t seq_pages(const StreamParams &p, uint32_t vs
 
 // pages per range for this launch: the same value in every wavefront of both kernels
 __device__ __forceinline__ uint32_t range_pages(const StreamParams &p, uint32_t total) {
-    uint32_t per = (total + p.n_ranges - 1) / p.n_ranges;
-    return per < p.min_pages ? p.min_pages : per;
+    return ixm::stream_range_pages(total, p.n_ranges, p.min_pages);
 }
 
 template <int SP, int KD, int VD, int WPE, bool PF, int TT = 1>
@@ -244,8 +244,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, W
             bool bad = len_b > max_ctx;
             if constexpr (PF) bad = p.seq_lens[b] > max_ctx;
             const uint32_t ctx = len_b > max_ctx ? max_ctx : len_b;
-            const uint32_t lo = (rlo > sb ? rlo : sb) - sb;            // first page of the segment, in the sequence
-            const uint32_t hi = (rhi < eb ? rhi : eb) - sb;
+            uint32_t lo, hi;                                           // pages [lo, hi) of the sequence: this segment
+            ixm::stream_segment(rlo, rhi, sb, eb, &lo, &hi);
             const uint32_t n = hi - lo;                                // pages of this segment (>= 1)
             const uint32_t *tab = p.tables + (uint64_t)b * p.max_blocks_per_seq + lo;
 
@@ -515,7 +515,8 @@ __global__ void __launch_bounds__(256) decode_stream_merge_kernel(StreamParams p
     pre = s_pre[0] + s_pre[1] + s_pre[2] + s_pre[3];
     const uint32_t npg = seq_pages<false>(p, b, max_ctx);
     const uint32_t per = range_pages(p, tot);
-    const uint32_t r_lo = npg ? pre / per : 1, r_hi = npg ? (pre + npg - 1) / per : 0;   // empty sequence: no partials
+    uint32_t r_lo, r_hi;
+    ixm::stream_merge_ranges(pre, npg, per, &r_lo, &r_hi);   // empty sequence: no partials
     float mx = -INFINITY;
     float acc = 0.0f, den = 0.0f;
     constexpr int kOneTrip = 8;
@@ -621,7 +622,8 @@ __global__ void __launch_bounds__(kPrefillMergeThreads)
     }
     const uint32_t npg = seq_pages<true>(p, vq, max_ctx);
     const uint32_t per = range_pages(p, tot);
-    const uint32_t r_lo = npg ? pre / per : 1, r_hi = npg ? (pre + npg - 1) / per : 0;   // nothing streamed: no partials
+    uint32_t r_lo, r_hi;
+    ixm::stream_merge_ranges(pre, npg, per, &r_lo, &r_hi);   // nothing streamed: no partials
     const uint32_t seq = vq / p.qt, tiles = p.tpv / p.tpt, cols = p.tpt * p.group;
     const bool violation = p.seq_lens[seq] < p.l_new;              // possible only with unvalidated device tables
     for (uint32_t ci = part; ci < tiles * cols; ci += kSlots) {
@@ -700,7 +702,8 @@ __global__ void __launch_bounds__(1024) decode_stream_merge_quantize_kernel(Stre
     }
     const uint32_t npg = seq_pages<false>(p, b, max_ctx);
     const uint32_t per = range_pages(p, tot);
-    const uint32_t r_lo = npg ? pre / per : 1, r_hi = npg ? (pre + npg - 1) / per : 0;   // empty sequence: no partials
+    uint32_t r_lo, r_hi;
+    ixm::stream_merge_ranges(pre, npg, per, &r_lo, &r_hi);   // empty sequence: no partials
 
     // blockDim.x == num_heads * 32: thread (h, q) owns dims 4 q .. 4 q + 3 of head h
     const uint32_t h = threadIdx.x / 32, d4 = (threadIdx.x % 32) * 4;

@@ -9,6 +9,7 @@
 #include <type_traits>
 
 #include "device_utils.hpp"
+#include "index_models.hpp"
 #include "kernels.hpp"
 
 namespace fa {
@@ -762,9 +763,7 @@ __device__ __forceinline__ uint32_t meet_ticket(uint32_t *counter, uint32_t *slo
 // block -> (group, member) of a split-k launch: see above
 template <int S>
 __device__ __forceinline__ void ksplit_ids(uint32_t *group, uint32_t *member) {
-    const uint32_t xcd = blockIdx.x % 8, q = blockIdx.x / 8;
-    *group = (q / S) * 8 + xcd;
-    *member = q % S;
+    ixm::ksplit_block(blockIdx.x, S, group, member);
 }
 
 // W8A8, plain epilogue.  Item idx = (i * S + j) * 4 + e of a block is accumulator element e of row tile i, column
@@ -781,7 +780,8 @@ __global__ void __launch_bounds__(512)
     ksplit_ids<S>(&group, &member);
     if (group >= n_groups) return;                   // the same for every member of the group
     const uint32_t nt0 = group * S;
-    const uint32_t kt_lo = (uint32_t)((uint64_t)k_tiles * member / S), kt_hi = (uint32_t)((uint64_t)k_tiles * (member + 1) / S);
+    uint32_t kt_lo, kt_hi;
+    ixm::ksplit_k_range(k_tiles, member, S, &kt_lo, &kt_hi);
     const uint32_t len = kt_hi - kt_lo;
     const uint32_t cnt = len > (uint32_t)wave ? (len - wave + NW - 1) / NW : 0;
 
@@ -855,7 +855,7 @@ __global__ void __launch_bounds__(512)
             for (int e = 0; e < 4; ++e) red[wave][(i * S + j) * 4 + e][lane] = acc[i][j][e];
     __syncthreads();
     int own[NE];
-    int32_t *mine = partial + ((uint64_t)group * S + member) * (NACC * 64);
+    int32_t *mine = partial + ixm::ksplit_partial_base(group, member, S, NACC);
 #pragma unroll
     for (int q = 0; q < NE; ++q) {
         const int idx = wave + q * NW;
@@ -873,7 +873,7 @@ __global__ void __launch_bounds__(512)
     for (int q = 0; q < NE; ++q)
 #pragma unroll
         for (int r = 0; r < S; ++r)
-            other[q][r] = meet_load<LOCAL>(partial + ((uint64_t)group * S + r) * (NACC * 64) + (wave + q * NW) * 64 + lane);
+            other[q][r] = meet_load<LOCAL>(partial + ixm::ksplit_partial_base(group, r, S, NACC) + (wave + q * NW) * 64 + lane);
 #pragma unroll
     for (int q = 0; q < NE; ++q) {
         const int idx = wave + q * NW;
@@ -912,7 +912,8 @@ __global__ void __launch_bounds__(512)
     if (group >= n_groups) return;
     const uint32_t nt0 = group * S;
     const uint64_t k = (uint64_t)k_tiles * 64;
-    const uint32_t kt_lo = (uint32_t)((uint64_t)k_tiles * member / S), kt_hi = (uint32_t)((uint64_t)k_tiles * (member + 1) / S);
+    uint32_t kt_lo, kt_hi;
+    ixm::ksplit_k_range(k_tiles, member, S, &kt_lo, &kt_hi);
     const uint32_t len = kt_hi - kt_lo;
     const uint32_t cnt = len > (uint32_t)wave ? (len - wave + NW - 1) / NW : 0;
 
@@ -988,7 +989,7 @@ __global__ void __launch_bounds__(512)
             for (int e = 0; e < 4; ++e) red[wave][(i * S + j) * 4 + e][lane] = acc[i][j][e];
     __syncthreads();
     float own[NE];
-    float *mine = partial + ((uint64_t)group * S + member) * (NACC * 64);
+    float *mine = partial + ixm::ksplit_partial_base(group, member, S, NACC);
 #pragma unroll
     for (int q = 0; q < NE; ++q) {
         const int idx = wave + q * NW;
@@ -1006,7 +1007,7 @@ __global__ void __launch_bounds__(512)
     for (int q = 0; q < NE; ++q)
 #pragma unroll
         for (int r2 = 0; r2 < S; ++r2)
-            other[q][r2] = meet_load<LOCAL>(partial + ((uint64_t)group * S + r2) * (NACC * 64) + (wave + q * NW) * 64 + lane);
+            other[q][r2] = meet_load<LOCAL>(partial + ixm::ksplit_partial_base(group, r2, S, NACC) + (wave + q * NW) * 64 + lane);
 #pragma unroll
     for (int q = 0; q < NE; ++q) {
         const int idx = wave + q * NW;

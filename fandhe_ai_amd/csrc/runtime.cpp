@@ -459,6 +459,9 @@ fa_status fa_topology_query(const fa_context *ctx, int32_t *xcd_local, int32_t *
 
 fa_status fa_context_destroy(fa_context *ctx) {
     if (!ctx || ctx->magic != kCtxMagic) return fail(FA_ERR_INVALID_ARGUMENT, "fa_context_destroy: not a context");
+    if (ctx->live_graphs != 0)
+        return fail(FA_ERR_INVALID_ARGUMENT, "fa_context_destroy: " + std::to_string(ctx->live_graphs) +
+                                                 " graph(s) recorded on this context are still alive; destroy them first");
     (void)hipSetDevice(ctx->device);
     (void)hipStreamSynchronize(ctx->stream);
     std::pair<uint64_t, void *> ent;
@@ -706,6 +709,8 @@ fa_status fa_graph_capture_end(fa_context *ctx, fa_graph **out) {
         return fail(FA_ERR_ALLOCATION_FAILED, "host allocation of the graph handle failed");
     }
     gr->magic = kGraphMagic;
+    gr->ctx = ctx;
+    ctx->live_graphs += 1;
     gr->graph = g;
     gr->exec = exec;
     gr->owned.swap(ctx->capture_owned);
@@ -716,6 +721,7 @@ fa_status fa_graph_capture_end(fa_context *ctx, fa_graph **out) {
 fa_status fa_graph_launch(fa_context *ctx, fa_graph *graph) {
     if (fa_status s = check_ctx(ctx)) return s;
     if (!graph || graph->magic != kGraphMagic) return fail(FA_ERR_INVALID_ARGUMENT, "fa_graph_launch: not a graph");
+    if (graph->ctx != ctx) return fail(FA_ERR_DEVICE_MISMATCH, "fa_graph_launch: the graph was recorded on another context");
     if (ctx->capturing) return fail(FA_ERR_CAPTURE_IN_PROGRESS, "fa_graph_launch during capture");
     hipError_t e = hipGraphLaunch(graph->exec, ctx->stream);
     if (e != hipSuccess) return hip_fail(ctx, e, "hipGraphLaunch", FA_ERR_KERNEL_LAUNCH_FAILED);
@@ -725,9 +731,11 @@ fa_status fa_graph_launch(fa_context *ctx, fa_graph *graph) {
 fa_status fa_graph_destroy(fa_context *ctx, fa_graph *graph) {
     if (!graph) return FA_OK;
     if (graph->magic != kGraphMagic) return fail(FA_ERR_INVALID_ARGUMENT, "fa_graph_destroy: not a graph");
-    if (!graph->owned.empty() && !(ctx && ctx->magic == kCtxMagic))
-        return fail(FA_ERR_INVALID_ARGUMENT, "fa_graph_destroy: the graph owns device blocks, its context is needed");
-    if (ctx && ctx->magic == kCtxMagic) (void)hipStreamSynchronize(ctx->stream);
+    // The blocks a graph owns come from the pool of the context that recorded it and go back there, so that context
+    // and no other has to be passed (and has to be alive: fa_context_destroy refuses while graphs of it live).
+    if (!ctx || ctx->magic != kCtxMagic) return fail(FA_ERR_INVALID_ARGUMENT, "fa_graph_destroy: the graph's context is needed");
+    if (graph->ctx != ctx) return fail(FA_ERR_DEVICE_MISMATCH, "fa_graph_destroy: the graph was recorded on another context");
+    (void)hipStreamSynchronize(ctx->stream);
     (void)hipGraphExecDestroy(graph->exec);
     (void)hipGraphDestroy(graph->graph);
     // every replay has finished (synchronized above): the scratch the recorded kernels used is free again
@@ -736,6 +744,7 @@ fa_status fa_graph_destroy(fa_context *ctx, fa_graph *graph) {
         pool_free(ctx, b.ptr, b.bytes, b.cls);
     }
     graph->owned.clear();
+    if (ctx->live_graphs) ctx->live_graphs -= 1;
     graph->magic = 0;
     delete graph;
     return FA_OK;

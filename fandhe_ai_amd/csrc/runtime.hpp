@@ -95,6 +95,9 @@ struct fa_context {
     // are zero whenever no such launch is running)
     fa::k::SplitKArea splitk;
     int xcd_count = 0;            // distinct XCDs seen by the probe launch at creation
+    // graphs recorded on this context that are still alive; a context is not destroyed while one of them holds
+    // device blocks of its pool
+    uint64_t live_graphs = 0;
 };
 
 struct fa_buffer {
@@ -119,6 +122,7 @@ struct fa_qweight {
 
 struct fa_graph {
     uint32_t magic;
+    fa_context *ctx;          // the context whose stream recorded it: the only one that may replay or destroy it
     hipGraph_t graph;
     hipGraphExec_t exec;
     // device blocks whose addresses the recorded kernels hold; returned to the pool when the graph is destroyed

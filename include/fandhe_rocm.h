@@ -449,7 +449,11 @@ fa_status fa_paged_cache_restore_table(fa_paged_cache *cache, const fa_block_tab
  * (BackendOps::linear_chain_forward_captured, backend_ops.rs:4814;
  * docs/inference-chain-single-sync-design.md:175-186).  Between begin and end
  * every call on the context is recorded instead of executed; calls that
- * synchronize or allocate return FA_ERR_CAPTURE_IN_PROGRESS. */
+ * synchronize or allocate return FA_ERR_CAPTURE_IN_PROGRESS.  A graph belongs
+ * to the context that recorded it: only that context may launch or destroy it
+ * (another one gets FA_ERR_DEVICE_MISMATCH), the scratch blocks its kernels use
+ * return to that context's pool when it is destroyed, and fa_context_destroy
+ * refuses (FA_ERR_INVALID_ARGUMENT) while graphs of the context are alive. */
 typedef struct fa_graph fa_graph;
 fa_status fa_graph_capture_begin(fa_context *ctx);
 fa_status fa_graph_capture_end(fa_context *ctx, fa_graph **out);

@@ -20,6 +20,16 @@ def test_cpp_host_layer_on_a_toy_decoder():
     assert "checks ok" in r.stdout
 
 
+def test_kernel_index_arithmetic_on_the_host():
+    """The functions the large-tile GEMM, the streamed attention and the split-k linears use for their block, tile,
+    stage, LDS and workspace offsets (fandhe_ai_amd/csrc/index_models.hpp), walked on the host for every instantiation:
+    offsets in bounds, a stage's bytes where the operand reads expect them, every output written exactly once
+    (tests/cpp/host_index_model_test.cpp)."""
+    r = subprocess.run([host_binary("host_index_model_test")], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "checks ok" in r.stdout
+
+
 def test_cpp_header_compiles_standalone_with_warnings_as_errors(tmp_path):
     src = tmp_path / "t.cpp"
     src.write_text('#include "fandhe_rocm.hpp"\nint main() { return 0; }\n')

@@ -297,6 +297,36 @@ def test_sync_points_are_rejected_during_graph_capture_and_graph_replays():
     fa.check(lib.fa_graph_destroy(be._ctx, g))
 
 
+def test_a_graph_belongs_to_the_context_that_recorded_it():
+    """Another context may neither replay nor destroy a graph (its scratch blocks would land in the wrong pool), and a
+    context is not destroyed while one of its graphs is alive."""
+    import fandhe_ai_amd as fa
+    lib = fa.capi.lib
+    one, two = C.c_void_p(), C.c_void_p()
+    fa.check(lib.fa_context_create(0, C.byref(one)))
+    fa.check(lib.fa_context_create(0, C.byref(two)))
+    a, out = C.c_void_p(), C.c_void_p()
+    host = np.full(64, 2.0, np.float32)
+    fa.check(lib.fa_upload(one, fa.capi.F32, host.ctypes.data, 64, C.byref(a)))
+    fa.check(lib.fa_alloc_zeroed(one, fa.capi.F32, 64, C.byref(out)))
+    fa.check(lib.fa_graph_capture_begin(one))
+    fa.check(lib.fa_add(one, a, a, 64, out))
+    g = C.c_void_p()
+    fa.check(lib.fa_graph_capture_end(one, C.byref(g)))
+    assert lib.fa_graph_launch(two, g) == fa.capi.DEVICE_MISMATCH
+    assert lib.fa_graph_destroy(two, g) == fa.capi.DEVICE_MISMATCH
+    assert lib.fa_context_destroy(one) == fa.capi.INVALID_ARGUMENT and b"still alive" in lib.fa_last_error_message()
+    fa.check(lib.fa_graph_launch(one, g))
+    got = np.empty(64, np.float32)
+    fa.check(lib.fa_download(one, out, 0, got.ctypes.data, 64))
+    assert np.all(got == 4.0)
+    fa.check(lib.fa_graph_destroy(one, g))
+    for b in (a, out):
+        fa.check(lib.fa_buffer_free(one, b))
+    fa.check(lib.fa_context_destroy(one))
+    fa.check(lib.fa_context_destroy(two))
+
+
 def _capture(fa, be, fn):
     lib = fa.capi.lib
     g = C.c_void_p()

@@ -191,7 +191,10 @@ ACCEPT_CASES = [(17, 1, 0.3), (1000, 4, 0.5), (32000, 3, 0.2), (50257, 7, 1.0), 
 def test_speculative_acceptance_equals_the_oracle(vocab, k, spread):
     """fa_speculative_accept against verify_sampling of the oracle over many rounds with one running generator:
     drafts drawn on the device from the draft's weights (k = 0 calls), then the acceptance step; accepted count,
-    token and generator state must all equal the oracle's, for drafts close to and far from the target."""
+    token and generator state must all equal the oracle's, for drafts close to and far from the target.
+    The device adds the f64 normalisers and the cumulative draw as block-wide trees, the oracle (like the reference)
+    in index order: a sum may differ in its last bit, so agreement is shown for these seeds and inputs, not by
+    construction (parity unpinned at the last-bit level; same-seed token identity is not a contract)."""
     fa = _fa()
     be = ops()
     rng = np.random.default_rng(vocab * 31 + k)
