@@ -13,7 +13,7 @@ using namespace fa;
 namespace fa {
 namespace k {
 extern int g_gemm_f32_form, g_weight_prefetch, g_probe_plain_loads, g_rows_wide;
-extern int g_skinny_ksplit, g_skinny_ksplit_s;
+extern int g_skinny_ksplit, g_skinny_ksplit_s, g_row_fusion;
 extern int g_skinny_ntw, g_skinny_waves, g_skinny_astat, g_gemm_small_tiles, g_gemm_waves, g_gemm_ntb, g_gemm_split_fill;
 }
 int g_decode_waves = 0;
@@ -94,6 +94,7 @@ fa_status fa_set_tuning(int32_t key, int32_t value) {
         case 16: k::g_skinny_ksplit = value; return FA_OK;
         case 17: k::g_skinny_ksplit_s = value; return FA_OK;
         case 18: k::g_rows_wide = value; return FA_OK;
+        case 19: k::g_row_fusion = value; return FA_OK;
     }
     return fail(FA_ERR_INVALID_ARGUMENT, "fa_set_tuning: unknown key");
 }

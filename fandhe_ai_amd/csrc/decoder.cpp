@@ -162,6 +162,16 @@ fa_status enqueue_step(fa_context *ctx, fa_decoder *d, int stop_after = -1) {
         ep.out_bf16 = 0;
         return ep;
     };
+    auto norm_prologue = [&](const float *norm_w) {
+        k::RowPrologue pro;
+        pro.x = (const float *)d->h->ptr;
+        pro.norm_w = norm_w;
+        pro.eps = c.rms_eps;
+        pro.inv_n = 1.0f / (float)D;
+        pro.xq_tiled_out = (int8_t *)d->xq->ptr;
+        pro.sx_out = (float *)d->sx->ptr;
+        return pro;
+    };
     auto linear = [&](const fa_qweight *w, void *out, const float *residual) {
         k::linear_w8a8_skinny((const int8_t *)d->xq->ptr, (const int8_t *)w->codes->ptr, B, w->n, w->n_pad, w->k_pad,
                               epilogue(w, out, residual), cus, s, &ctx->splitk);
@@ -182,15 +192,21 @@ fa_status enqueue_step(fa_context *ctx, fa_decoder *d, int stop_after = -1) {
         const k::QkvRopeTargets t{(const float *)d->cos_sin->ptr, (const uint32_t *)d->slots->ptr, (uint16_t *)d->q_bf->ptr,
                                   (uint16_t *)L.k_pool->ptr, (uint16_t *)L.v_pool->ptr, c.n_heads, c.n_kv_heads,
                                   c.head_dim, pool_rows};
-        k::rmsnorm_quantize_i8((const float *)d->h->ptr, (const float *)L.attn_norm->ptr, c.rms_eps, nullptr,
-                               (int8_t *)d->xq->ptr, (float *)d->sx->ptr, B, m_pad, D, s,
-                               k::prefetch_for_linear_w8a8_qkv_rope_skinny((const int8_t *)L.wqkv->codes->ptr, B, L.wqkv->n_pad,
-                                                                           L.wqkv->k_pad, t, kPullQkv));
+        // With at most four rows the linears redo the row work in front of them inside their own launch
+        // (k::RowPrologue): the row stage then launches nothing and its outputs (codes, scales) appear with the
+        // linear's stage, written by one block of it.
+        const bool fuse_qkv = k::qkv_rope_fuses_norm(B, L.wqkv->k_pad);
+        if (!fuse_qkv)
+            k::rmsnorm_quantize_i8((const float *)d->h->ptr, (const float *)L.attn_norm->ptr, c.rms_eps, nullptr,
+                                   (int8_t *)d->xq->ptr, (float *)d->sx->ptr, B, m_pad, D, s,
+                                   k::prefetch_for_linear_w8a8_qkv_rope_skinny((const int8_t *)L.wqkv->codes->ptr, B, L.wqkv->n_pad,
+                                                                               L.wqkv->k_pad, t, kPullQkv));
         if (stop_here()) break;
         {
+            const k::RowPrologue pro = norm_prologue((const float *)L.attn_norm->ptr);
             k::linear_w8a8_qkv_rope_skinny((const int8_t *)d->xq->ptr, (const int8_t *)L.wqkv->codes->ptr,
                                            (const float *)d->sx->ptr, (const float *)L.wqkv->scales->ptr, B,
-                                           L.wqkv->n_pad, L.wqkv->k_pad, t, s);
+                                           L.wqkv->n_pad, L.wqkv->k_pad, t, s, fuse_qkv ? &pro : nullptr);
         }
         if (stop_here()) break;
         if (c.n_heads <= 32) {
@@ -210,17 +226,36 @@ fa_status enqueue_step(fa_context *ctx, fa_decoder *d, int stop_after = -1) {
         if (stop_here()) break;
         linear(L.wo, d->h->ptr, (const float *)d->h->ptr);
         if (stop_here()) break;
-        k::rmsnorm_quantize_i8((const float *)d->h->ptr, (const float *)L.ffn_norm->ptr, c.rms_eps, nullptr,
-                               (int8_t *)d->xq->ptr, (float *)d->sx->ptr, B, m_pad, D, s);
+        const bool fuse_gu = k::swiglu_fuses_norm(B, L.wgu->n_pad, L.wgu->k_pad, cus);
+        if (!fuse_gu)
+            k::rmsnorm_quantize_i8((const float *)d->h->ptr, (const float *)L.ffn_norm->ptr, c.rms_eps, nullptr,
+                                   (int8_t *)d->xq->ptr, (float *)d->sx->ptr, B, m_pad, D, s);
         if (stop_here()) break;
-        k::linear_w8a8_swiglu_skinny((const int8_t *)d->xq->ptr, (const int8_t *)L.wgu->codes->ptr,
-                                     (const float *)d->sx->ptr, (const float *)L.wgu->scales->ptr, B, L.wgu->n,
-                                     L.wgu->n_pad, L.wgu->k_pad, (float *)d->act->ptr, (float *)d->pmax->ptr, 4, cus, s);
+        {
+            const k::RowPrologue pro = norm_prologue((const float *)L.ffn_norm->ptr);
+            k::linear_w8a8_swiglu_skinny((const int8_t *)d->xq->ptr, (const int8_t *)L.wgu->codes->ptr,
+                                         (const float *)d->sx->ptr, (const float *)L.wgu->scales->ptr, B, L.wgu->n,
+                                         L.wgu->n_pad, L.wgu->k_pad, (float *)d->act->ptr, (float *)d->pmax->ptr, 4, cus, s,
+                                         fuse_gu ? &pro : nullptr);
+        }
         if (stop_here()) break;
-        k::quantize_rows_from_pmax(d->act->ptr, false, (const float *)d->pmax->ptr, (uint32_t)(F / 16),
-                                   (int8_t *)d->xq->ptr, (float *)d->sx->ptr, B, m_pad, F, s);
+        const bool fuse_down = F % 64 == 0 && k::plain_fuses_pmax_quantizer(B, L.wdown->n_pad, L.wdown->k_pad, cus);
+        if (!fuse_down)
+            k::quantize_rows_from_pmax(d->act->ptr, false, (const float *)d->pmax->ptr, (uint32_t)(F / 16),
+                                       (int8_t *)d->xq->ptr, (float *)d->sx->ptr, B, m_pad, F, s);
         if (stop_here()) break;
-        linear(L.wdown, d->h->ptr, (const float *)d->h->ptr);
+        if (fuse_down) {
+            k::RowPrologue pro;
+            pro.x = (const float *)d->act->ptr;
+            pro.pmax = (const float *)d->pmax->ptr;
+            pro.parts = (uint32_t)(F / 16);
+            pro.xq_tiled_out = (int8_t *)d->xq->ptr;
+            pro.sx_out = (float *)d->sx->ptr;
+            k::linear_w8a8_skinny(nullptr, (const int8_t *)L.wdown->codes->ptr, B, L.wdown->n, L.wdown->n_pad, L.wdown->k_pad,
+                                  epilogue(L.wdown, d->h->ptr, (const float *)d->h->ptr), cus, s, nullptr, &pro);
+        } else {
+            linear(L.wdown, d->h->ptr, (const float *)d->h->ptr);
+        }
         if (stop_here()) break;
     }
     if (stop_after >= 0 && stage > stop_after) return after_launch(ctx, "decoder step (partial)");

@@ -86,6 +86,19 @@ __global__ void gather_rows_kernel(const float *__restrict__ table, uint64_t tab
     for (uint64_t c = threadIdx.x; c < cols; c += blockDim.x) dst[c] = ok ? src[c] : __uint_as_float(0x7fc00000u);
 }
 
+// The same with 16-byte moves, one per thread, for rows whose length is a multiple of four: the few rows of a
+// decode step spread over as many threads as they have elements / 4, so the copy is one memory round trip.
+__global__ void __launch_bounds__(256)
+    gather_rows_vec_kernel(const v4f *__restrict__ table, uint64_t table_rows, uint64_t vec_cols, const int32_t *__restrict__ idx,
+                           v4f *__restrict__ out) {
+    const uint64_t r = blockIdx.y, c = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (c >= vec_cols) return;
+    const int32_t id = idx[r];
+    const bool ok = id >= 0 && (uint64_t)id < table_rows;
+    const float nan = __uint_as_float(0x7fc00000u);
+    out[r * vec_cols + c] = ok ? table[(uint64_t)id * vec_cols + c] : v4f{nan, nan, nan, nan};
+}
+
 __global__ void f32_to_bf16_kernel(const float *__restrict__ in, uint16_t *__restrict__ out, uint64_t n) {
     uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
     uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
@@ -178,6 +191,11 @@ void argmax_rows_f32(const float *x, int32_t *out, uint64_t rows, uint64_t cols,
 void gather_rows_f32(const float *table, uint64_t table_rows, uint64_t cols, const int32_t *idx, float *out,
                      uint64_t rows, hipStream_t s) {
     if (rows == 0 || cols == 0) return;
+    if (cols % 4 == 0 && rows <= 65535 && (uintptr_t)table % 16 == 0 && (uintptr_t)out % 16 == 0) {
+        const dim3 grid((unsigned)((cols / 4 + 255) / 256), (unsigned)rows);
+        gather_rows_vec_kernel<<<grid, 256, 0, s>>>((const v4f *)table, table_rows, cols / 4, idx, (v4f *)out);
+        return;
+    }
     gather_rows_kernel<<<(unsigned)rows, 256, 0, s>>>(table, table_rows, cols, idx, out);
 }
 void convert_f32_to_bf16(const float *in, uint16_t *out, uint64_t n, hipStream_t s) {

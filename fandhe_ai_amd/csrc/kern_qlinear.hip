@@ -11,6 +11,7 @@
 #include "device_utils.hpp"
 #include "index_models.hpp"
 #include "kernels.hpp"
+#include "row_prologue.hpp"
 
 namespace fa {
 namespace k {
@@ -23,6 +24,7 @@ int g_skinny_astat = 0;     // activation-stationary kernel: 0 by shape, 1 never
 int g_skinny_ksplit = 0;    // split k over the blocks of an XCD: 0 by shape, 1 never, 2 whenever it can run (agent-scope
                             // meeting), 3 whenever it can run (meeting in the XCD's L2), 4 by shape but agent scope
 int g_skinny_ksplit_s = 0;  // members per group of the split (0 by shape, 2 or 4)
+int g_row_fusion = 0;       // row work inside the linears for at most four rows: 0 by shape, 1 never
 
 namespace {
 
@@ -53,14 +55,21 @@ enum { kEpiPlain = 0, kEpiSwiglu = 1, kEpiRope = 2 };
 // a + head_dim/32 of one head, i.e. the two halves that the rotation pairs, rotates q and k heads by the
 // row's position (products rounded separately, no contraction), rounds once to bf16 and stores q rows
 // and the new K / V cache rows directly, so the f32 projection never reaches memory.
-template <int MT, int NTW, int NWAVES, int MODE>
+// PRO != 0 (at most four rows, eight wavefronts): the block makes its own activation codes from `pro` behind its first
+// weight loads (row_prologue.hpp: 1 RMSNorm + quantizer, 2 quantizer from partial maxima) and reads the activation
+// operand from LDS; xq_tiled is not read.
+template <int MT, int NTW, int NWAVES, int MODE, int PRO = 0>
 __global__ void __launch_bounds__(NWAVES * 64)
     w8a8_skinny_kernel(const int8_t *__restrict__ xq_tiled, const int8_t *__restrict__ w_tiles, uint32_t m,
-                       uint32_t n, uint32_t n_tiles, uint32_t k_tiles, EpiI8 ep) {
+                       uint32_t n, uint32_t n_tiles, uint32_t k_tiles, EpiI8 ep, RowPrologue pro) {
     constexpr bool SWIGLU = MODE == kEpiSwiglu, ROPE = MODE == kEpiRope;
     static_assert(MODE == kEpiPlain || NTW == 2, "the fused epilogues pair two tiles");
+    static_assert(PRO == 0 || (MT == 1 && NWAVES * 64 == kPrologueThreads), "row prologues: one row tile, 512 threads");
     constexpr int NACC = MT * NTW * 4;
     __shared__ int red[NWAVES][NACC][64];
+    extern __shared__ __attribute__((aligned(16))) int8_t pro_codes[];      // PRO: [m][k] activation codes
+    __shared__ float pro_sx[PRO ? kPrologueMaxRows : 1], pro_f[PRO ? 16 : 1];
+    __shared__ double pro_d[PRO ? 16 : 1];
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
     const uint32_t half_tiles = ROPE ? ep.head_dim / 32 : 0;
     const uint32_t nt0 = SWIGLU ? blockIdx.x
@@ -108,7 +117,7 @@ __global__ void __launch_bounds__(NWAVES * 64)
             const int e = idx % 4, j = (idx / 4) % NTW, i = idx / (4 * NTW);
             const uint32_t row = i * 16 + 4 * (lane / 16) + e, col = (nt0 + j) * 16 + lane % 16;
             if (idx < NACC && row < m && col < n) {
-                p_sx[q] = ep.sx[row];
+                if constexpr (PRO == 0) p_sx[q] = ep.sx[row];
                 p_sw0[q] = ep.sw[col];
                 if (ep.bias) p_x0[q] = ep.bias[col];
                 if (ep.residual) p_x1[q] = ep.residual[(uint64_t)row * n + col];
@@ -118,7 +127,7 @@ __global__ void __launch_bounds__(NWAVES * 64)
             const uint32_t row = i * 16 + 4 * (lane / 16) + e, col = nt0 * 16 + lane % 16;
             const uint32_t pair = SWIGLU ? n / 2 : ep.head_dim / 2;      // distance to the partner column
             if (idx < MT * 4 && row < m && col + pair < n) {
-                p_sx[q] = ep.sx[row];
+                if constexpr (PRO == 0) p_sx[q] = ep.sx[row];
                 p_sw0[q] = ep.sw[col];
                 p_sw1[q] = ep.sw[col + pair];
                 if constexpr (ROPE) {
@@ -135,7 +144,9 @@ __global__ void __launch_bounds__(NWAVES * 64)
     __builtin_amdgcn_sched_barrier(0);
 
     v4i a[D][MT], b[D][NTW];
-    auto load_slot = [&](int s, uint32_t it) {
+    // PRO: lane (g, r) reads k-group g of row r of the block's own codes; rows at or past m read row 0 (never stored)
+    const uint32_t pro_off = ((uint32_t)lane % 16 < m ? (uint32_t)lane % 16 : 0u) * (k_tiles * 64) + ((uint32_t)lane / 16) * 16;
+    auto load_b = [&](int s, uint32_t it) {
         const uint32_t kt = wave + (it < cnt ? it : cnt - 1) * NWAVES;
 #pragma unroll
         for (int j = 0; j < NTW; ++j) {
@@ -143,8 +154,19 @@ __global__ void __launch_bounds__(NWAVES * 64)
             nt = nt < n_tiles ? nt : n_tiles - 1;            // a tile past the edge is loaded clamped, never stored
             b[s][j] = stream_load<true>((const v4i *)(b_base + ((uint64_t)nt * k_tiles + kt) * 1024));
         }
+    };
+    auto load_a = [&](int s, uint32_t it) {
+        const uint32_t kt = wave + (it < cnt ? it : cnt - 1) * NWAVES;
+        if constexpr (PRO != 0) {
+            a[s][0] = *(const v4i *)(pro_codes + pro_off + kt * 64);
+        } else {
 #pragma unroll
-        for (int i = 0; i < MT; ++i) a[s][i] = *(const v4i *)(xq_tiled + ((uint64_t)i * k_tiles + kt) * 1024 + a_off[i]);
+            for (int i = 0; i < MT; ++i) a[s][i] = *(const v4i *)(xq_tiled + ((uint64_t)i * k_tiles + kt) * 1024 + a_off[i]);
+        }
+    };
+    auto load_slot = [&](int s, uint32_t it) {
+        load_b(s, it);
+        load_a(s, it);
     };
     auto mma_slot = [&](int s) {
 #pragma unroll
@@ -153,9 +175,36 @@ __global__ void __launch_bounds__(NWAVES * 64)
             for (int j = 0; j < NTW; ++j)
                 acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[s][i], b[s][j], acc[i][j], 0, 0, 0);
     };
-    if (cnt != 0) {
+    if constexpr (PRO != 0) {
+        // the rows are requested first, the first weight tiles behind them: the row work runs while the tiles travel
+        typename std::conditional<PRO == 1, NormRows, PmaxRows>::type rows;
+        if constexpr (PRO == 1) prologue_norm_load(pro, m, k_tiles * 64, rows);
+        else prologue_pmax_load(pro, m, k_tiles * 64, rows);
+        __builtin_amdgcn_sched_barrier(0);
+        if (cnt != 0) {
 #pragma unroll
-        for (int s = 0; s < D; ++s) load_slot(s, (uint32_t)s);
+            for (int s = 0; s < D; ++s) load_b(s, (uint32_t)s);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (PRO == 1) prologue_rmsnorm_quantize(pro, rows, m, k_tiles * 64, pro_codes, pro_sx, pro_d, pro_f);
+        else prologue_quantize_from_pmax(pro, rows, m, k_tiles * 64, pro_codes, pro_sx, pro_f);
+        prologue_publish(pro, m, k_tiles * 64, pro_codes, pro_sx);
+#pragma unroll
+        for (int q = 0; q < NE; ++q) {
+            const int idx = wave + q * NWAVES;
+            const uint32_t row = (uint32_t)(4 * (lane / 16) + idx % 4);      // one row tile: element idx % 4 of the lane
+            p_sx[q] = row < m ? pro_sx[row] : 0.0f;
+        }
+        if (cnt != 0) {
+#pragma unroll
+            for (int s = 0; s < D; ++s) load_a(s, (uint32_t)s);
+        }
+    }
+    if (cnt != 0) {
+        if constexpr (PRO == 0) {
+#pragma unroll
+            for (int s = 0; s < D; ++s) load_slot(s, (uint32_t)s);
+        }
         uint32_t it0 = 0;
         for (; it0 + D < cnt; it0 += D) {                     // a further group exists: refill while multiplying
 #pragma unroll
@@ -292,26 +341,34 @@ __global__ void __launch_bounds__(NWAVES * 64)
 // meet in LDS (two buffers, one barrier per unit) and wavefront w finishes the rows
 // 4 (l / 16) + w % 4 of row tile w / 4 for both tiles of the unit, so SwiGLU has
 // gate and up of an element in the same lane.
-template <int MT, int KTW, int MODE>
+// PRO == 1 (at most four rows): the block makes its own activation codes (RMSNorm + quantizer of `pro`, see
+// row_prologue.hpp) behind the weight loads of its first unit and takes its activation registers from LDS.
+template <int MT, int KTW, int MODE, int PRO = 0>
 __global__ void __launch_bounds__(512)
     w8a8_astat_kernel(const int8_t *__restrict__ xq_tiled, const int8_t *__restrict__ w_tiles, uint32_t m, uint32_t n,
-                      uint32_t n_tiles, uint32_t k_tiles, uint32_t n_units, EpiI8 ep) {
+                      uint32_t n_tiles, uint32_t k_tiles, uint32_t n_units, EpiI8 ep, RowPrologue pro) {
     constexpr bool SWIGLU = MODE == kEpiSwiglu;
     constexpr int NW = 8, NACC = MT * 2 * 4;
+    static_assert(PRO == 0 || (PRO == 1 && MT == 1), "row prologue: norm + quantizer, one row tile");
     __shared__ int red[2][NW][NACC][64];
+    extern __shared__ __attribute__((aligned(16))) int8_t pro_codes[];      // PRO: [m][k] activation codes
+    __shared__ float pro_sx[PRO ? kPrologueMaxRows : 1], pro_f[PRO ? 16 : 1];
+    __shared__ double pro_d[PRO ? 16 : 1];
     const int lane = threadIdx.x % 64;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
     const uint32_t last_kt = k_tiles - 1, last_tile = n_tiles - 1;
 
     // activations of this wavefront's k-tiles (clamped repeats past the end are never multiplied)
     v4i a[KTW][MT];
+    if constexpr (PRO == 0) {
 #pragma unroll
-    for (int t = 0; t < KTW; ++t) {
-        uint32_t kt = wave + NW * t;
-        kt = kt < k_tiles ? kt : last_kt;
+        for (int t = 0; t < KTW; ++t) {
+            uint32_t kt = wave + NW * t;
+            kt = kt < k_tiles ? kt : last_kt;
 #pragma unroll
-        for (int i = 0; i < MT; ++i)
-            a[t][i] = *(const v4i *)(xq_tiled + ((uint64_t)i * k_tiles + kt) * 1024 + (uint64_t)lane * 16);
+            for (int i = 0; i < MT; ++i)
+                a[t][i] = *(const v4i *)(xq_tiled + ((uint64_t)i * k_tiles + kt) * 1024 + (uint64_t)lane * 16);
+        }
     }
     auto tile_of = [&](uint32_t u, int j) -> uint32_t {
         uint32_t nt = SWIGLU ? u + j * (n_tiles / 2) : 2 * u + j;
@@ -326,7 +383,7 @@ __global__ void __launch_bounds__(512)
     };
     const uint32_t e_row = (wave / 4) * 16 + 4 * (lane / 16) + wave % 4;
     const bool e_wave = wave < MT * 4 && e_row < m;
-    const float e_sx = e_wave ? ep.sx[e_row] : 0.0f;
+    float e_sx = (PRO == 0 && e_wave) ? ep.sx[e_row] : 0.0f;
     auto load_unit = [&](uint32_t u, v4i (&b)[KTW][2], UnitEpi &ue) {
         u = u < n_units ? u : n_units - 1;
 #pragma unroll
@@ -423,7 +480,26 @@ __global__ void __launch_bounds__(512)
     v4i b0[KTW][2], b1[KTW][2];
     UnitEpi ue0, ue1;
     uint32_t u = blockIdx.x;
+    NormRows rows;
+    if constexpr (PRO != 0) {
+        // the rows are requested first, the first unit's weights behind them: the row work runs while they travel
+        prologue_norm_load(pro, m, k_tiles * 64, rows);
+        __builtin_amdgcn_sched_barrier(0);
+    }
     load_unit(u, b0, ue0);
+    if constexpr (PRO != 0) {
+        __builtin_amdgcn_sched_barrier(0);
+        prologue_rmsnorm_quantize(pro, rows, m, k_tiles * 64, pro_codes, pro_sx, pro_d, pro_f);
+        prologue_publish(pro, m, k_tiles * 64, pro_codes, pro_sx);
+        e_sx = e_wave ? pro_sx[e_row] : 0.0f;
+        const uint32_t off = ((uint32_t)lane % 16 < m ? (uint32_t)lane % 16 : 0u) * (k_tiles * 64) + ((uint32_t)lane / 16) * 16;
+#pragma unroll
+        for (int t = 0; t < KTW; ++t) {
+            uint32_t kt = wave + NW * t;
+            kt = kt < k_tiles ? kt : last_kt;
+            a[t][0] = *(const v4i *)(pro_codes + off + kt * 64);
+        }
+    }
     for (; u < n_units; u += 2 * gridDim.x) {
         load_unit(u + gridDim.x, b1, ue1);
         finish_unit(u, b0, ue0, 0);
@@ -1167,9 +1243,9 @@ void launch_w8a8_rows(uint64_t m, int waves, unsigned grid, hipStream_t s, A... 
     auto go = [&](auto mt) {
         constexpr int MT = decltype(mt)::value;
         if (waves == 8)
-            w8a8_skinny_kernel<MT, NTW, 8, MODE><<<grid, 512, 0, s>>>(args...);
+            w8a8_skinny_kernel<MT, NTW, 8, MODE><<<grid, 512, 0, s>>>(args..., RowPrologue{});
         else
-            w8a8_skinny_kernel<MT, NTW, 4, MODE><<<grid, 256, 0, s>>>(args...);
+            w8a8_skinny_kernel<MT, NTW, 4, MODE><<<grid, 256, 0, s>>>(args..., RowPrologue{});
     };
     if (m <= 16)
         go(std::integral_constant<int, 1>{});
@@ -1338,10 +1414,46 @@ WeightPrefetch prefetch_for_linear_w8a8_qkv_rope_skinny(const int8_t *w_tiles, u
     return make_prefetch(w_tiles, n / 32, (uint32_t)(n_pad / 16), (uint32_t)(k_pad / 64), half_tiles, 1, half_tiles, budget);
 }
 
+namespace {
+// bytes of LDS a block needs for its own activation codes
+inline size_t prologue_lds_bytes(uint64_t m, uint64_t k_pad) { return (size_t)((m * k_pad + 15) / 16 * 16); }
+inline bool norm_prologue_shape(uint64_t m, uint64_t k_pad) {
+    // the stand-alone kernel whose f64 association the prologue reproduces is the 1024-thread, one-group-per-thread form
+    return g_row_fusion != 1 && m >= 1 && m <= 4 && k_pad > 1024 && k_pad <= 4096 && k_pad % 64 == 0;
+}
+}  // namespace
+
+bool qkv_rope_fuses_norm(uint64_t m, uint64_t k_pad) { return norm_prologue_shape(m, k_pad) && !g_skinny_waves; }
+bool swiglu_fuses_norm(uint64_t m, uint64_t n_pad, uint64_t k_pad, int num_cus) {
+    return norm_prologue_shape(m, k_pad) && astat_applies(n_pad / 32, k_pad / 64, num_cus);
+}
+bool plain_fuses_pmax_quantizer(uint64_t m, uint64_t n_pad, uint64_t k_pad, int num_cus) {
+    if (g_row_fusion == 1 || m == 0 || m > 2 || k_pad % 64 != 0 || k_pad > 16384) return false;     // PmaxRows
+    if (k_pad / 16 > 1024) return false;                     // partial maxima per row the prologue reads
+    const uint64_t n_tiles = n_pad / 16, k_tiles = k_pad / 64;
+    if (astat_applies((n_tiles + 1) / 2, k_tiles, num_cus)) return false;
+    int ntw, waves;
+    pick_config(n_tiles, k_tiles, num_cus, &ntw, &waves);
+    return ntw == 1 && waves == 8;                          // the form the fused kernel is built in
+}
+
 void linear_w8a8_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t m, uint64_t n, uint64_t n_pad,
-                        uint64_t k_pad, const EpilogueI8 &ep, int num_cus, hipStream_t s, const SplitKArea *sk) {
+                        uint64_t k_pad, const EpilogueI8 &ep, int num_cus, hipStream_t s, const SplitKArea *sk,
+                        const RowPrologue *pro) {
     if (m == 0 || n == 0) return;
     uint32_t n_tiles = (uint32_t)(n_pad / 16), k_tiles = (uint32_t)(k_pad / 64);
+    if (pro) {                                              // the caller asked plain_fuses_pmax_quantizer first
+        EpiI8 e{};
+        e.sw = ep.sw;
+        e.bias = ep.bias;
+        e.residual = ep.residual;
+        e.acc_out = ep.acc_out;
+        e.out = ep.out;
+        e.out_bf16 = ep.out_bf16;
+        w8a8_skinny_kernel<1, 1, 8, kEpiPlain, 2><<<n_tiles, 512, prologue_lds_bytes(m, k_pad), s>>>(
+            nullptr, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e, *pro);
+        return;
+    }
     EpiI8 e{};
     e.sx = ep.sx;
     e.sw = ep.sw;
@@ -1363,9 +1475,9 @@ void linear_w8a8_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t 
         unsigned n_units = (n_tiles + 1) / 2;
         unsigned blocks = (unsigned)std::min<uint64_t>(n_units, (uint64_t)num_cus);
         if (m <= 16)
-            w8a8_astat_kernel<1, 8, kEpiPlain><<<blocks, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, n_units, e);
+            w8a8_astat_kernel<1, 8, kEpiPlain><<<blocks, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, n_units, e, RowPrologue{});
         else
-            w8a8_astat_kernel<2, 8, kEpiPlain><<<blocks, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, n_units, e);
+            w8a8_astat_kernel<2, 8, kEpiPlain><<<blocks, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, n_units, e, RowPrologue{});
         return;
     }
     int ntw, waves;
@@ -1379,7 +1491,7 @@ void linear_w8a8_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t 
 
 void linear_w8a8_swiglu_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, const float *sx, const float *sw,
                                uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad, float *act, float *pmax,
-                               int waves, int num_cus, hipStream_t s) {
+                               int waves, int num_cus, hipStream_t s, const RowPrologue *pro) {
     if (m == 0 || n == 0) return;
     uint32_t n_tiles = (uint32_t)(n_pad / 16), k_tiles = (uint32_t)(k_pad / 64);
     if (g_skinny_waves) waves = g_skinny_waves;
@@ -1388,19 +1500,26 @@ void linear_w8a8_swiglu_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, co
     e.sw = sw;
     e.out = act;
     e.pmax = pmax;
+    if (pro) {                                              // the caller asked swiglu_fuses_norm first
+        unsigned blocks = (unsigned)std::min<uint64_t>(n_tiles / 2, (uint64_t)num_cus);
+        w8a8_astat_kernel<1, 8, kEpiSwiglu, 1><<<blocks, 512, prologue_lds_bytes(m, k_pad), s>>>(
+            nullptr, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, n_tiles / 2, e, *pro);
+        return;
+    }
     if (m <= 32 && astat_applies(n_tiles / 2, k_tiles, num_cus)) {
         unsigned blocks = (unsigned)std::min<uint64_t>(n_tiles / 2, (uint64_t)num_cus);
         if (m <= 16)
-            w8a8_astat_kernel<1, 8, kEpiSwiglu><<<blocks, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, n_tiles / 2, e);
+            w8a8_astat_kernel<1, 8, kEpiSwiglu><<<blocks, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, n_tiles / 2, e, RowPrologue{});
         else
-            w8a8_astat_kernel<2, 8, kEpiSwiglu><<<blocks, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, n_tiles / 2, e);
+            w8a8_astat_kernel<2, 8, kEpiSwiglu><<<blocks, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, n_tiles / 2, e, RowPrologue{});
         return;
     }
     launch_w8a8_rows<2, kEpiSwiglu>(m, waves, n_tiles / 2, s, xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e);
 }
 
 void linear_w8a8_qkv_rope_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, const float *sx, const float *sw,
-                                 uint64_t m, uint64_t n_pad, uint64_t k_pad, const QkvRopeTargets &t, hipStream_t s) {
+                                 uint64_t m, uint64_t n_pad, uint64_t k_pad, const QkvRopeTargets &t, hipStream_t s,
+                                 const RowPrologue *pro) {
     if (m == 0) return;
     uint32_t n = (t.heads + 2 * t.kv_heads) * t.head_dim;
     uint32_t n_tiles = (uint32_t)(n_pad / 16), k_tiles = (uint32_t)(k_pad / 64);
@@ -1417,6 +1536,11 @@ void linear_w8a8_qkv_rope_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, 
     e.head_dim = t.head_dim;
     e.pool_rows = t.pool_rows;
     unsigned grid = n / 32;                                  // one block per pair of 16-column tiles
+    if (pro) {                                               // the caller asked qkv_rope_fuses_norm first
+        w8a8_skinny_kernel<1, 2, 8, kEpiRope, 1><<<grid, 512, prologue_lds_bytes(m, k_pad), s>>>(nullptr, w_tiles, (uint32_t)m, n, n_tiles,
+                                                                                              k_tiles, e, *pro);
+        return;
+    }
     int waves = g_skinny_waves ? g_skinny_waves : 8;
     launch_w8a8_rows<2, kEpiRope>(m, waves, grid, s, xq_tiled, w_tiles, (uint32_t)m, n, n_tiles, k_tiles, e);
 }

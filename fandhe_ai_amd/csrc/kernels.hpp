@@ -138,17 +138,37 @@ struct SplitKArea {
 };
 // out[b] = hardware id of the XCD workgroup b of the probe launch ran on (b < blocks)
 void xcc_id_probe(uint32_t *out, uint32_t blocks, hipStream_t s);
+// Row work that a decode-shape linear of at most four rows does for itself (row_prologue.hpp) instead of reading
+// ready-made codes: the RMSNorm + per-token quantizer of x (norm_w set), or the quantizer of x from `parts` partial
+// absolute maxima per row (norm_w null).  Same arithmetic as the stand-alone row kernels, so the linear's result
+// is bit-identical to theirs followed by the unfused linear.  xq_tiled_out / sx_out (nullable) receive what the
+// stand-alone kernel would have written (one block of the linear writes them).
+struct RowPrologue {
+    const float *x = nullptr;       // [m, k] f32
+    const float *norm_w = nullptr;  // [k]
+    const float *pmax = nullptr;    // [m, parts]
+    uint32_t parts = 0;
+    float eps = 0.0f, inv_n = 0.0f;
+    int8_t *xq_tiled_out = nullptr;
+    float *sx_out = nullptr;
+};
+// Whether the three linears of a decode step take the row work in front of them into their own launch for m rows
+// (the caller then skips the row kernel and passes a RowPrologue): q | k | v and gate | up take the norm + quantizer,
+// the down projection the quantizer from partial maxima.
+bool qkv_rope_fuses_norm(uint64_t m, uint64_t k_pad);
+bool swiglu_fuses_norm(uint64_t m, uint64_t n_pad, uint64_t k_pad, int num_cus);
+bool plain_fuses_pmax_quantizer(uint64_t m, uint64_t n_pad, uint64_t k_pad, int num_cus);
 // xq_tiled: activation tiles (see quantize_rows_i8); m <= 64 (one to four row tiles of 16 per block).
 // sk (optional): lets narrow weights split k over groups of blocks (m <= 32).
 void linear_w8a8_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t m, uint64_t n,
                         uint64_t n_pad, uint64_t k_pad, const EpilogueI8 &ep, int num_cus,
-                        hipStream_t s, const SplitKArea *sk = nullptr);
+                        hipStream_t s, const SplitKArea *sk = nullptr, const RowPrologue *pro = nullptr);
 // gate_up projection fused with SwiGLU: the weight is [k, n] with gate columns [0, n/2) and up columns
 // [n/2, n), n/2 a multiple of 16; act[m, n/2] = silu(gate) * up (f32) and pmax[m, n/32] receives the
 // absmax of every 16-column block of act (consumed by quantize_rows_from_pmax).
 void linear_w8a8_swiglu_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, const float *sx, const float *sw,
                                uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad, float *act, float *pmax,
-                               int waves, int num_cus, hipStream_t s);
+                               int waves, int num_cus, hipStream_t s, const RowPrologue *pro = nullptr);
 // Fused q | k | v projection of a decode step: the weight is [k, (heads + 2 kv_heads) head_dim], head_dim a
 // multiple of 32; q and k heads are rotated (rotate-half pairing, cos/sin of the row's position from
 // cos_sin[m][head_dim]) and rounded once to bf16; q goes to q_out [m, heads * head_dim], the new K / V rows
@@ -161,7 +181,8 @@ struct QkvRopeTargets {
     uint64_t pool_rows;
 };
 void linear_w8a8_qkv_rope_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, const float *sx, const float *sw,
-                                 uint64_t m, uint64_t n_pad, uint64_t k_pad, const QkvRopeTargets &t, hipStream_t s);
+                                 uint64_t m, uint64_t n_pad, uint64_t k_pad, const QkvRopeTargets &t, hipStream_t s,
+                                 const RowPrologue *pro = nullptr);
 // a: bf16 [m, k] row-major (k == k_pad required), m <= 32.
 void linear_w8a16_skinny(const uint16_t *a, const int8_t *w_tiles, const float *sw, uint64_t m,
                          uint64_t n, uint64_t n_pad, uint64_t k_pad, void *out, int out_bf16,

@@ -83,7 +83,10 @@ fa_status fa_probe_l2_path(fa_context *ctx, const fa_buffer *cold, uint64_t cold
  *        meeting in the XCD's L2, 4 by shape but meeting in memory;
  * key 17: blocks per group of that form: 0 by shape, 2 or 4;
  * key 18: 1 keeps the 256-thread form of the row kernels (norm, quantizer, norm + quantizer) for every row count
- *        instead of the up-to-1024-thread form used for at most 256 rows. */
+ *        instead of the up-to-1024-thread form used for at most 256 rows;
+ * key 19: 1 keeps the norm + quantizer and quantizer kernels of a decode step as launches of their own for every batch
+ *        size; 0: for at most four rows the linears that follow do that row work themselves (takes effect when a step
+ *        is recorded). */
 fa_status fa_set_tuning(int32_t key, int32_t value);
 
 /* What the context found when it was created: xcd_local = 1 when workgroups b and b + 8 of a launch were seen to

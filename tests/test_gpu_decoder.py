@@ -82,6 +82,108 @@ def test_decode_steps_match_the_oracle_eager_and_graph(shape, astat):
         fa.check(fa.capi.lib.fa_set_tuning(5, 0))
 
 
+@pytest.mark.parametrize("shape", [
+    dict(n_layers=2, d_model=2048, n_heads=16, n_kv_heads=4, d_ffn=3072, vocab=3000),
+    # the benchmark's width, one layer: gate / up takes the activation-stationary kernel by shape
+    dict(n_layers=1, d_model=4096, n_heads=32, n_kv_heads=8, d_ffn=14336, vocab=32000),
+], ids=["2048-wide", "benchmark-wide"])
+@pytest.mark.parametrize("batch", [1, 2, 3, 4])
+def test_small_batches_do_the_row_work_inside_the_linears(shape, batch):
+    """With one to four rows the q | k | v and gate | up projections do the norm + quantizer in front of them
+    themselves, and with one or two rows the down projection does its quantizer (no launch of their own for the row
+    kernels).  The steps must meet the oracle like any other batch, and every logit, token and cache row must be
+    bit-identical to the same steps with the row kernels launched separately (tuning key 19 = 1): a sequence decodes to
+    the same bits whatever batch it sits in.  The codes and scales the fused linears publish are those of the
+    stand-alone kernels as well (read back after the step: the down projection's)."""
+    import ctypes as C
+    import fandhe_ai_amd as fa
+    be = ops()
+    lib = fa.capi.lib
+    wide = shape["d_model"] == 4096
+    ctxs = [3, 130, 17, 64][:batch]
+    m = build_model(seed=21 + batch, steps=4, batch=batch, ctxs=ctxs, numpy_fill=wide, **shape)
+    if not wide:
+        fa.check(lib.fa_set_tuning(5, 2))                 # narrow test model: force the kernel gate / up uses at full width
+    outs, stages = {}, {}
+    try:
+        for fused in (True, False):
+            fa.check(lib.fa_set_tuning(19, 0 if fused else 1))
+            dec = GpuDecoder(be, m)
+            try:
+                # what the row stages leave behind, read after the linear that would consume it: the q | k | v projection
+                # (stage 2: the attention norm's codes and scales), gate | up (stage 6: the ffn norm's) and the down
+                # projection (stage 8: the SwiGLU quantizer's) of the first layer
+                got = []
+                for stage, k_cols in ((2, shape["d_model"]), (6, shape["d_model"]), (8, shape["d_ffn"])):
+                    dec.set_state(m.seq_lens, m.tokens)
+                    fa.check(lib.fa_decoder_debug_step_until(be._ctx, dec.h, stage))
+                    xq, sx = C.c_void_p(), C.c_void_p()
+                    fa.check(lib.fa_decoder_debug_buffer(dec.h, 1, C.byref(xq)))
+                    fa.check(lib.fa_decoder_debug_buffer(dec.h, 2, C.byref(sx)))
+                    codes = np.empty(16 * k_cols, np.int8)
+                    scales = np.empty(batch, np.float32)
+                    fa.check(lib.fa_download(be._ctx, xq, 0, codes.ctypes.data, codes.size))
+                    fa.check(lib.fa_download(be._ctx, sx, 0, scales.ctypes.data, batch))
+                    got.append((codes, scales))
+                stages[fused] = got
+                lens, tokens = m.seq_lens.copy(), m.tokens.copy()
+                trace = []
+                for step in range(3):
+                    dec.set_state(lens, tokens)
+                    dec.step(step > 0)
+                    trace.append((dec.logits().copy(), dec.tokens().copy(), [tuple(x.copy() for x in dec.kv_pool(li))
+                                                                             for li in range(shape["n_layers"])]))
+                    lens = lens + 1
+                    tokens = trace[-1][1]
+                outs[fused] = trace
+            finally:
+                dec.close()
+        for i, ((ca, sa), (cb, sb)) in enumerate(zip(stages[True], stages[False])):
+            assert np.array_equal(sa, sb), "scales of row stage %d differ between the fused and the separate row work" % i
+            assert np.array_equal(ca, cb), "codes of row stage %d differ between the fused and the separate row work" % i
+            assert np.any(ca != 0)
+        for step, (a, b) in enumerate(zip(outs[True], outs[False])):
+            assert np.array_equal(a[0], b[0]), "logits of step %d differ between the fused and the separate row work" % step
+            assert np.array_equal(a[1], b[1])
+            for (ak, av), (bk, bv) in zip(a[2], b[2]):
+                assert np.array_equal(ak, bk) and np.array_equal(av, bv)
+        # against the oracle, with the fused path
+        fa.check(lib.fa_set_tuning(19, 0))
+        dec = GpuDecoder(be, m)
+        try:
+            lens, tokens = m.seq_lens.copy(), m.tokens.copy()
+            for step in range(2):
+                tokens = _check_small(m, dec, lens, tokens, step > 0, "fused rows:B%d:step%d" % (batch, step))
+                dec.set_state(lens, tokens)
+        finally:
+            dec.close()
+    finally:
+        fa.check(lib.fa_set_tuning(19, 0))
+        fa.check(lib.fa_set_tuning(5, 0))
+
+
+def _check_small(m, dec, lens, tokens, use_graph, tag):
+    """_check_step with the bar for a handful of rows: a flipped code is not diluted by other rows, so every row is
+    held to mean < 4e-3 of its logit range and the median row to 2e-4."""
+    want_next, want_logits = oracle_step(m, lens, tokens)
+    dec.step(use_graph)
+    got_logits, got_next = dec.logits(), dec.tokens()
+    spread = want_logits.max(axis=1, keepdims=True) - want_logits.min(axis=1, keepdims=True)
+    err = np.abs(got_logits - want_logits) / spread
+    rows = err.mean(axis=1)
+    print("DECODE_STEP_PARITY\t%s\tmax_err/range=%.3e\trow means=%s" % (tag, err.max(), np.array2string(rows, precision=2)), flush=True)
+    assert rows.max() < 4e-3 and np.median(rows) < 2e-4 and err.max() < 2e-2
+    top2 = np.sort(want_logits, axis=1)[:, -2:]
+    decisive = (top2[:, 1] - top2[:, 0]) > 4e-2 * spread[:, 0]
+    assert np.array_equal(got_next[decisive], want_next[decisive])
+    assert np.array_equal(dec.seq_lens(), lens)
+    for li, L in enumerate(m.layers):
+        gk, gv = dec.kv_pool(li)
+        L["k_pool"][:] = gk
+        L["v_pool"][:] = gv
+    return got_next
+
+
 def test_decode_step_at_the_benchmark_width():
     """One layer of the benchmark's decoder at its full width (d_model 4096, 32 / 8 heads, FFN 14336, vocab
     32000), batch 32, contexts uniform in [1024, 8192]: the shapes at which the step's kernels are timed
