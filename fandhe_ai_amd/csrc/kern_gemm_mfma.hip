@@ -364,6 +364,12 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
             if constexpr (FP8) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
             else acc[i][j] = v4i{0, 0, 0, 0};
         }
+    // the per-tensor scales of the e4m3 epilogue are fetched here, not after the last stage, where the two dependent
+    // scalar loads would be a memory round trip that nothing overlaps
+    float fscale = 0.0f;
+    if constexpr (FP8) {
+        if (ep.sx == nullptr) fscale = __fmul_rn(*ep.a_scale, *ep.w_scale);
+    }
 
     // Per stage a wavefront issues its B loads of stage ks + 1 first and its A loads of stage ks + 2 after
     // them, so the wait at the top of stage ks + 1 can leave exactly those 2 TPW A loads outstanding.  Past
@@ -475,13 +481,11 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
     int row_l0, col_l0;                               // block-local row of this lane in row tile 0, first column in tile 0
     ixm::big_out_elem<NTB, WM>(wm, wn, 0, 0, 0, lane, &row_l0, &col_l0);
     const int g = lane / 16;
-    float fscale = 0.0f;
     bool extras = false;
     const bool out_bf16 = ep.out_bf16 != 0;
     bool f8_rows = false;
     if constexpr (FP8) {
         f8_rows = ep.sx != nullptr;
-        if (!f8_rows) fscale = __fmul_rn(*ep.a_scale, *ep.w_scale);
         extras = f8_rows && ep.bias != nullptr;
     } else {
         extras = ep.acc_out != nullptr || ep.bias != nullptr || ep.residual != nullptr;

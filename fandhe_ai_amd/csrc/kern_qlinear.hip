@@ -836,6 +836,24 @@ __device__ __forceinline__ uint32_t meet_ticket(uint32_t *counter, uint32_t *slo
     return *slot;
 }
 
+// LOCAL only: the members of a group must share an XCD, or the partial tiles above were exchanged through two
+// different L2s.  Every member notes the XCD it runs on before it takes its ticket; the last arriver compares and
+// reports a mismatch in host memory (the context then refuses further work: the launch's results are wrong).
+__device__ __forceinline__ uint32_t this_xcc() {
+    uint32_t id;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(id));
+    return id & 15u;
+}
+template <int S>
+__device__ __forceinline__ void meet_check_xcd(const uint32_t *xcc_seen, uint32_t group, uint32_t *fault) {
+    if (threadIdx.x != 0 || !xcc_seen) return;
+    const uint32_t mine = this_xcc();
+    bool same = true;
+#pragma unroll
+    for (int r = 0; r < S; ++r) same = same && meet_load<true>(xcc_seen + (uint64_t)group * S + r) == mine + 1u;
+    if (!same) __hip_atomic_store(fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
 // block -> (group, member) of a split-k launch: see above
 template <int S>
 __device__ __forceinline__ void ksplit_ids(uint32_t *group, uint32_t *member) {
@@ -847,7 +865,8 @@ __device__ __forceinline__ void ksplit_ids(uint32_t *group, uint32_t *member) {
 template <int MT, int S, int D, bool LOCAL>
 __global__ void __launch_bounds__(512)
     w8a8_ksplit_kernel(const int8_t *__restrict__ xq_tiled, const int8_t *__restrict__ w_tiles, uint32_t m, uint32_t n,
-                       uint32_t n_tiles, uint32_t k_tiles, uint32_t n_groups, EpiI8 ep, int32_t *partial, uint32_t *counters) {
+                       uint32_t n_tiles, uint32_t k_tiles, uint32_t n_groups, EpiI8 ep, int32_t *partial, uint32_t *counters,
+                       uint32_t *xcc_seen, uint32_t *fault) {
     constexpr int NW = 8, NACC = MT * S * 4, NE = NACC / NW;
     static_assert(NACC % NW == 0, "items divide over the wavefronts");
     __shared__ int red[NW][NACC][64];
@@ -941,9 +960,11 @@ __global__ void __launch_bounds__(512)
         own[q] = sum;
         meet_store<LOCAL>(mine + idx * 64 + lane, sum);
     }
+    if (LOCAL && xcc_seen && threadIdx.x == 0) meet_store<true>(xcc_seen + (uint64_t)group * S + member, this_xcc() + 1u);
     const uint32_t ticket = meet_ticket<LOCAL>(counters + group, (uint32_t *)&red[0][0][0]);
     if (ticket != S - 1) return;
     if (threadIdx.x == 0) meet_store<LOCAL>(counters + group, 0u);      // for the next launch
+    if constexpr (LOCAL) meet_check_xcd<S>(xcc_seen, group, fault);
     int other[NE][S];
 #pragma unroll
     for (int q = 0; q < NE; ++q)
@@ -977,7 +998,7 @@ template <int MT, int S, int D, bool LOCAL>
 __global__ void __launch_bounds__(512)
     w8a16_ksplit_kernel(const uint16_t *__restrict__ a, const int8_t *__restrict__ w_tiles, const float *__restrict__ sw,
                         uint32_t m, uint32_t n, uint32_t n_tiles, uint32_t k_tiles, uint32_t n_groups, void *__restrict__ out,
-                        int out_bf16, float *partial, uint32_t *counters) {
+                        int out_bf16, float *partial, uint32_t *counters, uint32_t *xcc_seen, uint32_t *fault) {
     constexpr int NW = 8, NACC = MT * S * 4, NE = NACC / NW;
     static_assert(NACC % NW == 0, "items divide over the wavefronts");
     __shared__ float red[NW][NACC][64];
@@ -1075,9 +1096,11 @@ __global__ void __launch_bounds__(512)
         own[q] = sum;
         meet_store<LOCAL>(mine + idx * 64 + lane, sum);
     }
+    if (LOCAL && xcc_seen && threadIdx.x == 0) meet_store<true>(xcc_seen + (uint64_t)group * S + member, this_xcc() + 1u);
     const uint32_t ticket = meet_ticket<LOCAL>(counters + group, (uint32_t *)&red[0][0][0]);
     if (ticket != S - 1) return;
     if (threadIdx.x == 0) meet_store<LOCAL>(counters + group, 0u);
+    if constexpr (LOCAL) meet_check_xcd<S>(xcc_seen, group, fault);
     float other[NE][S];
 #pragma unroll
     for (int q = 0; q < NE; ++q)
@@ -1313,6 +1336,11 @@ inline bool ksplit_plan(uint64_t m, uint32_t n_tiles, uint32_t k_tiles, int num_
     return true;
 }
 
+// the XCD notes of a launch, when the area has room for one word per block and a place to report to
+inline uint32_t *xcc_seen_for(const SplitKArea *sk, const KsplitPlan &p) {
+    return (sk->xcc_seen && sk->fault && (uint64_t)p.n_groups * p.s <= sk->n_xcc_seen) ? sk->xcc_seen : nullptr;
+}
+
 // Calls go(MT, S, D, LOCAL) with the plan's values as integral constants.
 template <typename F>
 void ksplit_dispatch(uint64_t m, const KsplitPlan &p, F &&go) {
@@ -1467,7 +1495,7 @@ void linear_w8a8_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t 
         ksplit_dispatch(m, kp, [&](auto mt, auto ss, auto d, auto local) {
             w8a8_ksplit_kernel<decltype(mt)::value, decltype(ss)::value, decltype(d)::value, decltype(local)::value>
                 <<<kp.blocks, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, kp.n_groups, e,
-                                           (int32_t *)sk->partial, sk->counters);
+                                           (int32_t *)sk->partial, sk->counters, xcc_seen_for(sk, kp), sk->fault);
         });
         return;
     }
@@ -1576,7 +1604,7 @@ void linear_w8a16_skinny(const uint16_t *a, const int8_t *w_tiles, const float *
         ksplit_dispatch(m, kp, [&](auto mt, auto ss, auto d, auto local) {
             w8a16_ksplit_kernel<decltype(mt)::value, decltype(ss)::value, decltype(d)::value, decltype(local)::value>
                 <<<kp.blocks, 512, 0, s>>>(a, w_tiles, sw, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, kp.n_groups, out, out_bf16,
-                                           (float *)sk->partial, sk->counters);
+                                           (float *)sk->partial, sk->counters, xcc_seen_for(sk, kp), sk->fault);
         });
         return;
     }

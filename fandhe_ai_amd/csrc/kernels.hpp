@@ -135,6 +135,12 @@ struct SplitKArea {
     uint32_t *counters = nullptr;
     uint32_t n_counters = 0;
     int xcd_local = 0;          // probed: workgroups b and b + 8 of a launch run on the same XCD (share an L2)
+    // Where the members of a group note the XCD they run on (one word per block of a launch, beside the partial
+    // tiles) and where the last arriver reports a group whose members did not share one: a word of pinned host
+    // memory that the device writes and the host reads at every entry (the results of that launch are wrong).
+    uint32_t *xcc_seen = nullptr;
+    uint32_t n_xcc_seen = 0;
+    uint32_t *fault = nullptr;
 };
 // out[b] = hardware id of the XCD workgroup b of the probe launch ran on (b < blocks)
 void xcc_id_probe(uint32_t *out, uint32_t blocks, hipStream_t s);

@@ -131,6 +131,11 @@ fa_pool_stats SizeClassPool::stats() {
 fa_status check_ctx(const fa_context *ctx) {
     if (!ctx || ctx->magic != kCtxMagic) return fail(FA_ERR_INVALID_ARGUMENT, "context: null or not a context");
     if (ctx->poisoned) return fail(FA_ERR_CONTEXT_POISONED, "context: poisoned by an earlier device failure");
+    // a split-k linear found the blocks of a group on different XCDs although the probe at creation said they share
+    // one: its partial tiles met through two L2s and what it wrote cannot be trusted
+    if (ctx->splitk.fault && *(volatile uint32_t *)ctx->splitk.fault != 0)
+        return fail(FA_ERR_CONTEXT_POISONED, "context: a split-k linear ran its groups across XCDs (results invalid); "
+                                             "recreate the context, or set tuning key 16 to 4 to let partial tiles meet in memory");
     return FA_OK;
 }
 fa_status check_buf(const fa_context *ctx, const fa_buffer *b, const char *what) {
@@ -411,9 +416,9 @@ fa_status fa_context_create(int32_t ordinal, fa_context **out) {
     // workgroups report the XCD they run on.  Without that property the partial tiles meet in memory instead.
     {
         constexpr uint64_t kPartial = 16ull << 20;
-        constexpr uint32_t kCounters = 4096, kProbe = 2048;
+        constexpr uint32_t kCounters = 4096, kProbe = 2048, kXccSeen = 16384;
         void *area = nullptr;
-        if (hipMalloc(&area, kPartial + kCounters * 4) == hipSuccess) {
+        if (hipMalloc(&area, kPartial + (kCounters + kXccSeen) * 4) == hipSuccess) {
             uint32_t *counters = (uint32_t *)((uint8_t *)area + kPartial);
             std::vector<uint32_t> ids(kProbe, 0xffu);
             fa::k::xcc_id_probe(counters, kProbe, ctx->stream);
@@ -429,7 +434,7 @@ fa_status fa_context_create(int32_t ordinal, fa_context **out) {
                 for (uint32_t b = 0; b < kProbe; ++b) seen[ids[b] & 15u] = true;
                 for (bool x : seen) ctx->xcd_count += x ? 1 : 0;
             }
-            ok = ok && hipMemsetAsync(area, 0, kPartial + kCounters * 4, ctx->stream) == hipSuccess &&
+            ok = ok && hipMemsetAsync(area, 0, kPartial + (kCounters + kXccSeen) * 4, ctx->stream) == hipSuccess &&
                  hipStreamSynchronize(ctx->stream) == hipSuccess;
             if (ok) {
                 ctx->splitk.partial = area;
@@ -437,6 +442,18 @@ fa_status fa_context_create(int32_t ordinal, fa_context **out) {
                 ctx->splitk.counters = counters;
                 ctx->splitk.n_counters = kCounters;
                 ctx->splitk.xcd_local = round_robin ? 1 : 0;
+                // one word per block of a launch (the groups' XCD notes) behind the counters, and the word of pinned
+                // host memory a launch reports a split group to
+                ctx->splitk.xcc_seen = counters + kCounters;
+                ctx->splitk.n_xcc_seen = kXccSeen;
+                void *flag = nullptr;
+                if (hipHostMalloc(&flag, 64, hipHostMallocMapped) == hipSuccess) {
+                    *(volatile uint32_t *)flag = 0;
+                    ctx->splitk.fault = (uint32_t *)flag;
+                } else {
+                    (void)hipGetLastError();
+                    ctx->splitk.xcc_seen = nullptr;        // nowhere to report to: no notes
+                }
             } else {
                 (void)hipGetLastError();
                 (void)hipFree(area);                 // the linears then keep to their unsplit forms
@@ -469,6 +486,7 @@ fa_status fa_context_destroy(fa_context *ctx) {
     if (ctx->table_stage) (void)hipFree(ctx->table_stage);
     if (ctx->workspace) (void)hipFree(ctx->workspace);
     if (ctx->splitk.partial) (void)hipFree(ctx->splitk.partial);
+    if (ctx->splitk.fault) (void)hipHostFree(ctx->splitk.fault);
     for (void *w : ctx->retired_workspaces) (void)hipFree(w);
     for (auto &b : ctx->capture_owned) (void)hipFree(b.ptr);   // a capture that was never ended
     for (void *p : ctx->deferred_frees) (void)hipFree(p);
