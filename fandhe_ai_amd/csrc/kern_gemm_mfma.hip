@@ -8,6 +8,7 @@
 // read at lane * 16.
 #include <algorithm>
 #include <type_traits>
+#include <utility>
 
 #include "device_utils.hpp"
 #include "index_models.hpp"
@@ -264,6 +265,51 @@ __device__ __forceinline__ void drain_row(T (&r)[8]) {
                  : "+a"(r[0]), "+a"(r[1]), "+a"(r[2]), "+a"(r[3]), "+a"(r[4]), "+a"(r[5]), "+a"(r[6]), "+a"(r[7]));
 }
 
+// LDS fragment reads and the waits for them, as assembly, for the large-tile kernel's main loop.  A read's result
+// may only be touched after an lds_wait that names it: the wait takes the registers as in/out operands, so every
+// use the compiler sees comes after it.  addr is an LDS byte address, OFF an immediate offset below 65536.
+template <int OFF>
+__device__ __forceinline__ void lds_read16(v4i &dst, uint32_t addr) {
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+}
+// At most N LDS reads issued before this point are still outstanding afterwards (N = 0 emits no instruction: the
+// caller has just waited for all of them).
+template <int N>
+__device__ __forceinline__ void lds_wait(v4i &x, v4i &y) {
+    if constexpr (N == 0) asm volatile("" : "+v"(x), "+v"(y));
+    else asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(x), "+v"(y) : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void lds_wait_all_a(v4i (&a)[2][2], v4i (&b)[2]) {
+    asm volatile("s_waitcnt lgkmcnt(%6)"
+                 : "+v"(a[0][0]), "+v"(a[0][1]), "+v"(a[1][0]), "+v"(a[1][1]), "+v"(b[0]), "+v"(b[1])
+                 : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void lds_wait_all_a(v4i (&a)[4][2], v4i (&b)[2]) {
+    asm volatile("s_waitcnt lgkmcnt(%10)"
+                 : "+v"(a[0][0]), "+v"(a[0][1]), "+v"(a[1][0]), "+v"(a[1][1]), "+v"(a[2][0]), "+v"(a[2][1]), "+v"(a[3][0]),
+                   "+v"(a[3][1]), "+v"(b[0]), "+v"(b[1])
+                 : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void lds_wait_all_a(v4i (&a)[8][2], v4i (&b)[2]) {
+    asm volatile("s_waitcnt lgkmcnt(%18)"
+                 : "+v"(a[0][0]), "+v"(a[0][1]), "+v"(a[1][0]), "+v"(a[1][1]), "+v"(a[2][0]), "+v"(a[2][1]), "+v"(a[3][0]),
+                   "+v"(a[3][1]), "+v"(a[4][0]), "+v"(a[4][1]), "+v"(a[5][0]), "+v"(a[5][1]), "+v"(a[6][0]), "+v"(a[6][1]),
+                   "+v"(a[7][0]), "+v"(a[7][1]), "+v"(b[0]), "+v"(b[1])
+                 : "n"(N));
+}
+template <int... I, typename F>
+__device__ __forceinline__ void static_for_seq(std::integer_sequence<int, I...>, F &&f) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a constant expression
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+    static_for_seq(std::make_integer_sequence<int, N>{}, f);
+}
+
 // ------------------------------------------------------------ large tiles
 // Block tile 256 rows x NTB * 16 columns, four wavefronts in 2 x 2, one per
 // SIMD, each owning 128 rows x NTB / 2 column tiles of accumulators (up to 256
@@ -393,25 +439,37 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
     // The loads overwrite the buffers of stage ks - 1; they are issued after the barrier that opened
     // stage ks, which a wavefront reaches only after all its reads of stage ks - 1 have completed.
     int slot_a = 0;
-    const uint8_t *la = lds + (wm * AI) * TILE;
-    const uint8_t *lb = lds_b0 + ixm::big_b_frag_off<NTB>(wn, 0, 0, lane);      // fragment j, slice h at + j * TILE + h * 1024
+    // Fragment reads are written as assembly with their own lgkmcnt waits (lds_read16 / lds_wait above): left to
+    // the compiler, every wait for a fragment becomes lgkmcnt(0), which also waits for the fragment of the NEXT
+    // group that was issued a moment earlier, and the read-ahead is lost.  Addresses are LDS byte offsets.
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(lptr)lds;
+    const uint32_t la_lane[2] = {lds0 + (wm * AI) * TILE + a_off[0], lds0 + (wm * AI) * TILE + a_off[1]};
+    const uint32_t lb_lane = lds0 + NSA * A_STAGE + ixm::big_b_frag_off<NTB>(wn, 0, 0, lane);
+    uint32_t la[2] = {la_lane[0], la_lane[1]};        // A fragment (i, sub) at la[sub] + i * TILE
+    uint32_t lb = lb_lane;                            // B fragment j, slice h at lb + j * TILE + h * 1024
     __builtin_amdgcn_s_waitcnt(0x0F70 | NLD);         // stage 0 of this wavefront has landed (A of stage 1 may not)
     __builtin_amdgcn_s_barrier();                     // a bare barrier: __syncthreads would add a fence on top
-    v4i a[AI][2], b[2][2];                            // [..][slice]
-#pragma unroll
-    for (int i = 0; i < AI; ++i) {
-        a[i][0] = *(const v4i *)(la + i * TILE + a_off[0]);
-        a[i][1] = *(const v4i *)(la + i * TILE + a_off[1]);
-    }
-    b[0][0] = *(const v4i *)(lb);
-    b[0][1] = *(const v4i *)(lb + 1024);
+    // B fragments go through three registers sets: group 0 of a stage multiplies from set 2, group j >= 1 from set
+    // (j - 1) % 2.  Fragment j + 1 is read under the multiplies of group j, and fragment 0 of the next stage is read
+    // into set 2 right behind the barrier that makes that stage visible, ahead of the last group's multiplies, so
+    // no stage begins by waiting for an LDS read it has only just issued.  LDS reads complete in the order they were
+    // issued, so with the two reads of fragment j + 1 the only younger ones, lgkmcnt(2) says fragment j (and, in
+    // group 0, every A fragment) has arrived.
+    v4i a[AI][2], b[3][2];                            // [..][slice]
+    static_for<AI>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        lds_read16<i * TILE>(a[i][0], la[0]);
+        lds_read16<i * TILE>(a[i][1], la[1]);
+    });
+    lds_read16<0>(b[2][0], lb);
+    lds_read16<1024>(b[2][1], lb);
     uint32_t ks = 0;
     do {                                              // k_steps >= 1: the launcher returns early otherwise
         const int buf = ks % NSB;
         const uint32_t ks_b = ks + 1 < last ? ks + 1 : last, ks_a = ks + 2 < last ? ks + 2 : last;
         const int slot_a2 = slot_a == 0 ? 2 : slot_a - 1;             // (slot_a + 2) % 3
-#pragma unroll
-        for (int j = 0; j < WNT; ++j) {
+        static_for<WNT>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
             {
                 // 2 NLD load instructions over the first multiply groups, B before A
                 constexpr int PER = (2 * NLD + WNT - 3) / (WNT - 2);
@@ -422,49 +480,56 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
                     else if (idx < 2 * NLD) issue_a(ks_a, slot_a2, idx - NLD);
                 }
             }
-            const int cur = j % 2;
-            if (j + 1 < WNT) {                        // next fragment under the multiplies
-                b[cur ^ 1][0] = *(const v4i *)(lb + (j + 1) * TILE);
-                b[cur ^ 1][1] = *(const v4i *)(lb + (j + 1) * TILE + 1024);
+            constexpr int cur = j == 0 ? 2 : (j - 1) % 2, nxt = j % 2;   // sets of group j and of group j + 1
+            constexpr bool tail = j + 1 == WNT;
+            if constexpr (!tail) {                    // next fragment under the multiplies
+                lds_read16<(j + 1) * TILE>(b[nxt][0], lb);
+                lds_read16<(j + 1) * TILE + 1024>(b[nxt][1], lb);
+                if constexpr (j == 0) lds_wait_all_a<2>(a, b[cur]);
+                else lds_wait<2>(b[cur][0], b[cur][1]);
             } else {
                 // lgkmcnt(0), vmcnt(NLD): every read of stage ks by this wavefront is complete and its
                 // loads of stage ks + 1 have landed (the A loads of stage ks + 2 may be outstanding)
                 __builtin_amdgcn_s_waitcnt(0x0070 | NLD);
+                lds_wait<0>(b[cur][0], b[cur][1]);    // no instruction: ties the fragment to the wait above
                 __builtin_amdgcn_s_barrier();         // stage ks + 1 visible to all; stage ks no longer read
                 slot_a = slot_a == 2 ? 0 : slot_a + 1;
-                la = lds + slot_a * A_STAGE + (wm * AI) * TILE;
-                lb = lds_b0 + (buf ^ 1) * B_STAGE + ixm::big_b_frag_off<NTB>(wn, 0, 0, lane);
+                la[0] = la_lane[0] + slot_a * A_STAGE;
+                la[1] = la_lane[1] + slot_a * A_STAGE;
+                lb = lb_lane + (buf ^ 1) * B_STAGE;
+                lds_read16<0>(b[2][0], lb);           // fragment 0 of the next stage (set 2 was last used by group 0)
+                lds_read16<1024>(b[2][1], lb);
             }
-            const bool tail = j + 1 == WNT;           // past the last stage the reads fetch stale, unused data
+            // past the last stage the tail's reads fetch stale, unused data
             if constexpr (FP8) {
-#pragma unroll
-                for (int i = 0; i < AI; ++i) {
+                static_for<AI>([&](auto ic) {
+                    constexpr int i = decltype(ic)::value;
                     const v4i &x0 = a[i][0], &x1 = a[i][1], &y0 = b[cur][0], &y1 = b[cur][1];
                     // weight fragment first: the accumulator tile comes out transposed (see the epilogue)
                     mfma_acc(acc[i][j], v8i{y0[0], y0[1], y0[2], y0[3], y1[0], y1[1], y1[2], y1[3]},
                              v8i{x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]});
-                    if (tail) {
-                        a[i][0] = *(const v4i *)(la + i * TILE + a_off[0]);
-                        a[i][1] = *(const v4i *)(la + i * TILE + a_off[1]);
+                    if constexpr (tail) {
+                        lds_read16<i * TILE>(a[i][0], la[0]);
+                        lds_read16<i * TILE>(a[i][1], la[1]);
                     }
-                }
+                });
             } else {
                 // the two k-steps of a tile are eight instructions apart, so no instruction waits for the
                 // accumulator of the one before it
-#pragma unroll
-                for (int h = 0; h < 2; ++h)
-#pragma unroll
-                    for (int i = 0; i < AI; ++i) {
+                static_for<2>([&](auto hc) {
+                    constexpr int h = decltype(hc)::value;
+                    static_for<AI>([&](auto ic) {
+                        constexpr int i = decltype(ic)::value;
                         mfma_acc(acc[i][j], b[cur][h], a[i][h]);
-                        if (tail) a[i][h] = *(const v4i *)(la + i * TILE + a_off[h]);
-                    }
+                        if constexpr (tail) lds_read16<i * TILE>(a[i][h], la[h]);
+                    });
+                });
             }
-            if (tail) {                               // after the multiplies: with an odd WNT they read b[0]
-                b[0][0] = *(const v4i *)(lb);
-                b[0][1] = *(const v4i *)(lb + 1024);
-            }
-        }
+        });
     } while (++ks < k_steps);
+    // the reads the last pass issued for a stage that does not exist are still on their way to registers that are
+    // dead from here on: hold those registers until the reads have written them
+    lds_wait_all_a<0>(a, b[2]);
     // The compiler cannot see that the asm statements are matrix instructions, so it does not insert the
     // wait states their results need before other instructions read the accumulators (it may even peel
     // the last pass and start copying accumulators between its multiplies).  Every accumulator therefore
