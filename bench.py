@@ -620,33 +620,38 @@ def floor_sizes(cfg, att_bytes):
 
 
 # ---------------------------------------------------------------- CPU baseline
-def cpu_baseline(cfg, batch, ctxs, threads):
+def cpu_baseline(fa, be, cfg, batch, ctxs, threads, keep, tables, max_blocks, num_blocks):
     """The CPU oracle (a restatement of the reference's backend-cpu algorithms; the Rust crate cannot be
-    built on this host) on ONE layer plus the lm_head of the same workload, scaled to the full depth."""
+    built on this host) on ONE layer plus the lm_head of the same workload, scaled to the full depth.  The operands
+    are the GPU's own: layer 0's norms, quantized weights (codes and channel scales exported from the device), the
+    embedding, the head, the block tables, and layer 0's K / V pools regenerated from the seeds that filled them."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     import oracle_lib as o
     from decoder_common import Model, oracle_step
-    rng = np.random.default_rng(1)
+    lib = fa.capi.lib
     one = dict(cfg, n_layers=1)
     m = Model()
     m.cfg, m.batch = dict(one), batch
-    tables, max_blocks, num_blocks = make_tables(rng, ctxs, 2, cfg["block_size"])
     m.cfg["max_blocks_per_seq"], m.cfg["num_blocks"], m.tables = max_blocks, num_blocks, tables
-    D, F, V = cfg["d_model"], cfg["d_ffn"], cfg["vocab"]
-    EQ, EKV = cfg["n_heads"] * cfg["head_dim"], cfg["n_kv_heads"] * cfg["head_dim"]
+    V = cfg["vocab"]
+    EKV = cfg["n_kv_heads"] * cfg["head_dim"]
+    # build_decoder keeps, per layer: attn norm, ffn norm, qkv, o, gate|up, down; then embedding, final norm, head
+    n1, n2, wqkv, wo, wgu, wdown = keep[:6]
+    embed, final_norm, lm = keep[-3:]
+    m.embed = be.download(embed)
+    m.final_norm = be.download(final_norm)
+    m.lm = lm.export()
 
-    def qw(k, n):
-        return (rng.integers(-127, 128, size=(k, n), dtype=np.int8), rng.uniform(1e-4, 2e-4, size=n).astype(np.float32))
+    def pool(seed):
+        t = be.alloc_uninit((num_blocks, cfg["block_size"], EKV), fa.capi.BF16)
+        fa.check(lib.fa_fill_normal(be._ctx, t._h, 0, t.numel(), seed, 0.0, 1.0))
+        h = be.download(t)
+        t.free()
+        return h
 
-    def bf16_noise(shape):
-        return (rng.integers(0x3C00, 0x4000, size=shape, dtype=np.uint16) | (rng.integers(0, 2, size=shape, dtype=np.uint16) << 15))
-
-    m.embed = rng.standard_normal((V, D), dtype=np.float32)
-    m.final_norm = np.ones(D, np.float32)
-    m.lm = qw(D, V)
-    m.layers = [dict(attn_norm=np.ones(D, np.float32), ffn_norm=np.ones(D, np.float32), wqkv=qw(D, EQ + 2 * EKV),
-                     wo=qw(EQ, D), wgu=qw(D, 2 * F), wdown=qw(F, D),
-                     k_pool=bf16_noise((num_blocks, 16, EKV)), v_pool=bf16_noise((num_blocks, 16, EKV)))]
+    m.layers = [dict(attn_norm=be.download(n1), ffn_norm=be.download(n2), wqkv=wqkv.export(), wo=wo.export(),
+                     wgu=wgu.export(), wdown=wdown.export(), k_pool=pool(1000 + 7), v_pool=pool(1000 + 8))]
+    rng = np.random.default_rng(1)
     tokens = rng.integers(0, V, size=batch).astype(np.int32)
     oracle_step(m, np.asarray(ctxs, dtype=np.uint32).copy(), tokens, threads=threads)   # warm-up
     times = []
@@ -657,7 +662,7 @@ def cpu_baseline(cfg, batch, ctxs, threads):
         times.append(time.perf_counter() - t0)
     t_one = float(np.median(times))
     # separate the lm_head share: time a zero-layer-equivalent by timing the head alone
-    x = rng.standard_normal((batch, D), dtype=np.float32)
+    x = rng.standard_normal((batch, cfg["d_model"]), dtype=np.float32)
     o.set_threads(threads)
     t0 = time.perf_counter()
     o.linear_w8a8(x, m.lm[0], m.lm[1])
@@ -667,7 +672,8 @@ def cpu_baseline(cfg, batch, ctxs, threads):
     t_full = t_layer * cfg["n_layers"] + t_head
     return dict(value=batch / t_full, unit="tokens/s", cores=threads, kind="port",
                 sample="CPU oracle (C++ restatement of backend-cpu, not the Rust binary): 1 of %d layers + lm_head at "
-                       "batch %d, same contexts, warm-up 1 + median of 3 timed passes, %.2f s per layer measured, scaled "
+                       "batch %d on the GPU's own layer-0 weights, head, tables and K / V contents, same contexts, warm-up 1 + "
+                       "median of 3 timed passes, %.2f s per layer measured, scaled "
                        "to the full depth" % (cfg["n_layers"], batch, t_layer))
 
 
@@ -945,6 +951,10 @@ def main():
         log("continuous batching: %d requests, %d generated tokens in %.2f s -> %.0f generated tokens/s "
             "(mean %.1f active rows)" % (batching["requests"], batching["generated_tokens"], batching["seconds"],
                                          batching["generated_tokens_per_s"], batching["mean_active_rows"]))
+    threads = min(16, os.cpu_count() or 1)
+    cpu_base = None
+    if not a.no_cpu_baseline:                            # before the model's buffers go: the CPU is timed on them
+        cpu_base = cpu_baseline(fa, be, cfg, batch, ctxs, threads, keep, tables, max_blocks, num_blocks)
     lib.fa_decoder_destroy(be._ctx, dec)
     for x in keep:
         x.free()
@@ -995,13 +1005,10 @@ def main():
                    "batch": batch, "sum_ctx": int(sum(mid_ctx)), "graph": bool(use_graph)},
         "roofline": roofline, "extras": extras,
     }
+    out["cpu_baseline"] = cpu_base
     if not a.no_cpu_baseline:
-        threads = min(16, os.cpu_count() or 1)
-        out["cpu_baseline"] = cpu_baseline(cfg, batch, ctxs, threads)
         if not a.no_extras:
             extras["cpu_operator_baselines"] = cpu_operator_baselines(fa, be, threads)
-    else:
-        out["cpu_baseline"] = None
     be.close()
     print(json.dumps(out), flush=True)
 
