@@ -95,6 +95,7 @@ fa_status fa_set_tuning(int32_t key, int32_t value) {
         case 17: k::g_skinny_ksplit_s = value; return FA_OK;
         case 18: k::g_rows_wide = value; return FA_OK;
         case 19: k::g_row_fusion = value; return FA_OK;
+        case 20: k::g_decode_one = value; return FA_OK;
     }
     return fail(FA_ERR_INVALID_ARGUMENT, "fa_set_tuning: unknown key");
 }

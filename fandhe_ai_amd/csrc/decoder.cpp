@@ -116,6 +116,15 @@ void enqueue_pick(fa_decoder *d, hipStream_t s) {
                        d->cfg.vocab, d->strategy == FA_SAMPLE_TOP_K, d->temperature, d->top_k, s);
 }
 
+// Whether the step about to be enqueued (the host lengths already count its token) sees only short contexts: its
+// attention then takes the one-launch form, and the recorded graphs of the two kinds are kept apart.
+bool step_is_short(const fa_decoder *d) {
+    if (k::g_decode_one == 1) return false;
+    uint32_t longest = 0;
+    for (uint32_t b = 0; b < d->batch && b < d->host_lens.size(); ++b) longest = std::max(longest, d->host_lens[b]);
+    return d->batch != 0 && d->batch <= 2 && longest <= k::kDecodeOneMaxCtx;
+}
+
 // The kernels of one step, enqueued on the context's stream.  stop_after (test aid, -1 in normal use) ends the
 // step after the given stage: stage 0 is the per-step bookkeeping and the embedding gather, stage
 // 1 + 8 * layer + i (i = 0 .. 7) is the i-th launch of that layer (norm + quantizer, qkv projection with RoPE
@@ -137,6 +146,7 @@ fa_status enqueue_step(fa_context *ctx, fa_decoder *d, int stop_after = -1) {
     k::gather_rows_f32((const float *)d->embed->ptr, V, D, (const int32_t *)d->tokens->ptr, (float *)d->h->ptr, B, s);
     int stage = 0;
     auto stop_here = [&]() { return stop_after >= 0 && stage++ == stop_after; };
+    const bool short_ctx = step_is_short(d);
     if (stop_here()) return after_launch(ctx, "decoder step (partial)");
 
     k::PagedShape ps;
@@ -196,6 +206,11 @@ fa_status enqueue_step(fa_context *ctx, fa_decoder *d, int stop_after = -1) {
         // (k::RowPrologue): the row stage then launches nothing and its outputs (codes, scales) appear with the
         // linear's stage, written by one block of it.
         const bool fuse_qkv = k::qkv_rope_fuses_norm(B, L.wqkv->k_pad);
+        // One or two short sequences: the attention finishes in one launch (a block per sequence and kv head; no
+        // partial results, no merge launch) and leaves its output and the heads' maxima for the o projection, which
+        // does the per-token quantizer itself.
+        const bool one_attn = short_ctx && c.n_heads <= 32 && F >= EQ && EQ % 64 == 0 &&
+                              k::plain_fuses_pmax_quantizer(B, L.wo->n_pad, L.wo->k_pad, cus);
         if (!fuse_qkv)
             k::rmsnorm_quantize_i8((const float *)d->h->ptr, (const float *)L.attn_norm->ptr, c.rms_eps, nullptr,
                                    (int8_t *)d->xq->ptr, (float *)d->sx->ptr, B, m_pad, D, s,
@@ -209,7 +224,12 @@ fa_status enqueue_step(fa_context *ctx, fa_decoder *d, int stop_after = -1) {
                                            L.wqkv->n_pad, L.wqkv->k_pad, t, s, fuse_qkv ? &pro : nullptr);
         }
         if (stop_here()) break;
-        if (c.n_heads <= 32) {
+        if (one_attn) {
+            k::paged_attention_decode_one_bf16((const uint16_t *)d->q_bf->ptr, (const uint16_t *)L.k_pool->ptr,
+                                               (const uint16_t *)L.v_pool->ptr, (const uint32_t *)d->tables->ptr,
+                                               (const uint32_t *)d->seq_lens->ptr, ps, (float *)d->act->ptr,
+                                               (float *)d->pmax->ptr, s);
+        } else if (c.n_heads <= 32) {
             k::paged_attention_decode_bf16((const uint16_t *)d->q_bf->ptr, (const uint16_t *)L.k_pool->ptr,
                                            (const uint16_t *)L.v_pool->ptr, (const uint32_t *)d->tables->ptr,
                                            (const uint32_t *)d->seq_lens->ptr, ps, (uint32_t)g_decode_waves, ctx->workspace,
@@ -224,7 +244,18 @@ fa_status enqueue_step(fa_context *ctx, fa_decoder *d, int stop_after = -1) {
                                        (float *)d->sx->ptr, B, m_pad, EQ, s);
         }
         if (stop_here()) break;
-        linear(L.wo, d->h->ptr, (const float *)d->h->ptr);
+        if (one_attn) {
+            k::RowPrologue pro;
+            pro.x = (const float *)d->act->ptr;
+            pro.pmax = (const float *)d->pmax->ptr;
+            pro.parts = c.n_heads;
+            pro.xq_tiled_out = (int8_t *)d->xq->ptr;
+            pro.sx_out = (float *)d->sx->ptr;
+            k::linear_w8a8_skinny(nullptr, (const int8_t *)L.wo->codes->ptr, B, L.wo->n, L.wo->n_pad, L.wo->k_pad,
+                                  epilogue(L.wo, d->h->ptr, (const float *)d->h->ptr), cus, s, nullptr, &pro);
+        } else {
+            linear(L.wo, d->h->ptr, (const float *)d->h->ptr);
+        }
         if (stop_here()) break;
         const bool fuse_gu = k::swiglu_fuses_norm(B, L.wgu->n_pad, L.wgu->k_pad, cus);
         if (!fuse_gu)
@@ -661,10 +692,14 @@ fa_status fa_decoder_step(fa_context *ctx, fa_decoder *d, int32_t use_graph) {
         return es;
     }
     if (d->graph_waves != g_decode_waves) drop_graphs(d);
-    auto it = d->graphs.find(d->batch);
+    // a graph per batch size and kind of step (bit 31: the short-context form, decided on the lengths after this step)
+    advance(1);
+    const uint32_t key = d->batch | (step_is_short(d) ? 0x80000000u : 0u);
+    advance(-1);
+    auto it = d->graphs.find(key);
     if (it == d->graphs.end()) {
         try {
-            it = d->graphs.emplace(d->batch, nullptr).first;
+            it = d->graphs.emplace(key, nullptr).first;
         } catch (const std::exception &) {
             return fail(FA_ERR_ALLOCATION_FAILED, "decoder_step: out of host memory");      // lengths not advanced yet
         }

@@ -165,6 +165,9 @@ struct StreamParams {
     // per tpv new tokens.  One launch covers the new tokens [t0, t0 + qt * tpv) of every sequence.
     // Decode: l_new = tpt = tpv = qt = 1, t0 = 0.
     uint32_t l_new, tpt, tpv, qt, t0, n_vseq;
+    // ONE form only (decode_stream_kernel<..., ONE = true>): the finished attention output, f32 values already rounded
+    // to bf16 (the operator's output type), [batch][num_heads][128], and the absmax of every head's slice
+    float *one_out = nullptr, *one_pmax = nullptr;
 };
 
 // Length of (virtual) sequence vs: all cached positions up to the last new token of its tile.  A row whose
@@ -193,59 +196,50 @@ __device__ __forceinline__ uint32_t range_pages(const StreamParams &p, uint32_t 
     return ixm::stream_range_pages(total, p.n_ranges, p.min_pages);
 }
 
-template <int SP, int KD, int VD, int WPE, bool PF, int TT = 1>
+// ONE (decode only): one block per (sequence, kv head) instead of one wavefront per (range, kv head).  The four
+// wavefronts of the block take a quarter of the sequence's pages each, their results meet in LDS, and the first
+// wavefront normalises and stores the finished output (p.one_out, p.one_pmax): no partial results in memory, no
+// merge launch.  For a few short sequences (a compute unit per kv head streams a whole sequence); the arithmetic of
+// the meeting is that of the merge kernels.
+template <int SP, int KD, int VD, int WPE, bool PF, int TT = 1, bool ONE = false>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) decode_stream_kernel(StreamParams p) {
     static_assert(PF || TT == 1, "several token tiles per wavefront exist only in the prefill form");
+    static_assert(!ONE || !PF, "the one-block form is a decode form");
     static_assert(SP % KD == 0 && SP % VD == 0, "static register indices need SP to be a multiple of the depths");
     __shared__ __attribute__((aligned(16))) uint16_t v_s[4][kPage * kVPitch];
+    __shared__ float one_o[ONE ? 4 : 1][ONE ? 64 : 1][ONE ? 33 : 1];       // [wavefront][lane][its 32 dims], padded
+    __shared__ float one_ml[ONE ? 4 : 1][2][16], one_amax[ONE ? 4 : 1][16];
     const int lane = threadIdx.x % 64;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
     const int g = lane / 16, c = lane % 16;
-    const uint32_t item_id = blockIdx.x * 4 + wave;
-    const uint32_t kvh = item_id % p.num_kv_heads, r = item_id / p.num_kv_heads;
-    if (r >= p.n_ranges) return;
+    const uint32_t item_id = ONE ? blockIdx.x : blockIdx.x * 4 + wave;
+    const uint32_t kvh = item_id % p.num_kv_heads, r = item_id / p.num_kv_heads;   // ONE: r is the sequence
+    if (r >= (ONE ? p.batch : p.n_ranges)) return;
     const uint32_t max_ctx = p.max_blocks_per_seq * kPage;
     const uint32_t nv = PF ? p.n_vseq : p.batch;
-    uint32_t total = 0;
-    for (uint32_t b = lane; b < nv; b += 64) total += seq_pages<PF>(p, b, max_ctx);
-    total = __builtin_amdgcn_readfirstlane(wave_sum_dpp<uint32_t>(total));
-    const uint32_t per = range_pages(p, total);
-    const uint64_t rlo64 = (uint64_t)r * per;
-    if (rlo64 >= total) return;
-    const uint32_t rlo = (uint32_t)rlo64, rhi = rlo + per < total ? rlo + per : total;
+    uint32_t rlo = 0, rhi = 0;
+    if constexpr (!ONE) {
+        uint32_t total = 0;
+        for (uint32_t b = lane; b < nv; b += 64) total += seq_pages<PF>(p, b, max_ctx);
+        total = __builtin_amdgcn_readfirstlane(wave_sum_dpp<uint32_t>(total));
+        const uint32_t per = range_pages(p, total);
+        const uint64_t rlo64 = (uint64_t)r * per;
+        if (rlo64 >= total) return;
+        rlo = (uint32_t)rlo64;
+        rhi = rlo + per < total ? rlo + per : total;
+    }
 
     const uint64_t page_elems = (uint64_t)kPage * p.e_kv;
     const uint64_t k_lane = (uint64_t)c * p.e_kv + (uint64_t)kvh * kDh + 8 * g;       // token c, dims 8g..
     const uint64_t v_lane = (uint64_t)(4 * g) * p.e_kv + (uint64_t)kvh * kDh + 8 * c;  // tokens 4g.., dims 8c..
     uint16_t *vs = &v_s[wave][0];
 
-    uint32_t base = 0;
-    for (uint32_t b0 = 0; b0 < nv; b0 += 64) {
-        uint32_t len = b0 + lane < nv ? vseq_len<PF>(p, b0 + lane) : 0;
-        uint32_t len_c = len > max_ctx ? max_ctx : len;
-        uint32_t npg = (len_c + kPage - 1) / kPage;
-        uint32_t incl = npg;
-#pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-            uint32_t up = __shfl_up(incl, off, 64);
-            if (lane >= off) incl += up;
-        }
-        const uint32_t s_b = base + incl - npg, e_b = base + incl;
-        uint64_t mask = __ballot(npg != 0 && s_b < rhi && e_b > rlo);
-        base += __shfl(incl, 63, 64);
-        while (mask != 0) {
-            const int src = __builtin_ctzll(mask);
-            mask &= mask - 1;
-            const uint32_t vq = b0 + src;                                // (virtual) sequence
+    // pages [lo, hi) (hi > lo) of (virtual) sequence vq, whose length is len_b
+    auto segment = [&](const uint32_t vq, const uint32_t lo, const uint32_t hi, const uint32_t len_b) {
             const uint32_t b = PF ? vq / p.qt : vq;
-            const uint32_t sb = __builtin_amdgcn_readfirstlane(__shfl(s_b, src, 64));
-            const uint32_t eb = __builtin_amdgcn_readfirstlane(__shfl(e_b, src, 64));
-            const uint32_t len_b = __builtin_amdgcn_readfirstlane(__shfl(len, src, 64));
             bool bad = len_b > max_ctx;
             if constexpr (PF) bad = p.seq_lens[b] > max_ctx;
             const uint32_t ctx = len_b > max_ctx ? max_ctx : len_b;
-            uint32_t lo, hi;                                           // pages [lo, hi) of the sequence: this segment
-            ixm::stream_segment(rlo, rhi, sb, eb, &lo, &hi);
             const uint32_t n = hi - lo;                                // pages of this segment (>= 1)
             const uint32_t *tab = p.tables + (uint64_t)b * p.max_blocks_per_seq + lo;
 
@@ -464,6 +458,23 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, W
                 win = adv ? win + 64 : win;
             }
             // lane (g, c) holds, for column c: dims 32 bp + 8 g + {0..7} = {o[2bp][0], o[2bp+1][0], o[2bp][1], ...}
+            if constexpr (ONE) {
+                float l = l_run[0];
+                l += __shfl_xor(l, 16, 64);
+                l += __shfl_xor(l, 32, 64);
+#pragma unroll
+                for (int bp = 0; bp < 4; ++bp) {
+                    float *d = &one_o[wave][lane][8 * bp];
+                    d[0] = o[0][2 * bp][0], d[1] = o[0][2 * bp + 1][0], d[2] = o[0][2 * bp][1], d[3] = o[0][2 * bp + 1][1];
+                    d[4] = o[0][2 * bp][2], d[5] = o[0][2 * bp + 1][2], d[6] = o[0][2 * bp][3], d[7] = o[0][2 * bp + 1][3];
+                }
+                if (g == 0) {
+                    const float nanv = __uint_as_float(0x7fc00000u);
+                    one_ml[wave][0][c] = bad ? nanv : m_run[0];
+                    one_ml[wave][1][c] = bad ? nanv : l;
+                }
+                return;
+            }
             const uint64_t item = (uint64_t)(r + vq) * p.num_kv_heads + kvh;
 #pragma unroll
             for (int tt = 0; tt < TT; ++tt) {
@@ -483,6 +494,85 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, W
                         p.part_ml[(item * TT + tt) * (2 * p.g_pad) + p.g_pad + c] = bad ? nanv : l;
                     }
                 }
+            }
+    };
+    if constexpr (ONE) {
+        const uint32_t len_b = p.seq_lens[r];
+        const uint32_t len_c = len_b > max_ctx ? max_ctx : len_b;
+        const uint32_t npg = (len_c + kPage - 1) / kPage;
+        const uint32_t lo = (uint32_t)((uint64_t)npg * (uint32_t)wave / 4), hi = (uint32_t)((uint64_t)npg * ((uint32_t)wave + 1) / 4);
+        if (hi > lo) {
+            segment(r, lo, hi, len_b);
+        } else {                                                       // no pages for this wavefront: weight zero
+#pragma unroll
+            for (int j = 0; j < 32; ++j) one_o[wave][lane][j] = 0.0f;
+            if (g == 0) {
+                one_ml[wave][0][c] = -INFINITY;
+                one_ml[wave][1][c] = 0.0f;
+            }
+        }
+        __syncthreads();
+        // the meeting, as decode_stream_merge_quantize_kernel does it: maximum (NaN marks a violation), weights,
+        // weighted sums in wavefront order, one division, one rounding to bf16; wavefront w finishes dims
+        // 32 w + 8 g .. + 7 of every column
+        float mx = -INFINITY, den = 0.0f, acc[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const float m = one_ml[w][0][c];
+            mx = (m != m || mx != mx) ? __uint_as_float(0x7fc00000u) : fmaxf(mx, m);
+        }
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const float wt = expf(one_ml[w][0][c] - mx);
+            den = __builtin_fmaf(wt, one_ml[w][1][c], den);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(wt, one_o[w][lane][8 * wave + e], acc[e]);
+        }
+        float amax = 0.0f, v[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float res = npg == 0 ? 0.0f : __fdiv_rn(acc[e], den);
+            v[e] = bf16_to_f32(f32_to_bf16(res));
+            amax = fmaxf(amax, fabsf(v[e]));
+        }
+        if ((uint32_t)c < p.group) {
+            float *dst = p.one_out + ((uint64_t)r * p.num_heads + (uint64_t)kvh * p.group + c) * kDh + 32 * wave + 8 * g;
+            *(v4f *)dst = v4f{v[0], v[1], v[2], v[3]};
+            *(v4f *)(dst + 4) = v4f{v[4], v[5], v[6], v[7]};
+        }
+        amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+        amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+        if (g == 0) one_amax[wave][c] = amax;
+        __syncthreads();
+        if (wave == 0 && g == 0 && (uint32_t)c < p.group)
+            p.one_pmax[(uint64_t)r * p.num_heads + (uint64_t)kvh * p.group + c] =
+                fmaxf(fmaxf(one_amax[0][c], one_amax[1][c]), fmaxf(one_amax[2][c], one_amax[3][c]));
+    } else {
+        uint32_t base = 0;
+        for (uint32_t b0 = 0; b0 < nv; b0 += 64) {
+            uint32_t len = b0 + lane < nv ? vseq_len<PF>(p, b0 + lane) : 0;
+            uint32_t len_c = len > max_ctx ? max_ctx : len;
+            uint32_t npg = (len_c + kPage - 1) / kPage;
+            uint32_t incl = npg;
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                uint32_t up = __shfl_up(incl, off, 64);
+                if (lane >= off) incl += up;
+            }
+            const uint32_t s_b = base + incl - npg, e_b = base + incl;
+            uint64_t mask = __ballot(npg != 0 && s_b < rhi && e_b > rlo);
+            base += __shfl(incl, 63, 64);
+            while (mask != 0) {
+                const int src = __builtin_ctzll(mask);
+                mask &= mask - 1;
+                const uint32_t sb = __builtin_amdgcn_readfirstlane(__shfl(s_b, src, 64));
+                const uint32_t eb = __builtin_amdgcn_readfirstlane(__shfl(e_b, src, 64));
+                const uint32_t len_b = __builtin_amdgcn_readfirstlane(__shfl(len, src, 64));
+                uint32_t lo, hi;                                       // pages [lo, hi) of the sequence: this segment
+                ixm::stream_segment(rlo, rhi, sb, eb, &lo, &hi);
+                segment(b0 + src, lo, hi, len_b);
             }
         }
     }
@@ -1333,6 +1423,41 @@ void paged_attention_decode_bf16(const uint16_t *q, const uint16_t *k_pool, cons
     }
     dim3 grid2(ps.num_heads, ps.batch);
     decode_stream_merge_kernel<<<grid2, 256, 0, s>>>(sp, out, out_bf16, pmax);
+}
+
+// Decode attention of a few short sequences with the finished output in one launch (decode_stream_kernel's ONE
+// form): out_f32 [batch][num_heads][128] holds the output values rounded to bf16, pmax [batch][num_heads] the absmax
+// of every head's slice, which is what a per-token quantizer in front of the next projection needs.  A compute unit
+// per (sequence, kv head) streams the whole sequence, so this is for contexts of at most kDecodeOneMaxCtx tokens;
+// longer ones go through paged_attention_decode_bf16.
+int g_decode_one = 0;
+void paged_attention_decode_one_bf16(const uint16_t *q, const uint16_t *k_pool, const uint16_t *v_pool, const uint32_t *tables,
+                                     const uint32_t *seq_lens, const PagedShape &ps, float *out_f32, float *pmax, hipStream_t s) {
+    if (ps.batch == 0) return;
+    StreamParams sp;
+    sp.q = q;
+    sp.k_pool = k_pool;
+    sp.v_pool = v_pool;
+    sp.tables = tables;
+    sp.seq_lens = seq_lens;
+    sp.part_o = sp.part_ml = nullptr;
+    sp.num_blocks = ps.num_blocks;
+    sp.e_kv = ps.e_kv;
+    sp.batch = ps.batch;
+    sp.num_heads = ps.num_heads;
+    sp.num_kv_heads = ps.num_kv_heads;
+    sp.group = ps.num_heads / ps.num_kv_heads;
+    sp.g_pad = (uint32_t)group_pad(sp.group);
+    sp.max_blocks_per_seq = ps.max_blocks_per_seq;
+    sp.n_ranges = ps.batch;
+    sp.min_pages = 1;
+    sp.scale = ps.scale;
+    sp.l_new = sp.tpt = sp.tpv = sp.qt = 1;
+    sp.t0 = 0;
+    sp.n_vseq = ps.batch;
+    sp.one_out = out_f32;
+    sp.one_pmax = pmax;
+    decode_stream_kernel<4, 4, 2, 2, false, 1, true><<<ps.batch * ps.num_kv_heads, 256, 0, s>>>(sp);
 }
 
 // Prefill (l_new > 1) on the same streaming kernel: groups of kPrefillTT token tiles of 16 / group new tokens

@@ -260,6 +260,15 @@ void paged_attention_decode_bf16(const uint16_t *q, const uint16_t *k_pool, cons
                                  int8_t *xq_tiled, float *sx, uint32_t m_pad, hipStream_t s,
                                  const WeightPrefetch &pull = WeightPrefetch{});
 
+// Decode attention of a few short sequences, finished in one launch (a block per (sequence, kv head), no partial
+// results, no merge): out_f32 [batch][num_heads][128] = the output values rounded to bf16 (the operator's output
+// type), pmax [batch][num_heads] = absmax of every head's slice, for a per-token quantizer inside the projection that
+// follows (RowPrologue).  Same shapes as the fast path above; meant for contexts up to kDecodeOneMaxCtx tokens.
+constexpr uint32_t kDecodeOneMaxCtx = 1024;
+extern int g_decode_one;      // 0: by shape and context, 1: never (tuning aid)
+void paged_attention_decode_one_bf16(const uint16_t *q, const uint16_t *k_pool, const uint16_t *v_pool, const uint32_t *tables,
+                                     const uint32_t *seq_lens, const PagedShape &ps, float *out_f32, float *pmax, hipStream_t s);
+
 // Prefill fast path: bf16, head_dim 128, block_size 16, l_new > 1, group <= 16.  Causal over the cached
 // positions: new token t of a row sees positions below seq_len - l_new + t + 1.
 uint64_t paged_prefill_workspace_bytes(const PagedShape &ps, uint32_t waves_per_cu);

@@ -86,7 +86,10 @@ fa_status fa_probe_l2_path(fa_context *ctx, const fa_buffer *cold, uint64_t cold
  *        instead of the up-to-1024-thread form used for at most 256 rows;
  * key 19: 1 keeps the norm + quantizer and quantizer kernels of a decode step as launches of their own for every batch
  *        size; 0: for at most four rows the linears that follow do that row work themselves (takes effect when a step
- *        is recorded). */
+ *        is recorded);
+ * key 20: 1 keeps the streamed attention with its merge launch for every decode step; 0: a step of one or two
+ *        sequences whose contexts are at most 1024 tokens runs the attention as one launch (a block per sequence
+ *        and kv head) and lets the o projection do the quantizer (takes effect when a step is recorded). */
 fa_status fa_set_tuning(int32_t key, int32_t value);
 
 /* What the context found when it was created: xcd_local = 1 when workgroups b and b + 8 of a launch were seen to

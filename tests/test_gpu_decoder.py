@@ -106,6 +106,9 @@ def test_small_batches_do_the_row_work_inside_the_linears(shape, batch):
         fa.check(lib.fa_set_tuning(5, 2))                 # narrow test model: force the kernel gate / up uses at full width
     outs, stages = {}, {}
     try:
+        # (the attention keeps its usual form in both runs: how a sequence's pages are divided among wavefronts decides
+        # the last bits of its output, and the one-launch form for short contexts divides them its own way)
+        fa.check(lib.fa_set_tuning(20, 1))
         for fused in (True, False):
             fa.check(lib.fa_set_tuning(19, 0 if fused else 1))
             dec = GpuDecoder(be, m)
@@ -147,8 +150,9 @@ def test_small_batches_do_the_row_work_inside_the_linears(shape, batch):
             assert np.array_equal(a[1], b[1])
             for (ak, av), (bk, bv) in zip(a[2], b[2]):
                 assert np.array_equal(ak, bk) and np.array_equal(av, bv)
-        # against the oracle, with the fused path
+        # against the oracle, with the fused path (and, for one and two rows, the one-launch attention)
         fa.check(lib.fa_set_tuning(19, 0))
+        fa.check(lib.fa_set_tuning(20, 0))
         dec = GpuDecoder(be, m)
         try:
             lens, tokens = m.seq_lens.copy(), m.tokens.copy()
@@ -159,12 +163,63 @@ def test_small_batches_do_the_row_work_inside_the_linears(shape, batch):
             dec.close()
     finally:
         fa.check(lib.fa_set_tuning(19, 0))
+        fa.check(lib.fa_set_tuning(20, 0))
         fa.check(lib.fa_set_tuning(5, 0))
+
+
+@pytest.mark.parametrize("ctxs", [[1], [16], [17, 3], [130, 64], [1000, 1], [1023, 777]], ids=lambda c: "ctx" + "_".join(map(str, c)))
+def test_short_contexts_finish_the_attention_in_one_launch(ctxs):
+    """One or two sequences of at most 1024 tokens: the attention runs as one launch (a block per sequence and kv
+    head whose four wavefronts share the pages) and the o projection does the per-token quantizer.  What the o
+    projection publishes (codes and scales of the attention output, stage 4 of the first layer) must be what the
+    streamed attention + merge + quantizer leave (tuning key 20 = 1) up to the last bits of the attention output: equal
+    scales to 1e-6 relative and codes at most one step apart, nearly all equal.  The steps meet the oracle, eager
+    and replayed, also when a context grows past the limit and the step changes form (1023 -> 1026)."""
+    import ctypes as C
+    import fandhe_ai_amd as fa
+    be = ops()
+    lib = fa.capi.lib
+    batch = len(ctxs)
+    shape = dict(n_layers=2, d_model=2048, n_heads=16, n_kv_heads=4, d_ffn=3072, vocab=3000)
+    m = build_model(seed=40 + sum(ctxs), steps=5, batch=batch, ctxs=ctxs, **shape)
+    got = {}
+    try:
+        for one in (True, False):
+            fa.check(lib.fa_set_tuning(20, 0 if one else 1))
+            dec = GpuDecoder(be, m)
+            try:
+                dec.set_state(m.seq_lens, m.tokens)
+                fa.check(lib.fa_decoder_debug_step_until(be._ctx, dec.h, 4))
+                xq, sx = C.c_void_p(), C.c_void_p()
+                fa.check(lib.fa_decoder_debug_buffer(dec.h, 1, C.byref(xq)))
+                fa.check(lib.fa_decoder_debug_buffer(dec.h, 2, C.byref(sx)))
+                codes = np.empty(16 * shape["d_model"], np.int8)
+                scales = np.empty(batch, np.float32)
+                fa.check(lib.fa_download(be._ctx, xq, 0, codes.ctypes.data, codes.size))
+                fa.check(lib.fa_download(be._ctx, sx, 0, scales.ctypes.data, batch))
+                got[one] = (codes.astype(np.int32), scales)
+            finally:
+                dec.close()
+        (ca, sa), (cb, sb) = got[True], got[False]
+        assert np.all(sb > 0) and np.allclose(sa, sb, rtol=1e-6, atol=0)
+        assert np.abs(ca - cb).max() <= 1 and (ca != cb).mean() < 2e-3 and np.any(ca != 0)
+        fa.check(lib.fa_set_tuning(20, 0))
+        dec = GpuDecoder(be, m)
+        try:
+            lens, tokens = m.seq_lens.copy(), m.tokens.copy()
+            for step in range(4):
+                tokens = _check_small(m, dec, lens, tokens, step > 0, "one-launch attention:%s:step%d" % (ctxs, step))
+                dec.set_state(lens, tokens)
+        finally:
+            dec.close()
+    finally:
+        fa.check(lib.fa_set_tuning(20, 0))
 
 
 def _check_small(m, dec, lens, tokens, use_graph, tag):
     """_check_step with the bar for a handful of rows: a flipped code is not diluted by other rows, so every row is
-    held to mean < 4e-3 of its logit range and the median row to 2e-4."""
+    held to mean < 4e-3 of its logit range and, with three rows or more, the median row to 2e-4 (with one or two rows
+    a single flipped code is the median)."""
     want_next, want_logits = oracle_step(m, lens, tokens)
     dec.step(use_graph)
     got_logits, got_next = dec.logits(), dec.tokens()
@@ -172,7 +227,7 @@ def _check_small(m, dec, lens, tokens, use_graph, tag):
     err = np.abs(got_logits - want_logits) / spread
     rows = err.mean(axis=1)
     print("DECODE_STEP_PARITY\t%s\tmax_err/range=%.3e\trow means=%s" % (tag, err.max(), np.array2string(rows, precision=2)), flush=True)
-    assert rows.max() < 4e-3 and np.median(rows) < 2e-4 and err.max() < 2e-2
+    assert rows.max() < 4e-3 and (len(rows) < 3 or np.median(rows) < 2e-4) and err.max() < 2e-2
     top2 = np.sort(want_logits, axis=1)[:, -2:]
     decisive = (top2[:, 1] - top2[:, 0]) > 4e-2 * spread[:, 0]
     assert np.array_equal(got_next[decisive], want_next[decisive])
