@@ -32,7 +32,7 @@ MFMA_PEAK_TOPS = 5000.0          # dense int8 and fp8 on MI355X
 # HBM bytes per launch of decode_stream_kernel at this benchmark's shape, from hardware counters
 # (rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE, each scaled by the same counter's reading for a plain
 # row-copy kernel of known size; the figures are in profiles/decode_stream_kernel_config5_pmc.txt).
-ATTENTION_TRAFFIC_BYTES = 635879260
+ATTENTION_TRAFFIC_BYTES = 635875453
 U32MAX = 0xFFFFFFFF
 SERVING_ROWS = 64          # rows of the continuous-batching run (the decoder's limit)
 
@@ -812,7 +812,7 @@ def main():
                     help="with --only decode-linears: one of the four layer shapes (0 .. 3) instead of all, so that "
                          "a counter run sees launches of one shape only")
     ap.add_argument("--only", choices=("attention", "copy", "linears", "decode-linears", "prefill", "prefill-attention", "mfma",
-                                       "prompt", "stream-floor", "gemm-f32", "l2-path"), default=None,
+                                       "prompt", "stream-floor", "gemm-f32", "l2-path", "single-stream"), default=None,
                     help="profiling aid: run only the dominant kernel at the workload's shape, or a plain "
                          "copy kernel of known size (counter calibration), a few launches, no JSON line")
     a = ap.parse_args()
@@ -848,6 +848,14 @@ def main():
             for r in bench_short_prompts(fa, be, dec, cfg, tables):
                 log("one prompt of %d tokens%s through %d layers: %.2f ms, %.0f tokens/s" %
                     (r["l_new"], " after %d cached" % r["cached"] if r["cached"] else "", cfg["n_layers"], r["ms"], r["tokens_per_s"]))
+            lib.fa_decoder_destroy(be._ctx, dec)
+            be.close()
+            return
+        if a.only == "single-stream":
+            dec, keep, tables, _, _ = build_decoder(fa, be, cfg, batch, ctxs, 300, max_batch=batch)
+            r = bench_single_stream(fa, be, dec, cfg, tables)
+            log("one sequence decoding alone through %d layers: %.3f ms per token; verifying 5 positions in one step: %.3f ms" %
+                (cfg["n_layers"], r["ms_per_token"], r["verify_5_positions_ms"]))
             lib.fa_decoder_destroy(be._ctx, dec)
             be.close()
             return
