@@ -546,30 +546,43 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
     int row_l0, col_l0;                               // block-local row of this lane in row tile 0, first column in tile 0
     ixm::big_out_elem<NTB, WM>(wm, wn, 0, 0, 0, lane, &row_l0, &col_l0);
     const int g = lane / 16;
-    bool extras = false;
+    bool extras = false, raw_out = false;
     const bool out_bf16 = ep.out_bf16 != 0;
     bool f8_rows = false;
+    const float *bias = nullptr, *residual = nullptr;
     if constexpr (FP8) {
         f8_rows = ep.sx != nullptr;
         extras = f8_rows && ep.bias != nullptr;
+        if (extras) bias = ep.bias;
     } else {
         extras = ep.acc_out != nullptr || ep.bias != nullptr || ep.residual != nullptr;
+        raw_out = ep.acc_out != nullptr;
+        bias = ep.bias;
+        residual = ep.residual;
     }
     const uint32_t col0 = (nt0 + wn * WNT) * 16;      // first column of this wavefront
     const bool full_cols = nt0 + wn * WNT + WNT <= n_tiles && col0 + WNT * 16 <= n;
     const bool row_scales = !FP8 || f8_rows;
-    if (!extras && full_cols && n % 8 == 0) {
-        v4f swc[WNT];
-        if (row_scales) {
+    if (!raw_out && full_cols && n % 8 == 0) {
+        // bias and residual are added in the order of the general form below: (product + bias), then residual + that
+        v4f swc[WNT], bc[WNT];
 #pragma unroll
-            for (int j = 0; j < WNT; ++j) swc[j] = *(const v4f *)(ep.sw + col0 + j * 16 + 4 * g);
+        for (int j = 0; j < WNT; ++j) {
+            if (row_scales) swc[j] = *(const v4f *)(ep.sw + col0 + j * 16 + 4 * g);
+            if (bias) bc[j] = *(const v4f *)(bias + col0 + j * 16 + 4 * g);
         }
 #pragma unroll
         for (int i = 0; i < AI; ++i) {
             const uint32_t row = m0 + row_l0 + i * 16;
             const bool row_ok = row < m;
             const float sxr = row_scales ? ep.sx[row_ok ? row : m - 1] : 0.0f;
-            uint8_t *orow = (uint8_t *)ep.out + ((uint64_t)(row_ok ? row : m - 1) * n + nt0 * 16 + col_l0) * (out_bf16 ? 2 : 4);
+            const uint64_t o0 = (uint64_t)(row_ok ? row : m - 1) * n + nt0 * 16 + col_l0;
+            uint8_t *orow = (uint8_t *)ep.out + o0 * (out_bf16 ? 2 : 4);
+            v4f res[WNT];
+            if (residual) {
+#pragma unroll
+                for (int j = 0; j < WNT; ++j) res[j] = *(const v4f *)(residual + o0 + j * 16);
+            }
 #pragma unroll
             for (int j = 0; j < WNT; ++j) {
                 float v[4];
@@ -577,6 +590,8 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
                 for (int e = 0; e < 4; ++e) {
                     if constexpr (FP8) v[e] = __fmul_rn(acc[i][j][e], f8_rows ? __fmul_rn(sxr, swc[j][e]) : fscale);
                     else v[e] = __fmul_rn((float)acc[i][j][e], __fmul_rn(sxr, swc[j][e]));
+                    if (bias) v[e] = __fadd_rn(v[e], bc[j][e]);
+                    if (residual) v[e] = __fadd_rn(res[j][e], v[e]);
                 }
                 if (!row_ok) continue;
                 if (out_bf16)

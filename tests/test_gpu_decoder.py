@@ -321,6 +321,39 @@ def test_prompt_prefill_matches_the_oracle_decoding_the_prompt_token_by_token(sh
         dec.close()
 
 
+def test_prompt_pass_on_large_tiles_equals_the_pass_on_128_tiles_bit_for_bit():
+    """The projections of a prompt pass on the large-tile GEMM (forced: 256 x 224 tiles; its epilogue adds the
+    residual of the o and down projections from registers, four outputs of a row per lane) against the same pass on
+    the 128 x 128 kernel (its own epilogue code): int32 sums are exact and both epilogues apply scale, then
+    residual, in the same order, so logits, tokens and every cache row must be identical."""
+    import fandhe_ai_amd as fa
+    be = ops()
+    lib = fa.capi.lib
+    shape = dict(n_layers=2, d_model=512, n_heads=4, n_kv_heads=2, d_ffn=1024, vocab=700, batch=3, ctxs=[0, 9, 40])
+    l_new = 100                                           # 300 rows: two row blocks of 256, the second ragged
+    m = build_model(seed=77, steps=l_new + 2, **shape)
+    prompt = o.Rng(6).randint(0, shape["vocab"], shape["batch"] * l_new).astype(np.int32).reshape(shape["batch"], l_new)
+    got = {}
+    try:
+        for big in (True, False):
+            fa.check(lib.fa_set_tuning(7, 14 if big else 0))
+            fa.check(lib.fa_set_tuning(4, 0 if big else 1))
+            dec = GpuDecoder(be, m)
+            try:
+                dec.prefill(prompt)
+                got[big] = (dec.logits().copy(), dec.tokens().copy(), [tuple(x.copy() for x in dec.kv_pool(li)) for li in range(2)])
+            finally:
+                dec.close()
+    finally:
+        fa.check(lib.fa_set_tuning(7, 0))
+        fa.check(lib.fa_set_tuning(4, 0))
+    a, b = got[True], got[False]
+    assert np.all(np.isfinite(a[0])) and np.any(a[0] != 0)
+    assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1])
+    for (ak, av), (bk, bv) in zip(a[2], b[2]):
+        assert np.array_equal(ak, bk) and np.array_equal(av, bv)
+
+
 @pytest.mark.parametrize("shape", [
     dict(n_layers=2, d_model=256, n_heads=4, n_kv_heads=2, d_ffn=512, vocab=1000, batch=3, ctxs=[0, 5, 40], l_new=6),
     dict(n_layers=1, d_model=256, n_heads=2, n_kv_heads=1, d_ffn=256, vocab=300, batch=1, ctxs=[21], l_new=40),

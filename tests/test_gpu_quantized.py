@@ -579,6 +579,32 @@ def test_fp8_large_tile_kernel_ragged_shape():
     assert np.array_equal(small, got)
 
 
+@pytest.mark.parametrize("n", [9008, 9004], ids=["whole-tiles", "ragged-columns"])
+def test_int8_large_tile_kernel_bias_without_raw_sums(n):
+    """fa_linear_w8a8 on 1000 rows (quantizer + large-tile GEMM) with a bias and no raw-accumulator output: with a
+    column count that is a multiple of 8 the epilogue adds the bias from registers and stores four outputs of a row
+    per lane; otherwise it takes the general element-by-element form.  Both bit-exact against the oracle, f32 and
+    bf16 outputs."""
+    fa = _fa()
+    be = ops()
+    m, k = 1000, 1024
+    rng = o.Rng(47 + n)
+    x = rng.randn((m, k))
+    w = rng.randn((k, n), std=0.05)
+    bias = rng.randn((n,))
+    o.set_threads(8)
+    wq, ws = o.quantize_cols_i8(w)
+    _, want = o.linear_w8a8(x, wq, ws, bias)
+    o.set_threads(1)
+    qw = be.import_quantized_weight(wq, ws)
+    assert _gemm_plan(fa, be, m, qw).big_ntb in (14, 16)
+    dbias = fa.DeviceBufferView(be.upload(bias), 0, (n,))
+    got = be.download_owned(be.linear_w8a8(be.upload(x), qw, bias=dbias))
+    assert np.array_equal(got, want)
+    out_bf = be.download_owned(be.linear_w8a8(be.upload(x), qw, bias=dbias, out_dtype=fa.capi.BF16))
+    assert_bf16_rounding_of("w8a8 large tile bias bf16", out_bf, got)
+
+
 def test_int8_large_tile_kernel_wavefront_variants_are_bit_exact():
     """The 4- and 16-wavefront variants and both tile widths of the large-tile int8 kernel against the oracle
     on sampled rows of a ragged shape (exact integers: any difference is an indexing error)."""
