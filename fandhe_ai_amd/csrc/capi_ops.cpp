@@ -14,6 +14,7 @@ namespace fa {
 namespace k {
 extern int g_gemm_f32_form, g_weight_prefetch, g_probe_plain_loads, g_rows_wide;
 extern int g_skinny_ksplit, g_skinny_ksplit_s, g_row_fusion;
+extern int g_rows_kernel;
 extern int g_skinny_ntw, g_skinny_waves, g_skinny_astat, g_gemm_small_tiles, g_gemm_waves, g_gemm_ntb, g_gemm_split_fill;
 }
 int g_decode_waves = 0;
@@ -96,6 +97,7 @@ fa_status fa_set_tuning(int32_t key, int32_t value) {
         case 18: k::g_rows_wide = value; return FA_OK;
         case 19: k::g_row_fusion = value; return FA_OK;
         case 20: k::g_decode_one = value; return FA_OK;
+        case 21: k::g_rows_kernel = value; return FA_OK;
     }
     return fail(FA_ERR_INVALID_ARGUMENT, "fa_set_tuning: unknown key");
 }
@@ -340,6 +342,13 @@ fa_status fa_linear_w8a8(fa_context *ctx, const fa_buffer *x, uint64_t m, const 
                             qw->k_pad, ctx->stream);
         k::linear_w8a8_skinny((const int8_t *)xq.ptr, (const int8_t *)qw->codes->ptr, m, qw->n, qw->n_pad, qw->k_pad,
                               ep, ctx->props.multiProcessorCount, ctx->stream, &ctx->splitk);
+    } else if (qw->k == qw->k_pad && k::linear_w8a8_rows_applies(m, qw->n_pad, qw->k_pad, ctx->props.multiProcessorCount)) {
+        uint64_t m_pad = round_up(m, 16);
+        if (fa_status s = xq.get(m_pad * qw->k_pad)) return s;
+        k::quantize_rows_i8(x->ptr, x->dtype == FA_BF16, nullptr, (int8_t *)xq.ptr, (float *)sx.ptr, m, m_pad, qw->k,
+                            qw->k_pad, ctx->stream);
+        k::linear_w8a8_rows((const int8_t *)xq.ptr, (const int8_t *)qw->codes->ptr, m, qw->n, qw->n_pad, qw->k_pad, ep,
+                            ctx->props.multiProcessorCount, ctx->stream);
     } else {
         if (qw->k != qw->k_pad) return fail(FA_ERR_UNSUPPORTED, "linear_w8a8: m > 64 needs k to be a multiple of 64");
         if (fa_status s = xq.get(mk)) return s;

@@ -363,6 +363,13 @@ fa_status enqueue_prefill_chunk(fa_context *ctx, fa_decoder *d, PrefillBuffers &
     ps.scale = 1.0f / std::sqrt((float)c.head_dim);
     for (uint32_t b = 0; b < B; ++b) ps.ctx_hint = std::max(ps.ctx_hint, d->host_lens[b] + lc);
 
+    // A pass of 65 to a few hundred rows runs its narrow projections on the weight-stationary kernel, which takes
+    // activation tiles (the decode kernels' layout) instead of row-major codes: the quantizer in front of such a
+    // projection writes that layout.
+    const uint64_t M_pad = round_up(M, 16);
+    // (at most 64 rows: every projection on the decode kernels, which take the same layout)
+    const bool decode_form = M <= 64 && k::g_rows_kernel != 1;
+    auto rows_form = [&](const fa_qweight *w) { return decode_form || k::linear_w8a8_rows_applies(M, w->n_pad, w->k_pad, cus); };
     // y = dequant(xq @ w) (+ residual) for the rows quantized into t.xq / t.sx just before
     auto gemm = [&](const fa_qweight *w, float *out, const float *residual) {
         k::EpilogueI8 ep;
@@ -373,14 +380,25 @@ fa_status enqueue_prefill_chunk(fa_context *ctx, fa_decoder *d, PrefillBuffers &
         ep.acc_out = nullptr;
         ep.out = out;
         ep.out_bf16 = 0;
-        k::gemm_w8a8_mfma(t.xq.as<int8_t>(), (const int8_t *)w->codes->ptr, M, w->n, w->n_pad, w->k_pad, ep, cus, s,
-                          t.splitk.ptr, t.splitk.bytes);
+        if (decode_form)
+            k::linear_w8a8_skinny(t.xq.as<int8_t>(), (const int8_t *)w->codes->ptr, M, w->n, w->n_pad, w->k_pad, ep, cus, s,
+                                  &ctx->splitk);
+        else if (rows_form(w))
+            k::linear_w8a8_rows(t.xq.as<int8_t>(), (const int8_t *)w->codes->ptr, M, w->n, w->n_pad, w->k_pad, ep, cus, s);
+        else
+            k::gemm_w8a8_mfma(t.xq.as<int8_t>(), (const int8_t *)w->codes->ptr, M, w->n, w->n_pad, w->k_pad, ep, cus, s,
+                              t.splitk.ptr, t.splitk.bytes);
+    };
+    auto norm_quantize = [&](const float *norm_w, const fa_qweight *w) {
+        if (rows_form(w))
+            k::rmsnorm_quantize_i8(t.h.as<float>(), norm_w, c.rms_eps, nullptr, t.xq.as<int8_t>(), t.sx.as<float>(), M, M_pad, D, s);
+        else
+            k::rmsnorm_quantize_rows_i8(t.h.as<float>(), norm_w, c.rms_eps, t.xq.as<int8_t>(), t.sx.as<float>(), M, D, s);
     };
 
     for (uint32_t li = 0; li < c.n_layers; ++li) {
         const fa_decoder::Layer &L = d->layers[li];
-        k::rmsnorm_quantize_rows_i8(t.h.as<float>(), (const float *)L.attn_norm->ptr, c.rms_eps, t.xq.as<int8_t>(),
-                                    t.sx.as<float>(), M, D, s);
+        norm_quantize((const float *)L.attn_norm->ptr, L.wqkv);
         gemm(L.wqkv, t.qkv.as<float>(), nullptr);
         k::rope_append(t.qkv.as<float>(), t.cos_sin.as<float>(), t.slots.as<uint32_t>(), t.q_bf.as<uint16_t>(),
                        (uint16_t *)L.k_pool->ptr, (uint16_t *)L.v_pool->ptr, M, c.n_heads, c.n_kv_heads, c.head_dim,
@@ -389,19 +407,20 @@ fa_status enqueue_prefill_chunk(fa_context *ctx, fa_decoder *d, PrefillBuffers &
                                         (const uint16_t *)L.v_pool->ptr, (const uint32_t *)d->tables->ptr,
                                         (const uint32_t *)d->seq_lens->ptr, ps, (uint32_t)g_decode_waves, ctx->workspace,
                                         t.attn.ptr, 1, s);
-        k::quantize_rows_i8(t.attn.ptr, true, t.xq.as<int8_t>(), nullptr, t.sx.as<float>(), M, M, L.wo->k, L.wo->k_pad, s);
+        if (rows_form(L.wo))
+            k::quantize_rows_i8(t.attn.ptr, true, nullptr, t.xq.as<int8_t>(), t.sx.as<float>(), M, M_pad, L.wo->k, L.wo->k_pad, s);
+        else
+            k::quantize_rows_i8(t.attn.ptr, true, t.xq.as<int8_t>(), nullptr, t.sx.as<float>(), M, M, L.wo->k, L.wo->k_pad, s);
         gemm(L.wo, t.h.as<float>(), t.h.as<float>());
-        k::rmsnorm_quantize_rows_i8(t.h.as<float>(), (const float *)L.ffn_norm->ptr, c.rms_eps, t.xq.as<int8_t>(),
-                                    t.sx.as<float>(), M, D, s);
+        norm_quantize((const float *)L.ffn_norm->ptr, L.wgu);
         gemm(L.wgu, t.gu.as<float>(), nullptr);
-        k::swiglu_quantize_rows_i8(t.gu.as<float>(), t.xq.as<int8_t>(), t.sx.as<float>(), M, F, s);
+        k::swiglu_quantize_rows_i8(t.gu.as<float>(), t.xq.as<int8_t>(), t.sx.as<float>(), M, F, s, rows_form(L.wdown));
         gemm(L.wdown, t.h.as<float>(), t.h.as<float>());
     }
     if (padded) k::trim_seq_lens((uint32_t *)d->seq_lens->ptr, t.row_lens.as<uint32_t>(), B, lc, s);
     if (every_row) {
         // verification: the head over every row of the chunk (row b * lc + t is token t of sequence b)
-        k::rmsnorm_quantize_rows_i8(t.h.as<float>(), (const float *)d->final_norm->ptr, c.rms_eps, t.xq.as<int8_t>(),
-                                    t.sx.as<float>(), M, D, s);
+        norm_quantize((const float *)d->final_norm->ptr, d->lm_head);
         gemm(d->lm_head, t.all_logits.as<float>(), nullptr);
         k::argmax_rows_f32(t.all_logits.as<float>(), t.all_picked.as<int32_t>(), M, V, s);
     }
@@ -778,7 +797,7 @@ static fa_status prefill_impl(fa_context *ctx, fa_decoder *d, const int32_t *tok
     };
     get(t.tok, M * 4);
     get(t.h, M * D * 4);
-    get(t.xq, M * kmax);
+    get(t.xq, round_up(M, 16) * kmax);                    // row-major codes, or activation tiles with rows padded to 16
     get(t.sx, M * 4);
     get(t.qkv, M * (EQ + 2 * EKV) * 4);
     get(t.q_bf, M * EQ * 2);

@@ -391,7 +391,7 @@ __global__ void __launch_bounds__(THREADS)
 template <bool ONE>
 __global__ void __launch_bounds__(ONE ? 1024 : kBlock)
     swiglu_quantize_rows_kernel(const float *__restrict__ gu, int8_t *__restrict__ xq_row, float *__restrict__ sx,
-                                uint64_t f) {
+                                uint64_t f, int tiled) {
     constexpr int THREADS = ONE ? 1024 : kBlock;
     __shared__ float smem[THREADS / 64];
     const uint64_t r = blockIdx.x;
@@ -430,7 +430,7 @@ __global__ void __launch_bounds__(ONE ? 1024 : kBlock)
             uint32_t words[4] = {0, 0, 0, 0};
 #pragma unroll
             for (int e = 0; e < 16; ++e) words[e / 4] |= ((uint32_t)quant_i8(prod[e], scale) & 0xffu) << (8 * (e % 4));
-            *(v4u *)(xq_row + r * f + c * 16) = v4u{words[0], words[1], words[2], words[3]};
+            *(v4u *)(xq_row + (tiled ? tiled_chunk_offset(r, c, f / 64) : r * f + c * 16)) = v4u{words[0], words[1], words[2], words[3]};
         }
     } else {
         for (uint64_t c = threadIdx.x; c < f / 16; c += THREADS) {
@@ -441,7 +441,7 @@ __global__ void __launch_bounds__(ONE ? 1024 : kBlock)
 #pragma unroll
             for (int e = 0; e < 16; ++e)
                 words[e / 4] |= ((uint32_t)quant_i8(silu_f32(g[e]) * u[e], scale) & 0xffu) << (8 * (e % 4));
-            *(v4u *)(xq_row + r * f + c * 16) = v4u{words[0], words[1], words[2], words[3]};
+            *(v4u *)(xq_row + (tiled ? tiled_chunk_offset(r, c, f / 64) : r * f + c * 16)) = v4u{words[0], words[1], words[2], words[3]};
         }
     }
 }
@@ -634,12 +634,12 @@ void rmsnorm_quantize_rows_i8(const float *x, const float *w, float eps, int8_t 
         rmsnorm_quantize_kernel<4, true><<<grid, kBlock, 0, s>>>(x, w, eps, inv_n, nullptr, xq_rowmajor, sx, m, hidden, grid, WeightPrefetch{});
 }
 
-void swiglu_quantize_rows_i8(const float *gu, int8_t *xq_rowmajor, float *sx, uint64_t m, uint64_t f, hipStream_t s) {
+void swiglu_quantize_rows_i8(const float *gu, int8_t *xq, float *sx, uint64_t m, uint64_t f, hipStream_t s, bool tiled) {
     if (m == 0 || f == 0) return;
     if (f <= 16384)
-        swiglu_quantize_rows_kernel<true><<<(unsigned)m, 1024, 0, s>>>(gu, xq_rowmajor, sx, f);
+        swiglu_quantize_rows_kernel<true><<<(unsigned)m, 1024, 0, s>>>(gu, xq, sx, f, tiled ? 1 : 0);
     else
-        swiglu_quantize_rows_kernel<false><<<(unsigned)m, kBlock, 0, s>>>(gu, xq_rowmajor, sx, f);
+        swiglu_quantize_rows_kernel<false><<<(unsigned)m, kBlock, 0, s>>>(gu, xq, sx, f, tiled ? 1 : 0);
 }
 
 void quantize_rows_from_pmax(const void *x, bool in_bf16, const float *pmax, uint32_t parts, int8_t *xq_tiled,

@@ -20,6 +20,7 @@ using namespace fa::dev;
 int g_skinny_ntw = 0;      // tuning overrides (0 = heuristic)
 int g_skinny_waves = 0;
 int g_weight_prefetch = 0;   // 1: row kernels pull nothing for the linear that follows them
+int g_rows_kernel = 0;      // weight-stationary kernel for a few hundred rows: 0 by shape, 1 never, 2 whenever it can run
 int g_skinny_astat = 0;     // activation-stationary kernel: 0 by shape, 1 never, 2 whenever it can run
 int g_skinny_ksplit = 0;    // split k over the blocks of an XCD: 0 by shape, 1 never, 2 whenever it can run (agent-scope
                             // meeting), 3 whenever it can run (meeting in the XCD's L2), 4 by shape but agent scope
@@ -325,6 +326,128 @@ __global__ void __launch_bounds__(NWAVES * 64)
                 ((uint16_t *)ep.out)[o] = f32_to_bf16(v);
             else
                 ((float *)ep.out)[o] = v;
+        }
+    }
+}
+
+// ------------------------------------------------- W8A8, weight stationary (a few hundred rows)
+// Between the decode shapes (at most 64 rows, kernels above) and the tiled GEMMs (which need a few hundred output
+// tiles to fill the device): a prompt of 65 to a few hundred tokens against a weight with about one column tile per
+// compute unit.  A block owns NTW column tiles for all rows.  Its eight wavefronts divide k as above, but every
+// wavefront loads the weight tiles of its k-tiles once and keeps them in registers for the whole kernel; the
+// rows then pass by in groups of 64: the wavefront streams the activation tiles of its k-tiles for the group
+// (a ring of four k-tiles, refilled behind every multiply, running on into the next group), the eight partial
+// tiles meet in LDS and are finished exactly as in the kernel above.  The weight leaves HBM once, an activation
+// byte is read from L2 once per block, and once the weights are in, nothing a wavefront loads comes from HBM, so
+// no L2 hit waits behind a miss.  k_tiles <= 8 KTW; the tiled activation layout of the decode kernels.
+template <int KTW, int NTW>
+__global__ void __launch_bounds__(512)
+    w8a8_wstat_kernel(const int8_t *__restrict__ xq_tiled, const int8_t *__restrict__ w_tiles, uint32_t m, uint32_t n,
+                      uint32_t n_tiles, uint32_t k_tiles, EpiI8 ep) {
+    constexpr int NW = 8, MT = 4, NACC = MT * NTW * 4, DS = 4;
+    static_assert(KTW % DS == 0, "the ring restarts at slot 0 with every row group");
+    __shared__ int red[NW][NACC][64];
+    const int lane = threadIdx.x % 64;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+    const uint32_t nt0 = blockIdx.x * NTW;
+    const uint32_t cnt = k_tiles > (uint32_t)wave ? (k_tiles - wave + NW - 1) / NW : 0;      // k-tiles of this wavefront
+    const uint32_t row_tiles = (m + 15) / 16, groups = (row_tiles + MT - 1) / MT;
+
+    // the weights of this wavefront's k-tiles (clamped repeats past its last one are never multiplied)
+    v4i w[KTW][NTW];
+#pragma unroll
+    for (int t = 0; t < KTW; ++t) {
+        const uint32_t kt = wave + ((uint32_t)t < cnt ? (uint32_t)t : (cnt ? cnt - 1 : 0)) * NW;
+#pragma unroll
+        for (int j = 0; j < NTW; ++j) {
+            uint32_t nt = nt0 + j;
+            nt = nt < n_tiles ? nt : n_tiles - 1;
+            w[t][j] = stream_load<true>((const v4i *)(w_tiles + ((uint64_t)nt * k_tiles + (kt < k_tiles ? kt : 0)) * 1024 + (uint64_t)lane * 16));
+        }
+    }
+    // channel scale and bias of the accumulator elements this wavefront finishes (item q = element wave + 8 q)
+    constexpr int NE = NACC / NW;
+    float p_sw[NE], p_bias[NE];
+#pragma unroll
+    for (int q = 0; q < NE; ++q) {
+        const int idx = wave + q * NW, j = (idx / 4) % NTW;
+        const uint32_t col = (nt0 + j) * 16 + lane % 16;
+        p_sw[q] = col < n ? ep.sw[col] : 0.0f;
+        p_bias[q] = (ep.bias && col < n) ? ep.bias[col] : 0.0f;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // step (g, t): the MT activation tiles of k-tile t of this wavefront for row group g; row tiles past the last
+    // one repeat it (their sums are never stored)
+    v4i a[DS][MT];
+    auto load_step = [&](int slot, uint32_t g, int t) {
+        const uint32_t kt = wave + ((uint32_t)t < cnt ? (uint32_t)t : (cnt ? cnt - 1 : 0)) * NW;
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            uint32_t rt = g * MT + i;
+            rt = rt < row_tiles ? rt : row_tiles - 1;
+            a[slot][i] = *(const v4i *)(xq_tiled + ((uint64_t)rt * k_tiles + (kt < k_tiles ? kt : 0)) * 1024 + (uint64_t)lane * 16);
+        }
+    };
+#pragma unroll
+    for (int t = 0; t < DS; ++t) load_step(t, 0, t);
+    for (uint32_t g = 0; g < groups; ++g) {
+        // what the epilogue of this group needs, asked for ahead of its multiplies
+        float p_sx[NE], p_res[NE];
+#pragma unroll
+        for (int q = 0; q < NE; ++q) {
+            const int idx = wave + q * NW, e = idx % 4, j = (idx / 4) % NTW, i = idx / (4 * NTW);
+            const uint32_t row = (g * MT + i) * 16 + 4 * (lane / 16) + e, col = (nt0 + j) * 16 + lane % 16;
+            const bool ok = row < m && col < n;
+            p_sx[q] = ok ? ep.sx[row] : 0.0f;
+            p_res[q] = (ok && ep.residual) ? ep.residual[(uint64_t)row * n + col] : 0.0f;
+        }
+        v4i acc[MT][NTW];
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int j = 0; j < NTW; ++j) acc[i][j] = v4i{0, 0, 0, 0};
+#pragma unroll
+        for (int t = 0; t < KTW; ++t) {
+            if ((uint32_t)t < cnt) {
+#pragma unroll
+                for (int i = 0; i < MT; ++i)
+#pragma unroll
+                    for (int j = 0; j < NTW; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[t % DS][i], w[t][j], acc[i][j], 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);                // the refill right behind its consumer
+            if (t + DS < KTW) load_step(t % DS, g, t + DS);
+            else load_step(t % DS, g + 1 < groups ? g + 1 : g, t + DS - KTW);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        __syncthreads();                                      // everybody has read the sums of the group before
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int j = 0; j < NTW; ++j)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) red[wave][(i * NTW + j) * 4 + e][lane] = acc[i][j][e];
+        __syncthreads();
+#pragma unroll
+        for (int q = 0; q < NE; ++q) {
+            const int idx = wave + q * NW;
+            int sum = 0;
+#pragma unroll
+            for (int ww = 0; ww < NW; ++ww) sum += red[ww][idx][lane];
+            const int e = idx % 4, j = (idx / 4) % NTW, i = idx / (4 * NTW);
+            const uint32_t row = (g * MT + i) * 16 + 4 * (lane / 16) + e, col = (nt0 + j) * 16 + lane % 16;
+            if (row < m && col < n) {
+                const uint64_t o = (uint64_t)row * n + col;
+                if (ep.acc_out) ep.acc_out[o] = sum;
+                float v = __fmul_rn((float)sum, __fmul_rn(p_sx[q], p_sw[q]));
+                if (ep.bias) v = __fadd_rn(v, p_bias[q]);
+                if (ep.residual) v = __fadd_rn(p_res[q], v);
+                if (ep.out_bf16)
+                    ((uint16_t *)ep.out)[o] = f32_to_bf16(v);
+                else
+                    ((float *)ep.out)[o] = v;
+            }
         }
     }
 }
@@ -1515,6 +1638,50 @@ void linear_w8a8_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t 
         launch_w8a8_rows<1, kEpiPlain>(m, waves, grid, s, xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e);
     else
         launch_w8a8_rows<2, kEpiPlain>(m, waves, grid, s, xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e);
+}
+
+// Whether a linear of m rows takes the weight-stationary kernel: more rows than the decode kernels hold, a weight
+// with at most about two column tiles per compute unit, k within what a wavefront keeps in registers, and a block's
+// activation bytes (m x k, read from L2 once per block) below what the tiled GEMM with its k split costs.
+bool linear_w8a8_rows_applies(uint64_t m, uint64_t n_pad, uint64_t k_pad, int num_cus) {
+    if (g_rows_kernel == 1) return false;
+    const uint64_t n_tiles = n_pad / 16, k_tiles = k_pad / 64;
+    if (m <= 64 || n_tiles == 0 || k_tiles == 0 || k_tiles > 224) return false;
+    if (g_rows_kernel == 2) return true;
+    // measured against the tiled GEMM with its k split (both with their row quantizer, us): 4096 -> 4096 at 65 / 128 / 300 /
+    // 512 rows 13.9 / 14.8 / 25.7 / 37.1 against 24.3 / 27.5 / 33.2 / 41.1; 14336 -> 4096 at 128 rows 36.9 against 41.5, at 200
+    // rows 54.9 against 48.7: what it costs is the m x k bytes of activations every block pulls from L2
+    return n_tiles <= 2 * (uint64_t)num_cus && m * k_pad <= (2ull << 20);
+}
+
+void linear_w8a8_rows(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad,
+                      const EpilogueI8 &ep, int num_cus, hipStream_t s) {
+    if (m == 0 || n == 0) return;
+    EpiI8 e{};
+    e.sx = ep.sx;
+    e.sw = ep.sw;
+    e.bias = ep.bias;
+    e.residual = ep.residual;
+    e.acc_out = ep.acc_out;
+    e.out = ep.out;
+    e.out_bf16 = ep.out_bf16;
+    const uint32_t n_tiles = (uint32_t)(n_pad / 16), k_tiles = (uint32_t)(k_pad / 64);
+    // two column tiles per block once there are more tiles than compute units (every activation tile then feeds two
+    // multiplies), where the registers allow it
+    const bool two = n_tiles > (uint32_t)num_cus && k_tiles <= 64;
+    const unsigned grid = two ? (n_tiles + 1) / 2 : n_tiles;
+    auto go = [&](auto ktw, auto ntw) {
+        w8a8_wstat_kernel<decltype(ktw)::value, decltype(ntw)::value><<<grid, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n,
+                                                                                           n_tiles, k_tiles, e);
+    };
+    using std::integral_constant;
+    if (two) {
+        go(integral_constant<int, 8>{}, integral_constant<int, 2>{});
+    } else {
+        if (k_tiles <= 64) go(integral_constant<int, 8>{}, integral_constant<int, 1>{});
+        else if (k_tiles <= 128) go(integral_constant<int, 16>{}, integral_constant<int, 1>{});
+        else go(integral_constant<int, 28>{}, integral_constant<int, 1>{});
+    }
 }
 
 void linear_w8a8_swiglu_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, const float *sx, const float *sw,

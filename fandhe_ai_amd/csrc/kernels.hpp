@@ -72,9 +72,11 @@ void rmsnorm_quantize_i8(const float *x, const float *w, float eps, float *out_f
 // multiple of 16 and at most 16384.
 void rmsnorm_quantize_rows_i8(const float *x, const float *w, float eps, int8_t *xq_rowmajor, float *sx, uint64_t m,
                               uint64_t hidden, hipStream_t s);
-// act = silu(gate) * up of gu [m, 2 f] (gate columns first) quantized per token, row-major codes [m, f];
-// the f32 products are not stored.  f a multiple of 16.
-void swiglu_quantize_rows_i8(const float *gu, int8_t *xq_rowmajor, float *sx, uint64_t m, uint64_t f, hipStream_t s);
+// act = silu(gate) * up of gu [m, 2 f] (gate columns first) quantized per token, row-major codes [m, f] or
+// (tiled, f a multiple of 64) activation tiles with rows padded to 16; the f32 products are not stored.  f a
+// multiple of 16.
+void swiglu_quantize_rows_i8(const float *gu, int8_t *xq, float *sx, uint64_t m, uint64_t f, hipStream_t s,
+                             bool tiled = false);
 // Per-tensor absmax -> scale = absmax / 448 (one f32) then e4m3 codes.
 void quantize_tensor_e4m3(const float *x, uint8_t *q, float *scale, float *absmax_scratch, uint64_t n,
                           hipStream_t s);
@@ -193,6 +195,14 @@ void linear_w8a8_qkv_rope_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, 
 void linear_w8a16_skinny(const uint16_t *a, const int8_t *w_tiles, const float *sw, uint64_t m,
                          uint64_t n, uint64_t n_pad, uint64_t k_pad, void *out, int out_bf16,
                          int num_cus, hipStream_t s, const SplitKArea *sk = nullptr);
+
+// A few hundred rows (65 up) against a weight with about one column tile per compute unit: the weight-stationary
+// kernel (weights in registers, rows streamed in groups of 64).  xq_tiled: activation tiles with rows padded to 16,
+// as for linear_w8a8_skinny.  linear_w8a8_rows_applies says whether a shape should take it.
+extern int g_rows_kernel;     // 0: by shape, 1: never (the tiled GEMMs for every prompt pass), 2: whenever it can run
+bool linear_w8a8_rows_applies(uint64_t m, uint64_t n_pad, uint64_t k_pad, int num_cus);
+void linear_w8a8_rows(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad,
+                      const EpilogueI8 &ep, int num_cus, hipStream_t s);
 
 // ---- prefill-shape MFMA GEMMs (kern_gemm_mfma.hip) -----------------------------
 // aq: int8 [m, k_pad] row-major.  workspace (optional, gemm_w8a8_workspace_bytes): lets a matrix with too few

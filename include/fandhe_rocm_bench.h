@@ -89,7 +89,11 @@ fa_status fa_probe_l2_path(fa_context *ctx, const fa_buffer *cold, uint64_t cold
  *        is recorded);
  * key 20: 1 keeps the streamed attention with its merge launch for every decode step; 0: a step of one or two
  *        sequences whose contexts are at most 1024 tokens runs the attention as one launch (a block per sequence
- *        and kv head) and lets the o projection do the quantizer (takes effect when a step is recorded). */
+ *        and kv head) and lets the o projection do the quantizer (takes effect when a step is recorded);
+ * key 21: the int8 linears of 65 to a few hundred rows (fa_linear_w8a8, prompt passes of the decoder): 0 the
+ *        weight-stationary kernel where the shape rule picks it (a weight with at most about two column tiles per
+ *        compute unit, m x k at most 2 MiB) and the decode kernels for prompt passes of at most 64 rows, 1 the tiled
+ *        GEMMs always, 2 the weight-stationary kernel whenever it can run. */
 fa_status fa_set_tuning(int32_t key, int32_t value);
 
 /* What the context found when it was created: xcd_local = 1 when workgroups b and b + 8 of a launch were seen to

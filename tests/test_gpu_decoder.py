@@ -354,6 +354,38 @@ def test_prompt_pass_on_large_tiles_equals_the_pass_on_128_tiles_bit_for_bit():
         assert np.array_equal(ak, bk) and np.array_equal(av, bv)
 
 
+@pytest.mark.parametrize("batch,l_new", [(1, 70), (3, 100), (2, 33)], ids=["70-rows", "300-rows", "66-rows"])
+def test_prompt_pass_on_the_weight_stationary_kernel_equals_the_pass_on_the_tiled_gemm(batch, l_new):
+    """A prompt pass of 66 to 300 rows with every projection on the weight-stationary kernel (forced, tuning key
+    21 = 2: activation tiles from the quantizers, weights held in registers, rows in groups of 64) against the same
+    pass on the tiled GEMMs (key 21 = 1): int32 sums are exact and the epilogues apply scale, then residual, in the
+    same order, so logits, tokens and every cache row must be identical; the verification pass (head over every row)
+    as well."""
+    import fandhe_ai_amd as fa
+    be = ops()
+    lib = fa.capi.lib
+    shape = dict(n_layers=2, d_model=512, n_heads=4, n_kv_heads=2, d_ffn=1024, vocab=700, batch=batch, ctxs=[0, 9, 40][:batch])
+    m = build_model(seed=78, steps=l_new + 2, **shape)
+    prompt = o.Rng(7).randint(0, shape["vocab"], batch * l_new).astype(np.int32).reshape(batch, l_new)
+    got = {}
+    try:
+        for rows in (True, False):
+            fa.check(lib.fa_set_tuning(21, 2 if rows else 1))
+            dec = GpuDecoder(be, m)
+            try:
+                dec.prefill(prompt)
+                got[rows] = (dec.logits().copy(), dec.tokens().copy(), [tuple(x.copy() for x in dec.kv_pool(li)) for li in range(2)])
+            finally:
+                dec.close()
+    finally:
+        fa.check(lib.fa_set_tuning(21, 0))
+    a, b = got[True], got[False]
+    assert np.all(np.isfinite(a[0])) and np.any(a[0] != 0)
+    assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1])
+    for (ak, av), (bk, bv) in zip(a[2], b[2]):
+        assert np.array_equal(ak, bk) and np.array_equal(av, bv)
+
+
 @pytest.mark.parametrize("shape", [
     dict(n_layers=2, d_model=256, n_heads=4, n_kv_heads=2, d_ffn=512, vocab=1000, batch=3, ctxs=[0, 5, 40], l_new=6),
     dict(n_layers=1, d_model=256, n_heads=2, n_kv_heads=1, d_ffn=256, vocab=300, batch=1, ctxs=[21], l_new=40),

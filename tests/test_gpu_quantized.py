@@ -175,6 +175,42 @@ def test_w8a8_split_k_gemm_is_bit_exact(m, k, n):
     assert np.array_equal(got2, o.linear_w8a8(x, wq, ws)[1])
 
 
+@pytest.mark.parametrize("m,k,n", [(65, 4096, 4096), (128, 4096, 6144), (300, 4096, 4096), (512, 4096, 4096), (100, 14336, 4096),
+                                   (200, 2048, 1000), (77, 8192, 528), (260, 1024, 16), (512, 4096, 8192)])
+def test_w8a8_weight_stationary_kernel_for_a_few_hundred_rows(m, k, n):
+    """More rows than the decode kernels hold against a narrow weight: the weights stay in registers and the rows pass
+    by in groups of 64 (forced here for every shape, tuning key 21 = 2).  Raw sums and outputs bit-exact against the
+    oracle, with a bias, f32 and bf16 outputs, ragged row and column counts, one and two column tiles per block, all
+    three register depths; and equal to what the tiled GEMM path (key 21 = 1) returns."""
+    fa = _fa()
+    be = ops()
+    lib = fa.capi.lib
+    rng = o.Rng(3 * m + n)
+    x = rng.randn((m, k))
+    w = rng.randn((k, n), std=0.02)
+    bias = rng.randn((n,))
+    o.set_threads(8)
+    wq, ws = o.quantize_cols_i8(w)
+    want_acc, want = o.linear_w8a8(x, wq, ws, bias)
+    o.set_threads(1)
+    qw = be.import_quantized_weight(wq, ws)
+    dbias = fa.DeviceBufferView(be.upload(bias), 0, (n,))
+    dx = be.upload(x)
+    try:
+        fa.check(lib.fa_set_tuning(21, 2))
+        for rep in range(2):
+            out, acc = be.linear_w8a8(dx, qw, bias=dbias, want_acc=True)
+            assert np.array_equal(be.download_owned(acc), want_acc), rep
+            got = be.download_owned(out)
+            assert np.array_equal(got, want), rep
+        out_bf = be.linear_w8a8(dx, qw, bias=dbias, out_dtype=fa.capi.BF16)
+        assert_bf16_rounding_of("w8a8 weight-stationary bf16", be.download_owned(out_bf), got)
+        fa.check(lib.fa_set_tuning(21, 1))
+        assert np.array_equal(be.download_owned(be.linear_w8a8(dx, qw, bias=dbias)), got)
+    finally:
+        fa.check(lib.fa_set_tuning(21, 0))
+
+
 def test_w8a8_ragged_shapes():
     """Shapes off every tile size, with and without a bias, under one and two column tiles per block and four and
     eight wavefronts (wavefronts without a k-tile, fewer k-tiles than ring slots, a clamped last column tile): the
