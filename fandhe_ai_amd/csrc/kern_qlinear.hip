@@ -1436,18 +1436,21 @@ struct KsplitPlan {
 };
 inline bool ksplit_plan(uint64_t m, uint32_t n_tiles, uint32_t k_tiles, int num_cus, const SplitKArea *sk, int act_bytes,
                         KsplitPlan *p) {
-    if (!sk || !sk->partial || !sk->counters || g_skinny_ksplit == 1 || m == 0 || m > 32 || n_tiles == 0) return false;
+    // int8 activations: up to four row tiles (64 rows), in pairs of blocks; bf16 activations: up to two
+    const uint64_t m_max = act_bytes == 1 ? 64 : 32;
+    if (!sk || !sk->partial || !sk->counters || g_skinny_ksplit == 1 || m == 0 || m > m_max || n_tiles == 0) return false;
     const bool forced = g_skinny_ksplit == 2 || g_skinny_ksplit == 3;
     // By shape: the projections with about one column tile per compute unit whose blocks would each pull 256 KiB of
     // activations or more (measured in a decode step's kernel trace at 32 rows: 14336 -> 4096 int8 17.3 -> 14.6 us,
     // while 4096 -> 4096 int8, 128 KiB per block, loses 0.7 us to the meeting); wider weights keep their activations
     // in registers (w8a8_astat_kernel).
-    const uint64_t a_bytes = (uint64_t)(m <= 16 ? 16 : 32) * k_tiles * 64 * (uint64_t)act_bytes;
+    const int mt = m <= 16 ? 1 : m <= 32 ? 2 : 4;
+    const uint64_t a_bytes = (uint64_t)(16 * mt) * k_tiles * 64 * (uint64_t)act_bytes;
     if (!forced && ((uint64_t)n_tiles > 2 * (uint64_t)num_cus || a_bytes < (256u << 10))) return false;
     int s = g_skinny_ksplit_s ? g_skinny_ksplit_s : (k_tiles >= 128 ? 4 : 2);
+    if (mt == 4) s = 2;                                        // the partial tiles of four row tiles x four members do not fit LDS
     if (s != 2 && s != 4) return false;
     if (k_tiles / (uint32_t)s < 16) return false;              // two k-tiles per wavefront at least
-    const int mt = m <= 16 ? 1 : 2;
     const uint32_t n_groups = (n_tiles + s - 1) / s;
     const uint64_t bytes = (uint64_t)n_groups * s * ((uint64_t)mt * s * 4 * 64 * 4);
     if (n_groups > sk->n_counters || bytes > sk->partial_bytes) return false;
@@ -1487,8 +1490,10 @@ void ksplit_dispatch(uint64_t m, const KsplitPlan &p, F &&go) {
     };
     if (m <= 16)
         with_s(std::integral_constant<int, 1>{});
-    else
+    else if (m <= 32)
         with_s(std::integral_constant<int, 2>{});
+    else
+        with_d(std::integral_constant<int, 4>{}, std::integral_constant<int, 2>{});      // 33 .. 64 rows: pairs only
 }
 
 }  // namespace

@@ -368,7 +368,7 @@ def test_split_k_decode_linears_match_the_oracle():
     o.set_threads(8)
     try:
         for m, k, n in ((32, 4096, 4096), (32, 14336, 4096), (7, 2048, 33), (17, 4160, 1000), (32, 11008, 100), (1, 4096, 16),
-                        (20, 2112, 4112), (16, 8192, 528)):
+                        (20, 2112, 4112), (16, 8192, 528), (64, 14336, 4096), (33, 4096, 1000), (50, 2112, 4112)):
             rng = o.Rng(m + k + n)
             x = rng.randn((m, k))
             w = rng.randn((k, n), std=0.05)
@@ -378,7 +378,7 @@ def test_split_k_decode_linears_match_the_oracle():
             dx = be.upload(x)
             dbias = fa.DeviceBufferView(be.upload(bias), 0, (n,))
             want_acc, want = o.linear_w8a8(x, wq, ws, bias)
-            a16 = o.to_bf16(rng.randn((m, k))) if k % 64 == 0 else None
+            a16 = o.to_bf16(rng.randn((m, k))) if k % 64 == 0 and m <= 32 else None      # bf16 activations: at most 32 rows
             want16 = o.linear_w8a16(a16, wq, ws) if a16 is not None else None
             da16 = be.upload(a16) if a16 is not None else None
             for mode in modes:
