@@ -1446,7 +1446,9 @@ inline bool ksplit_plan(uint64_t m, uint32_t n_tiles, uint32_t k_tiles, int num_
     // in registers (w8a8_astat_kernel).
     const int mt = m <= 16 ? 1 : m <= 32 ? 2 : 4;
     const uint64_t a_bytes = (uint64_t)(16 * mt) * k_tiles * 64 * (uint64_t)act_bytes;
-    if (!forced && ((uint64_t)n_tiles > 2 * (uint64_t)num_cus || a_bytes < (256u << 10))) return false;
+    // (with four row tiles a pair of blocks halves the bytes: worth it from 512 KiB on; in a 64-row step's trace
+    // 4096 -> 4096 at 256 KiB went from 6 to 7.4 us, 14336 -> 4096 from 24 to 21.7 us)
+    if (!forced && ((uint64_t)n_tiles > 2 * (uint64_t)num_cus || a_bytes < ((mt == 4 ? 512u : 256u) << 10))) return false;
     int s = g_skinny_ksplit_s ? g_skinny_ksplit_s : (k_tiles >= 128 ? 4 : 2);
     if (mt == 4) s = 2;                                        // the partial tiles of four row tiles x four members do not fit LDS
     if (s != 2 && s != 4) return false;
