@@ -43,13 +43,19 @@ FA_HD void big_block_tile(uint32_t bid, uint32_t m_blocks, uint32_t n_blocks, ui
 template <int NWAVES>
 FA_HD int big_a_tile(int wave, int i) { return wave + NWAVES * i; }
 FA_HD int big_a_row(int lane) { return lane / 4; }
-// Byte offset inside the row's 128 stage bytes that lane `lane` fetches with load x (0 or 1) of a pair: the
-// 16-byte piece q = 2 ((p - rot) mod 4) + x, p = lane % 4, rot = r / 2 (e4m3) or r / 2 + 2 x (int8), r = lane / 4.
+// Byte offset inside the row's 128 stage bytes that lane `lane` fetches with load x (0 or 1) of a pair, r = lane / 4,
+// p = lane % 4 its slot in the row's four slots of slice x.  e4m3: the 16-byte piece q = 2 ((p - r / 2) mod 4) + x.
+// int8: piece q = 2 j + x sits in slot (x + 2 (j % 2) + j / 2 + r / 2) mod 4, so that the four k-groups g of k-step s
+// (pieces 4 s + g: j = 2 s + g / 2, x = g % 2) read slots (g + s + r / 2) mod 4, the e4m3 pattern: the LDS serves a
+// 16-byte read sixteen lanes per cycle, lanes of two neighbouring k-groups together, and any other spacing of their
+// slots halves its rate (measured: 8 instead of 4 cycles per instruction).
 template <bool FP8>
 FA_HD int big_a_src_byte(int lane, int x) {
     const int r = lane / 4, p4 = lane % 4;
-    const int pp = (p4 - r / 2 - (FP8 ? 0 : 2 * x)) & 3;
-    return pp * 32 + x * 16;
+    if (FP8) return ((p4 - r / 2) & 3) * 32 + x * 16;
+    const int t = (p4 - x - r / 2) & 3;              // = 2 (j % 2) + j / 2
+    const int j = ((t & 1) << 1) | (t >> 1);
+    return j * 32 + x * 16;
 }
 // LDS byte offset of the slice that load (tile, h) of stage slot `slot` fills (the lane's 16 bytes go to + lane * 16).
 template <int NTB>
@@ -61,8 +67,7 @@ template <bool FP8>
 FA_HD int big_a_frag_off(int lane, int sub) {
     const int g = lane / 16, r = lane % 16;
     if (FP8) return sub * 1024 + (4 * r + ((g + r / 2) & 3)) * 16;
-    const int q = 4 * sub + g, x = q & 1;
-    return x * 1024 + (4 * r + (((q >> 1) + r / 2 + 2 * x) & 3)) * 16;
+    return (g & 1) * 1024 + (4 * r + ((g + sub + r / 2) & 3)) * 16;
 }
 
 // B tile (block-local column tile) that wavefront `wave` moves with load pair i: a block of 14 tiles has no tiles

@@ -354,12 +354,12 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
     // A rows are row-major in memory: a row's 128 bytes of a stage are eight 16-byte pieces q.  Load
     // instruction x takes the pieces with q % 2 == x, four consecutive lanes sharing one row, so every
     // lane quad touches one whole cache line per instruction (the L1 fetches it once; the second
-    // instruction hits) instead of one line per lane.  Lane 4 r + p fills LDS slot 4 r + p of slice x
-    // with piece q = 2 ((p - rot) mod 4) + x.  The rotation spreads the fragment reads over the LDS
-    // banks: rot = r / 2 for e4m3, whose k-group g of the matrix instruction is pieces 2 g, 2 g + 1, i.e.
-    // slot 4 r + (g + r / 2) mod 4 of both slices; rot = r / 2 + 2 x for int8, whose k-group g of k-step s
-    // is the single piece q = 4 s + g in slice q % 2, slot 4 r + (q / 2 + rot) mod 4 (without the 2 x
-    // term the lanes of k-groups g and g + 1 would read the same banks of the two slices).
+    // instruction hits) instead of one line per lane.  Lane 4 r + p fills LDS slot 4 r + p of slice x; which
+    // piece that is rotates with the row, so that the fragment reads spread over the LDS banks: e4m3's k-group g
+    // of the matrix instruction is pieces 2 g, 2 g + 1, kept in slot 4 r + (g + r / 2) mod 4 of both slices; int8's
+    // k-group g of k-step s is the single piece 4 s + g in slice g % 2, kept in slot 4 r + (g + s + r / 2) mod 4
+    // (the LDS serves sixteen lanes of a 16-byte read per cycle, the lanes of two neighbouring k-groups together:
+    // their slots have to differ by an odd number, or the read runs at half rate).
     constexpr int B_H = FP8 ? 16 : 1024;             // byte offset of slice h in a stage's weight tile in memory
     static_assert(ixm::big_b_src_byte<FP8>(0, 1) == B_H && ixm::kBigTk == TK && ixm::kBigTile == TILE, "index model out of step");
     const uint8_t *a_src[TPW][2];
@@ -583,6 +583,7 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
 #pragma unroll
                 for (int j = 0; j < WNT; ++j) res[j] = *(const v4f *)(residual + o0 + j * 16);
             }
+            v2u pk[WNT];                              // bf16 output: the four columns of tile j, packed
 #pragma unroll
             for (int j = 0; j < WNT; ++j) {
                 float v[4];
@@ -593,11 +594,22 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
                     if (bias) v[e] = __fadd_rn(v[e], bc[j][e]);
                     if (residual) v[e] = __fadd_rn(res[j][e], v[e]);
                 }
-                if (!row_ok) continue;
-                if (out_bf16)
-                    *(v2u *)(orow + j * 32) = v2u{f32x2_to_bf16x2(v[0], v[1]), f32x2_to_bf16x2(v[2], v[3])};
-                else
-                    *(v4f *)(orow + j * 64) = v4f{v[0], v[1], v[2], v[3]};
+                if (out_bf16) pk[j] = v2u{f32x2_to_bf16x2(v[0], v[1]), f32x2_to_bf16x2(v[2], v[3])};
+                else if (row_ok) *(v4f *)(orow + j * 64) = v4f{v[0], v[1], v[2], v[3]};
+            }
+            if (out_bf16) {
+                // Two tiles at a time, the lanes of column groups g = 1, 3 trade their four columns of the first tile
+                // for the four columns that groups g - 1 hold of the second (v_permlane16_swap: rows of sixteen lanes
+                // 1, 3 of one register against rows 0, 2 of the other).  Then g = 0, 2 hold columns 0 .. 7 and 8 .. 15
+                // of the first tile and g = 1, 3 those of the second: one 16-byte store per lane, 64 contiguous bytes
+                // per output row and instruction instead of 32.
+#pragma unroll
+                for (int j = 0; j + 1 < WNT; j += 2) {
+                    const auto lo = __builtin_amdgcn_permlane16_swap(pk[j][0], pk[j + 1][0], false, false);
+                    const auto hi = __builtin_amdgcn_permlane16_swap(pk[j][1], pk[j + 1][1], false, false);
+                    if (row_ok) *(v4u *)(orow - 8 * g + (j + (g & 1)) * 32 + (g >> 1) * 16) = v4u{lo[0], hi[0], lo[1], hi[1]};
+                }
+                if (WNT % 2 == 1 && row_ok) *(v2u *)(orow + (WNT - 1) * 32) = pk[WNT - 1];
             }
         }
         return;

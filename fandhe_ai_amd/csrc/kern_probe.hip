@@ -35,20 +35,32 @@ __global__ void __launch_bounds__(256) matrix_rate_kernel(const v4i *__restrict_
     for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc32[i][e] = 0;
+    // The instructions are written out with their accumulators tied to the accumulation registers: through the
+    // builtins the register allocator moved accumulators between the two register files around every instruction
+    // of the 16 x 16 x 64 form, and the loop then measured those moves (half the instruction's rate).
     for (uint32_t it = 0; it < iters; ++it) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             const v4i &x = a[i % 8], &y = b[(i * 3) % 8];
-            if constexpr (KIND == 0) acc16[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(x, y, acc16[i], 0, 0, 0);
-            if constexpr (KIND == 1) acc32[i % 4] = __builtin_amdgcn_mfma_i32_32x32x32_i8(x, y, acc32[i % 4], 0, 0, 0);
+            if constexpr (KIND == 0) asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(acc16[i]) : "v"(x), "v"(y));
+            if constexpr (KIND == 1) asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+a"(acc32[i % 4]) : "v"(x), "v"(y));
             if constexpr (KIND == 2) {
                 const v4i &x1 = a[(i + 1) % 8], &y1 = b[(i * 3 + 1) % 8];
-                accf[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                    v8i{x[0], x[1], x[2], x[3], x1[0], x1[1], x1[2], x1[3]},
-                    v8i{y[0], y[1], y[2], y[3], y1[0], y1[1], y1[2], y1[3]}, accf[i], 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
+                const v8i xx = v8i{x[0], x[1], x[2], x[3], x1[0], x1[1], x1[2], x1[3]};
+                const v8i yy = v8i{y[0], y[1], y[2], y[3], y1[0], y1[1], y1[2], y1[3]};
+                const int unit = 0x7f7f7f7f;          // block scales 2^0
+                asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %3 op_sel_hi:[0,0,0]"
+                             : "+a"(accf[i])
+                             : "v"(xx), "v"(yy), "v"(unit));
             }
         }
     }
+    // the compiler does not know that the statements above are matrix instructions: wait out the pipeline before
+    // anything reads an accumulator
+#pragma unroll
+    for (int i = 0; i < 16; ++i) asm volatile("s_nop 15\n\ts_nop 15" : "+a"(acc16[i]), "+a"(accf[i]));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) asm volatile("s_nop 15\n\ts_nop 15" : "+a"(acc32[i]));
     int s = 0;
 #pragma unroll
     for (int i = 0; i < 16; ++i) s += acc16[i][0] + (int)accf[i][0];

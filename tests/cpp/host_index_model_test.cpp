@@ -79,7 +79,7 @@ static void gemm_case() {
         CHECK((int)seen.size() == kBigRows * kBigTk);
 
         // operand reads.  A: lane (g, r) of row tile t wants row 16 t + r and, e4m3, k bytes 32 g + 16 sub .. + 15;
-        // int8, k bytes 64 sub + 16 g .. + 15.  16-byte reads must also be bank-conflict free eight lanes at a time.
+        // int8, k bytes 64 sub + 16 g .. + 15.  16-byte reads must also be bank-conflict free.
         for (int wm = 0; wm < WM; ++wm)
             for (int i = 0; i < AI; ++i)
                 for (int sub = 0; sub < 2; ++sub) {
@@ -98,6 +98,17 @@ static void gemm_case() {
                         for (int l = 0; l < 8; ++l) banks.insert((big_a_frag_off<FP8>(oct * 8 + l, sub) / 16) % 8);
                         CHECK(banks.size() == 8);
                     }
+                    // the full-rate rule as measured on the device: eight lanes of one k-group and the same eight of
+                    // the neighbouring group (lanes l and l + 16) are served in one cycle and must cover the 64 banks
+                    // (sixteen 16-byte columns) exactly once
+                    for (int pair = 0; pair < 2; ++pair)
+                        for (int half = 0; half < 2; ++half) {
+                            std::set<int> cols;
+                            for (int l = 0; l < 8; ++l)
+                                for (int gg = 0; gg < 2; ++gg)
+                                    cols.insert((big_a_frag_off<FP8>(32 * pair + 16 * gg + 8 * half + l, sub) / 16) % 16);
+                            CHECK(cols.size() == 16);
+                        }
                 }
         // B: lane l of fragment j of wavefront column wn wants slice h of its own 16 bytes of tile wn * WNT + j
         for (int wn = 0; wn < 2; ++wn)
