@@ -342,13 +342,17 @@ fa_status fa_linear_w8a8(fa_context *ctx, const fa_buffer *x, uint64_t m, const 
                             qw->k_pad, ctx->stream);
         k::linear_w8a8_skinny((const int8_t *)xq.ptr, (const int8_t *)qw->codes->ptr, m, qw->n, qw->n_pad, qw->k_pad,
                               ep, ctx->props.multiProcessorCount, ctx->stream, &ctx->splitk);
-    } else if (qw->k == qw->k_pad && k::linear_w8a8_rows_applies(m, qw->n_pad, qw->k_pad, ctx->props.multiProcessorCount)) {
+    } else if (qw->k == qw->k_pad &&
+               k::linear_w8a8_rows_applies(m, qw->n_pad, qw->k_pad, ctx->props.multiProcessorCount, &ctx->splitk)) {
         uint64_t m_pad = round_up(m, 16);
         if (fa_status s = xq.get(m_pad * qw->k_pad)) return s;
+        Scratch ws(ctx);
+        if (uint64_t wsb = k::linear_w8a8_rows_workspace_bytes(m, qw->n_pad, qw->k_pad, ctx->props.multiProcessorCount, &ctx->splitk))
+            if (fa_status s = ws.get(wsb)) return s;
         k::quantize_rows_i8(x->ptr, x->dtype == FA_BF16, nullptr, (int8_t *)xq.ptr, (float *)sx.ptr, m, m_pad, qw->k,
                             qw->k_pad, ctx->stream);
         k::linear_w8a8_rows((const int8_t *)xq.ptr, (const int8_t *)qw->codes->ptr, m, qw->n, qw->n_pad, qw->k_pad, ep,
-                            ctx->props.multiProcessorCount, ctx->stream);
+                            ctx->props.multiProcessorCount, ctx->stream, &ctx->splitk, ws.ptr, ws.bytes);
     } else {
         if (qw->k != qw->k_pad) return fail(FA_ERR_UNSUPPORTED, "linear_w8a8: m > 64 needs k to be a multiple of 64");
         if (fa_status s = xq.get(mk)) return s;

@@ -369,7 +369,7 @@ fa_status enqueue_prefill_chunk(fa_context *ctx, fa_decoder *d, PrefillBuffers &
     const uint64_t M_pad = round_up(M, 16);
     // (at most 64 rows: every projection on the decode kernels, which take the same layout)
     const bool decode_form = M <= 64 && k::g_rows_kernel != 1;
-    auto rows_form = [&](const fa_qweight *w) { return decode_form || k::linear_w8a8_rows_applies(M, w->n_pad, w->k_pad, cus); };
+    auto rows_form = [&](const fa_qweight *w) { return decode_form || k::linear_w8a8_rows_applies(M, w->n_pad, w->k_pad, cus, &ctx->splitk); };
     // y = dequant(xq @ w) (+ residual) for the rows quantized into t.xq / t.sx just before
     auto gemm = [&](const fa_qweight *w, float *out, const float *residual) {
         k::EpilogueI8 ep;
@@ -384,7 +384,8 @@ fa_status enqueue_prefill_chunk(fa_context *ctx, fa_decoder *d, PrefillBuffers &
             k::linear_w8a8_skinny(t.xq.as<int8_t>(), (const int8_t *)w->codes->ptr, M, w->n, w->n_pad, w->k_pad, ep, cus, s,
                                   &ctx->splitk);
         else if (rows_form(w))
-            k::linear_w8a8_rows(t.xq.as<int8_t>(), (const int8_t *)w->codes->ptr, M, w->n, w->n_pad, w->k_pad, ep, cus, s);
+            k::linear_w8a8_rows(t.xq.as<int8_t>(), (const int8_t *)w->codes->ptr, M, w->n, w->n_pad, w->k_pad, ep, cus, s,
+                                &ctx->splitk, t.splitk.ptr, t.splitk.bytes);
         else
             k::gemm_w8a8_mfma(t.xq.as<int8_t>(), (const int8_t *)w->codes->ptr, M, w->n, w->n_pad, w->k_pad, ep, cus, s,
                               t.splitk.ptr, t.splitk.bytes);
@@ -812,7 +813,8 @@ static fa_status prefill_impl(fa_context *ctx, fa_decoder *d, const int32_t *tok
         const int cus = ctx->props.multiProcessorCount;
         for (const auto &l : d->layers)
             for (const fa_qweight *w : {l.wqkv, l.wo, l.wgu, l.wdown})
-                need = std::max(need, k::gemm_w8a8_workspace_bytes(M, w->n, w->n_pad, w->k_pad, cus));
+                need = std::max({need, k::gemm_w8a8_workspace_bytes(M, w->n, w->n_pad, w->k_pad, cus),
+                                 k::linear_w8a8_rows_workspace_bytes(M, w->n_pad, w->k_pad, cus, &ctx->splitk)});
         if (verify)
             need = std::max(need, k::gemm_w8a8_workspace_bytes(M, d->lm_head->n, d->lm_head->n_pad, d->lm_head->k_pad, cus));
         get(t.splitk, need);

@@ -131,6 +131,12 @@ FA_HD void ksplit_k_range(uint32_t k_tiles, uint32_t member, uint32_t s, uint32_
 FA_HD uint64_t ksplit_partial_base(uint32_t group, uint32_t member, uint32_t s, uint32_t nacc) {
     return ((uint64_t)group * s + member) * ((uint64_t)nacc * 64);
 }
+// The weight-stationary split-k linear (w8a8_wstat_ksplit_kernel) leaves a partial tile set per row group: first
+// element of the set of (group, member, row group) in its workspace; nacc = row tiles of a row group x S x 4 items.
+FA_HD uint64_t rows_ksplit_partial_base(uint32_t group, uint32_t member, uint32_t s, uint32_t row_groups, uint32_t row_group,
+                                        uint32_t nacc) {
+    return (((uint64_t)group * s + member) * row_groups + row_group) * ((uint64_t)nacc * 64);
+}
 
 }  // namespace ixm
 }  // namespace fa

@@ -330,6 +330,29 @@ __global__ void __launch_bounds__(NWAVES * 64)
     }
 }
 
+// Stores that the compiler's wait-count bookkeeping does not see.  On this target loads and stores share one
+// counter (vmcnt) but complete out of order with respect to each other, so with a store pending the compiler turns
+// every wait for a load into vmcnt(0): in a loop that keeps a ring of loads in flight and stores results once per
+// pass, every pass then starts by draining the ring.  Issued like this the stores still raise the hardware counter,
+// which only makes a wait for "at most N loads outstanding" stricter than it had to be (loads complete in order
+// among themselves), never laxer.  Nothing in the kernels that use them reads the stored locations back through
+// the compiler's loads.  POLICY 0: plain, 1: sc0 (workgroup scope), 2: sc1 (agent scope).
+template <int POLICY>
+__device__ __forceinline__ void store_unseen_b32(void *p, uint32_t v) {
+    if constexpr (POLICY == 0) asm volatile("global_store_dword %0, %1, off" : : "v"(p), "v"(v));
+    else if constexpr (POLICY == 1) asm volatile("global_store_dword %0, %1, off sc0" : : "v"(p), "v"(v));
+    else asm volatile("global_store_dword %0, %1, off sc1" : : "v"(p), "v"(v));
+}
+template <int POLICY>
+__device__ __forceinline__ void store_unseen_b128(void *p, v4i v) {
+    if constexpr (POLICY == 0) asm volatile("global_store_dwordx4 %0, %1, off" : : "v"(p), "v"(v));
+    else if constexpr (POLICY == 1) asm volatile("global_store_dwordx4 %0, %1, off sc0" : : "v"(p), "v"(v));
+    else asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v));
+}
+__device__ __forceinline__ void store_unseen_b16(void *p, uint32_t v) {
+    asm volatile("global_store_short %0, %1, off" : : "v"(p), "v"(v));
+}
+
 // ------------------------------------------------- W8A8, weight stationary (a few hundred rows)
 // Between the decode shapes (at most 64 rows, kernels above) and the tiled GEMMs (which need a few hundred output
 // tiles to fill the device): a prompt of 65 to a few hundred tokens against a weight with about one column tile per
@@ -353,7 +376,8 @@ __global__ void __launch_bounds__(512)
     const uint32_t cnt = k_tiles > (uint32_t)wave ? (k_tiles - wave + NW - 1) / NW : 0;      // k-tiles of this wavefront
     const uint32_t row_tiles = (m + 15) / 16, groups = (row_tiles + MT - 1) / MT;
 
-    // the weights of this wavefront's k-tiles (clamped repeats past its last one are never multiplied)
+    // the weights of this wavefront's k-tiles; past its last one zeros, so that every step multiplies and the row
+    // loop below is straight-line code (the compiler then counts the loads of the activation ring exactly)
     v4i w[KTW][NTW];
 #pragma unroll
     for (int t = 0; t < KTW; ++t) {
@@ -362,7 +386,8 @@ __global__ void __launch_bounds__(512)
         for (int j = 0; j < NTW; ++j) {
             uint32_t nt = nt0 + j;
             nt = nt < n_tiles ? nt : n_tiles - 1;
-            w[t][j] = stream_load<true>((const v4i *)(w_tiles + ((uint64_t)nt * k_tiles + (kt < k_tiles ? kt : 0)) * 1024 + (uint64_t)lane * 16));
+            const v4i x = stream_load<true>((const v4i *)(w_tiles + ((uint64_t)nt * k_tiles + (kt < k_tiles ? kt : 0)) * 1024 + (uint64_t)lane * 16));
+            w[t][j] = (uint32_t)t < cnt ? x : v4i{0, 0, 0, 0};
         }
     }
     // channel scale and bias of the accumulator elements this wavefront finishes (item q = element wave + 8 q)
@@ -409,13 +434,11 @@ __global__ void __launch_bounds__(512)
             for (int j = 0; j < NTW; ++j) acc[i][j] = v4i{0, 0, 0, 0};
 #pragma unroll
         for (int t = 0; t < KTW; ++t) {
-            if ((uint32_t)t < cnt) {
 #pragma unroll
-                for (int i = 0; i < MT; ++i)
+            for (int i = 0; i < MT; ++i)
 #pragma unroll
-                    for (int j = 0; j < NTW; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[t % DS][i], w[t][j], acc[i][j], 0, 0, 0);
-            }
+                for (int j = 0; j < NTW; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[t % DS][i], w[t][j], acc[i][j], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);                // the refill right behind its consumer
             if (t + DS < KTW) load_step(t % DS, g, t + DS);
             else load_step(t % DS, g + 1 < groups ? g + 1 : g, t + DS - KTW);
@@ -439,14 +462,14 @@ __global__ void __launch_bounds__(512)
             const uint32_t row = (g * MT + i) * 16 + 4 * (lane / 16) + e, col = (nt0 + j) * 16 + lane % 16;
             if (row < m && col < n) {
                 const uint64_t o = (uint64_t)row * n + col;
-                if (ep.acc_out) ep.acc_out[o] = sum;
+                if (ep.acc_out) store_unseen_b32<0>(ep.acc_out + o, (uint32_t)sum);
                 float v = __fmul_rn((float)sum, __fmul_rn(p_sx[q], p_sw[q]));
                 if (ep.bias) v = __fadd_rn(v, p_bias[q]);
                 if (ep.residual) v = __fadd_rn(p_res[q], v);
                 if (ep.out_bf16)
-                    ((uint16_t *)ep.out)[o] = f32_to_bf16(v);
+                    store_unseen_b16((uint16_t *)ep.out + o, f32_to_bf16(v));
                 else
-                    ((float *)ep.out)[o] = v;
+                    store_unseen_b32<0>((float *)ep.out + o, __float_as_uint(v));
             }
         }
     }
@@ -941,6 +964,21 @@ __device__ __forceinline__ T meet_load(const T *p) {
     else
         return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// Four consecutive words of a partial tile set, requested with the cache policy of meet_load (a wider relaxed atomic
+// load does not exist; the words were written by one 16-byte store whose acknowledgement the writer awaited before its
+// ticket).  The request is an assembly statement, so the compiler neither waits for it nor knows that `v` is in
+// flight: `v` may only be touched after an unseen_wait_all that names it.
+template <bool LOCAL>
+__device__ __forceinline__ void meet_request_b128(v4i &v, const int32_t *p) {
+    if constexpr (LOCAL) asm volatile("global_load_dwordx4 %0, %1, off sc0" : "=&v"(v) : "v"(p));
+    else asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=&v"(v) : "v"(p));
+}
+__device__ __forceinline__ void unseen_wait_all(v4i (&x)[4][4]) {
+    asm volatile("s_waitcnt vmcnt(0)"
+                 : "+v"(x[0][0]), "+v"(x[0][1]), "+v"(x[0][2]), "+v"(x[0][3]), "+v"(x[1][0]), "+v"(x[1][1]), "+v"(x[1][2]),
+                   "+v"(x[1][3]), "+v"(x[2][0]), "+v"(x[2][1]), "+v"(x[2][2]), "+v"(x[2][3]), "+v"(x[3][0]), "+v"(x[3][1]),
+                   "+v"(x[3][2]), "+v"(x[3][3]));
+}
 // Ticket of this block in its group (0 .. S - 1), the same value in every thread.  `slot` is one LDS word that
 // nobody else uses between the two barriers.  Call with all of the block's partial stores issued.
 template <bool LOCAL>
@@ -1112,6 +1150,154 @@ __global__ void __launch_bounds__(512)
                 ((uint16_t *)ep.out)[o] = f32_to_bf16(v);
             else
                 ((float *)ep.out)[o] = v;
+        }
+    }
+}
+
+// W8A8, weight stationary, for 65 to a few hundred rows against a deep, narrow weight (k of 8192 and more, about one
+// column tile per compute unit): w8a8_wstat_kernel above would pull m x k activation bytes through every compute
+// unit.  Here a group of S = 4 same-XCD blocks owns four column tiles and member j keeps the weights of k-range j of
+// all four in registers (KTW k-tiles per wavefront x 4 tiles); the rows pass by in groups of 32, every member
+// streaming only its quarter of their k.  The sums of a row group over the eight wavefronts meet in LDS and go to
+// the workspace as one partial tile set per (member, row group); when the rows are through, the member takes a
+// ticket as in w8a8_ksplit_kernel, and the last arriver adds the four partial sets of every row group (int32:
+// exact in any order) and runs the epilogue for all rows of the group's 64 columns.  Nobody waits for anybody.
+template <int KTW, int DS, bool LOCAL>
+__global__ void __launch_bounds__(512)
+    w8a8_wstat_ksplit_kernel(const int8_t *__restrict__ xq_tiled, const int8_t *__restrict__ w_tiles, uint32_t m, uint32_t n,
+                             uint32_t n_tiles, uint32_t k_tiles, uint32_t n_groups, EpiI8 ep, int32_t *partial,
+                             uint32_t *counters, uint32_t *xcc_seen, uint32_t *fault) {
+    constexpr int NW = 8, S = 4, MT = 2, NACC = MT * S * 4;
+    static_assert(MT * S == NW, "one accumulator tile of a row group per wavefront");
+    static_assert(KTW % DS == 0, "the ring restarts at slot 0 with every row group");
+    __shared__ v4i red[2][NW][MT * S][64];            // two buffers: one barrier per row group
+    const int lane = threadIdx.x % 64;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+    uint32_t group, member;
+    ksplit_ids<S>(&group, &member);
+    if (group >= n_groups) return;                   // the same for every member of the group
+    const uint32_t nt0 = group * S;
+    uint32_t kt_lo, kt_hi;
+    ixm::ksplit_k_range(k_tiles, member, S, &kt_lo, &kt_hi);
+    const uint32_t len = kt_hi - kt_lo;
+    const uint32_t cnt = len > (uint32_t)wave ? (len - wave + NW - 1) / NW : 0;       // k-tiles of this wavefront (<= KTW)
+    const uint32_t row_tiles = (m + 15) / 16, row_groups = (row_tiles + MT - 1) / MT;
+    // k-tile of step t (steps past the wavefront's last k-tile repeat it and multiply it with zeros)
+    auto kt_of = [&](int t) -> uint32_t {
+        const uint32_t kt = kt_lo + wave + ((uint32_t)t < cnt ? (uint32_t)t : (cnt ? cnt - 1 : 0)) * NW;
+        return kt < k_tiles ? kt : k_tiles - 1;
+    };
+
+    v4i w[KTW][S];                                   // zeros past the wavefront's last k-tile: every step multiplies
+#pragma unroll
+    for (int t = 0; t < KTW; ++t) {
+        const uint32_t kt = kt_of(t);
+#pragma unroll
+        for (int j = 0; j < S; ++j) {
+            uint32_t nt = nt0 + j;
+            nt = nt < n_tiles ? nt : n_tiles - 1;            // a tile past the edge is loaded clamped, never stored
+            const v4i x = stream_load<true>((const v4i *)(w_tiles + ((uint64_t)nt * k_tiles + kt) * 1024 + (uint64_t)lane * 16));
+            w[t][j] = (uint32_t)t < cnt ? x : v4i{0, 0, 0, 0};
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    v4i a[DS][MT];
+    auto load_step = [&](int slot, uint32_t g, int t) {
+        const uint32_t kt = kt_of(t);
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            uint32_t rt = g * MT + i;
+            rt = rt < row_tiles ? rt : row_tiles - 1;
+            a[slot][i] = *(const v4i *)(xq_tiled + ((uint64_t)rt * k_tiles + kt) * 1024 + (uint64_t)lane * 16);
+        }
+    };
+#pragma unroll
+    for (int t = 0; t < DS; ++t) load_step(t, 0, t);
+    for (uint32_t g = 0; g < row_groups; ++g) {
+        v4i acc[MT][S];
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int j = 0; j < S; ++j) acc[i][j] = v4i{0, 0, 0, 0};
+#pragma unroll
+        for (int t = 0; t < KTW; ++t) {
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+#pragma unroll
+                for (int j = 0; j < S; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[t % DS][i], w[t][j], acc[i][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);                // the refill right behind its consumer
+            if (t + DS < KTW) load_step(t % DS, g, t + DS);
+            else load_step(t % DS, g + 1 < row_groups ? g + 1 : g, t + DS - KTW);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // the sums of row group g - 2 were read from this buffer before the barrier of group g - 1
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int j = 0; j < S; ++j) red[g & 1][wave][i * S + j][lane] = acc[i][j];
+        __syncthreads();
+        // wavefront w adds the eight partial tiles of tile w = (row tile w / S, column tile w % S)
+        v4i sum = v4i{0, 0, 0, 0};
+#pragma unroll
+        for (int ww = 0; ww < NW; ++ww) sum += red[g & 1][ww][wave][lane];
+        int32_t *mine = partial + ixm::rows_ksplit_partial_base(group, member, S, row_groups, g, NACC);
+        store_unseen_b128<LOCAL ? 1 : 2>(mine + (wave * 64 + lane) * 4, sum);       // the policy meet_store uses
+    }
+    if (LOCAL && xcc_seen && threadIdx.x == 0) meet_store<true>(xcc_seen + (uint64_t)group * S + member, this_xcc() + 1u);
+    const uint32_t ticket = meet_ticket<LOCAL>(counters + group, (uint32_t *)&red[0][0][0][0]);
+    if (ticket != S - 1) return;
+    if (threadIdx.x == 0) meet_store<LOCAL>(counters + group, 0u);      // for the next launch
+    if constexpr (LOCAL) meet_check_xcd<S>(xcc_seen, group, fault);
+    // this wavefront's tile of every row group: rows 4 (lane / 16) + e of row tile wave / S, column lane % 16 of
+    // column tile wave % S; the four members' sums are added in member order (int32: exact in any order)
+    const int ti = wave / S, tj = wave % S;
+    const uint32_t col = (nt0 + tj) * 16 + lane % 16;
+    const bool col_ok = col < n;
+    const float p_sw = col_ok ? ep.sw[col] : 0.0f;
+    const float p_bias = (ep.bias && col_ok) ? ep.bias[col] : 0.0f;
+    for (uint32_t g0 = 0; g0 < row_groups; g0 += 4) {            // four row groups' partial sets in flight
+        v4i part[4][S];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const uint32_t g = g0 + u < row_groups ? g0 + u : row_groups - 1;
+#pragma unroll
+            for (int r = 0; r < S; ++r)
+                meet_request_b128<LOCAL>(part[u][r], partial + ixm::rows_ksplit_partial_base(group, r, S, row_groups, g, NACC) + (wave * 64 + lane) * 4);
+        }
+        float p_sx[4][4], p_res[4][4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const uint32_t row0 = ((g0 + u) * MT + ti) * 16 + 4 * (lane / 16);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const bool ok = row0 + e < m && col_ok;
+                p_sx[u][e] = ok ? ep.sx[row0 + e] : 0.0f;
+                p_res[u][e] = (ok && ep.residual) ? ep.residual[(uint64_t)(row0 + e) * n + col] : 0.0f;
+            }
+        }
+        unseen_wait_all(part);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const uint32_t row0 = ((g0 + u) * MT + ti) * 16 + 4 * (lane / 16);
+            v4i sum = part[u][0];
+#pragma unroll
+            for (int r = 1; r < S; ++r) sum += part[u][r];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (row0 + e < m && col_ok) {                     // also false for the row groups past the last one
+                    const uint64_t o = (uint64_t)(row0 + e) * n + col;
+                    if (ep.acc_out) store_unseen_b32<0>(ep.acc_out + o, (uint32_t)sum[e]);
+                    float v = __fmul_rn((float)sum[e], __fmul_rn(p_sx[u][e], p_sw));
+                    if (ep.bias) v = __fadd_rn(v, p_bias);
+                    if (ep.residual) v = __fadd_rn(p_res[u][e], v);
+                    if (ep.out_bf16)
+                        store_unseen_b16((uint16_t *)ep.out + o, f32_to_bf16(v));
+                    else
+                        store_unseen_b32<0>((float *)ep.out + o, __float_as_uint(v));
+                }
+            }
         }
     }
 }
@@ -1647,12 +1833,46 @@ void linear_w8a8_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t 
         launch_w8a8_rows<2, kEpiPlain>(m, waves, grid, s, xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e);
 }
 
-// Whether a linear of m rows takes the weight-stationary kernel: more rows than the decode kernels hold, a weight
+// The split-k form of the weight-stationary kernel (w8a8_wstat_ksplit_kernel): deep, narrow weights (k from 8192 up to
+// what four members x eight wavefronts x eight k-tiles hold, about one column tile per compute unit), more rows than
+// the decode kernels take, and a quarter of the activations (m x k / 4 bytes per block) within what a compute unit
+// pulls from L2 in the time of the tiled GEMM.
+namespace {
+struct RowsKsplitPlan {
+    uint32_t n_groups, blocks, row_groups;
+    uint64_t workspace_bytes;
+    bool local;
+};
+inline bool rows_ksplit_plan(uint64_t m, uint32_t n_tiles, uint32_t k_tiles, int num_cus, const SplitKArea *sk, RowsKsplitPlan *p) {
+    if (!sk || !sk->counters || g_rows_kernel == 1 || g_rows_kernel == 2 || g_skinny_ksplit == 1) return false;
+    // (k up to what the kernel without the split holds as well, so that a caller without a workspace still has a form)
+    if (m <= 64 || n_tiles == 0 || k_tiles < 128 || k_tiles > 224) return false;
+    // measured against the tiled GEMM with its k split and the kernel without the split (us incl. the row quantizer, 65 / 128 /
+    // 200 / 300 / 512 rows): 14336 -> 4096 27.7 / 31.6 / 45.4 / 57.8 / 79.3 against 37.6 / 41.8 / 49.3 / 67.7 / 90.7 and 32.7 /
+    // 36.6 / 53.8 / 69.1 / 102; 11008 -> 4096 26.0 / 29.7 / 43.8 / 53.9 / 71.6 against 34.6 / 39.9 / 43.5 / 56.0 / 76.3; at
+    // 8192 -> 4096 the kernel without the split is the faster one while its rule admits it and the three are level above
+    if (g_rows_kernel != 3 && k_tiles < 160) return false;
+    if (g_rows_kernel != 3 && (m > 512 || (uint64_t)n_tiles > 2 * (uint64_t)num_cus)) return false;
+    const uint32_t n_groups = (n_tiles + 3) / 4;
+    if (n_groups > sk->n_counters) return false;
+    p->n_groups = n_groups;
+    p->blocks = 32u * ((n_groups + 7) / 8);                    // whole groups on every XCD; surplus groups return at once
+    p->row_groups = (uint32_t)((m + 31) / 32);
+    p->workspace_bytes = (uint64_t)n_groups * 4 * p->row_groups * (2 * 4 * 4 * 64 * 4);
+    p->local = g_skinny_ksplit == 3 || ((g_skinny_ksplit == 0) && sk->xcd_local);
+    return true;
+}
+}  // namespace
+
+// Whether a linear of m rows takes a weight-stationary kernel: more rows than the decode kernels hold, a weight
 // with at most about two column tiles per compute unit, k within what a wavefront keeps in registers, and a block's
-// activation bytes (m x k, read from L2 once per block) below what the tiled GEMM with its k split costs.
-bool linear_w8a8_rows_applies(uint64_t m, uint64_t n_pad, uint64_t k_pad, int num_cus) {
+// activation bytes (m x k, read from L2 once per block) below what the tiled GEMM with its k split costs.  With a
+// split-k area given, deep weights take the form that splits k over four blocks of an XCD.
+bool linear_w8a8_rows_applies(uint64_t m, uint64_t n_pad, uint64_t k_pad, int num_cus, const SplitKArea *sk) {
     if (g_rows_kernel == 1) return false;
     const uint64_t n_tiles = n_pad / 16, k_tiles = k_pad / 64;
+    RowsKsplitPlan kp;
+    if (rows_ksplit_plan(m, (uint32_t)n_tiles, (uint32_t)k_tiles, num_cus, sk, &kp)) return true;
     if (m <= 64 || n_tiles == 0 || k_tiles == 0 || k_tiles > 224) return false;
     if (g_rows_kernel == 2) return true;
     // measured against the tiled GEMM with its k split (both with their row quantizer, us): 4096 -> 4096 at 65 / 128 / 300 /
@@ -1661,8 +1881,14 @@ bool linear_w8a8_rows_applies(uint64_t m, uint64_t n_pad, uint64_t k_pad, int nu
     return n_tiles <= 2 * (uint64_t)num_cus && m * k_pad <= (2ull << 20);
 }
 
+uint64_t linear_w8a8_rows_workspace_bytes(uint64_t m, uint64_t n_pad, uint64_t k_pad, int num_cus, const SplitKArea *sk) {
+    RowsKsplitPlan kp;
+    return rows_ksplit_plan(m, (uint32_t)(n_pad / 16), (uint32_t)(k_pad / 64), num_cus, sk, &kp) ? kp.workspace_bytes : 0;
+}
+
 void linear_w8a8_rows(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad,
-                      const EpilogueI8 &ep, int num_cus, hipStream_t s) {
+                      const EpilogueI8 &ep, int num_cus, hipStream_t s, const SplitKArea *sk, void *workspace,
+                      uint64_t workspace_bytes) {
     if (m == 0 || n == 0) return;
     EpiI8 e{};
     e.sx = ep.sx;
@@ -1673,6 +1899,28 @@ void linear_w8a8_rows(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t m,
     e.out = ep.out;
     e.out_bf16 = ep.out_bf16;
     const uint32_t n_tiles = (uint32_t)(n_pad / 16), k_tiles = (uint32_t)(k_pad / 64);
+    RowsKsplitPlan kp;
+    if (workspace && rows_ksplit_plan(m, n_tiles, k_tiles, num_cus, sk, &kp) && workspace_bytes >= kp.workspace_bytes) {
+        KsplitPlan as_ks{};
+        as_ks.s = 4;
+        as_ks.n_groups = kp.n_groups;
+        uint32_t *seen = xcc_seen_for(sk, as_ks);
+        auto go = [&](auto ktw, auto ds, auto local) {
+            w8a8_wstat_ksplit_kernel<decltype(ktw)::value, decltype(ds)::value, decltype(local)::value><<<kp.blocks, 512, 0, s>>>(
+                xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, kp.n_groups, e, (int32_t *)workspace, sk->counters, seen,
+                sk->fault);
+        };
+        using std::integral_constant;
+        auto with_local = [&](auto ktw, auto ds) {
+            if (kp.local) go(ktw, ds, std::true_type{});
+            else go(ktw, ds, std::false_type{});
+        };
+        // k-tiles of a wavefront: a quarter of k over eight wavefronts, rounded up
+        const uint32_t per_wave = ((k_tiles + 3) / 4 + 7) / 8;
+        if (per_wave <= 4) with_local(integral_constant<int, 4>{}, integral_constant<int, 4>{});
+        else with_local(integral_constant<int, 7>{}, integral_constant<int, 7>{});      // k_tiles <= 224
+        return;
+    }
     // two column tiles per block once there are more tiles than compute units (every activation tile then feeds two
     // multiplies), where the registers allow it
     const bool two = n_tiles > (uint32_t)num_cus && k_tiles <= 64;

@@ -199,10 +199,17 @@ void linear_w8a16_skinny(const uint16_t *a, const int8_t *w_tiles, const float *
 // A few hundred rows (65 up) against a weight with about one column tile per compute unit: the weight-stationary
 // kernel (weights in registers, rows streamed in groups of 64).  xq_tiled: activation tiles with rows padded to 16,
 // as for linear_w8a8_skinny.  linear_w8a8_rows_applies says whether a shape should take it.
-extern int g_rows_kernel;     // 0: by shape, 1: never (the tiled GEMMs for every prompt pass), 2: whenever it can run
-bool linear_w8a8_rows_applies(uint64_t m, uint64_t n_pad, uint64_t k_pad, int num_cus);
+// With a split-k area (and then a workspace of linear_w8a8_rows_workspace_bytes for the launch), weights with a deep
+// k (8192 .. 14336) take a form that splits k over four blocks of an XCD, each keeping its quarter of the weights in
+// registers: a block then pulls a quarter of the activations.
+// g_rows_kernel: 0: by shape, 1: never (the tiled GEMMs for every prompt pass), 2: the form without the split
+// whenever it can run, 3: the split form whenever it can run
+extern int g_rows_kernel;
+bool linear_w8a8_rows_applies(uint64_t m, uint64_t n_pad, uint64_t k_pad, int num_cus, const SplitKArea *sk = nullptr);
+uint64_t linear_w8a8_rows_workspace_bytes(uint64_t m, uint64_t n_pad, uint64_t k_pad, int num_cus, const SplitKArea *sk);
 void linear_w8a8_rows(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad,
-                      const EpilogueI8 &ep, int num_cus, hipStream_t s);
+                      const EpilogueI8 &ep, int num_cus, hipStream_t s, const SplitKArea *sk = nullptr, void *workspace = nullptr,
+                      uint64_t workspace_bytes = 0);
 
 // ---- prefill-shape MFMA GEMMs (kern_gemm_mfma.hip) -----------------------------
 // aq: int8 [m, k_pad] row-major.  workspace (optional, gemm_w8a8_workspace_bytes): lets a matrix with too few

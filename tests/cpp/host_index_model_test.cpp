@@ -262,7 +262,42 @@ static void ksplit_cases() {
                 }
 }
 
+// The weight-stationary split-k linear: partial tile sets of (group, member, row group) tile its workspace without
+// gaps or overlaps, and the k-tiles of a member's eight wavefronts (step t of wavefront w: lo + w + 8 t) cover the
+// member's range exactly once within the kernel's register depth.
+static void rows_ksplit_cases() {
+    const uint32_t s = 4, nacc = 2 * s * 4;
+    for (uint32_t n_groups : {1u, 8u, 64u, 65u})
+        for (uint32_t row_groups : {3u, 10u, 16u}) {
+            std::set<uint64_t> bases;
+            const uint64_t total = (uint64_t)n_groups * s * row_groups * nacc * 64;
+            for (uint32_t g = 0; g < n_groups; ++g)
+                for (uint32_t m = 0; m < s; ++m)
+                    for (uint32_t rg = 0; rg < row_groups; ++rg) {
+                        const uint64_t base = rows_ksplit_partial_base(g, m, s, row_groups, rg, nacc);
+                        CHECK(base % ((uint64_t)nacc * 64) == 0 && base + (uint64_t)nacc * 64 <= total);
+                        CHECK(bases.insert(base).second);
+                    }
+            CHECK(bases.size() * nacc * 64 == total);
+        }
+    for (uint32_t k_tiles : {128u, 160u, 172u, 224u}) {
+        const uint32_t per_wave = ((k_tiles + 3) / 4 + 7) / 8, ktw = per_wave <= 4 ? 4 : 7;
+        for (uint32_t m = 0; m < s; ++m) {
+            uint32_t lo, hi;
+            ksplit_k_range(k_tiles, m, s, &lo, &hi);
+            std::set<uint32_t> seen;
+            for (uint32_t w = 0; w < 8; ++w) {
+                const uint32_t len = hi - lo, cnt = len > w ? (len - w + 7) / 8 : 0;
+                CHECK(cnt <= ktw);
+                for (uint32_t t = 0; t < cnt; ++t) CHECK(seen.insert(lo + w + 8 * t).second);
+            }
+            CHECK(seen.size() == hi - lo && (seen.empty() || (*seen.begin() == lo && *seen.rbegin() == hi - 1)));
+        }
+    }
+}
+
 int main() {
+    rows_ksplit_cases();
     gemm_case<true, 14, 4>();
     gemm_case<true, 16, 4>();
     gemm_case<false, 14, 4>();

@@ -211,6 +211,47 @@ def test_w8a8_weight_stationary_kernel_for_a_few_hundred_rows(m, k, n):
         fa.check(lib.fa_set_tuning(21, 0))
 
 
+@pytest.mark.parametrize("m,k,n", [(300, 14336, 4096), (65, 8192, 4096), (512, 14336, 1000), (129, 11008, 528), (97, 14336, 16)])
+def test_w8a8_weight_stationary_kernel_with_k_split_over_an_xcd(m, k, n):
+    """Deep, narrow weights under more rows than the decode kernels hold: groups of four blocks keep a quarter of k of
+    four column tiles in registers, every row group's partial sums meet in a workspace and the last arriver of a
+    group finishes all rows (forced for every shape, tuning key 21 = 3; partial tiles exchanged inside the XCD's L2,
+    key 16 = 3, and with agent-scope accesses, key 16 = 2).  Raw sums and outputs bit-exact against the oracle with a
+    bias, f32 and bf16 outputs, ragged rows and columns, both register depths, three calls in a row (the counters
+    return to zero), and equal to the tiled GEMM path (key 21 = 1)."""
+    fa = _fa()
+    be = ops()
+    lib = fa.capi.lib
+    rng = o.Rng(5 * m + n)
+    x = rng.randn((m, k))
+    w = rng.randn((k, n), std=0.02)
+    bias = rng.randn((n,))
+    o.set_threads(8)
+    wq, ws = o.quantize_cols_i8(w)
+    want_acc, want = o.linear_w8a8(x, wq, ws, bias)
+    o.set_threads(1)
+    qw = be.import_quantized_weight(wq, ws)
+    dbias = fa.DeviceBufferView(be.upload(bias), 0, (n,))
+    dx = be.upload(x)
+    try:
+        fa.check(lib.fa_set_tuning(21, 3))
+        for scope in (3, 2):
+            fa.check(lib.fa_set_tuning(16, scope))
+            for rep in range(3):
+                out, acc = be.linear_w8a8(dx, qw, bias=dbias, want_acc=True)
+                assert np.array_equal(be.download_owned(acc), want_acc), (scope, rep)
+                got = be.download_owned(out)
+                assert np.array_equal(got, want), (scope, rep)
+        fa.check(lib.fa_set_tuning(16, 0))
+        out_bf = be.linear_w8a8(dx, qw, bias=dbias, out_dtype=fa.capi.BF16)
+        assert_bf16_rounding_of("w8a8 weight-stationary split-k bf16", be.download_owned(out_bf), got)
+        fa.check(lib.fa_set_tuning(21, 1))
+        assert np.array_equal(be.download_owned(be.linear_w8a8(dx, qw, bias=dbias)), got)
+    finally:
+        fa.check(lib.fa_set_tuning(21, 0))
+        fa.check(lib.fa_set_tuning(16, 0))
+
+
 def test_w8a8_ragged_shapes():
     """Shapes off every tile size, with and without a bias, under one and two column tiles per block and four and
     eight wavefronts (wavefronts without a k-tile, fewer k-tiles than ring slots, a clamped last column tile): the
