@@ -98,6 +98,7 @@ fa_status fa_set_tuning(int32_t key, int32_t value) {
         case 19: k::g_row_fusion = value; return FA_OK;
         case 20: k::g_decode_one = value; return FA_OK;
         case 21: k::g_rows_kernel = value; return FA_OK;
+        case 22: k::g_gemm_swiglu = value; return FA_OK;
     }
     return fail(FA_ERR_INVALID_ARGUMENT, "fa_set_tuning: unknown key");
 }

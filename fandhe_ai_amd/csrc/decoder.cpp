@@ -414,8 +414,15 @@ fa_status enqueue_prefill_chunk(fa_context *ctx, fa_decoder *d, PrefillBuffers &
             k::quantize_rows_i8(t.attn.ptr, true, t.xq.as<int8_t>(), nullptr, t.sx.as<float>(), M, M, L.wo->k, L.wo->k_pad, s);
         gemm(L.wo, t.h.as<float>(), t.h.as<float>());
         norm_quantize((const float *)L.ffn_norm->ptr, L.wgu);
-        gemm(L.wgu, t.gu.as<float>(), nullptr);
-        k::swiglu_quantize_rows_i8(t.gu.as<float>(), t.xq.as<int8_t>(), t.sx.as<float>(), M, F, s, rows_form(L.wdown));
+        // on the large-tile GEMM the gate | up projection takes SwiGLU into its epilogue and leaves the products
+        // ([M, F] instead of [M, 2 F] written and read back); the quantizer behind it is the same either way
+        const bool swiglu_in_gemm = !rows_form(L.wgu) && L.wgu->n == 2 * F && k::gemm_w8a8_swiglu_applies(M, F, L.wgu->n_pad, L.wgu->k_pad);
+        if (swiglu_in_gemm)
+            k::gemm_w8a8_swiglu_mfma(t.xq.as<int8_t>(), (const int8_t *)L.wgu->codes->ptr, t.sx.as<float>(),
+                                     (const float *)L.wgu->scales->ptr, M, F, L.wgu->k_pad, t.gu.as<float>(), s);
+        else
+            gemm(L.wgu, t.gu.as<float>(), nullptr);
+        k::swiglu_quantize_rows_i8(t.gu.as<float>(), t.xq.as<int8_t>(), t.sx.as<float>(), M, F, s, rows_form(L.wdown), swiglu_in_gemm);
         gemm(L.wdown, t.h.as<float>(), t.h.as<float>());
     }
     if (padded) k::trim_seq_lens((uint32_t *)d->seq_lens->ptr, t.row_lens.as<uint32_t>(), B, lc, s);

@@ -86,6 +86,18 @@ FA_HD int big_b_lds_slice(int slot, int tile, int h) {
 template <int NTB>
 FA_HD int big_b_frag_off(int wn, int j, int h, int lane) { return (wn * (NTB / 2) + j) * kBigTile + h * 1024 + lane * 16; }
 
+// SwiGLU form of the large-tile kernel (weight = gate columns, then up columns, f_tiles column tiles each): the block
+// of column index nb owns NTB / 2 tiles of the product; block-local tile `local` = wn * (NTB / 2) + j of wavefront
+// column wn is, for j < NTB / 4, gate tile nb * NTB / 2 + wn * NTB / 4 + j, and for j >= NTB / 4 the up tile of the
+// same product tile as j - NTB / 4: gate and up of an element sit in the same lane of accumulator tiles j and
+// j + NTB / 4.
+template <int NTB>
+FA_HD uint32_t big_swiglu_tile(uint32_t nb, int local, uint32_t f_tiles) {
+    const int wn = local / (NTB / 2), j = local % (NTB / 2);
+    const uint32_t prod_tile = nb * (NTB / 2) + wn * (NTB / 4) + j % (NTB / 4);
+    return (j < NTB / 4 ? 0 : f_tiles) + prod_tile;
+}
+
 // Output element e (0 .. 3) of accumulator tile (i, j) of wavefront (wm, wn) in lane `lane`, block-local: the matrix
 // instructions take the weight fragment first, so a lane holds row lane % 16 and columns 4 (lane / 16) + e.
 template <int NTB, int WM>

@@ -19,6 +19,7 @@ namespace k {
 using namespace fa::dev;
 
 int g_gemm_small_tiles = 0;   // tuning: nonzero keeps the 128 x 128 kernel for every shape
+int g_gemm_swiglu = 0;        // tuning: 1 keeps SwiGLU out of the gate | up GEMM's epilogue (prompt passes)
 int g_gemm_waves = 0;
 int g_gemm_split_fill = 0;    // tuning: blocks per compute unit a split-k launch aims for (default 2)
 int g_gemm_ntb = 0;           // tuning: 14 or 16 fixes the column tiles per large-tile block         // tuning: 4 = four wavefronts per large-tile block instead of eight
@@ -30,6 +31,12 @@ struct EpiI8 {
     int32_t *acc_out;
     void *out;
     int out_bf16;
+};
+// int8, large-tile kernel only: the weight is gate | up (f columns each) and the kernel leaves silu(gate) * up, f32 [m, f]
+struct EpiI8Swiglu {
+    const float *sx, *sw;
+    float *out;
+    uint32_t f;
 };
 struct EpiF8 {
     const float *a_scale, *w_scale;   // one scale each (per-tensor form) ...
@@ -337,6 +344,8 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
     constexpr int A_STAGE = 16 * TILE, B_STAGE = NTB * TILE;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];   // [3][A_STAGE] then [2][B_STAGE]
 
+    constexpr bool SWI = std::is_same<Epi, EpiI8Swiglu>::value;
+    static_assert(!SWI || (!FP8 && NTB % 4 == 0), "the SwiGLU form pairs gate and up tiles inside a wavefront");
     const int tid = threadIdx.x, lane = tid % 64;
     const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
     const int wm = wave / 2, wn = wave % 2;
@@ -375,6 +384,7 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
         // 0, 1 instead (same bytes to the same place, served by the L1), which keeps the main loop
         // free of branches
         uint32_t t = nt0 + ixm::big_b_tile<NTB, NWAVES>(wave, i);
+        if constexpr (SWI) t = ixm::big_swiglu_tile<NTB>(nb, ixm::big_b_tile<NTB, NWAVES>(wave, i), ep.f / 16);
         t = t < n_tiles ? t : n_tiles - 1;
         b_src[i] = w_tiles + (uint64_t)t * k_steps * TILE + ixm::big_b_src_byte<FP8>(lane, 0);
     }
@@ -412,7 +422,7 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
         }
     // the per-tensor scales of the e4m3 epilogue are fetched here, not after the last stage, where the two dependent
     // scalar loads would be a memory round trip that nothing overlaps
-    float fscale = 0.0f;
+    [[maybe_unused]] float fscale = 0.0f;
     if constexpr (FP8) {
         if (ep.sx == nullptr) fscale = __fmul_rn(*ep.a_scale, *ep.w_scale);
     }
@@ -546,6 +556,38 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
     int row_l0, col_l0;                               // block-local row of this lane in row tile 0, first column in tile 0
     ixm::big_out_elem<NTB, WM>(wm, wn, 0, 0, 0, lane, &row_l0, &col_l0);
     const int g = lane / 16;
+    if constexpr (SWI) {
+        // accumulator tiles j and j + WNT / 2 hold gate and up of product tile nb * NTB / 2 + wn * WNT / 2 + j: the
+        // decode step's expressions (dequantize both, silu(gate) * up), four consecutive columns per lane
+        constexpr int HT = WNT / 2;
+        const uint32_t f = ep.f;
+        const uint32_t hc0 = (nb * (NTB / 2) + wn * HT) * 16 + 4 * g;      // this lane's first product column
+        v4f swg[HT], swu[HT];
+#pragma unroll
+        for (int j = 0; j < HT; ++j) {
+            swg[j] = *(const v4f *)(ep.sw + hc0 + j * 16);
+            swu[j] = *(const v4f *)(ep.sw + f + hc0 + j * 16);
+        }
+#pragma unroll
+        for (int i = 0; i < AI; ++i) {
+            const uint32_t row = m0 + row_l0 + i * 16;
+            const bool row_ok = row < m;
+            const float sxr = ep.sx[row_ok ? row : m - 1];
+            float *orow = ep.out + (uint64_t)(row_ok ? row : m - 1) * f + hc0;
+#pragma unroll
+            for (int j = 0; j < HT; ++j) {
+                float v[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float vg = __fmul_rn((float)acc[i][j][e], __fmul_rn(sxr, swg[j][e]));
+                    const float vu = __fmul_rn((float)acc[i][j + HT][e], __fmul_rn(sxr, swu[j][e]));
+                    v[e] = silu_f32(vg) * vu;
+                }
+                if (row_ok) *(v4f *)(orow + j * 16) = v4f{v[0], v[1], v[2], v[3]};
+            }
+        }
+        return;
+    } else {
     bool extras = false, raw_out = false;
     const bool out_bf16 = ep.out_bf16 != 0;
     bool f8_rows = false;
@@ -647,6 +689,7 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
             }
         }
     }
+    }                                                 // !SWI
 }
 
 // Column tiles per block for the large-tile kernel: the width that leaves the fewest idle block slots
@@ -765,6 +808,32 @@ void gemm_w8a8_mfma(const int8_t *aq, const int8_t *w_tiles, uint64_t m, uint64_
         const unsigned blocks = (unsigned)std::min<uint64_t>((quads + 255) / 256, (uint64_t)num_cus * 8);
         splitk_epilogue_i8_kernel<<<blocks, 256, 0, s>>>((const int32_t *)workspace, p.splits, (uint32_t)m, (uint32_t)n, e);
     }
+}
+
+// gate | up projection of a prompt pass with SwiGLU in the epilogue: w_tiles is the [k, 2 f] weight (gate columns first),
+// out receives silu(gate) * up as f32 [m, f], every value what the plain GEMM followed by the SwiGLU pass computes
+// (the same two dequantizations and the same product).  Large-tile kernel only, 256 x 256 block tiles whose column
+// tiles are eight gate tiles and the eight up tiles of the same product columns.
+bool gemm_w8a8_swiglu_applies(uint64_t m, uint64_t f, uint64_t n_pad, uint64_t k_pad) {
+    return g_gemm_swiglu != 1 && !g_gemm_small_tiles && m >= 256 && f != 0 && f % 128 == 0 && n_pad == 2 * f && k_pad != 0 &&
+           k_pad % 128 == 0;
+}
+void gemm_w8a8_swiglu_mfma(const int8_t *aq, const int8_t *w_tiles, const float *sx, const float *sw, uint64_t m, uint64_t f,
+                           uint64_t k_pad, float *out, hipStream_t s) {
+    if (m == 0 || f == 0) return;
+    const EpiI8Swiglu e{sx, sw, out, (uint32_t)f};
+    constexpr int NTB = 16;
+    const size_t smem = (3 * 16 + 2 * (size_t)NTB) * 2048;
+    static bool configured = false;
+    if (!configured) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_mfma_big_kernel<false, NTB, 4, EpiI8Swiglu>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        configured = true;
+    }
+    const uint32_t mb = (uint32_t)((m + 255) / 256), nb = (uint32_t)(f / 128);
+    gemm_mfma_big_kernel<false, NTB, 4, EpiI8Swiglu><<<mb * nb, 512, smem, s>>>((const uint8_t *)aq, (const uint8_t *)w_tiles, (uint32_t)m,
+                                                                              (uint32_t)(2 * f), (uint32_t)(2 * f / 16),
+                                                                              (uint32_t)(k_pad / 128), mb, nb, e);
 }
 
 static void launch_e4m3(const uint8_t *aq, const uint8_t *w_tiles, const EpiF8 &e, uint64_t m, uint64_t n, uint64_t n_pad,

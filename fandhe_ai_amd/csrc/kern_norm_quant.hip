@@ -388,14 +388,28 @@ __global__ void __launch_bounds__(THREADS)
 // writes their codes, so the f32 products never go to memory.  f a multiple of 16.
 // ONE = true: 1024 threads and at most one 16-element chunk per thread (f <= 16384): the products stay in
 // registers between the two passes, so every element is loaded and its exponential taken once.
-template <bool ONE>
+// PROD = true: gu is the products themselves, [m, f] (the gate | up GEMM took SwiGLU into its epilogue): the same
+// quantizer over values that are the same bit for bit.
+template <bool ONE, bool PROD = false>
 __global__ void __launch_bounds__(ONE ? 1024 : kBlock)
     swiglu_quantize_rows_kernel(const float *__restrict__ gu, int8_t *__restrict__ xq_row, float *__restrict__ sx,
                                 uint64_t f, int tiled) {
     constexpr int THREADS = ONE ? 1024 : kBlock;
     __shared__ float smem[THREADS / 64];
     const uint64_t r = blockIdx.x;
-    const float *gate = gu + r * 2 * f, *up = gate + f;
+    const float *gate = gu + r * (PROD ? 1 : 2) * f, *up = gate + f;
+    // the product of chunk c: silu(gate) * up, or the stored product
+    auto products = [&](uint64_t c, float (&p)[16]) {
+        if constexpr (PROD) {
+            load16<false>(gate, c * 16, p);
+        } else {
+            float g[16], u[16];
+            load16<false>(gate, c * 16, g);
+            load16<false>(up, c * 16, u);
+#pragma unroll
+            for (int e = 0; e < 16; ++e) p[e] = silu_f32(g[e]) * u[e];
+        }
+    };
     float amax = 0.0f;
     float prod[16];
     if constexpr (ONE) {
@@ -403,22 +417,16 @@ __global__ void __launch_bounds__(ONE ? 1024 : kBlock)
 #pragma unroll
         for (int e = 0; e < 16; ++e) prod[e] = 0.0f;
         if (c < f / 16) {
-            float g[16], u[16];
-            load16<false>(gate, c * 16, g);
-            load16<false>(up, c * 16, u);
+            products(c, prod);
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                prod[e] = silu_f32(g[e]) * u[e];
-                amax = fmaxf(amax, fabsf(prod[e]));
-            }
+            for (int e = 0; e < 16; ++e) amax = fmaxf(amax, fabsf(prod[e]));
         }
     } else {
         for (uint64_t c = threadIdx.x; c < f / 16; c += THREADS) {
-            float g[16], u[16];
-            load16<false>(gate, c * 16, g);
-            load16<false>(up, c * 16, u);
+            float pr[16];
+            products(c, pr);
 #pragma unroll
-            for (int e = 0; e < 16; ++e) amax = fmaxf(amax, fabsf(silu_f32(g[e]) * u[e]));
+            for (int e = 0; e < 16; ++e) amax = fmaxf(amax, fabsf(pr[e]));
         }
     }
     amax = block_max<THREADS / 64>(amax, smem);
@@ -434,13 +442,11 @@ __global__ void __launch_bounds__(ONE ? 1024 : kBlock)
         }
     } else {
         for (uint64_t c = threadIdx.x; c < f / 16; c += THREADS) {
-            float g[16], u[16];
-            load16<false>(gate, c * 16, g);
-            load16<false>(up, c * 16, u);
+            float pr[16];
+            products(c, pr);
             uint32_t words[4] = {0, 0, 0, 0};
 #pragma unroll
-            for (int e = 0; e < 16; ++e)
-                words[e / 4] |= ((uint32_t)quant_i8(silu_f32(g[e]) * u[e], scale) & 0xffu) << (8 * (e % 4));
+            for (int e = 0; e < 16; ++e) words[e / 4] |= ((uint32_t)quant_i8(pr[e], scale) & 0xffu) << (8 * (e % 4));
             *(v4u *)(xq_row + (tiled ? tiled_chunk_offset(r, c, f / 64) : r * f + c * 16)) = v4u{words[0], words[1], words[2], words[3]};
         }
     }
@@ -634,8 +640,16 @@ void rmsnorm_quantize_rows_i8(const float *x, const float *w, float eps, int8_t 
         rmsnorm_quantize_kernel<4, true><<<grid, kBlock, 0, s>>>(x, w, eps, inv_n, nullptr, xq_rowmajor, sx, m, hidden, grid, WeightPrefetch{});
 }
 
-void swiglu_quantize_rows_i8(const float *gu, int8_t *xq, float *sx, uint64_t m, uint64_t f, hipStream_t s, bool tiled) {
+void swiglu_quantize_rows_i8(const float *gu, int8_t *xq, float *sx, uint64_t m, uint64_t f, hipStream_t s, bool tiled,
+                             bool products) {
     if (m == 0 || f == 0) return;
+    if (products) {
+        if (f <= 16384)
+            swiglu_quantize_rows_kernel<true, true><<<(unsigned)m, 1024, 0, s>>>(gu, xq, sx, f, tiled ? 1 : 0);
+        else
+            swiglu_quantize_rows_kernel<false, true><<<(unsigned)m, kBlock, 0, s>>>(gu, xq, sx, f, tiled ? 1 : 0);
+        return;
+    }
     if (f <= 16384)
         swiglu_quantize_rows_kernel<true><<<(unsigned)m, 1024, 0, s>>>(gu, xq, sx, f, tiled ? 1 : 0);
     else

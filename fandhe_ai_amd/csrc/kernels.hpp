@@ -74,9 +74,9 @@ void rmsnorm_quantize_rows_i8(const float *x, const float *w, float eps, int8_t 
                               uint64_t hidden, hipStream_t s);
 // act = silu(gate) * up of gu [m, 2 f] (gate columns first) quantized per token, row-major codes [m, f] or
 // (tiled, f a multiple of 64) activation tiles with rows padded to 16; the f32 products are not stored.  f a
-// multiple of 16.
+// multiple of 16.  products: gu is [m, f] and holds the products already (gemm_w8a8_swiglu_mfma), only the quantizer runs.
 void swiglu_quantize_rows_i8(const float *gu, int8_t *xq, float *sx, uint64_t m, uint64_t f, hipStream_t s,
-                             bool tiled = false);
+                             bool tiled = false, bool products = false);
 // Per-tensor absmax -> scale = absmax / 448 (one f32) then e4m3 codes.
 void quantize_tensor_e4m3(const float *x, uint8_t *q, float *scale, float *absmax_scratch, uint64_t n,
                           hipStream_t s);
@@ -219,6 +219,13 @@ void gemm_w8a8_mfma(const int8_t *aq, const int8_t *w_tiles, uint64_t m, uint64_
                     uint64_t k_pad, const EpilogueI8 &ep, int num_cus, hipStream_t s, void *workspace = nullptr,
                     uint64_t workspace_bytes = 0);
 uint64_t gemm_w8a8_workspace_bytes(uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad, int num_cus);
+// The gate | up projection with SwiGLU in its epilogue (large-tile kernel, m >= 256, f a multiple of 128, k_pad of 128):
+// w_tiles is the [k, 2 f] weight with the gate columns first; out receives silu(gate) * up, f32 [m, f], bit for bit
+// what gemm_w8a8_mfma into an [m, 2 f] buffer followed by the SwiGLU pass computes.
+extern int g_gemm_swiglu;     // 1: never (the plain GEMM and the SwiGLU pass of the row quantizer)
+bool gemm_w8a8_swiglu_applies(uint64_t m, uint64_t f, uint64_t n_pad, uint64_t k_pad);
+void gemm_w8a8_swiglu_mfma(const int8_t *aq, const int8_t *w_tiles, const float *sx, const float *sw, uint64_t m, uint64_t f,
+                           uint64_t k_pad, float *out, hipStream_t s);
 // Which kernel the two launchers pick for a shape under the current tuning knobs: big_ntb column tiles of
 // 16 per block of the large-tile kernel (0: the 128 x 128 kernel), wavefronts per block, k splits.
 struct GemmPlan {

@@ -296,7 +296,27 @@ static void rows_ksplit_cases() {
     }
 }
 
+// SwiGLU form of the large-tile kernel: over all blocks every gate tile and every up tile of the weight is taken exactly
+// once, and accumulator tiles j and j + NTB / 4 of a wavefront column are gate and up of the same product tile.
+template <int NTB>
+static void swiglu_tile_case(uint32_t f_tiles) {
+    std::set<uint32_t> seen;
+    const uint32_t n_blocks = f_tiles / (NTB / 2);
+    for (uint32_t nb = 0; nb < n_blocks; ++nb)
+        for (int wn = 0; wn < 2; ++wn)
+            for (int j = 0; j < NTB / 4; ++j) {
+                const uint32_t g = big_swiglu_tile<NTB>(nb, wn * (NTB / 2) + j, f_tiles);
+                const uint32_t u = big_swiglu_tile<NTB>(nb, wn * (NTB / 2) + j + NTB / 4, f_tiles);
+                CHECK(g < f_tiles && u == g + f_tiles);
+                CHECK(g == nb * (NTB / 2) + wn * (NTB / 4) + j);           // the product tile the epilogue writes
+                CHECK(seen.insert(g).second && seen.insert(u).second);
+            }
+    CHECK(seen.size() == 2 * (size_t)f_tiles);
+}
+
 int main() {
+    swiglu_tile_case<16>(8);
+    swiglu_tile_case<16>(896);
     rows_ksplit_cases();
     gemm_case<true, 14, 4>();
     gemm_case<true, 16, 4>();

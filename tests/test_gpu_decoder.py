@@ -323,9 +323,11 @@ def test_prompt_prefill_matches_the_oracle_decoding_the_prompt_token_by_token(sh
 
 def test_prompt_pass_on_large_tiles_equals_the_pass_on_128_tiles_bit_for_bit():
     """The projections of a prompt pass on the large-tile GEMM (forced: 256 x 224 tiles; its epilogue adds the
-    residual of the o and down projections from registers, four outputs of a row per lane) against the same pass on
-    the 128 x 128 kernel (its own epilogue code): int32 sums are exact and both epilogues apply scale, then
-    residual, in the same order, so logits, tokens and every cache row must be identical."""
+    residual of the o and down projections from registers, four outputs of a row per lane, and the gate | up
+    projection takes SwiGLU into its epilogue) against the same pass with SwiGLU left to the row quantizer and against
+    the pass on the 128 x 128 kernel (its own epilogue code): int32 sums are exact, the epilogues apply scale, then
+    residual, in the same order, and the products are the same expressions of the same values, so logits, tokens and
+    every cache row must be identical."""
     import fandhe_ai_amd as fa
     be = ops()
     lib = fa.capi.lib
@@ -335,23 +337,30 @@ def test_prompt_pass_on_large_tiles_equals_the_pass_on_128_tiles_bit_for_bit():
     prompt = o.Rng(6).randint(0, shape["vocab"], shape["batch"] * l_new).astype(np.int32).reshape(shape["batch"], l_new)
     got = {}
     try:
-        for big in (True, False):
-            fa.check(lib.fa_set_tuning(7, 14 if big else 0))
-            fa.check(lib.fa_set_tuning(4, 0 if big else 1))
+        # "big": large tiles, the gate | up GEMM with SwiGLU in its epilogue (256 x 256 tiles of eight gate and eight
+        # up column tiles, products written); "plain": large tiles, SwiGLU left to the row quantizer (key 22 = 1);
+        # "small": the 128 x 128 kernel everywhere
+        for form in ("big", "plain", "small"):
+            fa.check(lib.fa_set_tuning(7, 0 if form == "small" else 14))
+            fa.check(lib.fa_set_tuning(4, 1 if form == "small" else 0))
+            fa.check(lib.fa_set_tuning(22, 1 if form == "plain" else 0))
             dec = GpuDecoder(be, m)
             try:
                 dec.prefill(prompt)
-                got[big] = (dec.logits().copy(), dec.tokens().copy(), [tuple(x.copy() for x in dec.kv_pool(li)) for li in range(2)])
+                got[form] = (dec.logits().copy(), dec.tokens().copy(), [tuple(x.copy() for x in dec.kv_pool(li)) for li in range(2)])
             finally:
                 dec.close()
     finally:
         fa.check(lib.fa_set_tuning(7, 0))
         fa.check(lib.fa_set_tuning(4, 0))
-    a, b = got[True], got[False]
+        fa.check(lib.fa_set_tuning(22, 0))
+    a = got["big"]
     assert np.all(np.isfinite(a[0])) and np.any(a[0] != 0)
-    assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1])
-    for (ak, av), (bk, bv) in zip(a[2], b[2]):
-        assert np.array_equal(ak, bk) and np.array_equal(av, bv)
+    for other in ("plain", "small"):
+        b = got[other]
+        assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1]), other
+        for (ak, av), (bk, bv) in zip(a[2], b[2]):
+            assert np.array_equal(ak, bk) and np.array_equal(av, bv), other
 
 
 @pytest.mark.parametrize("batch,l_new", [(1, 70), (3, 100), (2, 33)], ids=["70-rows", "300-rows", "66-rows"])
