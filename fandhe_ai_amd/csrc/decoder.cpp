@@ -400,10 +400,19 @@ fa_status enqueue_prefill_chunk(fa_context *ctx, fa_decoder *d, PrefillBuffers &
     for (uint32_t li = 0; li < c.n_layers; ++li) {
         const fa_decoder::Layer &L = d->layers[li];
         norm_quantize((const float *)L.attn_norm->ptr, L.wqkv);
-        gemm(L.wqkv, t.qkv.as<float>(), nullptr);
-        k::rope_append(t.qkv.as<float>(), t.cos_sin.as<float>(), t.slots.as<uint32_t>(), t.q_bf.as<uint16_t>(),
-                       (uint16_t *)L.k_pool->ptr, (uint16_t *)L.v_pool->ptr, M, c.n_heads, c.n_kv_heads, c.head_dim,
-                       pool_rows, s);
+        // on the large-tile GEMM the q | k | v projection does RoPE, the bf16 rounding and the K / V append in its epilogue
+        if (!rows_form(L.wqkv) &&
+            k::gemm_w8a8_qkv_rope_applies(M, L.wqkv->n, L.wqkv->n_pad, L.wqkv->k_pad, c.n_heads, c.n_kv_heads, c.head_dim, cus)) {
+            const k::QkvRopeTargets qt{t.cos_sin.as<float>(), t.slots.as<uint32_t>(), t.q_bf.as<uint16_t>(), (uint16_t *)L.k_pool->ptr,
+                                       (uint16_t *)L.v_pool->ptr, c.n_heads, c.n_kv_heads, c.head_dim, pool_rows};
+            k::gemm_w8a8_qkv_rope_mfma(t.xq.as<int8_t>(), (const int8_t *)L.wqkv->codes->ptr, t.sx.as<float>(),
+                                       (const float *)L.wqkv->scales->ptr, M, L.wqkv->k_pad, qt, s);
+        } else {
+            gemm(L.wqkv, t.qkv.as<float>(), nullptr);
+            k::rope_append(t.qkv.as<float>(), t.cos_sin.as<float>(), t.slots.as<uint32_t>(), t.q_bf.as<uint16_t>(),
+                           (uint16_t *)L.k_pool->ptr, (uint16_t *)L.v_pool->ptr, M, c.n_heads, c.n_kv_heads, c.head_dim,
+                           pool_rows, s);
+        }
         k::paged_attention_prefill_bf16(t.q_bf.as<uint16_t>(), (const uint16_t *)L.k_pool->ptr,
                                         (const uint16_t *)L.v_pool->ptr, (const uint32_t *)d->tables->ptr,
                                         (const uint32_t *)d->seq_lens->ptr, ps, (uint32_t)g_decode_waves, ctx->workspace,

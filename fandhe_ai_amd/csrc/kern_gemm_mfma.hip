@@ -19,7 +19,8 @@ namespace k {
 using namespace fa::dev;
 
 int g_gemm_small_tiles = 0;   // tuning: nonzero keeps the 128 x 128 kernel for every shape
-int g_gemm_swiglu = 0;        // tuning: 1 keeps SwiGLU out of the gate | up GEMM's epilogue (prompt passes)
+int g_gemm_swiglu = 0;        // tuning, prompt passes: bit 0 keeps SwiGLU out of the gate | up GEMM's epilogue, bit 1 RoPE
+                              // and the K / V append out of the q | k | v GEMM's
 int g_gemm_waves = 0;
 int g_gemm_split_fill = 0;    // tuning: blocks per compute unit a split-k launch aims for (default 2)
 int g_gemm_ntb = 0;           // tuning: 14 or 16 fixes the column tiles per large-tile block         // tuning: 4 = four wavefronts per large-tile block instead of eight
@@ -37,6 +38,15 @@ struct EpiI8Swiglu {
     const float *sx, *sw;
     float *out;
     uint32_t f;
+};
+// int8, large-tile kernel only: the weight is q | k | v (heads of 128 dims) and the kernel leaves what the plain GEMM followed
+// by the RoPE + append pass leaves: q rotated, bf16 [m, heads * 128]; K rotated and V as they are, bf16, in pool row slots[r]
+struct EpiI8QkvRope {
+    const float *sx, *sw, *cos_sin;
+    const uint32_t *slots;
+    uint16_t *q_out, *k_pool, *v_pool;
+    uint32_t heads, kv_heads;
+    uint64_t pool_rows;
 };
 struct EpiF8 {
     const float *a_scale, *w_scale;   // one scale each (per-tensor form) ...
@@ -344,8 +354,9 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
     constexpr int A_STAGE = 16 * TILE, B_STAGE = NTB * TILE;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];   // [3][A_STAGE] then [2][B_STAGE]
 
-    constexpr bool SWI = std::is_same<Epi, EpiI8Swiglu>::value;
+    constexpr bool SWI = std::is_same<Epi, EpiI8Swiglu>::value, ROPE = std::is_same<Epi, EpiI8QkvRope>::value;
     static_assert(!SWI || (!FP8 && NTB % 4 == 0), "the SwiGLU form pairs gate and up tiles inside a wavefront");
+    static_assert(!ROPE || (!FP8 && NTB == 16), "the RoPE form: a head of 128 dims is the eight column tiles of one wavefront");
     const int tid = threadIdx.x, lane = tid % 64;
     const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
     const int wm = wave / 2, wn = wave % 2;
@@ -556,7 +567,64 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
     int row_l0, col_l0;                               // block-local row of this lane in row tile 0, first column in tile 0
     ixm::big_out_elem<NTB, WM>(wm, wn, 0, 0, 0, lane, &row_l0, &col_l0);
     const int g = lane / 16;
-    if constexpr (SWI) {
+    if constexpr (ROPE) {
+        // The eight column tiles of this wavefront are head hd = 2 nb + wn of q | k | v; tiles j and j + 4 hold dims d
+        // and d + 64 of the rotate-half pairs (four consecutive d per lane).  The arithmetic is rope_append's: dequantize,
+        // x0 c - x1 s and x1 c + x0 s with explicit roundings, one rounding to bf16.
+        const uint32_t hd = nb * 2 + wn, heads = ep.heads, kv = ep.kv_heads;
+        const uint64_t eq = (uint64_t)heads * 128, ekv = (uint64_t)kv * 128;
+        const uint32_t c0 = hd * 128 + 4 * g;                              // this lane's first column in tile 0
+        v4f sw0[4], sw1[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            sw0[j] = *(const v4f *)(ep.sw + c0 + j * 16);
+            sw1[j] = *(const v4f *)(ep.sw + c0 + 64 + j * 16);
+        }
+#pragma unroll
+        for (int i = 0; i < AI; ++i) {
+            const uint32_t row = m0 + row_l0 + i * 16;
+            const bool row_ok = row < m;
+            const uint32_t rc = row_ok ? row : m - 1;
+            const float sxr = ep.sx[rc];
+            uint16_t *dst = nullptr;
+            if (hd < heads) {
+                dst = ep.q_out + (uint64_t)rc * eq + (uint64_t)hd * 128;
+            } else {
+                const uint64_t slot = ep.slots[rc];
+                if (slot < ep.pool_rows)
+                    dst = hd < heads + kv ? ep.k_pool + slot * ekv + (uint64_t)(hd - heads) * 128
+                                          : ep.v_pool + slot * ekv + (uint64_t)(hd - heads - kv) * 128;
+            }
+            const bool rotate = hd < heads + kv;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                v4f cs = v4f{0.f, 0.f, 0.f, 0.f}, sn = cs;
+                if (rotate) {
+                    cs = *(const v4f *)(ep.cos_sin + (uint64_t)rc * 128 + j * 16 + 4 * g);
+                    sn = *(const v4f *)(ep.cos_sin + (uint64_t)rc * 128 + 64 + j * 16 + 4 * g);
+                }
+                float y0[4], y1[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float x0 = __fmul_rn((float)acc[i][j][e], __fmul_rn(sxr, sw0[j][e]));
+                    float x1 = __fmul_rn((float)acc[i][j + 4][e], __fmul_rn(sxr, sw1[j][e]));
+                    if (rotate) {
+                        const float r0 = __fsub_rn(__fmul_rn(x0, cs[e]), __fmul_rn(x1, sn[e]));
+                        const float r1 = __fadd_rn(__fmul_rn(x1, cs[e]), __fmul_rn(x0, sn[e]));
+                        x0 = r0;
+                        x1 = r1;
+                    }
+                    y0[e] = x0;
+                    y1[e] = x1;
+                }
+                if (row_ok && dst) {
+                    *(v2u *)(dst + j * 16 + 4 * g) = v2u{f32x2_to_bf16x2(y0[0], y0[1]), f32x2_to_bf16x2(y0[2], y0[3])};
+                    *(v2u *)(dst + 64 + j * 16 + 4 * g) = v2u{f32x2_to_bf16x2(y1[0], y1[1]), f32x2_to_bf16x2(y1[2], y1[3])};
+                }
+            }
+        }
+        return;
+    } else if constexpr (SWI) {
         // accumulator tiles j and j + WNT / 2 hold gate and up of product tile nb * NTB / 2 + wn * WNT / 2 + j: the
         // decode step's expressions (dequantize both, silu(gate) * up), four consecutive columns per lane
         constexpr int HT = WNT / 2;
@@ -815,7 +883,7 @@ void gemm_w8a8_mfma(const int8_t *aq, const int8_t *w_tiles, uint64_t m, uint64_
 // (the same two dequantizations and the same product).  Large-tile kernel only, 256 x 256 block tiles whose column
 // tiles are eight gate tiles and the eight up tiles of the same product columns.
 bool gemm_w8a8_swiglu_applies(uint64_t m, uint64_t f, uint64_t n_pad, uint64_t k_pad) {
-    return g_gemm_swiglu != 1 && !g_gemm_small_tiles && m >= 256 && f != 0 && f % 128 == 0 && n_pad == 2 * f && k_pad != 0 &&
+    return !(g_gemm_swiglu & 1) && !g_gemm_small_tiles && m >= 256 && f != 0 && f % 128 == 0 && n_pad == 2 * f && k_pad != 0 &&
            k_pad % 128 == 0;
 }
 void gemm_w8a8_swiglu_mfma(const int8_t *aq, const int8_t *w_tiles, const float *sx, const float *sw, uint64_t m, uint64_t f,
@@ -834,6 +902,34 @@ void gemm_w8a8_swiglu_mfma(const int8_t *aq, const int8_t *w_tiles, const float 
     gemm_mfma_big_kernel<false, NTB, 4, EpiI8Swiglu><<<mb * nb, 512, smem, s>>>((const uint8_t *)aq, (const uint8_t *)w_tiles, (uint32_t)m,
                                                                               (uint32_t)(2 * f), (uint32_t)(2 * f / 16),
                                                                               (uint32_t)(k_pad / 128), mb, nb, e);
+}
+
+// q | k | v projection of a prompt pass with RoPE, the bf16 rounding and the K / V append in the epilogue (heads of 128 dims:
+// a head is the eight column tiles of one wavefront of a 256 x 256 block tile).  Taken where the plain GEMM would run on the
+// large-tile kernel too.
+bool gemm_w8a8_qkv_rope_applies(uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad, uint32_t heads, uint32_t kv_heads,
+                                uint32_t head_dim, int num_cus) {
+    if ((g_gemm_swiglu & 2) || g_gemm_small_tiles || head_dim != 128 || m < 256 || k_pad == 0 || k_pad % 128) return false;
+    if (n != (uint64_t)(heads + 2 * kv_heads) * 128 || n_pad != n || (heads + 2 * kv_heads) % 2) return false;
+    return pick_big_ntb(m, n_pad / 16, num_cus) != 0;
+}
+void gemm_w8a8_qkv_rope_mfma(const int8_t *aq, const int8_t *w_tiles, const float *sx, const float *sw, uint64_t m, uint64_t k_pad,
+                             const QkvRopeTargets &t, hipStream_t s) {
+    if (m == 0) return;
+    const EpiI8QkvRope e{sx, sw, t.cos_sin, t.slots, t.q_out, t.k_pool, t.v_pool, t.heads, t.kv_heads, t.pool_rows};
+    constexpr int NTB = 16;
+    const size_t smem = (3 * 16 + 2 * (size_t)NTB) * 2048;
+    static bool configured = false;
+    if (!configured) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_mfma_big_kernel<false, NTB, 4, EpiI8QkvRope>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        configured = true;
+    }
+    const uint64_t n = (uint64_t)(t.heads + 2 * t.kv_heads) * 128;
+    const uint32_t mb = (uint32_t)((m + 255) / 256), nb = (uint32_t)(n / 256);
+    gemm_mfma_big_kernel<false, NTB, 4, EpiI8QkvRope><<<mb * nb, 512, smem, s>>>((const uint8_t *)aq, (const uint8_t *)w_tiles,
+                                                                               (uint32_t)m, (uint32_t)n, (uint32_t)(n / 16),
+                                                                               (uint32_t)(k_pad / 128), mb, nb, e);
 }
 
 static void launch_e4m3(const uint8_t *aq, const uint8_t *w_tiles, const EpiF8 &e, uint64_t m, uint64_t n, uint64_t n_pad,

@@ -191,6 +191,12 @@ struct QkvRopeTargets {
 void linear_w8a8_qkv_rope_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, const float *sx, const float *sw,
                                  uint64_t m, uint64_t n_pad, uint64_t k_pad, const QkvRopeTargets &t, hipStream_t s,
                                  const RowPrologue *pro = nullptr);
+// The q | k | v projection of a prompt pass on the large-tile GEMM with rope_append's work in its epilogue (aq row-major
+// codes): bit for bit what gemm_w8a8_mfma into an [m, n] f32 buffer followed by rope_append leaves in q_out and the pools.
+bool gemm_w8a8_qkv_rope_applies(uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad, uint32_t heads, uint32_t kv_heads,
+                                uint32_t head_dim, int num_cus);
+void gemm_w8a8_qkv_rope_mfma(const int8_t *aq, const int8_t *w_tiles, const float *sx, const float *sw, uint64_t m, uint64_t k_pad,
+                             const QkvRopeTargets &t, hipStream_t s);
 // a: bf16 [m, k] row-major (k == k_pad required), m <= 32.
 void linear_w8a16_skinny(const uint16_t *a, const int8_t *w_tiles, const float *sw, uint64_t m,
                          uint64_t n, uint64_t n_pad, uint64_t k_pad, void *out, int out_bf16,
@@ -222,7 +228,7 @@ uint64_t gemm_w8a8_workspace_bytes(uint64_t m, uint64_t n, uint64_t n_pad, uint6
 // The gate | up projection with SwiGLU in its epilogue (large-tile kernel, m >= 256, f a multiple of 128, k_pad of 128):
 // w_tiles is the [k, 2 f] weight with the gate columns first; out receives silu(gate) * up, f32 [m, f], bit for bit
 // what gemm_w8a8_mfma into an [m, 2 f] buffer followed by the SwiGLU pass computes.
-extern int g_gemm_swiglu;     // 1: never (the plain GEMM and the SwiGLU pass of the row quantizer)
+extern int g_gemm_swiglu;     // bit 0: SwiGLU stays a pass of its own; bit 1: so do RoPE and the K / V append (below)
 bool gemm_w8a8_swiglu_applies(uint64_t m, uint64_t f, uint64_t n_pad, uint64_t k_pad);
 void gemm_w8a8_swiglu_mfma(const int8_t *aq, const int8_t *w_tiles, const float *sx, const float *sw, uint64_t m, uint64_t f,
                            uint64_t k_pad, float *out, hipStream_t s);

@@ -95,8 +95,10 @@ fa_status fa_probe_l2_path(fa_context *ctx, const fa_buffer *cold, uint64_t cold
  *        compute unit, m x k at most 2 MiB; k of 8192 .. 14336: the form that splits k over four blocks of an XCD,
  *        up to 512 rows) and the decode kernels for prompt passes of at most 64 rows, 1 the tiled GEMMs always, 2 the
  *        weight-stationary kernel without the split whenever it can run, 3 the split form whenever it can run;
- * key 22: 1 keeps SwiGLU out of the epilogue of the gate | up GEMM of prompt passes (the plain GEMM into [rows, 2 d_ffn]
- *        and the SwiGLU pass of the row quantizer); 0: on the large-tile kernel the GEMM leaves the products. */
+ * key 22: prompt passes on the large-tile GEMM, bits: 1 keeps SwiGLU out of the epilogue of the gate | up GEMM (the plain
+ *        GEMM into [rows, 2 d_ffn] and the SwiGLU pass of the row quantizer), 2 keeps RoPE, the bf16 rounding and the K / V
+ *        append out of the epilogue of the q | k | v GEMM (the plain GEMM and the RoPE + append pass); 0: both in the
+ *        epilogues. */
 fa_status fa_set_tuning(int32_t key, int32_t value);
 
 /* What the context found when it was created: xcd_local = 1 when workgroups b and b + 8 of a launch were seen to

@@ -323,8 +323,9 @@ def test_prompt_prefill_matches_the_oracle_decoding_the_prompt_token_by_token(sh
 
 def test_prompt_pass_on_large_tiles_equals_the_pass_on_128_tiles_bit_for_bit():
     """The projections of a prompt pass on the large-tile GEMM (forced: 256 x 224 tiles; its epilogue adds the
-    residual of the o and down projections from registers, four outputs of a row per lane, and the gate | up
-    projection takes SwiGLU into its epilogue) against the same pass with SwiGLU left to the row quantizer and against
+    residual of the o and down projections from registers, four outputs of a row per lane, the gate | up projection
+    takes SwiGLU into its epilogue and the q | k | v projection RoPE and the K / V append) against the same pass with
+    SwiGLU left to the row quantizer and RoPE to its own pass, and against
     the pass on the 128 x 128 kernel (its own epilogue code): int32 sums are exact, the epilogues apply scale, then
     residual, in the same order, and the products are the same expressions of the same values, so logits, tokens and
     every cache row must be identical."""
@@ -338,12 +339,13 @@ def test_prompt_pass_on_large_tiles_equals_the_pass_on_128_tiles_bit_for_bit():
     got = {}
     try:
         # "big": large tiles, the gate | up GEMM with SwiGLU in its epilogue (256 x 256 tiles of eight gate and eight
-        # up column tiles, products written); "plain": large tiles, SwiGLU left to the row quantizer (key 22 = 1);
+        # up column tiles, products written) and the q | k | v GEMM with RoPE, the bf16 rounding and the K / V append
+        # in its epilogue (a head per wavefront); "plain": large tiles, both left to their own passes (key 22 = 3);
         # "small": the 128 x 128 kernel everywhere
         for form in ("big", "plain", "small"):
             fa.check(lib.fa_set_tuning(7, 0 if form == "small" else 14))
             fa.check(lib.fa_set_tuning(4, 1 if form == "small" else 0))
-            fa.check(lib.fa_set_tuning(22, 1 if form == "plain" else 0))
+            fa.check(lib.fa_set_tuning(22, 3 if form == "plain" else 0))
             dec = GpuDecoder(be, m)
             try:
                 dec.prefill(prompt)
