@@ -19,7 +19,7 @@ extern int g_skinny_ntw, g_skinny_waves, g_skinny_astat, g_gemm_small_tiles, g_g
 }
 int g_decode_waves = 0;
 int g_prefill_generic = 0;
-extern int g_decode_partials_only, g_prefill_block_form, g_prefill_block_waves, g_prefill_block_split;
+extern int g_decode_partials_only, g_prefill_block_form, g_prefill_block_waves, g_prefill_block_split, g_prefill_block_cols;
 }  // namespace fa
 
 namespace {
@@ -99,6 +99,7 @@ fa_status fa_set_tuning(int32_t key, int32_t value) {
         case 20: k::g_decode_one = value; return FA_OK;
         case 21: k::g_rows_kernel = value; return FA_OK;
         case 22: k::g_gemm_swiglu = value; return FA_OK;
+        case 23: fa::g_prefill_block_cols = value; return FA_OK;
     }
     return fail(FA_ERR_INVALID_ARGUMENT, "fa_set_tuning: unknown key");
 }

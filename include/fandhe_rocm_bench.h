@@ -98,7 +98,9 @@ fa_status fa_probe_l2_path(fa_context *ctx, const fa_buffer *cold, uint64_t cold
  * key 22: prompt passes on the large-tile GEMM, bits: 1 keeps SwiGLU out of the epilogue of the gate | up GEMM (the plain
  *        GEMM into [rows, 2 d_ffn] and the SwiGLU pass of the row quantizer), 2 keeps RoPE, the bf16 rounding and the K / V
  *        append out of the epilogue of the q | k | v GEMM (the plain GEMM and the RoPE + append pass); 0: both in the
- *        epilogues. */
+ *        epilogues;
+ * key 23: columns (new token x head) per wavefront of the block form of the prefill attention: 0 by shape (16 while
+ *        blocks of 32 would not fill the device more than once, else 32), 1: 16 whenever the form allows, 2: 32. */
 fa_status fa_set_tuning(int32_t key, int32_t value);
 
 /* What the context found when it was created: xcd_local = 1 when workgroups b and b + 8 of a launch were seen to

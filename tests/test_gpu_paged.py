@@ -285,11 +285,13 @@ def test_bf16_prefill_on_the_streaming_kernel_against_the_oracle(heads, kv_heads
     fa.check(fa.capi.lib.fa_set_tuning(10, 2))
     # tiles of 256 / group and of 128 / group new tokens; the smaller blocks also with the cache walk of a tile
     # shared by several blocks (as many as the shape allows, or two) and a merge pass
-    for block_waves, split in ((8, 1), (4, 1), (4, 0), (4, 2)):
+    # (cols: 32 columns per wavefront, key 23 = 2, or 16, key 23 = 1: half the multiplies per step, twice the blocks)
+    for block_waves, split, cols in ((8, 1, 2), (4, 1, 2), (4, 1, 1), (4, 0, 2), (4, 2, 2)):
         fa.check(fa.capi.lib.fa_set_tuning(11, block_waves))
         fa.check(fa.capi.lib.fa_set_tuning(12, split))
+        fa.check(fa.capi.lib.fa_set_tuning(23, cols))
         blk = be.download_owned(be.paged_attention_forward(dq, dk, dv, tables, seq_lens, args, out_dtype=fa.capi.F32))
-        assert_parity("PAGED_PREFILL_PARITY", f"H{heads}/{kv_heads}:L{l_new}:block form, {block_waves} wavefronts, split {split}", blk, want)
+        assert_parity("PAGED_PREFILL_PARITY", f"H{heads}/{kv_heads}:L{l_new}:block form, {block_waves} wavefronts, split {split}, cols {cols}", blk, want)
         blk_bf = be.download_owned(be.paged_attention_forward(dq, dk, dv, tables, seq_lens, args))
         assert_bf16_rounding_of("paged prefill bf16, block form", blk_bf, blk)
         blk_dev = be.download_owned(be.paged_attention_forward_device(dq, dk, dv, be.upload(tables), be.upload(seq_lens), args,
@@ -303,6 +305,7 @@ def test_bf16_prefill_on_the_streaming_kernel_against_the_oracle(heads, kv_heads
             assert np.array_equal(blk_bf[0, 0, h * 128:(h + 1) * 128], vp[tables[0, 0], 0, gq * 128:(gq + 1) * 128])
     fa.check(fa.capi.lib.fa_set_tuning(11, 0))
     fa.check(fa.capi.lib.fa_set_tuning(12, 0))
+    fa.check(fa.capi.lib.fa_set_tuning(23, 0))
     # whatever the shape selects by itself (host tables: the longest row is known; device tables: the table width)
     fa.check(fa.capi.lib.fa_set_tuning(10, 0))
     auto = be.download_owned(be.paged_attention_forward(dq, dk, dv, tables, seq_lens, args, out_dtype=fa.capi.F32))
@@ -434,9 +437,10 @@ def test_block_form_prefill_flags_violations_per_column():
     bad_l[2] = l_new - 1                            # row 2: fewer positions than new tokens
     fa.check(fa.capi.lib.fa_set_tuning(10, 2))
     try:
-        for block_waves, split in ((4, 1), (4, 0), (8, 1)):
+        for block_waves, split, cols in ((4, 1, 2), (4, 1, 1), (4, 0, 2), (8, 1, 2)):
             fa.check(fa.capi.lib.fa_set_tuning(11, block_waves))
             fa.check(fa.capi.lib.fa_set_tuning(12, split))
+            fa.check(fa.capi.lib.fa_set_tuning(23, cols))
             got = be.download_owned(be.paged_attention_forward_device(
                 be.upload(q), be.upload(kp), be.upload(vp), be.upload(bad_t), be.upload(bad_l), args, out_dtype=fa.capi.F32))
             assert_parity("PAGED_PREFILL_PARITY", "row 0 beside violations", got[0:1], want[0:1])
@@ -447,6 +451,7 @@ def test_block_form_prefill_flags_violations_per_column():
         fa.check(fa.capi.lib.fa_set_tuning(10, 0))
         fa.check(fa.capi.lib.fa_set_tuning(11, 0))
         fa.check(fa.capi.lib.fa_set_tuning(12, 0))
+        fa.check(fa.capi.lib.fa_set_tuning(23, 0))
 
 
 def test_bf16_prefill_properties_at_prompt_size():
