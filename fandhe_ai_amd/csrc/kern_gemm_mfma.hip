@@ -277,6 +277,10 @@ __device__ __forceinline__ void drain_row(T (&r)[7]) {
                  : "+a"(r[0]), "+a"(r[1]), "+a"(r[2]), "+a"(r[3]), "+a"(r[4]), "+a"(r[5]), "+a"(r[6]));
 }
 template <typename T>
+__device__ __forceinline__ void drain_row(T (&r)[4]) {
+    asm volatile("s_nop 15\n\ts_nop 15" : "+a"(r[0]), "+a"(r[1]), "+a"(r[2]), "+a"(r[3]));
+}
+template <typename T>
 __device__ __forceinline__ void drain_row(T (&r)[8]) {
     asm volatile("s_nop 15\n\ts_nop 15"
                  : "+a"(r[0]), "+a"(r[1]), "+a"(r[2]), "+a"(r[3]), "+a"(r[4]), "+a"(r[5]), "+a"(r[6]), "+a"(r[7]));
@@ -828,6 +832,12 @@ static W8a8Plan plan_w8a8(uint64_t m, uint64_t n_pad, uint64_t k_pad, int num_cu
     const bool big_ok = !(g_gemm_small_tiles || k_pad % 128 || k_pad == 0) && n_tiles >= 14;
     if (big_ok && m >= 256) {
         if (int ntb = pick_big_ntb(m, n_tiles, num_cus)) return {ntb, 1};
+        // Too few 256 x 224 tiles for the device, but 256 x 128 tiles for at least half of it (about a thousand rows
+        // against a 4096- or 6144-column weight): the large-tile kernel on the narrower tile keeps its rate per compute
+        // unit, where the 128 x 128 kernel with its k split and second pass ran at a third of it (1024 rows, us: q | k | v
+        // 65 + 18 -> 40, o 65 + 18 -> 37)
+        const uint64_t blocks8 = ((m + 255) / 256) * ((n_tiles + 7) / 8);
+        if (g_gemm_ntb == 0 && blocks8 * 2 >= (uint64_t)num_cus) return {8, 1};
     }
     const uint64_t blocks = ((n_tiles + NT - 1) / NT) * ((m + BM - 1) / BM);
     if (blocks == 0 || blocks * 2 > fill) return {0, 1};
@@ -863,6 +873,8 @@ void gemm_w8a8_mfma(const int8_t *aq, const int8_t *w_tiles, uint64_t m, uint64_
     int32_t *partial = p.splits > 1 ? (int32_t *)workspace : nullptr;
     if (p.ntb == 16) {
         launch_big<false, 16, EpiI8>((const uint8_t *)aq, (const uint8_t *)w_tiles, m, n, n_pad / 16, k_pad / 128, e, s);
+    } else if (p.ntb == 8) {
+        launch_big<false, 8, EpiI8>((const uint8_t *)aq, (const uint8_t *)w_tiles, m, n, n_pad / 16, k_pad / 128, e, s);
     } else if (p.ntb) {
         launch_big<false, 14, EpiI8>((const uint8_t *)aq, (const uint8_t *)w_tiles, m, n, n_pad / 16, k_pad / 128, e, s);
     } else {

@@ -322,6 +322,7 @@ int main() {
     gemm_case<true, 16, 4>();
     gemm_case<false, 14, 4>();
     gemm_case<false, 16, 4>();
+    gemm_case<false, 8, 4>();
     gemm_case<true, 14, 2>();
     gemm_case<true, 16, 2>();
     gemm_case<false, 14, 2>();

@@ -682,6 +682,43 @@ def test_int8_large_tile_kernel_bias_without_raw_sums(n):
     assert_bf16_rounding_of("w8a8 large tile bias bf16", out_bf, got)
 
 
+@pytest.mark.parametrize("m,k,n", [(1024, 512, 4096), (1000, 1024, 6144), (800, 256, 4104)])
+def test_int8_large_tile_kernel_on_256_x_128_tiles(m, k, n):
+    """About a thousand rows against a weight of 4096 to 6144 columns: too few 256 x 224 tiles for the device, so the
+    large-tile kernel runs on 256 x 128 tiles (plan: 8 column tiles per block).  Raw sums and outputs bit-exact against
+    the oracle with a bias and a residual-free epilogue, f32 and bf16 outputs, ragged rows and columns; equal to the
+    128 x 128 kernel (key 4 = 1)."""
+    fa = _fa()
+    be = ops()
+    lib = fa.capi.lib
+    rng = o.Rng(7 * m + n)
+    x = rng.randn((m, k))
+    w = rng.randn((k, n), std=0.05)
+    bias = rng.randn((n,))
+    o.set_threads(8)
+    wq, ws = o.quantize_cols_i8(w)
+    want_acc, want = o.linear_w8a8(x, wq, ws, bias)
+    o.set_threads(1)
+    qw = be.import_quantized_weight(wq, ws)
+    dbias = fa.DeviceBufferView(be.upload(bias), 0, (n,))
+    dx = be.upload(x)
+    try:
+        fa.check(lib.fa_set_tuning(21, 1))                # no weight-stationary kernel: the tiled GEMMs
+        assert _gemm_plan(fa, be, m, qw).big_ntb == 8
+        out, acc = be.linear_w8a8(dx, qw, bias=dbias, want_acc=True)
+        assert np.array_equal(be.download_owned(acc), want_acc)
+        got = be.download_owned(be.linear_w8a8(dx, qw, bias=dbias))
+        assert np.array_equal(be.download_owned(out), want) and np.array_equal(got, want)
+        out_bf = be.download_owned(be.linear_w8a8(dx, qw, bias=dbias, out_dtype=fa.capi.BF16))
+        assert_bf16_rounding_of("w8a8 256 x 128 tiles bf16", out_bf, got)
+        fa.check(lib.fa_set_tuning(4, 1))
+        assert _gemm_plan(fa, be, m, qw).big_ntb == 0
+        assert np.array_equal(be.download_owned(be.linear_w8a8(dx, qw, bias=dbias)), got)
+    finally:
+        fa.check(lib.fa_set_tuning(4, 0))
+        fa.check(lib.fa_set_tuning(21, 0))
+
+
 def test_int8_large_tile_kernel_wavefront_variants_are_bit_exact():
     """The 4- and 16-wavefront variants and both tile widths of the large-tile int8 kernel against the oracle
     on sampled rows of a ragged shape (exact integers: any difference is an indexing error)."""
