@@ -100,6 +100,7 @@ fa_status fa_set_tuning(int32_t key, int32_t value) {
         case 21: k::g_rows_kernel = value; return FA_OK;
         case 22: k::g_gemm_swiglu = value; return FA_OK;
         case 23: fa::g_prefill_block_cols = value; return FA_OK;
+        case 24: k::g_gemm_pair = value; return FA_OK;
     }
     return fail(FA_ERR_INVALID_ARGUMENT, "fa_set_tuning: unknown key");
 }
@@ -364,7 +365,7 @@ fa_status fa_linear_w8a8(fa_context *ctx, const fa_buffer *x, uint64_t m, const 
         if (uint64_t wsb = k::gemm_w8a8_workspace_bytes(m, qw->n, qw->n_pad, qw->k_pad, ctx->props.multiProcessorCount))
             if (fa_status s = ws.get(wsb)) return s;
         k::gemm_w8a8_mfma((const int8_t *)xq.ptr, (const int8_t *)qw->codes->ptr, m, qw->n, qw->n_pad, qw->k_pad, ep,
-                          ctx->props.multiProcessorCount, ctx->stream, ws.ptr, ws.bytes);
+                          ctx->props.multiProcessorCount, ctx->stream, ws.ptr, ws.bytes, &ctx->splitk);
     }
     return after_launch(ctx, "linear_w8a8");
 }
@@ -395,7 +396,7 @@ fa_status fa_gemm_w8a8(fa_context *ctx, const fa_buffer *aq, const fa_buffer *sx
     if (uint64_t wsb = k::gemm_w8a8_workspace_bytes(m, qw->n, qw->n_pad, qw->k_pad, ctx->props.multiProcessorCount))
         if (fa_status s = ws.get(wsb)) return s;
     k::gemm_w8a8_mfma((const int8_t *)aq->ptr, (const int8_t *)qw->codes->ptr, m, qw->n, qw->n_pad, qw->k_pad, ep,
-                      ctx->props.multiProcessorCount, ctx->stream, ws.ptr, ws.bytes);
+                      ctx->props.multiProcessorCount, ctx->stream, ws.ptr, ws.bytes, &ctx->splitk);
     return after_launch(ctx, "gemm_w8a8_mfma");
 }
 

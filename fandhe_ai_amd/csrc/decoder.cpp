@@ -388,7 +388,7 @@ fa_status enqueue_prefill_chunk(fa_context *ctx, fa_decoder *d, PrefillBuffers &
                                 &ctx->splitk, t.splitk.ptr, t.splitk.bytes);
         else
             k::gemm_w8a8_mfma(t.xq.as<int8_t>(), (const int8_t *)w->codes->ptr, M, w->n, w->n_pad, w->k_pad, ep, cus, s,
-                              t.splitk.ptr, t.splitk.bytes);
+                              t.splitk.ptr, t.splitk.bytes, &ctx->splitk);
     };
     auto norm_quantize = [&](const float *norm_w, const fa_qweight *w) {
         if (rows_form(w))

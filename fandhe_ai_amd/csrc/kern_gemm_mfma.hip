@@ -19,6 +19,7 @@ namespace k {
 using namespace fa::dev;
 
 int g_gemm_small_tiles = 0;   // tuning: nonzero keeps the 128 x 128 kernel for every shape
+int g_gemm_pair = 0;          // tuning: 1 keeps one block per tile on the 256 x 128 tiles of the large-tile kernel
 int g_gemm_swiglu = 0;        // tuning, prompt passes: bit 0 keeps SwiGLU out of the gate | up GEMM's epilogue, bit 1 RoPE
                               // and the K / V append out of the q | k | v GEMM's
 int g_gemm_waves = 0;
@@ -32,6 +33,13 @@ struct EpiI8 {
     int32_t *acc_out;
     void *out;
     int out_bf16;
+    // Large-tile kernel, k split over a pair of blocks (split_partial != null): blocks b and b + 8 of a launch (one
+    // XCD) own one output tile and half of k each; both leave their raw sums in split_partial, wait for their stores and
+    // take a ticket from the tile's counter, and the one that draws the second ticket adds the other's sums (int32:
+    // exact in either order) and runs the epilogue.  split_local: the exchange stays in the XCD's L2.
+    int32_t *split_partial = nullptr;
+    uint32_t *split_counters = nullptr;
+    int split_local = 0;
 };
 // int8, large-tile kernel only: the weight is gate | up (f columns each) and the kernel leaves silu(gate) * up, f32 [m, f]
 struct EpiI8Swiglu {
@@ -365,7 +373,18 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
     const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
     const int wm = wave / 2, wn = wave % 2;
     uint32_t mb, nb;
-    ixm::big_block_tile(blockIdx.x, m_blocks, n_blocks, &mb, &nb);
+    uint32_t tile_id = blockIdx.x, half = 0, ks_lo = 0, ks_n = k_steps;
+    [[maybe_unused]] bool split = false;
+    if constexpr (std::is_same<Epi, EpiI8>::value) {
+        if (ep.split_partial) {
+            split = true;
+            ixm::ksplit_block(blockIdx.x, 2, &tile_id, &half);        // partners b and b + 8: one XCD
+            if (tile_id >= m_blocks * n_blocks) return;               // the same for both partners
+            ks_lo = half ? k_steps / 2 : 0;
+            ks_n = half ? k_steps - k_steps / 2 : k_steps / 2;
+        }
+    }
+    ixm::big_block_tile(tile_id, m_blocks, n_blocks, &mb, &nb);
     const uint32_t m0 = mb * 256, nt0 = nb * NTB;
     const uint64_t k_bytes = (uint64_t)k_steps * TK;
 
@@ -394,14 +413,14 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
         uint32_t row = m0 + ixm::big_a_tile<NWAVES>(wave, i) * 16 + ixm::big_a_row(lane);
         row = row < m ? row : m - 1;
 #pragma unroll
-        for (int x = 0; x < 2; ++x) a_src[i][x] = aq + (uint64_t)row * k_bytes + ixm::big_a_src_byte<FP8>(lane, x);
+        for (int x = 0; x < 2; ++x) a_src[i][x] = aq + (uint64_t)row * k_bytes + (uint64_t)ks_lo * TK + ixm::big_a_src_byte<FP8>(lane, x);
         // a block of NTB = 14 has no tiles 14, 15: the wavefronts that would move them repeat tiles
         // 0, 1 instead (same bytes to the same place, served by the L1), which keeps the main loop
         // free of branches
         uint32_t t = nt0 + ixm::big_b_tile<NTB, NWAVES>(wave, i);
         if constexpr (SWI) t = ixm::big_swiglu_tile<NTB>(nb, ixm::big_b_tile<NTB, NWAVES>(wave, i), ep.f / 16);
         t = t < n_tiles ? t : n_tiles - 1;
-        b_src[i] = w_tiles + (uint64_t)t * k_steps * TILE + ixm::big_b_src_byte<FP8>(lane, 0);
+        b_src[i] = w_tiles + ((uint64_t)t * k_steps + ks_lo) * TILE + ixm::big_b_src_byte<FP8>(lane, 0);
     }
     // byte offsets of this lane's two A operand reads inside a tile
     const int a_off[2] = {ixm::big_a_frag_off<FP8>(lane, 0), ixm::big_a_frag_off<FP8>(lane, 1)};
@@ -447,7 +466,7 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
     // the end the loads are repeated from the last stage into slots nobody reads again, which keeps the
     // count of outstanding loads the same in every pass.
     constexpr int NLD = 2 * TPW;                     // A load instructions per wavefront and stage
-    const uint32_t last = k_steps - 1;
+    const uint32_t last = ks_n - 1;                  // stages are counted from the block's first one
 #pragma unroll
     for (int idx = 0; idx < NLD; ++idx) issue_a(0, 0, idx);
 #pragma unroll
@@ -489,7 +508,7 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
     lds_read16<0>(b[2][0], lb);
     lds_read16<1024>(b[2][1], lb);
     uint32_t ks = 0;
-    do {                                              // k_steps >= 1: the launcher returns early otherwise
+    do {                                              // ks_n >= 1: the launcher sees to it
         const int buf = ks % NSB;
         const uint32_t ks_b = ks + 1 < last ? ks + 1 : last, ks_a = ks + 2 < last ? ks + 2 : last;
         const int slot_a2 = slot_a == 0 ? 2 : slot_a - 1;             // (slot_a + 2) % 3
@@ -551,7 +570,7 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
                 });
             }
         });
-    } while (++ks < k_steps);
+    } while (++ks < ks_n);
     // the reads the last pass issued for a stage that does not exist are still on their way to registers that are
     // dead from here on: hold those registers until the reads have written them
     lds_wait_all_a<0>(a, b[2]);
@@ -562,6 +581,51 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
 #pragma unroll
     for (int i = 0; i < AI; ++i) drain_row(acc[i]);
     __builtin_amdgcn_s_waitcnt(0x0F70);               // the repeated loads of the tail have landed too
+
+    if constexpr (std::is_same<Epi, EpiI8>::value) {
+        if (split) {
+            // raw sums of this half of k: word (i, j, e) of thread t at [(i * WNT + j) * 4 + e][t], 2 KiB per store
+            constexpr int WORDS = AI * WNT * 4;
+            int32_t *mine = ep.split_partial + ((uint64_t)tile_id * 2 + half) * ((uint64_t)WORDS * 128 * WM);
+            const int32_t *other = ep.split_partial + ((uint64_t)tile_id * 2 + (half ^ 1)) * ((uint64_t)WORDS * 128 * WM);
+            const bool local = ep.split_local != 0;
+#pragma unroll
+            for (int i = 0; i < AI; ++i)
+#pragma unroll
+                for (int j = 0; j < WNT; ++j)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        int32_t *p = mine + ((i * WNT + j) * 4 + e) * (128 * WM) + tid;
+                        if (local) __hip_atomic_store(p, (int32_t)acc[i][j][e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                        else __hip_atomic_store(p, (int32_t)acc[i][j][e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+            __builtin_amdgcn_s_waitcnt(0);            // this thread's stores are acknowledged
+            __syncthreads();                          // ... and everybody's; nobody reads the stages any more
+            uint32_t *slot = (uint32_t *)lds;
+            if (tid == 0) {
+                uint32_t *ctr = ep.split_counters + tile_id;
+                const uint32_t t = local ? __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)
+                                         : __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (t == 1) {                         // both are in: the counter returns to zero for the next launch
+                    if (local) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    else __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+                *slot = t;
+            }
+            __syncthreads();
+            if (*slot == 0) return;                   // the partner finishes the tile
+#pragma unroll
+            for (int i = 0; i < AI; ++i)
+#pragma unroll
+                for (int j = 0; j < WNT; ++j)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int32_t *p = other + ((i * WNT + j) * 4 + e) * (128 * WM) + tid;
+                        acc[i][j][e] += local ? __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)
+                                              : __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+        }
+    }
 
     // Epilogue.  The matrix instructions took the weight fragment as their first operand, so an accumulator tile is
     // the transpose of the usual one: lane l holds row l % 16 of the output tile and its columns 4 (l / 16) + e,
@@ -824,6 +888,7 @@ void launch_big(const uint8_t *aq, const uint8_t *w_tiles, uint64_t m, uint64_t 
 struct W8a8Plan {
     int ntb;
     uint32_t splits;
+    bool pair = false;     // large-tile kernel on 256 x 128 tiles with k split over pairs of same-XCD blocks
 };
 
 static W8a8Plan plan_w8a8(uint64_t m, uint64_t n_pad, uint64_t k_pad, int num_cus) {
@@ -837,7 +902,10 @@ static W8a8Plan plan_w8a8(uint64_t m, uint64_t n_pad, uint64_t k_pad, int num_cu
         // unit, where the 128 x 128 kernel with its k split and second pass ran at a third of it (1024 rows, us: q | k | v
         // 65 + 18 -> 40, o 65 + 18 -> 37)
         const uint64_t blocks8 = ((m + 255) / 256) * ((n_tiles + 7) / 8);
-        if (g_gemm_ntb == 0 && blocks8 * 2 >= (uint64_t)num_cus) return {8, 1};
+        // ... and when those tiles cover at most half of it, two blocks share a tile, half of k each (one prompt of 1024
+        // tokens through 32 layers: 14.0 -> 12.4 ms)
+        if (g_gemm_ntb == 0 && blocks8 * 2 >= (uint64_t)num_cus)
+            return {8, 1, g_gemm_pair != 1 && blocks8 * 2 <= (uint64_t)num_cus && k_pad / 128 >= 32};
     }
     const uint64_t blocks = ((n_tiles + NT - 1) / NT) * ((m + BM - 1) / BM);
     if (blocks == 0 || blocks * 2 > fill) return {0, 1};
@@ -860,14 +928,37 @@ GemmPlan gemm_plan(bool fp8, uint64_t m, uint64_t n_pad, uint64_t k_pad, int num
 
 uint64_t gemm_w8a8_workspace_bytes(uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad, int num_cus) {
     const W8a8Plan p = plan_w8a8(m, n_pad, k_pad, num_cus);
+    if (p.pair) return ((m + 255) / 256) * ((n_pad / 16 + 7) / 8) * 2 * (uint64_t)(256 * 128 * 4);
     return p.splits > 1 ? (uint64_t)p.splits * m * n * 4 : 0;
 }
 
 void gemm_w8a8_mfma(const int8_t *aq, const int8_t *w_tiles, uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad,
-                    const EpilogueI8 &ep, int num_cus, hipStream_t s, void *workspace, uint64_t workspace_bytes) {
+                    const EpilogueI8 &ep, int num_cus, hipStream_t s, void *workspace, uint64_t workspace_bytes,
+                    const SplitKArea *sk) {
     if (m == 0 || n == 0) return;
     EpiI8 e{ep.sx, ep.sw, ep.bias, ep.residual, ep.acc_out, ep.out, ep.out_bf16};
     W8a8Plan p = plan_w8a8(m, n_pad, k_pad, num_cus);
+    if (p.pair) {
+        const uint64_t tiles = ((m + 255) / 256) * ((n_pad / 16 + 7) / 8), need = tiles * 2 * (uint64_t)(256 * 128 * 4);
+        if (sk && sk->counters && tiles <= sk->n_counters && workspace && workspace_bytes >= need && g_gemm_waves != 4 && g_gemm_waves != 16) {
+            e.split_partial = (int32_t *)workspace;
+            e.split_counters = sk->counters;
+            e.split_local = sk->xcd_local;
+            constexpr int NTB = 8;
+            const size_t smem = (3 * 16 + 2 * (size_t)NTB) * 2048;
+            static bool configured = false;
+            if (!configured) {
+                (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_mfma_big_kernel<false, NTB, 4, EpiI8>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+                configured = true;
+            }
+            const uint32_t mb = (uint32_t)((m + 255) / 256), nb = (uint32_t)((n_pad / 16 + NTB - 1) / NTB);
+            const unsigned grid = 16u * (unsigned)((tiles + 7) / 8);           // whole pairs on every XCD; surplus pairs return at once
+            gemm_mfma_big_kernel<false, NTB, 4, EpiI8><<<grid, 512, smem, s>>>((const uint8_t *)aq, (const uint8_t *)w_tiles, (uint32_t)m,
+                                                                           (uint32_t)n, (uint32_t)(n_pad / 16), (uint32_t)(k_pad / 128), mb, nb, e);
+            return;
+        }
+    }
     if (p.splits > 1 && (!workspace || workspace_bytes < (uint64_t)p.splits * m * n * 4))
         p.splits = 1;                                 // no room for partial sums: one block per tile
     int32_t *partial = p.splits > 1 ? (int32_t *)workspace : nullptr;

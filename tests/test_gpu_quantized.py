@@ -682,12 +682,14 @@ def test_int8_large_tile_kernel_bias_without_raw_sums(n):
     assert_bf16_rounding_of("w8a8 large tile bias bf16", out_bf, got)
 
 
-@pytest.mark.parametrize("m,k,n", [(1024, 512, 4096), (1000, 1024, 6144), (800, 256, 4104)])
+@pytest.mark.parametrize("m,k,n", [(1024, 512, 4096), (1000, 1024, 6144), (800, 256, 4104), (1024, 4096, 4096), (800, 8320, 4096)])
 def test_int8_large_tile_kernel_on_256_x_128_tiles(m, k, n):
     """About a thousand rows against a weight of 4096 to 6144 columns: too few 256 x 224 tiles for the device, so the
     large-tile kernel runs on 256 x 128 tiles (plan: 8 column tiles per block).  Raw sums and outputs bit-exact against
     the oracle with a bias and a residual-free epilogue, f32 and bf16 outputs, ragged rows and columns; equal to the
-    128 x 128 kernel (key 4 = 1)."""
+    128 x 128 kernel (key 4 = 1).  With k of 4096 and more and tiles for at most half the device, pairs of same-XCD blocks
+    share a tile, half of k each, and meet in a workspace (the last two shapes, an odd number of k stages among them):
+    three calls in a row, and identical to one block per tile (key 24 = 1)."""
     fa = _fa()
     be = ops()
     lib = fa.capi.lib
@@ -709,6 +711,10 @@ def test_int8_large_tile_kernel_on_256_x_128_tiles(m, k, n):
         assert np.array_equal(be.download_owned(acc), want_acc)
         got = be.download_owned(be.linear_w8a8(dx, qw, bias=dbias))
         assert np.array_equal(be.download_owned(out), want) and np.array_equal(got, want)
+        assert np.array_equal(be.download_owned(be.linear_w8a8(dx, qw, bias=dbias)), want)      # counters back at zero
+        fa.check(lib.fa_set_tuning(24, 1))
+        assert np.array_equal(be.download_owned(be.linear_w8a8(dx, qw, bias=dbias)), want)
+        fa.check(lib.fa_set_tuning(24, 0))
         out_bf = be.download_owned(be.linear_w8a8(dx, qw, bias=dbias, out_dtype=fa.capi.BF16))
         assert_bf16_rounding_of("w8a8 256 x 128 tiles bf16", out_bf, got)
         fa.check(lib.fa_set_tuning(4, 1))
@@ -717,6 +723,7 @@ def test_int8_large_tile_kernel_on_256_x_128_tiles(m, k, n):
     finally:
         fa.check(lib.fa_set_tuning(4, 0))
         fa.check(lib.fa_set_tuning(21, 0))
+        fa.check(lib.fa_set_tuning(24, 0))
 
 
 def test_int8_large_tile_kernel_wavefront_variants_are_bit_exact():
