@@ -19,7 +19,8 @@ namespace k {
 using namespace fa::dev;
 
 int g_gemm_small_tiles = 0;   // tuning: nonzero keeps the 128 x 128 kernel for every shape
-int g_gemm_pair = 0;          // tuning: 1 keeps one block per tile on the 256 x 128 tiles of the large-tile kernel
+int g_gemm_pair = 0;          // tuning, 256 x 128 tiles of the large-tile kernel: 1 keeps one block per tile, 2 shares a tile
+                              // only where the tiles alone would cover half the device
 int g_gemm_swiglu = 0;        // tuning, prompt passes: bit 0 keeps SwiGLU out of the gate | up GEMM's epilogue, bit 1 RoPE
                               // and the K / V append out of the q | k | v GEMM's
 int g_gemm_waves = 0;
@@ -33,13 +34,14 @@ struct EpiI8 {
     int32_t *acc_out;
     void *out;
     int out_bf16;
-    // Large-tile kernel, k split over a pair of blocks (split_partial != null): blocks b and b + 8 of a launch (one
-    // XCD) own one output tile and half of k each; both leave their raw sums in split_partial, wait for their stores and
-    // take a ticket from the tile's counter, and the one that draws the second ticket adds the other's sums (int32:
-    // exact in either order) and runs the epilogue.  split_local: the exchange stays in the XCD's L2.
+    // Large-tile kernel, k split over split_s = 2 or 4 blocks (split_partial != null): blocks b, b + 8, ... of a launch
+    // (one XCD) own one output tile and a share of k each; all leave their raw sums in split_partial, wait for their
+    // stores and take a ticket from the tile's counter, and the one that draws the last ticket adds the others' sums
+    // (int32: exact in any order) and runs the epilogue.  split_local: the exchange stays in the XCD's L2.
     int32_t *split_partial = nullptr;
     uint32_t *split_counters = nullptr;
     int split_local = 0;
+    uint32_t split_s = 2;
 };
 // int8, large-tile kernel only: the weight is gate | up (f columns each) and the kernel leaves silu(gate) * up, f32 [m, f]
 struct EpiI8Swiglu {
@@ -378,10 +380,11 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
     if constexpr (std::is_same<Epi, EpiI8>::value) {
         if (ep.split_partial) {
             split = true;
-            ixm::ksplit_block(blockIdx.x, 2, &tile_id, &half);        // partners b and b + 8: one XCD
-            if (tile_id >= m_blocks * n_blocks) return;               // the same for both partners
-            ks_lo = half ? k_steps / 2 : 0;
-            ks_n = half ? k_steps - k_steps / 2 : k_steps / 2;
+            ixm::ksplit_block(blockIdx.x, ep.split_s, &tile_id, &half);      // partners b, b + 8, ...: one XCD
+            if (tile_id >= m_blocks * n_blocks) return;               // the same for all partners
+            uint32_t ks_hi;
+            ixm::ksplit_k_range(k_steps, half, ep.split_s, &ks_lo, &ks_hi);
+            ks_n = ks_hi - ks_lo;
         }
     }
     ixm::big_block_tile(tile_id, m_blocks, n_blocks, &mb, &nb);
@@ -586,8 +589,8 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
         if (split) {
             // raw sums of this half of k: word (i, j, e) of thread t at [(i * WNT + j) * 4 + e][t], 2 KiB per store
             constexpr int WORDS = AI * WNT * 4;
-            int32_t *mine = ep.split_partial + ((uint64_t)tile_id * 2 + half) * ((uint64_t)WORDS * 128 * WM);
-            const int32_t *other = ep.split_partial + ((uint64_t)tile_id * 2 + (half ^ 1)) * ((uint64_t)WORDS * 128 * WM);
+            const uint32_t S = ep.split_s;
+            int32_t *mine = ep.split_partial + ((uint64_t)tile_id * S + half) * ((uint64_t)WORDS * 128 * WM);
             const bool local = ep.split_local != 0;
 #pragma unroll
             for (int i = 0; i < AI; ++i)
@@ -606,24 +609,28 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
                 uint32_t *ctr = ep.split_counters + tile_id;
                 const uint32_t t = local ? __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)
                                          : __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                if (t == 1) {                         // both are in: the counter returns to zero for the next launch
+                if (t == S - 1) {                     // all are in: the counter returns to zero for the next launch
                     if (local) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                     else __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
                 *slot = t;
             }
             __syncthreads();
-            if (*slot == 0) return;                   // the partner finishes the tile
+            if (*slot != S - 1) return;               // a partner finishes the tile
+            for (uint32_t r = 0; r < S; ++r) {
+                if (r == half) continue;
+                const int32_t *other = ep.split_partial + ((uint64_t)tile_id * S + r) * ((uint64_t)WORDS * 128 * WM);
 #pragma unroll
-            for (int i = 0; i < AI; ++i)
+                for (int i = 0; i < AI; ++i)
 #pragma unroll
-                for (int j = 0; j < WNT; ++j)
+                    for (int j = 0; j < WNT; ++j)
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const int32_t *p = other + ((i * WNT + j) * 4 + e) * (128 * WM) + tid;
-                        acc[i][j][e] += local ? __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)
-                                              : __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    }
+                        for (int e = 0; e < 4; ++e) {
+                            const int32_t *p = other + ((i * WNT + j) * 4 + e) * (128 * WM) + tid;
+                            acc[i][j][e] += local ? __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)
+                                                  : __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        }
+            }
         }
     }
 
@@ -888,10 +895,10 @@ void launch_big(const uint8_t *aq, const uint8_t *w_tiles, uint64_t m, uint64_t 
 struct W8a8Plan {
     int ntb;
     uint32_t splits;
-    bool pair = false;     // large-tile kernel on 256 x 128 tiles with k split over pairs of same-XCD blocks
+    uint32_t share = 1;    // large-tile kernel on 256 x 128 tiles: same-XCD blocks that share a tile, a part of k each
 };
 
-static W8a8Plan plan_w8a8(uint64_t m, uint64_t n_pad, uint64_t k_pad, int num_cus) {
+static W8a8Plan plan_w8a8(uint64_t m, uint64_t n_pad, uint64_t k_pad, int num_cus, bool may_share = true) {
     const uint64_t n_tiles = n_pad / 16;
     const uint64_t fill = (uint64_t)num_cus * (g_gemm_split_fill > 0 ? g_gemm_split_fill : 2);
     const bool big_ok = !(g_gemm_small_tiles || k_pad % 128 || k_pad == 0) && n_tiles >= 14;
@@ -901,11 +908,16 @@ static W8a8Plan plan_w8a8(uint64_t m, uint64_t n_pad, uint64_t k_pad, int num_cu
         // against a 4096- or 6144-column weight): the large-tile kernel on the narrower tile keeps its rate per compute
         // unit, where the 128 x 128 kernel with its k split and second pass ran at a third of it (1024 rows, us: q | k | v
         // 65 + 18 -> 40, o 65 + 18 -> 37)
-        const uint64_t blocks8 = ((m + 255) / 256) * ((n_tiles + 7) / 8);
-        // ... and when those tiles cover at most half of it, two blocks share a tile, half of k each (one prompt of 1024
-        // tokens through 32 layers: 14.0 -> 12.4 ms)
+        const uint64_t blocks8 = ((m + 255) / 256) * ((n_tiles + 7) / 8), k_steps = k_pad / 128;
+        // ... and when those tiles cover a quarter to a half of it, two blocks share a tile, half of k each (one prompt
+        // of 1024 tokens through 32 layers: 14.0 -> 12.4 ms; 600 / 767 rows, us incl. the row quantizer: 4096 -> 4096
+        // 46 / 53 -> 41 / 41, 14336 -> 4096 105 / 133 -> 93 / 95), at least sixteen stages of k per block.  Four blocks a
+        // tile measured slower than every other form (14336 -> 4096 at 257 .. 512 rows: 82 - 87 us against 55 - 78 us).
         if (g_gemm_ntb == 0 && blocks8 * 2 >= (uint64_t)num_cus)
-            return {8, 1, g_gemm_pair != 1 && blocks8 * 2 <= (uint64_t)num_cus && k_pad / 128 >= 32};
+            return {8, 1, (may_share && g_gemm_pair != 1 && blocks8 * 2 <= (uint64_t)num_cus && k_steps >= 32) ? 2u : 1u};
+        if (may_share && g_gemm_ntb == 0 && g_gemm_pair != 1 && g_gemm_pair != 2) {
+            if (blocks8 * 4 >= (uint64_t)num_cus && blocks8 * 2 <= (uint64_t)num_cus && k_steps >= 32) return {8, 1, 2};
+        }
     }
     const uint64_t blocks = ((n_tiles + NT - 1) / NT) * ((m + BM - 1) / BM);
     if (blocks == 0 || blocks * 2 > fill) return {0, 1};
@@ -928,7 +940,7 @@ GemmPlan gemm_plan(bool fp8, uint64_t m, uint64_t n_pad, uint64_t k_pad, int num
 
 uint64_t gemm_w8a8_workspace_bytes(uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad, int num_cus) {
     const W8a8Plan p = plan_w8a8(m, n_pad, k_pad, num_cus);
-    if (p.pair) return ((m + 255) / 256) * ((n_pad / 16 + 7) / 8) * 2 * (uint64_t)(256 * 128 * 4);
+    if (p.share > 1) return ((m + 255) / 256) * ((n_pad / 16 + 7) / 8) * p.share * (uint64_t)(256 * 128 * 4);
     return p.splits > 1 ? (uint64_t)p.splits * m * n * 4 : 0;
 }
 
@@ -938,12 +950,13 @@ void gemm_w8a8_mfma(const int8_t *aq, const int8_t *w_tiles, uint64_t m, uint64_
     if (m == 0 || n == 0) return;
     EpiI8 e{ep.sx, ep.sw, ep.bias, ep.residual, ep.acc_out, ep.out, ep.out_bf16};
     W8a8Plan p = plan_w8a8(m, n_pad, k_pad, num_cus);
-    if (p.pair) {
-        const uint64_t tiles = ((m + 255) / 256) * ((n_pad / 16 + 7) / 8), need = tiles * 2 * (uint64_t)(256 * 128 * 4);
+    if (p.share > 1) {
+        const uint64_t tiles = ((m + 255) / 256) * ((n_pad / 16 + 7) / 8), need = tiles * p.share * (uint64_t)(256 * 128 * 4);
         if (sk && sk->counters && tiles <= sk->n_counters && workspace && workspace_bytes >= need && g_gemm_waves != 4 && g_gemm_waves != 16) {
             e.split_partial = (int32_t *)workspace;
             e.split_counters = sk->counters;
             e.split_local = sk->xcd_local;
+            e.split_s = p.share;
             constexpr int NTB = 8;
             const size_t smem = (3 * 16 + 2 * (size_t)NTB) * 2048;
             static bool configured = false;
@@ -953,11 +966,12 @@ void gemm_w8a8_mfma(const int8_t *aq, const int8_t *w_tiles, uint64_t m, uint64_
                 configured = true;
             }
             const uint32_t mb = (uint32_t)((m + 255) / 256), nb = (uint32_t)((n_pad / 16 + NTB - 1) / NTB);
-            const unsigned grid = 16u * (unsigned)((tiles + 7) / 8);           // whole pairs on every XCD; surplus pairs return at once
+            const unsigned grid = 8u * p.share * (unsigned)((tiles + 7) / 8);   // whole groups on every XCD; surplus groups return at once
             gemm_mfma_big_kernel<false, NTB, 4, EpiI8><<<grid, 512, smem, s>>>((const uint8_t *)aq, (const uint8_t *)w_tiles, (uint32_t)m,
                                                                            (uint32_t)n, (uint32_t)(n_pad / 16), (uint32_t)(k_pad / 128), mb, nb, e);
             return;
         }
+        p = plan_w8a8(m, n_pad, k_pad, num_cus, false);      // no counters or no room: the plan without shared tiles
     }
     if (p.splits > 1 && (!workspace || workspace_bytes < (uint64_t)p.splits * m * n * 4))
         p.splits = 1;                                 // no room for partial sums: one block per tile

@@ -221,8 +221,8 @@ void linear_w8a8_rows(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t m,
 // aq: int8 [m, k_pad] row-major.  workspace (optional, gemm_w8a8_workspace_bytes): lets a matrix with too few
 // output tiles to occupy the device split k across blocks; the int32 partial sums meet there and are
 // added exactly, so the result does not depend on the split.
-// sk (optional): with it and the workspace, a launch of at most about half a device of 256 x 128 tiles lets two blocks
-// of an XCD share a tile, half of k each (they meet in the workspace; the second to arrive finishes the tile).
+// sk (optional): with it and the workspace, a launch of at most half a device of 256 x 128 tiles lets two or four blocks
+// of an XCD share a tile, a part of k each (they meet in the workspace; the last to arrive finishes the tile).
 void gemm_w8a8_mfma(const int8_t *aq, const int8_t *w_tiles, uint64_t m, uint64_t n, uint64_t n_pad,
                     uint64_t k_pad, const EpilogueI8 &ep, int num_cus, hipStream_t s, void *workspace = nullptr,
                     uint64_t workspace_bytes = 0, const SplitKArea *sk = nullptr);
@@ -230,7 +230,8 @@ uint64_t gemm_w8a8_workspace_bytes(uint64_t m, uint64_t n, uint64_t n_pad, uint6
 // The gate | up projection with SwiGLU in its epilogue (large-tile kernel, m >= 256, f a multiple of 128, k_pad of 128):
 // w_tiles is the [k, 2 f] weight with the gate columns first; out receives silu(gate) * up, f32 [m, f], bit for bit
 // what gemm_w8a8_mfma into an [m, 2 f] buffer followed by the SwiGLU pass computes.
-extern int g_gemm_pair;       // 1: never two blocks per tile on the 256 x 128 tiles of the large-tile kernel
+extern int g_gemm_pair;       // 1: one block per tile on the 256 x 128 tiles of the large-tile kernel; 2: shared tiles only
+                              // where the tiles alone cover half the device
 extern int g_gemm_swiglu;     // bit 0: SwiGLU stays a pass of its own; bit 1: so do RoPE and the K / V append (below)
 bool gemm_w8a8_swiglu_applies(uint64_t m, uint64_t f, uint64_t n_pad, uint64_t k_pad);
 void gemm_w8a8_swiglu_mfma(const int8_t *aq, const int8_t *w_tiles, const float *sx, const float *sw, uint64_t m, uint64_t f,

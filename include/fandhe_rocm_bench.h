@@ -101,8 +101,9 @@ fa_status fa_probe_l2_path(fa_context *ctx, const fa_buffer *cold, uint64_t cold
  *        epilogues;
  * key 23: columns (new token x head) per wavefront of the block form of the prefill attention: 0 by shape (16 while
  *        blocks of 32 would not fill the device more than once, else 32), 1: 16 whenever the form allows, 2: 32;
- * key 24: 1 keeps one block per tile where the large-tile int8 GEMM runs on 256 x 128 tiles (0: when those tiles cover
- *        at most about half the device, pairs of same-XCD blocks share a tile, half of k each). */
+ * key 24: the large-tile int8 GEMM on 256 x 128 tiles: 0: when those tiles cover at most half the device, two or four
+ *        same-XCD blocks share a tile, a part of k each; 1: one block per tile; 2: shared tiles only where the tiles
+ *        alone cover half the device (pairs). */
 fa_status fa_set_tuning(int32_t key, int32_t value);
 
 /* What the context found when it was created: xcd_local = 1 when workgroups b and b + 8 of a launch were seen to
