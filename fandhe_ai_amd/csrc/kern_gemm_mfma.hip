@@ -19,6 +19,7 @@ namespace k {
 using namespace fa::dev;
 
 int g_gemm_small_tiles = 0;   // tuning: nonzero keeps the 128 x 128 kernel for every shape
+extern int g_skinny_ksplit;   // kern_qlinear.hip
 int g_gemm_pair = 0;          // tuning, 256 x 128 tiles of the large-tile kernel: 1 keeps one block per tile, 2 shares a tile
                               // only where the tiles alone would cover half the device
 int g_gemm_swiglu = 0;        // tuning, prompt passes: bit 0 keeps SwiGLU out of the gate | up GEMM's epilogue, bit 1 RoPE
@@ -955,7 +956,8 @@ void gemm_w8a8_mfma(const int8_t *aq, const int8_t *w_tiles, uint64_t m, uint64_
         if (sk && sk->counters && tiles <= sk->n_counters && workspace && workspace_bytes >= need && g_gemm_waves != 4 && g_gemm_waves != 16) {
             e.split_partial = (int32_t *)workspace;
             e.split_counters = sk->counters;
-            e.split_local = sk->xcd_local;
+            // (the scope knob of the split-k decode linears forces either form here as well: 2 agent scope, 3 the XCD's L2)
+            e.split_local = g_skinny_ksplit == 2 ? 0 : g_skinny_ksplit == 3 ? 1 : sk->xcd_local;
             e.split_s = p.share;
             constexpr int NTB = 8;
             const size_t smem = (3 * 16 + 2 * (size_t)NTB) * 2048;

@@ -712,6 +712,10 @@ def test_int8_large_tile_kernel_on_256_x_128_tiles(m, k, n):
         got = be.download_owned(be.linear_w8a8(dx, qw, bias=dbias))
         assert np.array_equal(be.download_owned(out), want) and np.array_equal(got, want)
         assert np.array_equal(be.download_owned(be.linear_w8a8(dx, qw, bias=dbias)), want)      # counters back at zero
+        for scope in (2, 3):                              # partial sums exchanged with agent-scope accesses / in the XCD's L2
+            fa.check(lib.fa_set_tuning(16, scope))
+            assert np.array_equal(be.download_owned(be.linear_w8a8(dx, qw, bias=dbias)), want), scope
+        fa.check(lib.fa_set_tuning(16, 0))
         fa.check(lib.fa_set_tuning(24, 1))
         assert np.array_equal(be.download_owned(be.linear_w8a8(dx, qw, bias=dbias)), want)
         fa.check(lib.fa_set_tuning(24, 0))
@@ -724,6 +728,7 @@ def test_int8_large_tile_kernel_on_256_x_128_tiles(m, k, n):
         fa.check(lib.fa_set_tuning(4, 0))
         fa.check(lib.fa_set_tuning(21, 0))
         fa.check(lib.fa_set_tuning(24, 0))
+        fa.check(lib.fa_set_tuning(16, 0))
 
 
 def test_int8_large_tile_kernel_wavefront_variants_are_bit_exact():
