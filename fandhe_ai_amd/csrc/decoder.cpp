@@ -118,11 +118,17 @@ void enqueue_pick(fa_decoder *d, hipStream_t s) {
 
 // Whether the step about to be enqueued (the host lengths already count its token) sees only short contexts: its
 // attention then takes the one-launch form, and the recorded graphs of the two kinds are kept apart.
+// With at most one block (sequence x kv head) per compute unit: a scheduler's batch of up to a few dozen short
+// conversations, whose few pages the streamed form would cut into ranges of a dozen, leaving partial results and a
+// merge launch (measured through 32 layers at 4 .. 32 rows and contexts up to 1000: 2 - 14 % of the step; from 36 rows
+// on, with more blocks than compute units and their unequal lengths, the streamed form is the faster one).
 bool step_is_short(const fa_decoder *d) {
     if (k::g_decode_one == 1) return false;
     uint32_t longest = 0;
     for (uint32_t b = 0; b < d->batch && b < d->host_lens.size(); ++b) longest = std::max(longest, d->host_lens[b]);
-    return d->batch != 0 && d->batch <= 2 && longest <= k::kDecodeOneMaxCtx;
+    if (d->batch == 0 || longest > k::kDecodeOneMaxCtx) return false;
+    const uint64_t blocks = (uint64_t)d->batch * d->cfg.n_kv_heads;
+    return k::g_decode_one == 2 || blocks <= (uint64_t)d->ctx->props.multiProcessorCount;
 }
 
 // The kernels of one step, enqueued on the context's stream.  stop_after (test aid, -1 in normal use) ends the
@@ -209,8 +215,8 @@ fa_status enqueue_step(fa_context *ctx, fa_decoder *d, int stop_after = -1) {
         // One or two short sequences: the attention finishes in one launch (a block per sequence and kv head; no
         // partial results, no merge launch) and leaves its output and the heads' maxima for the o projection, which
         // does the per-token quantizer itself.
-        const bool one_attn = short_ctx && c.n_heads <= 32 && F >= EQ && EQ % 64 == 0 &&
-                              k::plain_fuses_pmax_quantizer(B, L.wo->n_pad, L.wo->k_pad, cus);
+        const bool one_form = short_ctx && c.n_heads <= 32 && F >= EQ && EQ % 64 == 0;
+        const bool one_attn = one_form && k::plain_fuses_pmax_quantizer(B, L.wo->n_pad, L.wo->k_pad, cus);
         if (!fuse_qkv)
             k::rmsnorm_quantize_i8((const float *)d->h->ptr, (const float *)L.attn_norm->ptr, c.rms_eps, nullptr,
                                    (int8_t *)d->xq->ptr, (float *)d->sx->ptr, B, m_pad, D, s,
@@ -229,6 +235,15 @@ fa_status enqueue_step(fa_context *ctx, fa_decoder *d, int stop_after = -1) {
                                                (const uint16_t *)L.v_pool->ptr, (const uint32_t *)d->tables->ptr,
                                                (const uint32_t *)d->seq_lens->ptr, ps, (float *)d->act->ptr,
                                                (float *)d->pmax->ptr, s);
+        } else if (one_form) {
+            // the same launch for more rows than the o projection quantizes for itself: the quantizer from the heads'
+            // maxima is a launch of its own (the output is f32 values already rounded to bf16, the operator's output type)
+            k::paged_attention_decode_one_bf16((const uint16_t *)d->q_bf->ptr, (const uint16_t *)L.k_pool->ptr,
+                                               (const uint16_t *)L.v_pool->ptr, (const uint32_t *)d->tables->ptr,
+                                               (const uint32_t *)d->seq_lens->ptr, ps, (float *)d->act->ptr,
+                                               (float *)d->pmax->ptr, s);
+            k::quantize_rows_from_pmax(d->act->ptr, false, (const float *)d->pmax->ptr, c.n_heads, (int8_t *)d->xq->ptr,
+                                       (float *)d->sx->ptr, B, m_pad, EQ, s);
         } else if (c.n_heads <= 32) {
             k::paged_attention_decode_bf16((const uint16_t *)d->q_bf->ptr, (const uint16_t *)L.k_pool->ptr,
                                            (const uint16_t *)L.v_pool->ptr, (const uint32_t *)d->tables->ptr,

@@ -87,9 +87,10 @@ fa_status fa_probe_l2_path(fa_context *ctx, const fa_buffer *cold, uint64_t cold
  * key 19: 1 keeps the norm + quantizer and quantizer kernels of a decode step as launches of their own for every batch
  *        size; 0: for at most four rows the linears that follow do that row work themselves (takes effect when a step
  *        is recorded);
- * key 20: 1 keeps the streamed attention with its merge launch for every decode step; 0: a step of one or two
- *        sequences whose contexts are at most 1024 tokens runs the attention as one launch (a block per sequence
- *        and kv head) and lets the o projection do the quantizer (takes effect when a step is recorded);
+ * key 20: 1 keeps the streamed attention with its merge launch for every decode step; 0: a step whose contexts are
+ *        at most 1024 tokens runs the attention as one launch (a block per sequence and kv head) while there is at
+ *        most one such block per compute unit (with one or two sequences the o projection then does the quantizer);
+ *        2: whenever the contexts are that short (takes effect when a step is recorded);
  * key 21: the int8 linears of 65 to a few hundred rows (fa_linear_w8a8, prompt passes of the decoder): 0 the
  *        weight-stationary kernel where the shape rule picks it (a weight with at most about two column tiles per
  *        compute unit, m x k at most 2 MiB; k of 8192 .. 14336: the form that splits k over four blocks of an XCD,

@@ -167,14 +167,20 @@ def test_small_batches_do_the_row_work_inside_the_linears(shape, batch):
         fa.check(lib.fa_set_tuning(5, 0))
 
 
-@pytest.mark.parametrize("ctxs", [[1], [16], [17, 3], [130, 64], [1000, 1], [1023, 777]], ids=lambda c: "ctx" + "_".join(map(str, c)))
+_MANY_SHORT = [int(x) for x in np.random.default_rng(5).integers(1, 700, size=33)]
+
+
+@pytest.mark.parametrize("ctxs", [[1], [16], [17, 3], [130, 64], [1000, 1], [1023, 777], [40, 7, 300, 1, 64], _MANY_SHORT],
+                         ids=lambda c: "ctx" + "_".join(map(str, c[:6])) + ("_etc" if len(c) > 6 else ""))
 def test_short_contexts_finish_the_attention_in_one_launch(ctxs):
-    """One or two sequences of at most 1024 tokens: the attention runs as one launch (a block per sequence and kv
-    head whose four wavefronts share the pages) and the o projection does the per-token quantizer.  What the o
-    projection publishes (codes and scales of the attention output, stage 4 of the first layer) must be what the
-    streamed attention + merge + quantizer leave (tuning key 20 = 1) up to the last bits of the attention output: equal
-    scales to 1e-6 relative and codes at most one step apart, nearly all equal.  The steps meet the oracle, eager
-    and replayed, also when a context grows past the limit and the step changes form (1023 -> 1026)."""
+    """Sequences of at most 1024 tokens: the attention runs as one launch (a block per sequence and kv head whose
+    four wavefronts share the pages); with one or two sequences the o projection does the per-token quantizer, with
+    more (up to one block per compute unit by itself; forced here for every batch, tuning key 20 = 2) the quantizer
+    from the heads' maxima is a launch of its own.  The codes and scales of the attention output (stage 4
+    of the first layer) must be what the streamed attention + merge + quantizer leave (tuning key 20 = 1) up to the
+    last bits of the attention output: equal scales to 1e-6 relative and codes at most one step apart, nearly all
+    equal.  The steps meet the oracle, eager and replayed, also when a context grows past the limit and the step
+    changes form (1023 -> 1026)."""
     import ctypes as C
     import fandhe_ai_amd as fa
     be = ops()
@@ -185,7 +191,7 @@ def test_short_contexts_finish_the_attention_in_one_launch(ctxs):
     got = {}
     try:
         for one in (True, False):
-            fa.check(lib.fa_set_tuning(20, 0 if one else 1))
+            fa.check(lib.fa_set_tuning(20, 2 if one else 1))
             dec = GpuDecoder(be, m)
             try:
                 dec.set_state(m.seq_lens, m.tokens)
@@ -203,7 +209,7 @@ def test_short_contexts_finish_the_attention_in_one_launch(ctxs):
         (ca, sa), (cb, sb) = got[True], got[False]
         assert np.all(sb > 0) and np.allclose(sa, sb, rtol=1e-6, atol=0)
         assert np.abs(ca - cb).max() <= 1 and (ca != cb).mean() < 2e-3 and np.any(ca != 0)
-        fa.check(lib.fa_set_tuning(20, 0))
+        fa.check(lib.fa_set_tuning(20, 2))
         dec = GpuDecoder(be, m)
         try:
             lens, tokens = m.seq_lens.copy(), m.tokens.copy()
