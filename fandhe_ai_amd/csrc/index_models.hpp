@@ -143,6 +143,17 @@ FA_HD void ksplit_k_range(uint32_t k_tiles, uint32_t member, uint32_t s, uint32_
 FA_HD uint64_t ksplit_partial_base(uint32_t group, uint32_t member, uint32_t s, uint32_t nacc) {
     return ((uint64_t)group * s + member) * ((uint64_t)nacc * 64);
 }
+// Activation operand of the decode-shape int8 kernels (w8a8_skinny_kernel, w8a8_ksplit_kernel): byte offset of the 16
+// bytes lane `lane` fetches for row tile i and k-tile kt from the tiled codes of m rows (ceil(m / 16) row tiles of
+// k_tiles x 1 KiB; lane l holds row l % 16, k-group l / 16).  The lanes of rows at or past m fetch row 0 of their
+// k-group instead, and a row tile that lies wholly at or past m (a kernel built for four row tiles under 33 to 48
+// rows) is fetched from row tile 0: the buffer holds no such tile.  What they fetch only reaches accumulator rows
+// that are never stored.
+FA_HD uint32_t decode_a_tile(uint32_t i, uint32_t m) { return i * 16 < m ? i : 0u; }          // the same in every lane
+FA_HD uint32_t decode_a_lane_byte(uint32_t i, uint32_t lane, uint32_t m) { return (i * 16 + lane % 16 < m ? lane : lane & 48u) * 16; }
+FA_HD uint64_t decode_a_byte(uint32_t i, uint32_t kt, uint32_t lane, uint32_t m, uint32_t k_tiles) {
+    return ((uint64_t)decode_a_tile(i, m) * k_tiles + kt) * 1024 + decode_a_lane_byte(i, lane, m);
+}
 // The weight-stationary split-k linear (w8a8_wstat_ksplit_kernel) leaves a partial tile set per row group: first
 // element of the set of (group, member, row group) in its workspace; nacc = row tiles of a row group x S x 4 items.
 FA_HD uint64_t rows_ksplit_partial_base(uint32_t group, uint32_t member, uint32_t s, uint32_t row_groups, uint32_t row_group,

@@ -101,7 +101,7 @@ __global__ void __launch_bounds__(NWAVES * 64)
     // skipped by predicate would make the count of outstanding loads depend on m.)
     uint32_t a_off[MT];
 #pragma unroll
-    for (int i = 0; i < MT; ++i) a_off[i] = ((uint32_t)i * 16 + (uint32_t)lane % 16 < m ? (uint32_t)lane : (uint32_t)lane & 48u) * 16;
+    for (int i = 0; i < MT; ++i) a_off[i] = ixm::decode_a_lane_byte((uint32_t)i, (uint32_t)lane, m);
     // What the epilogue needs from memory (scales, bias, residual, rotation, cache slot) is requested here,
     // ahead of the weight stream: asked for after the reduction it would cost the kernel one more memory
     // round trip with nothing else in flight.  Item q of this wavefront is accumulator wave + q * NWAVES
@@ -162,7 +162,7 @@ __global__ void __launch_bounds__(NWAVES * 64)
             a[s][0] = *(const v4i *)(pro_codes + pro_off + kt * 64);
         } else {
 #pragma unroll
-            for (int i = 0; i < MT; ++i) a[s][i] = *(const v4i *)(xq_tiled + ((uint64_t)i * k_tiles + kt) * 1024 + a_off[i]);
+            for (int i = 0; i < MT; ++i) a[s][i] = *(const v4i *)(xq_tiled + ((uint64_t)ixm::decode_a_tile((uint32_t)i, m) * k_tiles + kt) * 1024 + a_off[i]);
         }
     };
     auto load_slot = [&](int s, uint32_t it) {
@@ -343,11 +343,13 @@ __device__ __forceinline__ void store_unseen_b32(void *p, uint32_t v) {
     else if constexpr (POLICY == 1) asm volatile("global_store_dword %0, %1, off sc0" : : "v"(p), "v"(v));
     else asm volatile("global_store_dword %0, %1, off sc1" : : "v"(p), "v"(v));
 }
+// (a store of more than 64 bits must not be followed at once by a write to its data registers; for its own store
+// instructions the compiler keeps that distance, for these it cannot know: the s_nop keeps it)
 template <int POLICY>
 __device__ __forceinline__ void store_unseen_b128(void *p, v4i v) {
-    if constexpr (POLICY == 0) asm volatile("global_store_dwordx4 %0, %1, off" : : "v"(p), "v"(v));
-    else if constexpr (POLICY == 1) asm volatile("global_store_dwordx4 %0, %1, off sc0" : : "v"(p), "v"(v));
-    else asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v));
+    if constexpr (POLICY == 0) asm volatile("global_store_dwordx4 %0, %1, off\n\ts_nop 1" : : "v"(p), "v"(v));
+    else if constexpr (POLICY == 1) asm volatile("global_store_dwordx4 %0, %1, off sc0\n\ts_nop 1" : : "v"(p), "v"(v));
+    else asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(p), "v"(v));
 }
 __device__ __forceinline__ void store_unseen_b16(void *p, uint32_t v) {
     asm volatile("global_store_short %0, %1, off" : : "v"(p), "v"(v));
@@ -1046,9 +1048,11 @@ __global__ void __launch_bounds__(512)
     for (int i = 0; i < MT; ++i)
 #pragma unroll
         for (int j = 0; j < S; ++j) acc[i][j] = v4i{0, 0, 0, 0};
+    // (a row tile that lies wholly at or past m, the fourth one of 33 to 48 rows, need not exist in xq_tiled: its lanes
+    // fetch from row tile 0)
     uint32_t a_off[MT];
 #pragma unroll
-    for (int i = 0; i < MT; ++i) a_off[i] = ((uint32_t)i * 16 + (uint32_t)lane % 16 < m ? (uint32_t)lane : (uint32_t)lane & 48u) * 16;
+    for (int i = 0; i < MT; ++i) a_off[i] = ixm::decode_a_lane_byte((uint32_t)i, (uint32_t)lane, m);
     // epilogue operands, requested ahead of the weight stream by every member (only the last one uses them)
     float p_sx[NE], p_sw[NE], p_bias[NE], p_res[NE];
 #pragma unroll
@@ -1077,7 +1081,7 @@ __global__ void __launch_bounds__(512)
             b[s][j] = stream_load<true>((const v4i *)(b_base + ((uint64_t)nt * k_tiles + kt) * 1024));
         }
 #pragma unroll
-        for (int i = 0; i < MT; ++i) a[s][i] = *(const v4i *)(xq_tiled + ((uint64_t)i * k_tiles + kt) * 1024 + a_off[i]);
+        for (int i = 0; i < MT; ++i) a[s][i] = *(const v4i *)(xq_tiled + ((uint64_t)ixm::decode_a_tile((uint32_t)i, m) * k_tiles + kt) * 1024 + a_off[i]);
     };
     auto mma_slot = [&](int s) {
 #pragma unroll

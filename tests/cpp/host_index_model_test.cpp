@@ -296,6 +296,33 @@ static void rows_ksplit_cases() {
     }
 }
 
+// Activation fetch of the decode-shape int8 kernels: for every row count the kernels take, under the exact number of
+// row tiles (w8a8_skinny_kernel) and under the 1 / 2 / 4 the split-k form is built in (four row tiles from 33 rows on),
+// every lane's 16 bytes lie inside the tiled codes of ceil(m / 16) row tiles, a lane of a row below m fetches its own
+// row and k-group, and every other lane fetches bytes that some lane of a row below m fetches too.
+static void decode_a_cases() {
+    for (uint32_t k_tiles : {1u, 2u, 65u, 224u})
+        for (uint32_t m = 1; m <= 64; ++m) {
+            const uint32_t tiles = (m + 15) / 16;
+            const uint64_t bytes = (uint64_t)tiles * k_tiles * 1024;
+            for (uint32_t mt : {tiles, m <= 16 ? 1u : m <= 32 ? 2u : 4u})
+                for (uint32_t kt : {0u, k_tiles / 2, k_tiles - 1}) {
+                    std::set<uint64_t> own;
+                    for (uint32_t i = 0; i < mt; ++i)
+                        for (uint32_t lane = 0; lane < 64; ++lane) {
+                            const uint64_t b = decode_a_byte(i, kt, lane, m, k_tiles);
+                            CHECK(b % 16 == 0 && b + 16 <= bytes);
+                            if (i * 16 + lane % 16 < m) {
+                                CHECK(b == ((uint64_t)i * k_tiles + kt) * 1024 + lane * 16);
+                                own.insert(b);
+                            }
+                        }
+                    for (uint32_t i = 0; i < mt; ++i)
+                        for (uint32_t lane = 0; lane < 64; ++lane) CHECK(own.count(decode_a_byte(i, kt, lane, m, k_tiles)) == 1);
+                }
+        }
+}
+
 // SwiGLU form of the large-tile kernel: over all blocks every gate tile and every up tile of the weight is taken exactly
 // once, and accumulator tiles j and j + NTB / 4 of a wavefront column are gate and up of the same product tile.
 template <int NTB>
@@ -317,7 +344,10 @@ static void swiglu_tile_case(uint32_t f_tiles) {
 int main() {
     swiglu_tile_case<16>(8);
     swiglu_tile_case<16>(896);
+    swiglu_tile_case<8>(8);
+    swiglu_tile_case<8>(896);
     rows_ksplit_cases();
+    decode_a_cases();
     gemm_case<true, 14, 4>();
     gemm_case<true, 16, 4>();
     gemm_case<false, 14, 4>();

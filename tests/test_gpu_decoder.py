@@ -344,6 +344,8 @@ def test_prompt_pass_on_large_tiles_equals_the_pass_on_128_tiles_bit_for_bit():
     prompt = o.Rng(6).randint(0, shape["vocab"], shape["batch"] * l_new).astype(np.int32).reshape(shape["batch"], l_new)
     got = {}
     try:
+        # (every projection on the tiled GEMMs: at this width the weight-stationary kernel would take them, key 21 = 1)
+        fa.check(lib.fa_set_tuning(21, 1))
         # "big": large tiles, the gate | up GEMM with SwiGLU in its epilogue (256 x 256 tiles of eight gate and eight
         # up column tiles, products written) and the q | k | v GEMM with RoPE, the bf16 rounding and the K / V append
         # in its epilogue (a head per wavefront); "plain": large tiles, both left to their own passes (key 22 = 3);
@@ -362,6 +364,7 @@ def test_prompt_pass_on_large_tiles_equals_the_pass_on_128_tiles_bit_for_bit():
         fa.check(lib.fa_set_tuning(7, 0))
         fa.check(lib.fa_set_tuning(4, 0))
         fa.check(lib.fa_set_tuning(22, 0))
+        fa.check(lib.fa_set_tuning(21, 0))
     a = got["big"]
     assert np.all(np.isfinite(a[0])) and np.any(a[0] != 0)
     for other in ("plain", "small"):
