@@ -443,7 +443,7 @@ fa_status enqueue_prefill_chunk(fa_context *ctx, fa_decoder *d, PrefillBuffers &
         const bool swiglu_in_gemm = !rows_form(L.wgu) && L.wgu->n == 2 * F && k::gemm_w8a8_swiglu_applies(M, F, L.wgu->n_pad, L.wgu->k_pad);
         if (swiglu_in_gemm)
             k::gemm_w8a8_swiglu_mfma(t.xq.as<int8_t>(), (const int8_t *)L.wgu->codes->ptr, t.sx.as<float>(),
-                                     (const float *)L.wgu->scales->ptr, M, F, L.wgu->k_pad, t.gu.as<float>(), s);
+                                     (const float *)L.wgu->scales->ptr, M, F, L.wgu->k_pad, t.gu.as<float>(), cus, s);
         else
             gemm(L.wgu, t.gu.as<float>(), nullptr);
         k::swiglu_quantize_rows_i8(t.gu.as<float>(), t.xq.as<int8_t>(), t.sx.as<float>(), M, F, s, rows_form(L.wdown), swiglu_in_gemm);

@@ -1002,14 +1002,14 @@ void gemm_w8a8_mfma(const int8_t *aq, const int8_t *w_tiles, uint64_t m, uint64_
 // (the same two dequantizations and the same product).  Large-tile kernel only, 256 x 256 block tiles whose column
 // tiles are eight gate tiles and the eight up tiles of the same product columns.
 bool gemm_w8a8_swiglu_applies(uint64_t m, uint64_t f, uint64_t n_pad, uint64_t k_pad) {
-    return !(g_gemm_swiglu & 1) && !g_gemm_small_tiles && m >= 256 && f != 0 && f % 128 == 0 && n_pad == 2 * f && k_pad != 0 &&
+    // from 129 rows: below, the 128 x 128 kernel has one row of tiles for the whole device (one prompt of 130 / 200 / 250
+    // tokens through 32 layers: 5.50 / 6.06 / 6.36 -> 4.86 / 5.56 / 5.81 ms with the large tiles from 129 rows on)
+    return !(g_gemm_swiglu & 1) && !g_gemm_small_tiles && m >= 129 && f != 0 && f % 128 == 0 && n_pad == 2 * f && k_pad != 0 &&
            k_pad % 128 == 0;
 }
-void gemm_w8a8_swiglu_mfma(const int8_t *aq, const int8_t *w_tiles, const float *sx, const float *sw, uint64_t m, uint64_t f,
-                           uint64_t k_pad, float *out, hipStream_t s) {
-    if (m == 0 || f == 0) return;
-    const EpiI8Swiglu e{sx, sw, out, (uint32_t)f};
-    constexpr int NTB = 16;
+namespace {
+template <int NTB>
+void launch_swiglu(const int8_t *aq, const int8_t *w_tiles, const EpiI8Swiglu &e, uint64_t m, uint64_t f, uint64_t k_pad, hipStream_t s) {
     const size_t smem = (3 * 16 + 2 * (size_t)NTB) * 2048;
     static bool configured = false;
     if (!configured) {
@@ -1017,10 +1017,24 @@ void gemm_w8a8_swiglu_mfma(const int8_t *aq, const int8_t *w_tiles, const float 
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
         configured = true;
     }
-    const uint32_t mb = (uint32_t)((m + 255) / 256), nb = (uint32_t)(f / 128);
+    const uint32_t mb = (uint32_t)((m + 255) / 256), nb = (uint32_t)(f / (8 * NTB));      // NTB / 2 product tiles per block
     gemm_mfma_big_kernel<false, NTB, 4, EpiI8Swiglu><<<mb * nb, 512, smem, s>>>((const uint8_t *)aq, (const uint8_t *)w_tiles, (uint32_t)m,
                                                                               (uint32_t)(2 * f), (uint32_t)(2 * f / 16),
                                                                               (uint32_t)(k_pad / 128), mb, nb, e);
+}
+}  // namespace
+void gemm_w8a8_swiglu_mfma(const int8_t *aq, const int8_t *w_tiles, const float *sx, const float *sw, uint64_t m, uint64_t f,
+                           uint64_t k_pad, float *out, int num_cus, hipStream_t s) {
+    if (m == 0 || f == 0) return;
+    const EpiI8Swiglu e{sx, sw, out, (uint32_t)f};
+    // 256 x 256 tiles (eight gate and eight up column tiles), or 256 x 128 where the wide tiles would cover at most half the
+    // device (up to 256 rows at d_ffn 14336: 112 wide tiles, 224 narrow ones; one prompt of 200 tokens through 32 layers
+    // 5.56 -> 5.21 ms).  With more rows three rounds of narrow tiles measured no better than two of wide ones.
+    const uint64_t mb = (m + 255) / 256;
+    if (g_gemm_ntb == 8 || (g_gemm_ntb == 0 && mb * (f / 128) * 2 <= (uint64_t)num_cus))
+        launch_swiglu<8>(aq, w_tiles, e, m, f, k_pad, s);
+    else
+        launch_swiglu<16>(aq, w_tiles, e, m, f, k_pad, s);
 }
 
 // q | k | v projection of a prompt pass with RoPE, the bf16 rounding and the K / V append in the epilogue (heads of 128 dims:

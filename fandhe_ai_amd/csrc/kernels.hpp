@@ -227,7 +227,7 @@ void gemm_w8a8_mfma(const int8_t *aq, const int8_t *w_tiles, uint64_t m, uint64_
                     uint64_t k_pad, const EpilogueI8 &ep, int num_cus, hipStream_t s, void *workspace = nullptr,
                     uint64_t workspace_bytes = 0, const SplitKArea *sk = nullptr);
 uint64_t gemm_w8a8_workspace_bytes(uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad, int num_cus);
-// The gate | up projection with SwiGLU in its epilogue (large-tile kernel, m >= 256, f a multiple of 128, k_pad of 128):
+// The gate | up projection with SwiGLU in its epilogue (large-tile kernel, m >= 129, f a multiple of 128, k_pad of 128):
 // w_tiles is the [k, 2 f] weight with the gate columns first; out receives silu(gate) * up, f32 [m, f], bit for bit
 // what gemm_w8a8_mfma into an [m, 2 f] buffer followed by the SwiGLU pass computes.
 extern int g_gemm_pair;       // 1: one block per tile on the 256 x 128 tiles of the large-tile kernel; 2: shared tiles only
@@ -235,7 +235,7 @@ extern int g_gemm_pair;       // 1: one block per tile on the 256 x 128 tiles of
 extern int g_gemm_swiglu;     // bit 0: SwiGLU stays a pass of its own; bit 1: so do RoPE and the K / V append (below)
 bool gemm_w8a8_swiglu_applies(uint64_t m, uint64_t f, uint64_t n_pad, uint64_t k_pad);
 void gemm_w8a8_swiglu_mfma(const int8_t *aq, const int8_t *w_tiles, const float *sx, const float *sw, uint64_t m, uint64_t f,
-                           uint64_t k_pad, float *out, hipStream_t s);
+                           uint64_t k_pad, float *out, int num_cus, hipStream_t s);
 // Which kernel the two launchers pick for a shape under the current tuning knobs: big_ntb column tiles of
 // 16 per block of the large-tile kernel (0: the 128 x 128 kernel), wavefronts per block, k splits.
 struct GemmPlan {
