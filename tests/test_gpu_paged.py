@@ -407,6 +407,10 @@ def test_device_tables_flag_violations_with_nan():
     got = o.from_bf16(be.download_owned(be.paged_attention_forward_device(
         be.upload(q), be.upload(kp), be.upload(vp), be.upload(bad), be.upload(lens), args)))
     assert np.all(np.isfinite(got[0])) and np.all(np.isnan(got[1]))
+    # a row of length zero (device lengths are not validated) streams nothing and comes back as zeros
+    got0 = o.from_bf16(be.download_owned(be.paged_attention_forward_device(
+        be.upload(q), be.upload(kp), be.upload(vp), be.upload(tables), be.upload(np.array([0, 20], np.uint32)), args)))
+    assert not got0[0].any() and np.all(np.isfinite(got0[1])) and got0[1].any()
     # append with device slots: out-of-range slots are skipped, valid ones written
     kpool, vpool = be.alloc_zeroed((num_blocks, 16, e_kv), fa.capi.BF16), be.alloc_zeroed((num_blocks, 16, e_kv), fa.capi.BF16)
     rows = o.to_bf16(rng.randn((2, e_kv)))
