@@ -432,7 +432,6 @@ __global__ void __launch_bounds__(128 * WM) __attribute__((amdgpu_waves_per_eu(W
     // requests stay in flight across the wait at the top of a stage (with both operands one stage ahead
     // the path from L2 runs dry there; a third stage of both does not fit).
     constexpr int NSA = 3, NSB = 2;
-    uint8_t *const lds_b0 = lds + NSA * A_STAGE;
     // Load instruction `idx` of a stage: tile wave + NWAVES (idx / 2), slice idx % 2.  They are spread over
     // the multiply groups of the stage before, which keeps a steady stream of requests going to the L2
     // instead of one burst per stage.
