@@ -19,6 +19,7 @@ using namespace fa;
 
 namespace fa {
 extern int g_decode_waves;
+int g_prefill_rows = 0;      // rows per chunk of a prompt pass (tuning key 25; below 256: the built-in figure)
 namespace k {
 extern int g_weight_prefetch;
 }
@@ -814,9 +815,14 @@ static fa_status prefill_impl(fa_context *ctx, fa_decoder *d, const int32_t *tok
                 return fail(FA_ERR_INVALID_ARGUMENT, "paged_kv: row " + std::to_string(b) + " entry " + std::to_string(i) +
                                                          " is not a valid block id");
     }
-    // chunks of at most kRows rows per pass bound the activation memory (the widest is [rows, 2 d_ffn] f32)
-    constexpr uint64_t kRows = 4096;
-    if ((verify || padded) && (uint64_t)B * l_new > kRows)
+    // chunks of at most kRows rows per pass bound the activation memory (the widest is [rows, 2 d_ffn] f32: 0.9 GB at the
+    // benchmark's width).  8192 rather than 4096: the q | k | v projection at 6144 columns is 24 column blocks of the
+    // large-tile GEMM, 384 tiles = one and a half rounds of the device at 4096 rows, 768 = three whole rounds at 8192
+    // (a prompt pass of 4 x 2048 tokens on one box: 75.9 ms in chunks of 4096 rows, 74.9 in one of 8192; tuning key 25).
+    // Passes that keep every row's logits stay at 4096.
+    const uint64_t kRows = g_prefill_rows >= 256 ? (uint64_t)g_prefill_rows : 8192;
+    constexpr uint64_t kRowsChecked = 4096;
+    if ((verify || padded) && (uint64_t)B * l_new > kRowsChecked)
         return fail(FA_ERR_INVALID_ARGUMENT, "decoder: at most 4096 rows (batch x tokens) per verification or padded prompt pass");
     const uint32_t lc_max = (uint32_t)std::max<uint64_t>(1, std::min<uint64_t>(l_new, kRows / B));
     const uint64_t M = (uint64_t)B * lc_max;

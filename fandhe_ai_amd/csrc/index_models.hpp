@@ -32,9 +32,19 @@ struct BigLds {
 };
 
 // Blocks of one XCD (the hardware deals consecutive ids round-robin over 8 XCDs) take consecutive tiles, m fastest.
+// With eight or more row blocks and a whole number of column blocks per XCD, an XCD walks its column blocks for eight
+// row blocks at a time: the 32 tiles its compute units hold together are then 8 x 4 (12 operand panels per k step)
+// rather than 16 x 2 or 32 x 1 (18 or 33), which is what its L2 has to fetch.
 FA_HD void big_block_tile(uint32_t bid, uint32_t m_blocks, uint32_t n_blocks, uint32_t *mb, uint32_t *nb) {
     const uint32_t total = m_blocks * n_blocks;
     if (total % 8 == 0) bid = (bid % 8) * (total / 8) + bid / 8;
+    if (n_blocks % 8 == 0 && m_blocks % 8 == 0) {
+        const uint32_t nb8 = n_blocks / 8, xcd = bid / (total / 8), l = bid % (total / 8);
+        const uint32_t chunk = l / (8 * nb8), r = l % (8 * nb8);
+        *mb = chunk * 8 + r % 8;
+        *nb = xcd * nb8 + r / 8;
+        return;
+    }
     *mb = bid % m_blocks;
     *nb = bid / m_blocks;
 }

@@ -515,7 +515,7 @@ fa_status fa_decoder_read_row_sampling(fa_context *ctx, fa_decoder *dec, fa_row_
 /* Prompt ingestion: l_new tokens per installed sequence (tokens [batch, l_new],
  * host array), written behind what each sequence has cached, on the
  * prefill-shape GEMMs and the prefill form of the attention kernel, in chunks of
- * at most 4096 rows.  Leaves the logits of every sequence's last prompt token
+ * at most 8192 rows.  Leaves the logits of every sequence's last prompt token
  * and its greedy next token resident, exactly as a decode step does, so
  * fa_decoder_step continues from there.  The per-row arithmetic is the decode
  * step's: a prompt token leaves the K / V rows it would leave if it were

@@ -146,8 +146,8 @@ static void gemm_case() {
 }
 
 static void gemm_block_map() {
-    for (uint32_t mbs : {1u, 2u, 3u, 8u, 9u})
-        for (uint32_t nbs : {1u, 4u, 7u, 56u, 64u}) {
+    for (uint32_t mbs : {1u, 2u, 3u, 8u, 9u, 16u, 32u})
+        for (uint32_t nbs : {1u, 4u, 7u, 16u, 24u, 56u, 64u, 112u}) {
             std::set<std::pair<uint32_t, uint32_t>> tiles;
             for (uint32_t bid = 0; bid < mbs * nbs; ++bid) {
                 uint32_t mb, nb;

@@ -272,9 +272,9 @@ PREFILL_SHAPES = [
     # the benchmark's width: 72 rows against 4096 / 6144 / 28672 / 4096-column weights (k split across blocks)
     dict(n_layers=1, d_model=4096, n_heads=32, n_kv_heads=8, d_ffn=14336, vocab=32000, batch=3, ctxs=[0, 37, 400], l_new=24,
          numpy_fill=True),
-    # 8 x 600 rows: two chunks (512 + 88 tokens per sequence)
+    # 8 x 1100 rows: two chunks (1024 + 76 tokens per sequence)
     dict(n_layers=1, d_model=256, n_heads=4, n_kv_heads=1, d_ffn=256, vocab=300, batch=8, ctxs=[0, 3, 9, 20, 0, 64, 7, 15],
-         l_new=600),
+         l_new=1100),
 ]
 
 

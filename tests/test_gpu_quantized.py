@@ -489,6 +489,35 @@ def test_int8_prefill_gemm_rows_sampled_at_full_size():
     assert_bf16_rounding_of("gemm_w8a8 bf16", out_bf, got)
 
 
+@pytest.mark.parametrize("m,k,n", [(4000, 256, 2048), (8192, 128, 4096), (4096, 384, 6144)], ids=["16x8", "32x16", "16x24"])
+def test_int8_large_tile_kernel_tile_order_with_many_row_blocks(m, k, n):
+    """Sixteen and thirty-two row blocks of 256 against a multiple of eight column blocks: every XCD walks its column
+    blocks for eight row blocks at a time.  Sampled rows of every row block bit-exact against the oracle, and the
+    column sums of all accumulators equal (sum of the rows of a) @ w: every tile was written once, by the right block."""
+    fa = _fa()
+    be = ops()
+    lib = fa.capi.lib
+    rng = np.random.default_rng(m + n)
+    aq = rng.integers(-127, 128, size=(m, k), dtype=np.int8)
+    wq = rng.integers(-127, 128, size=(k, n), dtype=np.int8)
+    sx = rng.uniform(0.01, 0.05, size=m).astype(np.float32)
+    sw = rng.uniform(1e-4, 1e-3, size=n).astype(np.float32)
+    qw = be.import_quantized_weight(wq, sw)
+    try:
+        fa.check(lib.fa_set_tuning(7, 16))                # 256 x 256 tiles whatever the shape would pick
+        assert _gemm_plan(fa, be, m, qw).big_ntb == 16
+        out, acc = be.gemm_w8a8(be.upload(aq), be.upload(sx), qw, fa.capi.F32, want_acc=True)
+    finally:
+        fa.check(lib.fa_set_tuning(7, 0))
+    got_acc, got = be.download_owned(acc), be.download_owned(out)
+    rows = np.unique(np.r_[np.arange(0, m, 256), np.arange(255, m, 256), m - 1, 1000:1003])
+    want_acc = o.gemm_i8_i32(np.ascontiguousarray(aq[rows]), wq)
+    assert np.array_equal(got_acc[rows], want_acc)
+    assert np.array_equal(got[rows], o.dequant_i32(want_acc, np.ascontiguousarray(sx[rows]), sw))
+    colsum = aq.astype(np.int64).sum(axis=0)
+    assert np.array_equal(got_acc.astype(np.int64).sum(axis=0), colsum @ wq.astype(np.int64))
+
+
 def test_fp8_quantizer_bit_exact_and_gemm_within_stated_bound():
     """e4m3 per-tensor: codes and scale bit-exact.  GEMM: the oracle sums the exact products in f64 and
     rounds once.  The f8f6f4 matrix instruction aligns the 128 products of one issue to their largest
