@@ -21,7 +21,7 @@ int g_skinny_ntw = 0;      // tuning overrides (0 = heuristic)
 int g_skinny_waves = 0;
 int g_weight_prefetch = 0;   // 1: row kernels pull nothing for the linear that follows them
 int g_rows_kernel = 0;      // weight-stationary kernel for a few hundred rows: 0 by shape, 1 never, 2 whenever it can run
-int g_skinny_astat = 0;     // activation-stationary kernel: 0 by shape, 1 never, 2 whenever it can run
+int g_skinny_astat = 0;     // activation-stationary kernel: 0 by shape, 1 never, 2 whenever it can run, 3 by shape but not the 33 to 64 row form
 int g_skinny_ksplit = 0;    // split k over the blocks of an XCD: 0 by shape, 1 never, 2 whenever it can run (agent-scope
                             // meeting), 3 whenever it can run (meeting in the XCD's L2), 4 by shape but agent scope
 int g_skinny_ksplit_s = 0;  // members per group of the split (0 by shape, 2 or 4)
@@ -654,6 +654,165 @@ __global__ void __launch_bounds__(512)
         if (u + gridDim.x >= n_units) break;
         load_unit(u + 2 * gridDim.x, b0, ue0);
         finish_unit(u + gridDim.x, b1, ue1, 1);
+    }
+}
+
+// The same for 33 to 64 rows (three or four row tiles).  The activations of four row tiles fill half of a wavefront's
+// registers, so the weights have one register set instead of two: every k-tile's pair of weight tiles is multiplied
+// and its registers are refilled at once with the same k-tile of the block's next unit, which keeps a whole unit of
+// weight loads in flight all the time.  A wavefront finishes two of the 4 MT (row tile, element) items of a unit.
+// The partial tiles of two units (2 x 8 wavefronts x 8 MT items x 256 bytes) live in dynamic LDS.
+template <int MT, int MODE>
+__global__ void __launch_bounds__(512)
+    w8a8_astat_wide_kernel(const int8_t *__restrict__ xq_tiled, const int8_t *__restrict__ w_tiles, uint32_t m, uint32_t n,
+                           uint32_t n_tiles, uint32_t k_tiles, uint32_t n_units, EpiI8 ep) {
+    constexpr bool SWIGLU = MODE == kEpiSwiglu;
+    constexpr int NW = 8, KTW = 8, NACC = MT * 2 * 4, NQ = (MT * 4 + NW - 1) / NW;
+    static_assert(MT == 3 || MT == 4, "three or four row tiles; fewer take w8a8_astat_kernel");
+    extern __shared__ __attribute__((aligned(16))) int red_wide[];          // [2][NW][NACC][64]
+    auto red = [&](int buf, int w, int idx) -> int * { return red_wide + (((size_t)buf * NW + w) * NACC + idx) * 64; };
+    const int lane = threadIdx.x % 64;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+    const uint32_t last_kt = k_tiles - 1, last_tile = n_tiles - 1;
+
+    // activations of this wavefront's k-tiles (clamped repeats past the end are never multiplied)
+    v4i a[KTW][MT];
+#pragma unroll
+    for (int t = 0; t < KTW; ++t) {
+        uint32_t kt = wave + NW * t;
+        kt = kt < k_tiles ? kt : last_kt;
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+            a[t][i] = *(const v4i *)(xq_tiled + ((uint64_t)ixm::decode_a_tile((uint32_t)i, m) * k_tiles + kt) * 1024 + (uint64_t)lane * 16);
+    }
+    auto tile_of = [&](uint32_t u, int j) -> uint32_t {
+        uint32_t nt = SWIGLU ? u + j * (n_tiles / 2) : 2 * u + j;
+        return nt < last_tile ? nt : last_tile;
+    };
+    // item q of this wavefront: element idx % 4 of row tile idx / 4, idx = wave + 8 q
+    uint32_t e_row[NQ];
+    bool e_ok[NQ];
+    float e_sx[NQ];
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+        const int idx = wave + NW * q;
+        e_row[q] = (uint32_t)(idx / 4) * 16 + 4 * ((uint32_t)lane / 16) + (uint32_t)(idx % 4);
+        e_ok[q] = idx < MT * 4 && e_row[q] < m;
+        e_sx[q] = e_ok[q] ? ep.sx[e_row[q]] : 0.0f;
+    }
+    struct UnitEpi {
+        float sw[2], bias[2], res[NQ][2];
+    };
+    auto load_epi = [&](uint32_t u, UnitEpi &ue) {
+        u = u < n_units ? u : n_units - 1;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            ue.sw[j] = ue.bias[j] = 0.0f;
+            const uint32_t col = SWIGLU ? u * 16 + lane % 16 + j * (n / 2) : (2 * u + j) * 16 + lane % 16;
+            if (col < n) {
+                ue.sw[j] = ep.sw[col];
+                if constexpr (!SWIGLU) {
+                    if (ep.bias) ue.bias[j] = ep.bias[col];
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) {
+                ue.res[q][j] = 0.0f;
+                if constexpr (!SWIGLU) {
+                    if (ep.residual && e_ok[q] && col < n) ue.res[q][j] = ep.residual[(uint64_t)e_row[q] * n + col];
+                }
+            }
+        }
+    };
+    v4i b[KTW][2];
+    auto load_w = [&](uint32_t u, int t) {
+        u = u < n_units ? u : n_units - 1;
+        uint32_t kt = wave + NW * t;
+        kt = kt < k_tiles ? kt : last_kt;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+            b[t][j] = stream_load<true>((const v4i *)(w_tiles + ((uint64_t)tile_of(u, j) * k_tiles + kt) * 1024 + (uint64_t)lane * 16));
+    };
+
+    UnitEpi ue;
+    uint32_t u = blockIdx.x;
+    load_epi(u, ue);
+#pragma unroll
+    for (int t = 0; t < KTW; ++t) load_w(u, t);
+    for (int it = 0; u < n_units; u += gridDim.x, ++it) {
+        const int buf = it & 1;
+        UnitEpi ue_next;
+        load_epi(u + gridDim.x, ue_next);
+        v4i acc[MT][2];
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) acc[i][j] = v4i{0, 0, 0, 0};
+#pragma unroll
+        for (int t = 0; t < KTW; ++t) {
+            if ((uint32_t)(wave + NW * t) < k_tiles) {
+#pragma unroll
+                for (int i = 0; i < MT; ++i)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[t][i], b[t][j], acc[i][j], 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);                // the refill right behind its consumer
+            load_w(u + gridDim.x, t);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) red(buf, wave, (i * 2 + j) * 4 + e)[lane] = acc[i][j][e];
+        __syncthreads();      // buffer buf is rewritten two units later, behind the barrier of the unit in between
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) {
+            const int idx = wave + NW * q;
+            if (idx >= MT * 4) break;
+            const int i = idx / 4, e = idx % 4;
+            int s0 = 0, s1 = 0;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) {
+                s0 += red(buf, w, (i * 2 + 0) * 4 + e)[lane];
+                s1 += red(buf, w, (i * 2 + 1) * 4 + e)[lane];
+            }
+            const uint32_t row = e_row[q];
+            if constexpr (SWIGLU) {
+                const uint32_t f = n / 2, col = u * 16 + lane % 16;
+                float av = 0.0f;
+                if (row < m && col < f) {
+                    float vg = __fmul_rn((float)s0, __fmul_rn(e_sx[q], ue.sw[0]));
+                    float vu = __fmul_rn((float)s1, __fmul_rn(e_sx[q], ue.sw[1]));
+                    float act = silu_f32(vg) * vu;
+                    ((float *)ep.out)[(uint64_t)row * f + col] = act;
+                    av = fabsf(act);
+                }
+#pragma unroll
+                for (int off = 1; off < 16; off <<= 1) av = fmaxf(av, __shfl_xor(av, off, 64));
+                if (lane % 16 == 0 && row < m) ep.pmax[(uint64_t)row * (n_tiles / 2) + u] = av;
+            } else {
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const uint32_t col = (2 * u + j) * 16 + lane % 16;
+                    const int sum = j ? s1 : s0;
+                    if (row < m && col < n) {
+                        uint64_t o = (uint64_t)row * n + col;
+                        if (ep.acc_out) ep.acc_out[o] = sum;
+                        float v = __fmul_rn((float)sum, __fmul_rn(e_sx[q], ue.sw[j]));
+                        if (ep.bias) v = __fadd_rn(v, ue.bias[j]);
+                        if (ep.residual) v = __fadd_rn(ue.res[q][j], v);
+                        if (ep.out_bf16)
+                            ((uint16_t *)ep.out)[o] = f32_to_bf16(v);
+                        else
+                            ((float *)ep.out)[o] = v;
+                    }
+                }
+            }
+        }
+        ue = ue_next;
     }
 }
 
@@ -1573,6 +1732,30 @@ inline bool astat_applies(uint64_t n_units, uint64_t k_tiles, int num_cus) {
     return n_units >= 3 * (uint64_t)num_cus;
 }
 
+// w8a8_astat_wide_kernel for 33 to 64 rows: as many blocks as compute units (or units), 96 / 128 KiB of dynamic LDS
+template <int MODE>
+void launch_astat_wide(uint64_t m, unsigned blocks, hipStream_t s, const int8_t *xq_tiled, const int8_t *w_tiles, uint32_t n,
+                       uint32_t n_tiles, uint32_t k_tiles, uint32_t n_units, const EpiI8 &e) {
+    auto go = [&](auto mt) {
+        constexpr int MT = decltype(mt)::value;
+        const size_t smem = (size_t)2 * 8 * (MT * 8) * 64 * 4;
+        static bool configured = false;
+        if (!configured) {
+            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&w8a8_astat_wide_kernel<MT, MODE>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+            configured = true;
+        }
+        w8a8_astat_wide_kernel<MT, MODE><<<blocks, 512, smem, s>>>(xq_tiled, w_tiles, (uint32_t)m, n, n_tiles, k_tiles, n_units, e);
+    };
+    if (m <= 48)
+        go(std::integral_constant<int, 3>{});
+    else
+        go(std::integral_constant<int, 4>{});
+}
+inline bool astat_wide_applies(uint64_t m, uint64_t n_units, uint64_t k_tiles, int num_cus) {
+    return g_skinny_astat != 3 && m > 32 && m <= 64 && astat_applies(n_units, k_tiles, num_cus);
+}
+
 // Row tiles per block by the number of rows (16 each, at most 64 rows), 4 or 8 wavefronts.
 template <int NTW, int MODE, typename... A>
 void launch_w8a8_rows(uint64_t m, int waves, unsigned grid, hipStream_t s, A... args) {
@@ -1744,7 +1927,8 @@ WeightPrefetch prefetch_for_linear_w8a8_skinny(const int8_t *w_tiles, uint64_t m
         pf.ksplit = (uint32_t)kp.s;
         return pf;
     }
-    if (m <= 32 && astat_applies((n_tiles + 1) / 2, k_tiles, num_cus)) {      // block b starts with unit b = tiles 2 b, 2 b + 1
+    if ((m <= 32 && astat_applies((n_tiles + 1) / 2, k_tiles, num_cus)) ||
+        astat_wide_applies(m, (n_tiles + 1) / 2, k_tiles, num_cus)) {           // block b starts with unit b = tiles 2 b, 2 b + 1
         const uint32_t n_units = (n_tiles + 1) / 2;
         return make_prefetch(w_tiles, (uint32_t)std::min<uint64_t>(n_units, (uint64_t)num_cus), n_tiles, k_tiles, 0, 2, n_tiles > 1 ? 1 : 0, budget);
     }
@@ -1826,6 +2010,12 @@ void linear_w8a8_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t 
             w8a8_astat_kernel<1, 8, kEpiPlain><<<blocks, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, n_units, e, RowPrologue{});
         else
             w8a8_astat_kernel<2, 8, kEpiPlain><<<blocks, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, n_units, e, RowPrologue{});
+        return;
+    }
+    if (astat_wide_applies(m, (n_tiles + 1) / 2, k_tiles, num_cus)) {
+        const unsigned n_units = (n_tiles + 1) / 2;
+        launch_astat_wide<kEpiPlain>(m, (unsigned)std::min<uint64_t>(n_units, (uint64_t)num_cus), s, xq_tiled, w_tiles, (uint32_t)n, n_tiles,
+                                     k_tiles, n_units, e);
         return;
     }
     int ntw, waves;
@@ -1966,6 +2156,11 @@ void linear_w8a8_swiglu_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, co
             w8a8_astat_kernel<1, 8, kEpiSwiglu><<<blocks, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, n_tiles / 2, e, RowPrologue{});
         else
             w8a8_astat_kernel<2, 8, kEpiSwiglu><<<blocks, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, n_tiles / 2, e, RowPrologue{});
+        return;
+    }
+    if (astat_wide_applies(m, n_tiles / 2, k_tiles, num_cus)) {
+        launch_astat_wide<kEpiSwiglu>(m, (unsigned)std::min<uint64_t>(n_tiles / 2, (uint64_t)num_cus), s, xq_tiled, w_tiles, (uint32_t)n,
+                                      n_tiles, k_tiles, n_tiles / 2, e);
         return;
     }
     launch_w8a8_rows<2, kEpiSwiglu>(m, waves, n_tiles / 2, s, xq_tiled, w_tiles, (uint32_t)m, (uint32_t)n, n_tiles, k_tiles, e);

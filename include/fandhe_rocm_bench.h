@@ -58,7 +58,8 @@ fa_status fa_probe_l2_path(fa_context *ctx, const fa_buffer *cold, uint64_t cold
  * key 3: nonzero launches only the streaming kernel of the decode attention and
  *        leaves the output unwritten (for timing that kernel by itself);
  * key 4: nonzero keeps the 128 x 128 block tile of the prefill GEMMs for every shape;
- * key 5: activation-stationary decode linears: 1 never, 2 whenever the shape allows;
+ * key 5: activation-stationary decode linears: 1 never, 2 whenever the shape allows, 3 by shape but 33 to 64 rows stay
+ *        on the block-per-tile kernels;
  * key 6: wavefronts per block of the large-tile prefill GEMMs (4 or 16; default 8);
  * key 7: column tiles of 16 per block of the large-tile prefill GEMMs (14 or 16);
  * key 8: nonzero sends attention with more than one new token per row to the generic

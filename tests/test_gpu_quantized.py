@@ -285,7 +285,8 @@ def test_w8a8_ragged_shapes():
 def test_w8a8_activation_stationary_kernel_is_bit_exact():
     """The decode-shape linear that keeps the activations in registers and walks several column-tile
     pairs per block (chosen by shape for wide weights; forced here so that few units per block, ragged
-    widths and k-tile counts that do not fill every wavefront are covered too)."""
+    widths and k-tile counts that do not fill every wavefront are covered too).  33 to 64 rows take the form with one
+    weight register set refilled behind every multiply (three and four row tiles, two items per wavefront)."""
     fa = _fa()
     be = ops()
     rng = o.Rng(77)
@@ -293,7 +294,7 @@ def test_w8a8_activation_stationary_kernel_is_bit_exact():
     fa.check(lib.fa_set_tuning(5, 2))
     try:
         for m, k, n in ((32, 4096, 28672), (16, 4096, 6144), (3, 100, 37), (32, 130, 70), (7, 4096, 33), (17, 1000, 16400),
-                        (1, 64, 16)):
+                        (1, 64, 16), (33, 4096, 6144), (48, 1000, 16400), (49, 130, 70), (64, 4096, 32000), (40, 64, 16)):
             x = rng.randn((m, k))
             w = rng.randn((k, n), std=0.05)
             bias = rng.randn((n,))
