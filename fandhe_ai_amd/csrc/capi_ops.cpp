@@ -19,7 +19,7 @@ extern int g_skinny_ntw, g_skinny_waves, g_skinny_astat, g_gemm_small_tiles, g_g
 }
 int g_decode_waves = 0;
 int g_prefill_generic = 0;
-extern int g_prefill_rows, g_decode_partials_only, g_prefill_block_form, g_prefill_block_waves, g_prefill_block_split, g_prefill_block_cols;
+extern int g_prefill_rows, g_prefill_fused_rows, g_decode_partials_only, g_prefill_block_form, g_prefill_block_waves, g_prefill_block_split, g_prefill_block_cols;
 }  // namespace fa
 
 namespace {
@@ -102,6 +102,7 @@ fa_status fa_set_tuning(int32_t key, int32_t value) {
         case 23: fa::g_prefill_block_cols = value; return FA_OK;
         case 24: k::g_gemm_pair = value; return FA_OK;
         case 25: fa::g_prefill_rows = value; return FA_OK;
+        case 26: fa::g_prefill_fused_rows = value; return FA_OK;
     }
     return fail(FA_ERR_INVALID_ARGUMENT, "fa_set_tuning: unknown key");
 }

@@ -20,6 +20,7 @@ using namespace fa;
 namespace fa {
 extern int g_decode_waves;
 int g_prefill_rows = 0;      // rows per chunk of a prompt pass (tuning key 25; below 256: the built-in figure)
+int g_prefill_fused_rows = 0;   // prompt passes of at most 64 rows: 0 the decode step's fused projections, 1 plain ones (tuning key 26)
 namespace k {
 extern int g_weight_prefetch;
 }
@@ -416,8 +417,14 @@ fa_status enqueue_prefill_chunk(fa_context *ctx, fa_decoder *d, PrefillBuffers &
     for (uint32_t li = 0; li < c.n_layers; ++li) {
         const fa_decoder::Layer &L = d->layers[li];
         norm_quantize((const float *)L.attn_norm->ptr, L.wqkv);
-        // on the large-tile GEMM the q | k | v projection does RoPE, the bf16 rounding and the K / V append in its epilogue
-        if (!rows_form(L.wqkv) &&
+        // at most 64 rows: the decode step's fused projection (RoPE, the bf16 rounding and the K / V append in the epilogue
+        // of the decode kernel); on the large-tile GEMM the q | k | v projection does the same in its epilogue
+        if (decode_form && g_prefill_fused_rows != 1) {
+            const k::QkvRopeTargets qt{t.cos_sin.as<float>(), t.slots.as<uint32_t>(), t.q_bf.as<uint16_t>(), (uint16_t *)L.k_pool->ptr,
+                                       (uint16_t *)L.v_pool->ptr, c.n_heads, c.n_kv_heads, c.head_dim, pool_rows};
+            k::linear_w8a8_qkv_rope_skinny(t.xq.as<int8_t>(), (const int8_t *)L.wqkv->codes->ptr, t.sx.as<float>(),
+                                           (const float *)L.wqkv->scales->ptr, M, L.wqkv->n_pad, L.wqkv->k_pad, qt, s);
+        } else if (!rows_form(L.wqkv) &&
             k::gemm_w8a8_qkv_rope_applies(M, L.wqkv->n, L.wqkv->n_pad, L.wqkv->k_pad, c.n_heads, c.n_kv_heads, c.head_dim, cus)) {
             const k::QkvRopeTargets qt{t.cos_sin.as<float>(), t.slots.as<uint32_t>(), t.q_bf.as<uint16_t>(), (uint16_t *)L.k_pool->ptr,
                                        (uint16_t *)L.v_pool->ptr, c.n_heads, c.n_kv_heads, c.head_dim, pool_rows};
@@ -439,6 +446,17 @@ fa_status enqueue_prefill_chunk(fa_context *ctx, fa_decoder *d, PrefillBuffers &
             k::quantize_rows_i8(t.attn.ptr, true, t.xq.as<int8_t>(), nullptr, t.sx.as<float>(), M, M, L.wo->k, L.wo->k_pad, s);
         gemm(L.wo, t.h.as<float>(), t.h.as<float>());
         norm_quantize((const float *)L.ffn_norm->ptr, L.wgu);
+        if (decode_form && g_prefill_fused_rows != 1 && L.wgu->n == 2 * F && F / 16 <= (uint64_t)c.n_heads * c.head_dim + 2 * EKV) {
+            // at most 64 rows: the decode step's gate | up kernel (SwiGLU in the epilogue: products and their partial
+            // maxima per 16 columns) and its quantizer from those maxima; t.qkv is free here and holds the maxima
+            k::linear_w8a8_swiglu_skinny(t.xq.as<int8_t>(), (const int8_t *)L.wgu->codes->ptr, t.sx.as<float>(),
+                                         (const float *)L.wgu->scales->ptr, M, L.wgu->n, L.wgu->n_pad, L.wgu->k_pad, t.gu.as<float>(),
+                                         t.qkv.as<float>(), 4, cus, s, nullptr);
+            k::quantize_rows_from_pmax(t.gu.ptr, false, t.qkv.as<float>(), (uint32_t)(F / 16), t.xq.as<int8_t>(), t.sx.as<float>(), M,
+                                       M_pad, F, s);
+            gemm(L.wdown, t.h.as<float>(), t.h.as<float>());
+            continue;
+        }
         // on the large-tile GEMM the gate | up projection takes SwiGLU into its epilogue and leaves the products
         // ([M, F] instead of [M, 2 F] written and read back); the quantizer behind it is the same either way
         const bool swiglu_in_gemm = !rows_form(L.wgu) && L.wgu->n == 2 * F && k::gemm_w8a8_swiglu_applies(M, F, L.wgu->n_pad, L.wgu->k_pad);

@@ -106,7 +106,9 @@ fa_status fa_probe_l2_path(fa_context *ctx, const fa_buffer *cold, uint64_t cold
  * key 24: the large-tile int8 GEMM on 256 x 128 tiles: 0: when those tiles cover at most half the device, two or four
  *        same-XCD blocks share a tile, a part of k each; 1: one block per tile; 2: shared tiles only where the tiles
  *        alone cover half the device (pairs);
- * key 25: rows (sequences x tokens) per chunk of a prompt pass, from 256 up; anything smaller: the built-in 8192. */
+ * key 25: rows (sequences x tokens) per chunk of a prompt pass, from 256 up; anything smaller: the built-in 8192;
+ * key 26: prompt passes of at most 64 rows: 0: q | k | v and gate | up on the decode step's fused kernels (RoPE and the
+ *        K / V append, SwiGLU, in the epilogues), 1: plain projections and separate passes. */
 fa_status fa_set_tuning(int32_t key, int32_t value);
 
 /* What the context found when it was created: xcd_local = 1 when workgroups b and b + 8 of a launch were seen to
