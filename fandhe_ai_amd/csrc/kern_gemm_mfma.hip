@@ -1001,9 +1001,10 @@ void gemm_w8a8_mfma(const int8_t *aq, const int8_t *w_tiles, uint64_t m, uint64_
 // (the same two dequantizations and the same product).  Large-tile kernel only, 256 x 256 block tiles whose column
 // tiles are eight gate tiles and the eight up tiles of the same product columns.
 bool gemm_w8a8_swiglu_applies(uint64_t m, uint64_t f, uint64_t n_pad, uint64_t k_pad) {
-    // from 129 rows: below, the 128 x 128 kernel has one row of tiles for the whole device (one prompt of 130 / 200 / 250
-    // tokens through 32 layers: 5.50 / 6.06 / 6.36 -> 4.86 / 5.56 / 5.81 ms with the large tiles from 129 rows on)
-    return !(g_gemm_swiglu & 1) && !g_gemm_small_tiles && m >= 129 && f != 0 && f % 128 == 0 && n_pad == 2 * f && k_pad != 0 &&
+    // from 65 rows (fewer take the decode kernels): the 128 x 128 kernel has one or two rows of tiles for the whole device
+    // there, and this launch streams the weight once whatever the row count (one prompt of 65 / 100 / 128 / 130 / 200 / 250
+    // tokens through 32 layers: 4.25 / 4.54 / 4.76 / 5.50 / 6.06 / 6.36 -> 4.01 / 4.19 / 4.28 / 4.59 / 5.21 / 5.46 ms)
+    return !(g_gemm_swiglu & 1) && !g_gemm_small_tiles && m >= 65 && f != 0 && f % 128 == 0 && n_pad == 2 * f && k_pad != 0 &&
            k_pad % 128 == 0;
 }
 namespace {

@@ -227,7 +227,7 @@ void gemm_w8a8_mfma(const int8_t *aq, const int8_t *w_tiles, uint64_t m, uint64_
                     uint64_t k_pad, const EpilogueI8 &ep, int num_cus, hipStream_t s, void *workspace = nullptr,
                     uint64_t workspace_bytes = 0, const SplitKArea *sk = nullptr);
 uint64_t gemm_w8a8_workspace_bytes(uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad, int num_cus);
-// The gate | up projection with SwiGLU in its epilogue (large-tile kernel, m >= 129, f a multiple of 128, k_pad of 128):
+// The gate | up projection with SwiGLU in its epilogue (large-tile kernel, m >= 65, f a multiple of 128, k_pad of 128):
 // w_tiles is the [k, 2 f] weight with the gate columns first; out receives silu(gate) * up, f32 [m, f], bit for bit
 // what gemm_w8a8_mfma into an [m, 2 f] buffer followed by the SwiGLU pass computes.
 extern int g_gemm_pair;       // 1: one block per tile on the 256 x 128 tiles of the large-tile kernel; 2: shared tiles only
