@@ -103,6 +103,7 @@ fa_status fa_set_tuning(int32_t key, int32_t value) {
         case 24: k::g_gemm_pair = value; return FA_OK;
         case 25: fa::g_prefill_rows = value; return FA_OK;
         case 26: fa::g_prefill_fused_rows = value; return FA_OK;
+        case 27: k::g_rows_rope = value; return FA_OK;
     }
     return fail(FA_ERR_INVALID_ARGUMENT, "fa_set_tuning: unknown key");
 }

@@ -424,6 +424,13 @@ fa_status enqueue_prefill_chunk(fa_context *ctx, fa_decoder *d, PrefillBuffers &
                                        (uint16_t *)L.v_pool->ptr, c.n_heads, c.n_kv_heads, c.head_dim, pool_rows};
             k::linear_w8a8_qkv_rope_skinny(t.xq.as<int8_t>(), (const int8_t *)L.wqkv->codes->ptr, t.sx.as<float>(),
                                            (const float *)L.wqkv->scales->ptr, M, L.wqkv->n_pad, L.wqkv->k_pad, qt, s);
+        } else if (const k::QkvRopeTargets qt{t.cos_sin.as<float>(), t.slots.as<uint32_t>(), t.q_bf.as<uint16_t>(),
+                                              (uint16_t *)L.k_pool->ptr, (uint16_t *)L.v_pool->ptr, c.n_heads, c.n_kv_heads,
+                                              c.head_dim, pool_rows};
+                   !decode_form && k::linear_w8a8_qkv_rope_rows_applies(M, L.wqkv->n_pad, L.wqkv->k_pad, cus, &ctx->splitk, qt)) {
+            // 65 to a few hundred rows: the same in the epilogue of the weight-stationary kernel
+            k::linear_w8a8_qkv_rope_rows(t.xq.as<int8_t>(), (const int8_t *)L.wqkv->codes->ptr, t.sx.as<float>(),
+                                         (const float *)L.wqkv->scales->ptr, M, L.wqkv->n_pad, L.wqkv->k_pad, qt, s);
         } else if (!rows_form(L.wqkv) &&
             k::gemm_w8a8_qkv_rope_applies(M, L.wqkv->n, L.wqkv->n_pad, L.wqkv->k_pad, c.n_heads, c.n_kv_heads, c.head_dim, cus)) {
             const k::QkvRopeTargets qt{t.cos_sin.as<float>(), t.slots.as<uint32_t>(), t.q_bf.as<uint16_t>(), (uint16_t *)L.k_pool->ptr,

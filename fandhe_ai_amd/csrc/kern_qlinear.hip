@@ -20,6 +20,7 @@ using namespace fa::dev;
 int g_skinny_ntw = 0;      // tuning overrides (0 = heuristic)
 int g_skinny_waves = 0;
 int g_weight_prefetch = 0;   // 1: row kernels pull nothing for the linear that follows them
+int g_rows_rope = 0;         // q | k | v of a prompt pass on the weight-stationary kernel: 0 RoPE and the append in its epilogue, 1 a pass of their own
 int g_rows_kernel = 0;      // weight-stationary kernel for a few hundred rows: 0 by shape, 1 never, 2 whenever it can run
 int g_skinny_astat = 0;     // activation-stationary kernel: 0 by shape, 1 never, 2 whenever it can run, 3 by shape but not the 33 to 64 row form
 int g_skinny_ksplit = 0;    // split k over the blocks of an XCD: 0 by shape, 1 never, 2 whenever it can run (agent-scope
@@ -365,16 +366,23 @@ __device__ __forceinline__ void store_unseen_b16(void *p, uint32_t v) {
 // tiles meet in LDS and are finished exactly as in the kernel above.  The weight leaves HBM once, an activation
 // byte is read from L2 once per block, and once the weights are in, nothing a wavefront loads comes from HBM, so
 // no L2 hit waits behind a miss.  k_tiles <= 8 KTW; the tiled activation layout of the decode kernels.
-template <int KTW, int NTW>
+// ROPE (two column tiles): the weight is the fused q | k | v projection and the block's tiles are the two halves of a head
+// that the rotation pairs (tile a and tile a + head_dim / 32, as in w8a8_skinny_kernel's mode of that name); the epilogue
+// rotates q and k heads by the row's position, rounds once to bf16 and stores q rows and the new K / V cache rows, with
+// rope_append's expressions, so the f32 projection never reaches memory and the rotation costs no launch.
+template <int KTW, int NTW, bool ROPE = false>
 __global__ void __launch_bounds__(512)
     w8a8_wstat_kernel(const int8_t *__restrict__ xq_tiled, const int8_t *__restrict__ w_tiles, uint32_t m, uint32_t n,
                       uint32_t n_tiles, uint32_t k_tiles, EpiI8 ep) {
     constexpr int NW = 8, MT = 4, NACC = MT * NTW * 4, DS = 4;
     static_assert(KTW % DS == 0, "the ring restarts at slot 0 with every row group");
+    static_assert(!ROPE || NTW == 2, "the rotation pairs two tiles");
     __shared__ int red[NW][NACC][64];
     const int lane = threadIdx.x % 64;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
-    const uint32_t nt0 = blockIdx.x * NTW;
+    const uint32_t half_tiles = ROPE ? ep.head_dim / 32 : 0;
+    const uint32_t nt0 = ROPE ? (blockIdx.x / half_tiles) * 2 * half_tiles + blockIdx.x % half_tiles : blockIdx.x * NTW;
+    const uint32_t nt_step = ROPE ? half_tiles : 1;
     const uint32_t cnt = k_tiles > (uint32_t)wave ? (k_tiles - wave + NW - 1) / NW : 0;      // k-tiles of this wavefront
     const uint32_t row_tiles = (m + 15) / 16, groups = (row_tiles + MT - 1) / MT;
 
@@ -386,7 +394,7 @@ __global__ void __launch_bounds__(512)
         const uint32_t kt = wave + ((uint32_t)t < cnt ? (uint32_t)t : (cnt ? cnt - 1 : 0)) * NW;
 #pragma unroll
         for (int j = 0; j < NTW; ++j) {
-            uint32_t nt = nt0 + j;
+            uint32_t nt = nt0 + j * nt_step;
             nt = nt < n_tiles ? nt : n_tiles - 1;
             const v4i x = stream_load<true>((const v4i *)(w_tiles + ((uint64_t)nt * k_tiles + (kt < k_tiles ? kt : 0)) * 1024 + (uint64_t)lane * 16));
             w[t][j] = (uint32_t)t < cnt ? x : v4i{0, 0, 0, 0};
@@ -398,10 +406,17 @@ __global__ void __launch_bounds__(512)
 #pragma unroll
     for (int q = 0; q < NE; ++q) {
         const int idx = wave + q * NW, j = (idx / 4) % NTW;
-        const uint32_t col = (nt0 + j) * 16 + lane % 16;
+        const uint32_t col = (nt0 + j * nt_step) * 16 + lane % 16;
         p_sw[q] = col < n ? ep.sw[col] : 0.0f;
-        p_bias[q] = (ep.bias && col < n) ? ep.bias[col] : 0.0f;
+        p_bias[q] = (!ROPE && ep.bias && col < n) ? ep.bias[col] : 0.0f;
     }
+    // ROPE: the wavefront finishes pairs instead: pair q = (row tile, element) wave + 8 q of both tiles; the first tile's
+    // column, its head and dim, and the channel scales of the two halves
+    constexpr int NP = ROPE ? MT * 4 / NW : 1;
+    const uint32_t r_col = nt0 * 16 + lane % 16, r_half = ROPE ? ep.head_dim / 2 : 0;
+    const uint32_t r_head = ROPE ? r_col / ep.head_dim : 0, r_dim = ROPE ? r_col % ep.head_dim : 0;
+    const bool r_live = ROPE && r_col + r_half < n;
+    const float r_sw0 = r_live ? ep.sw[r_col] : 0.0f, r_sw1 = r_live ? ep.sw[r_col + r_half] : 0.0f;
     __builtin_amdgcn_sched_barrier(0);
 
     // step (g, t): the MT activation tiles of k-tile t of this wavefront for row group g; row tiles past the last
@@ -421,13 +436,33 @@ __global__ void __launch_bounds__(512)
     for (uint32_t g = 0; g < groups; ++g) {
         // what the epilogue of this group needs, asked for ahead of its multiplies
         float p_sx[NE], p_res[NE];
+        float r_sx[NP], r_cos[NP], r_sin[NP];
+        uint32_t r_slot[NP];
+        if constexpr (ROPE) {
 #pragma unroll
-        for (int q = 0; q < NE; ++q) {
-            const int idx = wave + q * NW, e = idx % 4, j = (idx / 4) % NTW, i = idx / (4 * NTW);
-            const uint32_t row = (g * MT + i) * 16 + 4 * (lane / 16) + e, col = (nt0 + j) * 16 + lane % 16;
-            const bool ok = row < m && col < n;
-            p_sx[q] = ok ? ep.sx[row] : 0.0f;
-            p_res[q] = (ok && ep.residual) ? ep.residual[(uint64_t)row * n + col] : 0.0f;
+            for (int q = 0; q < NP; ++q) {
+                const int idx = wave + q * NW;
+                const uint32_t row = (g * MT + idx / 4) * 16 + 4 * (lane / 16) + idx % 4;
+                r_sx[q] = r_cos[q] = r_sin[q] = 0.0f;
+                r_slot[q] = 0xffffffffu;
+                if (row < m && r_live) {
+                    r_sx[q] = ep.sx[row];
+                    if (r_head < ep.heads + ep.kv_heads) {
+                        r_cos[q] = ep.cos_sin[(uint64_t)row * ep.head_dim + r_dim];
+                        r_sin[q] = ep.cos_sin[(uint64_t)row * ep.head_dim + r_half + r_dim];
+                    }
+                    if (r_head >= ep.heads) r_slot[q] = ep.slots[row];
+                }
+            }
+        } else {
+#pragma unroll
+            for (int q = 0; q < NE; ++q) {
+                const int idx = wave + q * NW, e = idx % 4, j = (idx / 4) % NTW, i = idx / (4 * NTW);
+                const uint32_t row = (g * MT + i) * 16 + 4 * (lane / 16) + e, col = (nt0 + j) * 16 + lane % 16;
+                const bool ok = row < m && col < n;
+                p_sx[q] = ok ? ep.sx[row] : 0.0f;
+                p_res[q] = (ok && ep.residual) ? ep.residual[(uint64_t)row * n + col] : 0.0f;
+            }
         }
         v4i acc[MT][NTW];
 #pragma unroll
@@ -454,6 +489,46 @@ __global__ void __launch_bounds__(512)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) red[wave][(i * NTW + j) * 4 + e][lane] = acc[i][j][e];
         __syncthreads();
+        if constexpr (ROPE) {
+            const uint32_t eq = ep.heads * ep.head_dim, ekv = ep.kv_heads * ep.head_dim;
+#pragma unroll
+            for (int q = 0; q < NP; ++q) {
+                const int idx = wave + q * NW, i = idx / 4, e = idx % 4;
+                int s0 = 0, s1 = 0;
+#pragma unroll
+                for (int ww = 0; ww < NW; ++ww) {
+                    s0 += red[ww][(i * 2 + 0) * 4 + e][lane];
+                    s1 += red[ww][(i * 2 + 1) * 4 + e][lane];
+                }
+                const uint32_t row = (g * MT + i) * 16 + 4 * (lane / 16) + e;
+                if (row < m && r_live) {
+                    float x0 = __fmul_rn((float)s0, __fmul_rn(r_sx[q], r_sw0));
+                    float x1 = __fmul_rn((float)s1, __fmul_rn(r_sx[q], r_sw1));
+                    uint16_t *dst = nullptr;
+                    if (r_head < ep.heads) {
+                        dst = ep.q_out + (uint64_t)row * eq + (uint64_t)r_head * ep.head_dim + r_dim;
+                    } else {
+                        const uint64_t slot = r_slot[q];
+                        if (slot < ep.pool_rows) {
+                            const uint32_t hk = r_head - ep.heads;
+                            dst = (hk < ep.kv_heads ? ep.k_pool + slot * ekv + (uint64_t)hk * ep.head_dim
+                                                    : ep.v_pool + slot * ekv + (uint64_t)(hk - ep.kv_heads) * ep.head_dim) + r_dim;
+                        }
+                    }
+                    if (r_head < ep.heads + ep.kv_heads) {
+                        const float r0 = __fsub_rn(__fmul_rn(x0, r_cos[q]), __fmul_rn(x1, r_sin[q]));
+                        const float r1 = __fadd_rn(__fmul_rn(x1, r_cos[q]), __fmul_rn(x0, r_sin[q]));
+                        x0 = r0;
+                        x1 = r1;
+                    }
+                    if (dst) {
+                        store_unseen_b16(dst, f32_to_bf16(x0));
+                        store_unseen_b16(dst + r_half, f32_to_bf16(x1));
+                    }
+                }
+            }
+            continue;
+        }
 #pragma unroll
         for (int q = 0; q < NE; ++q) {
             const int idx = wave + q * NW;
@@ -2131,6 +2206,38 @@ void linear_w8a8_rows(const int8_t *xq_tiled, const int8_t *w_tiles, uint64_t m,
         else if (k_tiles <= 128) go(integral_constant<int, 16>{}, integral_constant<int, 1>{});
         else go(integral_constant<int, 28>{}, integral_constant<int, 1>{});
     }
+}
+
+// The q | k | v projection of a prompt pass of 65 to a few hundred rows on the weight-stationary kernel with RoPE, the
+// bf16 rounding and the K / V append in its epilogue (w8a8_wstat_kernel<8, 2, true>: a block per pair of tiles that the
+// rotation pairs).  Applies where linear_w8a8_rows would take the unsplit kernel and a wavefront holds its k-tiles.
+bool linear_w8a8_qkv_rope_rows_applies(uint64_t m, uint64_t n_pad, uint64_t k_pad, int num_cus, const SplitKArea *sk,
+                                       const QkvRopeTargets &t) {
+    if (g_rows_rope == 1 || k_pad == 0 || k_pad / 64 > 64 || t.head_dim == 0 || t.head_dim % 32 != 0) return false;
+    const uint64_t n = (uint64_t)(t.heads + 2 * t.kv_heads) * t.head_dim;
+    if (n == 0 || n != n_pad) return false;
+    RowsKsplitPlan kp;
+    if (rows_ksplit_plan(m, (uint32_t)(n_pad / 16), (uint32_t)(k_pad / 64), num_cus, sk, &kp)) return false;
+    return linear_w8a8_rows_applies(m, n_pad, k_pad, num_cus, sk);
+}
+void linear_w8a8_qkv_rope_rows(const int8_t *xq_tiled, const int8_t *w_tiles, const float *sx, const float *sw, uint64_t m,
+                               uint64_t n_pad, uint64_t k_pad, const QkvRopeTargets &t, hipStream_t s) {
+    if (m == 0) return;
+    const uint32_t n = (t.heads + 2 * t.kv_heads) * t.head_dim;
+    EpiI8 e{};
+    e.sx = sx;
+    e.sw = sw;
+    e.cos_sin = t.cos_sin;
+    e.slots = t.slots;
+    e.q_out = t.q_out;
+    e.k_pool = t.k_pool;
+    e.v_pool = t.v_pool;
+    e.heads = t.heads;
+    e.kv_heads = t.kv_heads;
+    e.head_dim = t.head_dim;
+    e.pool_rows = t.pool_rows;
+    w8a8_wstat_kernel<8, 2, true><<<n / 32, 512, 0, s>>>(xq_tiled, w_tiles, (uint32_t)m, n, (uint32_t)(n_pad / 16),
+                                                       (uint32_t)(k_pad / 64), e);
 }
 
 void linear_w8a8_swiglu_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, const float *sx, const float *sw,

@@ -191,6 +191,13 @@ struct QkvRopeTargets {
 void linear_w8a8_qkv_rope_skinny(const int8_t *xq_tiled, const int8_t *w_tiles, const float *sx, const float *sw,
                                  uint64_t m, uint64_t n_pad, uint64_t k_pad, const QkvRopeTargets &t, hipStream_t s,
                                  const RowPrologue *pro = nullptr);
+// The same for 65 to a few hundred rows, on the weight-stationary kernel (see linear_w8a8_rows): whether it applies to a
+// shape, and the launch.  Bit for bit what linear_w8a8_rows into an [m, n] f32 buffer followed by rope_append leaves.
+extern int g_rows_rope;
+bool linear_w8a8_qkv_rope_rows_applies(uint64_t m, uint64_t n_pad, uint64_t k_pad, int num_cus, const SplitKArea *sk,
+                                       const QkvRopeTargets &t);
+void linear_w8a8_qkv_rope_rows(const int8_t *xq_tiled, const int8_t *w_tiles, const float *sx, const float *sw, uint64_t m,
+                               uint64_t n_pad, uint64_t k_pad, const QkvRopeTargets &t, hipStream_t s);
 // The q | k | v projection of a prompt pass on the large-tile GEMM with rope_append's work in its epilogue (aq row-major
 // codes): bit for bit what gemm_w8a8_mfma into an [m, n] f32 buffer followed by rope_append leaves in q_out and the pools.
 bool gemm_w8a8_qkv_rope_applies(uint64_t m, uint64_t n, uint64_t n_pad, uint64_t k_pad, uint32_t heads, uint32_t kv_heads,

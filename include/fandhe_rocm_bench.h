@@ -108,7 +108,9 @@ fa_status fa_probe_l2_path(fa_context *ctx, const fa_buffer *cold, uint64_t cold
  *        alone cover half the device (pairs);
  * key 25: rows (sequences x tokens) per chunk of a prompt pass, from 256 up; anything smaller: the built-in 8192;
  * key 26: prompt passes of at most 64 rows: 0: q | k | v and gate | up on the decode step's fused kernels (RoPE and the
- *        K / V append, SwiGLU, in the epilogues), 1: plain projections and separate passes. */
+ *        K / V append, SwiGLU, in the epilogues), 1: plain projections and separate passes;
+ * key 27: prompt passes whose q | k | v projection runs on the weight-stationary kernel: 0: RoPE, the bf16 rounding and
+ *        the K / V append in that kernel's epilogue, 1: a pass of their own behind it. */
 fa_status fa_set_tuning(int32_t key, int32_t value);
 
 /* What the context found when it was created: xcd_local = 1 when workgroups b and b + 8 of a launch were seen to
