@@ -210,13 +210,13 @@ fa_status enqueue_step(fa_context *ctx, fa_decoder *d, int stop_after = -1) {
         const k::QkvRopeTargets t{(const float *)d->cos_sin->ptr, (const uint32_t *)d->slots->ptr, (uint16_t *)d->q_bf->ptr,
                                   (uint16_t *)L.k_pool->ptr, (uint16_t *)L.v_pool->ptr, c.n_heads, c.n_kv_heads,
                                   c.head_dim, pool_rows};
-        // With at most four rows the linears redo the row work in front of them inside their own launch
-        // (k::RowPrologue): the row stage then launches nothing and its outputs (codes, scales) appear with the
-        // linear's stage, written by one block of it.
+        // With one or two rows (by measurement; the kernels take four) the linears redo the row work in front of them
+        // inside their own launch (k::RowPrologue): the row stage then launches nothing and its outputs (codes,
+        // scales) appear with the linear's stage, written by one block of it.
         const bool fuse_qkv = k::qkv_rope_fuses_norm(B, L.wqkv->k_pad);
-        // One or two short sequences: the attention finishes in one launch (a block per sequence and kv head; no
+        // Short sequences: the attention finishes in one launch (a block per sequence and kv head; no
         // partial results, no merge launch) and leaves its output and the heads' maxima for the o projection, which
-        // does the per-token quantizer itself.
+        // does the per-token quantizer itself when there is one row (a launch of its own otherwise).
         const bool one_form = short_ctx && c.n_heads <= 32 && F >= EQ && EQ % 64 == 0;
         const bool one_attn = one_form && k::plain_fuses_pmax_quantizer(B, L.wo->n_pad, L.wo->k_pad, cus);
         if (!fuse_qkv)

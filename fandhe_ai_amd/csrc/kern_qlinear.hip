@@ -26,7 +26,7 @@ int g_skinny_astat = 0;     // activation-stationary kernel: 0 by shape, 1 never
 int g_skinny_ksplit = 0;    // split k over the blocks of an XCD: 0 by shape, 1 never, 2 whenever it can run (agent-scope
                             // meeting), 3 whenever it can run (meeting in the XCD's L2), 4 by shape but agent scope
 int g_skinny_ksplit_s = 0;  // members per group of the split (0 by shape, 2 or 4)
-int g_row_fusion = 0;       // row work inside the linears for at most four rows: 0 by shape, 1 never
+int g_row_fusion = 0;       // row work inside the linears: 0 where it measured faster (norm: two rows, quantizer: one), 1 never, 2 up to the kernels' four / two rows
 
 namespace {
 
@@ -2026,7 +2026,10 @@ namespace {
 inline size_t prologue_lds_bytes(uint64_t m, uint64_t k_pad) { return (size_t)((m * k_pad + 15) / 16 * 16); }
 inline bool norm_prologue_shape(uint64_t m, uint64_t k_pad) {
     // the stand-alone kernel whose f64 association the prologue reproduces is the 1024-thread, one-group-per-thread form
-    return g_row_fusion != 1 && m >= 1 && m <= 4 && k_pad > 1024 && k_pad <= 4096 && k_pad % 64 == 0;
+    // by measurement one or two rows (whole steps of 1 / 2 / 3 / 4 rows through 32 layers, contexts 100-200: 2.10 / 2.22 / 2.35 /
+    // 2.47 ms with the row work in here against 2.30 / 2.34 / 2.29 / 2.30 ms with the row kernels); the kernels take four
+    const uint64_t rows = g_row_fusion == 2 ? 4 : 2;
+    return g_row_fusion != 1 && m >= 1 && m <= rows && k_pad > 1024 && k_pad <= 4096 && k_pad % 64 == 0;
 }
 }  // namespace
 
@@ -2035,7 +2038,9 @@ bool swiglu_fuses_norm(uint64_t m, uint64_t n_pad, uint64_t k_pad, int num_cus) 
     return norm_prologue_shape(m, k_pad) && astat_applies(n_pad / 32, k_pad / 64, num_cus);
 }
 bool plain_fuses_pmax_quantizer(uint64_t m, uint64_t n_pad, uint64_t k_pad, int num_cus) {
-    if (g_row_fusion == 1 || m == 0 || m > 2 || k_pad % 64 != 0 || k_pad > 16384) return false;     // PmaxRows
+    // by measurement one row (two rows: 2.22 ms a step without, 2.34 ms with); the kernel takes two
+    const uint64_t rows = g_row_fusion == 2 ? 2 : 1;
+    if (g_row_fusion == 1 || m == 0 || m > rows || k_pad % 64 != 0 || k_pad > 16384) return false;     // PmaxRows
     if (k_pad / 16 > 1024) return false;                     // partial maxima per row the prologue reads
     const uint64_t n_tiles = n_pad / 16, k_tiles = k_pad / 64;
     if (astat_applies((n_tiles + 1) / 2, k_tiles, num_cus)) return false;

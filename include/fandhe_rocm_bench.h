@@ -86,8 +86,9 @@ fa_status fa_probe_l2_path(fa_context *ctx, const fa_buffer *cold, uint64_t cold
  * key 18: 1 keeps the 256-thread form of the row kernels (norm, quantizer, norm + quantizer) for every row count
  *        instead of the up-to-1024-thread form used for at most 256 rows;
  * key 19: 1 keeps the norm + quantizer and quantizer kernels of a decode step as launches of their own for every batch
- *        size; 0: for at most four rows the linears that follow do that row work themselves (takes effect when a step
- *        is recorded);
+ *        size; 0: the linears that follow do that row work themselves where that measured faster (norm + quantizer: one
+ *        or two rows, quantizer from partial maxima: one row); 2: wherever the kernels can (four / two rows); takes
+ *        effect when a step is recorded;
  * key 20: 1 keeps the streamed attention with its merge launch for every decode step; 0: a step whose contexts are
  *        at most 1024 tokens runs the attention as one launch (a block per sequence and kv head) while there is at
  *        most one such block per compute unit (with one or two sequences the o projection then does the quantizer);

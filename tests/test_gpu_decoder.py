@@ -110,7 +110,7 @@ def test_small_batches_do_the_row_work_inside_the_linears(shape, batch):
         # the last bits of its output, and the one-launch form for short contexts divides them its own way)
         fa.check(lib.fa_set_tuning(20, 1))
         for fused in (True, False):
-            fa.check(lib.fa_set_tuning(19, 0 if fused else 1))
+            fa.check(lib.fa_set_tuning(19, 2 if fused else 1))
             dec = GpuDecoder(be, m)
             try:
                 # what the row stages leave behind, read after the linear that would consume it: the q | k | v projection
